@@ -1,0 +1,610 @@
+/*
+ * iom_oracle.c — CPU restatement of the reference CPU backend (see
+ * iom_oracle.h).  TEST INFRASTRUCTURE ONLY: nothing shipped may link this.
+ *
+ * Build without FMA contraction and without ISA flags (plain -O2
+ * -ffp-contract=off): the reference's sequential F32 recurrences
+ * `sum + v*v` and `(v*inverse)*scale` must stay two roundings.
+ */
+#include "iom_oracle.h"
+
+#include <math.h>
+#include <string.h>
+
+#define TILE 16u
+#define TILE_SLOTS 256u
+
+/* ------------------------------------------------------------------ */
+/* Layout (src/tensor.cpp:76-164)                                       */
+/* ------------------------------------------------------------------ */
+
+size_t iomo_leaf_bytes(int dtype) {
+    switch (dtype) {
+        case IOMO_DT_BF16: return 2;
+        case IOMO_DT_I32:
+        case IOMO_DT_U32:
+        case IOMO_DT_F32: return 4;
+        default: return 0;
+    }
+}
+
+static uint64_t tiles_of(uint64_t extent) { return (extent + TILE - 1) / TILE; }
+
+uint64_t iomo_plane_elems(uint64_t rows, uint64_t cols) {
+    return tiles_of(rows) * tiles_of(cols) * TILE_SLOTS;
+}
+
+uint64_t iomo_plane_slot(uint64_t rows, uint64_t cols, uint64_t plane,
+                         uint64_t row, uint64_t col) {
+    const uint64_t tile_cols = tiles_of(cols);
+    const uint64_t tiles_per_plane = tiles_of(rows) * tile_cols;
+    const uint64_t tile = plane * tiles_per_plane + (row / TILE) * tile_cols
+            + col / TILE;
+    return tile * TILE_SLOTS + (row % TILE) * TILE + col % TILE;
+}
+
+static uint64_t load_leaf(const void* base, uint64_t slot, size_t bytes) {
+    if (bytes == 2) {
+        uint16_t v;
+        memcpy(&v, (const unsigned char*)base + slot * 2, 2);
+        return v;
+    }
+    uint32_t v;
+    memcpy(&v, (const unsigned char*)base + slot * 4, 4);
+    return v;
+}
+
+static void store_leaf(void* base, uint64_t slot, size_t bytes, uint64_t raw) {
+    if (bytes == 2) {
+        const uint16_t v = (uint16_t)raw;
+        memcpy((unsigned char*)base + slot * 2, &v, 2);
+    } else {
+        const uint32_t v = (uint32_t)raw;
+        memcpy((unsigned char*)base + slot * 4, &v, 4);
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* Named-format codec (src/shared/scalar_binary_codec.hpp:30-148)       */
+/* ------------------------------------------------------------------ */
+
+typedef struct {
+    unsigned ebits, fbits;
+    int bias;
+} fmt_t;
+
+static int float_format(int dtype, fmt_t* f) {
+    if (dtype == IOMO_DT_BF16) { f->ebits = 8; f->fbits = 7; f->bias = 127; return 1; }
+    if (dtype == IOMO_DT_F32) { f->ebits = 8; f->fbits = 23; f->bias = 127; return 1; }
+    return 0;
+}
+
+/* :45-65 — both in-scope float leaves have infinities and NaNs. */
+static long double codec_decode(uint64_t raw, fmt_t f) {
+    const uint64_t emask = (1ull << f.ebits) - 1;
+    const uint64_t sign = (raw >> (f.ebits + f.fbits)) & 1;
+    const uint64_t frac = raw & ((1ull << f.fbits) - 1);
+    const uint64_t exp = (raw >> f.fbits) & emask;
+    long double v;
+    if (exp == emask) {
+        if (frac != 0) return (long double)NAN;
+        return sign ? -(long double)INFINITY : (long double)INFINITY;
+    }
+    if (exp != 0) {
+        v = ldexpl((long double)((1ull << f.fbits) + frac),
+                   (int)exp - f.bias - (int)f.fbits);
+    } else {
+        v = ldexpl((long double)frac, 1 - f.bias - (int)f.fbits);
+    }
+    return sign ? -v : v;
+}
+
+/* :110-118 */
+static uint64_t codec_round_even(long double v) {
+    const long double whole = floorl(v);
+    const long double rest = v - whole;
+    uint64_t q = (uint64_t)whole;
+    if (rest > 0.5L || (rest == 0.5L && (q & 1))) ++q;
+    return q;
+}
+
+/* :67-108 */
+static uint64_t codec_encode(long double v, fmt_t f) {
+    const uint64_t sign = signbit(v) ? 1 : 0;
+    const uint64_t emask = (1ull << f.ebits) - 1;
+    const unsigned shift = f.ebits + f.fbits;
+    const uint64_t inf_bits = (sign << shift) | (emask << f.fbits);
+    v = fabsl(v);
+    if (isnan(v)) return (sign << shift) | (emask << f.fbits) | (1ull << (f.fbits - 1));
+    if (isinf(v)) return inf_bits;
+    if (v == 0) return sign << shift;
+    const int min_sub = 1 - f.bias - (int)f.fbits;
+    const int max_exp = (int)(emask - 1) - f.bias;
+    int e = 0;
+    (void)frexpl(v, &e);
+    --e;
+    if (e < min_sub + (int)f.fbits) {
+        const uint64_t q = codec_round_even(ldexpl(v, -min_sub));
+        if (q == (1ull << f.fbits)) return (sign << shift) | (1ull << f.fbits);
+        return (sign << shift) | q;
+    }
+    if (e > max_exp) return inf_bits;
+    uint64_t frac = codec_round_even(
+            ldexpl(v, (int)f.fbits - e) - (long double)(1ull << f.fbits));
+    if (frac == (1ull << f.fbits)) { ++e; frac = 0; }
+    if (e > max_exp) return inf_bits;
+    return (sign << shift) | ((uint64_t)(e + f.bias) << f.fbits) | frac;
+}
+
+/* :120-148 */
+static long double codec_arith(int op, long double x, long double y) {
+    if (isnan(x) || isnan(y)) return (long double)NAN;
+    if (op == IOMO_OP_ADD) {
+        if (isinf(x) && isinf(y) && signbit(x) != signbit(y)) return (long double)NAN;
+        if (x == 0 && y == 0) return (signbit(x) && signbit(y)) ? -0.0L : 0.0L;
+        const long double r = x + y;
+        return r == 0 ? 0.0L : r;
+    }
+    if (op == IOMO_OP_MUL) {
+        if ((isinf(x) && y == 0) || (isinf(y) && x == 0)) return (long double)NAN;
+        return x * y;
+    }
+    if (isinf(x) && isinf(y) && signbit(x) == signbit(y)) return (long double)NAN;
+    return x - y;
+}
+
+/* The codec stores every NaN as sign 0, exponent all-ones, top fraction bit
+ * (:79-84, quiet_nan() has a clear sign on x86-64). */
+uint64_t iomo_scalar_binary(int op, int dtype, uint64_t a, uint64_t b) {
+    if (dtype == IOMO_DT_I32 || dtype == IOMO_DT_U32) {
+        const uint64_t mask = 0xFFFFFFFFull;
+        if (op == IOMO_OP_ADD) return (a + b) & mask;
+        if (op == IOMO_OP_MUL) return (a * b) & mask;
+        return (a - b) & mask;
+    }
+    fmt_t f;
+    if (!float_format(dtype, &f)) return 0;
+    const long double r = codec_arith(op, codec_decode(a, f), codec_decode(b, f));
+    if (isnan(r)) return (((1ull << f.ebits) - 1) << f.fbits) | (1ull << (f.fbits - 1));
+    return codec_encode(r, f);
+}
+
+uint16_t iomo_encode_bf16(float value) {
+    fmt_t f;
+    float_format(IOMO_DT_BF16, &f);
+    if (isnan(value)) return 0x7FC0u;
+    return (uint16_t)codec_encode((long double)value, f);
+}
+
+/* ---- closed form: IEEE-754 binary32 single rounding ---------------- */
+
+static float f32_from_bits(uint32_t b) { float f; memcpy(&f, &b, 4); return f; }
+static uint32_t f32_bits(float f) { uint32_t b; memcpy(&b, &f, 4); return b; }
+
+static uint16_t bf16_rne_bits(uint32_t bits) {
+    if ((bits & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0u;
+    return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
+}
+
+uint64_t iomo_scalar_binary_ieee(int op, int dtype, uint64_t a, uint64_t b) {
+    if (dtype == IOMO_DT_I32 || dtype == IOMO_DT_U32) {
+        const uint32_t x = (uint32_t)a, y = (uint32_t)b;
+        if (op == IOMO_OP_ADD) return (uint32_t)(x + y);
+        if (op == IOMO_OP_MUL) return (uint32_t)(x * y);
+        return (uint32_t)(x - y);
+    }
+    if (dtype == IOMO_DT_F32) {
+        const volatile float x = f32_from_bits((uint32_t)a);
+        const volatile float y = f32_from_bits((uint32_t)b);
+        volatile float r;
+        if (op == IOMO_OP_ADD) r = x + y;
+        else if (op == IOMO_OP_MUL) r = x * y;
+        else r = x - y;
+        if (r != r) return 0x7FC00000u;
+        return f32_bits(r);
+    }
+    if (dtype == IOMO_DT_BF16) {
+        const float x = f32_from_bits((uint32_t)a << 16);
+        const float y = f32_from_bits((uint32_t)b << 16);
+        if (op == IOMO_OP_MUL) {
+            /* The product of two 8-bit significands is exact in binary64 and
+             * binary64 has the exponent range for it, so one rounding from the
+             * exact value is what remains.  Round on the BF16 grid directly. */
+            const double p = (double)x * (double)y;
+            if (p != p) return 0x7FC0u;
+            if (isinf(p)) return p < 0 ? 0xFF80u : 0x7F80u;
+            const double m = fabs(p);
+            const uint64_t sign = signbit(p) ? 0x8000u : 0;
+            if (m == 0) return sign;
+            int e;
+            (void)frexp(m, &e); /* m = f * 2^e, f in [0.5,1) */
+            --e;
+            int quantum = e - 7;              /* normal BF16 ulp exponent */
+            if (quantum < -133) quantum = -133; /* subnormal grid 2^-133   */
+            const double scaled = ldexp(m, -quantum); /* exact */
+            double q = floor(scaled);
+            const double rest = scaled - q;
+            if (rest > 0.5 || (rest == 0.5 && fmod(q, 2.0) != 0)) q += 1;
+            const double rounded = ldexp(q, quantum);
+            if (rounded > 3.3895313892515355e38) return sign | 0x7F80u;
+            const float back = (float)rounded; /* exact: on the BF16 grid */
+            return sign | (f32_bits(back) >> 16);
+        }
+        const volatile float r = (op == IOMO_OP_ADD) ? x + y : x - y;
+        return bf16_rne_bits(f32_bits(r));
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* SiLU (src/shared/scalar_silu.hpp:69-97, float carrier)               */
+/* ------------------------------------------------------------------ */
+
+static float silu_f32(float x) {
+    if (isnan(x)) return NAN;
+    if (isinf(x)) return signbit(x) ? -0.0f : INFINITY;
+    if (x == 0.0f) return x;
+    if (x >= 0.0f) {
+        const volatile float e = expf(-x);
+        const volatile float d = 1.0f + e;
+        return x / d;
+    }
+    const volatile float t = expf(x * 0.5f);
+    const volatile float xt = x * t;
+    const volatile float num = xt * t;
+    const volatile float tt = t * t;
+    const volatile float den = 1.0f + tt;
+    return num / den;
+}
+
+uint64_t iomo_scalar_silu(int dtype, uint64_t raw) {
+    fmt_t f;
+    if (!float_format(dtype, &f)) return 0;
+    /* decode through the codec in the float carrier: exact for both leaves */
+    const float x = (float)codec_decode(raw, f);
+    const float y = silu_f32(x);
+    if (isnan(y)) return (((1ull << f.ebits) - 1) << f.fbits) | (1ull << (f.fbits - 1));
+    return codec_encode((long double)y, f);
+}
+
+/* ------------------------------------------------------------------ */
+/* View helpers                                                         */
+/* ------------------------------------------------------------------ */
+
+static int view_ok(const iomo_view* v) {
+    if (!v || !v->base || v->rank < 2 || v->rank > 8) return 0;
+    for (uint32_t i = 0; i < v->rank; ++i) if (v->dims[i] == 0) return 0;
+    return 1;
+}
+
+static uint64_t view_rows(const iomo_view* v) { return v->dims[v->rank - 2]; }
+static uint64_t view_cols(const iomo_view* v) { return v->dims[v->rank - 1]; }
+
+/* Row-major walk over the leading coordinates of `dims[0..leading)`. */
+static int next_coord(uint64_t* coord, const uint64_t* dims, uint32_t leading) {
+    for (uint32_t i = leading; i-- > 0;) {
+        if (++coord[i] < dims[i]) return 1;
+        coord[i] = 0;
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* Binary (src/cpu/queue.cpp:414-536)                                   */
+/* ------------------------------------------------------------------ */
+
+typedef struct {
+    uint64_t strides[6]; /* result-aligned, 0 on broadcast / missing axes */
+    int bcast_rows, bcast_cols;
+} bsnap_t;
+
+/* src/device_ops_binary.cpp:61-100 */
+static void snapshot(const iomo_view* v, const uint64_t* rdims, uint32_t rrank,
+                     bsnap_t* s) {
+    const uint32_t offset = rrank - v->rank;
+    const uint32_t rleading = rrank - 2;
+    for (uint32_t axis = 0; axis < rleading; ++axis) {
+        s->strides[axis] = 0;
+        if (axis < offset) continue;
+        const uint32_t src = axis - offset;
+        if (v->dims[src] == 1 && rdims[axis] != 1) continue;
+        s->strides[axis] = v->plane_strides[src];
+    }
+    s->bcast_rows = view_rows(v) == 1 && rdims[rrank - 2] != 1;
+    s->bcast_cols = view_cols(v) == 1 && rdims[rrank - 1] != 1;
+}
+
+int iomo_binary(int op, int dtype, const iomo_view* lhs, const iomo_view* rhs,
+                const iomo_view* out, int use_ieee) {
+    const size_t bytes = iomo_leaf_bytes(dtype);
+    if (!bytes) return IOMO_ERR_UNSUPPORTED;
+    if (op < IOMO_OP_ADD || op > IOMO_OP_SUB) return IOMO_ERR_INVALID;
+    if (!view_ok(lhs) || !view_ok(rhs) || !view_ok(out)) return IOMO_ERR_INVALID;
+    /* src/device_ops_binary.cpp:121-143: right-aligned broadcast */
+    const uint32_t rank = lhs->rank > rhs->rank ? lhs->rank : rhs->rank;
+    uint64_t rdims[8];
+    for (uint32_t i = 0; i < rank; ++i) {
+        const uint64_t l = i < rank - lhs->rank ? 1 : lhs->dims[i - (rank - lhs->rank)];
+        const uint64_t r = i < rank - rhs->rank ? 1 : rhs->dims[i - (rank - rhs->rank)];
+        if (l != r && l != 1 && r != 1) return IOMO_ERR_INVALID;
+        rdims[i] = l > r ? l : r;
+    }
+    if (out->rank != rank) return IOMO_ERR_INVALID;
+    for (uint32_t i = 0; i < rank; ++i)
+        if (out->dims[i] != rdims[i]) return IOMO_ERR_INVALID;
+
+    bsnap_t ls, rs, os;
+    snapshot(lhs, rdims, rank, &ls);
+    snapshot(rhs, rdims, rank, &rs);
+    snapshot(out, rdims, rank, &os);
+    const uint32_t leading = rank - 2;
+    const uint64_t rows = rdims[rank - 2], cols = rdims[rank - 1];
+    uint64_t coord[8] = {0};
+    do {
+        uint64_t lp = lhs->plane_offset, rp = rhs->plane_offset, op_ = out->plane_offset;
+        for (uint32_t a = 0; a < leading; ++a) {
+            lp += coord[a] * ls.strides[a];
+            rp += coord[a] * rs.strides[a];
+            op_ += coord[a] * os.strides[a];
+        }
+        for (uint64_t r = 0; r < rows; ++r) {
+            for (uint64_t c = 0; c < cols; ++c) {
+                const uint64_t lslot = iomo_plane_slot(
+                        view_rows(lhs), view_cols(lhs), lp,
+                        ls.bcast_rows ? 0 : r, ls.bcast_cols ? 0 : c);
+                const uint64_t rslot = iomo_plane_slot(
+                        view_rows(rhs), view_cols(rhs), rp,
+                        rs.bcast_rows ? 0 : r, rs.bcast_cols ? 0 : c);
+                const uint64_t oslot = iomo_plane_slot(rows, cols, op_, r, c);
+                const uint64_t a = load_leaf(lhs->base, lslot, bytes);
+                const uint64_t b = load_leaf(rhs->base, rslot, bytes);
+                const uint64_t y = use_ieee
+                        ? iomo_scalar_binary_ieee(op, dtype, a, b)
+                        : iomo_scalar_binary(op, dtype, a, b);
+                store_leaf(out->base, oslot, bytes, y);
+            }
+        }
+    } while (next_coord(coord, rdims, leading));
+    return IOMO_OK;
+}
+
+/* ------------------------------------------------------------------ */
+/* RMSNorm (src/cpu/queue.cpp:1144-1296, float carrier)                 */
+/* ------------------------------------------------------------------ */
+
+int iomo_rmsnorm(int dtype, const iomo_view* x, const iomo_view* scale,
+                 const iomo_view* out, float eps) {
+    fmt_t f;
+    if (!view_ok(x) || !view_ok(scale) || !view_ok(out)) return IOMO_ERR_INVALID;
+    if (x->rank != out->rank) return IOMO_ERR_INVALID;
+    for (uint32_t i = 0; i < x->rank; ++i)
+        if (x->dims[i] != out->dims[i]) return IOMO_ERR_INVALID;
+    const uint64_t rows = view_rows(x), feats = view_cols(x);
+    if (scale->rank != 2 || scale->dims[0] != 1 || scale->dims[1] != feats)
+        return IOMO_ERR_INVALID;
+    if (out->base == x->base || out->base == scale->base) return IOMO_ERR_INVALID;
+    if (!float_format(dtype, &f)) return IOMO_ERR_UNSUPPORTED;
+    if (!isfinite(eps) || eps < 0.0f) return IOMO_ERR_INVALID;
+    const size_t bytes = iomo_leaf_bytes(dtype);
+    const uint32_t leading = x->rank - 2;
+    const float divisor = (float)feats;
+    uint64_t coord[8] = {0};
+    do {
+        uint64_t xp = x->plane_offset, yp = out->plane_offset;
+        for (uint32_t a = 0; a < leading; ++a) {
+            xp += coord[a] * x->plane_strides[a];
+            yp += coord[a] * out->plane_strides[a];
+        }
+        for (uint64_t r = 0; r < rows; ++r) {
+            volatile float sum = 0.0f;
+            for (uint64_t c = 0; c < feats; ++c) {
+                const float v = (float)codec_decode(
+                        load_leaf(x->base, iomo_plane_slot(rows, feats, xp, r, c), bytes), f);
+                const volatile float sq = v * v;
+                sum = sum + sq;
+            }
+            const volatile float mean = sum / divisor;
+            const volatile float shifted = mean + eps;
+            const volatile float root = sqrtf(shifted);
+            const volatile float inverse = 1.0f / root;
+            for (uint64_t c = 0; c < feats; ++c) {
+                const float v = (float)codec_decode(
+                        load_leaf(x->base, iomo_plane_slot(rows, feats, xp, r, c), bytes), f);
+                const float w = (float)codec_decode(
+                        load_leaf(scale->base,
+                                  iomo_plane_slot(1, feats, scale->plane_offset, 0, c), bytes), f);
+                const volatile float normalized = v * inverse;
+                const volatile float y = normalized * w;
+                uint64_t raw;
+                if (y != y) raw = (((1ull << f.ebits) - 1) << f.fbits) | (1ull << (f.fbits - 1));
+                else raw = codec_encode((long double)y, f);
+                store_leaf(out->base, iomo_plane_slot(rows, feats, yp, r, c), bytes, raw);
+            }
+        }
+    } while (next_coord(coord, x->dims, leading));
+    return IOMO_OK;
+}
+
+/* ------------------------------------------------------------------ */
+/* SiLU / copy: two-view plane walks                                    */
+/* ------------------------------------------------------------------ */
+
+static int same_shape(const iomo_view* a, const iomo_view* b) {
+    if (a->rank != b->rank) return 0;
+    for (uint32_t i = 0; i < a->rank; ++i) if (a->dims[i] != b->dims[i]) return 0;
+    return 1;
+}
+
+int iomo_silu(int dtype, const iomo_view* x, const iomo_view* y) {
+    fmt_t f;
+    if (!view_ok(x) || !view_ok(y) || !same_shape(x, y)) return IOMO_ERR_INVALID;
+    if (!float_format(dtype, &f)) return IOMO_ERR_UNSUPPORTED;
+    const size_t bytes = iomo_leaf_bytes(dtype);
+    const uint64_t rows = view_rows(x), cols = view_cols(x);
+    const uint32_t leading = x->rank - 2;
+    uint64_t coord[8] = {0};
+    do {
+        uint64_t xp = x->plane_offset, yp = y->plane_offset;
+        for (uint32_t a = 0; a < leading; ++a) {
+            xp += coord[a] * x->plane_strides[a];
+            yp += coord[a] * y->plane_strides[a];
+        }
+        for (uint64_t r = 0; r < rows; ++r)
+            for (uint64_t c = 0; c < cols; ++c)
+                store_leaf(y->base, iomo_plane_slot(rows, cols, yp, r, c), bytes,
+                           iomo_scalar_silu(dtype, load_leaf(
+                                   x->base, iomo_plane_slot(rows, cols, xp, r, c), bytes)));
+    } while (next_coord(coord, x->dims, leading));
+    return IOMO_OK;
+}
+
+int iomo_copy(int dtype, const iomo_view* src, const iomo_view* dst) {
+    const size_t bytes = iomo_leaf_bytes(dtype);
+    if (!bytes) return IOMO_ERR_UNSUPPORTED;
+    if (!view_ok(src) || !view_ok(dst) || !same_shape(src, dst)) return IOMO_ERR_INVALID;
+    const uint64_t rows = view_rows(src), cols = view_cols(src);
+    const uint32_t leading = src->rank - 2;
+    uint64_t coord[8] = {0};
+    do {
+        uint64_t sp = src->plane_offset, dp = dst->plane_offset;
+        for (uint32_t a = 0; a < leading; ++a) {
+            sp += coord[a] * src->plane_strides[a];
+            dp += coord[a] * dst->plane_strides[a];
+        }
+        for (uint64_t r = 0; r < rows; ++r)
+            for (uint64_t c = 0; c < cols; ++c)
+                store_leaf(dst->base, iomo_plane_slot(rows, cols, dp, r, c), bytes,
+                           load_leaf(src->base, iomo_plane_slot(rows, cols, sp, r, c), bytes));
+    } while (next_coord(coord, src->dims, leading));
+    return IOMO_OK;
+}
+
+/* src/cpu/tensor.cpp:79-167: the logical side is dense row-major over the
+ * view's own shape. */
+int iomo_scatter(int dtype, const iomo_view* dst, const void* logical) {
+    const size_t bytes = iomo_leaf_bytes(dtype);
+    if (!bytes) return IOMO_ERR_UNSUPPORTED;
+    if (!view_ok(dst) || !logical) return IOMO_ERR_INVALID;
+    const uint64_t rows = view_rows(dst), cols = view_cols(dst);
+    const uint32_t leading = dst->rank - 2;
+    uint64_t coord[8] = {0};
+    uint64_t index = 0;
+    do {
+        uint64_t dp = dst->plane_offset;
+        for (uint32_t a = 0; a < leading; ++a) dp += coord[a] * dst->plane_strides[a];
+        for (uint64_t r = 0; r < rows; ++r)
+            for (uint64_t c = 0; c < cols; ++c, ++index)
+                store_leaf(dst->base, iomo_plane_slot(rows, cols, dp, r, c), bytes,
+                           load_leaf(logical, index, bytes));
+    } while (next_coord(coord, dst->dims, leading));
+    return IOMO_OK;
+}
+
+int iomo_gather(int dtype, const iomo_view* src, void* logical) {
+    const size_t bytes = iomo_leaf_bytes(dtype);
+    if (!bytes) return IOMO_ERR_UNSUPPORTED;
+    if (!view_ok(src) || !logical) return IOMO_ERR_INVALID;
+    const uint64_t rows = view_rows(src), cols = view_cols(src);
+    const uint32_t leading = src->rank - 2;
+    uint64_t coord[8] = {0};
+    uint64_t index = 0;
+    do {
+        uint64_t sp = src->plane_offset;
+        for (uint32_t a = 0; a < leading; ++a) sp += coord[a] * src->plane_strides[a];
+        for (uint64_t r = 0; r < rows; ++r)
+            for (uint64_t c = 0; c < cols; ++c, ++index)
+                store_leaf(logical, index, bytes,
+                           load_leaf(src->base, iomo_plane_slot(rows, cols, sp, r, c), bytes));
+    } while (next_coord(coord, src->dims, leading));
+    return IOMO_OK;
+}
+
+/* ------------------------------------------------------------------ */
+/* Softmax stage (src/cpu/sdpa.cpp:214-309)                             */
+/* ------------------------------------------------------------------ */
+
+static uint64_t stage_offset(const iomo_stage_layout* l, uint64_t plane,
+                             uint64_t head, uint64_t row, uint64_t col) {
+    return l->plane_offset + plane * l->plane_stride + head * l->head_stride
+            + row * l->row_stride + col * l->column_stride;
+}
+
+int iomo_softmax(const iomo_softmax_desc* d) {
+    if (!d || !d->scores || !d->p_bf16) return IOMO_ERR_INVALID;
+    if (d->L == 0 || d->rows == 0 || d->heads == 0 || d->planes == 0) return IOMO_ERR_INVALID;
+    const iomo_stage_layout* sl = &d->scores_layout;
+    const iomo_stage_layout* pl = &d->probability_layout;
+    if (pl->rows < d->rows || pl->columns < d->L) return IOMO_ERR_INVALID;
+    for (uint64_t plane = 0; plane < d->planes; ++plane)
+    for (uint64_t head = 0; head < d->heads; ++head)
+    for (uint64_t row = 0; row < pl->rows; ++row) {
+        uint16_t* prow = d->p_bf16;
+        if (row >= d->rows) {
+            /* physical rows past the logical extent are canonical +0
+             * (src/rocm/sdpa_softmax.hpp:24-27) */
+            for (uint64_t t = 0; t < pl->columns; ++t)
+                prow[stage_offset(pl, plane, head, row, t)] = 0;
+            continue;
+        }
+        const uint64_t reach = d->a + row + 1;
+        const uint64_t visible = reach < d->L ? reach : d->L;
+        int has_nan = 0, all_ninf = 1;
+        uint64_t pinf = 0;
+        for (uint64_t t = 0; t < visible; ++t) {
+            const volatile float s =
+                    d->scores[stage_offset(sl, plane, head, row, t)] * d->scale;
+            has_nan = has_nan || isnan(s);
+            pinf += (s == INFINITY) ? 1 : 0;
+            all_ninf = all_ninf && isinf(s) && signbit(s);
+        }
+        if (has_nan || all_ninf) {
+            for (uint64_t t = 0; t < pl->columns; ++t)
+                prow[stage_offset(pl, plane, head, row, t)] =
+                        t < visible ? 0x7FC0u : 0;
+            continue;
+        }
+        if (pinf != 0) {
+            const volatile float p = 1.0f / (float)pinf;
+            for (uint64_t t = 0; t < pl->columns; ++t) {
+                uint16_t e = 0;
+                if (t < visible) {
+                    const volatile float s =
+                            d->scores[stage_offset(sl, plane, head, row, t)] * d->scale;
+                    e = iomo_encode_bf16(s == INFINITY ? p : 0.0f);
+                }
+                prow[stage_offset(pl, plane, head, row, t)] = e;
+            }
+            continue;
+        }
+        float maximum = -INFINITY;
+        for (uint64_t t = 0; t < visible; ++t) {
+            const volatile float s =
+                    d->scores[stage_offset(sl, plane, head, row, t)] * d->scale;
+            if (s > maximum) maximum = s;
+        }
+        volatile float sum = 0.0f;
+        for (uint64_t t = 0; t < visible; ++t) {
+            const volatile float s =
+                    d->scores[stage_offset(sl, plane, head, row, t)] * d->scale;
+            if (isinf(s) && signbit(s)) continue;
+            const volatile float shifted = s - maximum;
+            const volatile float e = expf(shifted);
+            sum = sum + e;
+        }
+        for (uint64_t t = 0; t < pl->columns; ++t) {
+            uint16_t enc = 0;
+            if (t < visible) {
+                const volatile float s =
+                        d->scores[stage_offset(sl, plane, head, row, t)] * d->scale;
+                if (!(isinf(s) && signbit(s))) {
+                    const volatile float shifted = s - maximum;
+                    const volatile float e = expf(shifted);
+                    const volatile float p = e / sum;
+                    enc = iomo_encode_bf16(p);
+                }
+            }
+            prow[stage_offset(pl, plane, head, row, t)] = enc;
+        }
+    }
+    return IOMO_OK;
+}

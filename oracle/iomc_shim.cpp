@@ -1,0 +1,342 @@
+// iomc_shim.cpp — a plain-C handle API over IOM's public C++ interface
+// (iom::Device / iom::Tensor / iom::TensorView / iom::DeviceOps,
+// include/iom/{device,tensor,iom}.hpp), so that Python tests can drive a
+// backend exactly the way the reference's own conformance drivers do:
+// create_tensor -> copy_from_host -> queue->add/mul/sub/copy/rmsnorm/silu ->
+// wait -> copy_to_host.
+//
+// TEST INFRASTRUCTURE.  The file is compiled twice, against the reference's
+// headers where they lie:
+//   * with the reference CPU backend's own sources -> oracle/_ref/libiom_ref.so
+//     (factory: iom::make_cpu_device, include/iom/cpu/device.hpp:19-20);
+//   * -DIOMC_WITH_MI355X with this repository's backend ->
+//     iom_amd/lib/libiom_mi355x_shim.so (factory: iom::make_rocm_device,
+//     include/iom/rocm/device.hpp:22-24).
+// It holds no arithmetic of its own.
+#include <cstddef>
+#include <cstdint>
+#include <cstring>
+#include <exception>
+#include <memory>
+#include <new>
+#include <span>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "iom/alloc.hpp"
+#include "iom/cpu/device.hpp"
+#include "iom/device.hpp"
+#include "iom/iom.hpp"
+#include "iom/tensor.hpp"
+#include "src/iom_internal.hpp"  // iom::detail::UnsupportedOperation
+#ifdef IOMC_WITH_MI355X
+#include "iom/rocm/device.hpp"
+#endif
+
+namespace {
+
+thread_local std::string g_error;
+
+// Error classes mirror the negative OID mapping of src/device_ops.cpp:422-439.
+int classify(const std::exception_ptr& failure) {
+    try {
+        std::rethrow_exception(failure);
+    } catch (const iom::detail::UnsupportedOperation& e) {
+        g_error = std::string("unsupported: ") + e.what();
+        return -2;
+    } catch (const std::bad_alloc& e) {
+        g_error = std::string("bad_alloc: ") + e.what();
+        return -4;
+    } catch (const std::overflow_error& e) {
+        g_error = std::string("overflow_error: ") + e.what();
+        return -3;
+    } catch (const std::invalid_argument& e) {
+        g_error = std::string("invalid_argument: ") + e.what();
+        return -1;
+    } catch (const std::out_of_range& e) {
+        g_error = std::string("out_of_range: ") + e.what();
+        return -7;
+    } catch (const std::exception& e) {
+        g_error = std::string("exception: ") + e.what();
+        return -5;
+    } catch (...) {
+        g_error = "unknown failure";
+        return -6;
+    }
+}
+
+class HeapAllocator final : public iom::Allocator {
+public:
+    void* alloc(std::size_t size) override {
+        return ::operator new(size, std::align_val_t(64));
+    }
+    void free(void* buffer) override {
+        ::operator delete(buffer, std::align_val_t(64));
+    }
+    void reset() override {}
+};
+
+}  // namespace
+
+struct iomc_device {
+    HeapAllocator allocator;
+    std::unique_ptr<iom::Device> device;
+};
+struct iomc_tensor {
+    std::unique_ptr<iom::Tensor> tensor;
+};
+struct iomc_view {
+    iom::TensorView view;
+};
+struct iomc_queue {
+    std::unique_ptr<iom::DeviceOps> ops;
+};
+
+namespace {
+
+template <typename F>
+auto guarded(F&& body, decltype(body()) fallback) -> decltype(body()) {
+    try {
+        return body();
+    } catch (...) {
+        (void)classify(std::current_exception());
+        return fallback;
+    }
+}
+
+template <typename F>
+int guarded_status(F&& body) {
+    try {
+        body();
+        return 0;
+    } catch (...) {
+        return classify(std::current_exception());
+    }
+}
+
+// Host transfers on accelerator backends need a caller workspace of the
+// queried size (src/rocm/device_tensor.cpp:136-143); the CPU backend reports
+// {0,1}.
+std::unique_ptr<iom::RawWorkspace> transfer_workspace(
+        iom::Device& device, const iom::WorkspaceRequirements& need) {
+    if (need.bytes == 0) return nullptr;
+    return device.create_workspace(need.bytes);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* iomc_last_error() { return g_error.c_str(); }
+
+iomc_device* iomc_cpu_device_create(std::size_t max_in_flight) {
+    return guarded([&]() -> iomc_device* {
+        auto holder = std::make_unique<iomc_device>();
+        holder->device = iom::make_cpu_device(
+                holder->allocator, iom::QueueConfig{max_in_flight});
+        return holder.release();
+    }, nullptr);
+}
+
+#ifdef IOMC_WITH_MI355X
+iomc_device* iomc_mi355x_device_create(
+        std::uint32_t ordinal, std::size_t arena_bytes,
+        std::size_t max_in_flight) {
+    return guarded([&]() -> iomc_device* {
+        auto holder = std::make_unique<iomc_device>();
+        holder->device = iom::make_rocm_device(
+                ordinal, iom::DeviceMemoryConfig{arena_bytes},
+                iom::QueueConfig{max_in_flight});
+        return holder.release();
+    }, nullptr);
+}
+#endif
+
+void iomc_device_destroy(iomc_device* device) { delete device; }
+
+int iomc_device_backend_kind(const iomc_device* device) {
+    return static_cast<int>(device->device->backend_kind());
+}
+
+iomc_tensor* iomc_tensor_create(
+        iomc_device* device, int dtype, std::uint32_t rank,
+        const std::uint64_t* dims) {
+    return guarded([&]() -> iomc_tensor* {
+        std::vector<std::size_t> shape(dims, dims + rank);
+        iom::TensorSpec spec{
+                iom::TensorShape{std::move(shape)},
+                static_cast<iom::DataType>(dtype)};
+        auto holder = std::make_unique<iomc_tensor>();
+        holder->tensor = device->device->create_tensor(spec);
+        return holder.release();
+    }, nullptr);
+}
+
+void iomc_tensor_destroy(iomc_tensor* tensor) { delete tensor; }
+
+iomc_view* iomc_tensor_view(iomc_tensor* tensor) {
+    return guarded([&]() -> iomc_view* {
+        return new iomc_view{tensor->tensor->view()};
+    }, nullptr);
+}
+
+void iomc_view_destroy(iomc_view* view) { delete view; }
+
+iomc_view* iomc_view_slice(
+        const iomc_view* view, std::size_t dim, std::size_t first,
+        std::size_t count, std::size_t step) {
+    return guarded([&]() -> iomc_view* {
+        return new iomc_view{view->view.slice(dim, first, count, step)};
+    }, nullptr);
+}
+
+iomc_view* iomc_view_select(
+        const iomc_view* view, std::size_t dim, std::size_t index) {
+    return guarded([&]() -> iomc_view* {
+        return new iomc_view{view->view.select(dim, index)};
+    }, nullptr);
+}
+
+iomc_view* iomc_view_permute(
+        const iomc_view* view, const std::uint64_t* order, std::size_t count) {
+    return guarded([&]() -> iomc_view* {
+        std::vector<std::size_t> axes(order, order + count);
+        return new iomc_view{view->view.permute(axes)};
+    }, nullptr);
+}
+
+iomc_view* iomc_view_reshape_leading(
+        const iomc_view* view, const std::uint64_t* dims, std::size_t count) {
+    return guarded([&]() -> iomc_view* {
+        std::vector<std::size_t> leading(dims, dims + count);
+        return new iomc_view{view->view.reshape_leading(leading)};
+    }, nullptr);
+}
+
+std::uint32_t iomc_view_rank(const iomc_view* view) {
+    return static_cast<std::uint32_t>(view->view.spec().shape.rank());
+}
+
+void iomc_view_describe(
+        const iomc_view* view, std::uint64_t* dims, std::uint64_t* plane_offset,
+        std::uint64_t* plane_strides) {
+    const auto shape = view->view.spec().shape.dimensions();
+    for (std::size_t i = 0; i < shape.size(); ++i) dims[i] = shape[i];
+    *plane_offset = view->view.plane_offset();
+    const auto strides = view->view.plane_strides();
+    for (std::size_t i = 0; i < strides.size(); ++i) plane_strides[i] = strides[i];
+}
+
+std::uint64_t iomc_view_logical_nbytes(const iomc_view* view) {
+    return guarded([&]() -> std::uint64_t {
+        return view->view.spec().logical_nbytes();
+    }, 0);
+}
+
+std::uint64_t iomc_view_tiled_nbytes(const iomc_view* view) {
+    return guarded([&]() -> std::uint64_t {
+        return view->view.spec().tiled_storage_nbytes();
+    }, 0);
+}
+
+// Raw owner storage: host memory on the CPU backend, device memory on an
+// accelerator backend (include/iom/tensor.hpp:290-291).
+void* iomc_view_native_handle(iomc_view* view) {
+    return view->view.native_handle();
+}
+
+int iomc_view_from_host(
+        iomc_device* device, iomc_view* view, const void* bytes,
+        std::size_t nbytes) {
+    return guarded_status([&] {
+        auto workspace = transfer_workspace(
+                *device->device,
+                view->view.copy_from_host_workspace_requirements());
+        const std::span<const std::byte> source(
+                static_cast<const std::byte*>(bytes), nbytes);
+        if (workspace) view->view.copy_from_host(source, workspace->view());
+        else view->view.copy_from_host(source);
+    });
+}
+
+int iomc_view_to_host(
+        iomc_device* device, const iomc_view* view, void* bytes,
+        std::size_t nbytes) {
+    return guarded_status([&] {
+        auto workspace = transfer_workspace(
+                *device->device,
+                view->view.copy_to_host_workspace_requirements());
+        const std::span<std::byte> destination(
+                static_cast<std::byte*>(bytes), nbytes);
+        if (workspace) view->view.copy_to_host(destination, workspace->view());
+        else view->view.copy_to_host(destination);
+    });
+}
+
+iomc_queue* iomc_queue_create(iomc_device* device) {
+    return guarded([&]() -> iomc_queue* {
+        auto holder = std::make_unique<iomc_queue>();
+        holder->ops = device->device->create_ops();
+        return holder.release();
+    }, nullptr);
+}
+
+void iomc_queue_destroy(iomc_queue* queue) { delete queue; }
+
+// op: 0 add, 1 mul, 2 sub, 3 div (order of scalar_binary_codec.hpp:9).
+std::int64_t iomc_binary(
+        iomc_queue* queue, int op, const iomc_view* lhs, const iomc_view* rhs,
+        iomc_view* out) {
+    switch (op) {
+        case 0: return queue->ops->add(lhs->view, rhs->view, out->view);
+        case 1: return queue->ops->mul(lhs->view, rhs->view, out->view);
+        case 2: return queue->ops->sub(lhs->view, rhs->view, out->view);
+        case 3: return queue->ops->div(lhs->view, rhs->view, out->view);
+        default: return -1;
+    }
+}
+
+std::int64_t iomc_copy(
+        iomc_queue* queue, const iomc_view* source, iomc_view* destination) {
+    return queue->ops->copy(source->view, destination->view);
+}
+
+std::int64_t iomc_rmsnorm(
+        iomc_queue* queue, const iomc_view* x, const iomc_view* scale,
+        iomc_view* out, float eps) {
+    return queue->ops->rmsnorm(x->view, scale->view, out->view, eps);
+}
+
+std::int64_t iomc_silu(iomc_queue* queue, const iomc_view* x, iomc_view* y) {
+    return queue->ops->silu(x->view, y->view);
+}
+
+// Full attention through the public facade; the softmax stage has no public
+// entry of its own (docs/BACKEND_CONTRACT/scaled-dot-product-attention.md:9-10).
+std::int64_t iomc_sdpa(
+        iomc_device* device, iomc_queue* queue, const iomc_view* q,
+        const iomc_view* k, const iomc_view* v, iomc_view* out, std::size_t a,
+        std::size_t L) {
+    try {
+        const iom::WorkspaceRequirements need =
+                queue->ops->sdpa_workspace_requirements(
+                        q->view, k->view, v->view, out->view, a, L);
+        if (need.bytes == 0) {
+            return queue->ops->sdpa(q->view, k->view, v->view, out->view, a, L);
+        }
+        auto workspace = device->device->create_workspace(need.bytes);
+        const iom::oid token = queue->ops->sdpa(
+                q->view, k->view, v->view, out->view, a, L, workspace->view());
+        if (token > 0) queue->ops->wait(token);
+        return token;
+    } catch (...) {
+        return classify(std::current_exception());
+    }
+}
+
+int iomc_wait(iomc_queue* queue, std::int64_t token) {
+    return guarded_status([&] { queue->ops->wait(token); });
+}
+
+}  // extern "C"

@@ -1,0 +1,512 @@
+"""ctypes bindings for the test-only checkers.
+
+TEST INFRASTRUCTURE: only tests, the smoke check and the benchmark's
+CPU-baseline leg may import this module.  Two libraries are wrapped:
+
+* ``libiom_oracle.so`` – this repository's C restatement of the reference CPU
+  backend (``iom_oracle.h``).
+* ``_ref/libiom_ref.so`` – the reference's own CPU backend compiled from its
+  sources (``make ref``), driven through the ``iomc_*`` handle API of
+  ``iomc_shim.cpp``.  Present only where it has been built.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional, Sequence
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+DT_I32, DT_U32, DT_BF16, DT_F32 = 9, 10, 20, 21
+OP_ADD, OP_MUL, OP_SUB = 0, 1, 2
+TILE = 16
+
+NP_OF = {DT_I32: np.uint32, DT_U32: np.uint32, DT_BF16: np.uint16, DT_F32: np.uint32}
+"""Raw-bit numpy carrier of every leaf (all arithmetic is on bit patterns)."""
+
+
+def leaf_bytes(dtype: int) -> int:
+    return 2 if dtype == DT_BF16 else 4
+
+
+class View(C.Structure):
+    _fields_ = [
+        ("base", C.c_void_p),
+        ("rank", C.c_uint32),
+        ("dims", C.c_uint64 * 8),
+        ("plane_offset", C.c_uint64),
+        ("plane_strides", C.c_uint64 * 6),
+    ]
+
+
+class StageLayout(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in (
+        "plane_offset", "plane_stride", "head_stride", "row_stride",
+        "column_stride", "rows", "columns")]
+
+
+class SoftmaxDesc(C.Structure):
+    _fields_ = [
+        ("planes", C.c_uint64), ("heads", C.c_uint64), ("rows", C.c_uint64),
+        ("a", C.c_uint64), ("L", C.c_uint64), ("scale", C.c_float),
+        ("scores", C.c_void_p), ("p_bf16", C.c_void_p),
+        ("scores_layout", StageLayout), ("probability_layout", StageLayout),
+    ]
+
+
+def _load(path: str) -> C.CDLL:
+    if not os.path.exists(path):
+        raise FileNotFoundError(
+            f"{path} is not built; run `make -C {HERE}` (or __graft_entry__.build())")
+    return C.CDLL(path)
+
+
+_lib: Optional[C.CDLL] = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        l = _load(os.path.join(HERE, "libiom_oracle.so"))
+        VP = C.POINTER(View)
+        l.iomo_plane_slot.restype = C.c_uint64
+        l.iomo_plane_slot.argtypes = [C.c_uint64] * 5
+        l.iomo_plane_elems.restype = C.c_uint64
+        l.iomo_plane_elems.argtypes = [C.c_uint64] * 2
+        l.iomo_scalar_binary.restype = C.c_uint64
+        l.iomo_scalar_binary.argtypes = [C.c_int, C.c_int, C.c_uint64, C.c_uint64]
+        l.iomo_scalar_binary_ieee.restype = C.c_uint64
+        l.iomo_scalar_binary_ieee.argtypes = [C.c_int, C.c_int, C.c_uint64, C.c_uint64]
+        l.iomo_scalar_silu.restype = C.c_uint64
+        l.iomo_scalar_silu.argtypes = [C.c_int, C.c_uint64]
+        l.iomo_encode_bf16.restype = C.c_uint16
+        l.iomo_encode_bf16.argtypes = [C.c_float]
+        l.iomo_binary.argtypes = [C.c_int, C.c_int, VP, VP, VP, C.c_int]
+        l.iomo_rmsnorm.argtypes = [C.c_int, VP, VP, VP, C.c_float]
+        l.iomo_silu.argtypes = [C.c_int, VP, VP]
+        l.iomo_copy.argtypes = [C.c_int, VP, VP]
+        l.iomo_scatter.argtypes = [C.c_int, VP, C.c_void_p]
+        l.iomo_gather.argtypes = [C.c_int, VP, C.c_void_p]
+        l.iomo_softmax.argtypes = [C.POINTER(SoftmaxDesc)]
+        _lib = l
+    return _lib
+
+
+# --------------------------------------------------------------------------
+# Host-side tensors in tiled storage (numpy), with leading-axis views.
+# --------------------------------------------------------------------------
+
+def padded(n: int) -> int:
+    return (n + TILE - 1) // TILE * TILE
+
+
+def plane_elems(rows: int, cols: int) -> int:
+    return padded(rows) * padded(cols)
+
+
+class HostTensor:
+    """Owner storage in the standard 16x16 tiled layout, held in numpy.
+
+    Mirrors ``iom::Tensor`` + ``iom::TensorView`` (include/iom/tensor.hpp:262-411)
+    as far as the checkers need: a full view plus slice/select/permute/
+    reshape_leading returning new views over the same storage.
+    """
+
+    def __init__(self, dtype: int, dims: Sequence[int], fill: Optional[int] = None):
+        self.dtype = dtype
+        self.dims = tuple(int(d) for d in dims)
+        assert 2 <= len(self.dims) <= 8 and all(d > 0 for d in self.dims)
+        planes = int(np.prod(self.dims[:-2], dtype=np.int64)) if len(self.dims) > 2 else 1
+        self.planes = planes
+        n = planes * plane_elems(self.dims[-2], self.dims[-1])
+        self.storage = np.zeros(n, dtype=NP_OF[dtype])
+        if fill is not None:
+            self.storage.view(np.uint8)[:] = fill
+
+    def view(self) -> "HostView":
+        lead = self.dims[:-2]
+        strides = []
+        s = 1
+        for d in reversed(lead):
+            strides.append(s)
+            s *= d
+        return HostView(self, self.dims, 0, tuple(reversed(strides)))
+
+
+class HostView:
+    def __init__(self, owner: HostTensor, dims, plane_offset: int, plane_strides):
+        self.owner = owner
+        self.dims = tuple(int(d) for d in dims)
+        self.plane_offset = int(plane_offset)
+        self.plane_strides = tuple(int(s) for s in plane_strides)
+
+    @property
+    def dtype(self) -> int:
+        return self.owner.dtype
+
+    # src/tensor_view.cpp:99-256
+    def slice(self, dim, first, count, step=1):
+        lead = list(self.dims[:-2])
+        assert dim < len(lead) and count > 0 and step > 0
+        assert first + (count - 1) * step < lead[dim]
+        strides = list(self.plane_strides)
+        off = self.plane_offset + first * strides[dim]
+        lead[dim] = count
+        strides[dim] *= step
+        return HostView(self.owner, tuple(lead) + self.dims[-2:], off, strides)
+
+    def select(self, dim, index):
+        lead = list(self.dims[:-2])
+        assert dim < len(lead) and index < lead[dim]
+        strides = list(self.plane_strides)
+        off = self.plane_offset + index * strides[dim]
+        del lead[dim]
+        del strides[dim]
+        return HostView(self.owner, tuple(lead) + self.dims[-2:], off, strides)
+
+    def permute(self, order):
+        lead = self.dims[:-2]
+        assert sorted(order) == list(range(len(lead)))
+        return HostView(self.owner, tuple(lead[i] for i in order) + self.dims[-2:],
+                        self.plane_offset, [self.plane_strides[i] for i in order])
+
+    def reshape_leading(self, new_lead):
+        lead = self.dims[:-2]
+        assert int(np.prod(new_lead, dtype=np.int64)) == int(np.prod(lead, dtype=np.int64))
+        expected = 1
+        for d, s in zip(reversed(lead), reversed(self.plane_strides)):
+            if d > 1:
+                assert s == expected, "reshape requires a contiguous view"
+                expected *= d
+        strides = []
+        s = 1
+        for d in reversed(new_lead):
+            strides.append(s)
+            s *= d
+        return HostView(self.owner, tuple(new_lead) + self.dims[-2:], self.plane_offset,
+                        tuple(reversed(strides)))
+
+    def cview(self, base: Optional[int] = None) -> View:
+        v = View()
+        v.base = self.owner.storage.ctypes.data if base is None else base
+        v.rank = len(self.dims)
+        for i, d in enumerate(self.dims):
+            v.dims[i] = d
+        v.plane_offset = self.plane_offset
+        for i, s in enumerate(self.plane_strides):
+            v.plane_strides[i] = s
+        return v
+
+    @property
+    def logical_count(self) -> int:
+        return int(np.prod(self.dims, dtype=np.int64))
+
+    def from_logical(self, arr: np.ndarray) -> None:
+        """region_from_host: raw-bit array of the view's logical shape."""
+        arr = np.ascontiguousarray(arr, dtype=NP_OF[self.dtype]).reshape(-1)
+        assert arr.size == self.logical_count
+        cv = self.cview()
+        rc = lib().iomo_scatter(self.dtype, C.byref(cv), arr.ctypes.data)
+        assert rc == 0, rc
+
+    def to_logical(self) -> np.ndarray:
+        out = np.empty(self.logical_count, dtype=NP_OF[self.dtype])
+        cv = self.cview()
+        rc = lib().iomo_gather(self.dtype, C.byref(cv), out.ctypes.data)
+        assert rc == 0, rc
+        return out.reshape(self.dims)
+
+
+def tile_plane(logical: np.ndarray, fill=0) -> np.ndarray:
+    """Closed-form numpy tiling of [..., R, C] -> flat tiled storage (independent of
+    the C scatter): pad to 16, split into tiles, order plane/tile-row/tile-col/r/c."""
+    *lead, R, Cc = logical.shape
+    PR, PC = padded(R), padded(Cc)
+    buf = np.full(tuple(lead) + (PR, PC), fill, dtype=logical.dtype)
+    buf[..., :R, :Cc] = logical
+    nlead = len(lead)
+    buf = buf.reshape(tuple(lead) + (PR // TILE, TILE, PC // TILE, TILE))
+    axes = tuple(range(nlead)) + (nlead, nlead + 2, nlead + 1, nlead + 3)
+    return np.ascontiguousarray(buf.transpose(axes)).reshape(-1)
+
+
+def untile_plane(flat: np.ndarray, dims) -> np.ndarray:
+    *lead, R, Cc = dims
+    PR, PC = padded(R), padded(Cc)
+    nlead = len(lead)
+    buf = flat.reshape(tuple(lead) + (PR // TILE, PC // TILE, TILE, TILE))
+    axes = tuple(range(nlead)) + (nlead, nlead + 2, nlead + 1, nlead + 3)
+    buf = buf.transpose(axes).reshape(tuple(lead) + (PR, PC))
+    return np.ascontiguousarray(buf[..., :R, :Cc])
+
+
+# -- op wrappers -------------------------------------------------------------
+
+def binary(op: int, lhs: HostView, rhs: HostView, out: HostView, ieee: bool = False) -> int:
+    a, b, o = lhs.cview(), rhs.cview(), out.cview()
+    return lib().iomo_binary(op, out.dtype, C.byref(a), C.byref(b), C.byref(o), int(ieee))
+
+
+def rmsnorm(x: HostView, scale: HostView, out: HostView, eps: float) -> int:
+    a, b, o = x.cview(), scale.cview(), out.cview()
+    return lib().iomo_rmsnorm(out.dtype, C.byref(a), C.byref(b), C.byref(o), eps)
+
+
+def silu(x: HostView, y: HostView) -> int:
+    a, o = x.cview(), y.cview()
+    return lib().iomo_silu(y.dtype, C.byref(a), C.byref(o))
+
+
+def copy(src: HostView, dst: HostView) -> int:
+    a, o = src.cview(), dst.cview()
+    return lib().iomo_copy(dst.dtype, C.byref(a), C.byref(o))
+
+
+def dense_layout(heads: int, rows: int, cols: int) -> StageLayout:
+    l = StageLayout()
+    l.plane_offset = 0
+    l.plane_stride = heads * rows * cols
+    l.head_stride = rows * cols
+    l.row_stride = cols
+    l.column_stride = 1
+    l.rows = rows
+    l.columns = cols
+    return l
+
+
+def softmax(scores: np.ndarray, a: int, L: int, scale: float = 1.0,
+            rows: Optional[int] = None) -> np.ndarray:
+    """scores: float32 [planes, heads, phys_rows, phys_cols] -> uint16 same shape."""
+    scores = np.ascontiguousarray(scores, dtype=np.float32)
+    planes, heads, prow, pcol = scores.shape
+    out = np.full(scores.shape, 0xAAAA, dtype=np.uint16)
+    d = SoftmaxDesc()
+    d.planes, d.heads, d.rows = planes, heads, prow if rows is None else rows
+    d.a, d.L, d.scale = a, L, scale
+    d.scores, d.p_bf16 = scores.ctypes.data, out.ctypes.data
+    d.scores_layout = dense_layout(heads, prow, pcol)
+    d.probability_layout = dense_layout(heads, prow, pcol)
+    rc = lib().iomo_softmax(C.byref(d))
+    assert rc == 0, rc
+    return out
+
+
+# -- bf16 helpers (numpy, independent of the C code) --------------------------
+
+def f32_to_bf16_rne(x: np.ndarray) -> np.ndarray:
+    bits = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    nan = (bits & 0x7FFFFFFF) > 0x7F800000
+    r = ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16).astype(np.uint16)
+    r[nan] = 0x7FC0
+    return r
+
+
+def bf16_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+# --------------------------------------------------------------------------
+# The compiled reference CPU backend (optional).
+# --------------------------------------------------------------------------
+
+REF_PATH = os.path.join(HERE, "_ref", "libiom_ref.so")
+
+
+def ref_available() -> bool:
+    return os.path.exists(REF_PATH)
+
+
+def bind_iomc(l: C.CDLL) -> C.CDLL:
+    """Declare the iomc_* handle API (iomc_shim.cpp) on a loaded library."""
+    P = C.c_void_p
+    U64P = C.POINTER(C.c_uint64)
+    l.iomc_last_error.restype = C.c_char_p
+    l.iomc_cpu_device_create.restype = P
+    l.iomc_cpu_device_create.argtypes = [C.c_size_t]
+    if hasattr(l, "iomc_mi355x_device_create"):
+        l.iomc_mi355x_device_create.restype = P
+        l.iomc_mi355x_device_create.argtypes = [C.c_uint32, C.c_size_t, C.c_size_t]
+    l.iomc_device_destroy.argtypes = [P]
+    l.iomc_device_backend_kind.argtypes = [P]
+    l.iomc_tensor_create.restype = P
+    l.iomc_tensor_create.argtypes = [P, C.c_int, C.c_uint32, U64P]
+    l.iomc_tensor_destroy.argtypes = [P]
+    l.iomc_tensor_view.restype = P
+    l.iomc_tensor_view.argtypes = [P]
+    l.iomc_view_destroy.argtypes = [P]
+    l.iomc_view_slice.restype = P
+    l.iomc_view_slice.argtypes = [P, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t]
+    l.iomc_view_select.restype = P
+    l.iomc_view_select.argtypes = [P, C.c_size_t, C.c_size_t]
+    l.iomc_view_permute.restype = P
+    l.iomc_view_permute.argtypes = [P, U64P, C.c_size_t]
+    l.iomc_view_reshape_leading.restype = P
+    l.iomc_view_reshape_leading.argtypes = [P, U64P, C.c_size_t]
+    l.iomc_view_rank.restype = C.c_uint32
+    l.iomc_view_rank.argtypes = [P]
+    l.iomc_view_describe.argtypes = [P, U64P, U64P, U64P]
+    l.iomc_view_logical_nbytes.restype = C.c_uint64
+    l.iomc_view_logical_nbytes.argtypes = [P]
+    l.iomc_view_tiled_nbytes.restype = C.c_uint64
+    l.iomc_view_tiled_nbytes.argtypes = [P]
+    l.iomc_view_native_handle.restype = P
+    l.iomc_view_native_handle.argtypes = [P]
+    l.iomc_view_from_host.argtypes = [P, P, P, C.c_size_t]
+    l.iomc_view_to_host.argtypes = [P, P, P, C.c_size_t]
+    l.iomc_queue_create.restype = P
+    l.iomc_queue_create.argtypes = [P]
+    l.iomc_queue_destroy.argtypes = [P]
+    l.iomc_binary.restype = C.c_int64
+    l.iomc_binary.argtypes = [P, C.c_int, P, P, P]
+    l.iomc_copy.restype = C.c_int64
+    l.iomc_copy.argtypes = [P, P, P]
+    l.iomc_rmsnorm.restype = C.c_int64
+    l.iomc_rmsnorm.argtypes = [P, P, P, P, C.c_float]
+    l.iomc_silu.restype = C.c_int64
+    l.iomc_silu.argtypes = [P, P, P]
+    l.iomc_sdpa.restype = C.c_int64
+    l.iomc_sdpa.argtypes = [P, P, P, P, P, P, C.c_size_t, C.c_size_t]
+    l.iomc_wait.argtypes = [P, C.c_int64]
+    return l
+
+
+class IomTensor:
+    """One owner created through an iomc device, with view transforms."""
+
+    def __init__(self, backend: "IomBackend", dtype: int, dims: Sequence[int]):
+        self.b = backend
+        self.dtype = dtype
+        self.dims = tuple(int(d) for d in dims)
+        arr = (C.c_uint64 * len(self.dims))(*self.dims)
+        self.handle = backend.l.iomc_tensor_create(backend.dev, dtype, len(self.dims), arr)
+        if not self.handle:
+            raise RuntimeError(backend.error())
+        self.full = IomView(self, backend.l.iomc_tensor_view(self.handle))
+
+    def view(self) -> "IomView":
+        return self.full
+
+    def close(self):
+        if self.handle:
+            self.b.l.iomc_tensor_destroy(self.handle)
+            self.handle = None
+
+
+class IomView:
+    def __init__(self, owner: IomTensor, handle):
+        if not handle:
+            raise RuntimeError(owner.b.error())
+        self.owner = owner
+        self.h = handle
+
+    @property
+    def l(self):
+        return self.owner.b.l
+
+    def slice(self, dim, first, count, step=1):
+        return IomView(self.owner, self.l.iomc_view_slice(self.h, dim, first, count, step))
+
+    def select(self, dim, index):
+        return IomView(self.owner, self.l.iomc_view_select(self.h, dim, index))
+
+    def permute(self, order):
+        arr = (C.c_uint64 * len(order))(*order)
+        return IomView(self.owner, self.l.iomc_view_permute(self.h, arr, len(order)))
+
+    def reshape_leading(self, lead):
+        arr = (C.c_uint64 * len(lead))(*lead)
+        return IomView(self.owner, self.l.iomc_view_reshape_leading(self.h, arr, len(lead)))
+
+    def describe(self):
+        rank = self.l.iomc_view_rank(self.h)
+        dims = (C.c_uint64 * 8)()
+        strides = (C.c_uint64 * 6)()
+        off = C.c_uint64()
+        self.l.iomc_view_describe(self.h, dims, C.byref(off), strides)
+        return tuple(dims[:rank]), off.value, tuple(strides[:rank - 2])
+
+    def from_host(self, arr: np.ndarray):
+        arr = np.ascontiguousarray(arr, dtype=NP_OF[self.owner.dtype])
+        rc = self.l.iomc_view_from_host(self.owner.b.dev, self.h, arr.ctypes.data, arr.nbytes)
+        if rc != 0:
+            raise RuntimeError(self.owner.b.error())
+
+    def to_host(self) -> np.ndarray:
+        dims, _, _ = self.describe()
+        out = np.empty(int(np.prod(dims, dtype=np.int64)), dtype=NP_OF[self.owner.dtype])
+        rc = self.l.iomc_view_to_host(self.owner.b.dev, self.h, out.ctypes.data, out.nbytes)
+        if rc != 0:
+            raise RuntimeError(self.owner.b.error())
+        return out.reshape(dims)
+
+    def raw_storage(self) -> np.ndarray:
+        """Copy of the owner's raw tiled bytes (host-memory backends only)."""
+        n = self.l.iomc_view_tiled_nbytes(self.owner.full.h)
+        p = self.l.iomc_view_native_handle(self.h)
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), shape=(n,)).copy()
+
+
+class IomBackend:
+    """A device + one queue behind the iomc_* handle API."""
+
+    def __init__(self, l: C.CDLL, dev):
+        if not dev:
+            raise RuntimeError(l.iomc_last_error().decode())
+        self.l = l
+        self.dev = dev
+        self.queue = l.iomc_queue_create(dev)
+        if not self.queue:
+            raise RuntimeError(self.error())
+
+    def error(self) -> str:
+        return self.l.iomc_last_error().decode()
+
+    def tensor(self, dtype, dims) -> IomTensor:
+        return IomTensor(self, dtype, dims)
+
+    def wait(self, token: int) -> int:
+        return self.l.iomc_wait(self.queue, token)
+
+    def run(self, token: int) -> int:
+        """Wait when accepted; return the oid (negative = synchronous error)."""
+        if token > 0:
+            rc = self.wait(token)
+            if rc != 0:
+                raise RuntimeError(self.error())
+        return token
+
+    def binary(self, op, lhs: IomView, rhs: IomView, out: IomView) -> int:
+        return self.run(self.l.iomc_binary(self.queue, op, lhs.h, rhs.h, out.h))
+
+    def copy(self, src: IomView, dst: IomView) -> int:
+        return self.run(self.l.iomc_copy(self.queue, src.h, dst.h))
+
+    def rmsnorm(self, x, scale, out, eps) -> int:
+        return self.run(self.l.iomc_rmsnorm(self.queue, x.h, scale.h, out.h, eps))
+
+    def silu(self, x, y) -> int:
+        return self.run(self.l.iomc_silu(self.queue, x.h, y.h))
+
+    def sdpa(self, q, k, v, out, a, L) -> int:
+        return self.run(self.l.iomc_sdpa(self.dev, self.queue, q.h, k.h, v.h, out.h, a, L))
+
+    def close(self):
+        if self.queue:
+            self.l.iomc_queue_destroy(self.queue)
+            self.queue = None
+        if self.dev:
+            self.l.iomc_device_destroy(self.dev)
+            self.dev = None
+
+
+_ref_lib: Optional[C.CDLL] = None
+
+
+def ref_backend(max_in_flight: int = 16) -> IomBackend:
+    """The reference's own CPU backend (make_cpu_device)."""
+    global _ref_lib
+    if _ref_lib is None:
+        _ref_lib = bind_iomc(_load(REF_PATH))
+    return IomBackend(_ref_lib, _ref_lib.iomc_cpu_device_create(max_in_flight))
