@@ -1,0 +1,220 @@
+/*
+ * iomx.h — C ABI of the MI355X (gfx950) tensor-op library, libiomx.so.
+ *
+ * This is the only place where HIP is reached: an IOM backend's C++ host code
+ * (Device / Tensor / DeviceOps subclasses) includes this header and nothing of
+ * hip_runtime.  Each entry point names the interface of the rlewczuk/iom tree
+ * it stands in for (paths relative to that tree).  All functions return 0 on
+ * success, a NEGATIVE iomx_status for a request this library rejects before
+ * any launch, or a POSITIVE HIP error code; iomx_error_string() explains both.
+ *
+ * Tensors are owner storages in IOM's standard layout: leading planes in the
+ * owner's row-major order, each plane 16x16-tiled (tile row, tile column, row
+ * in tile, column in tile), padded to whole tiles.  A view selects planes with
+ * an offset and per-axis strides counted in whole planes
+ * (include/iom/tensor.hpp:262-335).  Padding slots are never written and never
+ * influence a logical result.
+ */
+#ifndef IOMX_H
+#define IOMX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status ------------------------------------------------------------- */
+
+/* Negative values mirror the OID error classes of include/iom/oid.hpp:16-23. */
+typedef enum iomx_status {
+    IOMX_OK = 0,
+    IOMX_ERR_INVALID = -1,     /* malformed request (std::invalid_argument)   */
+    IOMX_ERR_UNSUPPORTED = -2, /* leaf or shape outside this library's scope  */
+    IOMX_ERR_OVERFLOW = -3     /* address arithmetic would overflow           */
+} iomx_status;
+
+const char* iomx_error_string(int status);
+
+/* ---- leaves and operations --------------------------------------------- */
+
+/* Numeric values of iom::DataType (include/iom/tensor.hpp:10-33). */
+enum {
+    IOMX_DT_I32 = 9,
+    IOMX_DT_U32 = 10,
+    IOMX_DT_BF16 = 20,
+    IOMX_DT_F32 = 21
+};
+
+/* Order of BinaryOp in src/shared/scalar_binary_codec.hpp:9. */
+enum { IOMX_OP_ADD = 0, IOMX_OP_MUL = 1, IOMX_OP_SUB = 2 };
+
+/*
+ * One operand: what DeviceOps::BinaryViewSnapshot / CopyViewSnapshot carry
+ * (include/iom/iom.hpp:382-401,480-511) and what the reference uploads as
+ * BinaryMetadata / RmsnormMetadata / SiluMetadata
+ * (src/shared/standard_tiled_add.inl:43-65,
+ *  src/shared/standard_tiled_rmsnorm.inl:73-90, src/shared/gpu_queue.hpp:59-73).
+ * Passed by pointer on the host and by value to the kernels: no descriptor
+ * upload, no allocation.
+ */
+typedef struct iomx_view {
+    void* base;                /* device address of the OWNER storage          */
+    uint32_t rank;             /* 2..8                                         */
+    uint64_t dims[8];          /* the view's logical shape                     */
+    uint64_t plane_offset;     /* first selected owner plane                   */
+    uint64_t plane_strides[6]; /* per leading axis, in owner planes, nonzero   */
+} iomx_view;
+
+/* ---- runtime: device, memory, streams, events --------------------------- */
+
+typedef struct iomx_stream_s* iomx_stream_t; /* NULL = the default stream */
+typedef struct iomx_event_s* iomx_event_t;
+
+typedef struct iomx_device_props {
+    char name[64];     /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+    int compute_units;
+    int wavefront_size;
+    int lds_bytes_per_cu;
+    uint64_t global_bytes;
+} iomx_device_props;
+
+/* Stand in for the hip* calls of src/rocm/driver.hpp:20-81 and
+ * src/rocm/copy.hpp:121-185. */
+int iomx_device_count(int* count);
+int iomx_set_device(int ordinal);
+int iomx_get_device(int* ordinal);
+int iomx_get_device_props(int ordinal, iomx_device_props* props);
+int iomx_device_synchronize(void);
+
+int iomx_malloc(void** ptr, size_t bytes);
+int iomx_free(void* ptr);
+int iomx_host_alloc(void** ptr, size_t bytes); /* pinned, for staging mirrors */
+int iomx_host_free(void* ptr);
+/* src/rocm/device_tensor.cpp:22-41: is this a device allocation of `ordinal`? */
+int iomx_pointer_device(const void* ptr, int* ordinal);
+int iomx_fill_async(void* ptr, uint8_t value, size_t bytes, iomx_stream_t stream);
+int iomx_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int iomx_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int iomx_memcpy_h2d_async(void* dst, const void* src, size_t bytes, iomx_stream_t stream);
+int iomx_memcpy_d2h_async(void* dst, const void* src, size_t bytes, iomx_stream_t stream);
+int iomx_memcpy_d2d_async(void* dst, const void* src, size_t bytes, iomx_stream_t stream);
+
+/* Non-blocking stream at the default priority (src/rocm/copy.hpp:151-185). */
+int iomx_stream_create(iomx_stream_t* stream);
+int iomx_stream_destroy(iomx_stream_t stream);
+int iomx_stream_synchronize(iomx_stream_t stream);
+int iomx_event_create(iomx_event_t* event, int enable_timing);
+int iomx_event_destroy(iomx_event_t event);
+int iomx_event_record(iomx_event_t event, iomx_stream_t stream);
+int iomx_event_synchronize(iomx_event_t event);
+/* *done = 1 when the event has completed, 0 while it is pending. */
+int iomx_event_query(iomx_event_t event, int* done);
+int iomx_event_elapsed_ms(iomx_event_t start, iomx_event_t stop, float* ms);
+
+/* ---- operations ---------------------------------------------------------- */
+
+/*
+ * out = lhs (op) rhs with right-aligned broadcasting.  Replaces
+ * launch_grid_stride_binary / launch_alias_safe_binary
+ * (src/shared/standard_tiled_add.inl:445-464,297-441) behind
+ * DeviceOps::binary_impl (include/iom/iom.hpp:846-956); element rule of
+ * src/shared/scalar_binary_codec.hpp:120-178.  I32/U32 wrap modulo 2^32;
+ * F32 and BF16 are one IEEE operation with one round-to-nearest-even encode,
+ * gradual underflow, and every NaN result stored as the positive canonical
+ * quiet NaN.  An input that shares out's storage must select exactly out's
+ * window (src/device_ops_binary.cpp:152-169); anything else is rejected.
+ */
+int iomx_launch_binary(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs,
+                       const iomx_view* out, iomx_stream_t stream);
+
+/*
+ * out[...,r,:] = (x[...,r,:] / sqrt(mean(x^2)+eps)) * scale[0,:], F32
+ * accumulation.  Replaces standard_tiled_rmsnorm_kernel
+ * (src/shared/standard_tiled_rmsnorm.inl:436-637) behind
+ * DeviceOps::rmsnorm_impl; arithmetic order of src/cpu/queue.cpp:1187-1234:
+ * mean = sum/F, shifted = mean+eps, root = sqrt, inverse = 1/root,
+ * out = (x*inverse)*scale, no fused multiply-add.
+ */
+int iomx_launch_rmsnorm(int dtype, const iomx_view* x, const iomx_view* scale,
+                        const iomx_view* out, float eps, iomx_stream_t stream);
+
+/*
+ * y = x * sigmoid(x) in F32 with the stable two-branch form of
+ * src/shared/scalar_silu.hpp:69-97.  Replaces silu_kernel
+ * (src/rocm/copy.hip:1317-1454) behind DeviceOps::silu_impl.
+ */
+int iomx_launch_silu(int dtype, const iomx_view* x, const iomx_view* y, iomx_stream_t stream);
+
+/*
+ * y = silu(gate) * up with the intermediate rounded to the leaf exactly as the
+ * two-kernel sequence stores it (src/session.cpp:2022-2028 calls silu then
+ * mul).  A private fast path with no counterpart operation in the reference:
+ * its result equals iomx_launch_silu followed by iomx_launch_binary(MUL).
+ */
+int iomx_launch_silu_mul(int dtype, const iomx_view* gate, const iomx_view* up,
+                         const iomx_view* y, iomx_stream_t stream);
+
+/*
+ * Same-spec copy of the selected planes' logical elements.  Replaces
+ * grid_stride_copy_kernel (src/shared/standard_tiled_copy_metadata.inl:241-282)
+ * behind DeviceOps::copy_impl (src/device_ops_copy.cpp:9-52).
+ */
+int iomx_launch_copy(int dtype, const iomx_view* src, const iomx_view* dst, iomx_stream_t stream);
+
+/*
+ * Host-transfer staging: dense logical row-major bytes of the view's shape
+ * (already in device memory) <-> the tiled view.  Replace scatter_plane_kernel /
+ * gather_plane_kernel (src/shared/standard_tiled_copy.inl:286-310) under
+ * Tensor::region_from_host / region_to_host (src/rocm/device_tensor.cpp:145-167).
+ */
+int iomx_launch_scatter(int dtype, const iomx_view* dst, const void* logical, iomx_stream_t stream);
+int iomx_launch_gather(int dtype, const iomx_view* src, void* logical, iomx_stream_t stream);
+
+/* Element strides of one softmax-stage buffer (src/rocm/sdpa_softmax.hpp:14-22). */
+typedef struct iomx_stage_layout {
+    uint64_t plane_offset, plane_stride, head_stride, row_stride, column_stride;
+    uint64_t rows, columns; /* physical region the stage may write */
+} iomx_stage_layout;
+
+/*
+ * The softmax stage of attention: F32 scores in, BF16 probabilities out.
+ * Replaces launch_sdpa_softmax (src/rocm/sdpa_softmax.hpp:36-80,
+ * src/rocm/sdpa_softmax.hip:109-198); arithmetic of src/cpu/sdpa.cpp:214-309.
+ * Row r sees tokens t < min(L, a+r+1).  A row with a NaN or with only -inf
+ * becomes NaN; k scores of +inf share 1/k; otherwise exp(s-max)/sum, rounded to
+ * BF16 once.  Everything outside the visible range, and every physical row or
+ * column beyond the logical extent, is stored as +0.
+ */
+typedef struct iomx_softmax_desc {
+    uint64_t planes, heads, rows;
+    uint64_t a, L;
+    float scale;
+    const float* scores;
+    uint16_t* p_bf16;
+    iomx_stage_layout scores_layout;
+    iomx_stage_layout probability_layout;
+} iomx_softmax_desc;
+
+int iomx_launch_softmax(const iomx_softmax_desc* desc, iomx_stream_t stream);
+
+/* ---- introspection (no counterpart in the reference) --------------------- */
+
+/* Which kernel family the last successful launch on this thread selected
+ * ("binary_planes", "binary_rowvec", "binary_general", ...), and its grid. */
+typedef struct iomx_launch_info {
+    char kernel[48];
+    uint32_t grid, block;
+    uint64_t work_items;
+} iomx_launch_info;
+int iomx_last_launch(iomx_launch_info* info);
+
+/* Compares the hardware BF16 conversion with the software round-to-nearest-
+ * even rule over all 2^32 binary32 encodings; *mismatches receives the count. */
+int iomx_selftest_bf16_convert(uint64_t* mismatches, iomx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* IOMX_H */

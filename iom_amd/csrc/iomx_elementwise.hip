@@ -1,0 +1,505 @@
+// Elementwise operations on tiled, plane-strided, broadcast views:
+// ADD / SUB / MUL over I32, U32, F32, BF16; SiLU and SiLU*up over F32, BF16;
+// same-spec copy.  Two kernel families, selected on the host:
+//
+//   *_planes        every operand either covers whole 16x16-tiled planes
+//                   (FULL) or is a [.,1,F] row vector broadcast over rows
+//                   (ROWVEC); no padding.  Each lane moves 128-bit chunks of a
+//                   contiguous plane range: loads and stores are fully
+//                   coalesced, the plane index math runs on the scalar unit.
+//   *_general       anything else: tile padding, column broadcast, scalars.
+//                   One lane owns one 16-byte piece of one logical row and
+//                   masks the tail.
+//
+// Both read every input of a chunk before storing it, so an input that is the
+// exact alias of the output is safe without staging.
+#include "iomx_common.hpp"
+
+namespace iomx {
+
+enum { MODE_FULL = 0, MODE_ROWVEC = 1 };
+
+// Internal operation codes: the three public binary operations keep their ABI
+// values; the rest are private to this file.
+enum { OP_SILU_MUL = 3, OP_SILU = 4, OP_COPY = 5 };
+
+template <int OP>
+struct Arity { static constexpr int kInputs = (OP == OP_SILU || OP == OP_COPY) ? 1 : 2; };
+
+// x * sigmoid(x) in binary32.  Both branches of the reference form
+// (x >= 0: x / (1 + exp(-x)); x < 0: ((x*t)*t) / (1 + t*t), t = exp(x/2)) need
+// one exponential of a non-positive argument, so one evaluation serves both.
+// -inf maps to -0, +inf to +inf, zeros keep their sign, NaN stays NaN.
+__device__ __forceinline__ float silu_f32(float x) {
+    const bool pos = x >= 0.0f;
+    const float e = expf(pos ? -x : x * 0.5f);
+    const float xe = x * e;
+    float num = pos ? x : xe * e;
+    const float den = 1.0f + (pos ? e : e * e);
+    if (!pos && e == 0.0f) num = -0.0f;  // covers -inf (inf*0) and the flushed tail
+    return num / den;
+}
+
+struct BinaryArgs {
+    const uint8_t* src[2];
+    uint8_t* out;
+    PlaneWalk<3> walk;        // 0 lhs, 1 rhs, 2 out
+    uint64_t plane_bytes[3];  // bytes of one owner plane
+    uint64_t plane_chunks;    // 16-byte chunks of one result plane range
+    uint32_t blocks_per_plane;
+    uint32_t total_blocks;
+    uint32_t tile_cols;       // tile columns of the result (ROWVEC addressing)
+};
+
+struct GeneralArgs {
+    const uint8_t* src[2];
+    uint8_t* out;
+    PlaneWalk<3> walk;
+    uint64_t plane_elems[3];
+    uint64_t rows, cols;          // result matrix
+    uint64_t tile_cols[3];        // per operand
+    uint64_t pieces_per_row;      // 16-byte pieces covering one padded row
+    uint64_t total_pieces;
+    uint32_t brow[2], bcol[2];
+};
+
+template <int DT, int OP>
+__device__ __forceinline__ uint32_t op_word(uint32_t a, uint32_t b) {
+    if constexpr (OP == OP_COPY) {
+        return a;
+    } else if constexpr (OP == OP_SILU) {
+        if constexpr (DT == IOMX_DT_F32) return as_u32(canonical(silu_f32(as_f32(a))));
+        else return pack_bf16(silu_f32(bf16_lo(a)), silu_f32(bf16_hi(a)));
+    } else if constexpr (OP == OP_SILU_MUL) {
+        // the activation is rounded to the leaf before the product, exactly as
+        // the stored intermediate of the two-operation sequence
+        if constexpr (DT == IOMX_DT_F32) {
+            const float act = canonical(silu_f32(as_f32(a)));
+            return as_u32(canonical(act * as_f32(b)));
+        } else {
+            const uint32_t act = pack_bf16(silu_f32(bf16_lo(a)), silu_f32(bf16_hi(a)));
+            return pack_bf16(bf16_lo(act) * bf16_lo(b), bf16_hi(act) * bf16_hi(b));
+        }
+    } else if constexpr (DT == IOMX_DT_I32) {
+        if constexpr (OP == IOMX_OP_ADD) return a + b;
+        else if constexpr (OP == IOMX_OP_MUL) return a * b;
+        else return a - b;
+    } else if constexpr (DT == IOMX_DT_F32) {
+        const float x = as_f32(a), y = as_f32(b);
+        float r;
+        if constexpr (OP == IOMX_OP_ADD) r = x + y;
+        else if constexpr (OP == IOMX_OP_MUL) r = x * y;
+        else r = x - y;
+        return as_u32(canonical(r));
+    } else {
+        // BF16 pair.  The binary32 result of one operation on two BF16 values
+        // is exact or correctly rounded with enough guard bits that the single
+        // narrowing below is the only rounding that matters; binary32
+        // subnormals are kept, so tiny products round once as well.
+        const float xl = bf16_lo(a), yl = bf16_lo(b), xh = bf16_hi(a), yh = bf16_hi(b);
+        float rl, rh;
+        if constexpr (OP == IOMX_OP_ADD) { rl = xl + yl; rh = xh + yh; }
+        else if constexpr (OP == IOMX_OP_MUL) { rl = xl * yl; rh = xh * yh; }
+        else { rl = xl - yl; rh = xh - yh; }
+        return pack_bf16(rl, rh);
+    }
+}
+
+template <int DT, int OP>
+__device__ __forceinline__ u32x4 op_chunk(u32x4 a, u32x4 b) {
+    u32x4 r;
+    r.x = op_word<DT, OP>(a.x, b.x);
+    r.y = op_word<DT, OP>(a.y, b.y);
+    r.z = op_word<DT, OP>(a.z, b.z);
+    r.w = op_word<DT, OP>(a.w, b.w);
+    return r;
+}
+
+template <int DT>
+struct Leaf {
+    static constexpr uint32_t kBytes = (DT == IOMX_DT_BF16) ? 2 : 4;
+    static constexpr uint32_t kPerChunk = 16 / kBytes;          // elements per 16 bytes
+    static constexpr uint32_t kChunksPerRow = kTile / kPerChunk; // per tile row
+    static constexpr uint32_t kChunksPerTile = kTileSlots / kPerChunk;
+};
+
+constexpr int kUnroll = 4;
+constexpr uint32_t kBlock = 256;
+constexpr uint32_t kBlockChunks = kBlock * kUnroll;
+
+template <int DT, int OP, int LM, int RM>
+__global__ __launch_bounds__(kBlock) void elementwise_planes_kernel(const BinaryArgs a) {
+    using L = Leaf<DT>;
+    constexpr int kInputs = Arity<OP>::kInputs;
+    constexpr uint32_t kTilesPerBlock = kBlockChunks / L::kChunksPerTile;
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t w = blockIdx.x; w < a.total_blocks; w += gridDim.x) {
+        uint32_t p = 0, bip = w;
+        if (a.walk.nlead != 0) {
+            p = w / a.blocks_per_plane;
+            bip = w - p * a.blocks_per_plane;
+        }
+        uint64_t plane[3];
+        walk_planes(a.walk, p, plane);
+        const uint8_t* lbase = a.src[0] + plane[0] * a.plane_bytes[0];
+        const uint8_t* rbase = a.src[1] + plane[1] * a.plane_bytes[1];
+        uint8_t* obase = a.out + plane[2] * a.plane_bytes[2];
+        const uint64_t c0 = (uint64_t)bip * kBlockChunks;
+        // first tile column of this block, for row-vector operands
+        uint32_t tcol0 = 0;
+        if constexpr (LM == MODE_ROWVEC || RM == MODE_ROWVEC) {
+            tcol0 = (uint32_t)((c0 / L::kChunksPerTile) % a.tile_cols);
+        }
+        u32x4 va[kUnroll], vb[kUnroll];
+        bool ok[kUnroll];
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) {
+            const uint32_t local = i * kBlock + tid;
+            const uint64_t c = c0 + local;
+            ok[i] = c < a.plane_chunks;
+            uint64_t voff = 0;
+            if constexpr (LM == MODE_ROWVEC || RM == MODE_ROWVEC) {
+                uint32_t tc = tcol0 + local / L::kChunksPerTile;
+                if (a.tile_cols >= kTilesPerBlock) tc -= (tc >= a.tile_cols) ? a.tile_cols : 0;
+                else tc %= a.tile_cols;
+                voff = ((uint64_t)tc * L::kChunksPerTile + (local % L::kChunksPerRow)) * 16;
+            }
+            vb[i] = u32x4{0, 0, 0, 0};
+            if (ok[i]) {
+                va[i] = *reinterpret_cast<const u32x4*>(lbase + (LM == MODE_ROWVEC ? voff : c * 16));
+                if constexpr (kInputs == 2)
+                    vb[i] = *reinterpret_cast<const u32x4*>(rbase + (RM == MODE_ROWVEC ? voff : c * 16));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) {
+            const uint64_t c = c0 + i * kBlock + tid;
+            if (ok[i]) *reinterpret_cast<u32x4*>(obase + c * 16) = op_chunk<DT, OP>(va[i], vb[i]);
+        }
+    }
+}
+
+// One lane = one 16-byte piece (kPerChunk elements) of one logical result row.
+template <int DT, int OP>
+__global__ __launch_bounds__(kBlock) void elementwise_general_kernel(const GeneralArgs a) {
+    using L = Leaf<DT>;
+    constexpr int kInputs = Arity<OP>::kInputs;
+    for (uint64_t g = blockIdx.x * (uint64_t)kBlock + threadIdx.x; g < a.total_pieces;
+         g += (uint64_t)gridDim.x * kBlock) {
+        const uint64_t piece = g % a.pieces_per_row;
+        const uint64_t rowlin = g / a.pieces_per_row;
+        const uint64_t row = rowlin % a.rows;
+        const uint32_t p = (uint32_t)(rowlin / a.rows);
+        const uint64_t col0 = piece * L::kPerChunk;
+        if (col0 >= a.cols) continue;
+        const uint32_t valid = (a.cols - col0) < L::kPerChunk ? (uint32_t)(a.cols - col0) : L::kPerChunk;
+        uint64_t plane[3];
+        walk_planes(a.walk, p, plane);
+        u32x4 v[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}};
+#pragma unroll
+        for (int k = 0; k < kInputs; ++k) {
+            const uint64_t r = a.brow[k] ? 0 : row;
+            const uint64_t c = a.bcol[k] ? 0 : col0;
+            const uint64_t slot = plane[k] * a.plane_elems[k]
+                    + ((r / kTile) * a.tile_cols[k] + c / kTile) * kTileSlots
+                    + (r % kTile) * kTile + c % kTile;
+            if (a.bcol[k]) {
+                uint32_t word;
+                if constexpr (L::kBytes == 2) {
+                    const uint32_t e = *reinterpret_cast<const uint16_t*>(a.src[k] + slot * 2);
+                    word = e | (e << 16);
+                } else {
+                    word = *reinterpret_cast<const uint32_t*>(a.src[k] + slot * 4);
+                }
+                v[k] = u32x4{word, word, word, word};
+            } else {
+                v[k] = *reinterpret_cast<const u32x4*>(a.src[k] + slot * L::kBytes);
+            }
+        }
+        const u32x4 r = op_chunk<DT, OP>(v[0], v[1]);
+        const uint64_t oslot = plane[2] * a.plane_elems[2]
+                + ((row / kTile) * a.tile_cols[2] + col0 / kTile) * kTileSlots
+                + (row % kTile) * kTile + col0 % kTile;
+        uint8_t* dst = a.out + oslot * L::kBytes;
+        if (valid == L::kPerChunk) {
+            *reinterpret_cast<u32x4*>(dst) = r;
+        } else {
+            const uint32_t words[4] = {r.x, r.y, r.z, r.w};
+            for (uint32_t e = 0; e < valid; ++e) {
+                if constexpr (L::kBytes == 2) {
+                    reinterpret_cast<uint16_t*>(dst)[e] =
+                            (uint16_t)(words[e >> 1] >> ((e & 1) * 16));
+                } else {
+                    reinterpret_cast<uint32_t*>(dst)[e] = words[e];
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+
+namespace {
+
+struct Snapshot {
+    uint64_t stride[kMaxLead];
+    bool brow, bcol, broadcasts;
+};
+
+// Result-aligned plane strides with 0 on broadcast axes
+// (src/device_ops_binary.cpp:61-100).
+Snapshot snapshot(const iomx_view& v, const uint64_t* rdims, uint32_t rrank) {
+    Snapshot s = {};
+    const uint32_t offset = rrank - v.rank;
+    s.broadcasts = v.rank != rrank;
+    for (uint32_t axis = 0; axis + 2 < rrank; ++axis) {
+        if (axis < offset) { s.broadcasts = s.broadcasts || rdims[axis] != 1; continue; }
+        const uint32_t src = axis - offset;
+        if (v.dims[src] == 1 && rdims[axis] != 1) { s.broadcasts = true; continue; }
+        s.stride[axis] = v.plane_strides[src];
+    }
+    s.brow = v.dims[v.rank - 2] == 1 && rdims[rrank - 2] != 1;
+    s.bcol = v.dims[v.rank - 1] == 1 && rdims[rrank - 1] != 1;
+    s.broadcasts = s.broadcasts || s.brow || s.bcol;
+    return s;
+}
+
+bool same_window(const iomx_view& a, const iomx_view& b) {
+    if (a.rank != b.rank || a.plane_offset != b.plane_offset) return false;
+    for (uint32_t i = 0; i < a.rank; ++i) if (a.dims[i] != b.dims[i]) return false;
+    for (uint32_t i = 0; i + 2 < a.rank; ++i)
+        if (a.plane_strides[i] != b.plane_strides[i]) return false;
+    return true;
+}
+
+uint32_t grid_for(uint64_t blocks) {
+    // Enough resident waves to cover HBM latency on 256 CUs, few enough that the
+    // scalar plane walk amortises; the kernels loop over the remainder.
+    const uint64_t cap = 256ull * 64;
+    return (uint32_t)(blocks < cap ? blocks : cap);
+}
+
+const char* family(int op, bool planes, bool rowvec) {
+    const bool unary = op == OP_SILU || op == OP_COPY;
+    if (op == OP_SILU) return planes ? "silu_planes" : "silu_general";
+    if (op == OP_COPY) return planes ? "copy_planes" : "copy_general";
+    if (op == OP_SILU_MUL) return planes ? "silu_mul_planes" : "silu_mul_general";
+    (void)unary;
+    if (!planes) return "binary_general";
+    return rowvec ? "binary_rowvec" : "binary_planes";
+}
+
+template <int DT, int OP>
+int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs& ga,
+           hipStream_t s) {
+    if (planes) {
+        const uint32_t grid = grid_for(pa.total_blocks);
+#define IOMX_PLANES(LMV, RMV)                                                              \
+    hipLaunchKernelGGL((elementwise_planes_kernel<DT, OP, LMV, RMV>), dim3(grid),          \
+                       dim3(kBlock), 0, s, pa)
+        if (lm == MODE_FULL && rm == MODE_FULL) IOMX_PLANES(MODE_FULL, MODE_FULL);
+        else if constexpr (OP <= IOMX_OP_SUB) {
+            if (lm == MODE_FULL) IOMX_PLANES(MODE_FULL, MODE_ROWVEC);
+            else IOMX_PLANES(MODE_ROWVEC, MODE_FULL);
+        } else {
+            return IOMX_ERR_INVALID;
+        }
+#undef IOMX_PLANES
+        record_launch(family(OP, true, lm != MODE_FULL || rm != MODE_FULL), grid, kBlock,
+                      pa.total_blocks);
+    } else {
+        const uint64_t blocks = (ga.total_pieces + kBlock - 1) / kBlock;
+        const uint32_t grid = grid_for(blocks);
+        hipLaunchKernelGGL((elementwise_general_kernel<DT, OP>), dim3(grid), dim3(kBlock), 0, s, ga);
+        record_launch(family(OP, false, false), grid, kBlock, ga.total_pieces);
+    }
+    return IOMX_OK;
+}
+
+template <int DT>
+int dispatch(int op, bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs& ga,
+             hipStream_t s) {
+    switch (op) {
+        case IOMX_OP_ADD: return launch<DT, IOMX_OP_ADD>(planes, lm, rm, pa, ga, s);
+        case IOMX_OP_MUL: return launch<DT, IOMX_OP_MUL>(planes, lm, rm, pa, ga, s);
+        case IOMX_OP_SUB: return launch<DT, IOMX_OP_SUB>(planes, lm, rm, pa, ga, s);
+        case OP_COPY: return launch<DT, OP_COPY>(planes, lm, rm, pa, ga, s);
+        default: break;
+    }
+    if constexpr (DT != IOMX_DT_I32) {
+        if (op == OP_SILU) return launch<DT, OP_SILU>(planes, lm, rm, pa, ga, s);
+        if (op == OP_SILU_MUL) return launch<DT, OP_SILU_MUL>(planes, lm, rm, pa, ga, s);
+    }
+    return IOMX_ERR_UNSUPPORTED;
+}
+
+// Shared admission + planning of every elementwise operation.  `rhs` is null
+// for the one-input operations.
+enum AliasPolicy { ALIAS_NONE, ALIAS_EXACT, ALIAS_ANY };
+
+int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iomx_view* out,
+        AliasPolicy alias, iomx_stream_t stream) {
+    const uint32_t bytes = leaf_bytes(dtype);
+    if (!bytes) return IOMX_ERR_UNSUPPORTED;
+    IOMX_TRY(check_view(lhs, bytes));
+    if (rhs) IOMX_TRY(check_view(rhs, bytes));
+    IOMX_TRY(check_view(out, bytes));
+    const bool unary = rhs == nullptr;
+    if (unary) rhs = lhs;
+
+    // right-aligned broadcast and exact output shape (src/device_ops_binary.cpp:121-143)
+    const uint32_t rank = lhs->rank > rhs->rank ? lhs->rank : rhs->rank;
+    uint64_t rdims[8];
+    for (uint32_t i = 0; i < rank; ++i) {
+        const uint64_t l = i < rank - lhs->rank ? 1 : lhs->dims[i - (rank - lhs->rank)];
+        const uint64_t r = i < rank - rhs->rank ? 1 : rhs->dims[i - (rank - rhs->rank)];
+        if (l != r && l != 1 && r != 1) return IOMX_ERR_INVALID;
+        rdims[i] = l > r ? l : r;
+    }
+    if (out->rank != rank) return IOMX_ERR_INVALID;
+    for (uint32_t i = 0; i < rank; ++i) if (out->dims[i] != rdims[i]) return IOMX_ERR_INVALID;
+
+    const iomx_view* v[3] = {lhs, rhs, out};
+    Snapshot snap[3];
+    for (int k = 0; k < 3; ++k) snap[k] = snapshot(*v[k], rdims, rank);
+    // alias rule (src/device_ops_binary.cpp:152-169)
+    for (int k = 0; k < 2; ++k) {
+        if (v[k]->base != out->base || alias == ALIAS_ANY) continue;
+        if (alias == ALIAS_NONE || snap[k].broadcasts || !same_window(*v[k], *out))
+            return IOMX_ERR_INVALID;
+    }
+
+    Matrix m[3];
+    for (int k = 0; k < 3; ++k) m[k] = matrix_of(*v[k]);
+    uint64_t strides[3][kMaxLead];
+    uint64_t offsets[3];
+    for (int k = 0; k < 3; ++k) {
+        std::memcpy(strides[k], snap[k].stride, sizeof(strides[k]));
+        offsets[k] = v[k]->plane_offset;
+    }
+    PlaneWalk<3> walk;
+    IOMX_TRY(build_walk<3>(rank - 2, rdims, strides, offsets, &walk));
+
+    const uint64_t rows = rdims[rank - 2], cols = rdims[rank - 1];
+    const bool no_pad = rows % kTile == 0 && cols % kTile == 0;
+    int mode[2] = {MODE_FULL, MODE_FULL};
+    bool planes_ok = no_pad;
+    for (int k = 0; k < 2 && planes_ok; ++k) {
+        if (!snap[k].brow && !snap[k].bcol) mode[k] = MODE_FULL;
+        else if (snap[k].brow && !snap[k].bcol) mode[k] = MODE_ROWVEC;
+        else planes_ok = false;
+    }
+    if (planes_ok && mode[0] == MODE_ROWVEC && mode[1] == MODE_ROWVEC) planes_ok = false;
+    if (planes_ok && op > IOMX_OP_SUB && (mode[0] != MODE_FULL || mode[1] != MODE_FULL))
+        planes_ok = false;
+
+    BinaryArgs pa = {};
+    GeneralArgs ga = {};
+    if (planes_ok) {
+        pa.src[0] = static_cast<const uint8_t*>(lhs->base);
+        pa.src[1] = static_cast<const uint8_t*>(rhs->base);
+        pa.out = static_cast<uint8_t*>(out->base);
+        pa.walk = walk;
+        for (int k = 0; k < 3; ++k) pa.plane_bytes[k] = m[k].plane_elems * bytes;
+        pa.plane_chunks = m[2].plane_elems * bytes / 16;
+        if (m[2].tile_cols > 0xFFFFFFFFull) return IOMX_ERR_OVERFLOW;
+        pa.tile_cols = (uint32_t)m[2].tile_cols;
+        // A dense selection on every FULL operand folds all planes into one range.
+        bool fold = walk.nlead <= 1;
+        for (int k = 0; k < 3 && fold; ++k) {
+            const bool rowvec = k < 2 && mode[k] == MODE_ROWVEC;
+            if (rowvec) fold = walk.nlead == 0 || walk.stride[k][0] == 0;
+            else fold = walk_is_dense(walk, k);
+        }
+        if (fold && walk.planes > 1) {
+            if (mul_overflows(pa.plane_chunks, walk.planes, &pa.plane_chunks)) return IOMX_ERR_OVERFLOW;
+            pa.src[0] += offsets[0] * pa.plane_bytes[0];
+            pa.src[1] += offsets[1] * pa.plane_bytes[1];
+            pa.out += offsets[2] * pa.plane_bytes[2];
+            for (int k = 0; k < 3; ++k) pa.walk.offset[k] = 0;
+            pa.walk.nlead = 0;
+            pa.walk.planes = 1;
+        }
+        const uint64_t per_plane = (pa.plane_chunks + kBlockChunks - 1) / kBlockChunks;
+        uint64_t total;
+        if (mul_overflows(per_plane, pa.walk.planes, &total) || total > 0xFFFFFFFFull)
+            return IOMX_ERR_OVERFLOW;
+        pa.blocks_per_plane = (uint32_t)per_plane;
+        pa.total_blocks = (uint32_t)total;
+    } else {
+        ga.src[0] = static_cast<const uint8_t*>(lhs->base);
+        ga.src[1] = static_cast<const uint8_t*>(rhs->base);
+        ga.out = static_cast<uint8_t*>(out->base);
+        ga.walk = walk;
+        for (int k = 0; k < 3; ++k) { ga.plane_elems[k] = m[k].plane_elems; ga.tile_cols[k] = m[k].tile_cols; }
+        ga.rows = rows;
+        ga.cols = cols;
+        ga.pieces_per_row = m[2].tile_cols * (kTile * bytes / 16);
+        for (int k = 0; k < 2; ++k) { ga.brow[k] = snap[k].brow; ga.bcol[k] = snap[k].bcol; }
+        uint64_t t;
+        if (mul_overflows(walk.planes, rows, &t)) return IOMX_ERR_OVERFLOW;
+        if (mul_overflows(t, ga.pieces_per_row, &ga.total_pieces)) return IOMX_ERR_OVERFLOW;
+    }
+
+    const hipStream_t s = native(stream);
+    int rc;
+    if (dtype == IOMX_DT_BF16) rc = dispatch<IOMX_DT_BF16>(op, planes_ok, mode[0], mode[1], pa, ga, s);
+    else if (dtype == IOMX_DT_F32) rc = dispatch<IOMX_DT_F32>(op, planes_ok, mode[0], mode[1], pa, ga, s);
+    else rc = dispatch<IOMX_DT_I32>(op, planes_ok, mode[0], mode[1], pa, ga, s);
+    IOMX_TRY(rc);
+    IOMX_HIP(hipGetLastError());
+    return IOMX_OK;
+}
+
+bool same_shape(const iomx_view* a, const iomx_view* b) {
+    if (!a || !b || a->rank != b->rank || a->rank > 8) return false;
+    for (uint32_t i = 0; i < a->rank; ++i) if (a->dims[i] != b->dims[i]) return false;
+    return true;
+}
+
+}  // namespace
+}  // namespace iomx
+
+using namespace iomx;
+
+extern "C" {
+
+int iomx_launch_binary(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs,
+                       const iomx_view* out, iomx_stream_t stream) {
+    if (op < IOMX_OP_ADD || op > IOMX_OP_SUB) return IOMX_ERR_INVALID;
+    if (!rhs) return IOMX_ERR_INVALID;
+    return run(op, dtype, lhs, rhs, out, ALIAS_EXACT, stream);
+}
+
+// Admission of src/device_ops_neural.cpp:363-438: identical shapes, a floating
+// leaf, and an output that shares no storage with the input.
+int iomx_launch_silu(int dtype, const iomx_view* x, const iomx_view* y, iomx_stream_t stream) {
+    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32) return IOMX_ERR_UNSUPPORTED;
+    if (!same_shape(x, y)) return IOMX_ERR_INVALID;
+    return run(OP_SILU, dtype, x, nullptr, y, ALIAS_NONE, stream);
+}
+
+int iomx_launch_silu_mul(int dtype, const iomx_view* gate, const iomx_view* up,
+                         const iomx_view* y, iomx_stream_t stream) {
+    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32) return IOMX_ERR_UNSUPPORTED;
+    if (!same_shape(gate, y) || !same_shape(up, y)) return IOMX_ERR_INVALID;
+    return run(OP_SILU_MUL, dtype, gate, up, y, ALIAS_EXACT, stream);
+}
+
+// src/device_ops_copy.cpp:9-52: identical specs; an identical window is a
+// no-op.  Distinct windows of one owner are accepted as the reference accepts
+// them; windows that overlap partially have no defined result.
+int iomx_launch_copy(int dtype, const iomx_view* src, const iomx_view* dst, iomx_stream_t stream) {
+    if (!leaf_bytes(dtype)) return IOMX_ERR_UNSUPPORTED;
+    if (!same_shape(src, dst)) return IOMX_ERR_INVALID;
+    if (src->base == dst->base && same_window(*src, *dst)) {
+        IOMX_TRY(check_view(src, leaf_bytes(dtype)));
+        record_launch("copy_noop", 0, 0, 0);
+        return IOMX_OK;
+    }
+    return run(OP_COPY, dtype, src, nullptr, dst, ALIAS_ANY, stream);
+}
+
+}  // extern "C"

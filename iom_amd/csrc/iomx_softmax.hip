@@ -1,0 +1,269 @@
+// The softmax stage of attention: binary32 scores in, BF16 probabilities out.
+//
+// One wave owns one row.  In the fast kernel the lane holds the whole row in
+// registers (K 128-bit loads, fully coalesced across the wave), so HBM sees
+// every visible score once and every probability once; the maximum and the sum
+// are wave-wide butterfly reductions.  Rows are independent, so four waves of a
+// workgroup work on four rows without LDS or barriers.
+//
+//   softmax_rows     unit column strides, 16-byte aligned score rows, at most
+//                    4096 physical columns.
+//   softmax_generic  any strides and lengths: three strided passes per row.
+#include "iomx_common.hpp"
+
+namespace iomx {
+
+struct SoftmaxArgs {
+    const float* scores;
+    uint16_t* p;
+    iomx_stage_layout sl, pl;
+    uint64_t rows;       // logical rows per head
+    uint64_t a, L;
+    uint64_t heads;
+    uint64_t total_rows; // planes * heads * pl.rows
+    float scale;
+};
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = v + __shfl_xor(v, m);
+    return v;
+}
+
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = v + __shfl_xor(v, m);
+    return v;
+}
+
+constexpr uint32_t kNegInf = 0xFF800000u;
+constexpr uint32_t kPosInf = 0x7F800000u;
+
+__device__ __forceinline__ uint64_t stage_offset(const iomx_stage_layout& l, uint64_t plane,
+                                                 uint64_t head, uint64_t row) {
+    return l.plane_offset + plane * l.plane_stride + head * l.head_stride + row * l.row_stride;
+}
+
+template <int K>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint64_t wave = (blockIdx.x * (uint64_t)blockDim.x + threadIdx.x) >> 6;
+    const uint64_t waves = ((uint64_t)gridDim.x * blockDim.x) >> 6;
+    for (uint64_t g = wave; g < a.total_rows; g += waves) {
+        const uint64_t r = g % a.pl.rows;
+        const uint64_t ph = g / a.pl.rows;
+        const uint64_t head = ph % a.heads;
+        const uint64_t plane = ph / a.heads;
+        uint16_t* prow = a.p + stage_offset(a.pl, plane, head, r);
+        uint64_t visible = 0;
+        if (r < a.rows) {
+            const uint64_t reach = a.a + r + 1;
+            visible = reach < a.L ? reach : a.L;
+        }
+        const float* srow = a.scores + stage_offset(a.sl, plane, head, r < a.rows ? r : 0);
+
+        float s[K][4];
+        bool has_nan = false;
+        float vmax = as_f32(kNegInf);
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const uint64_t col = ((uint64_t)k * 64 + lane) * 4;
+            float x[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) x[j] = as_f32(kNegInf);
+            if (col + 4 <= visible) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(srow + col);
+                x[0] = as_f32(v.x) * a.scale; x[1] = as_f32(v.y) * a.scale;
+                x[2] = as_f32(v.z) * a.scale; x[3] = as_f32(v.w) * a.scale;
+            } else if (col < visible) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (col + j < visible) x[j] = srow[col + j] * a.scale;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                s[k][j] = x[j];
+                has_nan = has_nan || (x[j] != x[j]);
+                vmax = fmaxf(vmax, x[j]);  // fmaxf skips NaN; NaN rows are decided by has_nan
+            }
+        }
+        const bool row_nan = __any(has_nan);
+        const float m = wave_max(vmax);
+        const bool all_ninf = as_u32(m) == kNegInf;
+        const bool poisoned = row_nan || all_ninf;
+        uint32_t pinf = 0;
+        float inv_share = 0.0f;
+        float sum = 1.0f;
+        if (!poisoned) {
+            if (as_u32(m) == kPosInf) {
+                uint32_t cnt = 0;
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) cnt += as_u32(s[k][j]) == kPosInf ? 1u : 0u;
+                pinf = wave_sum_u32(cnt);
+                inv_share = 1.0f / (float)pinf;
+            } else {
+                float part = 0.0f;
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float e = expf(s[k][j] - m);  // exp(-inf) = 0 for masked and -inf scores
+                        s[k][j] = e;
+                        part = part + e;
+                    }
+                sum = wave_sum(part);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const uint64_t col = ((uint64_t)k * 64 + lane) * 4;
+            if (col >= a.pl.columns) continue;
+            float pr[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v;
+                if (poisoned) v = as_f32(kQuietNanF32);
+                else if (pinf != 0) v = as_u32(s[k][j]) == kPosInf ? inv_share : 0.0f;
+                else v = s[k][j] / sum;
+                pr[j] = (col + j < visible) ? v : 0.0f;
+            }
+            const uint32_t lo = pack_bf16(pr[0], pr[1]);
+            const uint32_t hi = pack_bf16(pr[2], pr[3]);
+            if (col + 4 <= a.pl.columns) {
+                *reinterpret_cast<u32x2*>(prow + col) = u32x2{lo, hi};
+            } else {
+                const uint32_t words[2] = {lo, hi};
+                for (int j = 0; j < 4; ++j)
+                    if (col + j < a.pl.columns)
+                        prow[col + j] = (uint16_t)(words[j >> 1] >> ((j & 1) * 16));
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void softmax_generic_kernel(const SoftmaxArgs a) {
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint64_t wave = (blockIdx.x * (uint64_t)blockDim.x + threadIdx.x) >> 6;
+    const uint64_t waves = ((uint64_t)gridDim.x * blockDim.x) >> 6;
+    for (uint64_t g = wave; g < a.total_rows; g += waves) {
+        const uint64_t r = g % a.pl.rows;
+        const uint64_t ph = g / a.pl.rows;
+        const uint64_t head = ph % a.heads;
+        const uint64_t plane = ph / a.heads;
+        uint16_t* prow = a.p + stage_offset(a.pl, plane, head, r);
+        uint64_t visible = 0;
+        if (r < a.rows) {
+            const uint64_t reach = a.a + r + 1;
+            visible = reach < a.L ? reach : a.L;
+        }
+        const float* srow = a.scores + stage_offset(a.sl, plane, head, r < a.rows ? r : 0);
+        bool has_nan = false;
+        float vmax = as_f32(kNegInf);
+        uint32_t cnt = 0;
+        for (uint64_t t = lane; t < visible; t += 64) {
+            const float x = srow[t * a.sl.column_stride] * a.scale;
+            has_nan = has_nan || (x != x);
+            vmax = fmaxf(vmax, x);
+            cnt += as_u32(x) == kPosInf ? 1u : 0u;
+        }
+        const bool row_nan = __any(has_nan);
+        const float m = wave_max(vmax);
+        const bool poisoned = row_nan || as_u32(m) == kNegInf;
+        const uint32_t pinf = wave_sum_u32(cnt);
+        float sum = 1.0f;
+        if (!poisoned && pinf == 0) {
+            float part = 0.0f;
+            for (uint64_t t = lane; t < visible; t += 64) {
+                const float x = srow[t * a.sl.column_stride] * a.scale;
+                part = part + expf(x - m);
+            }
+            sum = wave_sum(part);
+        }
+        const float inv_share = pinf ? 1.0f / (float)pinf : 0.0f;
+        for (uint64_t t = lane; t < a.pl.columns; t += 64) {
+            float v = 0.0f;
+            if (t < visible) {
+                const float x = srow[t * a.sl.column_stride] * a.scale;
+                if (poisoned) v = as_f32(kQuietNanF32);
+                else if (pinf != 0) v = as_u32(x) == kPosInf ? inv_share : 0.0f;
+                else v = expf(x - m) / sum;
+            }
+            prow[t * a.pl.column_stride] = (uint16_t)(pack_bf16(v, 0.0f) & 0xFFFFu);
+        }
+    }
+}
+
+}  // namespace iomx
+
+using namespace iomx;
+
+// Request checks of validate_sdpa_softmax_request (src/rocm/sdpa_softmax.hpp:64-69).
+extern "C" int iomx_launch_softmax(const iomx_softmax_desc* d, iomx_stream_t stream) {
+    if (!d || !d->scores || !d->p_bf16) return IOMX_ERR_INVALID;
+    if (d->planes == 0 || d->heads == 0 || d->rows == 0 || d->L == 0) return IOMX_ERR_INVALID;
+    const iomx_stage_layout& sl = d->scores_layout;
+    const iomx_stage_layout& pl = d->probability_layout;
+    if (pl.rows < d->rows || pl.columns < d->L) return IOMX_ERR_INVALID;
+    if (sl.rows < d->rows || sl.columns < d->L) return IOMX_ERR_INVALID;
+    if (sl.column_stride == 0 || pl.column_stride == 0) return IOMX_ERR_INVALID;
+    if (!(d->scale == d->scale)) return IOMX_ERR_INVALID;
+    uint64_t total;
+    if (mul_overflows(d->planes, d->heads, &total) || mul_overflows(total, pl.rows, &total))
+        return IOMX_ERR_OVERFLOW;
+    // the largest element offset either buffer can reach must stay addressable
+    const iomx_stage_layout* ls[2] = {&sl, &pl};
+    for (const iomx_stage_layout* l : ls) {
+        uint64_t reach = l->plane_offset, t;
+        if (mul_overflows(d->planes - 1, l->plane_stride, &t) || add_overflows(reach, t, &reach)
+            || mul_overflows(d->heads - 1, l->head_stride, &t) || add_overflows(reach, t, &reach)
+            || mul_overflows(l->rows - 1, l->row_stride, &t) || add_overflows(reach, t, &reach)
+            || mul_overflows(l->columns - 1, l->column_stride, &t) || add_overflows(reach, t, &reach)
+            || reach > (1ull << 44))
+            return IOMX_ERR_OVERFLOW;
+    }
+
+    SoftmaxArgs a = {};
+    a.scores = d->scores;
+    a.p = d->p_bf16;
+    a.sl = sl;
+    a.pl = pl;
+    a.rows = d->rows;
+    a.a = d->a;
+    a.L = d->L;
+    a.heads = d->heads;
+    a.total_rows = total;
+    a.scale = d->scale;
+
+    const bool aligned = sl.column_stride == 1 && pl.column_stride == 1
+            && (reinterpret_cast<uintptr_t>(d->scores) & 15u) == 0
+            && (reinterpret_cast<uintptr_t>(d->p_bf16) & 7u) == 0
+            && sl.plane_offset % 4 == 0 && sl.plane_stride % 4 == 0 && sl.head_stride % 4 == 0
+            && sl.row_stride % 4 == 0
+            && pl.plane_offset % 4 == 0 && pl.plane_stride % 4 == 0 && pl.head_stride % 4 == 0
+            && pl.row_stride % 4 == 0;
+    const uint64_t blocks = (total + 3) / 4;
+    const uint32_t grid = (uint32_t)(blocks < (1u << 20) ? blocks : (1u << 20));
+    const hipStream_t s = native(stream);
+    const uint64_t cols = pl.columns;
+    if (aligned && cols <= 4096) {
+        if (cols <= 256) hipLaunchKernelGGL(softmax_rows_kernel<1>, dim3(grid), dim3(256), 0, s, a);
+        else if (cols <= 512) hipLaunchKernelGGL(softmax_rows_kernel<2>, dim3(grid), dim3(256), 0, s, a);
+        else if (cols <= 1024) hipLaunchKernelGGL(softmax_rows_kernel<4>, dim3(grid), dim3(256), 0, s, a);
+        else if (cols <= 2048) hipLaunchKernelGGL(softmax_rows_kernel<8>, dim3(grid), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(softmax_rows_kernel<16>, dim3(grid), dim3(256), 0, s, a);
+        record_launch("softmax_rows", grid, 256, total);
+    } else {
+        hipLaunchKernelGGL(softmax_generic_kernel, dim3(grid), dim3(256), 0, s, a);
+        record_launch("softmax_generic", grid, 256, total);
+    }
+    IOMX_HIP(hipGetLastError());
+    return IOMX_OK;
+}

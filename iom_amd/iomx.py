@@ -1,0 +1,401 @@
+"""ctypes binding of include/iomx.h, plus small helpers to hold tiled tensors
+in device memory.  Everything here calls the HIP library; nothing computes on
+the host."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional, Sequence
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libiomx.so")
+
+DT_I32, DT_U32, DT_BF16, DT_F32 = 9, 10, 20, 21
+OP_ADD, OP_MUL, OP_SUB = 0, 1, 2
+TILE = 16
+
+NP_OF = {DT_I32: np.uint32, DT_U32: np.uint32, DT_BF16: np.uint16, DT_F32: np.uint32}
+
+# every symbol include/iomx.h declares
+SYMBOLS = [
+    "iomx_error_string", "iomx_device_count", "iomx_set_device", "iomx_get_device",
+    "iomx_get_device_props", "iomx_device_synchronize", "iomx_malloc", "iomx_free",
+    "iomx_host_alloc", "iomx_host_free", "iomx_pointer_device", "iomx_fill_async",
+    "iomx_memcpy_h2d", "iomx_memcpy_d2h", "iomx_memcpy_h2d_async", "iomx_memcpy_d2h_async",
+    "iomx_memcpy_d2d_async", "iomx_stream_create", "iomx_stream_destroy",
+    "iomx_stream_synchronize", "iomx_event_create", "iomx_event_destroy", "iomx_event_record",
+    "iomx_event_synchronize", "iomx_event_query", "iomx_event_elapsed_ms",
+    "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul",
+    "iomx_launch_copy", "iomx_launch_scatter", "iomx_launch_gather", "iomx_launch_softmax",
+    "iomx_last_launch", "iomx_selftest_bf16_convert",
+]
+
+
+class View(C.Structure):
+    _fields_ = [
+        ("base", C.c_void_p), ("rank", C.c_uint32), ("dims", C.c_uint64 * 8),
+        ("plane_offset", C.c_uint64), ("plane_strides", C.c_uint64 * 6),
+    ]
+
+
+class StageLayout(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in (
+        "plane_offset", "plane_stride", "head_stride", "row_stride", "column_stride",
+        "rows", "columns")]
+
+
+class SoftmaxDesc(C.Structure):
+    _fields_ = [
+        ("planes", C.c_uint64), ("heads", C.c_uint64), ("rows", C.c_uint64),
+        ("a", C.c_uint64), ("L", C.c_uint64), ("scale", C.c_float),
+        ("scores", C.c_void_p), ("p_bf16", C.c_void_p),
+        ("scores_layout", StageLayout), ("probability_layout", StageLayout),
+    ]
+
+
+class DeviceProps(C.Structure):
+    _fields_ = [("name", C.c_char * 64), ("compute_units", C.c_int), ("wavefront_size", C.c_int),
+                ("lds_bytes_per_cu", C.c_int), ("global_bytes", C.c_uint64)]
+
+
+class LaunchInfo(C.Structure):
+    _fields_ = [("kernel", C.c_char * 48), ("grid", C.c_uint32), ("block", C.c_uint32),
+                ("work_items", C.c_uint64)]
+
+
+class IomxError(RuntimeError):
+    def __init__(self, status: int, what: str):
+        super().__init__(f"{what}: status {status}: {lib().iomx_error_string(status).decode()}")
+        self.status = status
+
+
+_lib: Optional[C.CDLL] = None
+
+
+def lib() -> C.CDLL:
+    """The HIP library.  Raises when it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m iom_amd.build` "
+                "(__graft_entry__.build()); iom_amd has no CPU fallback")
+        l = C.CDLL(LIB_PATH)
+        VP, P = C.POINTER(View), C.c_void_p
+        l.iomx_error_string.restype = C.c_char_p
+        l.iomx_error_string.argtypes = [C.c_int]
+        l.iomx_device_count.argtypes = [C.POINTER(C.c_int)]
+        l.iomx_set_device.argtypes = [C.c_int]
+        l.iomx_get_device.argtypes = [C.POINTER(C.c_int)]
+        l.iomx_get_device_props.argtypes = [C.c_int, C.POINTER(DeviceProps)]
+        l.iomx_malloc.argtypes = [C.POINTER(P), C.c_size_t]
+        l.iomx_free.argtypes = [P]
+        l.iomx_host_alloc.argtypes = [C.POINTER(P), C.c_size_t]
+        l.iomx_host_free.argtypes = [P]
+        l.iomx_pointer_device.argtypes = [P, C.POINTER(C.c_int)]
+        l.iomx_fill_async.argtypes = [P, C.c_uint8, C.c_size_t, P]
+        for name in ("iomx_memcpy_h2d", "iomx_memcpy_d2h"):
+            getattr(l, name).argtypes = [P, P, C.c_size_t]
+        for name in ("iomx_memcpy_h2d_async", "iomx_memcpy_d2h_async", "iomx_memcpy_d2d_async"):
+            getattr(l, name).argtypes = [P, P, C.c_size_t, P]
+        l.iomx_stream_create.argtypes = [C.POINTER(P)]
+        l.iomx_stream_destroy.argtypes = [P]
+        l.iomx_stream_synchronize.argtypes = [P]
+        l.iomx_event_create.argtypes = [C.POINTER(P), C.c_int]
+        l.iomx_event_destroy.argtypes = [P]
+        l.iomx_event_record.argtypes = [P, P]
+        l.iomx_event_synchronize.argtypes = [P]
+        l.iomx_event_query.argtypes = [P, C.POINTER(C.c_int)]
+        l.iomx_event_elapsed_ms.argtypes = [P, P, C.POINTER(C.c_float)]
+        l.iomx_launch_binary.argtypes = [C.c_int, C.c_int, VP, VP, VP, P]
+        l.iomx_launch_rmsnorm.argtypes = [C.c_int, VP, VP, VP, C.c_float, P]
+        l.iomx_launch_silu.argtypes = [C.c_int, VP, VP, P]
+        l.iomx_launch_silu_mul.argtypes = [C.c_int, VP, VP, VP, P]
+        l.iomx_launch_copy.argtypes = [C.c_int, VP, VP, P]
+        l.iomx_launch_scatter.argtypes = [C.c_int, VP, P, P]
+        l.iomx_launch_gather.argtypes = [C.c_int, VP, P, P]
+        l.iomx_launch_softmax.argtypes = [C.POINTER(SoftmaxDesc), P]
+        l.iomx_last_launch.argtypes = [C.POINTER(LaunchInfo)]
+        l.iomx_selftest_bf16_convert.argtypes = [C.POINTER(C.c_uint64), P]
+        _lib = l
+    return _lib
+
+
+def check(status: int, what: str = "iomx") -> None:
+    if status != 0:
+        raise IomxError(status, what)
+
+
+def device_count() -> int:
+    n = C.c_int(0)
+    status = lib().iomx_device_count(C.byref(n))
+    return n.value if status == 0 else 0
+
+
+def device_props(ordinal: int = 0) -> DeviceProps:
+    p = DeviceProps()
+    check(lib().iomx_get_device_props(ordinal, C.byref(p)), "get_device_props")
+    return p
+
+
+def synchronize() -> None:
+    check(lib().iomx_device_synchronize(), "device_synchronize")
+
+
+def last_launch() -> LaunchInfo:
+    info = LaunchInfo()
+    check(lib().iomx_last_launch(C.byref(info)))
+    return info
+
+
+class Stream:
+    def __init__(self):
+        self.h = C.c_void_p()
+        check(lib().iomx_stream_create(C.byref(self.h)), "stream_create")
+
+    def synchronize(self):
+        check(lib().iomx_stream_synchronize(self.h), "stream_synchronize")
+
+    def close(self):
+        if self.h:
+            lib().iomx_stream_destroy(self.h)
+            self.h = C.c_void_p()
+
+
+class Event:
+    def __init__(self, timing: bool = True):
+        self.h = C.c_void_p()
+        check(lib().iomx_event_create(C.byref(self.h), int(timing)), "event_create")
+
+    def record(self, stream: Optional[Stream] = None):
+        check(lib().iomx_event_record(self.h, stream.h if stream else None), "event_record")
+
+    def synchronize(self):
+        check(lib().iomx_event_synchronize(self.h), "event_synchronize")
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = C.c_float()
+        check(lib().iomx_event_elapsed_ms(self.h, stop.h, C.byref(ms)), "event_elapsed")
+        return ms.value
+
+    def close(self):
+        if self.h:
+            lib().iomx_event_destroy(self.h)
+            self.h = C.c_void_p()
+
+
+class Buffer:
+    """One device allocation."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        self.ptr = C.c_void_p()
+        check(lib().iomx_malloc(C.byref(self.ptr), max(self.nbytes, 16)), "malloc")
+
+    def upload(self, arr: np.ndarray, offset: int = 0):
+        arr = np.ascontiguousarray(arr)
+        assert offset + arr.nbytes <= self.nbytes
+        check(lib().iomx_memcpy_h2d(self.ptr.value + offset, arr.ctypes.data, arr.nbytes), "h2d")
+
+    def download(self, dtype, count: Optional[int] = None, offset: int = 0) -> np.ndarray:
+        itemsize = np.dtype(dtype).itemsize
+        if count is None:
+            count = (self.nbytes - offset) // itemsize
+        out = np.empty(count, dtype=dtype)
+        check(lib().iomx_memcpy_d2h(out.ctypes.data, self.ptr.value + offset, out.nbytes), "d2h")
+        return out
+
+    def fill(self, byte: int, stream: Optional[Stream] = None):
+        check(lib().iomx_fill_async(self.ptr, byte, self.nbytes, stream.h if stream else None), "fill")
+
+    def free(self):
+        if self.ptr:
+            lib().iomx_free(self.ptr)
+            self.ptr = C.c_void_p()
+
+
+def padded(n: int) -> int:
+    return (n + TILE - 1) // TILE * TILE
+
+
+def leaf_bytes(dtype: int) -> int:
+    return 2 if dtype == DT_BF16 else 4
+
+
+class DeviceTensor:
+    """Owner storage in the standard tiled layout, in device memory, with the
+    leading-axis view transforms of iom::TensorView (src/tensor_view.cpp:99-256)."""
+
+    def __init__(self, dtype: int, dims: Sequence[int], fill: Optional[int] = 0):
+        self.dtype = dtype
+        self.dims = tuple(int(d) for d in dims)
+        lead = self.dims[:-2]
+        self.planes = int(np.prod(lead, dtype=np.int64)) if lead else 1
+        self.plane_elems = padded(self.dims[-2]) * padded(self.dims[-1])
+        self.nbytes = self.planes * self.plane_elems * leaf_bytes(dtype)
+        self.buf = Buffer(self.nbytes)
+        if fill is not None:
+            self.buf.fill(fill)
+
+    def view(self) -> "DeviceView":
+        lead = self.dims[:-2]
+        strides, s = [], 1
+        for d in reversed(lead):
+            strides.append(s)
+            s *= d
+        return DeviceView(self, self.dims, 0, tuple(reversed(strides)))
+
+    def raw(self) -> np.ndarray:
+        synchronize()
+        return self.buf.download(NP_OF[self.dtype])
+
+    def upload_raw(self, storage: np.ndarray):
+        assert storage.nbytes == self.nbytes
+        self.buf.upload(storage)
+
+    def free(self):
+        self.buf.free()
+
+
+class DeviceView:
+    def __init__(self, owner: DeviceTensor, dims, plane_offset, plane_strides):
+        self.owner = owner
+        self.dims = tuple(int(d) for d in dims)
+        self.plane_offset = int(plane_offset)
+        self.plane_strides = tuple(int(s) for s in plane_strides)
+
+    @property
+    def dtype(self):
+        return self.owner.dtype
+
+    def slice(self, dim, first, count, step=1):
+        lead = list(self.dims[:-2])
+        assert dim < len(lead) and count > 0 and step > 0 and first + (count - 1) * step < lead[dim]
+        strides = list(self.plane_strides)
+        off = self.plane_offset + first * strides[dim]
+        lead[dim] = count
+        strides[dim] *= step
+        return DeviceView(self.owner, tuple(lead) + self.dims[-2:], off, strides)
+
+    def select(self, dim, index):
+        lead = list(self.dims[:-2])
+        assert dim < len(lead) and index < lead[dim]
+        strides = list(self.plane_strides)
+        off = self.plane_offset + index * strides[dim]
+        del lead[dim]
+        del strides[dim]
+        return DeviceView(self.owner, tuple(lead) + self.dims[-2:], off, strides)
+
+    def permute(self, order):
+        lead = self.dims[:-2]
+        assert sorted(order) == list(range(len(lead)))
+        return DeviceView(self.owner, tuple(lead[i] for i in order) + self.dims[-2:],
+                          self.plane_offset, [self.plane_strides[i] for i in order])
+
+    def reshape_leading(self, new_lead):
+        lead = self.dims[:-2]
+        assert int(np.prod(new_lead, dtype=np.int64)) == int(np.prod(lead, dtype=np.int64))
+        expected = 1
+        for d, s in zip(reversed(lead), reversed(self.plane_strides)):
+            if d > 1:
+                assert s == expected
+                expected *= d
+        strides, s = [], 1
+        for d in reversed(new_lead):
+            strides.append(s)
+            s *= d
+        return DeviceView(self.owner, tuple(new_lead) + self.dims[-2:], self.plane_offset,
+                          tuple(reversed(strides)))
+
+    def cview(self) -> View:
+        v = View()
+        v.base = self.owner.buf.ptr.value
+        v.rank = len(self.dims)
+        for i, d in enumerate(self.dims):
+            v.dims[i] = d
+        v.plane_offset = self.plane_offset
+        for i, s in enumerate(self.plane_strides):
+            v.plane_strides[i] = s
+        return v
+
+    @property
+    def logical_count(self) -> int:
+        return int(np.prod(self.dims, dtype=np.int64))
+
+    def from_host(self, arr: np.ndarray, stream: Optional[Stream] = None):
+        """copy_from_host: logical row-major raw bits -> staging -> scatter kernel."""
+        arr = np.ascontiguousarray(arr, dtype=NP_OF[self.dtype]).reshape(-1)
+        assert arr.size == self.logical_count
+        staging = Buffer(arr.nbytes)
+        try:
+            staging.upload(arr)
+            cv = self.cview()
+            check(lib().iomx_launch_scatter(self.dtype, C.byref(cv), staging.ptr,
+                                            stream.h if stream else None), "scatter")
+            (stream.synchronize() if stream else synchronize())
+        finally:
+            staging.free()
+
+    def to_host(self, stream: Optional[Stream] = None) -> np.ndarray:
+        staging = Buffer(self.logical_count * leaf_bytes(self.dtype))
+        try:
+            cv = self.cview()
+            check(lib().iomx_launch_gather(self.dtype, C.byref(cv), staging.ptr,
+                                           stream.h if stream else None), "gather")
+            (stream.synchronize() if stream else synchronize())
+            return staging.download(NP_OF[self.dtype]).reshape(self.dims)
+        finally:
+            staging.free()
+
+
+def _h(stream):
+    return stream.h if stream else None
+
+
+def binary(op: int, lhs: DeviceView, rhs: DeviceView, out: DeviceView, stream=None) -> int:
+    a, b, o = lhs.cview(), rhs.cview(), out.cview()
+    return lib().iomx_launch_binary(op, out.dtype, C.byref(a), C.byref(b), C.byref(o), _h(stream))
+
+
+def rmsnorm(x: DeviceView, scale: DeviceView, out: DeviceView, eps: float, stream=None) -> int:
+    a, b, o = x.cview(), scale.cview(), out.cview()
+    return lib().iomx_launch_rmsnorm(out.dtype, C.byref(a), C.byref(b), C.byref(o), eps, _h(stream))
+
+
+def silu(x: DeviceView, y: DeviceView, stream=None) -> int:
+    a, o = x.cview(), y.cview()
+    return lib().iomx_launch_silu(y.dtype, C.byref(a), C.byref(o), _h(stream))
+
+
+def silu_mul(gate: DeviceView, up: DeviceView, y: DeviceView, stream=None) -> int:
+    a, b, o = gate.cview(), up.cview(), y.cview()
+    return lib().iomx_launch_silu_mul(y.dtype, C.byref(a), C.byref(b), C.byref(o), _h(stream))
+
+
+def copy(src: DeviceView, dst: DeviceView, stream=None) -> int:
+    a, o = src.cview(), dst.cview()
+    return lib().iomx_launch_copy(dst.dtype, C.byref(a), C.byref(o), _h(stream))
+
+
+def dense_layout(heads: int, rows: int, cols: int) -> StageLayout:
+    l = StageLayout()
+    l.plane_offset, l.plane_stride, l.head_stride = 0, heads * rows * cols, rows * cols
+    l.row_stride, l.column_stride, l.rows, l.columns = cols, 1, rows, cols
+    return l
+
+
+def softmax_desc(scores_ptr: int, p_ptr: int, planes: int, heads: int, prows: int, pcols: int,
+                 a: int, L: int, scale: float = 1.0, rows: Optional[int] = None) -> SoftmaxDesc:
+    d = SoftmaxDesc()
+    d.planes, d.heads, d.rows = planes, heads, prows if rows is None else rows
+    d.a, d.L, d.scale = a, L, scale
+    d.scores, d.p_bf16 = scores_ptr, p_ptr
+    d.scores_layout = dense_layout(heads, prows, pcols)
+    d.probability_layout = dense_layout(heads, prows, pcols)
+    return d
+
+
+def softmax(desc: SoftmaxDesc, stream=None) -> int:
+    return lib().iomx_launch_softmax(C.byref(desc), _h(stream))
