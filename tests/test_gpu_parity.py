@@ -6,8 +6,12 @@ Bars (written where they are applied):
   elementwise I32/F32/BF16      bit-exact, including untouched tile padding
   RMSNorm                       BF16 <= 1 ulp, F32 relative error <= 1e-5,
                                 special classes (NaN / signed zero) exact
-  SiLU                          BF16 <= 1 ulp, F32 <= 4 ulp (the reference's own
-                                ceiling, test/backend/test_scalar_silu.cpp:163-167)
+  SiLU                          BF16 <= 1 ulp against the CPU oracle; F32 <= 4 ulp
+                                against the exact value, the reference's own
+                                ceiling for every backend
+                                (test/backend/backend_conformance_silu.hpp:492-494,
+                                docs/BACKEND_CONTRACT/silu-activation.md:160-162),
+                                and so <= 8 ulp against the CPU oracle
   softmax stage                 <= 1 BF16 ulp, masked entries exactly +0,
                                 special rows exact
 """
@@ -288,6 +292,16 @@ def assert_float_close(got, want, dtype, what, bf16_ulp=1, f32_rel=1e-5, f32_ulp
         assert d.size == 0 or d.max() <= 64
 
 
+def silu_exact_f32_bits(x_bits):
+    """x*sigmoid(x) evaluated in binary64 and rounded once to binary32."""
+    x = x_bits.reshape(-1).view(np.float32).astype(np.float64)
+    with np.errstate(all="ignore"):
+        y = np.where(x < -700.0, x * np.exp(x), x / (1.0 + np.exp(-x)))
+        y = np.where(np.isneginf(x), -0.0, y)
+        y = np.where(x == 0, x, y)
+        return y.astype(np.float32).view(np.uint32)
+
+
 RMS_CASES = [
     ((1, 1), [], "rmsnorm_generic"), ((15, 16), [], "rmsnorm_band"), ((17, 33), [], "rmsnorm_generic"),
     ((16, 31), [], "rmsnorm_generic"), ((3, 5, 130), [], "rmsnorm_generic"),
@@ -385,8 +399,11 @@ def test_silu_against_oracle(dtype, dims, steps, family, kind):
     assert rc == 0, iomx.lib().iomx_error_string(rc)
     assert kernel_name() == family
     assert iomo.silu(hvx, ho.view()) == 0
-    assert_float_close(do.view().to_host(), ho.view().to_logical(), dtype, "silu",
-                       bf16_ulp=1, f32_ulp=4)
+    got = do.view().to_host()
+    assert_float_close(got, ho.view().to_logical(), dtype, "silu", bf16_ulp=1, f32_ulp=8)
+    if dtype == DT_F32:
+        assert_float_close(got, silu_exact_f32_bits(hvx.to_logical()), dtype, "silu vs exact",
+                           f32_ulp=4)
     pad = iomo.tile_plane(np.ones(hvx.dims, ho.storage.dtype)) == 0
     assert np.array_equal(do.raw()[pad], ho.storage[pad])
     dx.free()
@@ -417,7 +434,9 @@ def test_silu_f32_tails_and_specials():
     assert iomx.silu(dx.view(), do.view()) == 0
     assert iomo.silu(hx.view(), ho.view()) == 0
     got, want = do.view().to_host(), ho.view().to_logical()
-    assert_float_close(got, want, DT_F32, "silu tails", f32_ulp=4)
+    assert_float_close(got, want, DT_F32, "silu tails", f32_ulp=8)
+    assert_float_close(got, silu_exact_f32_bits(x.view(np.uint32)), DT_F32, "silu tails vs exact",
+                       f32_ulp=4)
     t = got.reshape(-1)[0]
     assert t & 0x80000000 and t & 0x7FFFFFFF          # -104 keeps a nonzero negative tail
     dx.free()
@@ -572,7 +591,7 @@ def test_reference_cpu_vectors(case):
         x, o = iomx.DeviceTensor(dtype, dims), iomx.DeviceTensor(dtype, dims)
         x.view().from_host(z[key + "_x"])
         assert iomx.silu(x.view(), o.view()) == 0
-        assert_float_close(o.view().to_host(), z[key + "_y"], dtype, key, bf16_ulp=1, f32_ulp=4)
+        assert_float_close(o.view().to_host(), z[key + "_y"], dtype, key, bf16_ulp=1, f32_ulp=8)
         tensors = [x, o]
     for t in tensors:
         t.free()
