@@ -1,0 +1,437 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X tensor-op hot path: achieved HBM GB/s on one GPU.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-detail] [--no-cpu]
+
+One "step" is one launch of the headline workload: broadcast ADD in BF16 of a
+[64,512,2048] activation with a [1,2048] vector (the configuration the metric is
+quoted on).  Inputs are resident in HBM before the timed region; buffers rotate
+over a footprint larger than the 256 MiB Infinity Cache so that every pass comes
+from HBM.  Prints ONE JSON line; `detail` holds the same measurement for every
+other configuration of the hot path, `roofline` the headline kernel against the
+8 TB/s HBM peak, `cpu_baseline` the reference CPU backend (or, where it was not
+built, the CPU restatement) timed on this host on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+import datagen  # noqa: E402  (seeded synthetic inputs, shared with the tests)
+from iom_amd import iomx  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+BF16, F32, I32 = iomx.DT_BF16, iomx.DT_F32, iomx.DT_I32
+ADD, MUL = iomx.OP_ADD, iomx.OP_MUL
+BASE = 1 << 22  # elements of the seeded base pattern that is repeated over big tensors
+
+
+# --------------------------------------------------------------------------- data
+
+def _repeat(base: np.ndarray, count: int) -> np.ndarray:
+    reps = (count + base.size - 1) // base.size
+    return np.tile(base, reps)[:count]
+
+
+def synth(dtype: int, count: int, kind: str, salt: int) -> np.ndarray:
+    """Raw leaf bits of `count` elements drawn from the named distribution."""
+    n = min(count, BASE)
+    if kind == "uniform_pm1":
+        v = datagen.uniform_f32(n, -1.0, 1.0, salt)
+    elif kind == "uniform_i20":
+        return _repeat(datagen.uniform_i32(n, -(1 << 20), 1 << 20, salt), count)
+    elif kind == "normal":
+        v = datagen.normal_f32(n, 0.0, 1.0, salt)
+    elif kind == "normal_0p02":
+        v = datagen.normal_f32(n, 0.0, 0.02, salt)
+    elif kind == "uniform_half_3half":
+        v = datagen.uniform_f32(n, 0.5, 1.5, salt)
+    else:
+        raise ValueError(kind)
+    bits = datagen.bf16_rne(v) if dtype == BF16 else v.view(np.uint32)
+    return _repeat(bits, count)
+
+
+def device_tensor(dtype, dims, kind=None, salt=0, outlier_rows=False):
+    """Owner in HBM.  Every benchmark shape is a multiple of 16 in both matrix axes,
+    so tiled storage equals a permutation of the logical data and the raw upload of
+    an i.i.d. pattern has the stated distribution."""
+    t = iomx.DeviceTensor(dtype, dims, fill=None)
+    if kind is not None:
+        n = t.nbytes // iomx.leaf_bytes(dtype)
+        bits = synth(dtype, n, kind, salt)
+        if outlier_rows:
+            # 1 % of the rows scaled by 50: whole 16-element tile-row segments of
+            # every 100th row of each band
+            f = (datagen.bf16_to_f32(bits) if dtype == BF16 else bits.view(np.float32)).copy()
+            seg = f.reshape(-1, 16)
+            cols16 = dims[-1] // 16
+            row_of_seg = (np.arange(seg.shape[0]) // (16 * cols16)) * 16 + np.arange(seg.shape[0]) % 16
+            seg[row_of_seg % 100 == 0] *= 50.0
+            bits = datagen.bf16_rne(seg.reshape(-1)) if dtype == BF16 else seg.reshape(-1).view(np.uint32)
+        t.upload_raw(bits)
+    return t
+
+
+# ------------------------------------------------------------------------ timing
+
+class Timer:
+    """HIP events on the launch stream + host wall clock around the same region."""
+
+    def __init__(self, stream):
+        self.stream = stream
+        self.start, self.stop = iomx.Event(True), iomx.Event(True)
+
+    def run(self, launch, steps: int, warmup: int):
+        for i in range(warmup):
+            launch(i)
+        self.stream.synchronize()
+        iomx.synchronize()
+        t0 = time.perf_counter()
+        self.start.record(self.stream)
+        for i in range(steps):
+            launch(warmup + i)
+        self.stop.record(self.stream)
+        self.stream.synchronize()
+        iomx.synchronize()
+        wall = time.perf_counter() - t0
+        return wall / steps * 1e3, self.start.elapsed_ms(self.stop) / steps
+
+
+def report(name, alg_bytes, elements, wall_ms, event_ms, kernel, extra=None):
+    gbs = alg_bytes / (event_ms * 1e-3) / 1e9
+    r = {
+        "workload": name, "kernel": kernel, "algorithmic_bytes": int(alg_bytes),
+        "elements": int(elements), "ms_per_launch": round(event_ms, 5),
+        "ms_per_step_wall": round(wall_ms, 5), "GB_per_s": round(gbs, 1),
+        "Gelem_per_s": round(elements / (event_ms * 1e-3) / 1e9, 2),
+        "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+    }
+    if extra:
+        r.update(extra)
+    return r
+
+
+# --------------------------------------------------------------------- workloads
+
+ROT = 4  # buffer sets rotated through, so the footprint exceeds the Infinity Cache
+
+
+def check(rc, what):
+    if rc != 0:
+        raise iomx.IomxError(rc, what)
+
+
+def wl_binary(timer, steps, warmup, name, dtype, op, dims, rhs_dims, kinds, lhs_view=None):
+    """lhs (op) rhs -> out over ROT rotating buffer sets."""
+    esize = iomx.leaf_bytes(dtype)
+    sets = []
+    for i in range(ROT):
+        if lhs_view is None:
+            lhs = device_tensor(dtype, dims, kinds[0], 11 + i)
+            lv = lhs.view()
+        else:
+            owner_dims, fn = lhs_view
+            lhs = device_tensor(dtype, owner_dims, kinds[0], 11 + i)
+            lv = fn(lhs.view())
+        rhs = device_tensor(dtype, rhs_dims, kinds[1], 23 + i)
+        out = device_tensor(dtype, dims)
+        sets.append((lhs, rhs, out, lv))
+    n = int(np.prod(dims))
+    nr = int(np.prod(rhs_dims))
+    alg = (2 * n + nr) * esize if nr != n else 3 * n * esize
+
+    def launch(i):
+        lhs, rhs, out, lv = sets[i % ROT]
+        check(iomx.binary(op, lv, rhs.view(), out.view(), timer.stream), name)
+
+    wall, ev = timer.run(launch, steps, warmup)
+    kernel = iomx.last_launch().kernel.decode()
+    for s in sets:
+        for t in s[:3]:
+            t.free()
+    return report(name, alg, n, wall, ev, kernel)
+
+
+def wl_rmsnorm(timer, steps, warmup, name, dtype, dims):
+    esize = iomx.leaf_bytes(dtype)
+    F = dims[-1]
+    w = device_tensor(dtype, (1, F), "uniform_half_3half", 5)
+    sets = [(device_tensor(dtype, dims, "normal", 31 + i, outlier_rows=True), device_tensor(dtype, dims))
+            for i in range(ROT)]
+    n = int(np.prod(dims))
+    alg = (2 * n + F) * esize
+
+    def launch(i):
+        x, o = sets[i % ROT]
+        check(iomx.rmsnorm(x.view(), w.view(), o.view(), 1e-5, timer.stream), name)
+
+    wall, ev = timer.run(launch, steps, warmup)
+    kernel = iomx.last_launch().kernel.decode()
+    for x, o in sets:
+        x.free()
+        o.free()
+    w.free()
+    return report(name, alg, n, wall, ev, kernel)
+
+
+def wl_silu_mul(timer, steps, warmup, dims):
+    """silu(gate) -> act (stored BF16), then act*up -> prod; also the fused private path."""
+    out = []
+    rot = 2
+    sets = [(device_tensor(BF16, dims, "normal", 41 + i), device_tensor(BF16, dims, "normal", 51 + i),
+             device_tensor(BF16, dims), device_tensor(BF16, dims)) for i in range(rot)]
+    n = int(np.prod(dims))
+
+    def silu(i):
+        g, u, a, p = sets[i % rot]
+        check(iomx.silu(g.view(), a.view(), timer.stream), "silu")
+
+    def mul(i):
+        g, u, a, p = sets[i % rot]
+        check(iomx.binary(MUL, a.view(), u.view(), p.view(), timer.stream), "mul")
+
+    def fused(i):
+        g, u, a, p = sets[i % rot]
+        check(iomx.silu_mul(g.view(), u.view(), p.view(), timer.stream), "silu_mul")
+
+    wall, ev = timer.run(silu, steps, warmup)
+    out.append(report("silu_bf16_[32768,5632]", 4 * n, n, wall, ev, iomx.last_launch().kernel.decode()))
+    wall, ev = timer.run(mul, steps, warmup)
+    out.append(report("mul_bf16_[32768,5632]", 6 * n, n, wall, ev, iomx.last_launch().kernel.decode()))
+    wall, ev = timer.run(fused, steps, warmup)
+    out.append(report("fused_silu_mul_bf16_[32768,5632] (private path)", 6 * n, n, wall, ev,
+                      iomx.last_launch().kernel.decode()))
+    for s in sets:
+        for t in s:
+            t.free()
+    return out
+
+
+def wl_softmax(timer, steps, warmup, planes, heads, rows, cols, causal_position):
+    """F32 scores [planes,heads,rows,cols] with the strict upper triangle = -inf as data.
+    causal_position=False: a = cols-1, every token is positionally visible (the mask
+    is data, all of it is read).  True: a = 0, only t <= r is read."""
+    n = planes * heads * rows * cols
+    one = datagen.normal_f32(rows * cols, 0.0, 3.0, 61).reshape(rows, cols)
+    one[np.triu_indices(rows, 1, cols)] = -np.inf
+    sb = iomx.Buffer(n * 4)
+    pb = iomx.Buffer(n * 2)
+    sb.upload(one)
+    mat = rows * cols * 4
+    copied = 1
+    total = planes * heads
+    while copied < total:  # doubling device-to-device copies
+        m = min(copied, total - copied)
+        check(iomx.lib().iomx_memcpy_d2d_async(sb.ptr.value + copied * mat, sb.ptr.value, m * mat,
+                                               timer.stream.h), "d2d")
+        timer.stream.synchronize()
+        copied += m
+    a = 0 if causal_position else cols - 1
+    d = iomx.softmax_desc(sb.ptr.value, pb.ptr.value, planes, heads, rows, cols, a, cols, 1.0)
+
+    def launch(i):
+        check(iomx.softmax(d, timer.stream), "softmax")
+
+    wall, ev = timer.run(launch, steps, warmup)
+    kernel = iomx.last_launch().kernel.decode()
+    sb.free()
+    pb.free()
+    if causal_position:
+        visible = planes * heads * (rows * (rows + 1) // 2)
+        alg = 4 * visible + 2 * n
+        name = f"softmax_f32_to_bf16_[{planes},{heads},{rows},{cols}]_positional_causal"
+    else:
+        alg = 6 * n
+        name = f"softmax_f32_to_bf16_[{planes},{heads},{rows},{cols}]_mask_as_data"
+    return report(name, alg, n, wall, ev, kernel)
+
+
+def wl_chain(timer, steps, warmup):
+    """Non-GEMM op chain of one TinyLlama-1.1B decoder layer over [64,512,.] BF16:
+    rmsnorm(x,w1)->n; add(x,attn)->x2; rmsnorm(x2,w2)->n2; silu(gate)->act;
+    mul(act,up)->prod; add(x2,down)->next (order of src/session.cpp:2842,2500,1996-2042)."""
+    B, S, H, FF = 64, 512, 2048, 5632
+    hd, fd = (B, S, H), (B, S, FF)
+    x, attn, down = (device_tensor(BF16, hd, "normal", s) for s in (1, 2, 3))
+    gate, up = device_tensor(BF16, fd, "normal", 4), device_tensor(BF16, fd, "normal", 5)
+    w1, w2 = (device_tensor(BF16, (1, H), "uniform_half_3half", s) for s in (6, 7))
+    n1, x2, n2, nxt = (device_tensor(BF16, hd) for _ in range(4))
+    act, prod = device_tensor(BF16, fd), device_tensor(BF16, fd)
+    st = timer.stream
+
+    def launch(i):
+        check(iomx.rmsnorm(x.view(), w1.view(), n1.view(), 1e-5, st), "rmsnorm1")
+        check(iomx.binary(ADD, x.view(), attn.view(), x2.view(), st), "add1")
+        check(iomx.rmsnorm(x2.view(), w2.view(), n2.view(), 1e-5, st), "rmsnorm2")
+        check(iomx.silu(gate.view(), act.view(), st), "silu")
+        check(iomx.binary(MUL, act.view(), up.view(), prod.view(), st), "mul")
+        check(iomx.binary(ADD, x2.view(), down.view(), nxt.view(), st), "add2")
+
+    wall, ev = timer.run(launch, steps, warmup)
+    nh, nf = B * S * H, B * S * FF
+    alg = 2 * (4 * nh + 2 * H) + 2 * (6 * nh) + 4 * nf + 6 * nf
+    for t in (x, attn, down, gate, up, w1, w2, n1, x2, n2, nxt, act, prod):
+        t.free()
+    return report("tinyllama_layer_non_gemm_chain_bf16_[64,512]", alg, 4 * nh + 2 * nf, wall, ev,
+                  "6 launches")
+
+
+# ------------------------------------------------------------------ CPU baseline
+
+def cpu_baseline():
+    """The reference CPU backend (one worker thread per queue, src/cpu/queue.cpp:230-235)
+    on a bounded sample of the headline workload: [8,512,2048] BF16 + [1,2048], median of
+    5 after 1 warm-up (the method of test/cpu/test_cpu_bench.cpp:45-83)."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import iomo
+    dims, vdims = (8, 512, 2048), (1, 2048)
+    n = int(np.prod(dims))
+    x = synth(BF16, n, "normal", 11).reshape(dims)
+    b = synth(BF16, 2048, "normal_0p02", 23).reshape(vdims)
+    alg = (2 * n + 2048) * 2
+    if iomo.ref_available():
+        ref = iomo.ref_backend()
+        tx, tb, to = ref.tensor(BF16, dims), ref.tensor(BF16, vdims), ref.tensor(BF16, dims)
+        tx.view().from_host(x)
+        tb.view().from_host(b)
+
+        def once():
+            t0 = time.perf_counter()
+            tok = ref.binary(iomo.OP_ADD, tx.view(), tb.view(), to.view())
+            assert tok > 0
+            return time.perf_counter() - t0
+        kind = "reference"
+    else:
+        hx, hb, ho = iomo.HostTensor(BF16, dims), iomo.HostTensor(BF16, vdims), iomo.HostTensor(BF16, dims)
+        hx.view().from_logical(x)
+        hb.view().from_logical(b)
+
+        def once():
+            t0 = time.perf_counter()
+            assert iomo.binary(iomo.OP_ADD, hx.view(), hb.view(), ho.view()) == 0
+            return time.perf_counter() - t0
+        kind = "port"
+    once()
+    samples = sorted(once() for _ in range(5))
+    med = samples[2]
+    return {
+        "value": round(alg / med / 1e9, 5), "unit": "GB/s", "cores": 1, "kind": kind,
+        "sample": "broadcast ADD BF16 [8,512,2048]+[1,2048] (1/8 of the GPU workload), "
+                  "submit to wait, median of 5 after 1 warm-up",
+        "Melem_per_s": round(n / med / 1e6, 3), "seconds_per_run": round(med, 4),
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def traffic_of(key):
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        return json.load(f).get(key, {}).get("hbm_bytes_per_launch")
+
+
+# -------------------------------------------------------------------------- main
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--only", default=None, help="run one workload of `detail` instead of everything")
+    ap.add_argument("--no-detail", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this backend has no multi-GPU path "
+              "(every op is independent per plane; shards need no exchange). Use --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+    if iomx.device_count() < 1:
+        print("no HIP device visible", file=sys.stderr)
+        sys.exit(1)
+    check(iomx.lib().iomx_set_device(0), "set_device")
+    props = iomx.device_props(0)
+    stream = iomx.Stream()
+    timer = Timer(stream)
+    K, W = args.steps, args.warmup
+    hd = (64, 512, 2048)
+
+    table = {
+        "bcast_add_bf16": lambda: wl_binary(timer, K, W, "bcast_add_bf16_[64,512,2048]+[1,2048]", BF16, ADD,
+                                            hd, (1, 2048), ("normal", "normal_0p02")),
+        "bcast_mul_bf16": lambda: wl_binary(timer, K, W, "bcast_mul_bf16_[64,512,2048]*[1,2048]", BF16, MUL,
+                                            hd, (1, 2048), ("normal", "normal_0p02")),
+        "bcast_add_bf16_sliced": lambda: wl_binary(
+            timer, K, W, "bcast_add_bf16_lhs=slice(0,0,64,2)of[128,512,2048]", BF16, ADD, hd, (1, 2048),
+            ("normal", "normal_0p02"), lhs_view=((128, 512, 2048), lambda v: v.slice(0, 0, 64, 2))),
+        "bcast_add_bf16_permuted": lambda: wl_binary(
+            timer, K, W, "bcast_add_bf16_lhs=permute(1,0)of[8,8,512,2048]", BF16, ADD, (8, 8, 512, 2048),
+            (1, 2048), ("normal", "normal_0p02"),
+            lhs_view=((8, 8, 512, 2048), lambda v: v.permute([1, 0]))),
+        "add_f32": lambda: wl_binary(timer, K, W, "add_f32_[4096,4096]", F32, ADD, (4096, 4096),
+                                     (4096, 4096), ("uniform_pm1", "uniform_pm1")),
+        "add_i32": lambda: wl_binary(timer, K, W, "add_i32_[4096,4096]", I32, ADD, (4096, 4096),
+                                     (4096, 4096), ("uniform_i20", "uniform_i20")),
+        "rmsnorm_bf16": lambda: wl_rmsnorm(timer, K, W, "rmsnorm_bf16_[32768,2048]", BF16, (32768, 2048)),
+        "rmsnorm_f32": lambda: wl_rmsnorm(timer, K, W, "rmsnorm_f32_[32768,2048]", F32, (32768, 2048)),
+        "silu_mul": lambda: wl_silu_mul(timer, max(K // 4, 5), max(W // 4, 2), (32768, 5632)),
+        "softmax": lambda: wl_softmax(timer, max(K // 20, 3), 2, 32, 32, 2048, 2048, False),
+        "softmax_causal": lambda: wl_softmax(timer, max(K // 20, 3), 2, 32, 32, 2048, 2048, True),
+        "chain": lambda: wl_chain(timer, max(K // 10, 5), max(W // 10, 2)),
+    }
+
+    if args.only:
+        for key in args.only.split(","):
+            r = table[key]()
+            for row in (r if isinstance(r, list) else [r]):
+                print(json.dumps({"only": key, "result": row}))
+        return
+
+    head = table["bcast_add_bf16"]()
+    detail = []
+    if not args.no_detail:
+        for key in ("bcast_mul_bf16", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "add_f32",
+                    "add_i32", "rmsnorm_bf16", "rmsnorm_f32", "silu_mul", "softmax", "softmax_causal",
+                    "chain"):
+            r = table[key]()
+            detail.extend(r if isinstance(r, list) else [r])
+    cpu = None if args.no_cpu else cpu_baseline()
+
+    line = {
+        "metric": "achieved HBM GB/s (% of MI355X peak) for ADD, broadcast ADD, RMSNorm",
+        "value": head["GB_per_s"],
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": head["ms_per_step_wall"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "broadcast ADD BF16 [64,512,2048] + [1,2048] (tiled 16x16, "
+                               "configs[1])", "elements": head["elements"],
+                   "algorithmic_bytes": head["algorithmic_bytes"],
+                   "hbm_frac_of_8TBps": head["hbm_frac"], "Gelem_per_s": head["Gelem_per_s"],
+                   "device": props.name.decode(), "compute_units": props.compute_units},
+        "roofline": {"bound": "hbm", "achieved": head["GB_per_s"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": head["hbm_frac"], "traffic": traffic_of("bcast_add_bf16"),
+                     "kernel": "elementwise_planes_kernel<BF16,ADD,FULL,ROWVEC>",
+                     "ms_per_launch": head["ms_per_launch"]},
+        "cpu_baseline": cpu,
+        "detail": detail,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

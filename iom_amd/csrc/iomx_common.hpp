@@ -200,22 +200,26 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return as_f32(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return as_f32(w & 0xFFFF0000u); }
 
-// Owner plane of operand k for the linear result plane p.
+// Owner plane of operand k for the linear result plane p.  The outermost
+// coordinate needs no division, and the loop stays rolled so that a launch with
+// one leading axis (the common case) pays for none.
 template <int N>
 __device__ __forceinline__ void walk_planes(const PlaneWalk<N>& w, uint32_t p, uint64_t* out) {
 #pragma unroll
     for (int k = 0; k < N; ++k) out[k] = w.offset[k];
+    if (w.nlead == 0) return;
+    uint32_t rem = p;
+#pragma clang loop unroll(disable)
+    for (uint32_t a = w.nlead - 1; a >= 1; --a) {
+        const uint32_t d = w.dims[a];
+        const uint32_t q = rem / d;
+        const uint32_t c = rem - q * d;
+        rem = q;
 #pragma unroll
-    for (int a = kMaxLead - 1; a >= 0; --a) {
-        if (a < (int)w.nlead) {
-            const uint32_t d = w.dims[a];
-            const uint32_t q = p / d;
-            const uint32_t c = p - q * d;
-            p = q;
-#pragma unroll
-            for (int k = 0; k < N; ++k) out[k] += (uint64_t)c * w.stride[k][a];
-        }
+        for (int k = 0; k < N; ++k) out[k] += (uint64_t)c * w.stride[k][a];
     }
+#pragma unroll
+    for (int k = 0; k < N; ++k) out[k] += (uint64_t)rem * w.stride[k][0];
 }
 
 #endif  // __HIPCC__

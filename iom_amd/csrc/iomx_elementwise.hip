@@ -40,15 +40,20 @@ __device__ __forceinline__ float silu_f32(float x) {
     return num / den;
 }
 
+// Work decomposition of the streaming kernel: a result plane (z) is cut into
+// segments (y) of seg_chunks 128-bit chunks, and a wave takes 64 consecutive
+// chunks of one segment (x).  With whole-plane operands only, the segment is the
+// plane (or every plane at once when the selection is dense).  With a row-vector
+// operand the segment is one tile-row band, so the vector chunk a lane needs
+// follows from its position in the segment by bit operations alone.
 struct BinaryArgs {
     const uint8_t* src[2];
     uint8_t* out;
-    PlaneWalk<3> walk;        // 0 lhs, 1 rhs, 2 out
+    uint64_t seg_chunks;
+    uint32_t segments;        // per plane
+    uint32_t planes;
     uint64_t plane_bytes[3];  // bytes of one owner plane
-    uint64_t plane_chunks;    // 16-byte chunks of one result plane range
-    uint32_t blocks_per_plane;
-    uint32_t total_blocks;
-    uint32_t tile_cols;       // tile columns of the result (ROWVEC addressing)
+    PlaneWalk<3> walk;        // 0 lhs, 1 rhs, 2 out
 };
 
 struct GeneralArgs {
@@ -123,59 +128,84 @@ struct Leaf {
     static constexpr uint32_t kChunksPerTile = kTileSlots / kPerChunk;
 };
 
-constexpr int kUnroll = 4;
-constexpr uint32_t kBlock = 256;
-constexpr uint32_t kBlockChunks = kBlock * kUnroll;
+// Launch shape of the streaming kernel.  Measured on MI355X with 64..1024 MiB
+// operands: one wave per workgroup, one 128-bit chunk per lane and streaming
+// (nontemporal) loads and stores sustain the most HBM bandwidth; larger
+// workgroups or deeper unrolling lose 3-15 %.
+constexpr uint32_t kPlanesBlock = 64;
+constexpr uint32_t kBlock = 256;  // general kernel
+
+__device__ __forceinline__ u32x4 load_stream(const uint8_t* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ void store_stream(uint8_t* p, u32x4 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+
+// Kernel arguments of the two cheap shapes: everything in one dense range
+// (FLAT), or one dense range cut into tile-row bands (BANDS).  A wave of these
+// kernels reads its few arguments, forms three addresses and issues its loads:
+// nothing else stands before the memory system.
+struct FlatArgs {
+    const uint8_t* src[2];
+    uint8_t* out;
+    uint64_t seg_chunks;
+    uint32_t segments;
+};
+
+enum { SHAPE_FLAT = 0, SHAPE_BANDS = 1, SHAPE_PLANES = 2 };
 
 template <int DT, int OP, int LM, int RM>
-__global__ __launch_bounds__(kBlock) void elementwise_planes_kernel(const BinaryArgs a) {
-    using L = Leaf<DT>;
+__device__ __forceinline__ void stream_chunk(const uint8_t* lbase, const uint8_t* rbase,
+                                             uint8_t* obase, uint64_t off, uint64_t voff) {
     constexpr int kInputs = Arity<OP>::kInputs;
-    constexpr uint32_t kTilesPerBlock = kBlockChunks / L::kChunksPerTile;
-    const uint32_t tid = threadIdx.x;
-    for (uint32_t w = blockIdx.x; w < a.total_blocks; w += gridDim.x) {
-        uint32_t p = 0, bip = w;
-        if (a.walk.nlead != 0) {
-            p = w / a.blocks_per_plane;
-            bip = w - p * a.blocks_per_plane;
-        }
+    // whole-plane operands stream past the caches; the row vector is reused by
+    // every row and stays cached
+    u32x4 va, vb = u32x4{0, 0, 0, 0};
+    if constexpr (LM == MODE_ROWVEC) va = *reinterpret_cast<const u32x4*>(lbase + voff);
+    else va = load_stream(lbase + off);
+    if constexpr (kInputs == 2) {
+        if constexpr (RM == MODE_ROWVEC) vb = *reinterpret_cast<const u32x4*>(rbase + voff);
+        else vb = load_stream(rbase + off);
+    }
+    store_stream(obase + off, op_chunk<DT, OP>(va, vb));
+}
+
+// chunk of row 0 of the lane's tile column, for row-vector operands
+template <int DT>
+__device__ __forceinline__ uint64_t rowvec_offset(uint64_t cb) {
+    using L = Leaf<DT>;
+    return ((cb & ~(uint64_t)(L::kChunksPerTile - 1)) | (cb & (L::kChunksPerRow - 1))) * 16;
+}
+
+template <int DT, int OP, int LM, int RM, int SHAPE>
+__global__ __launch_bounds__(kPlanesBlock) void elementwise_stream_kernel(const FlatArgs a) {
+    const uint64_t cb = (uint64_t)blockIdx.x * kPlanesBlock + threadIdx.x;
+    if (cb >= a.seg_chunks) return;
+    if constexpr (SHAPE == SHAPE_FLAT) {
+        stream_chunk<DT, OP, LM, RM>(a.src[0], a.src[1], a.out, cb * 16, 0);
+    } else {
+        const uint64_t voff = rowvec_offset<DT>(cb);
+        for (uint32_t y = blockIdx.y; y < a.segments; y += gridDim.y)
+            stream_chunk<DT, OP, LM, RM>(a.src[0], a.src[1], a.out,
+                                         ((uint64_t)y * a.seg_chunks + cb) * 16, voff);
+    }
+}
+
+template <int DT, int OP, int LM, int RM>
+__global__ __launch_bounds__(kPlanesBlock) void elementwise_planes_kernel(const BinaryArgs a) {
+    const uint64_t cb = (uint64_t)blockIdx.x * kPlanesBlock + threadIdx.x;
+    if (cb >= a.seg_chunks) return;
+    const uint64_t voff = rowvec_offset<DT>(cb);
+    for (uint32_t z = blockIdx.z; z < a.planes; z += gridDim.z) {
         uint64_t plane[3];
-        walk_planes(a.walk, p, plane);
+        walk_planes(a.walk, z, plane);
         const uint8_t* lbase = a.src[0] + plane[0] * a.plane_bytes[0];
         const uint8_t* rbase = a.src[1] + plane[1] * a.plane_bytes[1];
         uint8_t* obase = a.out + plane[2] * a.plane_bytes[2];
-        const uint64_t c0 = (uint64_t)bip * kBlockChunks;
-        // first tile column of this block, for row-vector operands
-        uint32_t tcol0 = 0;
-        if constexpr (LM == MODE_ROWVEC || RM == MODE_ROWVEC) {
-            tcol0 = (uint32_t)((c0 / L::kChunksPerTile) % a.tile_cols);
-        }
-        u32x4 va[kUnroll], vb[kUnroll];
-        bool ok[kUnroll];
-#pragma unroll
-        for (int i = 0; i < kUnroll; ++i) {
-            const uint32_t local = i * kBlock + tid;
-            const uint64_t c = c0 + local;
-            ok[i] = c < a.plane_chunks;
-            uint64_t voff = 0;
-            if constexpr (LM == MODE_ROWVEC || RM == MODE_ROWVEC) {
-                uint32_t tc = tcol0 + local / L::kChunksPerTile;
-                if (a.tile_cols >= kTilesPerBlock) tc -= (tc >= a.tile_cols) ? a.tile_cols : 0;
-                else tc %= a.tile_cols;
-                voff = ((uint64_t)tc * L::kChunksPerTile + (local % L::kChunksPerRow)) * 16;
-            }
-            vb[i] = u32x4{0, 0, 0, 0};
-            if (ok[i]) {
-                va[i] = *reinterpret_cast<const u32x4*>(lbase + (LM == MODE_ROWVEC ? voff : c * 16));
-                if constexpr (kInputs == 2)
-                    vb[i] = *reinterpret_cast<const u32x4*>(rbase + (RM == MODE_ROWVEC ? voff : c * 16));
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < kUnroll; ++i) {
-            const uint64_t c = c0 + i * kBlock + tid;
-            if (ok[i]) *reinterpret_cast<u32x4*>(obase + c * 16) = op_chunk<DT, OP>(va[i], vb[i]);
-        }
+        for (uint32_t y = blockIdx.y; y < a.segments; y += gridDim.y)
+            stream_chunk<DT, OP, LM, RM>(lbase, rbase, obase,
+                                         ((uint64_t)y * a.seg_chunks + cb) * 16, voff);
     }
 }
 
@@ -275,9 +305,9 @@ bool same_window(const iomx_view& a, const iomx_view& b) {
 }
 
 uint32_t grid_for(uint64_t blocks) {
-    // Enough resident waves to cover HBM latency on 256 CUs, few enough that the
-    // scalar plane walk amortises; the kernels loop over the remainder.
-    const uint64_t cap = 256ull * 64;
+    // One workgroup per block of work: the hardware dispatcher keeps the access
+    // stream in address order; the kernels loop only beyond the grid limit.
+    const uint64_t cap = 0x7FFFFFFFull;
     return (uint32_t)(blocks < cap ? blocks : cap);
 }
 
@@ -295,10 +325,25 @@ template <int DT, int OP>
 int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs& ga,
            hipStream_t s) {
     if (planes) {
-        const uint32_t grid = grid_for(pa.total_blocks);
-#define IOMX_PLANES(LMV, RMV)                                                              \
-    hipLaunchKernelGGL((elementwise_planes_kernel<DT, OP, LMV, RMV>), dim3(grid),          \
-                       dim3(kBlock), 0, s, pa)
+        const uint64_t gx = (pa.seg_chunks + kPlanesBlock - 1) / kPlanesBlock;
+        if (gx > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
+        const dim3 grid3((uint32_t)gx, pa.segments < 65535u ? pa.segments : 65535u,
+                         pa.planes < 65535u ? pa.planes : 65535u);
+        const uint32_t grid = grid3.x;
+        FlatArgs fa = {{pa.src[0], pa.src[1]}, pa.out, pa.seg_chunks, pa.segments};
+        const bool dense = pa.planes == 1 && pa.walk.nlead == 0;
+#define IOMX_PLANES(LMV, RMV)                                                                   \
+    do {                                                                                        \
+        if (dense && pa.segments == 1)                                                          \
+            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SHAPE_FLAT>), grid3, \
+                               dim3(kPlanesBlock), 0, s, fa);                                   \
+        else if (dense)                                                                         \
+            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SHAPE_BANDS>),      \
+                               grid3, dim3(kPlanesBlock), 0, s, fa);                            \
+        else                                                                                    \
+            hipLaunchKernelGGL((elementwise_planes_kernel<DT, OP, LMV, RMV>), grid3,            \
+                               dim3(kPlanesBlock), 0, s, pa);                                   \
+    } while (0)
         if (lm == MODE_FULL && rm == MODE_FULL) IOMX_PLANES(MODE_FULL, MODE_FULL);
         else if constexpr (OP <= IOMX_OP_SUB) {
             if (lm == MODE_FULL) IOMX_PLANES(MODE_FULL, MODE_ROWVEC);
@@ -307,8 +352,8 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
             return IOMX_ERR_INVALID;
         }
 #undef IOMX_PLANES
-        record_launch(family(OP, true, lm != MODE_FULL || rm != MODE_FULL), grid, kBlock,
-                      pa.total_blocks);
+        record_launch(family(OP, true, lm != MODE_FULL || rm != MODE_FULL), grid, kPlanesBlock,
+                      gx * pa.segments * pa.planes);
     } else {
         const uint64_t blocks = (ga.total_pieces + kBlock - 1) / kBlock;
         const uint32_t grid = grid_for(blocks);
@@ -403,31 +448,36 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
         pa.out = static_cast<uint8_t*>(out->base);
         pa.walk = walk;
         for (int k = 0; k < 3; ++k) pa.plane_bytes[k] = m[k].plane_elems * bytes;
-        pa.plane_chunks = m[2].plane_elems * bytes / 16;
-        if (m[2].tile_cols > 0xFFFFFFFFull) return IOMX_ERR_OVERFLOW;
-        pa.tile_cols = (uint32_t)m[2].tile_cols;
-        // A dense selection on every FULL operand folds all planes into one range.
+        const bool rowvec = mode[0] == MODE_ROWVEC || mode[1] == MODE_ROWVEC;
+        const uint64_t plane_chunks = m[2].plane_elems * bytes / 16;
+        const uint64_t band_chunks = m[2].tile_cols * (kTileSlots * bytes / 16);
+        uint64_t planes = walk.planes;
+        uint64_t segments = rowvec ? m[2].tile_rows : 1;
+        pa.seg_chunks = rowvec ? band_chunks : plane_chunks;
+        // A dense selection on every whole-plane operand (and a row vector shared by
+        // all planes) folds the planes into one range.
         bool fold = walk.nlead <= 1;
         for (int k = 0; k < 3 && fold; ++k) {
-            const bool rowvec = k < 2 && mode[k] == MODE_ROWVEC;
-            if (rowvec) fold = walk.nlead == 0 || walk.stride[k][0] == 0;
+            const bool vec = k < 2 && mode[k] == MODE_ROWVEC;
+            if (vec) fold = walk.nlead == 0 || walk.stride[k][0] == 0;
             else fold = walk_is_dense(walk, k);
         }
-        if (fold && walk.planes > 1) {
-            if (mul_overflows(pa.plane_chunks, walk.planes, &pa.plane_chunks)) return IOMX_ERR_OVERFLOW;
+        if (fold) {
             pa.src[0] += offsets[0] * pa.plane_bytes[0];
             pa.src[1] += offsets[1] * pa.plane_bytes[1];
             pa.out += offsets[2] * pa.plane_bytes[2];
             for (int k = 0; k < 3; ++k) pa.walk.offset[k] = 0;
             pa.walk.nlead = 0;
-            pa.walk.planes = 1;
+            if (rowvec) {
+                if (mul_overflows(segments, planes, &segments)) return IOMX_ERR_OVERFLOW;
+            } else if (mul_overflows(pa.seg_chunks, planes, &pa.seg_chunks)) {
+                return IOMX_ERR_OVERFLOW;
+            }
+            planes = 1;
         }
-        const uint64_t per_plane = (pa.plane_chunks + kBlockChunks - 1) / kBlockChunks;
-        uint64_t total;
-        if (mul_overflows(per_plane, pa.walk.planes, &total) || total > 0xFFFFFFFFull)
-            return IOMX_ERR_OVERFLOW;
-        pa.blocks_per_plane = (uint32_t)per_plane;
-        pa.total_blocks = (uint32_t)total;
+        if (segments > 0xFFFFFFFFull || planes > 0xFFFFFFFFull) return IOMX_ERR_OVERFLOW;
+        pa.segments = (uint32_t)segments;
+        pa.planes = (uint32_t)planes;
     } else {
         ga.src[0] = static_cast<const uint8_t*>(lhs->base);
         ga.src[1] = static_cast<const uint8_t*>(rhs->base);
