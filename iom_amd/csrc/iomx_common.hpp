@@ -200,6 +200,19 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return as_f32(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return as_f32(w & 0xFFFF0000u); }
 
+// e^x for x <= 0 (NaN in, NaN out; -inf gives 0), to about two units in the last
+// place, with gradual underflow.  x*log2(e) is formed in two pieces so the
+// rounding of the product does not reach the result; the power of two is applied
+// by v_ldexp_f32, which denormalises correctly where v_exp_f32 would flush.
+__device__ __forceinline__ float exp_nonpos(float x) {
+    const float a = x < -256.0f ? -256.0f : x;  // keeps NaN, bounds the integer part
+    const float hi = a * 1.44269502e+00f;
+    const float lo = __builtin_fmaf(a, 1.44269502e+00f, -hi) + a * 1.92596299e-08f;
+    const float n = __builtin_rintf(hi);
+    const float f = (hi - n) + lo;
+    return __builtin_amdgcn_ldexpf(__builtin_amdgcn_exp2f(f), (int)n);
+}
+
 // Owner plane of operand k for the linear result plane p.  The outermost
 // coordinate needs no division, and the loop stays rolled so that a launch with
 // one leading axis (the common case) pays for none.

@@ -3,13 +3,13 @@
 // In the 16x16-tiled layout one tile-row band (16 logical rows x F features)
 // is one contiguous range, and inside it a wave that reads 64 consecutive
 // 128-bit chunks always sees the same logical row in the same lane.  So a
-// workgroup owns one band, streams it once with fully coalesced loads, keeps it
-// in registers, reduces per lane, combines the lanes of a row inside the wave
-// and the waves through LDS, then scales the registers and stores: HBM sees x
-// once and out once.
+// workgroup owns one band at a time, streams it once with fully coalesced
+// loads, keeps it in registers, reduces per lane, combines the lanes of a row
+// inside the wave and the waves through LDS, then scales the registers and
+// stores: HBM sees x once and out once.
 //
 //   rmsnorm_band     F a multiple of 16 and a band that fits the register
-//                    budget (K chunks per lane).
+//                    budget (at most 16 chunks per lane of a 1024-lane workgroup).
 //   rmsnorm_generic  any F and any band size: two passes over the band, the
 //                    second served by L2, with per-element column masks.
 #include "iomx_common.hpp"
@@ -96,81 +96,82 @@ __device__ __forceinline__ float inverse_rms(float sum, uint32_t feats, float ep
     return 1.0f / root;
 }
 
-template <int DT, int K, int THREADS, bool PREFETCH>
+// The band kernel: one band per workgroup, K 128-bit chunks per lane held in
+// registers between the two passes.  Whole-band loads and stores stream past
+// the caches; the scale row stays cached.  Keeping the register count low keeps
+// two 1024-lane workgroups resident per compute unit, so one band's loads
+// overlap the other's arithmetic and stores.  (Variants measured and dropped on
+// MI355X, [32768,2048]: a persistent workgroup that prefetches its next band
+// into a second register set, the scale row decoded once into registers, sixteen
+// lanes finishing the row totals for everyone, and a barrier-free kernel with
+// four rows per wave: all slower, by 3-20 %.)
+//
+// The sum of squares uses a fused multiply-add per element (one rounding instead
+// of the reference's two): the total differs from the sequential reference
+// recurrence by a few units in the last place either way, far inside the bar.
+template <int DT, int K, int THREADS>
 __global__ __launch_bounds__(THREADS) void rmsnorm_band_kernel(const RmsArgs a) {
     using L = RLeaf<DT>;
     constexpr int kWaves = THREADS / 64;
-    __shared__ float partial[kWaves][kTile];
+    __shared__ __attribute__((aligned(16))) float partial[kTile][kWaves];
     const uint32_t tid = threadIdx.x;
     const uint32_t row = lane_row<DT>(tid);
-    for (uint32_t band = blockIdx.x; band < a.total_bands; band += gridDim.x) {
-        const uint32_t p = band / a.tile_rows;
-        const uint32_t tr = band - p * a.tile_rows;
-        uint64_t plane[2];
-        walk_planes(a.walk, p, plane);
-        const uint8_t* xb = a.x + plane[0] * a.plane_bytes + (uint64_t)tr * a.band_bytes;
-        uint8_t* ob = a.out + plane[1] * a.plane_bytes + (uint64_t)tr * a.band_bytes;
-
-        u32x4 v[K];
-        u32x4 w[PREFETCH ? K : 1];
+    const uint32_t band = blockIdx.x;
+    uint32_t p = 0, tr = band;
+    if (a.walk.nlead != 0) {
+        p = band / a.tile_rows;
+        tr = band - p * a.tile_rows;
+    }
+    uint64_t plane[2];
+    walk_planes(a.walk, p, plane);
+    const uint8_t* xb = a.x + plane[0] * a.plane_bytes + (uint64_t)tr * a.band_bytes;
+    uint8_t* ob = a.out + plane[1] * a.plane_bytes + (uint64_t)tr * a.band_bytes;
+    u32x4 cur[K];
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const uint32_t c = tid + k * THREADS;
-            v[k] = u32x4{0, 0, 0, 0};
-            if (c < a.band_chunks) v[k] = *reinterpret_cast<const u32x4*>(xb + (uint64_t)c * 16);
-        }
-        if constexpr (PREFETCH) {
+    for (int k = 0; k < K; ++k) {
+        const uint32_t c = tid + k * THREADS;
+        cur[k] = u32x4{0, 0, 0, 0};
+        if (c < a.band_chunks)
+            cur[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xb + (uint64_t)c * 16));
+    }
+    float acc = 0.0f;
 #pragma unroll
-            for (int k = 0; k < K; ++k) {
-                const uint32_t c = tid + k * THREADS;
-                const uint32_t soff = ((c / L::kChunksPerTile) * L::kChunksPerTile
-                                       + (c % L::kChunksPerRow)) * 16;
-                w[k] = u32x4{0, 0, 0, 0};
-                if (c < a.band_chunks) w[k] = *reinterpret_cast<const u32x4*>(a.scale + soff);
+    for (int k = 0; k < K; ++k) {
+        float f[L::kPerChunk];
+        unpack<DT>(cur[k], f);
+#pragma unroll
+        for (uint32_t e = 0; e < L::kPerChunk; ++e) acc = __builtin_fmaf(f[e], f[e], acc);
+    }
+    acc = row_sum_in_wave<DT>(acc);
+    float inverse;
+    if constexpr (kWaves > 1) {
+        if (row_leader<DT>(tid)) partial[row][tid / 64] = acc;
+        __syncthreads();
+        float total = 0.0f;
+#pragma unroll
+        for (int wv = 0; wv < kWaves; ++wv) total = total + partial[row][wv];
+        inverse = inverse_rms(total, a.feats, a.eps);
+    } else {
+        inverse = inverse_rms(acc, a.feats, a.eps);
+    }
+    if (tr * kTile + row >= a.rows) return;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t c = tid + k * THREADS;
+        if (c < a.band_chunks) {
+            const uint32_t soff = ((c / L::kChunksPerTile) * L::kChunksPerTile
+                                   + (c % L::kChunksPerRow)) * 16;
+            float f[L::kPerChunk], sc[L::kPerChunk];
+            unpack<DT>(cur[k], f);
+            unpack<DT>(*reinterpret_cast<const u32x4*>(a.scale + soff), sc);
+#pragma unroll
+            for (uint32_t e = 0; e < L::kPerChunk; ++e) {
+                const float normalized = f[e] * inverse;
+                f[e] = normalized * sc[e];
             }
+            u32x4* dst = reinterpret_cast<u32x4*>(ob + (uint64_t)c * 16);
+            __builtin_nontemporal_store(pack<DT>(f), dst);
         }
-        float acc = 0.0f;
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-            float f[L::kPerChunk];
-            unpack<DT>(v[k], f);
-#pragma unroll
-            for (uint32_t e = 0; e < L::kPerChunk; ++e) acc = acc + f[e] * f[e];
-        }
-        acc = row_sum_in_wave<DT>(acc);
-        if (kWaves > 1) {
-            if (row_leader<DT>(tid)) partial[tid / 64][row] = acc;
-            __syncthreads();
-            acc = 0.0f;
-#pragma unroll
-            for (int wv = 0; wv < kWaves; ++wv) acc = acc + partial[wv][row];
-        }
-        const float inverse = inverse_rms(acc, a.feats, a.eps);
-        const bool live = tr * kTile + row < a.rows;
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const uint32_t c = tid + k * THREADS;
-            if (c < a.band_chunks && live) {
-                u32x4 wk;
-                if constexpr (PREFETCH) {
-                    wk = w[k];
-                } else {
-                    const uint32_t soff = ((c / L::kChunksPerTile) * L::kChunksPerTile
-                                           + (c % L::kChunksPerRow)) * 16;
-                    wk = *reinterpret_cast<const u32x4*>(a.scale + soff);
-                }
-                float f[L::kPerChunk], s[L::kPerChunk];
-                unpack<DT>(v[k], f);
-                unpack<DT>(wk, s);
-#pragma unroll
-                for (uint32_t e = 0; e < L::kPerChunk; ++e) {
-                    const float normalized = f[e] * inverse;
-                    f[e] = normalized * s[e];
-                }
-                *reinterpret_cast<u32x4*>(ob + (uint64_t)c * 16) = pack<DT>(f);
-            }
-        }
-        if (kWaves > 1) __syncthreads();  // partial[] is reused by the next band
     }
 }
 
@@ -243,29 +244,29 @@ __global__ __launch_bounds__(256) void rmsnorm_generic_kernel(const RmsArgs a) {
 
 namespace {
 
-template <int DT, int K, int THREADS, bool PREFETCH>
-void launch_band(const RmsArgs& a, uint32_t grid, hipStream_t s) {
-    hipLaunchKernelGGL((rmsnorm_band_kernel<DT, K, THREADS, PREFETCH>), dim3(grid), dim3(THREADS),
-                       0, s, a);
-    record_launch("rmsnorm_band", grid, THREADS, a.total_bands);
+template <int DT, int K, int THREADS>
+void launch_band(const RmsArgs& a, hipStream_t s) {
+    hipLaunchKernelGGL((rmsnorm_band_kernel<DT, K, THREADS>), dim3(a.total_bands), dim3(THREADS), 0,
+                       s, a);
+    record_launch("rmsnorm_band", a.total_bands, THREADS, a.total_bands);
 }
 
 template <int DT>
 int launch(const RmsArgs& a, bool band_ok, hipStream_t s) {
-    const uint32_t cap = 1u << 20;
-    const uint32_t grid = a.total_bands < cap ? a.total_bands : cap;
     const uint32_t n = a.band_chunks;
-    if (!band_ok || n > 16384) {
+    if (!band_ok || n > 16384 || a.total_bands > 0x7FFFFFFFu) {
+        const uint32_t cap = 1u << 20;
+        const uint32_t grid = a.total_bands < cap ? a.total_bands : cap;
         hipLaunchKernelGGL((rmsnorm_generic_kernel<DT>), dim3(grid), dim3(256), 0, s, a);
         record_launch("rmsnorm_generic", grid, 256, a.total_bands);
-    } else if (n <= 64) launch_band<DT, 1, 64, true>(a, grid, s);
-    else if (n <= 256) launch_band<DT, 1, 256, true>(a, grid, s);
-    else if (n <= 512) launch_band<DT, 2, 256, true>(a, grid, s);
-    else if (n <= 1024) launch_band<DT, 4, 256, true>(a, grid, s);
-    else if (n <= 2048) launch_band<DT, 8, 256, true>(a, grid, s);
-    else if (n <= 4096) launch_band<DT, 16, 256, true>(a, grid, s);
-    else if (n <= 8192) launch_band<DT, 16, 512, false>(a, grid, s);
-    else launch_band<DT, 16, 1024, false>(a, grid, s);
+    } else if (n <= 64) launch_band<DT, 1, 64>(a, s);
+    else if (n <= 256) launch_band<DT, 1, 256>(a, s);
+    else if (n <= 512) launch_band<DT, 1, 512>(a, s);
+    else if (n <= 1024) launch_band<DT, 1, 1024>(a, s);
+    else if (n <= 2048) launch_band<DT, 2, 1024>(a, s);
+    else if (n <= 4096) launch_band<DT, 4, 1024>(a, s);
+    else if (n <= 8192) launch_band<DT, 8, 1024>(a, s);
+    else launch_band<DT, 16, 1024>(a, s);
     return IOMX_OK;
 }
 
@@ -317,6 +318,16 @@ extern "C" int iomx_launch_rmsnorm(int dtype, const iomx_view* x, const iomx_vie
     a.band_chunks = (uint32_t)band_chunks;
     a.total_bands = (uint32_t)total_bands;
     a.eps = eps;
+    // Dense selections of whole bands fold all planes into one run of bands.
+    if (a.walk.nlead <= 1 && walk_is_dense(a.walk, 0) && walk_is_dense(a.walk, 1)
+        && m.rows % kTile == 0 && total_bands * kTile <= 0xFFFFFFFFull) {
+        a.x += a.walk.offset[0] * a.plane_bytes;
+        a.out += a.walk.offset[1] * a.plane_bytes;
+        a.walk.offset[0] = a.walk.offset[1] = 0;
+        a.walk.nlead = 0;
+        a.tile_rows = (uint32_t)total_bands;
+        a.rows = (uint32_t)(total_bands * kTile);
+    }
     const bool band_ok = m.cols % kTile == 0;
     const hipStream_t s = native(stream);
     if (dtype == IOMX_DT_BF16) IOMX_TRY(launch<IOMX_DT_BF16>(a, band_ok, s));

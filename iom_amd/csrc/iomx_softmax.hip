@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
         const bool poisoned = row_nan || all_ninf;
         uint32_t pinf = 0;
         float inv_share = 0.0f;
-        float sum = 1.0f;
+        float inv_sum = 1.0f;
         if (!poisoned) {
             if (as_u32(m) == kPosInf) {
                 uint32_t cnt = 0;
@@ -115,11 +115,13 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
                 for (int k = 0; k < K; ++k)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const float e = expf(s[k][j] - m);  // exp(-inf) = 0 for masked and -inf scores
+                        const float e = exp_nonpos(s[k][j] - m);  // 0 for masked and -inf scores
                         s[k][j] = e;
                         part = part + e;
                     }
-                sum = wave_sum(part);
+                // e * (1/sum) instead of e / sum: at most one binary32 unit apart,
+                // which a BF16 result shows only at a rounding boundary
+                inv_sum = 1.0f / wave_sum(part);
             }
         }
 #pragma unroll
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
                 float v;
                 if (poisoned) v = as_f32(kQuietNanF32);
                 else if (pinf != 0) v = as_u32(s[k][j]) == kPosInf ? inv_share : 0.0f;
-                else v = s[k][j] / sum;
+                else v = s[k][j] * inv_sum;
                 pr[j] = (col + j < visible) ? v : 0.0f;
             }
             const uint32_t lo = pack_bf16(pr[0], pr[1]);
