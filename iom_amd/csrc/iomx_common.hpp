@@ -102,10 +102,31 @@ inline int check_view(const iomx_view* v, uint32_t bytes) {
 // Passed to kernels by value.
 // ---------------------------------------------------------------------------
 
+// Division of a 32-bit value by a launch-invariant divisor d >= 2 as a multiply
+// and two shifts (round-up method): with l = ceil(log2 d) and
+// m = floor(2^32 (2^l - d) / d) + 1, n / d = (t + ((n - t) >> 1)) >> (l - 1) where
+// t = mulhi(m, n), exact for every 32-bit n.  A wave that needs a plane
+// coordinate pays five scalar operations instead of a reciprocal sequence.
+struct FastDiv {
+    uint32_t mul;
+    uint32_t shift;  // l - 1
+};
+
+inline FastDiv make_fast_div(uint32_t d) {
+    FastDiv f = {0, 0};
+    if (d < 2) return f;
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    f.mul = (uint32_t)((((1ull << l) - d) << 32) / d + 1);
+    f.shift = l - 1;
+    return f;
+}
+
 template <int N>
 struct PlaneWalk {
     uint32_t nlead;                 // axes in use
     uint32_t dims[kMaxLead];        // extents, outermost first
+    FastDiv div[kMaxLead];          // division by dims[a]
     uint64_t stride[N][kMaxLead];   // owner planes per step, 0 = broadcast
     uint64_t offset[N];             // first owner plane
     uint64_t planes;                // product of dims
@@ -146,6 +167,7 @@ inline int build_walk(uint32_t nlead, const uint64_t* dims,
     for (uint32_t a = 0; a < n; ++a) {
         if (d[a] > 0xFFFFFFFFull) return IOMX_ERR_OVERFLOW;
         w->dims[a] = static_cast<uint32_t>(d[a]);
+        w->div[a] = make_fast_div(w->dims[a]);
         for (int k = 0; k < N; ++k) w->stride[k][a] = s[k][a];
     }
     w->nlead = n;
@@ -200,6 +222,11 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return as_f32(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return as_f32(w & 0xFFFF0000u); }
 
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, FastDiv f) {
+    const uint32_t t = __umulhi(f.mul, n);
+    return (t + ((n - t) >> 1)) >> f.shift;
+}
+
 // e^x for x <= 0 (NaN in, NaN out; -inf gives 0), to about two units in the last
 // place, with gradual underflow.  x*log2(e) is formed in two pieces so the
 // rounding of the product does not reach the result; the power of two is applied
@@ -225,7 +252,7 @@ __device__ __forceinline__ void walk_planes(const PlaneWalk<N>& w, uint32_t p, u
 #pragma clang loop unroll(disable)
     for (uint32_t a = w.nlead - 1; a >= 1; --a) {
         const uint32_t d = w.dims[a];
-        const uint32_t q = rem / d;
+        const uint32_t q = fast_div(rem, w.div[a]);
         const uint32_t c = rem - q * d;
         rem = q;
 #pragma unroll

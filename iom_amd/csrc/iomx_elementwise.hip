@@ -165,9 +165,17 @@ struct FlatArgs {
     uint8_t* out;
     uint64_t seg_chunks;
     uint32_t segments;
+    // one or two leading axes, as byte steps per coordinate (0 = broadcast)
+    uint32_t n0, n1;
+    uint64_t step0[3], step1[3];
 };
 
-enum { SHAPE_FLAT = 0, SHAPE_BANDS = 1, SHAPE_PLANES = 2 };
+// FLAT    one dense range.
+// BANDS   one dense range cut into tile-row bands (row-vector operand).
+// AXIS1   one strided leading axis on blockIdx.z, segments on blockIdx.y.
+// AXIS2   two strided leading axes on blockIdx.z / blockIdx.y, one segment.
+// PLANES  anything else: the generic plane walk.
+enum { SHAPE_FLAT = 0, SHAPE_BANDS = 1, SHAPE_AXIS1 = 2, SHAPE_AXIS2 = 3, SHAPE_PLANES = 4 };
 
 template <int DT, int OP, int LM, int RM>
 __device__ __forceinline__ void stream_chunk(const uint8_t* lbase, const uint8_t* rbase,
@@ -198,11 +206,24 @@ __global__ __launch_bounds__(kPlanesBlock) void elementwise_stream_kernel(const 
     if (cb >= a.seg_chunks) return;
     if constexpr (SHAPE == SHAPE_FLAT) {
         stream_chunk<DT, OP, LM, RM>(a.src[0], a.src[1], a.out, cb * 16, 0);
-    } else {
+    } else if constexpr (SHAPE == SHAPE_BANDS) {
         const uint64_t voff = rowvec_offset<DT>(cb);
         for (uint32_t y = blockIdx.y; y < a.segments; y += gridDim.y)
             stream_chunk<DT, OP, LM, RM>(a.src[0], a.src[1], a.out,
                                          ((uint64_t)y * a.seg_chunks + cb) * 16, voff);
+    } else if constexpr (SHAPE == SHAPE_AXIS1) {
+        const uint64_t voff = rowvec_offset<DT>(cb);
+        for (uint32_t z = blockIdx.z; z < a.n0; z += gridDim.z)
+            for (uint32_t y = blockIdx.y; y < a.segments; y += gridDim.y)
+                stream_chunk<DT, OP, LM, RM>(a.src[0] + z * a.step0[0], a.src[1] + z * a.step0[1],
+                                             a.out + z * a.step0[2],
+                                             ((uint64_t)y * a.seg_chunks + cb) * 16, voff);
+    } else {
+        for (uint32_t z = blockIdx.z; z < a.n0; z += gridDim.z)
+            for (uint32_t y = blockIdx.y; y < a.n1; y += gridDim.y)
+                stream_chunk<DT, OP, LM, RM>(a.src[0] + z * a.step0[0] + y * a.step1[0],
+                                             a.src[1] + z * a.step0[1] + y * a.step1[1],
+                                             a.out + z * a.step0[2] + y * a.step1[2], cb * 16, 0);
     }
 }
 
@@ -341,19 +362,42 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
     if (planes) {
         const uint64_t gx = (pa.seg_chunks + kPlanesBlock - 1) / kPlanesBlock;
         if (gx > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
-        const dim3 grid3((uint32_t)gx, pa.segments < 65535u ? pa.segments : 65535u,
-                         pa.planes < 65535u ? pa.planes : 65535u);
-        const uint32_t grid = grid3.x;
-        FlatArgs fa = {{pa.src[0], pa.src[1]}, pa.out, pa.seg_chunks, pa.segments};
-        const bool dense = pa.planes == 1 && pa.walk.nlead == 0;
+        const uint32_t grid = (uint32_t)gx;
+        FlatArgs fa = {};
+        fa.src[0] = pa.src[0];
+        fa.src[1] = pa.src[1];
+        fa.out = pa.out;
+        fa.seg_chunks = pa.seg_chunks;
+        fa.segments = pa.segments;
+        int shape = SHAPE_PLANES;
+        dim3 grid3((uint32_t)gx, pa.segments < 65535u ? pa.segments : 65535u,
+                   pa.planes < 65535u ? pa.planes : 65535u);
+        if (pa.planes == 1 && pa.walk.nlead == 0) {
+            shape = pa.segments == 1 ? SHAPE_FLAT : SHAPE_BANDS;
+        } else if (pa.walk.nlead == 1 || (pa.walk.nlead == 2 && pa.segments == 1)) {
+            shape = pa.walk.nlead == 1 ? SHAPE_AXIS1 : SHAPE_AXIS2;
+            fa.n0 = pa.walk.dims[0];
+            fa.n1 = pa.walk.nlead == 2 ? pa.walk.dims[1] : 1;
+            fa.src[0] += pa.walk.offset[0] * pa.plane_bytes[0];
+            fa.src[1] += pa.walk.offset[1] * pa.plane_bytes[1];
+            fa.out += pa.walk.offset[2] * pa.plane_bytes[2];
+            for (int k = 0; k < 3; ++k) {
+                fa.step0[k] = pa.walk.stride[k][0] * pa.plane_bytes[k];
+                fa.step1[k] = pa.walk.nlead == 2 ? pa.walk.stride[k][1] * pa.plane_bytes[k] : 0;
+            }
+            if (shape == SHAPE_AXIS2) grid3 = dim3((uint32_t)gx, fa.n1 < 65535u ? fa.n1 : 65535u,
+                                                   fa.n0 < 65535u ? fa.n0 : 65535u);
+            else grid3.z = fa.n0 < 65535u ? fa.n0 : 65535u;
+        }
+#define IOMX_STREAM(LMV, RMV, SH)                                                               \
+    hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SH>), grid3,                \
+                       dim3(kPlanesBlock), 0, s, fa)
 #define IOMX_PLANES(LMV, RMV)                                                                   \
     do {                                                                                        \
-        if (dense && pa.segments == 1)                                                          \
-            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SHAPE_FLAT>), grid3, \
-                               dim3(kPlanesBlock), 0, s, fa);                                   \
-        else if (dense)                                                                         \
-            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SHAPE_BANDS>),      \
-                               grid3, dim3(kPlanesBlock), 0, s, fa);                            \
+        if (shape == SHAPE_FLAT) IOMX_STREAM(LMV, RMV, SHAPE_FLAT);                             \
+        else if (shape == SHAPE_BANDS) IOMX_STREAM(LMV, RMV, SHAPE_BANDS);                      \
+        else if (shape == SHAPE_AXIS1) IOMX_STREAM(LMV, RMV, SHAPE_AXIS1);                      \
+        else if (shape == SHAPE_AXIS2) IOMX_STREAM(LMV, RMV, SHAPE_AXIS2);                      \
         else                                                                                    \
             hipLaunchKernelGGL((elementwise_planes_kernel<DT, OP, LMV, RMV>), grid3,            \
                                dim3(kPlanesBlock), 0, s, pa);                                   \
@@ -366,6 +410,7 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
             return IOMX_ERR_INVALID;
         }
 #undef IOMX_PLANES
+#undef IOMX_STREAM
         record_launch(family(OP, true, lm != MODE_FULL || rm != MODE_FULL), grid, kPlanesBlock,
                       gx * pa.segments * pa.planes);
     } else {

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
 #pragma unroll
             for (int j = 0; j < 4; ++j) x[j] = as_f32(kNegInf);
             if (col + 4 <= visible) {
-                const u32x4 v = *reinterpret_cast<const u32x4*>(srow + col);
+                const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(srow + col));
                 x[0] = as_f32(v.x) * a.scale; x[1] = as_f32(v.y) * a.scale;
                 x[2] = as_f32(v.z) * a.scale; x[3] = as_f32(v.w) * a.scale;
             } else if (col < visible) {
@@ -140,7 +140,7 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
             const uint32_t lo = pack_bf16(pr[0], pr[1]);
             const uint32_t hi = pack_bf16(pr[2], pr[3]);
             if (col + 4 <= a.pl.columns) {
-                *reinterpret_cast<u32x2*>(prow + col) = u32x2{lo, hi};
+                __builtin_nontemporal_store(u32x2{lo, hi}, reinterpret_cast<u32x2*>(prow + col));
             } else {
                 const uint32_t words[2] = {lo, hi};
                 for (int j = 0; j < 4; ++j)
