@@ -1,0 +1,656 @@
+// MI355X backend for IOM: iom::Device / iom::Tensor / iom::RawWorkspace /
+// iom::DeviceOps subclasses behind the factory iom::make_rocm_device
+// (include/iom/rocm/device.hpp:22-24), a drop-in for the reference's ROCm
+// backend on the memory-bound operations: add / mul / sub, copy, rmsnorm, silu
+// and the host transfers.  Everything else keeps the common default
+// (UnsupportedOperation, OID -2).
+//
+// This translation unit is plain C++20: it includes no HIP header and reaches
+// the GPU only through the C ABI of libiomx (include/iomx.h).
+//
+// Design (not a port of src/rocm or src/shared/gpu_queue*):
+//   * One device arena (a single iomx_malloc at setup, none afterwards), carved
+//     by the reference's ListAllocator at 256-byte alignment.  Kernel
+//     descriptors travel as kernel arguments, so there is no metadata arena and
+//     no per-operation upload.
+//   * A queue is one non-blocking stream, C completion events created eagerly,
+//     and one completion thread.  The admission dispatch itself launches the
+//     kernel and records an event (on whichever thread the common FIFO pump runs:
+//     the submitting thread or the completion thread); the completion thread
+//     waits for events in submission order, releases the registry entries and
+//     completes the sequence.  The common layer already bounds executing work to
+//     C, so an event is always free when a dispatch runs.
+//   * Host transfers are synchronous, serialised per device, and stage through
+//     the caller's raw workspace: host -> workspace, then the scatter kernel (or
+//     the gather kernel, then workspace -> host).
+#include <array>
+#include <condition_variable>
+#include <cstddef>
+#include <cstdint>
+#include <deque>
+#include <exception>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <new>
+#include <span>
+#include <stdexcept>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "iom/alloc.hpp"
+#include "iom/detail/gpu_arena_config.hpp"
+#include "iom/detail/outstanding_work_registry.hpp"
+#include "iom/device.hpp"
+#include "iom/gpu_algorithm.hpp"
+#include "iom/iom.hpp"
+#include "iom/rocm/device.hpp"
+#include "iom/tensor.hpp"
+#include "src/iom_internal.hpp"  // iom::detail::UnsupportedOperation, leaf_bits
+
+#include "iomx.h"
+
+namespace iom {
+namespace {
+
+constexpr std::size_t kArenaAlignment = 256;
+
+[[noreturn]] void throw_status(int status, const char* what) {
+    std::string message(what);
+    message += ": ";
+    message += iomx_error_string(status);
+    if (status == IOMX_ERR_INVALID) throw std::invalid_argument(message);
+    if (status == IOMX_ERR_OVERFLOW) throw std::overflow_error(message);
+    if (status == IOMX_ERR_UNSUPPORTED) throw detail::UnsupportedOperation();
+    throw std::runtime_error(message);
+}
+
+void check(int status, const char* what) {
+    if (status != IOMX_OK) throw_status(status, what);
+}
+
+// The leaves this backend stores and moves: every 16- and 32-bit leaf.  Their
+// payload is copied as raw bits, so one code per width serves copy and transfer.
+int transfer_code(DataType type) {
+    switch (detail::leaf_bits(type)) {
+        case 16: return IOMX_DT_BF16;
+        case 32: return IOMX_DT_I32;
+        default: return -1;
+    }
+}
+
+// Arithmetic leaves of the binary operations and of rmsnorm / silu.
+int binary_code(DataType type) {
+    switch (type) {
+        case DataType::I32: return IOMX_DT_I32;
+        case DataType::U32: return IOMX_DT_U32;
+        case DataType::F32: return IOMX_DT_F32;
+        case DataType::BF16: return IOMX_DT_BF16;
+        default: return -1;
+    }
+}
+
+int float_code(DataType type) {
+    if (type == DataType::F32) return IOMX_DT_F32;
+    if (type == DataType::BF16) return IOMX_DT_BF16;
+    return -1;
+}
+
+constexpr std::array<DataType, 7> kStoredLeaves = {
+        DataType::I16, DataType::U16, DataType::I32, DataType::U32,
+        DataType::F16, DataType::BF16, DataType::F32};
+
+iomx_view make_view(void* base, std::span<const std::size_t> dims, std::size_t plane_offset,
+                    std::span<const std::size_t> plane_strides) {
+    iomx_view v{};
+    v.base = base;
+    v.rank = static_cast<std::uint32_t>(dims.size());
+    for (std::size_t i = 0; i < dims.size(); ++i) v.dims[i] = dims[i];
+    v.plane_offset = plane_offset;
+    for (std::size_t i = 0; i + 2 < dims.size() && i < plane_strides.size(); ++i)
+        v.plane_strides[i] = plane_strides[i];
+    return v;
+}
+
+iomx_view make_view(const TensorView& view) {
+    return make_view(const_cast<void*>(view.native_handle()), view.spec().shape.dimensions(),
+                     view.plane_offset(), view.plane_strides());
+}
+
+class Mi355xDevice;
+
+// ---------------------------------------------------------------------------
+// Device
+// ---------------------------------------------------------------------------
+
+class Mi355xDevice final : public Device {
+public:
+    Mi355xDevice(std::uint32_t ordinal, std::size_t arena_bytes, QueueConfig queue_config)
+            : Device(queue_config), ordinal_(ordinal), arena_bytes_(arena_bytes) {
+        int count = 0;
+        if (iomx_device_count(&count) != IOMX_OK || ordinal >= static_cast<std::uint32_t>(count))
+            throw std::invalid_argument("MI355X device ordinal does not exist");
+        check(iomx_set_device(static_cast<int>(ordinal_)), "set device");
+        if (iomx_malloc(&arena_, arena_bytes_) != IOMX_OK || arena_ == nullptr)
+            throw std::bad_alloc();
+        try {
+            allocator_ = std::make_unique<ListAllocator>(arena_, arena_bytes_, kArenaAlignment);
+            check(iomx_stream_create(&transfer_stream_), "transfer stream");
+        } catch (...) {
+            (void)iomx_free(arena_);
+            throw;
+        }
+    }
+
+    ~Mi355xDevice() override {
+        (void)iomx_set_device(static_cast<int>(ordinal_));
+        if (transfer_stream_ != nullptr) {
+            (void)iomx_stream_synchronize(transfer_stream_);
+            (void)iomx_stream_destroy(transfer_stream_);
+        }
+        // Quarantined storage is returned to the allocator's host-side books when
+        // the registry state is destroyed (after this body); the device range
+        // itself can go now.
+        (void)iomx_device_synchronize();
+        (void)iomx_free(arena_);
+    }
+
+    [[nodiscard]] BackendKind backend_kind() const noexcept override { return BackendKind::ROCM; }
+    [[nodiscard]] std::uint32_t backend_device() const noexcept override { return ordinal_; }
+    [[nodiscard]] std::span<const DataType> supported_data_types() const noexcept override {
+        return kStoredLeaves;
+    }
+
+    [[nodiscard]] std::unique_ptr<Tensor> create_tensor(const TensorSpec& spec) override;
+    [[nodiscard]] std::unique_ptr<RawWorkspace> create_workspace(std::size_t bytes) override;
+    [[nodiscard]] std::unique_ptr<DeviceOps> create_ops() override;
+
+    [[nodiscard]] detail::RegistryState& registry_state() noexcept { return registry_state_; }
+    [[nodiscard]] int ordinal() const noexcept { return static_cast<int>(ordinal_); }
+
+    // Arena suballocation; exhaustion (including fragmentation) is std::bad_alloc.
+    [[nodiscard]] void* allocate(std::size_t bytes) {
+        std::lock_guard<std::mutex> lock(arena_mutex_);
+        void* address = allocator_->alloc(bytes);
+        if (address == nullptr) throw std::bad_alloc();
+        return address;
+    }
+    void release(void* address) noexcept {
+        if (address == nullptr) return;
+        std::lock_guard<std::mutex> lock(arena_mutex_);
+        try { allocator_->free(address); } catch (...) {}
+    }
+    [[nodiscard]] Allocator& data_allocator() noexcept { return *guarded_allocator_; }
+
+    // Host transfers: one at a time per device, never waiting on any queue.
+    void transfer(const TensorView& view, RawWorkspaceView workspace,
+                  std::span<const std::byte> source, std::span<std::byte> destination,
+                  bool from_host) {
+        const WorkspaceRequirements need = view.copy_from_host_workspace_requirements();
+        const std::array<TensorView, 1> operands{view};
+        const RawWorkspaceView checked = detail::WorkspaceValidation::validated(
+                *this, workspace, need.bytes, need.alignment, operands);
+        void* staging = detail::WorkspaceValidation::address(checked);
+        const int code = transfer_code(view.spec().data_type);
+        if (code < 0) throw detail::UnsupportedOperation();
+        const std::size_t nbytes = view.spec().logical_nbytes();
+        const iomx_view v = make_view(view);
+        std::lock_guard<std::mutex> lock(transfer_mutex_);
+        if (transfer_poisoned_) throw std::bad_alloc();
+        try {
+            check(iomx_set_device(ordinal()), "set device");
+            if (from_host) {
+                check(iomx_memcpy_h2d(staging, source.data(), nbytes), "host to staging");
+                check(iomx_launch_scatter(code, &v, staging, transfer_stream_), "scatter");
+                check(iomx_stream_synchronize(transfer_stream_), "scatter completion");
+            } else {
+                check(iomx_launch_gather(code, &v, staging, transfer_stream_), "gather");
+                check(iomx_stream_synchronize(transfer_stream_), "gather completion");
+                check(iomx_memcpy_d2h(destination.data(), staging, nbytes), "staging to host");
+            }
+        } catch (...) {
+            transfer_poisoned_ = true;  // a failed transfer leaves the stream's state unknown
+            throw;
+        }
+    }
+
+    void zero_fill(void* address, std::size_t bytes) {
+        std::lock_guard<std::mutex> lock(transfer_mutex_);
+        check(iomx_set_device(ordinal()), "set device");
+        check(iomx_fill_async(address, 0, bytes, transfer_stream_), "zero fill");
+        check(iomx_stream_synchronize(transfer_stream_), "zero fill completion");
+    }
+
+private:
+    // Allocator facade whose free() takes the arena lock: quarantined storage is
+    // released through it from whatever thread drains the quarantine.
+    class GuardedAllocator final : public Allocator {
+    public:
+        explicit GuardedAllocator(Mi355xDevice& device) : device_(device) {}
+        void* alloc(std::size_t bytes) override { return device_.allocate(bytes); }
+        void free(void* address) override { device_.release(address); }
+        void reset() override {}
+    private:
+        Mi355xDevice& device_;
+    };
+
+    std::uint32_t ordinal_;
+    std::size_t arena_bytes_;
+    void* arena_ = nullptr;
+    std::mutex arena_mutex_;
+    std::unique_ptr<ListAllocator> allocator_;
+    std::unique_ptr<GuardedAllocator> guarded_allocator_ = std::make_unique<GuardedAllocator>(*this);
+    iomx_stream_t transfer_stream_ = nullptr;
+    std::mutex transfer_mutex_;
+    bool transfer_poisoned_ = false;
+    // Destroyed first (declared last): draining its quarantine uses the allocator.
+    detail::RegistryState registry_state_;
+};
+
+// ---------------------------------------------------------------------------
+// Tensor and workspace owners
+// ---------------------------------------------------------------------------
+
+class Mi355xTensor final : public Tensor {
+public:
+    Mi355xTensor(const TensorSpec& spec, Mi355xDevice& device)
+            : Tensor(spec, device), device_(device) {
+        if (transfer_code(spec.data_type) < 0) throw detail::UnsupportedOperation();
+        bytes_ = view().spec().tiled_storage_nbytes();
+        address_ = device_.allocate(bytes_);
+        try {
+            device_.zero_fill(address_, bytes_);
+        } catch (...) {
+            device_.release(address_);
+            throw;
+        }
+    }
+
+    ~Mi355xTensor() noexcept override {
+        if (address_ == nullptr) return;
+        void* address = address_;
+        // Storage with unproven outstanding work is parked in the quarantine and
+        // returned to the arena only when the device goes away
+        // (include/iom/detail/outstanding_work_registry_core.hpp:235-275).
+        detail::release_or_quarantine(
+                device_.registry_state().registry, address,
+                [this, address] {
+                    try {
+                        device_.registry_state().quarantine
+                                .emplace<detail::AllocatorCleanupAction>(
+                                        device_.data_allocator(), address, bytes_);
+                    } catch (...) {
+                    }
+                    address_ = nullptr;
+                },
+                [this, address] {
+                    device_.release(address);
+                    address_ = nullptr;
+                });
+    }
+
+private:
+    [[nodiscard]] void* storage_handle() noexcept override { return address_; }
+    [[nodiscard]] WorkspaceRequirements host_transfer_workspace_requirements(
+            std::size_t checked_logical_nbytes) const override {
+        return {gpu_algorithm::compute_staging_size(checked_logical_nbytes), 32};
+    }
+    void region_from_host(const TensorView& destination, std::span<const std::byte> source,
+                          RawWorkspaceView workspace) override {
+        device_.transfer(destination, workspace, source, {}, true);
+    }
+    void region_to_host(const TensorView& source, std::span<std::byte> destination,
+                        RawWorkspaceView workspace) const override {
+        device_.transfer(source, workspace, {}, destination, false);
+    }
+
+    Mi355xDevice& device_;
+    void* address_ = nullptr;
+    std::size_t bytes_ = 0;
+};
+
+class Mi355xWorkspace final : public RawWorkspace {
+public:
+    Mi355xWorkspace(Mi355xDevice& device, std::size_t bytes)
+            : RawWorkspace(device, bytes), device_(device) {
+        if (bytes != 0) address_ = device_.allocate(bytes);
+    }
+    ~Mi355xWorkspace() noexcept override { device_.release(address_); }
+
+private:
+    [[nodiscard]] void* workspace_address() const noexcept override { return address_; }
+    Mi355xDevice& device_;
+    void* address_ = nullptr;
+};
+
+// ---------------------------------------------------------------------------
+// Queue
+// ---------------------------------------------------------------------------
+
+class Mi355xQueue final : public DeviceOps {
+public:
+    explicit Mi355xQueue(Mi355xDevice& device)
+            : DeviceOps(device), device_(device),
+              registry_queue_id_(detail::allocate_queue_id(device.registry_state())) {
+        const std::size_t capacity = device.queue_config().max_in_flight_per_queue;
+        try {
+            check(iomx_set_device(device_.ordinal()), "set device");
+            events_.reserve(capacity);
+            for (std::size_t i = 0; i < capacity; ++i) {
+                iomx_event_t event = nullptr;
+                check(iomx_event_create(&event, 0), "completion event");
+                events_.push_back(event);
+                free_events_.push_back(event);
+            }
+            check(iomx_stream_create(&stream_), "queue stream");
+            completer_ = std::thread([this] { run_completer(); });
+        } catch (...) {
+            destroy_native();
+            throw;
+        }
+    }
+
+    ~Mi355xQueue() override {
+        // Stop accepting, fail what never started, then let the completion thread
+        // finish everything that was launched before the native objects go away.
+        close_and_drain();
+        {
+            std::unique_lock<std::mutex> lock(mutex_);
+            shutdown_ = true;
+        }
+        cv_.notify_all();
+        if (completer_.joinable()) completer_.join();
+        close_and_drain();
+        (void)iomx_set_device(device_.ordinal());
+        if (stream_ != nullptr) (void)iomx_stream_synchronize(stream_);
+        destroy_native();
+        device_.registry_state().registry.invalidate_entries_for_queue(registry_queue_id_);
+    }
+
+    [[nodiscard]] std::string_view backend_label() const noexcept override { return "MI355X"; }
+
+private:
+    using Finish = std::function<void(bool failed)>;
+
+    struct InFlight {
+        std::uint64_t sequence = 0;
+        iomx_event_t event = nullptr;
+        std::exception_ptr failure;
+        Finish finish;
+    };
+
+    static detail::FenceResult fence_pending(const detail::Fence&) noexcept {
+        return detail::FenceResult::pending();
+    }
+    [[nodiscard]] static detail::Fence pending_fence() noexcept {
+        detail::Fence fence;
+        fence.invoke = &fence_pending;
+        return fence;
+    }
+
+    void destroy_native() noexcept {
+        for (iomx_event_t event : events_) (void)iomx_event_destroy(event);
+        events_.clear();
+        free_events_.clear();
+        if (stream_ != nullptr) (void)iomx_stream_destroy(stream_);
+        stream_ = nullptr;
+    }
+
+    // Runs inside the common admission dispatch: launch on the queue stream,
+    // record the completion event, hand the rest to the completion thread.
+    // Throws only before anything was launched.
+    template <typename Launch>
+    void start(std::uint64_t sequence, Launch&& launch, Finish finish) {
+        iomx_event_t event = nullptr;
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            if (shutdown_) throw std::logic_error("MI355X queue is shut down");
+            if (free_events_.empty()) throw detail::AdmissionResourceUnavailable();
+            event = free_events_.back();
+            free_events_.pop_back();
+        }
+        InFlight item;
+        item.sequence = sequence;
+        item.event = event;
+        item.finish = std::move(finish);
+        int status = iomx_set_device(device_.ordinal());
+        if (status == IOMX_OK) status = launch(stream_);
+        if (status == IOMX_OK) status = iomx_event_record(event, stream_);
+        if (status != IOMX_OK) {
+            try { throw_status(status, "MI355X kernel submission"); }
+            catch (...) { item.failure = std::current_exception(); }
+        }
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            in_flight_.push_back(std::move(item));
+        }
+        cv_.notify_all();
+    }
+
+    void run_completer() noexcept {
+        (void)iomx_set_device(device_.ordinal());
+        for (;;) {
+            InFlight item;
+            {
+                std::unique_lock<std::mutex> lock(mutex_);
+                cv_.wait(lock, [this] { return shutdown_ || !in_flight_.empty(); });
+                if (in_flight_.empty()) return;
+                item = std::move(in_flight_.front());
+                in_flight_.pop_front();
+            }
+            if (!item.failure) {
+                const int status = iomx_event_synchronize(item.event);
+                if (status != IOMX_OK) {
+                    try { throw_status(status, "MI355X kernel completion"); }
+                    catch (...) { item.failure = std::current_exception(); }
+                }
+            } else {
+                // the stream may still hold earlier work: keep completion in order
+                (void)iomx_stream_synchronize(stream_);
+            }
+            {
+                std::lock_guard<std::mutex> lock(mutex_);
+                free_events_.push_back(item.event);
+            }
+            try { if (item.finish) item.finish(static_cast<bool>(item.failure)); } catch (...) {}
+            try { complete(item.sequence, std::move(item.failure)); } catch (...) {}
+        }
+    }
+
+    // ---- hooks ----------------------------------------------------------------
+
+    oid copy_impl(const TensorView& source, TensorView& destination) override {
+        const int code = transfer_code(source.spec().data_type);
+        if (code < 0) throw detail::UnsupportedOperation();
+        std::lock_guard<std::mutex> order(submission_mutex_);
+        return submit_copy(
+                source, destination, device_.registry_state(), registry_queue_id_, pending_fence(),
+                [this, code](std::uint64_t sequence, const CopyRequest& captured,
+                             detail::EntryRegistration entries) {
+                    auto& registry = device_.registry_state().registry;
+                    try {
+                        start(sequence,
+                              [&captured, code](iomx_stream_t stream) {
+                                  if (captured.no_op) return static_cast<int>(IOMX_OK);
+                                  const iomx_view src = make_view(
+                                          captured.source.native_handle,
+                                          captured.source.spec.shape.dimensions(),
+                                          captured.source.plane_offset, captured.source.plane_strides);
+                                  const iomx_view dst = make_view(
+                                          captured.destination.native_handle,
+                                          captured.destination.spec.shape.dimensions(),
+                                          captured.destination.plane_offset,
+                                          captured.destination.plane_strides);
+                                  return iomx_launch_copy(code, &src, &dst, stream);
+                              },
+                              [&registry, entries](bool failed) {
+                                  const detail::SequenceOutcome outcome{
+                                          entries.source, entries.destination, nullptr, true};
+                                  (void)detail::release_or_invalidate_entries(
+                                          registry, outcome, failed, true);
+                              });
+                    } catch (...) {
+                        registry.remove_entry_if_present(
+                                entries.source, captured.source.native_handle);
+                        registry.remove_entry_if_present(
+                                entries.destination, captured.destination.native_handle);
+                        throw;
+                    }
+                });
+    }
+
+    oid binary_impl(const BinaryRequest& request) override {
+        const int code = binary_code(request.out.spec.data_type);
+        if (code < 0 || request.operation == BinaryOperation::Div)
+            throw detail::UnsupportedOperation();
+        int op = IOMX_OP_ADD;
+        if (request.operation == BinaryOperation::Mul) op = IOMX_OP_MUL;
+        if (request.operation == BinaryOperation::Sub) op = IOMX_OP_SUB;
+        std::lock_guard<std::mutex> order(submission_mutex_);
+        return submit_binary(
+                request, device_.registry_state(), registry_queue_id_, pending_fence(),
+                [this, code, op](std::uint64_t sequence, const BinaryRequest& captured,
+                                 detail::BinaryEntryRegistration entries) {
+                    auto& state = device_.registry_state();
+                    const detail::WorkspaceLease lease = captured.workspace_lease;
+                    try {
+                        start(sequence,
+                              [&captured, code, op](iomx_stream_t stream) {
+                                  const auto view_of = [](const BinaryViewSnapshot& s) {
+                                      return make_view(s.native_handle, s.spec.shape.dimensions(),
+                                                       s.plane_offset, s.plane_strides);
+                                  };
+                                  const iomx_view lhs = view_of(captured.lhs);
+                                  const iomx_view rhs = view_of(captured.rhs);
+                                  const iomx_view out = view_of(captured.out);
+                                  return iomx_launch_binary(op, code, &lhs, &rhs, &out, stream);
+                              },
+                              [&state, entries, lease](bool failed) {
+                                  (void)detail::release_or_invalidate_binary_entries(
+                                          state.registry, entries, failed, true);
+                                  detail::complete_workspace_lease(state, lease, true);
+                              });
+                    } catch (...) {
+                        state.registry.remove_entries(std::span<const detail::EntryId>(
+                                entries.entries.data(), entries.count));
+                        detail::complete_workspace_lease(state, lease, true);
+                        throw;
+                    }
+                });
+    }
+
+    [[nodiscard]] bool rmsnorm_supported(DataType data_type) const override {
+        return float_code(data_type) >= 0;
+    }
+
+    oid rmsnorm_impl(const RmsnormRequest& request) override {
+        const int code = float_code(request.x.spec.data_type);
+        if (code < 0) throw detail::UnsupportedOperation();
+        std::lock_guard<std::mutex> order(submission_mutex_);
+        return submit_rmsnorm(
+                request, device_.registry_state(), registry_queue_id_, pending_fence(),
+                [this, code](std::uint64_t sequence, const RmsnormRequest& captured,
+                             detail::BinaryEntryRegistration entries) {
+                    auto& registry = device_.registry_state().registry;
+                    try {
+                        start(sequence,
+                              [&captured, code](iomx_stream_t stream) {
+                                  const auto view_of = [](const CopyViewSnapshot& s) {
+                                      return make_view(s.native_handle, s.spec.shape.dimensions(),
+                                                       s.plane_offset, s.plane_strides);
+                                  };
+                                  const iomx_view x = view_of(captured.x);
+                                  const iomx_view scale = view_of(captured.scale);
+                                  const iomx_view out = view_of(captured.out);
+                                  return iomx_launch_rmsnorm(code, &x, &scale, &out,
+                                                             captured.epsilon, stream);
+                              },
+                              [&registry, entries](bool failed) {
+                                  (void)detail::release_or_invalidate_binary_entries(
+                                          registry, entries, failed, true);
+                              });
+                    } catch (...) {
+                        registry.remove_entries(std::span<const detail::EntryId>(
+                                entries.entries.data(), entries.count));
+                        throw;
+                    }
+                });
+    }
+
+    [[nodiscard]] WorkspaceRequirements silu_workspace_requirements_impl(
+            const SiLURequest& request) override {
+        if (float_code(request.x.data_type) < 0) throw detail::UnsupportedOperation();
+        return {0, 1};
+    }
+
+    oid silu_impl(const SiLURequest& request) override {
+        const int code = float_code(request.x.data_type);
+        if (code < 0) throw detail::UnsupportedOperation();
+        std::lock_guard<std::mutex> order(submission_mutex_);
+        return submit_silu(
+                request, device_.registry_state(), registry_queue_id_, pending_fence(),
+                [this, code](std::uint64_t sequence, const SiLURequest& captured,
+                             detail::BinaryEntryRegistration entries) {
+                    auto& registry = device_.registry_state().registry;
+                    try {
+                        start(sequence,
+                              [&captured, code](iomx_stream_t stream) {
+                                  const auto view_of = [](const SiLUViewSnapshot& s) {
+                                      return make_view(s.native_handle, s.shape_dimensions(),
+                                                       s.plane_offset, s.leading_plane_strides());
+                                  };
+                                  const iomx_view x = view_of(captured.x);
+                                  const iomx_view y = view_of(captured.y);
+                                  return iomx_launch_silu(code, &x, &y, stream);
+                              },
+                              [&registry, entries](bool failed) {
+                                  (void)detail::release_or_invalidate_binary_entries(
+                                          registry, entries, failed, true);
+                              });
+                    } catch (...) {
+                        registry.remove_entries(std::span<const detail::EntryId>(
+                                entries.entries.data(), entries.count));
+                        throw;
+                    }
+                });
+    }
+
+    Mi355xDevice& device_;
+    detail::QueueId registry_queue_id_;
+    std::mutex submission_mutex_;
+    iomx_stream_t stream_ = nullptr;
+    std::vector<iomx_event_t> events_;
+    std::mutex mutex_;
+    std::condition_variable cv_;
+    std::vector<iomx_event_t> free_events_;
+    std::deque<InFlight> in_flight_;
+    bool shutdown_ = false;
+    std::thread completer_;
+};
+
+std::unique_ptr<Tensor> Mi355xDevice::create_tensor(const TensorSpec& spec) {
+    return std::make_unique<Mi355xTensor>(spec, *this);
+}
+
+std::unique_ptr<RawWorkspace> Mi355xDevice::create_workspace(std::size_t bytes) {
+    return std::make_unique<Mi355xWorkspace>(*this, bytes);
+}
+
+std::unique_ptr<DeviceOps> Mi355xDevice::create_ops() {
+    return std::make_unique<Mi355xQueue>(*this);
+}
+
+}  // namespace
+
+// include/iom/rocm/device.hpp:22-24.  Configuration errors are reported before
+// any native effect (include/iom/detail/gpu_arena_config.hpp:18-53).
+std::unique_ptr<Device> make_rocm_device(std::uint32_t device_ordinal,
+                                         DeviceMemoryConfig memory_config,
+                                         QueueConfig queue_config) {
+    const std::size_t arena = detail::valid_tensor_arena_bytes(memory_config.tensor_arena_bytes);
+    (void)detail::standard_gpu_metadata_bytes(queue_config.max_in_flight_per_queue);
+    return std::make_unique<Mi355xDevice>(device_ordinal, arena, queue_config);
+}
+
+}  // namespace iom

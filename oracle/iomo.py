@@ -23,8 +23,10 @@ DT_I32, DT_U32, DT_BF16, DT_F32 = 9, 10, 20, 21
 OP_ADD, OP_MUL, OP_SUB = 0, 1, 2
 TILE = 16
 
-NP_OF = {DT_I32: np.uint32, DT_U32: np.uint32, DT_BF16: np.uint16, DT_F32: np.uint32}
-"""Raw-bit numpy carrier of every leaf (all arithmetic is on bit patterns)."""
+NP_OF = {DT_I32: np.uint32, DT_U32: np.uint32, DT_BF16: np.uint16, DT_F32: np.uint32,
+         5: np.uint8, 6: np.uint8, 7: np.uint16, 8: np.uint16, 19: np.uint16}
+"""Raw-bit numpy carrier of every leaf (all arithmetic is on bit patterns); the
+8- and 16-bit integer leaves and F16 appear only as opaque payloads of copies."""
 
 
 def leaf_bytes(dtype: int) -> int:
@@ -510,3 +512,30 @@ def ref_backend(max_in_flight: int = 16) -> IomBackend:
     if _ref_lib is None:
         _ref_lib = bind_iomc(_load(REF_PATH))
     return IomBackend(_ref_lib, _ref_lib.iomc_cpu_device_create(max_in_flight))
+
+
+MI355X_SHIM_PATH = os.path.join(HERE, "_ref", "libiom_mi355x_shim.so")
+_mi355x_lib: Optional[C.CDLL] = None
+
+
+def mi355x_available() -> bool:
+    return os.path.exists(MI355X_SHIM_PATH)
+
+
+def mi355x_lib() -> C.CDLL:
+    """The handle API over this repository's C++ backend (iom::make_rocm_device) and,
+    in the same process and over the same libiom core, the reference CPU backend."""
+    global _mi355x_lib
+    if _mi355x_lib is None:
+        _mi355x_lib = bind_iomc(_load(MI355X_SHIM_PATH))
+    return _mi355x_lib
+
+
+def mi355x_backend(arena_bytes: int = 1 << 30, max_in_flight: int = 16, ordinal: int = 0) -> IomBackend:
+    l = mi355x_lib()
+    return IomBackend(l, l.iomc_mi355x_device_create(ordinal, arena_bytes, max_in_flight))
+
+
+def cpu_backend_beside_mi355x(max_in_flight: int = 16) -> IomBackend:
+    l = mi355x_lib()
+    return IomBackend(l, l.iomc_cpu_device_create(max_in_flight))

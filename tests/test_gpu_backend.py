@@ -1,0 +1,204 @@
+"""The C++ backend (iom::make_rocm_device of iom_amd/host) driven through IOM's own
+Device / TensorView / DeviceOps API next to the reference CPU backend in one
+process, as the reference's conformance drivers do
+(test/backend/backend_conformance_common.hpp:310: reference + candidate devices).
+
+Skipped where the backend library was not built (it needs the reference headers)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import datagen
+import iomo
+from iomo import DT_BF16, DT_F32, DT_I32, OP_ADD, OP_MUL, OP_SUB
+
+pytestmark = pytest.mark.gpu
+
+BITS = {DT_BF16: 16, DT_F32: 32, DT_I32: 32, 19: 16, 7: 16}
+
+
+@pytest.fixture(scope="module")
+def devices():
+    if not iomo.mi355x_available():
+        pytest.skip("oracle/_ref/libiom_mi355x_shim.so not built (needs the reference headers)")
+    gpu = iomo.mi355x_backend(arena_bytes=1 << 30, max_in_flight=4)
+    cpu = iomo.cpu_backend_beside_mi355x()
+    yield cpu, gpu
+    gpu.close()
+    cpu.close()
+
+
+def apply(view, steps):
+    for name, args in steps:
+        view = getattr(view, name)(*args)
+    return view
+
+
+def both(devices, dtype, dims, salt=None, values=None):
+    cpu, gpu = devices
+    if salt is not None:
+        values = datagen.pattern_bits(BITS[dtype], int(np.prod(dims)), salt).reshape(dims)
+    out = []
+    for dev in (cpu, gpu):
+        t = dev.tensor(dtype, dims)
+        if values is not None:
+            t.view().from_host(values)
+        out.append(t)
+    return out
+
+
+def close(*tensors):
+    for t in tensors:
+        t.close()
+
+
+def test_device_identity(devices):
+    cpu, gpu = devices
+    assert gpu.l.iomc_device_backend_kind(gpu.dev) == 2      # BackendKind::ROCM
+    assert cpu.l.iomc_device_backend_kind(cpu.dev) == 0
+
+
+CASES = [
+    ((2, 17, 33), [], (2, 17, 33), [], (2, 17, 33), []),
+    ((2, 1, 33), [], (1, 17, 1), [], (2, 17, 33), []),
+    ((3, 32, 48), [], (1, 48), [], (3, 32, 48), []),
+    ((6, 20, 35), [("slice", (0, 1, 3, 2))], (3, 20, 35), [], (3, 20, 35), []),
+    ((4, 3, 16, 32), [("permute", ([1, 0],))], (3, 4, 16, 32), [], (3, 4, 16, 32), []),
+    ((4, 3, 16, 32), [("select", (0, 2))], (1, 16, 32), [], (5, 3, 16, 32), [("select", (0, 4))]),
+    ((8, 64, 256), [], (8, 64, 256), [], (8, 64, 256), []),
+]
+
+
+@pytest.mark.parametrize("dtype", [DT_I32, DT_F32, DT_BF16])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("case", range(len(CASES)))
+def test_binary_matches_reference_cpu_backend_bit_for_bit(devices, dtype, op, case):
+    cpu, gpu = devices
+    ld, ls, rd, rs, od, os_ = CASES[case]
+    cl, gl = both(devices, dtype, ld, salt=0x100 + case)
+    cr, gr = both(devices, dtype, rd, salt=0x200 + case)
+    co, go = both(devices, dtype, od, salt=0x300 + case)
+    tc = cpu.binary(op, apply(cl.view(), ls), apply(cr.view(), rs), apply(co.view(), os_))
+    tg = gpu.binary(op, apply(gl.view(), ls), apply(gr.view(), rs), apply(go.view(), os_))
+    assert tc > 0 and tg > 0, (tc, tg, gpu.error())
+    assert np.array_equal(co.view().to_host(), go.view().to_host())
+    close(cl, gl, cr, gr, co, go)
+
+
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F32])
+@pytest.mark.parametrize("dims,steps", [((17, 33), []), ((40, 2048), []),
+                                        ((2, 3, 17, 64), [("permute", ([1, 0],))])])
+def test_rmsnorm_and_silu_within_the_bar(devices, dtype, dims, steps):
+    cpu, gpu = devices
+    n = int(np.prod(dims))
+    x = datagen.normal_f32(n, 0, 1, 5)
+    w = datagen.uniform_f32(dims[-1], 0.5, 1.5, 6)
+    xl = (datagen.bf16_rne(x) if dtype == DT_BF16 else x.view(np.uint32)).reshape(dims)
+    wl = (datagen.bf16_rne(w) if dtype == DT_BF16 else w.view(np.uint32)).reshape(1, dims[-1])
+    cx, gx = both(devices, dtype, dims, values=xl)
+    cw, gw = both(devices, dtype, (1, dims[-1]), values=wl)
+    vdims = apply(cx.view(), steps).describe()[0]
+    co, go = both(devices, dtype, vdims)
+    assert cpu.rmsnorm(apply(cx.view(), steps), cw.view(), co.view(), 1e-5) > 0
+    assert gpu.rmsnorm(apply(gx.view(), steps), gw.view(), go.view(), 1e-5) > 0, gpu.error()
+    a, b = co.view().to_host(), go.view().to_host()
+    if dtype == DT_BF16:
+        assert np.abs(a.astype(np.int64) - b.astype(np.int64)).max() <= 1      # 1 BF16 ulp
+    else:
+        fa, fb = a.view(np.float32).astype(np.float64), b.view(np.float32).astype(np.float64)
+        assert np.max(np.abs(fa - fb) / np.maximum(np.abs(fa), 1e-30)) <= 1e-5
+    cs, gs = both(devices, dtype, vdims)
+    assert cpu.silu(apply(cx.view(), steps), cs.view()) > 0
+    assert gpu.silu(apply(gx.view(), steps), gs.view()) > 0, gpu.error()
+    a, b = cs.view().to_host().astype(np.int64), gs.view().to_host().astype(np.int64)
+    assert np.abs(a - b).max() <= (1 if dtype == DT_BF16 else 8)
+    close(cx, gx, cw, gw, co, go, cs, gs)
+
+
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F32, DT_I32, 19, 7])   # 19 = F16, 7 = I16: moved as bits
+def test_copy_and_host_transfer_round_trip(devices, dtype):
+    cpu, gpu = devices
+    dims = (6, 20, 35)
+    vals = datagen.pattern_bits(BITS[dtype], int(np.prod(dims)), 77).reshape(dims)
+    cs, gs = both(devices, dtype, dims, values=vals)
+    assert np.array_equal(gs.view().to_host(), vals)
+    cd, gd = both(devices, dtype, (3, 20, 35), salt=78)
+    assert cpu.copy(cs.view().slice(0, 1, 3, 2), cd.view()) > 0
+    assert gpu.copy(gs.view().slice(0, 1, 3, 2), gd.view()) > 0, gpu.error()
+    assert np.array_equal(cd.view().to_host(), gd.view().to_host())
+    close(cs, gs, cd, gd)
+
+
+def test_error_classes_match_the_reference(devices):
+    cpu, gpu = devices
+    for dev in (cpu, gpu):
+        a = dev.tensor(DT_F32, (2, 16, 16))
+        b = dev.tensor(DT_F32, (3, 16, 16))
+        o = dev.tensor(DT_F32, (2, 16, 16))
+        assert dev.binary(OP_ADD, a.view(), b.view(), o.view()) == -1        # InvalidArgument
+        assert dev.binary(OP_ADD, a.view(), a.view(), b.view()) == -1
+        w = dev.tensor(DT_F32, (1, 16))
+        assert dev.rmsnorm(a.view(), w.view(), a.view(), 1e-5) == -1         # output aliases input
+        assert dev.rmsnorm(a.view(), w.view(), o.view(), -1.0) == -1
+        assert dev.wait(12345) != 0                                           # foreign / unsubmitted token
+        close(a, b, o, w)
+    # leaves outside this backend's arithmetic scope are Unsupported, not wrong
+    h = gpu.tensor(19, (2, 16, 16))
+    assert gpu.binary(OP_ADD, h.view(), h.view(), h.view()) == -2
+    ho = gpu.tensor(19, (2, 16, 16))
+    assert gpu.silu(h.view(), ho.view()) == -2
+    close(h, ho)
+    with pytest.raises(RuntimeError):
+        gpu.tensor(5, (2, 16, 16))                                            # I8 storage is not offered
+    # a view of the other device is rejected by the queue
+    ca = cpu.tensor(DT_F32, (2, 16, 16))
+    ga = gpu.tensor(DT_F32, (2, 16, 16))
+    assert gpu.l.iomc_binary(gpu.queue, OP_ADD, ca.view().h, ga.view().h, ga.view().h) == -1
+    close(ca, ga)
+
+
+def test_in_order_queue_with_more_submissions_than_credits(devices):
+    """C = 4 in flight; 64 dependent submissions without waiting, then one wait."""
+    cpu, gpu = devices
+    dims = (4, 64, 128)
+    ones = np.full(dims, 1, np.uint32)
+    acc_c, acc_g = both(devices, DT_I32, dims, values=np.zeros(dims, np.uint32))
+    one_c, one_g = both(devices, DT_I32, dims, values=ones)
+    last = 0
+    for _ in range(64):
+        last = gpu.l.iomc_binary(gpu.queue, OP_ADD, acc_g.view().h, one_g.view().h, acc_g.view().h)
+        assert last > 0
+    assert gpu.wait(last) == 0
+    assert gpu.wait(last) == 0                      # repeat-waitable
+    assert np.all(acc_g.view().to_host() == 64)
+    close(acc_c, acc_g, one_c, one_g)
+
+
+def test_arena_exhaustion_and_reuse(devices):
+    cpu, gpu = devices
+    small = iomo.mi355x_backend(arena_bytes=1 << 20, max_in_flight=2)
+    try:
+        t = small.tensor(DT_F32, (256, 256))            # 256 KiB
+        with pytest.raises(RuntimeError, match="bad_alloc"):
+            small.tensor(DT_F32, (512, 512))            # 1 MiB does not fit beside it
+        t.close()
+        t2 = small.tensor(DT_F32, (384, 512))           # fits again once the first is gone
+        t2.close()
+        queues = [small.l.iomc_queue_create(small.dev) for _ in range(3)]   # + the backend's own = 4
+        assert all(queues)
+        assert not small.l.iomc_queue_create(small.dev)                      # the fifth is refused
+        for q in queues:
+            small.l.iomc_queue_destroy(q)
+    finally:
+        small.close()
+
+
+def test_bad_factory_configuration_is_rejected_before_any_native_effect():
+    if not iomo.mi355x_available():
+        pytest.skip("backend library not built")
+    l = iomo.mi355x_lib()
+    assert not l.iomc_mi355x_device_create(0, 0, 16)
+    assert b"invalid_argument" in l.iomc_last_error()
+    assert not l.iomc_mi355x_device_create(0, 1000, 16)           # not a multiple of 32
+    assert not l.iomc_mi355x_device_create(99, 1 << 20, 16)       # no such ordinal
