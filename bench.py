@@ -164,6 +164,24 @@ def wl_binary(timer, steps, warmup, name, dtype, op, dims, rhs_dims, kinds, lhs_
     return report(name, alg, n, wall, ev, kernel)
 
 
+def wl_copy(timer, steps, warmup, name, dtype, dims):
+    """Plain same-spec copy: the known-size kernel the HBM counters are scaled by."""
+    esize = iomx.leaf_bytes(dtype)
+    sets = [(device_tensor(dtype, dims, "normal", 61 + i), device_tensor(dtype, dims)) for i in range(ROT)]
+    n = int(np.prod(dims))
+
+    def launch(i):
+        src, dst = sets[i % ROT]
+        check(iomx.copy(src.view(), dst.view(), timer.stream), name)
+
+    wall, ev = timer.run(launch, steps, warmup)
+    kernel = iomx.last_launch().kernel.decode()
+    for src, dst in sets:
+        src.free()
+        dst.free()
+    return report(name, 2 * n * esize, n, wall, ev, kernel)
+
+
 def wl_rmsnorm(timer, steps, warmup, name, dtype, dims):
     esize = iomx.leaf_bytes(dtype)
     F = dims[-1]
@@ -381,6 +399,7 @@ def main():
             timer, K, W, "bcast_add_bf16_lhs=permute(1,0)of[8,8,512,2048]", BF16, ADD, (8, 8, 512, 2048),
             (1, 2048), ("normal", "normal_0p02"),
             lhs_view=((8, 8, 512, 2048), lambda v: v.permute([1, 0]))),
+        "copy_bf16": lambda: wl_copy(timer, K, W, "copy_bf16_[64,512,2048]", BF16, hd),
         "add_f32": lambda: wl_binary(timer, K, W, "add_f32_[4096,4096]", F32, ADD, (4096, 4096),
                                      (4096, 4096), ("uniform_pm1", "uniform_pm1")),
         "add_i32": lambda: wl_binary(timer, K, W, "add_i32_[4096,4096]", I32, ADD, (4096, 4096),
@@ -403,7 +422,7 @@ def main():
     head = table["bcast_add_bf16"]()
     detail = []
     if not args.no_detail:
-        for key in ("bcast_mul_bf16", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "add_f32",
+        for key in ("bcast_mul_bf16", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "copy_bf16", "add_f32",
                     "add_i32", "rmsnorm_bf16", "rmsnorm_f32", "silu_mul", "softmax", "softmax_causal",
                     "chain"):
             r = table[key]()
@@ -425,7 +444,7 @@ def main():
                    "device": props.name.decode(), "compute_units": props.compute_units},
         "roofline": {"bound": "hbm", "achieved": head["GB_per_s"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": head["hbm_frac"], "traffic": traffic_of("bcast_add_bf16"),
-                     "kernel": "elementwise_planes_kernel<BF16,ADD,FULL,ROWVEC>",
+                     "kernel": "elementwise_stream_kernel<BF16,ADD,FULL,ROWVEC,BANDS>",
                      "ms_per_launch": head["ms_per_launch"]},
         "cpu_baseline": cpu,
         "detail": detail,
