@@ -22,6 +22,9 @@ struct SoftmaxArgs {
     uint64_t heads;
     uint64_t total_rows; // planes * heads * pl.rows
     float scale;
+    // 32-bit copies for the row kernel (all fit when it is selected)
+    uint32_t rows32, prows32, heads32, pcols32, L32, a32;
+    FastDiv div_prows, div_heads;
 };
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -53,100 +56,108 @@ __device__ __forceinline__ uint64_t stage_offset(const iomx_stage_layout& l, uin
 template <int K>
 __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) {
     const uint32_t lane = threadIdx.x & 63u;
-    const uint64_t wave = (blockIdx.x * (uint64_t)blockDim.x + threadIdx.x) >> 6;
-    const uint64_t waves = ((uint64_t)gridDim.x * blockDim.x) >> 6;
-    for (uint64_t g = wave; g < a.total_rows; g += waves) {
-        const uint64_t r = g % a.pl.rows;
-        const uint64_t ph = g / a.pl.rows;
-        const uint64_t head = ph % a.heads;
-        const uint64_t plane = ph / a.heads;
-        uint16_t* prow = a.p + stage_offset(a.pl, plane, head, r);
-        uint64_t visible = 0;
-        if (r < a.rows) {
-            const uint64_t reach = a.a + r + 1;
-            visible = reach < a.L ? reach : a.L;
-        }
-        const float* srow = a.scores + stage_offset(a.sl, plane, head, r < a.rows ? r : 0);
+    const uint32_t g = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (g >= (uint32_t)a.total_rows) return;
+    // row -> (plane, head, r) with multiply-shift divisions
+    uint32_t ph = g, r = 0;
+    if (a.prows32 > 1) {
+        ph = fast_div(g, a.div_prows);
+        r = g - ph * a.prows32;
+    }
+    uint32_t plane = ph, head = 0;
+    if (a.heads32 > 1) {
+        plane = fast_div(ph, a.div_heads);
+        head = ph - plane * a.heads32;
+    }
+    uint16_t* prow = a.p + stage_offset(a.pl, plane, head, r);
+    uint32_t visible = 0;
+    if (r < a.rows32) {
+        const uint32_t reach = a.a32 + r + 1;  // a32 <= L32 <= 4096: no wrap
+        visible = reach < a.L32 ? reach : a.L32;
+    }
+    const float* srow = a.scores + stage_offset(a.sl, plane, head, r < a.rows32 ? r : 0);
 
-        float s[K][4];
-        bool has_nan = false;
-        float vmax = as_f32(kNegInf);
+    float s[K][4];
+    bool has_nan = false;
+    float vmax = as_f32(kNegInf);
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const uint64_t col = ((uint64_t)k * 64 + lane) * 4;
-            float x[4];
+    for (int k = 0; k < K; ++k) {
+        const uint32_t col = (k * 64u + lane) * 4u;
+        float x[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) x[j] = as_f32(kNegInf);
-            if (col + 4 <= visible) {
-                const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(srow + col));
-                x[0] = as_f32(v.x) * a.scale; x[1] = as_f32(v.y) * a.scale;
-                x[2] = as_f32(v.z) * a.scale; x[3] = as_f32(v.w) * a.scale;
-            } else if (col < visible) {
+        for (int j = 0; j < 4; ++j) x[j] = as_f32(kNegInf);
+        if (col + 4 <= visible) {
+            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(srow + col));
+            x[0] = as_f32(v.x) * a.scale; x[1] = as_f32(v.y) * a.scale;
+            x[2] = as_f32(v.z) * a.scale; x[3] = as_f32(v.w) * a.scale;
+        } else if (col < visible) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (col + j < visible) x[j] = srow[col + j] * a.scale;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                s[k][j] = x[j];
-                has_nan = has_nan || (x[j] != x[j]);
-                vmax = fmaxf(vmax, x[j]);  // fmaxf skips NaN; NaN rows are decided by has_nan
-            }
+            for (int j = 0; j < 4; ++j)
+                if (col + j < visible) x[j] = srow[col + j] * a.scale;
         }
-        const bool row_nan = __any(has_nan);
-        const float m = wave_max(vmax);
-        const bool all_ninf = as_u32(m) == kNegInf;
-        const bool poisoned = row_nan || all_ninf;
-        uint32_t pinf = 0;
-        float inv_share = 0.0f;
-        float inv_sum = 1.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            s[k][j] = x[j];
+            has_nan = has_nan || (x[j] != x[j]);
+            vmax = fmaxf(vmax, x[j]);  // fmaxf skips NaN; NaN rows are decided by has_nan
+        }
+    }
+    const bool row_nan = __any(has_nan);
+    const float m = wave_max(vmax);
+    const bool poisoned = row_nan || as_u32(m) == kNegInf;
+    if (poisoned || as_u32(m) == kPosInf) {
+        // rare rows: NaN / all -inf -> NaN over the visible range; k scores of +inf
+        // share 1/k
+        float share = as_f32(kQuietNanF32);
         if (!poisoned) {
-            if (as_u32(m) == kPosInf) {
-                uint32_t cnt = 0;
+            uint32_t cnt = 0;
 #pragma unroll
-                for (int k = 0; k < K; ++k)
+            for (int k = 0; k < K; ++k)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) cnt += as_u32(s[k][j]) == kPosInf ? 1u : 0u;
-                pinf = wave_sum_u32(cnt);
-                inv_share = 1.0f / (float)pinf;
-            } else {
-                float part = 0.0f;
-#pragma unroll
-                for (int k = 0; k < K; ++k)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float e = exp_nonpos(s[k][j] - m);  // 0 for masked and -inf scores
-                        s[k][j] = e;
-                        part = part + e;
-                    }
-                // e * (1/sum) instead of e / sum: at most one binary32 unit apart,
-                // which a BF16 result shows only at a rounding boundary
-                inv_sum = 1.0f / wave_sum(part);
-            }
+                for (int j = 0; j < 4; ++j) cnt += as_u32(s[k][j]) == kPosInf ? 1u : 0u;
+            share = 1.0f / (float)wave_sum_u32(cnt);
         }
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const uint64_t col = ((uint64_t)k * 64 + lane) * 4;
-            if (col >= a.pl.columns) continue;
-            float pr[4];
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                s[k][j] = (poisoned || as_u32(s[k][j]) == kPosInf) ? share : 0.0f;
+    } else {
+        float part = 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; ++k)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                float v;
-                if (poisoned) v = as_f32(kQuietNanF32);
-                else if (pinf != 0) v = as_u32(s[k][j]) == kPosInf ? inv_share : 0.0f;
-                else v = s[k][j] * inv_sum;
-                pr[j] = (col + j < visible) ? v : 0.0f;
+                const float e = exp_nonpos(s[k][j] - m);  // 0 for masked and -inf scores
+                s[k][j] = e;
+                part = part + e;
             }
-            const uint32_t lo = pack_bf16(pr[0], pr[1]);
-            const uint32_t hi = pack_bf16(pr[2], pr[3]);
-            if (col + 4 <= a.pl.columns) {
-                __builtin_nontemporal_store(u32x2{lo, hi}, reinterpret_cast<u32x2*>(prow + col));
-            } else {
-                const uint32_t words[2] = {lo, hi};
-                for (int j = 0; j < 4; ++j)
-                    if (col + j < a.pl.columns)
-                        prow[col + j] = (uint16_t)(words[j >> 1] >> ((j & 1) * 16));
-            }
+        // e * (1/sum) instead of e / sum: at most one binary32 unit apart, which a
+        // BF16 result shows only at a rounding boundary
+        const float inv_sum = 1.0f / wave_sum(part);
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s[k][j] = s[k][j] * inv_sum;
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t col = (k * 64u + lane) * 4u;
+        if (col >= a.pcols32) continue;
+        // elements at or beyond the visible limit are +0
+        const uint32_t nvis = visible > col ? visible - col : 0u;
+        float pr[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pr[j] = ((uint32_t)j < nvis) ? s[k][j] : 0.0f;
+        const uint32_t lo = pack_bf16(pr[0], pr[1]);
+        const uint32_t hi = pack_bf16(pr[2], pr[3]);
+        if (col + 4 <= a.pcols32) {
+            __builtin_nontemporal_store(u32x2{lo, hi}, reinterpret_cast<u32x2*>(prow + col));
+        } else {
+            const uint32_t words[2] = {lo, hi};
+            for (int j = 0; j < 4; ++j)
+                if (col + j < a.pcols32)
+                    prow[col + j] = (uint16_t)(words[j >> 1] >> ((j & 1) * 16));
         }
     }
 }
@@ -252,10 +263,20 @@ extern "C" int iomx_launch_softmax(const iomx_softmax_desc* d, iomx_stream_t str
             && pl.plane_offset % 4 == 0 && pl.plane_stride % 4 == 0 && pl.head_stride % 4 == 0
             && pl.row_stride % 4 == 0;
     const uint64_t blocks = (total + 3) / 4;
-    const uint32_t grid = (uint32_t)(blocks < (1u << 20) ? blocks : (1u << 20));
+    uint32_t grid = (uint32_t)(blocks < (1u << 20) ? blocks : (1u << 20));
     const hipStream_t s = native(stream);
     const uint64_t cols = pl.columns;
-    if (aligned && cols <= 4096) {
+    if (aligned && cols <= 4096 && blocks <= 0x7FFFFFFFull && d->rows <= 0xFFFFFFFFull
+        && pl.rows <= 0xFFFFFFFFull && d->heads <= 0xFFFFFFFFull) {
+        grid = (uint32_t)blocks;  // one wave per row, one-shot
+        a.rows32 = (uint32_t)d->rows;
+        a.prows32 = (uint32_t)pl.rows;
+        a.heads32 = (uint32_t)d->heads;
+        a.pcols32 = (uint32_t)cols;
+        a.L32 = (uint32_t)d->L;
+        a.a32 = (uint32_t)(d->a < d->L ? d->a : d->L);
+        a.div_prows = make_fast_div(a.prows32);
+        a.div_heads = make_fast_div(a.heads32);
         if (cols <= 256) hipLaunchKernelGGL(softmax_rows_kernel<1>, dim3(grid), dim3(256), 0, s, a);
         else if (cols <= 512) hipLaunchKernelGGL(softmax_rows_kernel<2>, dim3(grid), dim3(256), 0, s, a);
         else if (cols <= 1024) hipLaunchKernelGGL(softmax_rows_kernel<4>, dim3(grid), dim3(256), 0, s, a);
