@@ -104,7 +104,8 @@ __device__ __forceinline__ float inverse_rms(float sum, uint32_t feats, float ep
 // MI355X, [32768,2048]: a persistent workgroup that prefetches its next band
 // into a second register set, the scale row decoded once into registers, sixteen
 // lanes finishing the row totals for everyone, and a barrier-free kernel with
-// four rows per wave: all slower, by 3-20 %.)
+// four rows per wave, and two passes with the second read served by the caches:
+// all slower, by 3-20 %.)
 //
 // The sum of squares uses a fused multiply-add per element (one rounding instead
 // of the reference's two): the total differs from the sequential reference

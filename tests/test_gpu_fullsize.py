@@ -1,0 +1,307 @@
+"""The benchmark configurations at their full sizes, on the GPU, against closed
+forms evaluated with numpy (binary32 arithmetic is IEEE there), against the
+oracle on sampled planes / rows, and through size-independent properties.
+
+  config 1  ADD F32 / I32 [4096,4096]                       bit-exact, every element
+  config 2  broadcast ADD / MUL BF16 [64,512,2048]+[1,2048], dense, sliced and
+            permuted lhs                                    bit-exact, every element
+  config 3  RMSNorm BF16 / F32 [32768,2048]                 <= 1 BF16 ulp / 1e-5 relative
+  config 4  softmax F32->BF16 [8,8,2048,2048] (1/16 of the planes of the benchmark
+            shape; rows are independent) and SiLU then MUL BF16 [32768,5632]
+  config 5  the six-operation layer chain over [64,512,.]   end to end
+"""
+import numpy as np
+import pytest
+
+import datagen
+import iomo
+from iom_amd import iomx
+from iomo import DT_BF16, DT_F32, DT_I32, OP_ADD, OP_MUL
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    assert iomx.device_count() >= 1
+    iomx.check(iomx.lib().iomx_set_device(0))
+    yield
+
+
+def tiled_values(dtype, dims, kind, salt):
+    """Raw tiled storage with an i.i.d. pattern (shapes are multiples of 16, so any
+    permutation of an i.i.d. pattern has the stated distribution)."""
+    n = int(np.prod(dims))
+    base = min(n, 1 << 22)
+    if kind == "uniform_pm1":
+        v = datagen.uniform_f32(base, -1, 1, salt).view(np.uint32)
+    elif kind == "i20":
+        v = datagen.uniform_i32(base, -(1 << 20), 1 << 20, salt)
+    elif kind == "normal":
+        v = datagen.normal_f32(base, 0, 1, salt)
+        v = datagen.bf16_rne(v) if dtype == DT_BF16 else v.view(np.uint32)
+    elif kind == "normal_small":
+        v = datagen.bf16_rne(datagen.normal_f32(base, 0, 0.02, salt))
+    elif kind == "weight":
+        v = datagen.uniform_f32(base, 0.5, 1.5, salt)
+        v = datagen.bf16_rne(v) if dtype == DT_BF16 else v.view(np.uint32)
+    reps = (n + base - 1) // base
+    # rotate every repetition so that repeated blocks do not line up with tiles
+    return np.concatenate([np.roll(v, 977 * i) for i in range(reps)])[:n]
+
+
+def upload(dtype, dims, kind, salt):
+    t = iomx.DeviceTensor(dtype, dims, fill=None)
+    storage = tiled_values(dtype, dims, kind, salt)
+    t.upload_raw(storage)
+    return t, storage
+
+
+def bf16_op(a, b, op):
+    fa, fb = datagen.bf16_to_f32(a), datagen.bf16_to_f32(b)
+    with np.errstate(all="ignore"):
+        r = fa + fb if op == OP_ADD else fa * fb
+    return datagen.bf16_rne(r)
+
+
+@pytest.mark.parametrize("dtype,kind", [(DT_F32, "uniform_pm1"), (DT_I32, "i20")])
+def test_config1_add_2p24(dtype, kind):
+    dims = (4096, 4096)
+    a, sa = upload(dtype, dims, kind, 1)
+    b, sb = upload(dtype, dims, kind, 2)
+    o = iomx.DeviceTensor(dtype, dims)
+    assert iomx.binary(OP_ADD, a.view(), b.view(), o.view()) == 0
+    assert iomx.last_launch().kernel.decode() == "binary_planes"
+    got = o.raw()
+    if dtype == DT_F32:
+        want = (sa.view(np.float32) + sb.view(np.float32)).view(np.uint32)
+    else:
+        want = (sa + sb).astype(np.uint32)
+    assert np.array_equal(got, want)
+    # the closed form used above is itself the oracle's element rule on a sample
+    L = iomo.lib()
+    for i in range(0, got.size, 40009):
+        assert L.iomo_scalar_binary(OP_ADD, dtype, int(sa[i]), int(sb[i])) == int(want[i])
+    for t in (a, b, o):
+        t.free()
+
+
+def vector_storage(values16):
+    """Tiled storage of a [1,F] BF16 vector: row 0 of every tile."""
+    F = values16.size
+    st = np.zeros(F * 16, np.uint16)
+    st.reshape(F // 16, 16, 16)[:, 0, :] = values16.reshape(F // 16, 16)
+    return st
+
+
+def column_of_storage(dims):
+    """Logical column index of every slot of a tiled [..., R, C] storage."""
+    R, Cc = dims[-2], dims[-1]
+    planes = int(np.prod(dims[:-2]))
+    col = (np.arange(Cc // 16)[None, :, None, None] * 16 + np.arange(16)[None, None, None, :])
+    col = np.broadcast_to(col, (R // 16, Cc // 16, 16, 16)).reshape(-1)
+    return np.tile(col, planes)
+
+
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL])
+@pytest.mark.parametrize("layout", ["dense", "sliced", "permuted"])
+def test_config2_broadcast_bf16(op, layout):
+    F = 2048
+    vec = datagen.bf16_rne(datagen.normal_f32(F, 0, 0.02, 9))
+    v = iomx.DeviceTensor(DT_BF16, (1, F))
+    v.upload_raw(vector_storage(vec))
+    plane = 512 * F
+    if layout == "dense":
+        x, sx = upload(DT_BF16, (64, 512, F), "normal", 3)
+        xv, odims = x.view(), (64, 512, F)
+        src = sx
+    elif layout == "sliced":
+        x, sx = upload(DT_BF16, (128, 512, F), "normal", 3)
+        xv, odims = x.view().slice(0, 0, 64, 2), (64, 512, F)
+        src = sx.reshape(128, plane)[0::2].reshape(-1)
+    else:
+        x, sx = upload(DT_BF16, (8, 8, 512, F), "normal", 3)
+        xv, odims = x.view().permute([1, 0]), (8, 8, 512, F)
+        src = sx.reshape(8, 8, plane).transpose(1, 0, 2).reshape(-1)
+    o = iomx.DeviceTensor(DT_BF16, odims)
+    assert iomx.binary(op, xv, v.view(), o.view()) == 0
+    assert iomx.last_launch().kernel.decode() == "binary_rowvec"
+    got = o.raw()
+    want = bf16_op(src, vec[column_of_storage((512, F))][np.arange(src.size) % plane], op)
+    assert np.array_equal(got, want)
+    for t in (x, v, o):
+        t.free()
+
+
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F32])
+def test_config3_rmsnorm_32768x2048(dtype):
+    R, F = 32768, 2048
+    x, sx = upload(dtype, (R, F), "normal", 5)
+    # 1 % of the rows scaled by 50 (whole rows: every 100th)
+    xf = (datagen.bf16_to_f32(sx) if dtype == DT_BF16 else sx.view(np.float32)).copy()
+    seg = xf.reshape(R // 16, F // 16, 16, 16)            # band, tile col, row, col
+    rows = np.arange(R).reshape(R // 16, 16)
+    seg[(rows % 100 == 0)[:, None, :, None].repeat(F // 16, 1).repeat(16, 3)] *= 50.0
+    sx = datagen.bf16_rne(xf) if dtype == DT_BF16 else xf.view(np.uint32)
+    x.upload_raw(sx)
+    w = datagen.uniform_f32(F, 0.5, 1.5, 6)
+    wl = datagen.bf16_rne(w) if dtype == DT_BF16 else w.view(np.uint32)
+    wt = iomx.DeviceTensor(dtype, (1, F))
+    wt.view().from_host(wl.reshape(1, F))
+    o = iomx.DeviceTensor(dtype, (R, F))
+    assert iomx.rmsnorm(x.view(), wt.view(), o.view(), 1e-5) == 0
+    assert iomx.last_launch().kernel.decode() == "rmsnorm_band"
+    got = iomo.untile_plane(o.raw(), (R, F))
+    xl = iomo.untile_plane(sx, (R, F))
+    x64 = (datagen.bf16_to_f32(xl.reshape(-1)).reshape(R, F) if dtype == DT_BF16
+           else xl.view(np.float32)).astype(np.float64)
+    w64 = (datagen.bf16_to_f32(wl) if dtype == DT_BF16 else wl.view(np.float32)).astype(np.float64)
+    ref = x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + 1e-5) * w64
+    g = (datagen.bf16_to_f32(got.reshape(-1)).reshape(R, F) if dtype == DT_BF16
+         else got.view(np.float32)).astype(np.float64)
+    rel = np.abs(g - ref) / np.maximum(np.abs(ref), 1e-30)
+    assert rel.max() <= (2.0 ** -7 if dtype == DT_BF16 else 1e-5)
+    # the oracle itself on 64 sampled rows (4 bands): <= 1 BF16 ulp / 1e-5
+    bands = [0, 6, 1024, 2047]
+    sample = np.concatenate([xl[b * 16:(b + 1) * 16] for b in bands])
+    hx, hw, ho = iomo.HostTensor(dtype, sample.shape), iomo.HostTensor(dtype, (1, F)), iomo.HostTensor(dtype, sample.shape)
+    hx.view().from_logical(sample)
+    hw.view().from_logical(wl.reshape(1, F))
+    assert iomo.rmsnorm(hx.view(), hw.view(), ho.view(), 1e-5) == 0
+    want = ho.view().to_logical()
+    mine = np.concatenate([got[b * 16:(b + 1) * 16] for b in bands])
+    if dtype == DT_BF16:
+        assert np.abs(mine.astype(np.int64) - want.astype(np.int64)).max() <= 1
+    else:
+        a, b = mine.view(np.float32).astype(np.float64), want.view(np.float32).astype(np.float64)
+        assert (np.abs(a - b) / np.maximum(np.abs(b), 1e-30)).max() <= 1e-5
+    for t in (x, wt, o):
+        t.free()
+
+
+def test_config4_softmax_rows_of_2048():
+    planes, heads, R, Cc = 8, 8, 2048, 2048
+    one = datagen.normal_f32(R * Cc, 0, 3, 61).reshape(R, Cc)
+    one[np.triu_indices(R, 1, Cc)] = -np.inf
+    n = planes * heads * R * Cc
+    sb, pb = iomx.Buffer(n * 4), iomx.Buffer(n * 2)
+    for i in range(planes * heads):
+        sb.upload(one, offset=i * one.nbytes)
+    for a_pos, name in ((Cc - 1, "mask as data"), (0, "positional")):
+        pb.fill(0xAA)
+        d = iomx.softmax_desc(sb.ptr.value, pb.ptr.value, planes, heads, R, Cc, a_pos, Cc)
+        assert iomx.softmax(d) == 0
+        assert iomx.last_launch().kernel.decode() == "softmax_rows"
+        iomx.synchronize()
+        got = pb.download(np.uint16).reshape(planes * heads, R, Cc)
+        assert np.all(got[:, np.triu_indices(R, 1, Cc)[0], np.triu_indices(R, 1, Cc)[1]] == 0), name
+        assert np.array_equal(got[0], got[-1])                       # identical inputs, identical planes
+        p = datagen.bf16_to_f32(got[0].reshape(-1)).reshape(R, Cc).astype(np.float64)
+        assert np.abs(p.sum(axis=1) - 1.0).max() < 2.0 ** -6           # rows sum to one
+        x64 = one.astype(np.float64)
+        e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+        ref = e / e.sum(axis=1, keepdims=True)
+        nz = ref > 1e-30
+        assert (np.abs(p[nz] - ref[nz]) / ref[nz]).max() <= 2.0 ** -7
+        # oracle on 48 sampled rows: <= 1 BF16 ulp
+        rows = [0, 1, 15, 16, 17, 255, 1023, 1024, 2046, 2047] + list(range(500, 538))
+        want = iomo.softmax(one[rows].reshape(1, 1, len(rows), Cc), a=Cc - 1, L=Cc)[0, 0]
+        assert np.abs(got[0][rows].astype(np.int64) - want.astype(np.int64)).max() <= 1
+    sb.free()
+    pb.free()
+
+
+def silu64(x):
+    with np.errstate(all="ignore"):
+        return x / (1.0 + np.exp(-x))
+
+
+def test_config4_silu_then_mul_32768x5632():
+    dims = (32768, 5632)
+    g, sg = upload(DT_BF16, dims, "normal", 7)
+    u, su = upload(DT_BF16, dims, "normal", 8)
+    act, prod, fused = (iomx.DeviceTensor(DT_BF16, dims) for _ in range(3))
+    assert iomx.silu(g.view(), act.view()) == 0
+    assert iomx.binary(OP_MUL, act.view(), u.view(), prod.view()) == 0
+    assert iomx.silu_mul(g.view(), u.view(), fused.view()) == 0
+    ra, rp, rf = act.raw(), prod.raw(), fused.raw()
+    assert np.array_equal(rp, rf)                                        # private fused path == sequence
+    assert np.array_equal(rp, bf16_op(ra, su, OP_MUL))                   # MUL bit-exact given act
+    ref = datagen.bf16_rne(silu64(datagen.bf16_to_f32(sg).astype(np.float64)).astype(np.float32))
+    assert np.abs(ra.astype(np.int64) - ref.astype(np.int64)).max() <= 1  # SiLU <= 1 BF16 ulp
+    # the oracle (reference arithmetic) on 2^20 sampled elements
+    idx = np.arange(0, sg.size, sg.size // (1 << 20))[: 1 << 20]
+    hx, ho = iomo.HostTensor(DT_BF16, (1024, 1024)), iomo.HostTensor(DT_BF16, (1024, 1024))
+    hx.storage[:] = sg[idx]
+    assert iomo.silu(hx.view(), ho.view()) == 0
+    d = np.abs(ra[idx].astype(np.int64) - ho.storage.astype(np.int64))
+    assert d.max() <= 1
+    print("silu: %d of %d sampled elements differ from the CPU arithmetic by 1 ulp" % (int((d == 1).sum()), d.size), flush=True)
+    for t in (g, u, act, prod, fused):
+        t.free()
+
+
+def test_config5_layer_chain_end_to_end():
+    """rmsnorm(x,w1)->n; add(x,attn)->x2; rmsnorm(x2,w2)->n2; silu(gate)->act;
+    mul(act,up)->prod; add(x2,down)->next over [64,512,.]; the oracle runs the same
+    chain on 2 of the 64 planes."""
+    B, S, H, FF = 64, 512, 2048, 5632
+    hd, fd = (B, S, H), (B, S, FF)
+    x, sx = upload(DT_BF16, hd, "normal", 11)
+    attn, sa = upload(DT_BF16, hd, "normal", 12)
+    down, sd = upload(DT_BF16, hd, "normal", 13)
+    gate, sg = upload(DT_BF16, fd, "normal", 14)
+    up, su = upload(DT_BF16, fd, "normal", 15)
+    w1l = datagen.bf16_rne(datagen.uniform_f32(H, 0.5, 1.5, 16))
+    w2l = datagen.bf16_rne(datagen.uniform_f32(H, 0.5, 1.5, 17))
+    w1, w2 = iomx.DeviceTensor(DT_BF16, (1, H)), iomx.DeviceTensor(DT_BF16, (1, H))
+    w1.view().from_host(w1l.reshape(1, H))
+    w2.view().from_host(w2l.reshape(1, H))
+    n1, x2, n2, nxt = (iomx.DeviceTensor(DT_BF16, hd) for _ in range(4))
+    act, prod = iomx.DeviceTensor(DT_BF16, fd), iomx.DeviceTensor(DT_BF16, fd)
+    assert iomx.rmsnorm(x.view(), w1.view(), n1.view(), 1e-5) == 0
+    assert iomx.binary(OP_ADD, x.view(), attn.view(), x2.view()) == 0
+    assert iomx.rmsnorm(x2.view(), w2.view(), n2.view(), 1e-5) == 0
+    assert iomx.silu(gate.view(), act.view()) == 0
+    assert iomx.binary(OP_MUL, act.view(), up.view(), prod.view()) == 0
+    assert iomx.binary(OP_ADD, x2.view(), down.view(), nxt.view()) == 0
+    # full size, closed forms: the two residual adds are bit-exact
+    rx2 = x2.raw()
+    assert np.array_equal(rx2, bf16_op(sx, sa, OP_ADD))
+    assert np.array_equal(nxt.raw(), bf16_op(rx2, sd, OP_ADD))
+    assert np.array_equal(prod.raw(), bf16_op(act.raw(), su, OP_MUL))
+    # the oracle on planes 0 and 63
+    hp, fp = S * H, S * FF
+    stats = {}
+    for pl in (0, 63):
+        def host(dt_dims, storage, per):
+            t = iomo.HostTensor(DT_BF16, dt_dims)
+            t.storage[:] = storage[pl * per:(pl + 1) * per]
+            return t
+        hx, ha, hdn = host((S, H), sx, hp), host((S, H), sa, hp), host((S, H), sd, hp)
+        hg, hu = host((S, FF), sg, fp), host((S, FF), su, fp)
+        hw1, hw2 = iomo.HostTensor(DT_BF16, (1, H)), iomo.HostTensor(DT_BF16, (1, H))
+        hw1.view().from_logical(w1l.reshape(1, H))
+        hw2.view().from_logical(w2l.reshape(1, H))
+        hn1, hx2, hn2, hnx = (iomo.HostTensor(DT_BF16, (S, H)) for _ in range(4))
+        hact, hprod = iomo.HostTensor(DT_BF16, (S, FF)), iomo.HostTensor(DT_BF16, (S, FF))
+        assert iomo.rmsnorm(hx.view(), hw1.view(), hn1.view(), 1e-5) == 0
+        assert iomo.binary(OP_ADD, hx.view(), ha.view(), hx2.view(), ieee=True) == 0
+        assert iomo.rmsnorm(hx2.view(), hw2.view(), hn2.view(), 1e-5) == 0
+        assert iomo.silu(hg.view(), hact.view()) == 0
+        assert iomo.binary(OP_MUL, hact.view(), hu.view(), hprod.view(), ieee=True) == 0
+        assert iomo.binary(OP_ADD, hx2.view(), hdn.view(), hnx.view(), ieee=True) == 0
+        for name, dev, hostt, per in (("n", n1, hn1, hp), ("x2", x2, hx2, hp), ("n2", n2, hn2, hp),
+                                      ("act", act, hact, fp), ("prod", prod, hprod, fp),
+                                      ("next", nxt, hnx, hp)):
+            gotp = dev.raw()[pl * per:(pl + 1) * per].astype(np.int64)
+            d = np.abs(gotp - hostt.storage.astype(np.int64))
+            stats[name] = (max(stats.get(name, (0, 0))[0], int(d.max())),
+                           stats.get(name, (0, 0))[1] + int((d != 0).sum()))
+    print("layer chain vs CPU arithmetic (max ulp, mismatches over 2 planes):", stats, flush=True)
+    assert stats["x2"] == (0, 0) and stats["next"] == (0, 0)           # elementwise: bit-exact
+    assert stats["n"][0] <= 1 and stats["n2"][0] <= 1 and stats["act"][0] <= 1
+    # prod multiplies an activation that may differ by one ulp: at most one product ulp more
+    assert stats["prod"][0] <= 2
+    for t in (x, attn, down, gate, up, w1, w2, n1, x2, n2, nxt, act, prod):
+        t.free()
