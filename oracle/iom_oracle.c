@@ -18,14 +18,23 @@
 /* Layout (src/tensor.cpp:76-164)                                       */
 /* ------------------------------------------------------------------ */
 
-size_t iomo_leaf_bytes(int dtype) {
+unsigned iomo_leaf_bits(int dtype) {
     switch (dtype) {
-        case IOMO_DT_BF16: return 2;
-        case IOMO_DT_I32:
-        case IOMO_DT_U32:
-        case IOMO_DT_F32: return 4;
+        case IOMO_DT_I2: case IOMO_DT_U2: return 2;
+        case IOMO_DT_I4: case IOMO_DT_U4: case IOMO_DT_F4_E2M1: return 4;
+        case IOMO_DT_F6_E2M3: case IOMO_DT_F6_E3M2: return 6;
+        case IOMO_DT_BOOL: case IOMO_DT_I8: case IOMO_DT_U8: case IOMO_DT_F8_E4M3FN:
+        case IOMO_DT_F8_E5M2: case IOMO_DT_F8_E8M0: return 8;
+        case IOMO_DT_I16: case IOMO_DT_U16: case IOMO_DT_F16: case IOMO_DT_BF16: return 16;
+        case IOMO_DT_I32: case IOMO_DT_U32: case IOMO_DT_F32: return 32;
+        case IOMO_DT_I64: case IOMO_DT_U64: case IOMO_DT_F64: return 64;
         default: return 0;
     }
+}
+
+size_t iomo_leaf_bytes(int dtype) {
+    const unsigned bits = iomo_leaf_bits(dtype);
+    return bits % 8 == 0 ? bits / 8 : 0;
 }
 
 static uint64_t tiles_of(uint64_t extent) { return (extent + TILE - 1) / TILE; }
@@ -43,24 +52,37 @@ uint64_t iomo_plane_slot(uint64_t rows, uint64_t cols, uint64_t plane,
     return tile * TILE_SLOTS + (row % TILE) * TILE + col % TILE;
 }
 
-static uint64_t load_leaf(const void* base, uint64_t slot, size_t bytes) {
-    if (bytes == 2) {
-        uint16_t v;
-        memcpy(&v, (const unsigned char*)base + slot * 2, 2);
+/* Packed elements: element `slot` occupies bits [slot*bits, (slot+1)*bits) of a
+ * little-endian bit stream, least significant bit first
+ * (src/cpu/transfer_helpers.hpp:14-40). */
+static uint64_t load_leaf(const void* base, uint64_t slot, unsigned bits) {
+    const unsigned char* p = (const unsigned char*)base;
+    if (bits % 8 == 0) {
+        uint64_t v = 0;
+        memcpy(&v, p + slot * (bits / 8), bits / 8);
         return v;
     }
-    uint32_t v;
-    memcpy(&v, (const unsigned char*)base + slot * 4, 4);
+    uint64_t v = 0;
+    const uint64_t first = slot * bits;
+    for (unsigned i = 0; i < bits; ++i) {
+        const uint64_t bit = first + i;
+        v |= (uint64_t)((p[bit >> 3] >> (bit & 7)) & 1u) << i;
+    }
     return v;
 }
 
-static void store_leaf(void* base, uint64_t slot, size_t bytes, uint64_t raw) {
-    if (bytes == 2) {
-        const uint16_t v = (uint16_t)raw;
-        memcpy((unsigned char*)base + slot * 2, &v, 2);
-    } else {
-        const uint32_t v = (uint32_t)raw;
-        memcpy((unsigned char*)base + slot * 4, &v, 4);
+static void store_leaf(void* base, uint64_t slot, unsigned bits, uint64_t raw) {
+    unsigned char* p = (unsigned char*)base;
+    if (bits % 8 == 0) {
+        memcpy(p + slot * (bits / 8), &raw, bits / 8);
+        return;
+    }
+    const uint64_t first = slot * bits;
+    for (unsigned i = 0; i < bits; ++i) {
+        const uint64_t bit = first + i;
+        const unsigned char mask = (unsigned char)(1u << (bit & 7));
+        if ((raw >> i) & 1u) p[bit >> 3] |= mask;
+        else p[bit >> 3] &= (unsigned char)~mask;
     }
 }
 
@@ -71,24 +93,50 @@ static void store_leaf(void* base, uint64_t slot, size_t bytes, uint64_t raw) {
 typedef struct {
     unsigned ebits, fbits;
     int bias;
+    int finite_only; /* no infinities; NaN only when ebits >= 4 (all of the top exponent) */
+    int infs;
 } fmt_t;
 
+/* :30-43 */
 static int float_format(int dtype, fmt_t* f) {
-    if (dtype == IOMO_DT_BF16) { f->ebits = 8; f->fbits = 7; f->bias = 127; return 1; }
-    if (dtype == IOMO_DT_F32) { f->ebits = 8; f->fbits = 23; f->bias = 127; return 1; }
-    return 0;
+    switch (dtype) {
+        case IOMO_DT_F4_E2M1:   *f = (fmt_t){2, 1, 1, 1, 0}; return 1;
+        case IOMO_DT_F6_E2M3:   *f = (fmt_t){2, 3, 1, 1, 0}; return 1;
+        case IOMO_DT_F6_E3M2:   *f = (fmt_t){3, 2, 3, 1, 0}; return 1;
+        case IOMO_DT_F8_E4M3FN: *f = (fmt_t){4, 3, 7, 1, 0}; return 1;
+        case IOMO_DT_F8_E5M2:   *f = (fmt_t){5, 2, 15, 0, 1}; return 1;
+        case IOMO_DT_F16:       *f = (fmt_t){5, 10, 15, 0, 1}; return 1;
+        case IOMO_DT_BF16:      *f = (fmt_t){8, 7, 127, 0, 1}; return 1;
+        case IOMO_DT_F32:       *f = (fmt_t){8, 23, 127, 0, 1}; return 1;
+        case IOMO_DT_F64:       *f = (fmt_t){11, 52, 1023, 0, 1}; return 1;
+        default: return 0;
+    }
 }
 
-/* :45-65 — both in-scope float leaves have infinities and NaNs. */
+static unsigned integer_width(int dtype) {
+    switch (dtype) {
+        case IOMO_DT_I2: case IOMO_DT_U2: case IOMO_DT_I4: case IOMO_DT_U4:
+        case IOMO_DT_I8: case IOMO_DT_U8: case IOMO_DT_I16: case IOMO_DT_U16:
+        case IOMO_DT_I32: case IOMO_DT_U32: case IOMO_DT_I64: case IOMO_DT_U64:
+            return iomo_leaf_bits(dtype);
+        default: return 0;
+    }
+}
+
+/* The top exponent is special (infinity / NaN) unless the format is one of the
+ * finite-only ones narrower than four exponent bits (:50-55). */
+static int top_exponent_is_special(fmt_t f) { return !f.finite_only || f.ebits >= 4; }
+
+/* :45-65 */
 static long double codec_decode(uint64_t raw, fmt_t f) {
     const uint64_t emask = (1ull << f.ebits) - 1;
     const uint64_t sign = (raw >> (f.ebits + f.fbits)) & 1;
     const uint64_t frac = raw & ((1ull << f.fbits) - 1);
     const uint64_t exp = (raw >> f.fbits) & emask;
     long double v;
-    if (exp == emask) {
-        if (frac != 0) return (long double)NAN;
-        return sign ? -(long double)INFINITY : (long double)INFINITY;
+    if (exp == emask && top_exponent_is_special(f)) {
+        if (f.infs && frac == 0) return sign ? -(long double)INFINITY : (long double)INFINITY;
+        return (long double)NAN;
     }
     if (exp != 0) {
         v = ldexpl((long double)((1ull << f.fbits) + frac),
@@ -108,18 +156,28 @@ static uint64_t codec_round_even(long double v) {
     return q;
 }
 
-/* :67-108 */
+/* :67-108.  Overflow stores infinity where the format has one and the largest
+ * finite magnitude otherwise; NaN stores exponent all-ones with the top
+ * fraction bit (every fraction bit for F8_E4M3FN), and the largest finite
+ * magnitude in the formats that have no NaN at all. */
 static uint64_t codec_encode(long double v, fmt_t f) {
     const uint64_t sign = signbit(v) ? 1 : 0;
     const uint64_t emask = (1ull << f.ebits) - 1;
+    const uint64_t fmask = (1ull << f.fbits) - 1;
     const unsigned shift = f.ebits + f.fbits;
-    const uint64_t inf_bits = (sign << shift) | (emask << f.fbits);
+    const uint64_t finite_emax = top_exponent_is_special(f) ? emask - 1 : emask;
+    const uint64_t overflow = (sign << shift)
+            | (f.infs ? emask << f.fbits : (finite_emax << f.fbits) | fmask);
     v = fabsl(v);
-    if (isnan(v)) return (sign << shift) | (emask << f.fbits) | (1ull << (f.fbits - 1));
-    if (isinf(v)) return inf_bits;
+    if (isnan(v)) {
+        if (!top_exponent_is_special(f)) return overflow;
+        return (sign << shift) | (emask << f.fbits)
+                | (f.finite_only ? fmask : 1ull << (f.fbits - 1));
+    }
+    if (isinf(v)) return overflow;
     if (v == 0) return sign << shift;
     const int min_sub = 1 - f.bias - (int)f.fbits;
-    const int max_exp = (int)(emask - 1) - f.bias;
+    const int max_exp = (int)finite_emax - f.bias;
     int e = 0;
     (void)frexpl(v, &e);
     --e;
@@ -128,11 +186,11 @@ static uint64_t codec_encode(long double v, fmt_t f) {
         if (q == (1ull << f.fbits)) return (sign << shift) | (1ull << f.fbits);
         return (sign << shift) | q;
     }
-    if (e > max_exp) return inf_bits;
+    if (e > max_exp) return overflow;
     uint64_t frac = codec_round_even(
             ldexpl(v, (int)f.fbits - e) - (long double)(1ull << f.fbits));
     if (frac == (1ull << f.fbits)) { ++e; frac = 0; }
-    if (e > max_exp) return inf_bits;
+    if (e > max_exp) return overflow;
     return (sign << shift) | ((uint64_t)(e + f.bias) << f.fbits) | frac;
 }
 
@@ -153,19 +211,22 @@ static long double codec_arith(int op, long double x, long double y) {
     return x - y;
 }
 
+static long double positive_nan(void) { return fabsl((long double)NAN); }
+
 /* The codec stores every NaN as sign 0, exponent all-ones, top fraction bit
  * (:79-84, quiet_nan() has a clear sign on x86-64). */
 uint64_t iomo_scalar_binary(int op, int dtype, uint64_t a, uint64_t b) {
-    if (dtype == IOMO_DT_I32 || dtype == IOMO_DT_U32) {
-        const uint64_t mask = 0xFFFFFFFFull;
+    const unsigned width = integer_width(dtype);
+    if (width) {
+        const uint64_t mask = width == 64 ? ~0ull : (1ull << width) - 1;
         if (op == IOMO_OP_ADD) return (a + b) & mask;
         if (op == IOMO_OP_MUL) return (a * b) & mask;
         return (a - b) & mask;
     }
     fmt_t f;
     if (!float_format(dtype, &f)) return 0;
-    const long double r = codec_arith(op, codec_decode(a, f), codec_decode(b, f));
-    if (isnan(r)) return (((1ull << f.ebits) - 1) << f.fbits) | (1ull << (f.fbits - 1));
+    long double r = codec_arith(op, codec_decode(a, f), codec_decode(b, f));
+    if (isnan(r)) r = positive_nan();
     return codec_encode(r, f);
 }
 
@@ -176,22 +237,92 @@ uint16_t iomo_encode_bf16(float value) {
     return (uint16_t)codec_encode((long double)value, f);
 }
 
-/* ---- closed form: IEEE-754 binary32 single rounding ---------------- */
+/* ---- closed form: one IEEE-754 operation and one rounding ------------ */
 
 static float f32_from_bits(uint32_t b) { float f; memcpy(&f, &b, 4); return f; }
 static uint32_t f32_bits(float f) { uint32_t b; memcpy(&b, &f, 4); return b; }
+static double f64_from_bits(uint64_t b) { double f; memcpy(&f, &b, 8); return f; }
+static uint64_t f64_bits(double f) { uint64_t b; memcpy(&b, &f, 8); return b; }
 
 static uint16_t bf16_rne_bits(uint32_t bits) {
     if ((bits & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0u;
     return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
 }
 
+/* Value of a narrow encoding as a binary64 number, by integer construction
+ * (every format of at most 32 bits is a subset of binary64).  *special: 0 finite,
+ * 1 infinity, 2 NaN. */
+static double narrow_value(uint64_t raw, fmt_t f, int* special) {
+    const uint64_t emask = (1ull << f.ebits) - 1;
+    const int negative = (int)((raw >> (f.ebits + f.fbits)) & 1);
+    const uint64_t frac = raw & ((1ull << f.fbits) - 1);
+    const uint64_t exp = (raw >> f.fbits) & emask;
+    *special = 0;
+    if (exp == emask && top_exponent_is_special(f)) {
+        *special = (f.infs && frac == 0) ? 1 : 2;
+        if (*special == 2) return NAN;
+        return negative ? -INFINITY : INFINITY;
+    }
+    const int64_t m = (int64_t)(exp ? (1ull << f.fbits) + frac : frac);
+    const int scale = (int)(exp ? exp : 1) - f.bias - (int)f.fbits;
+    const double v = ldexp((double)m, scale);
+    return negative ? -v : v;
+}
+
+/* One round-to-nearest-even of a finite binary64 value onto a narrow format's
+ * grid, done on the integer significand (no floating-point operation rounds
+ * here).  `v` must be a normal binary64 number or zero. */
+static uint64_t narrow_round(double v, fmt_t f) {
+    const uint64_t emask = (1ull << f.ebits) - 1;
+    const uint64_t fmask = (1ull << f.fbits) - 1;
+    const unsigned shift = f.ebits + f.fbits;
+    const uint64_t b = f64_bits(v);
+    const uint64_t sign = (b >> 63) << shift;
+    const uint64_t finite_emax = top_exponent_is_special(f) ? emask - 1 : emask;
+    const uint64_t overflow = sign | (f.infs ? emask << f.fbits : (finite_emax << f.fbits) | fmask);
+    const uint64_t mag = b & 0x7FFFFFFFFFFFFFFFull;
+    if (mag == 0) return sign;
+    const int e = (int)(mag >> 52) - 1023;                  /* unbiased, v = 1.m * 2^e */
+    const uint64_t m = (mag & 0xFFFFFFFFFFFFFull) | (1ull << 52);
+    const int emin = 1 - f.bias;                             /* smallest normal exponent */
+    /* the kept integer q counts units of 2^(max(e,emin) - fbits) */
+    int drop = 52 - (int)f.fbits + (e < emin ? emin - e : 0);
+    uint64_t q, rest, half;
+    if (drop > 62) { q = 0; rest = 1; half = 2; }            /* far below half a unit */
+    else {
+        q = m >> drop;
+        rest = m & ((1ull << drop) - 1);
+        half = 1ull << (drop - 1);
+    }
+    if (rest > half || (rest == half && (q & 1))) ++q;
+    /* a normal q carries the implicit bit, which adds one to the exponent field;
+     * a subnormal q that reaches 2^fbits becomes the smallest normal the same way */
+    const uint64_t field = e < emin ? q : ((uint64_t)(e + f.bias - 1) << f.fbits) + q;
+    if ((field >> f.fbits) > finite_emax) return overflow;
+    return sign | field;
+}
+
+static uint64_t narrow_nan(fmt_t f) {
+    const uint64_t emask = (1ull << f.ebits) - 1;
+    const uint64_t fmask = (1ull << f.fbits) - 1;
+    if (!top_exponent_is_special(f)) return (emask << f.fbits) | fmask;   /* saturates */
+    return (emask << f.fbits) | (f.finite_only ? fmask : 1ull << (f.fbits - 1));
+}
+
 uint64_t iomo_scalar_binary_ieee(int op, int dtype, uint64_t a, uint64_t b) {
-    if (dtype == IOMO_DT_I32 || dtype == IOMO_DT_U32) {
+    const unsigned width = integer_width(dtype);
+    if (width == 64) {
+        if (op == IOMO_OP_ADD) return a + b;
+        if (op == IOMO_OP_MUL) return a * b;
+        return a - b;
+    }
+    if (width) {
+        /* two's-complement wrap in the native width */
         const uint32_t x = (uint32_t)a, y = (uint32_t)b;
-        if (op == IOMO_OP_ADD) return (uint32_t)(x + y);
-        if (op == IOMO_OP_MUL) return (uint32_t)(x * y);
-        return (uint32_t)(x - y);
+        const uint32_t mask = width == 32 ? 0xFFFFFFFFu : (1u << width) - 1;
+        if (op == IOMO_OP_ADD) return (uint32_t)(x + y) & mask;
+        if (op == IOMO_OP_MUL) return (uint32_t)(x * y) & mask;
+        return (uint32_t)(x - y) & mask;
     }
     if (dtype == IOMO_DT_F32) {
         const volatile float x = f32_from_bits((uint32_t)a);
@@ -202,6 +333,18 @@ uint64_t iomo_scalar_binary_ieee(int op, int dtype, uint64_t a, uint64_t b) {
         else r = x - y;
         if (r != r) return 0x7FC00000u;
         return f32_bits(r);
+    }
+    if (dtype == IOMO_DT_F64) {
+        /* binary64 carrier: the rule of a backend without an extended type
+         * (src/shared/standard_tiled_add.inl:116).  The x87 carrier of the host
+         * codec rounds twice here and may differ in the last place. */
+        const volatile double x = f64_from_bits(a), y = f64_from_bits(b);
+        volatile double r;
+        if (op == IOMO_OP_ADD) r = x + y;
+        else if (op == IOMO_OP_MUL) r = x * y;
+        else r = x - y;
+        if (r != r) return 0x7FF8000000000000ull;
+        return f64_bits(r);
     }
     if (dtype == IOMO_DT_BF16) {
         const float x = f32_from_bits((uint32_t)a << 16);
@@ -233,7 +376,34 @@ uint64_t iomo_scalar_binary_ieee(int op, int dtype, uint64_t a, uint64_t b) {
         const volatile float r = (op == IOMO_OP_ADD) ? x + y : x - y;
         return bf16_rne_bits(f32_bits(r));
     }
-    return 0;
+    fmt_t f;
+    if (!float_format(dtype, &f)) return 0;
+    /* F16 and the 4/6/8-bit formats: sums, differences and products of two
+     * values are exact in binary64 (at most 11 significand bits each, exponents
+     * within 2^-24 .. 2^16), so the single rounding below is the only one. */
+    int sx, sy;
+    const double x = narrow_value(a, f, &sx), y = narrow_value(b, f, &sy);
+    if (sx == 2 || sy == 2) return narrow_nan(f);
+    if (op == IOMO_OP_MUL) {
+        if ((sx == 1 && y == 0) || (sy == 1 && x == 0)) return narrow_nan(f);
+    } else if (sx == 1 && sy == 1) {
+        const int same = signbit(x) == signbit(y);
+        if ((op == IOMO_OP_ADD) != same) return narrow_nan(f);
+    }
+    double r;
+    if (op == IOMO_OP_ADD) {
+        if (x == 0 && y == 0) r = (signbit(x) && signbit(y)) ? -0.0 : 0.0;
+        else { r = x + y; if (r == 0) r = 0.0; }
+    } else if (op == IOMO_OP_MUL) {
+        r = x * y;
+    } else {
+        r = x - y;
+    }
+    if (isinf(r)) {
+        const uint64_t emask = (1ull << f.ebits) - 1;
+        return ((uint64_t)(signbit(r) ? 1 : 0) << (f.ebits + f.fbits)) | (emask << f.fbits);
+    }
+    return narrow_round(r, f);
 }
 
 /* ------------------------------------------------------------------ */
@@ -257,14 +427,33 @@ static float silu_f32(float x) {
     return num / den;
 }
 
+static double silu_f64(double x) {
+    if (isnan(x)) return NAN;
+    if (isinf(x)) return signbit(x) ? -0.0 : INFINITY;
+    if (x == 0.0) return x;
+    if (x >= 0.0) {
+        const volatile double e = exp(-x);
+        const volatile double d = 1.0 + e;
+        return x / d;
+    }
+    const volatile double t = exp(x * 0.5);
+    const volatile double xt = x * t;
+    const volatile double num = xt * t;
+    const volatile double tt = t * t;
+    const volatile double den = 1.0 + tt;
+    return num / den;
+}
+
+/* Carrier: binary32 for every leaf below F64, binary64 for F64
+ * (src/cpu/queue.cpp:1769-1773). */
 uint64_t iomo_scalar_silu(int dtype, uint64_t raw) {
     fmt_t f;
     if (!float_format(dtype, &f)) return 0;
-    /* decode through the codec in the float carrier: exact for both leaves */
-    const float x = (float)codec_decode(raw, f);
-    const float y = silu_f32(x);
-    if (isnan(y)) return (((1ull << f.ebits) - 1) << f.fbits) | (1ull << (f.fbits - 1));
-    return codec_encode((long double)y, f);
+    long double y;
+    if (dtype == IOMO_DT_F64) y = (long double)silu_f64((double)codec_decode(raw, f));
+    else y = (long double)silu_f32((float)codec_decode(raw, f));
+    if (isnan(y)) y = positive_nan();
+    return codec_encode(y, f);
 }
 
 /* ------------------------------------------------------------------ */
@@ -316,8 +505,10 @@ static void snapshot(const iomo_view* v, const uint64_t* rdims, uint32_t rrank,
 
 int iomo_binary(int op, int dtype, const iomo_view* lhs, const iomo_view* rhs,
                 const iomo_view* out, int use_ieee) {
-    const size_t bytes = iomo_leaf_bytes(dtype);
-    if (!bytes) return IOMO_ERR_UNSUPPORTED;
+    const unsigned bits = iomo_leaf_bits(dtype);
+    fmt_t numeric;
+    if (!bits || (!integer_width(dtype) && !float_format(dtype, &numeric)))
+        return IOMO_ERR_UNSUPPORTED;   /* BOOL and F8_E8M0 (src/device_ops_binary.cpp:26-46) */
     if (op < IOMO_OP_ADD || op > IOMO_OP_SUB) return IOMO_ERR_INVALID;
     if (!view_ok(lhs) || !view_ok(rhs) || !view_ok(out)) return IOMO_ERR_INVALID;
     /* src/device_ops_binary.cpp:121-143: right-aligned broadcast */
@@ -356,12 +547,12 @@ int iomo_binary(int op, int dtype, const iomo_view* lhs, const iomo_view* rhs,
                         view_rows(rhs), view_cols(rhs), rp,
                         rs.bcast_rows ? 0 : r, rs.bcast_cols ? 0 : c);
                 const uint64_t oslot = iomo_plane_slot(rows, cols, op_, r, c);
-                const uint64_t a = load_leaf(lhs->base, lslot, bytes);
-                const uint64_t b = load_leaf(rhs->base, rslot, bytes);
+                const uint64_t a = load_leaf(lhs->base, lslot, bits);
+                const uint64_t b = load_leaf(rhs->base, rslot, bits);
                 const uint64_t y = use_ieee
                         ? iomo_scalar_binary_ieee(op, dtype, a, b)
                         : iomo_scalar_binary(op, dtype, a, b);
-                store_leaf(out->base, oslot, bytes, y);
+                store_leaf(out->base, oslot, bits, y);
             }
         }
     } while (next_coord(coord, rdims, leading));
@@ -371,6 +562,38 @@ int iomo_binary(int op, int dtype, const iomo_view* lhs, const iomo_view* rhs,
 /* ------------------------------------------------------------------ */
 /* RMSNorm (src/cpu/queue.cpp:1144-1296, float carrier)                 */
 /* ------------------------------------------------------------------ */
+
+#define RMSNORM_ROWS(T, SQRT)                                                              \
+    do {                                                                                  \
+        const T divisor = (T)feats;                                                       \
+        const T epsilon = (T)eps;                                                         \
+        for (uint64_t r = 0; r < rows; ++r) {                                             \
+            volatile T sum = 0;                                                           \
+            for (uint64_t c = 0; c < feats; ++c) {                                        \
+                const T v = (T)codec_decode(                                              \
+                        load_leaf(x->base, iomo_plane_slot(rows, feats, xp, r, c), bits), f); \
+                const volatile T sq = v * v;                                              \
+                sum = sum + sq;                                                           \
+            }                                                                             \
+            const volatile T mean = sum / divisor;                                        \
+            const volatile T shifted = mean + epsilon;                                    \
+            const volatile T root = SQRT(shifted);                                        \
+            const volatile T inverse = (T)1 / root;                                       \
+            for (uint64_t c = 0; c < feats; ++c) {                                        \
+                const T v = (T)codec_decode(                                              \
+                        load_leaf(x->base, iomo_plane_slot(rows, feats, xp, r, c), bits), f); \
+                const T w = (T)codec_decode(                                              \
+                        load_leaf(scale->base,                                            \
+                                  iomo_plane_slot(1, feats, scale->plane_offset, 0, c), bits), f); \
+                const volatile T normalized = v * inverse;                                \
+                const volatile T y = normalized * w;                                      \
+                /* a NaN result is stored in its positive form (:1124-1134) */           \
+                const long double enc = (y != y) ? positive_nan() : (long double)y;       \
+                store_leaf(out->base, iomo_plane_slot(rows, feats, yp, r, c), bits,       \
+                           codec_encode(enc, f));                                         \
+            }                                                                             \
+        }                                                                                 \
+    } while (0)
 
 int iomo_rmsnorm(int dtype, const iomo_view* x, const iomo_view* scale,
                  const iomo_view* out, float eps) {
@@ -385,9 +608,8 @@ int iomo_rmsnorm(int dtype, const iomo_view* x, const iomo_view* scale,
     if (out->base == x->base || out->base == scale->base) return IOMO_ERR_INVALID;
     if (!float_format(dtype, &f)) return IOMO_ERR_UNSUPPORTED;
     if (!isfinite(eps) || eps < 0.0f) return IOMO_ERR_INVALID;
-    const size_t bytes = iomo_leaf_bytes(dtype);
+    const unsigned bits = iomo_leaf_bits(dtype);
     const uint32_t leading = x->rank - 2;
-    const float divisor = (float)feats;
     uint64_t coord[8] = {0};
     do {
         uint64_t xp = x->plane_offset, yp = out->plane_offset;
@@ -395,32 +617,9 @@ int iomo_rmsnorm(int dtype, const iomo_view* x, const iomo_view* scale,
             xp += coord[a] * x->plane_strides[a];
             yp += coord[a] * out->plane_strides[a];
         }
-        for (uint64_t r = 0; r < rows; ++r) {
-            volatile float sum = 0.0f;
-            for (uint64_t c = 0; c < feats; ++c) {
-                const float v = (float)codec_decode(
-                        load_leaf(x->base, iomo_plane_slot(rows, feats, xp, r, c), bytes), f);
-                const volatile float sq = v * v;
-                sum = sum + sq;
-            }
-            const volatile float mean = sum / divisor;
-            const volatile float shifted = mean + eps;
-            const volatile float root = sqrtf(shifted);
-            const volatile float inverse = 1.0f / root;
-            for (uint64_t c = 0; c < feats; ++c) {
-                const float v = (float)codec_decode(
-                        load_leaf(x->base, iomo_plane_slot(rows, feats, xp, r, c), bytes), f);
-                const float w = (float)codec_decode(
-                        load_leaf(scale->base,
-                                  iomo_plane_slot(1, feats, scale->plane_offset, 0, c), bytes), f);
-                const volatile float normalized = v * inverse;
-                const volatile float y = normalized * w;
-                uint64_t raw;
-                if (y != y) raw = (((1ull << f.ebits) - 1) << f.fbits) | (1ull << (f.fbits - 1));
-                else raw = codec_encode((long double)y, f);
-                store_leaf(out->base, iomo_plane_slot(rows, feats, yp, r, c), bytes, raw);
-            }
-        }
+        /* carrier: binary64 for the F64 leaf, binary32 below (:1312-1317) */
+        if (dtype == IOMO_DT_F64) RMSNORM_ROWS(double, sqrt);
+        else RMSNORM_ROWS(float, sqrtf);
     } while (next_coord(coord, x->dims, leading));
     return IOMO_OK;
 }
@@ -439,7 +638,7 @@ int iomo_silu(int dtype, const iomo_view* x, const iomo_view* y) {
     fmt_t f;
     if (!view_ok(x) || !view_ok(y) || !same_shape(x, y)) return IOMO_ERR_INVALID;
     if (!float_format(dtype, &f)) return IOMO_ERR_UNSUPPORTED;
-    const size_t bytes = iomo_leaf_bytes(dtype);
+    const unsigned bits = iomo_leaf_bits(dtype);
     const uint64_t rows = view_rows(x), cols = view_cols(x);
     const uint32_t leading = x->rank - 2;
     uint64_t coord[8] = {0};
@@ -451,16 +650,16 @@ int iomo_silu(int dtype, const iomo_view* x, const iomo_view* y) {
         }
         for (uint64_t r = 0; r < rows; ++r)
             for (uint64_t c = 0; c < cols; ++c)
-                store_leaf(y->base, iomo_plane_slot(rows, cols, yp, r, c), bytes,
+                store_leaf(y->base, iomo_plane_slot(rows, cols, yp, r, c), bits,
                            iomo_scalar_silu(dtype, load_leaf(
-                                   x->base, iomo_plane_slot(rows, cols, xp, r, c), bytes)));
+                                   x->base, iomo_plane_slot(rows, cols, xp, r, c), bits)));
     } while (next_coord(coord, x->dims, leading));
     return IOMO_OK;
 }
 
 int iomo_copy(int dtype, const iomo_view* src, const iomo_view* dst) {
-    const size_t bytes = iomo_leaf_bytes(dtype);
-    if (!bytes) return IOMO_ERR_UNSUPPORTED;
+    const unsigned bits = iomo_leaf_bits(dtype);
+    if (!bits) return IOMO_ERR_UNSUPPORTED;
     if (!view_ok(src) || !view_ok(dst) || !same_shape(src, dst)) return IOMO_ERR_INVALID;
     const uint64_t rows = view_rows(src), cols = view_cols(src);
     const uint32_t leading = src->rank - 2;
@@ -473,8 +672,8 @@ int iomo_copy(int dtype, const iomo_view* src, const iomo_view* dst) {
         }
         for (uint64_t r = 0; r < rows; ++r)
             for (uint64_t c = 0; c < cols; ++c)
-                store_leaf(dst->base, iomo_plane_slot(rows, cols, dp, r, c), bytes,
-                           load_leaf(src->base, iomo_plane_slot(rows, cols, sp, r, c), bytes));
+                store_leaf(dst->base, iomo_plane_slot(rows, cols, dp, r, c), bits,
+                           load_leaf(src->base, iomo_plane_slot(rows, cols, sp, r, c), bits));
     } while (next_coord(coord, src->dims, leading));
     return IOMO_OK;
 }
@@ -482,8 +681,8 @@ int iomo_copy(int dtype, const iomo_view* src, const iomo_view* dst) {
 /* src/cpu/tensor.cpp:79-167: the logical side is dense row-major over the
  * view's own shape. */
 int iomo_scatter(int dtype, const iomo_view* dst, const void* logical) {
-    const size_t bytes = iomo_leaf_bytes(dtype);
-    if (!bytes) return IOMO_ERR_UNSUPPORTED;
+    const unsigned bits = iomo_leaf_bits(dtype);
+    if (!bits) return IOMO_ERR_UNSUPPORTED;
     if (!view_ok(dst) || !logical) return IOMO_ERR_INVALID;
     const uint64_t rows = view_rows(dst), cols = view_cols(dst);
     const uint32_t leading = dst->rank - 2;
@@ -494,27 +693,32 @@ int iomo_scatter(int dtype, const iomo_view* dst, const void* logical) {
         for (uint32_t a = 0; a < leading; ++a) dp += coord[a] * dst->plane_strides[a];
         for (uint64_t r = 0; r < rows; ++r)
             for (uint64_t c = 0; c < cols; ++c, ++index)
-                store_leaf(dst->base, iomo_plane_slot(rows, cols, dp, r, c), bytes,
-                           load_leaf(logical, index, bytes));
+                store_leaf(dst->base, iomo_plane_slot(rows, cols, dp, r, c), bits,
+                           load_leaf(logical, index, bits));
     } while (next_coord(coord, dst->dims, leading));
     return IOMO_OK;
 }
 
 int iomo_gather(int dtype, const iomo_view* src, void* logical) {
-    const size_t bytes = iomo_leaf_bytes(dtype);
-    if (!bytes) return IOMO_ERR_UNSUPPORTED;
+    const unsigned bits = iomo_leaf_bits(dtype);
+    if (!bits) return IOMO_ERR_UNSUPPORTED;
     if (!view_ok(src) || !logical) return IOMO_ERR_INVALID;
     const uint64_t rows = view_rows(src), cols = view_cols(src);
     const uint32_t leading = src->rank - 2;
     uint64_t coord[8] = {0};
     uint64_t index = 0;
+    /* the unused high bits of a final partial byte read as zero
+     * (src/cpu/tensor.cpp:126-135) */
+    uint64_t count = 1;
+    for (uint32_t i = 0; i < src->rank; ++i) count *= src->dims[i];
+    if ((count * bits) % 8 != 0) ((unsigned char*)logical)[count * bits / 8] = 0;
     do {
         uint64_t sp = src->plane_offset;
         for (uint32_t a = 0; a < leading; ++a) sp += coord[a] * src->plane_strides[a];
         for (uint64_t r = 0; r < rows; ++r)
             for (uint64_t c = 0; c < cols; ++c, ++index)
-                store_leaf(logical, index, bytes,
-                           load_leaf(src->base, iomo_plane_slot(rows, cols, sp, r, c), bytes));
+                store_leaf(logical, index, bits,
+                           load_leaf(src->base, iomo_plane_slot(rows, cols, sp, r, c), bits));
     } while (next_coord(coord, src->dims, leading));
     return IOMO_OK;
 }

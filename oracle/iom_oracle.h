@@ -40,10 +40,13 @@ extern "C" {
 
 /* Leaf codes: numeric values of iom::DataType (include/iom/tensor.hpp:10-33). */
 enum {
-    IOMO_DT_I32 = 9,
-    IOMO_DT_U32 = 10,
-    IOMO_DT_BF16 = 20,
-    IOMO_DT_F32 = 21
+    IOMO_DT_BOOL = 0,
+    IOMO_DT_I2 = 1, IOMO_DT_U2 = 2, IOMO_DT_I4 = 3, IOMO_DT_U4 = 4,
+    IOMO_DT_I8 = 5, IOMO_DT_U8 = 6, IOMO_DT_I16 = 7, IOMO_DT_U16 = 8,
+    IOMO_DT_I32 = 9, IOMO_DT_U32 = 10, IOMO_DT_I64 = 11, IOMO_DT_U64 = 12,
+    IOMO_DT_F4_E2M1 = 13, IOMO_DT_F6_E2M3 = 14, IOMO_DT_F6_E3M2 = 15,
+    IOMO_DT_F8_E4M3FN = 16, IOMO_DT_F8_E5M2 = 17, IOMO_DT_F8_E8M0 = 18,
+    IOMO_DT_F16 = 19, IOMO_DT_BF16 = 20, IOMO_DT_F32 = 21, IOMO_DT_F64 = 22
 };
 
 /* Binary operations in the order of scalar_binary_codec.hpp:9. */
@@ -69,7 +72,9 @@ typedef struct iomo_view {
     uint64_t plane_strides[6];
 } iomo_view;
 
-/* src/tensor.cpp:107-134 (only the 16- and 32-bit leaves in scope). */
+/* src/tensor.cpp:107-134: bit width of a leaf (0 for an unknown code); bytes for
+ * the byte-sized ones (0 otherwise). */
+unsigned iomo_leaf_bits(int dtype);
 size_t iomo_leaf_bytes(int dtype);
 /* src/tensor.cpp:136-164: element slot of (plane,row,column). */
 uint64_t iomo_plane_slot(uint64_t rows, uint64_t cols, uint64_t plane,
@@ -80,7 +85,11 @@ uint64_t iomo_plane_elems(uint64_t rows, uint64_t cols);
 /* src/shared/scalar_binary_codec.hpp:163-178 with the long-double host traits
  * of src/shared/scalar_add.hpp:15-39. */
 uint64_t iomo_scalar_binary(int op, int dtype, uint64_t a, uint64_t b);
-/* Closed form: IEEE single op / wrap, canonical NaN; must equal the codec. */
+/* Closed form: one IEEE-754 operation in a carrier wide enough to be exact or
+ * innocuously rounded (binary32 for F32/BF16, binary64 for the narrower formats
+ * and for F64 itself), one rounding on the integer significand, canonical NaN,
+ * two's-complement wrap.  Must equal the codec for every leaf but F64, where
+ * the host codec's 64-bit-significand carrier rounds twice. */
 uint64_t iomo_scalar_binary_ieee(int op, int dtype, uint64_t a, uint64_t b);
 /* src/shared/scalar_silu.hpp:69-97 with the float carrier of
  * src/cpu/device_internal.hpp:20-49. */
@@ -100,7 +109,7 @@ int iomo_rmsnorm(int dtype, const iomo_view* x, const iomo_view* scale,
 int iomo_silu(int dtype, const iomo_view* x, const iomo_view* y);
 /* src/cpu/queue.cpp:2274-2303, src/device_ops_copy.cpp:9-52. */
 int iomo_copy(int dtype, const iomo_view* src, const iomo_view* dst);
-/* src/cpu/tensor.cpp:79-167: logical row-major bytes <-> tiled view. */
+/* src/cpu/tensor.cpp:79-167: logical row-major packed bits <-> tiled view. */
 int iomo_scatter(int dtype, const iomo_view* dst, const void* logical);
 int iomo_gather(int dtype, const iomo_view* src, void* logical);
 

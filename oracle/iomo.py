@@ -19,18 +19,58 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
-DT_I32, DT_U32, DT_BF16, DT_F32 = 9, 10, 20, 21
+# numeric values of iom::DataType (include/iom/tensor.hpp:10-33)
+(DT_BOOL, DT_I2, DT_U2, DT_I4, DT_U4, DT_I8, DT_U8, DT_I16, DT_U16, DT_I32, DT_U32, DT_I64,
+ DT_U64, DT_F4_E2M1, DT_F6_E2M3, DT_F6_E3M2, DT_F8_E4M3FN, DT_F8_E5M2, DT_F8_E8M0, DT_F16,
+ DT_BF16, DT_F32, DT_F64) = range(23)
+ALL_LEAVES = tuple(range(23))
+LEAF_NAME = ("BOOL I2 U2 I4 U4 I8 U8 I16 U16 I32 U32 I64 U64 F4_E2M1 F6_E2M3 F6_E3M2 "
+             "F8_E4M3FN F8_E5M2 F8_E8M0 F16 BF16 F32 F64").split()
+LEAF_BITS = (8, 2, 2, 4, 4, 8, 8, 16, 16, 32, 32, 64, 64, 4, 6, 6, 8, 8, 8, 16, 16, 32, 64)
+INTEGER_LEAVES = tuple(range(DT_I2, DT_U64 + 1))
+FLOAT_LEAVES = (DT_F4_E2M1, DT_F6_E2M3, DT_F6_E3M2, DT_F8_E4M3FN, DT_F8_E5M2, DT_F16, DT_BF16,
+                DT_F32, DT_F64)
+NUMERIC_LEAVES = INTEGER_LEAVES + FLOAT_LEAVES     # BOOL and F8_E8M0 carry no arithmetic
 OP_ADD, OP_MUL, OP_SUB = 0, 1, 2
 TILE = 16
 
-NP_OF = {DT_I32: np.uint32, DT_U32: np.uint32, DT_BF16: np.uint16, DT_F32: np.uint32,
-         5: np.uint8, 6: np.uint8, 7: np.uint16, 8: np.uint16, 19: np.uint16}
-"""Raw-bit numpy carrier of every leaf (all arithmetic is on bit patterns); the
-8- and 16-bit integer leaves and F16 appear only as opaque payloads of copies."""
+
+def carrier(dtype: int):
+    """Unsigned numpy type holding one raw element (all arithmetic is on bit patterns)."""
+    bits = LEAF_BITS[dtype]
+    return np.uint8 if bits <= 8 else {16: np.uint16, 32: np.uint32, 64: np.uint64}[bits]
+
+
+NP_OF = {d: carrier(d) for d in ALL_LEAVES}
 
 
 def leaf_bytes(dtype: int) -> int:
-    return 2 if dtype == DT_BF16 else 4
+    assert LEAF_BITS[dtype] % 8 == 0
+    return LEAF_BITS[dtype] // 8
+
+
+def pack_bits(values: np.ndarray, bits: int) -> np.ndarray:
+    """Elements -> the packed little-endian bit stream of the host format
+    (element i in bits [i*bits, (i+1)*bits), least significant bit first)."""
+    values = np.ascontiguousarray(values).reshape(-1)
+    if bits % 8 == 0:
+        return values.view(np.uint8).copy()
+    planes = np.unpackbits(values.astype(np.uint8)[:, None], axis=1, bitorder="little")[:, :bits]
+    return np.packbits(planes.reshape(-1), bitorder="little")
+
+
+def unpack_bits(stream: np.ndarray, bits: int, count: int) -> np.ndarray:
+    if bits % 8 == 0:
+        return stream.view({8: np.uint8, 16: np.uint16, 32: np.uint32, 64: np.uint64}[bits])[:count].copy()
+    flat = np.unpackbits(np.ascontiguousarray(stream, dtype=np.uint8), bitorder="little")
+    flat = flat[:count * bits].reshape(count, bits)
+    full = np.zeros((count, 8), np.uint8)
+    full[:, :bits] = flat
+    return np.packbits(full, axis=1, bitorder="little").reshape(-1)
+
+
+def packed_nbytes(count: int, bits: int) -> int:
+    return (count * bits + 7) // 8
 
 
 class View(C.Structure):
@@ -123,7 +163,12 @@ class HostTensor:
         planes = int(np.prod(self.dims[:-2], dtype=np.int64)) if len(self.dims) > 2 else 1
         self.planes = planes
         n = planes * plane_elems(self.dims[-2], self.dims[-1])
-        self.storage = np.zeros(n, dtype=NP_OF[dtype])
+        self.bits = LEAF_BITS[dtype]
+        # byte-sized leaves: one array item per slot; narrower ones: the packed bytes
+        if self.bits % 8 == 0:
+            self.storage = np.zeros(n, dtype=NP_OF[dtype])
+        else:
+            self.storage = np.zeros(n * self.bits // 8, dtype=np.uint8)
         if fill is not None:
             self.storage.view(np.uint8)[:] = fill
 
@@ -206,19 +251,28 @@ class HostView:
         return int(np.prod(self.dims, dtype=np.int64))
 
     def from_logical(self, arr: np.ndarray) -> None:
-        """region_from_host: raw-bit array of the view's logical shape."""
+        """region_from_host: one raw element per array item, in the view's logical shape."""
         arr = np.ascontiguousarray(arr, dtype=NP_OF[self.dtype]).reshape(-1)
         assert arr.size == self.logical_count
+        stream = pack_bits(arr, LEAF_BITS[self.dtype])
         cv = self.cview()
-        rc = lib().iomo_scatter(self.dtype, C.byref(cv), arr.ctypes.data)
+        rc = lib().iomo_scatter(self.dtype, C.byref(cv), stream.ctypes.data)
         assert rc == 0, rc
 
     def to_logical(self) -> np.ndarray:
-        out = np.empty(self.logical_count, dtype=NP_OF[self.dtype])
+        bits = LEAF_BITS[self.dtype]
+        stream = np.full(packed_nbytes(self.logical_count, bits), 0xEE, dtype=np.uint8)
         cv = self.cview()
-        rc = lib().iomo_gather(self.dtype, C.byref(cv), out.ctypes.data)
+        rc = lib().iomo_gather(self.dtype, C.byref(cv), stream.ctypes.data)
         assert rc == 0, rc
-        return out.reshape(self.dims)
+        return unpack_bits(stream, bits, self.logical_count).reshape(self.dims)
+
+    def slots(self) -> np.ndarray:
+        """Every slot of the owner storage as one raw element per item."""
+        o = self.owner
+        if o.bits % 8 == 0:
+            return o.storage.copy()
+        return unpack_bits(o.storage, o.bits, o.storage.size * 8 // o.bits)
 
 
 def tile_plane(logical: np.ndarray, fill=0) -> np.ndarray:
@@ -430,18 +484,27 @@ class IomView:
         return tuple(dims[:rank]), off.value, tuple(strides[:rank - 2])
 
     def from_host(self, arr: np.ndarray):
+        """One raw element per array item; packed to the host bit stream here."""
         arr = np.ascontiguousarray(arr, dtype=NP_OF[self.owner.dtype])
-        rc = self.l.iomc_view_from_host(self.owner.b.dev, self.h, arr.ctypes.data, arr.nbytes)
+        stream = pack_bits(arr, LEAF_BITS[self.owner.dtype])
+        rc = self.l.iomc_view_from_host(self.owner.b.dev, self.h, stream.ctypes.data, stream.nbytes)
         if rc != 0:
             raise RuntimeError(self.owner.b.error())
 
-    def to_host(self) -> np.ndarray:
+    def to_host_stream(self) -> np.ndarray:
+        """The packed host bytes exactly as the backend wrote them."""
         dims, _, _ = self.describe()
-        out = np.empty(int(np.prod(dims, dtype=np.int64)), dtype=NP_OF[self.owner.dtype])
-        rc = self.l.iomc_view_to_host(self.owner.b.dev, self.h, out.ctypes.data, out.nbytes)
+        bits = LEAF_BITS[self.owner.dtype]
+        stream = np.full(packed_nbytes(int(np.prod(dims, dtype=np.int64)), bits), 0xEE, np.uint8)
+        rc = self.l.iomc_view_to_host(self.owner.b.dev, self.h, stream.ctypes.data, stream.nbytes)
         if rc != 0:
             raise RuntimeError(self.owner.b.error())
-        return out.reshape(dims)
+        return stream
+
+    def to_host(self) -> np.ndarray:
+        dims, _, _ = self.describe()
+        count = int(np.prod(dims, dtype=np.int64))
+        return unpack_bits(self.to_host_stream(), LEAF_BITS[self.owner.dtype], count).reshape(dims)
 
     def raw_storage(self) -> np.ndarray:
         """Copy of the owner's raw tiled bytes (host-memory backends only)."""

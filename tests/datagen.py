@@ -24,9 +24,10 @@ def pattern_bits(bits: int, count: int, salt: int, start: int = 0) -> np.ndarray
     idx = np.arange(start, start + count, dtype=np.uint64)
     with np.errstate(over="ignore"):
         raw = splitmix64(splitmix64(idx * np.uint64(0x9E3779B97F4A7C15)) ^ np.uint64(salt))
-    if bits == 16:
-        return (raw & np.uint64(0xFFFF)).astype(np.uint16)
-    return (raw & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+    if bits == 64:
+        return raw
+    kind = np.uint8 if bits <= 8 else (np.uint16 if bits == 16 else np.uint32)
+    return (raw & np.uint64((1 << bits) - 1)).astype(kind)
 
 
 def uniform01(count: int, salt: int) -> np.ndarray:
