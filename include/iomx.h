@@ -39,12 +39,21 @@ const char* iomx_error_string(int status);
 
 /* ---- leaves and operations --------------------------------------------- */
 
-/* Numeric values of iom::DataType (include/iom/tensor.hpp:10-33). */
+/* Numeric values of iom::DataType (include/iom/tensor.hpp:10-33): the 23 leaves
+ * every standard tiled backend advertises (src/shared/standard_tiled_copy.hpp:17-31).
+ * Elements of 2, 4 and 6 bits are packed back to back, least significant bit
+ * first (src/cpu/transfer_helpers.hpp:14-40); a tile row of 16 elements is
+ * always a whole number of 32-bit words.  I32, U32, F32 and BF16 arithmetic runs
+ * on the bandwidth-tuned streaming kernels, every other leaf on the tile-row
+ * kernels. */
 enum {
-    IOMX_DT_I32 = 9,
-    IOMX_DT_U32 = 10,
-    IOMX_DT_BF16 = 20,
-    IOMX_DT_F32 = 21
+    IOMX_DT_BOOL = 0,
+    IOMX_DT_I2 = 1, IOMX_DT_U2 = 2, IOMX_DT_I4 = 3, IOMX_DT_U4 = 4,
+    IOMX_DT_I8 = 5, IOMX_DT_U8 = 6, IOMX_DT_I16 = 7, IOMX_DT_U16 = 8,
+    IOMX_DT_I32 = 9, IOMX_DT_U32 = 10, IOMX_DT_I64 = 11, IOMX_DT_U64 = 12,
+    IOMX_DT_F4_E2M1 = 13, IOMX_DT_F6_E2M3 = 14, IOMX_DT_F6_E3M2 = 15,
+    IOMX_DT_F8_E4M3FN = 16, IOMX_DT_F8_E5M2 = 17, IOMX_DT_F8_E8M0 = 18,
+    IOMX_DT_F16 = 19, IOMX_DT_BF16 = 20, IOMX_DT_F32 = 21, IOMX_DT_F64 = 22
 };
 
 /* Order of BinaryOp in src/shared/scalar_binary_codec.hpp:9. */
@@ -120,18 +129,26 @@ int iomx_event_elapsed_ms(iomx_event_t start, iomx_event_t stop, float* ms);
  * launch_grid_stride_binary / launch_alias_safe_binary
  * (src/shared/standard_tiled_add.inl:445-464,297-441) behind
  * DeviceOps::binary_impl (include/iom/iom.hpp:846-956); element rule of
- * src/shared/scalar_binary_codec.hpp:120-178.  I32/U32 wrap modulo 2^32;
- * F32 and BF16 are one IEEE operation with one round-to-nearest-even encode,
- * gradual underflow, and every NaN result stored as the positive canonical
- * quiet NaN.  An input that shares out's storage must select exactly out's
- * window (src/device_ops_binary.cpp:152-169); anything else is rejected.
+ * src/shared/scalar_binary_codec.hpp:120-178 over the 21 numeric leaves
+ * (src/device_ops_binary.cpp:26-46; BOOL and F8_E8M0 are IOMX_ERR_UNSUPPORTED).
+ * Integers wrap modulo 2^width.  Floating leaves are one IEEE operation with
+ * one round-to-nearest-even encode and gradual underflow; overflow gives
+ * infinity where the leaf has one and the largest finite magnitude otherwise
+ * (F8_E4M3FN reserves its whole top exponent for NaN and saturates at 240, as
+ * the reference codec does); every NaN result is the leaf's positive canonical
+ * NaN, or the largest finite magnitude in the 4- and 6-bit leaves, which have
+ * none.  F64 computes in binary64, the carrier of a device without an extended
+ * type (src/shared/standard_tiled_add.inl:116).  An input that shares out's
+ * storage must select exactly out's window (src/device_ops_binary.cpp:152-169);
+ * anything else is rejected.
  */
 int iomx_launch_binary(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs,
                        const iomx_view* out, iomx_stream_t stream);
 
 /*
- * out[...,r,:] = (x[...,r,:] / sqrt(mean(x^2)+eps)) * scale[0,:], F32
- * accumulation.  Replaces standard_tiled_rmsnorm_kernel
+ * out[...,r,:] = (x[...,r,:] / sqrt(mean(x^2)+eps)) * scale[0,:] over the 9
+ * floating leaves, accumulated in F32 (in F64 for the F64 leaf,
+ * src/cpu/queue.cpp:1312-1317).  Replaces standard_tiled_rmsnorm_kernel
  * (src/shared/standard_tiled_rmsnorm.inl:436-637) behind
  * DeviceOps::rmsnorm_impl; arithmetic order of src/cpu/queue.cpp:1187-1234:
  * mean = sum/F, shifted = mean+eps, root = sqrt, inverse = 1/root,
@@ -141,7 +158,8 @@ int iomx_launch_rmsnorm(int dtype, const iomx_view* x, const iomx_view* scale,
                         const iomx_view* out, float eps, iomx_stream_t stream);
 
 /*
- * y = x * sigmoid(x) in F32 with the stable two-branch form of
+ * y = x * sigmoid(x) over the 9 floating leaves, evaluated in F32 (F64 for the
+ * F64 leaf) with the stable two-branch form of
  * src/shared/scalar_silu.hpp:69-97.  Replaces silu_kernel
  * (src/rocm/copy.hip:1317-1454) behind DeviceOps::silu_impl.
  */
@@ -157,17 +175,22 @@ int iomx_launch_silu_mul(int dtype, const iomx_view* gate, const iomx_view* up,
                          const iomx_view* y, iomx_stream_t stream);
 
 /*
- * Same-spec copy of the selected planes' logical elements.  Replaces
+ * Same-spec copy of the selected planes' logical elements, any leaf.  Replaces
  * grid_stride_copy_kernel (src/shared/standard_tiled_copy_metadata.inl:241-282)
  * behind DeviceOps::copy_impl (src/device_ops_copy.cpp:9-52).
  */
 int iomx_launch_copy(int dtype, const iomx_view* src, const iomx_view* dst, iomx_stream_t stream);
 
 /*
- * Host-transfer staging: dense logical row-major bytes of the view's shape
- * (already in device memory) <-> the tiled view.  Replace scatter_plane_kernel /
- * gather_plane_kernel (src/shared/standard_tiled_copy.inl:286-310) under
- * Tensor::region_from_host / region_to_host (src/rocm/device_tensor.cpp:145-167).
+ * Host-transfer staging: the dense logical row-major bit stream of the view's
+ * shape (already in device memory) <-> the tiled view, any leaf.  Replace
+ * scatter_plane_kernel / gather_plane_kernel
+ * (src/shared/standard_tiled_copy.inl:286-310) under Tensor::region_from_host /
+ * region_to_host (src/rocm/device_tensor.cpp:145-167).  `logical` is 4-byte
+ * aligned and spans the logical byte count rounded up to 4, the size of the
+ * reference's transfer workspace (src/rocm/device_tensor.cpp:136-143): the
+ * kernels move whole 32-bit words, and gather stores the unused bits of the
+ * last word as zero (src/cpu/tensor.cpp:126-135).
  */
 int iomx_launch_scatter(int dtype, const iomx_view* dst, const void* logical, iomx_stream_t stream);
 int iomx_launch_gather(int dtype, const iomx_view* src, void* logical, iomx_stream_t stream);
@@ -202,7 +225,8 @@ int iomx_launch_softmax(const iomx_softmax_desc* desc, iomx_stream_t stream);
 /* ---- introspection (no counterpart in the reference) --------------------- */
 
 /* Which kernel family the last successful launch on this thread selected
- * ("binary_planes", "binary_rowvec", "binary_general", ...), and its grid. */
+ * ("binary_planes", "binary_rowvec", "binary_general", "rows_binary", ...), and
+ * its grid. */
 typedef struct iomx_launch_info {
     char kernel[48];
     uint32_t grid, block;

@@ -24,6 +24,7 @@ SOURCES = [
     "iomx_rmsnorm.hip",
     "iomx_softmax.hip",
     "iomx_transfer.hip",
+    "iomx_leaves.hip",
 ]
 
 # -ffp-contract=off: no fused multiply-add may replace the reference's two

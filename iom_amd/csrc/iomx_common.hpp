@@ -35,14 +35,21 @@ inline hipStream_t native(iomx_stream_t s) { return reinterpret_cast<hipStream_t
 
 void record_launch(const char* kernel, uint32_t grid, uint32_t block, uint64_t work);
 
+// Bit width of every leaf (src/tensor.cpp:107-134); 0 for an unknown code.
+inline uint32_t leaf_bits(int dtype) {
+    static const uint8_t kBits[23] = {8, 2, 2, 4, 4, 8, 8, 16, 16, 32, 32, 64, 64, 4, 6, 6,
+                                      8, 8, 8, 16, 16, 32, 64};
+    return (dtype >= 0 && dtype < 23) ? kBits[dtype] : 0;
+}
+
+// The leaves whose arithmetic runs on the streaming kernels.
+inline bool streaming_leaf(int dtype) {
+    return dtype == IOMX_DT_I32 || dtype == IOMX_DT_U32 || dtype == IOMX_DT_F32
+            || dtype == IOMX_DT_BF16;
+}
+
 inline uint32_t leaf_bytes(int dtype) {
-    switch (dtype) {
-        case IOMX_DT_BF16: return 2;
-        case IOMX_DT_I32:
-        case IOMX_DT_U32:
-        case IOMX_DT_F32: return 4;
-        default: return 0;
-    }
+    return streaming_leaf(dtype) ? leaf_bits(dtype) / 8 : 0;
 }
 
 inline bool mul_overflows(uint64_t a, uint64_t b, uint64_t* out) {
@@ -72,7 +79,7 @@ inline Matrix matrix_of(const iomx_view& v) {
 // Structural checks every operand must pass before any address is formed
 // (same facts as validate_checked_view, src/device_ops.cpp:112-206, minus the
 // owner identity that only the C++ layer knows).
-inline int check_view(const iomx_view* v, uint32_t bytes) {
+inline int check_view(const iomx_view* v, uint32_t bits) {
     if (!v || !v->base) return IOMX_ERR_INVALID;
     if (v->rank < 2 || v->rank > 8) return IOMX_ERR_INVALID;
     for (uint32_t i = 0; i < v->rank; ++i)
@@ -90,8 +97,8 @@ inline int check_view(const iomx_view* v, uint32_t bytes) {
     uint64_t end;
     if (add_overflows(max_plane, 1, &end)) return IOMX_ERR_OVERFLOW;
     if (mul_overflows(end, m.plane_elems, &end)) return IOMX_ERR_OVERFLOW;
-    if (mul_overflows(end, bytes, &end)) return IOMX_ERR_OVERFLOW;
-    if (end > (1ull << 47)) return IOMX_ERR_OVERFLOW;
+    if (mul_overflows(end, bits, &end)) return IOMX_ERR_OVERFLOW;
+    if (end / 8 > (1ull << 47)) return IOMX_ERR_OVERFLOW;
     if ((reinterpret_cast<uintptr_t>(v->base) & 15u) != 0) return IOMX_ERR_INVALID;
     return IOMX_OK;
 }

@@ -13,7 +13,7 @@
 //
 // Both read every input of a chunk before storing it, so an input that is the
 // exact alias of the output is safe without staging.
-#include "iomx_common.hpp"
+#include "iomx_leaves.hpp"
 
 namespace iomx {
 
@@ -446,11 +446,11 @@ enum AliasPolicy { ALIAS_NONE, ALIAS_EXACT, ALIAS_ANY };
 
 int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iomx_view* out,
         AliasPolicy alias, iomx_stream_t stream) {
-    const uint32_t bytes = leaf_bytes(dtype);
-    if (!bytes) return IOMX_ERR_UNSUPPORTED;
-    IOMX_TRY(check_view(lhs, bytes));
-    if (rhs) IOMX_TRY(check_view(rhs, bytes));
-    IOMX_TRY(check_view(out, bytes));
+    const uint32_t bits = leaf_bits(dtype);
+    if (!bits) return IOMX_ERR_UNSUPPORTED;
+    IOMX_TRY(check_view(lhs, bits));
+    if (rhs) IOMX_TRY(check_view(rhs, bits));
+    IOMX_TRY(check_view(out, bits));
     const bool unary = rhs == nullptr;
     if (unary) rhs = lhs;
 
@@ -500,6 +500,25 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
     if (planes_ok && op > IOMX_OP_SUB && (mode[0] != MODE_FULL || mode[1] != MODE_FULL))
         planes_ok = false;
 
+    // A copy of whole planes is a move of bytes whatever the leaf.  Everything else
+    // outside the four streaming leaves goes to the tile-row kernels.
+    const bool byte_copy = op == OP_COPY && planes_ok;
+    const bool streaming = streaming_leaf(dtype) || (op == OP_COPY && (bits == 16 || bits == 32));
+    if (!byte_copy && !streaming) {
+        RowsRequest r = {};
+        r.src[0] = static_cast<const uint8_t*>(lhs->base);
+        r.src[1] = static_cast<const uint8_t*>(rhs->base);
+        r.out = static_cast<uint8_t*>(out->base);
+        r.walk = walk;
+        for (int k = 0; k < 3; ++k) r.m[k] = m[k];
+        for (int k = 0; k < 2; ++k) { r.brow[k] = snap[k].brow; r.bcol[k] = snap[k].bcol; }
+        IOMX_TRY(launch_rows(op, dtype, r, native(stream)));
+        IOMX_HIP(hipGetLastError());
+        return IOMX_OK;
+    }
+    // byte counts below: exact for every width since a plane holds a multiple of 256 slots
+    const uint64_t bytes8 = bits;  // bits per element; sizes are formed as elems * bits / 8
+
     BinaryArgs pa = {};
     GeneralArgs ga = {};
     if (planes_ok) {
@@ -507,10 +526,10 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
         pa.src[1] = static_cast<const uint8_t*>(rhs->base);
         pa.out = static_cast<uint8_t*>(out->base);
         pa.walk = walk;
-        for (int k = 0; k < 3; ++k) pa.plane_bytes[k] = m[k].plane_elems * bytes;
+        for (int k = 0; k < 3; ++k) pa.plane_bytes[k] = m[k].plane_elems * bytes8 / 8;
         const bool rowvec = mode[0] == MODE_ROWVEC || mode[1] == MODE_ROWVEC;
-        const uint64_t plane_chunks = m[2].plane_elems * bytes / 16;
-        const uint64_t band_chunks = m[2].tile_cols * (kTileSlots * bytes / 16);
+        const uint64_t plane_chunks = m[2].plane_elems * bytes8 / 128;
+        const uint64_t band_chunks = m[2].tile_cols * (kTileSlots * bytes8 / 128);
         uint64_t planes = walk.planes;
         uint64_t segments = rowvec ? m[2].tile_rows : 1;
         pa.seg_chunks = rowvec ? band_chunks : plane_chunks;
@@ -546,7 +565,7 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
         for (int k = 0; k < 3; ++k) { ga.plane_elems[k] = m[k].plane_elems; ga.tile_cols[k] = m[k].tile_cols; }
         ga.rows = rows;
         ga.cols = cols;
-        ga.pieces_per_row = m[2].tile_cols * (kTile * bytes / 16);
+        ga.pieces_per_row = m[2].tile_cols * (kTile * bytes8 / 128);
         for (int k = 0; k < 2; ++k) { ga.brow[k] = snap[k].brow; ga.bcol[k] = snap[k].bcol; }
         uint64_t t;
         if (mul_overflows(walk.planes, rows, &t)) return IOMX_ERR_OVERFLOW;
@@ -555,7 +574,11 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
 
     const hipStream_t s = native(stream);
     int rc;
-    if (dtype == IOMX_DT_BF16) rc = dispatch<IOMX_DT_BF16>(op, planes_ok, mode[0], mode[1], pa, ga, s);
+    if (op == OP_COPY) {
+        // raw bits: the 16-bit kernels serve the padded 16-bit case, the 32-bit ones the rest
+        if (!planes_ok && bits == 16) rc = dispatch<IOMX_DT_BF16>(op, planes_ok, mode[0], mode[1], pa, ga, s);
+        else rc = dispatch<IOMX_DT_I32>(op, planes_ok, mode[0], mode[1], pa, ga, s);
+    } else if (dtype == IOMX_DT_BF16) rc = dispatch<IOMX_DT_BF16>(op, planes_ok, mode[0], mode[1], pa, ga, s);
     else if (dtype == IOMX_DT_F32) rc = dispatch<IOMX_DT_F32>(op, planes_ok, mode[0], mode[1], pa, ga, s);
     else rc = dispatch<IOMX_DT_I32>(op, planes_ok, mode[0], mode[1], pa, ga, s);
     IOMX_TRY(rc);
@@ -586,7 +609,8 @@ int iomx_launch_binary(int op, int dtype, const iomx_view* lhs, const iomx_view*
 // Admission of src/device_ops_neural.cpp:363-438: identical shapes, a floating
 // leaf, and an output that shares no storage with the input.
 int iomx_launch_silu(int dtype, const iomx_view* x, const iomx_view* y, iomx_stream_t stream) {
-    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32) return IOMX_ERR_UNSUPPORTED;
+    // the nine floating leaves (F8_E8M0 is a scale, not a number)
+    if (dtype < 13 || dtype > 22 || dtype == 18) return IOMX_ERR_UNSUPPORTED;
     if (!same_shape(x, y)) return IOMX_ERR_INVALID;
     return run(OP_SILU, dtype, x, nullptr, y, ALIAS_NONE, stream);
 }
@@ -602,10 +626,10 @@ int iomx_launch_silu_mul(int dtype, const iomx_view* gate, const iomx_view* up,
 // no-op.  Distinct windows of one owner are accepted as the reference accepts
 // them; windows that overlap partially have no defined result.
 int iomx_launch_copy(int dtype, const iomx_view* src, const iomx_view* dst, iomx_stream_t stream) {
-    if (!leaf_bytes(dtype)) return IOMX_ERR_UNSUPPORTED;
+    if (!leaf_bits(dtype)) return IOMX_ERR_UNSUPPORTED;
     if (!same_shape(src, dst)) return IOMX_ERR_INVALID;
     if (src->base == dst->base && same_window(*src, *dst)) {
-        IOMX_TRY(check_view(src, leaf_bytes(dtype)));
+        IOMX_TRY(check_view(src, leaf_bits(dtype)));
         record_launch("copy_noop", 0, 0, 0);
         return IOMX_OK;
     }

@@ -12,7 +12,7 @@
 //                    budget (at most 16 chunks per lane of a 1024-lane workgroup).
 //   rmsnorm_generic  any F and any band size: two passes over the band, the
 //                    second served by L2, with per-element column masks.
-#include "iomx_common.hpp"
+#include "iomx_leaves.hpp"
 
 namespace iomx {
 
@@ -280,18 +280,38 @@ using namespace iomx;
 // checked without owner identities).
 extern "C" int iomx_launch_rmsnorm(int dtype, const iomx_view* x, const iomx_view* scale,
                                    const iomx_view* out, float eps, iomx_stream_t stream) {
-    const uint32_t bytes = leaf_bytes(dtype);
-    if (!bytes) return IOMX_ERR_UNSUPPORTED;
-    IOMX_TRY(check_view(x, bytes));
-    IOMX_TRY(check_view(scale, bytes));
-    IOMX_TRY(check_view(out, bytes));
+    const uint32_t bits = leaf_bits(dtype);
+    if (!bits) return IOMX_ERR_UNSUPPORTED;
+    const uint32_t bytes = bits / 8;
+    IOMX_TRY(check_view(x, bits));
+    IOMX_TRY(check_view(scale, bits));
+    IOMX_TRY(check_view(out, bits));
     if (x->rank != out->rank) return IOMX_ERR_INVALID;
     for (uint32_t i = 0; i < x->rank; ++i) if (x->dims[i] != out->dims[i]) return IOMX_ERR_INVALID;
     const Matrix m = matrix_of(*x);
     if (scale->rank != 2 || scale->dims[0] != 1 || scale->dims[1] != m.cols) return IOMX_ERR_INVALID;
     if (out->base == x->base || out->base == scale->base) return IOMX_ERR_INVALID;
-    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32) return IOMX_ERR_UNSUPPORTED;
     if (!(eps >= 0.0f) || eps > 3.4028234e38f) return IOMX_ERR_INVALID;
+    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32) {
+        // the other floating leaves: one workgroup per row on packed tile rows
+        RowsRmsnormRequest r = {};
+        uint64_t rstrides[2][kMaxLead] = {};
+        uint64_t roffsets[2] = {x->plane_offset, out->plane_offset};
+        for (uint32_t i = 0; i + 2 < x->rank; ++i) {
+            rstrides[0][i] = x->plane_strides[i];
+            rstrides[1][i] = out->plane_strides[i];
+        }
+        IOMX_TRY(build_walk<2>(x->rank - 2, x->dims, rstrides, roffsets, &r.walk));
+        r.x = static_cast<const uint8_t*>(x->base);
+        r.out = static_cast<uint8_t*>(out->base);
+        r.scale = static_cast<const uint8_t*>(scale->base)
+                + scale->plane_offset * matrix_of(*scale).plane_elems * bits / 8;
+        r.m = m;
+        r.eps = eps;
+        IOMX_TRY(launch_rows_rmsnorm(dtype, r, native(stream)));
+        IOMX_HIP(hipGetLastError());
+        return IOMX_OK;
+    }
 
     RmsArgs a = {};
     uint64_t strides[2][kMaxLead] = {};

@@ -3,7 +3,7 @@
 // 16-byte piece of one logical row; a row of tiles is 32 or 64 bytes contiguous
 // on both sides, so both sides coalesce per piece.  Also the BF16 conversion
 // self test.
-#include "iomx_common.hpp"
+#include "iomx_leaves.hpp"
 
 namespace iomx {
 
@@ -71,10 +71,17 @@ namespace {
 
 int run_transfer(int dtype, const iomx_view* view, const void* logical, bool scatter,
                  iomx_stream_t stream) {
-    const uint32_t bytes = leaf_bytes(dtype);
-    if (!bytes) return IOMX_ERR_UNSUPPORTED;
-    IOMX_TRY(check_view(view, bytes));
+    const uint32_t bits = leaf_bits(dtype);
+    if (!bits) return IOMX_ERR_UNSUPPORTED;
+    IOMX_TRY(check_view(view, bits));
     if (!logical) return IOMX_ERR_INVALID;
+    if (bits != 16 && bits != 32) {
+        // every other width moves through the packed bit stream
+        IOMX_TRY(launch_bit_transfer(dtype, view, const_cast<void*>(logical), scatter, native(stream)));
+        IOMX_HIP(hipGetLastError());
+        return IOMX_OK;
+    }
+    const uint32_t bytes = bits / 8;
     const Matrix m = matrix_of(*view);
     TransferArgs a = {};
     uint64_t strides[1][kMaxLead] = {};

@@ -70,36 +70,40 @@ void check(int status, const char* what) {
     if (status != IOMX_OK) throw_status(status, what);
 }
 
-// The leaves this backend stores and moves: every 16- and 32-bit leaf.  Their
-// payload is copied as raw bits, so one code per width serves copy and transfer.
+// Leaf codes of the C ABI are the numeric values of iom::DataType.  Every leaf
+// is stored, copied and transferred; the 21 numeric leaves take the binary
+// operations (src/device_ops_binary.cpp:26-46); the 9 floating leaves take
+// rmsnorm and silu (F8_E8M0 is a scale encoding, not a number).
 int transfer_code(DataType type) {
-    switch (detail::leaf_bits(type)) {
-        case 16: return IOMX_DT_BF16;
-        case 32: return IOMX_DT_I32;
-        default: return -1;
-    }
+    const int code = static_cast<int>(type);
+    return (code >= 0 && code <= static_cast<int>(DataType::F64)) ? code : -1;
 }
 
-// Arithmetic leaves of the binary operations and of rmsnorm / silu.
 int binary_code(DataType type) {
-    switch (type) {
-        case DataType::I32: return IOMX_DT_I32;
-        case DataType::U32: return IOMX_DT_U32;
-        case DataType::F32: return IOMX_DT_F32;
-        case DataType::BF16: return IOMX_DT_BF16;
-        default: return -1;
-    }
+    if (type == DataType::BOOL || type == DataType::F8_E8M0) return -1;
+    return transfer_code(type);
 }
 
 int float_code(DataType type) {
-    if (type == DataType::F32) return IOMX_DT_F32;
-    if (type == DataType::BF16) return IOMX_DT_BF16;
-    return -1;
+    switch (type) {
+        case DataType::F4_E2M1: case DataType::F6_E2M3: case DataType::F6_E3M2:
+        case DataType::F8_E4M3FN: case DataType::F8_E5M2: case DataType::F16:
+        case DataType::BF16: case DataType::F32: case DataType::F64:
+            return static_cast<int>(type);
+        default:
+            return -1;
+    }
 }
 
-constexpr std::array<DataType, 7> kStoredLeaves = {
-        DataType::I16, DataType::U16, DataType::I32, DataType::U32,
-        DataType::F16, DataType::BF16, DataType::F32};
+// The 23 leaves of every standard tiled backend, in the order the reference
+// publishes them (src/shared/standard_tiled_copy.hpp:17-31).
+constexpr std::array<DataType, 23> kStoredLeaves = {
+        DataType::BOOL,
+        DataType::I2, DataType::U2, DataType::I4, DataType::U4, DataType::I8, DataType::U8,
+        DataType::I16, DataType::U16, DataType::I32, DataType::U32, DataType::I64, DataType::U64,
+        DataType::F4_E2M1, DataType::F6_E2M3, DataType::F6_E3M2,
+        DataType::F8_E4M3FN, DataType::F8_E5M2, DataType::F8_E8M0,
+        DataType::F16, DataType::BF16, DataType::F32, DataType::F64};
 
 iomx_view make_view(void* base, std::span<const std::size_t> dims, std::size_t plane_offset,
                     std::span<const std::size_t> plane_strides) {

@@ -12,11 +12,41 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libiomx.so")
 
-DT_I32, DT_U32, DT_BF16, DT_F32 = 9, 10, 20, 21
+# numeric values of iom::DataType (include/iom/tensor.hpp:10-33)
+(DT_BOOL, DT_I2, DT_U2, DT_I4, DT_U4, DT_I8, DT_U8, DT_I16, DT_U16, DT_I32, DT_U32, DT_I64,
+ DT_U64, DT_F4_E2M1, DT_F6_E2M3, DT_F6_E3M2, DT_F8_E4M3FN, DT_F8_E5M2, DT_F8_E8M0, DT_F16,
+ DT_BF16, DT_F32, DT_F64) = range(23)
+LEAF_BITS = (8, 2, 2, 4, 4, 8, 8, 16, 16, 32, 32, 64, 64, 4, 6, 6, 8, 8, 8, 16, 16, 32, 64)
 OP_ADD, OP_MUL, OP_SUB = 0, 1, 2
 TILE = 16
 
-NP_OF = {DT_I32: np.uint32, DT_U32: np.uint32, DT_BF16: np.uint16, DT_F32: np.uint32}
+
+def carrier(dtype: int):
+    """Unsigned numpy type that holds one raw element of the leaf."""
+    bits = LEAF_BITS[dtype]
+    return np.uint8 if bits <= 8 else {16: np.uint16, 32: np.uint32, 64: np.uint64}[bits]
+
+
+NP_OF = {d: carrier(d) for d in range(23)}
+
+
+def pack_bits(values: np.ndarray, bits: int) -> np.ndarray:
+    """One element per item -> the packed host format: element i in bits
+    [i*bits, (i+1)*bits) of a little-endian stream (src/cpu/transfer_helpers.hpp:14-40)."""
+    values = np.ascontiguousarray(values).reshape(-1)
+    if bits % 8 == 0:
+        return values.view(np.uint8)
+    planes = np.unpackbits(values.astype(np.uint8)[:, None], axis=1, bitorder="little")[:, :bits]
+    return np.packbits(planes.reshape(-1), bitorder="little")
+
+
+def unpack_bits(stream: np.ndarray, bits: int, count: int) -> np.ndarray:
+    if bits % 8 == 0:
+        return stream[:count * bits // 8].view(NP_OF[{8: 5, 16: 7, 32: 9, 64: 11}[bits]]).copy()
+    flat = np.unpackbits(np.ascontiguousarray(stream, dtype=np.uint8), bitorder="little")
+    full = np.zeros((count, 8), np.uint8)
+    full[:, :bits] = flat[:count * bits].reshape(count, bits)
+    return np.packbits(full, axis=1, bitorder="little").reshape(-1)
 
 # every symbol include/iomx.h declares
 SYMBOLS = [
@@ -221,7 +251,8 @@ def padded(n: int) -> int:
 
 
 def leaf_bytes(dtype: int) -> int:
-    return 2 if dtype == DT_BF16 else 4
+    assert LEAF_BITS[dtype] % 8 == 0
+    return LEAF_BITS[dtype] // 8
 
 
 class DeviceTensor:
@@ -234,7 +265,8 @@ class DeviceTensor:
         lead = self.dims[:-2]
         self.planes = int(np.prod(lead, dtype=np.int64)) if lead else 1
         self.plane_elems = padded(self.dims[-2]) * padded(self.dims[-1])
-        self.nbytes = self.planes * self.plane_elems * leaf_bytes(dtype)
+        self.bits = LEAF_BITS[dtype]
+        self.nbytes = self.planes * self.plane_elems * self.bits // 8
         self.buf = Buffer(self.nbytes)
         if fill is not None:
             self.buf.fill(fill)
@@ -248,8 +280,9 @@ class DeviceTensor:
         return DeviceView(self, self.dims, 0, tuple(reversed(strides)))
 
     def raw(self) -> np.ndarray:
+        """The owner storage: one item per slot for byte-sized leaves, bytes otherwise."""
         synchronize()
-        return self.buf.download(NP_OF[self.dtype])
+        return self.buf.download(NP_OF[self.dtype] if self.bits % 8 == 0 else np.uint8)
 
     def upload_raw(self, storage: np.ndarray):
         assert storage.nbytes == self.nbytes
@@ -325,12 +358,14 @@ class DeviceView:
         return int(np.prod(self.dims, dtype=np.int64))
 
     def from_host(self, arr: np.ndarray, stream: Optional[Stream] = None):
-        """copy_from_host: logical row-major raw bits -> staging -> scatter kernel."""
+        """copy_from_host: one raw element per item -> packed logical stream -> staging
+        (a whole number of 32-bit words, as the reference's workspace is) -> scatter."""
         arr = np.ascontiguousarray(arr, dtype=NP_OF[self.dtype]).reshape(-1)
         assert arr.size == self.logical_count
-        staging = Buffer(arr.nbytes)
+        stream_bytes = pack_bits(arr, LEAF_BITS[self.dtype])
+        staging = Buffer((stream_bytes.size + 3) // 4 * 4)
         try:
-            staging.upload(arr)
+            staging.upload(stream_bytes)
             cv = self.cview()
             check(lib().iomx_launch_scatter(self.dtype, C.byref(cv), staging.ptr,
                                             stream.h if stream else None), "scatter")
@@ -339,13 +374,21 @@ class DeviceView:
             staging.free()
 
     def to_host(self, stream: Optional[Stream] = None) -> np.ndarray:
-        staging = Buffer(self.logical_count * leaf_bytes(self.dtype))
+        return unpack_bits(self.to_host_stream(stream), LEAF_BITS[self.dtype],
+                           self.logical_count).reshape(self.dims)
+
+    def to_host_stream(self, stream: Optional[Stream] = None) -> np.ndarray:
+        """The packed logical bytes exactly as the gather kernel wrote them."""
+        nbytes = (self.logical_count * LEAF_BITS[self.dtype] + 7) // 8
+        staging = Buffer((nbytes + 3) // 4 * 4)
         try:
+            staging.fill(0xEE)
+            synchronize()
             cv = self.cview()
             check(lib().iomx_launch_gather(self.dtype, C.byref(cv), staging.ptr,
                                            stream.h if stream else None), "gather")
             (stream.synchronize() if stream else synchronize())
-            return staging.download(NP_OF[self.dtype]).reshape(self.dims)
+            return staging.download(np.uint8)[:nbytes]
         finally:
             staging.free()
 

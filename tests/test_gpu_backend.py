@@ -11,11 +11,12 @@ import pytest
 
 import datagen
 import iomo
-from iomo import DT_BF16, DT_F32, DT_I32, OP_ADD, OP_MUL, OP_SUB
+from iomo import (ALL_LEAVES, DT_BF16, DT_BOOL, DT_F32, DT_F64, DT_I32, FLOAT_LEAVES, LEAF_BITS,
+                  LEAF_NAME, NUMERIC_LEAVES, OP_ADD, OP_MUL, OP_SUB)
 
 pytestmark = pytest.mark.gpu
 
-BITS = {DT_BF16: 16, DT_F32: 32, DT_I32: 32, 19: 16, 7: 16}
+BITS = {d: LEAF_BITS[d] for d in ALL_LEAVES}
 
 
 @pytest.fixture(scope="module")
@@ -39,6 +40,8 @@ def both(devices, dtype, dims, salt=None, values=None):
     cpu, gpu = devices
     if salt is not None:
         values = datagen.pattern_bits(BITS[dtype], int(np.prod(dims)), salt).reshape(dims)
+        if dtype == DT_BOOL:
+            values = values & 1          # BOOL host bytes are zero or one (src/tensor_view.cpp:265-270)
     out = []
     for dev in (cpu, gpu):
         t = dev.tensor(dtype, dims)
@@ -116,18 +119,90 @@ def test_rmsnorm_and_silu_within_the_bar(devices, dtype, dims, steps):
     close(cx, gx, cw, gw, co, go, cs, gs)
 
 
-@pytest.mark.parametrize("dtype", [DT_BF16, DT_F32, DT_I32, 19, 7])   # 19 = F16, 7 = I16: moved as bits
+def test_every_standard_leaf_is_advertised_in_order(devices):
+    """23 leaves in the published order (src/shared/standard_tiled_copy.hpp:17-31); the
+    conformance drivers iterate exactly this list (test/rocm/test_rocm_conformance.cpp:225-240)."""
+    cpu, gpu = devices
+    for dtype in ALL_LEAVES:                     # creation is refused for an unadvertised leaf
+        t = gpu.tensor(dtype, (3, 5))
+        t.close()
+
+
+@pytest.mark.parametrize("dtype", ALL_LEAVES, ids=[LEAF_NAME[d] for d in ALL_LEAVES])
 def test_copy_and_host_transfer_round_trip(devices, dtype):
     cpu, gpu = devices
     dims = (6, 20, 35)
-    vals = datagen.pattern_bits(BITS[dtype], int(np.prod(dims)), 77).reshape(dims)
-    cs, gs = both(devices, dtype, dims, values=vals)
+    cs, gs = both(devices, dtype, dims, salt=77)
+    vals = cs.view().to_host()
     assert np.array_equal(gs.view().to_host(), vals)
+    assert np.array_equal(gs.view().to_host_stream(), cs.view().to_host_stream())
     cd, gd = both(devices, dtype, (3, 20, 35), salt=78)
     assert cpu.copy(cs.view().slice(0, 1, 3, 2), cd.view()) > 0
     assert gpu.copy(gs.view().slice(0, 1, 3, 2), gd.view()) > 0, gpu.error()
     assert np.array_equal(cd.view().to_host(), gd.view().to_host())
     close(cs, gs, cd, gd)
+
+
+OTHER_NUMERIC = [d for d in NUMERIC_LEAVES if d not in (DT_I32, iomo.DT_U32, DT_F32, DT_BF16)]
+
+
+@pytest.mark.parametrize("dtype", OTHER_NUMERIC, ids=[LEAF_NAME[d] for d in OTHER_NUMERIC])
+@pytest.mark.parametrize("case", [0, 1, 2, 3, 4])
+def test_binary_every_other_numeric_leaf(devices, dtype, case):
+    """Bit for bit against the reference CPU backend (F64 inputs are kept to values whose
+    sums and products are exact or far from a rounding tie of the 64-bit carrier)."""
+    cpu, gpu = devices
+    op = (OP_ADD, OP_MUL, OP_SUB)[case % 3]
+    ld, ls, rd, rs, od, os_ = CASES[case]
+    if dtype == DT_F64:
+        mk = lambda dims, salt: (datagen.uniform_i32(int(np.prod(dims)), -1000, 1000, salt)
+                                 .view(np.int32).astype(np.float64).view(np.uint64).reshape(dims))
+        cl, gl = both(devices, dtype, ld, values=mk(ld, 1 + case))
+        cr, gr = both(devices, dtype, rd, values=mk(rd, 2 + case))
+    else:
+        cl, gl = both(devices, dtype, ld, salt=0x100 + case)
+        cr, gr = both(devices, dtype, rd, salt=0x200 + case)
+    co, go = both(devices, dtype, od, salt=0x300 + case)
+    tc = cpu.binary(op, apply(cl.view(), ls), apply(cr.view(), rs), apply(co.view(), os_))
+    tg = gpu.binary(op, apply(gl.view(), ls), apply(gr.view(), rs), apply(go.view(), os_))
+    assert tc > 0 and tg > 0, (tc, tg, gpu.error())
+    assert np.array_equal(co.view().to_host(), go.view().to_host())
+    close(cl, gl, cr, gr, co, go)
+
+
+OTHER_FLOAT = [d for d in FLOAT_LEAVES if d not in (DT_F32, DT_BF16)]
+
+
+@pytest.mark.parametrize("dtype", OTHER_FLOAT, ids=[LEAF_NAME[d] for d in OTHER_FLOAT])
+def test_rmsnorm_and_silu_every_other_float_leaf(devices, dtype):
+    cpu, gpu = devices
+    dims = (3, 17, 40)
+    n = int(np.prod(dims))
+    if dtype == DT_F64:
+        xl = datagen.normal_f32(n, 0, 1, 5).astype(np.float64).view(np.uint64).reshape(dims)
+        wl = datagen.uniform_f32(40, 0.5, 1.5, 6).astype(np.float64).view(np.uint64).reshape(1, 40)
+    else:
+        # every finite-looking pattern: clear the top exponent bit so no NaN / infinity appears
+        ebits, fbits = {13: (2, 1), 14: (2, 3), 15: (3, 2), 16: (4, 3), 17: (5, 2), 19: (5, 10)}[dtype]
+        keep = ~(1 << (fbits + ebits - 1)) & ((1 << LEAF_BITS[dtype]) - 1)
+        xl = (datagen.pattern_bits(LEAF_BITS[dtype], n, 5) & keep).reshape(dims)
+        wl = (datagen.pattern_bits(LEAF_BITS[dtype], 40, 6) & keep).reshape(1, 40)
+    cx, gx = both(devices, dtype, dims, values=xl)
+    cw, gw = both(devices, dtype, (1, 40), values=wl)
+    co, go = both(devices, dtype, dims)
+    assert cpu.rmsnorm(cx.view(), cw.view(), co.view(), 1e-5) > 0
+    assert gpu.rmsnorm(gx.view(), gw.view(), go.view(), 1e-5) > 0, gpu.error()
+    cs, gs = both(devices, dtype, dims)
+    assert cpu.silu(cx.view(), cs.view()) > 0
+    assert gpu.silu(gx.view(), gs.view()) > 0, gpu.error()
+    for a, b in ((co, go), (cs, gs)):
+        a, b = a.view().to_host(), b.view().to_host()
+        if dtype == DT_F64:
+            fa, fb = a.view(np.float64), b.view(np.float64)
+            assert np.max(np.abs(fa - fb) / np.maximum(np.abs(fa), 1e-300)) <= 1e-12
+        else:
+            assert np.abs(a.astype(np.int64) - b.astype(np.int64)).max() <= 1   # one encoding step
+    close(cx, gx, cw, gw, co, go, cs, gs)
 
 
 def test_error_classes_match_the_reference(devices):
@@ -143,14 +218,19 @@ def test_error_classes_match_the_reference(devices):
         assert dev.rmsnorm(a.view(), w.view(), o.view(), -1.0) == -1
         assert dev.wait(12345) != 0                                           # foreign / unsubmitted token
         close(a, b, o, w)
-    # leaves outside this backend's arithmetic scope are Unsupported, not wrong
-    h = gpu.tensor(19, (2, 16, 16))
-    assert gpu.binary(OP_ADD, h.view(), h.view(), h.view()) == -2
-    ho = gpu.tensor(19, (2, 16, 16))
-    assert gpu.silu(h.view(), ho.view()) == -2
-    close(h, ho)
-    with pytest.raises(RuntimeError):
-        gpu.tensor(5, (2, 16, 16))                                            # I8 storage is not offered
+    # the two leaves that carry no arithmetic are Unsupported on both devices, and an
+    # integer leaf takes no silu
+    for dev in (cpu, gpu):
+        for dtype in (DT_BOOL, iomo.DT_F8_E8M0):
+            h = dev.tensor(dtype, (2, 16, 16))
+            ho = dev.tensor(dtype, (2, 16, 16))
+            assert dev.binary(OP_ADD, h.view(), h.view(), ho.view()) == -2
+            assert dev.silu(h.view(), ho.view()) == -2
+            close(h, ho)
+        i = dev.tensor(iomo.DT_I16, (2, 16, 16))
+        io = dev.tensor(iomo.DT_I16, (2, 16, 16))
+        assert dev.silu(i.view(), io.view()) == -2
+        close(i, io)
     # a view of the other device is rejected by the queue
     ca = cpu.tensor(DT_F32, (2, 16, 16))
     ga = gpu.tensor(DT_F32, (2, 16, 16))

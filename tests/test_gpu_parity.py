@@ -175,9 +175,10 @@ def test_binary_rejections_match_the_reference_rules():
     assert iomx.binary(OP_ADD, a.view(), b.view(), o.view()) == -1          # not broadcastable
     assert iomx.binary(OP_ADD, a.view(), a.view(), b.view()) == -1          # wrong output shape
     assert iomx.binary(7, a.view(), a.view(), o.view()) == -1               # unknown operation
-    assert iomx.lib().iomx_launch_binary(OP_ADD, 19, C.byref(a.view().cview()),
-                                         C.byref(a.view().cview()), C.byref(o.view().cview()),
-                                         None) == -2                          # F16 is out of scope
+    for code in (0, 18, 23, -1):         # BOOL, F8_E8M0: no arithmetic; unknown leaf codes
+        assert iomx.lib().iomx_launch_binary(OP_ADD, code, C.byref(a.view().cview()),
+                                             C.byref(a.view().cview()), C.byref(o.view().cview()),
+                                             None) == -2
     # an input sharing the output's storage through a different window is forbidden
     assert iomx.binary(OP_ADD, big.view().slice(0, 0, 2), a.view(), big.view().slice(0, 1, 2)) == -1
     for t in (a, b, o, big):
