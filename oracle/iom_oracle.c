@@ -724,6 +724,150 @@ int iomo_gather(int dtype, const iomo_view* src, void* logical) {
 }
 
 /* ------------------------------------------------------------------ */
+/* Cache append, embedding, RoPE                                        */
+/* ------------------------------------------------------------------ */
+
+/* src/cpu/queue.cpp:2227-2272, admission of src/device_ops_cache_append.cpp:160-270
+ * (what can be checked without owner identities). */
+int iomo_cache_append(int dtype, const iomo_view* src, const iomo_view* dst, uint64_t a) {
+    const unsigned bits = iomo_leaf_bits(dtype);
+    if (!view_ok(src) || !view_ok(dst)) return IOMO_ERR_INVALID;
+    if (src->rank < 3 || src->rank != dst->rank) return IOMO_ERR_INVALID;
+    const uint32_t rank = src->rank;
+    for (uint32_t i = 0; i + 2 < rank; ++i)
+        if (src->dims[i] != dst->dims[i]) return IOMO_ERR_INVALID;
+    if (view_cols(src) != view_cols(dst)) return IOMO_ERR_INVALID;
+    const uint64_t capacity = view_rows(dst), rows = view_rows(src), feats = view_cols(src);
+    if (a > capacity || rows > capacity - a) return IOMO_ERR_INVALID;
+    if (src->base == dst->base) return IOMO_ERR_INVALID;
+    if (!bits) return IOMO_ERR_UNSUPPORTED;
+    const uint32_t leading = rank - 2;
+    uint64_t coord[8] = {0};
+    do {
+        uint64_t sp = src->plane_offset, dp = dst->plane_offset;
+        for (uint32_t k = 0; k < leading; ++k) {
+            sp += coord[k] * src->plane_strides[k];
+            dp += coord[k] * dst->plane_strides[k];
+        }
+        for (uint64_t r = 0; r < rows; ++r)
+            for (uint64_t c = 0; c < feats; ++c)
+                store_leaf(dst->base, iomo_plane_slot(capacity, feats, dp, a + r, c), bits,
+                           load_leaf(src->base, iomo_plane_slot(rows, feats, sp, r, c), bits));
+    } while (next_coord(coord, src->dims, leading));
+    return IOMO_OK;
+}
+
+/* src/cpu/queue.cpp:941-1038.  table [V,F] (rank two, one selected plane), indices
+ * [...,1,R] of an integer leaf, out [...,R,F].  Every index is checked before
+ * anything is written; a negative or out-of-vocabulary one gives
+ * IOMO_ERR_INVALID (the CPU worker's deferred std::invalid_argument). */
+int iomo_embedding(int dtype, int index_dtype, const iomo_view* table, const iomo_view* indices,
+                   const iomo_view* out) {
+    const unsigned bits = iomo_leaf_bits(dtype);
+    const unsigned ibits = integer_width(index_dtype);
+    if (!view_ok(table) || !view_ok(indices) || !view_ok(out)) return IOMO_ERR_INVALID;
+    if (table->rank != 2 || indices->rank != out->rank) return IOMO_ERR_INVALID;
+    const uint32_t rank = out->rank;
+    for (uint32_t i = 0; i + 2 < rank; ++i)
+        if (indices->dims[i] != out->dims[i]) return IOMO_ERR_INVALID;
+    const uint64_t run = view_cols(indices), vocab = table->dims[0], feats = table->dims[1];
+    if (view_rows(indices) != 1 || view_rows(out) != run || view_cols(out) != feats)
+        return IOMO_ERR_INVALID;
+    if (out->base == table->base || out->base == indices->base) return IOMO_ERR_INVALID;
+    if (!bits || !ibits) return IOMO_ERR_UNSUPPORTED;
+    const int is_signed = index_dtype == IOMO_DT_I2 || index_dtype == IOMO_DT_I4
+            || index_dtype == IOMO_DT_I8 || index_dtype == IOMO_DT_I16
+            || index_dtype == IOMO_DT_I32 || index_dtype == IOMO_DT_I64;
+    const uint32_t leading = rank - 2;
+    for (int pass = 0; pass < 2; ++pass) {
+        uint64_t coord[8] = {0};
+        do {
+            uint64_t ip = indices->plane_offset, op = out->plane_offset;
+            for (uint32_t k = 0; k < leading; ++k) {
+                ip += coord[k] * indices->plane_strides[k];
+                op += coord[k] * out->plane_strides[k];
+            }
+            for (uint64_t r = 0; r < run; ++r) {
+                const uint64_t raw = load_leaf(indices->base, iomo_plane_slot(1, run, ip, 0, r), ibits);
+                if (pass == 0) {
+                    if (is_signed && ((raw >> (ibits - 1)) & 1)) return IOMO_ERR_INVALID;
+                    if (raw >= vocab) return IOMO_ERR_INVALID;
+                    continue;
+                }
+                for (uint64_t f = 0; f < feats; ++f)
+                    store_leaf(out->base, iomo_plane_slot(run, feats, op, r, f), bits,
+                               load_leaf(table->base,
+                                         iomo_plane_slot(vocab, feats, table->plane_offset, raw, f), bits));
+            }
+        } while (next_coord(coord, out->dims, leading));
+    }
+    return IOMO_OK;
+}
+
+/* src/cpu/queue.cpp:1341-1581: split-half rotary encoding of [...,H,R,D] in the
+ * carrier T (binary32 below F64, binary64 for F64).  A row at absolute position 0
+ * is a raw copy; otherwise for c < D/2: frequency = pow(theta, -2c/D),
+ * angle = position * frequency, and the four products and the following
+ * subtraction / addition stay separate roundings. */
+#define ROPE_ROWS(T, POW, SIN, COS)                                                        \
+    do {                                                                                  \
+        const T base = (T)theta;                                                          \
+        for (uint64_t r = 0; r < rows; ++r) {                                             \
+            const uint64_t position = a + r;                                              \
+            if (position == 0) {                                                          \
+                for (uint64_t c = 0; c < width; ++c)                                      \
+                    store_leaf(out->base, iomo_plane_slot(rows, width, yp, r, c), bits,   \
+                               load_leaf(x->base, iomo_plane_slot(rows, width, xp, r, c), bits)); \
+                continue;                                                                 \
+            }                                                                             \
+            for (uint64_t c = 0; c < half; ++c) {                                         \
+                const T first = (T)codec_decode(                                          \
+                        load_leaf(x->base, iomo_plane_slot(rows, width, xp, r, c), bits), f); \
+                const T second = (T)codec_decode(                                         \
+                        load_leaf(x->base, iomo_plane_slot(rows, width, xp, r, c + half), bits), f); \
+                const T exponent = (T)((-2.0 * (double)c) / (double)width);               \
+                const T frequency = POW(base, exponent);                                  \
+                const T angle = (T)position * frequency;                                  \
+                const T sine = SIN(angle), cosine = COS(angle);                           \
+                const volatile T p0 = first * cosine;                                     \
+                const volatile T p1 = second * sine;                                      \
+                const volatile T o0 = p0 - p1;                                            \
+                const volatile T p2 = second * cosine;                                    \
+                const volatile T p3 = first * sine;                                       \
+                const volatile T o1 = p2 + p3;                                            \
+                store_leaf(out->base, iomo_plane_slot(rows, width, yp, r, c), bits,       \
+                           codec_encode((long double)o0, f));                             \
+                store_leaf(out->base, iomo_plane_slot(rows, width, yp, r, c + half), bits, \
+                           codec_encode((long double)o1, f));                             \
+            }                                                                             \
+        }                                                                                 \
+    } while (0)
+
+int iomo_rope(int dtype, const iomo_view* x, const iomo_view* out, uint64_t a, double theta) {
+    fmt_t f;
+    if (!view_ok(x) || !view_ok(out) || !same_shape(x, out) || x->rank < 3) return IOMO_ERR_INVALID;
+    const uint64_t rows = view_rows(x), width = view_cols(x), half = width / 2;
+    if (width % 2 != 0) return IOMO_ERR_INVALID;
+    if (a + (rows - 1) > (1ull << 24)) return IOMO_ERR_INVALID;   /* binary32-exact positions */
+    if (out->base == x->base) return IOMO_ERR_INVALID;
+    if (!isfinite(theta) || theta < 1.0 || theta > 3.4028234663852886e38) return IOMO_ERR_INVALID;
+    if (!float_format(dtype, &f)) return IOMO_ERR_UNSUPPORTED;
+    const unsigned bits = iomo_leaf_bits(dtype);
+    const uint32_t leading = x->rank - 2;
+    uint64_t coord[8] = {0};
+    do {
+        uint64_t xp = x->plane_offset, yp = out->plane_offset;
+        for (uint32_t k = 0; k < leading; ++k) {
+            xp += coord[k] * x->plane_strides[k];
+            yp += coord[k] * out->plane_strides[k];
+        }
+        if (dtype == IOMO_DT_F64) ROPE_ROWS(double, pow, sin, cos);
+        else ROPE_ROWS(float, powf, sinf, cosf);
+    } while (next_coord(coord, x->dims, leading));
+    return IOMO_OK;
+}
+
+/* ------------------------------------------------------------------ */
 /* Softmax stage (src/cpu/sdpa.cpp:214-309)                             */
 /* ------------------------------------------------------------------ */
 

@@ -24,6 +24,10 @@
  *   iomo_softmax         special-row KATs test/rocm/test_rocm_sdpa_nonmatrix.cpp:607-648,
  *                        sum-to-one invariant, and the compiled reference's sdpa
  *                        driven with identity K and V.
+ *   iomo_cache_append / iomo_embedding / iomo_rope
+ *                        compiled reference, bit for bit (rope with the same libm);
+ *                        rope also against a float64 evaluation and the identity
+ *                        at position 0.
  *   iomo_copy / scatter / gather
  *                        bit identity and the closed-form slot formula
  *                        (test/test_iom.cpp:614-706), compiled reference.
@@ -112,6 +116,17 @@ int iomo_copy(int dtype, const iomo_view* src, const iomo_view* dst);
 /* src/cpu/tensor.cpp:79-167: logical row-major packed bits <-> tiled view. */
 int iomo_scatter(int dtype, const iomo_view* dst, const void* logical);
 int iomo_gather(int dtype, const iomo_view* src, void* logical);
+
+/* destination[..., h, a + r, d] = source[..., h, r, d]
+ * (src/cpu/queue.cpp:2227-2272, src/device_ops_cache_append.cpp:160-270). */
+int iomo_cache_append(int dtype, const iomo_view* src, const iomo_view* dst, uint64_t a);
+/* out[..., r, f] = table[indices[..., 0, r], f] (src/cpu/queue.cpp:941-1038);
+ * IOMO_ERR_INVALID for a negative or out-of-vocabulary index. */
+int iomo_embedding(int dtype, int index_dtype, const iomo_view* table,
+                   const iomo_view* indices, const iomo_view* out);
+/* Split-half rotary position encoding (src/cpu/queue.cpp:1341-1581,
+ * src/device_ops_neural.cpp:241-362). */
+int iomo_rope(int dtype, const iomo_view* x, const iomo_view* out, uint64_t a, double theta);
 
 /*
  * Softmax stage.  Request shape follows src/rocm/sdpa_softmax.hpp:14-62

@@ -335,6 +335,52 @@ std::int64_t iomc_sdpa(
     }
 }
 
+// destination[..., h, a + r, d] = source[..., h, r, d] (include/iom/iom.hpp:171-182).
+std::int64_t iomc_cache_append(
+        iomc_queue* queue, const iomc_view* source, iomc_view* destination, std::size_t a) {
+    return queue->ops->cache_append(source->view, destination->view, a);
+}
+
+// Split-half rotary position encoding (include/iom/iom.hpp:343-357).
+std::int64_t iomc_rope(
+        iomc_queue* queue, const iomc_view* x, iomc_view* out, std::size_t a, double theta) {
+    return queue->ops->rope(x->view, out->view, a, theta);
+}
+
+// out[b, r, f] = table[indices[b, 0, r], f] (include/iom/iom.hpp:188-223).  A backend
+// that asks for control scratch gets a workspace of exactly that size; the call then
+// waits so the scratch can be released, and reports the wait's outcome apart from the
+// submission's (0 = completed, negative = the retained failure's class).
+std::int64_t iomc_embedding(
+        iomc_device* device, iomc_queue* queue, const iomc_view* table,
+        const iomc_view* indices, iomc_view* out, int* wait_status) {
+    if (wait_status) *wait_status = 0;
+    try {
+        const iom::WorkspaceRequirements need =
+                queue->ops->embedding_workspace_requirements(
+                        table->view, indices->view, out->view);
+        std::unique_ptr<iom::RawWorkspace> workspace;
+        iom::oid token;
+        if (need.bytes == 0) {
+            token = queue->ops->embedding(table->view, indices->view, out->view);
+        } else {
+            workspace = device->device->create_workspace(need.bytes);
+            token = queue->ops->embedding(
+                    table->view, indices->view, out->view, workspace->view());
+        }
+        if (token > 0) {
+            try {
+                queue->ops->wait(token);
+            } catch (...) {
+                if (wait_status) *wait_status = static_cast<int>(classify(std::current_exception()));
+            }
+        }
+        return token;
+    } catch (...) {
+        return classify(std::current_exception());
+    }
+}
+
 int iomc_wait(iomc_queue* queue, std::int64_t token) {
     return guarded_status([&] { queue->ops->wait(token); });
 }

@@ -132,6 +132,9 @@ def lib() -> C.CDLL:
         l.iomo_scatter.argtypes = [C.c_int, VP, C.c_void_p]
         l.iomo_gather.argtypes = [C.c_int, VP, C.c_void_p]
         l.iomo_softmax.argtypes = [C.POINTER(SoftmaxDesc)]
+        l.iomo_cache_append.argtypes = [C.c_int, VP, VP, C.c_uint64]
+        l.iomo_embedding.argtypes = [C.c_int, C.c_int, VP, VP, VP]
+        l.iomo_rope.argtypes = [C.c_int, VP, VP, C.c_uint64, C.c_double]
         _lib = l
     return _lib
 
@@ -320,6 +323,21 @@ def copy(src: HostView, dst: HostView) -> int:
     return lib().iomo_copy(dst.dtype, C.byref(a), C.byref(o))
 
 
+def cache_append(src: HostView, dst: HostView, a: int) -> int:
+    s, d = src.cview(), dst.cview()
+    return lib().iomo_cache_append(dst.dtype, C.byref(s), C.byref(d), a)
+
+
+def embedding(table: HostView, indices: HostView, out: HostView) -> int:
+    t, i, o = table.cview(), indices.cview(), out.cview()
+    return lib().iomo_embedding(out.dtype, indices.dtype, C.byref(t), C.byref(i), C.byref(o))
+
+
+def rope(x: HostView, out: HostView, a: int, theta: float) -> int:
+    s, o = x.cview(), out.cview()
+    return lib().iomo_rope(out.dtype, C.byref(s), C.byref(o), a, theta)
+
+
 def dense_layout(heads: int, rows: int, cols: int) -> StageLayout:
     l = StageLayout()
     l.plane_offset = 0
@@ -425,6 +443,12 @@ def bind_iomc(l: C.CDLL) -> C.CDLL:
     l.iomc_sdpa.restype = C.c_int64
     l.iomc_sdpa.argtypes = [P, P, P, P, P, P, C.c_size_t, C.c_size_t]
     l.iomc_wait.argtypes = [P, C.c_int64]
+    l.iomc_cache_append.restype = C.c_int64
+    l.iomc_cache_append.argtypes = [P, P, P, C.c_size_t]
+    l.iomc_rope.restype = C.c_int64
+    l.iomc_rope.argtypes = [P, P, P, C.c_size_t, C.c_double]
+    l.iomc_embedding.restype = C.c_int64
+    l.iomc_embedding.argtypes = [P, P, P, P, P, C.POINTER(C.c_int)]
     return l
 
 
@@ -553,6 +577,18 @@ class IomBackend:
 
     def silu(self, x, y) -> int:
         return self.run(self.l.iomc_silu(self.queue, x.h, y.h))
+
+    def cache_append(self, src, dst, a) -> int:
+        return self.run(self.l.iomc_cache_append(self.queue, src.h, dst.h, a))
+
+    def rope(self, x, out, a, theta) -> int:
+        return self.run(self.l.iomc_rope(self.queue, x.h, out.h, a, theta))
+
+    def embedding(self, table, indices, out):
+        """(token or negative oid, wait status: 0 or the retained failure's class)."""
+        status = C.c_int(0)
+        token = self.l.iomc_embedding(self.dev, self.queue, table.h, indices.h, out.h, C.byref(status))
+        return token, status.value
 
     def sdpa(self, q, k, v, out, a, L) -> int:
         return self.run(self.l.iomc_sdpa(self.dev, self.queue, q.h, k.h, v.h, out.h, a, L))
