@@ -195,6 +195,47 @@ int iomx_launch_copy(int dtype, const iomx_view* src, const iomx_view* dst, iomx
 int iomx_launch_scatter(int dtype, const iomx_view* dst, const void* logical, iomx_stream_t stream);
 int iomx_launch_gather(int dtype, const iomx_view* src, void* logical, iomx_stream_t stream);
 
+/*
+ * destination[..., h, a + r, d] = source[..., h, r, d]: appends R rows to a cache
+ * of capacity C at the explicit row offset a, any leaf, raw bits.  Replaces the
+ * cache-append kernel of the standard tiled backends (src/rocm/copy.hip:132)
+ * behind DeviceOps::cache_append_impl; admission of
+ * src/device_ops_cache_append.cpp:160-270: ranks three to eight, equal leading
+ * tuples, head counts and feature widths, a <= C and then R <= C - a, distinct
+ * storages.
+ */
+int iomx_launch_cache_append(int dtype, const iomx_view* source, const iomx_view* destination,
+                             uint64_t a, iomx_stream_t stream);
+
+/*
+ * out[..., r, f] = table[indices[..., 0, r], f]: table [V,F] of rank two, indices
+ * [...,1,R] of one of the twelve integer leaves, out [...,R,F] of the table's
+ * leaf; payload bits are copied unchanged.  Replaces the gather kernel of
+ * src/shared/standard_tiled_embedding.inl behind DeviceOps::embedding_impl.
+ * `status` is one 32-bit word of device memory (the first word of the 32-byte
+ * control packet of docs/BACKEND_CONTRACT/embedding-lookup.md:178-201): the call
+ * resets it to 0 in stream order, and any negative or out-of-vocabulary id sets it
+ * to 1 without forming a table address; the caller transfers and interprets it
+ * after completion.
+ */
+int iomx_launch_embedding(int dtype, int index_dtype, const iomx_view* table,
+                          const iomx_view* indices, const iomx_view* out, uint32_t* status,
+                          iomx_stream_t stream);
+
+/*
+ * Split-half rotary position encoding of x[..., H, R, D] into out (same shape,
+ * distinct storage), row r at absolute position a + r, base theta in
+ * [1, FLT_MAX], over the 9 floating leaves: frequency = pow(theta, -2c/D),
+ * angle = position * frequency, out[c] = x[c] cos - x[c+D/2] sin,
+ * out[c+D/2] = x[c+D/2] cos + x[c] sin, evaluated in F32 (F64 for the F64 leaf)
+ * with separately rounded products; a row at position 0 is copied unchanged.
+ * Replaces the kernels of src/shared/standard_tiled_rope.inl behind
+ * DeviceOps::rope_impl; arithmetic of src/cpu/queue.cpp:1357-1411, admission of
+ * src/device_ops_neural.cpp:241-362.
+ */
+int iomx_launch_rope(int dtype, const iomx_view* x, const iomx_view* out, uint64_t a, double theta,
+                     iomx_stream_t stream);
+
 /* Element strides of one softmax-stage buffer (src/rocm/sdpa_softmax.hpp:14-22). */
 typedef struct iomx_stage_layout {
     uint64_t plane_offset, plane_stride, head_stride, row_stride, column_stride;

@@ -25,6 +25,7 @@ SOURCES = [
     "iomx_softmax.hip",
     "iomx_transfer.hip",
     "iomx_leaves.hip",
+    "iomx_layer.hip",
 ]
 
 # -ffp-contract=off: no fused multiply-add may replace the reference's two

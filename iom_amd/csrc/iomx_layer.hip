@@ -1,0 +1,476 @@
+// The remaining non-contraction operations of a transformer layer: cache-row
+// append, embedding row lookup, split-half rotary position encoding.  All three
+// work on tile rows (sixteen packed elements, whole 32-bit words) of any leaf.
+#include "iomx_rows.hpp"
+
+namespace iomx {
+
+// ---------------------------------------------------------------------------
+// Cache append: destination[..., a + r, :] = source[..., r, :]
+// ---------------------------------------------------------------------------
+
+struct AppendArgs {
+    const uint8_t* src;
+    uint8_t* dst;
+    PlaneWalk<2> walk;  // 0 source, 1 destination
+    uint64_t plane_bytes[2];
+    uint32_t tile_cols, rows, cols;
+    uint32_t rows_per_plane;  // padded tile rows of one source plane
+    FastDiv div_tile_cols;
+    uint32_t planes;
+    uint32_t a;
+};
+
+template <int BITS>
+__global__ __launch_bounds__(256) void cache_append_kernel(const AppendArgs a) {
+    constexpr int K = BITS / 2;
+    constexpr uint32_t kRowBytes = 2 * BITS, kTileBytes = 32 * BITS;
+    const TileRow t = tile_row_of(blockIdx.x * 256u + threadIdx.x, a.rows_per_plane, a.tile_cols,
+                                  a.div_tile_cols, a.rows, a.cols);
+    if (!t.live) return;
+    const uint32_t drow = a.a + t.row;
+    const uint64_t soff = ((uint64_t)(t.row >> 4) * a.tile_cols + t.tc) * kTileBytes + (t.row & 15u) * kRowBytes;
+    const uint64_t doff = ((uint64_t)(drow >> 4) * a.tile_cols + t.tc) * kTileBytes + (drow & 15u) * kRowBytes;
+    for (uint32_t p = blockIdx.y; p < a.planes; p += gridDim.y) {
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        uint32_t w[K];
+        load_row<BITS>(a.src + plane[0] * a.plane_bytes[0] + soff, w);
+        store_row<BITS>(a.dst + plane[1] * a.plane_bytes[1] + doff, w, t.ncols);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Embedding: out[..., r, :] = table[indices[..., 0, r], :]
+// ---------------------------------------------------------------------------
+
+struct EmbedArgs {
+    const uint8_t* table;    // the selected table plane
+    const uint8_t* indices;
+    uint8_t* out;
+    uint32_t* status;        // set to 1 by any lane that meets an invalid id
+    PlaneWalk<2> walk;       // 0 indices, 1 out
+    uint64_t index_plane_bytes, out_plane_bytes;
+    uint32_t tile_cols, run, feats;
+    uint32_t rows_per_plane;
+    FastDiv div_tile_cols;
+    uint32_t planes;
+    uint32_t index_signed;
+    uint64_t vocabulary;
+};
+
+__global__ void store_word_kernel(uint32_t* p, uint32_t v) { *p = v; }
+
+// An id is decoded at its full width, its sign bit is inspected before any
+// conversion and the unsigned value is compared with the vocabulary before any
+// address is formed (docs/BACKEND_CONTRACT/embedding-lookup.md:262-268); an
+// invalid id raises the status word and its output row is left alone.
+template <int BITS, int IBITS>
+__global__ __launch_bounds__(256) void embedding_kernel(const EmbedArgs a) {
+    constexpr int K = BITS / 2;
+    constexpr uint32_t kRowBytes = 2 * BITS, kTileBytes = 32 * BITS;
+    const TileRow t = tile_row_of(blockIdx.x * 256u + threadIdx.x, a.rows_per_plane, a.tile_cols,
+                                  a.div_tile_cols, a.run, a.feats);
+    if (!t.live) return;
+    // element r of an [1,R] plane: row 0 of tile r/16
+    const uint64_t index_bit = ((uint64_t)(t.row >> 4) * kTileSlots + (t.row & 15u)) * IBITS;
+    const uint64_t ooff = ((uint64_t)(t.row >> 4) * a.tile_cols + t.tc) * kTileBytes + (t.row & 15u) * kRowBytes;
+    for (uint32_t p = blockIdx.y; p < a.planes; p += gridDim.y) {
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        const uint64_t raw = read_bits<IBITS>(
+                reinterpret_cast<const uint32_t*>(a.indices + plane[0] * a.index_plane_bytes), index_bit);
+        const bool negative = a.index_signed && ((raw >> (IBITS - 1)) & 1ull);
+        if (negative || raw >= a.vocabulary) {
+            *a.status = 1u;
+            continue;
+        }
+        const uint64_t toff = ((raw >> 4) * a.tile_cols + t.tc) * kTileBytes + (raw & 15ull) * kRowBytes;
+        uint32_t w[K];
+        load_row<BITS>(a.table + toff, w);
+        store_row<BITS>(a.out + plane[1] * a.out_plane_bytes + ooff, w, t.ncols);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// RoPE (split halves): for c < D/2 and position = a + row,
+//   frequency = pow(theta, -2c/D), angle = position * frequency,
+//   out[c]       = x[c] * cos - x[c + D/2] * sin
+//   out[c + D/2] = x[c + D/2] * cos + x[c] * sin
+// in binary32 (binary64 for F64), four products and one subtraction / addition
+// as separate roundings, one encode per result; a row at position 0 is a raw
+// copy (src/cpu/queue.cpp:1357-1411,1498-1521).  The angle depends on the row
+// and the column only, so a lane evaluates its sixteen sine / cosine pairs once
+// and reuses them for every plane it walks.
+// ---------------------------------------------------------------------------
+
+struct RopeArgs {
+    const uint8_t* x;
+    uint8_t* out;
+    PlaneWalk<2> walk;  // 0 x, 1 out
+    uint64_t plane_bytes;
+    uint32_t rows, width, half, tile_cols;
+    uint32_t col_tiles;       // tiles a lane index runs over: pair tiles (aligned) or all tiles
+    uint32_t lanes_per_plane;
+    FastDiv div_col_tiles;
+    uint32_t planes;
+    uint32_t a;
+    double theta;
+};
+
+template <int DT, typename T>
+__device__ __forceinline__ T rope_decode(uint64_t raw) {
+    if constexpr (DT == DT_BF16) return (T)as_f32((uint32_t)raw << 16);
+    else if constexpr (DT == DT_F32) return (T)as_f32((uint32_t)raw);
+    else return (T)decode<DT>(raw);
+}
+
+template <int DT, typename T>
+__device__ __forceinline__ uint64_t rope_encode(T v) {
+    if constexpr (DT == DT_BF16) return bf16_rne_sw(as_u32((float)v));
+    else if constexpr (DT == DT_F32) return as_u32(canonical((float)v));
+    else return encode<DT>((double)v);
+}
+
+__device__ __forceinline__ void rope_angle(uint32_t column, uint32_t width, uint32_t position,
+                                           float theta, float* sine, float* cosine) {
+    const float exponent = (float)((-2.0 * (double)column) / (double)width);
+    const float frequency = powf(theta, exponent);
+    const float angle = (float)position * frequency;
+    sincosf(angle, sine, cosine);
+}
+__device__ __forceinline__ void rope_angle(uint32_t column, uint32_t width, uint32_t position,
+                                           double theta, double* sine, double* cosine) {
+    const double exponent = (-2.0 * (double)column) / (double)width;
+    const double frequency = pow(theta, exponent);
+    const double angle = (double)position * frequency;
+    sincos(angle, sine, cosine);
+}
+
+// D/2 a multiple of 16: a lane owns tile rows tc and tc + D/32 of one row.
+template <int DT, typename T>
+__global__ __launch_bounds__(256) void rope_pairs_kernel(const RopeArgs a) {
+    constexpr int BITS = bits_of(DT);
+    constexpr int K = BITS / 2;
+    constexpr uint32_t kRowBytes = 2 * BITS, kTileBytes = 32 * BITS;
+    const uint32_t g = blockIdx.x * 256u + threadIdx.x;
+    if (g >= a.lanes_per_plane) return;
+    const uint32_t r = g & 15u, q = g >> 4;
+    const uint32_t tr = a.col_tiles > 1 ? fast_div(q, a.div_col_tiles) : q;
+    const uint32_t ptc = q - tr * a.col_tiles;
+    const uint32_t row = tr * kTile + r;
+    if (row >= a.rows) return;
+    const uint32_t position = a.a + row;
+    T sine[kTile], cosine[kTile];
+    if (position != 0) {
+#pragma unroll
+        for (int i = 0; i < (int)kTile; ++i)
+            rope_angle(ptc * kTile + i, a.width, position, (T)a.theta, &sine[i], &cosine[i]);
+    }
+    const uint64_t off0 = ((uint64_t)tr * a.tile_cols + ptc) * kTileBytes + r * kRowBytes;
+    const uint64_t off1 = off0 + (uint64_t)(a.half >> 4) * kTileBytes;
+    for (uint32_t p = blockIdx.y; p < a.planes; p += gridDim.y) {
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        const uint8_t* xb = a.x + plane[0] * a.plane_bytes;
+        uint8_t* ob = a.out + plane[1] * a.plane_bytes;
+        uint32_t w0[K], w1[K];
+        load_row<BITS>(xb + off0, w0);
+        load_row<BITS>(xb + off1, w1);
+        if (position != 0) {
+            uint32_t r0[K], r1[K];
+#pragma unroll
+            for (int j = 0; j < K; ++j) { r0[j] = 0; r1[j] = 0; }
+#pragma unroll
+            for (int i = 0; i < (int)kTile; ++i) {
+                const T first = rope_decode<DT, T>(get<BITS>(w0, i));
+                const T second = rope_decode<DT, T>(get<BITS>(w1, i));
+                const T fc = first * cosine[i], ss = second * sine[i];
+                const T sc = second * cosine[i], fs = first * sine[i];
+                put<BITS>(r0, i, rope_encode<DT, T>(fc - ss));
+                put<BITS>(r1, i, rope_encode<DT, T>(sc + fs));
+            }
+            store_row<BITS>(ob + off0, r0, kTile);
+            store_row<BITS>(ob + off1, r1, kTile);
+        } else {
+            store_row<BITS>(ob + off0, w0, kTile);
+            store_row<BITS>(ob + off1, w1, kTile);
+        }
+    }
+}
+
+// Any even D: a lane owns one output tile row and fetches each partner element
+// from wherever the other half puts it.
+template <int DT, typename T>
+__global__ __launch_bounds__(256) void rope_general_kernel(const RopeArgs a) {
+    constexpr int BITS = bits_of(DT);
+    constexpr int K = BITS / 2;
+    constexpr uint32_t kRowBytes = 2 * BITS, kTileBytes = 32 * BITS;
+    const TileRow t = tile_row_of(blockIdx.x * 256u + threadIdx.x, a.lanes_per_plane, a.tile_cols,
+                                  a.div_col_tiles, a.rows, a.width);
+    if (!t.live) return;
+    const uint32_t position = a.a + t.row;
+    T sine[kTile], cosine[kTile];
+    if (position != 0) {
+#pragma unroll
+        for (int i = 0; i < (int)kTile; ++i) {
+            const uint32_t c = t.tc * kTile + i;
+            if (c < a.width)
+                rope_angle(c < a.half ? c : c - a.half, a.width, position, (T)a.theta, &sine[i], &cosine[i]);
+        }
+    }
+    const uint64_t row_base = (uint64_t)(t.row >> 4) * a.tile_cols * kTileBytes + (t.row & 15u) * kRowBytes;
+    const uint64_t off = row_base + (uint64_t)t.tc * kTileBytes;
+    for (uint32_t p = blockIdx.y; p < a.planes; p += gridDim.y) {
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        const uint8_t* xb = a.x + plane[0] * a.plane_bytes;
+        uint32_t w[K], res[K];
+        load_row<BITS>(xb + off, w);
+        if (position != 0) {
+#pragma unroll
+            for (int j = 0; j < K; ++j) res[j] = 0;
+#pragma unroll
+            for (int i = 0; i < (int)kTile; ++i) {
+                const uint32_t c = t.tc * kTile + i;
+                if (c >= a.width) continue;
+                const bool low = c < a.half;
+                const uint32_t partner = low ? c + a.half : c - a.half;
+                // bit address of the partner inside this row of tiles
+                const uint64_t bit = (row_base + (uint64_t)(partner >> 4) * kTileBytes) * 8ull
+                        + (uint64_t)(partner & 15u) * BITS;
+                const T own = rope_decode<DT, T>(get<BITS>(w, i));
+                const T other = rope_decode<DT, T>(read_bits<BITS>(reinterpret_cast<const uint32_t*>(xb), bit));
+                // low half: first*cos - second*sin; high half: second*cos + first*sin, where
+                // this lane's own element is `first` in the low half and `second` in the high
+                const T oc = own * cosine[i], os = other * sine[i];
+                const T y = low ? oc - os : oc + os;
+                put<BITS>(res, i, rope_encode<DT, T>(y));
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < K; ++j) res[j] = w[j];
+        }
+        store_row<BITS>(a.out + plane[1] * a.plane_bytes + off, res, t.ncols);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+
+namespace {
+
+bool same_leading(const iomx_view* a, const iomx_view* b, uint32_t axes) {
+    for (uint32_t i = 0; i < axes; ++i) if (a->dims[i] != b->dims[i]) return false;
+    return true;
+}
+
+template <int N>
+int walk_of(const iomx_view* const (&v)[N], const uint64_t* dims, uint32_t nlead, PlaneWalk<N>* w) {
+    uint64_t strides[N][kMaxLead] = {};
+    uint64_t offsets[N];
+    for (int k = 0; k < N; ++k) {
+        offsets[k] = v[k]->plane_offset;
+        for (uint32_t i = 0; i < nlead; ++i) strides[k][i] = v[k]->plane_strides[i];
+    }
+    return build_walk<N>(nlead, dims, strides, offsets, w);
+}
+
+bool is_signed_index(int dtype) {
+    return dtype == DT_I2 || dtype == DT_I4 || dtype == DT_I8 || dtype == DT_I16 || dtype == DT_I32
+            || dtype == DT_I64;
+}
+
+bool is_index_leaf(int dtype) { return dtype >= DT_I2 && dtype <= DT_U64; }
+
+// Enough planes per lane to reuse its angles, enough lanes to fill the device.
+uint32_t planes_in_grid(uint64_t lanes_per_plane, uint64_t planes) {
+    const uint64_t target = 1ull << 19;
+    uint64_t y = (target + lanes_per_plane - 1) / lanes_per_plane;
+    if (y < 1) y = 1;
+    if (y > planes) y = planes;
+    if (y > 65535) y = 65535;
+    return (uint32_t)y;
+}
+
+template <int DT, typename T>
+void launch_rope(const RopeArgs& a, bool aligned, dim3 grid, hipStream_t s) {
+    if (aligned) hipLaunchKernelGGL((rope_pairs_kernel<DT, T>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((rope_general_kernel<DT, T>), grid, dim3(256), 0, s, a);
+}
+
+}  // namespace
+}  // namespace iomx
+
+using namespace iomx;
+
+extern "C" {
+
+// Admission of src/device_ops_cache_append.cpp:160-270 (everything checkable
+// without owner identities).
+int iomx_launch_cache_append(int dtype, const iomx_view* source, const iomx_view* destination,
+                             uint64_t a, iomx_stream_t stream) {
+    const uint32_t bits = leaf_bits(dtype);
+    if (!bits) return IOMX_ERR_UNSUPPORTED;
+    IOMX_TRY(check_view(source, bits));
+    IOMX_TRY(check_view(destination, bits));
+    if (source->rank < 3 || source->rank != destination->rank) return IOMX_ERR_INVALID;
+    const uint32_t rank = source->rank;
+    if (!same_leading(source, destination, rank - 2)) return IOMX_ERR_INVALID;
+    const Matrix sm = matrix_of(*source), dm = matrix_of(*destination);
+    if (sm.cols != dm.cols) return IOMX_ERR_INVALID;
+    if (a > dm.rows || sm.rows > dm.rows - a) return IOMX_ERR_INVALID;   // in this order
+    if (source->base == destination->base) return IOMX_ERR_INVALID;
+    if (dm.rows > 0xFFFFFFFFull || sm.cols > 0xFFFFFFFFull) return IOMX_ERR_OVERFLOW;
+    AppendArgs k = {};
+    const iomx_view* v[2] = {source, destination};
+    IOMX_TRY(walk_of<2>(v, source->dims, rank - 2, &k.walk));
+    k.src = static_cast<const uint8_t*>(source->base);
+    k.dst = static_cast<uint8_t*>(destination->base);
+    k.plane_bytes[0] = sm.plane_elems * bits / 8;
+    k.plane_bytes[1] = dm.plane_elems * bits / 8;
+    k.tile_cols = (uint32_t)sm.tile_cols;
+    k.rows = (uint32_t)sm.rows;
+    k.cols = (uint32_t)sm.cols;
+    k.div_tile_cols = make_fast_div(k.tile_cols);
+    k.planes = (uint32_t)k.walk.planes;
+    k.a = (uint32_t)a;
+    dim3 grid;
+    IOMX_TRY(plane_grid(sm.tile_rows, sm.tile_cols, k.walk.planes, &k.rows_per_plane, &grid));
+    const hipStream_t s = native(stream);
+#define IOMX_APPEND(B) hipLaunchKernelGGL((cache_append_kernel<B>), grid, dim3(256), 0, s, k)
+    switch (bits) {
+        case 2: IOMX_APPEND(2); break;
+        case 4: IOMX_APPEND(4); break;
+        case 6: IOMX_APPEND(6); break;
+        case 8: IOMX_APPEND(8); break;
+        case 16: IOMX_APPEND(16); break;
+        case 32: IOMX_APPEND(32); break;
+        default: IOMX_APPEND(64); break;
+    }
+#undef IOMX_APPEND
+    record_launch("cache_append", grid.x, 256, (uint64_t)k.rows_per_plane * k.planes);
+    IOMX_HIP(hipGetLastError());
+    return IOMX_OK;
+}
+
+// Structural admission of src/device_ops_embedding.cpp (shape rules of
+// include/iom/iom.hpp:188-200).
+int iomx_launch_embedding(int dtype, int index_dtype, const iomx_view* table,
+                          const iomx_view* indices, const iomx_view* out, uint32_t* status,
+                          iomx_stream_t stream) {
+    const uint32_t bits = leaf_bits(dtype), ibits = leaf_bits(index_dtype);
+    if (!bits || !ibits) return IOMX_ERR_UNSUPPORTED;
+    IOMX_TRY(check_view(table, bits));
+    IOMX_TRY(check_view(indices, ibits));
+    IOMX_TRY(check_view(out, bits));
+    if (!status || (reinterpret_cast<uintptr_t>(status) & 3u)) return IOMX_ERR_INVALID;
+    if (table->rank != 2 || indices->rank != out->rank) return IOMX_ERR_INVALID;
+    const uint32_t rank = out->rank;
+    if (!same_leading(indices, out, rank - 2)) return IOMX_ERR_INVALID;
+    const Matrix tm = matrix_of(*table), im = matrix_of(*indices), om = matrix_of(*out);
+    if (im.rows != 1 || om.rows != im.cols || om.cols != tm.cols) return IOMX_ERR_INVALID;
+    if (out->base == table->base || out->base == indices->base) return IOMX_ERR_INVALID;
+    if (!is_index_leaf(index_dtype)) return IOMX_ERR_UNSUPPORTED;
+    if (om.rows > 0xFFFFFFFFull || om.cols > 0xFFFFFFFFull) return IOMX_ERR_OVERFLOW;
+    EmbedArgs k = {};
+    const iomx_view* v[2] = {indices, out};
+    IOMX_TRY(walk_of<2>(v, out->dims, rank - 2, &k.walk));
+    k.table = static_cast<const uint8_t*>(table->base) + table->plane_offset * (tm.plane_elems * bits / 8);
+    k.indices = static_cast<const uint8_t*>(indices->base);
+    k.out = static_cast<uint8_t*>(out->base);
+    k.status = status;
+    k.index_plane_bytes = im.plane_elems * ibits / 8;
+    k.out_plane_bytes = om.plane_elems * bits / 8;
+    k.tile_cols = (uint32_t)om.tile_cols;
+    k.run = (uint32_t)om.rows;
+    k.feats = (uint32_t)om.cols;
+    k.div_tile_cols = make_fast_div(k.tile_cols);
+    k.planes = (uint32_t)k.walk.planes;
+    k.index_signed = is_signed_index(index_dtype);
+    k.vocabulary = tm.rows;
+    dim3 grid;
+    IOMX_TRY(plane_grid(om.tile_rows, om.tile_cols, k.walk.planes, &k.rows_per_plane, &grid));
+    const hipStream_t s = native(stream);
+    hipLaunchKernelGGL(store_word_kernel, dim3(1), dim3(1), 0, s, status, 0u);
+#define IOMX_EMBED_I(B)                                                                          \
+    switch (ibits) {                                                                             \
+        case 2: hipLaunchKernelGGL((embedding_kernel<B, 2>), grid, dim3(256), 0, s, k); break;   \
+        case 4: hipLaunchKernelGGL((embedding_kernel<B, 4>), grid, dim3(256), 0, s, k); break;   \
+        case 8: hipLaunchKernelGGL((embedding_kernel<B, 8>), grid, dim3(256), 0, s, k); break;   \
+        case 16: hipLaunchKernelGGL((embedding_kernel<B, 16>), grid, dim3(256), 0, s, k); break; \
+        case 32: hipLaunchKernelGGL((embedding_kernel<B, 32>), grid, dim3(256), 0, s, k); break; \
+        default: hipLaunchKernelGGL((embedding_kernel<B, 64>), grid, dim3(256), 0, s, k); break; \
+    }
+    switch (bits) {
+        case 2: IOMX_EMBED_I(2); break;
+        case 4: IOMX_EMBED_I(4); break;
+        case 6: IOMX_EMBED_I(6); break;
+        case 8: IOMX_EMBED_I(8); break;
+        case 16: IOMX_EMBED_I(16); break;
+        case 32: IOMX_EMBED_I(32); break;
+        default: IOMX_EMBED_I(64); break;
+    }
+#undef IOMX_EMBED_I
+    record_launch("embedding", grid.x, 256, (uint64_t)k.rows_per_plane * k.planes);
+    IOMX_HIP(hipGetLastError());
+    return IOMX_OK;
+}
+
+// Admission of src/device_ops_neural.cpp:241-362.
+int iomx_launch_rope(int dtype, const iomx_view* x, const iomx_view* out, uint64_t a, double theta,
+                     iomx_stream_t stream) {
+    const uint32_t bits = leaf_bits(dtype);
+    if (!bits) return IOMX_ERR_UNSUPPORTED;
+    IOMX_TRY(check_view(x, bits));
+    IOMX_TRY(check_view(out, bits));
+    if (x->rank < 3 || x->rank != out->rank) return IOMX_ERR_INVALID;
+    if (!same_leading(x, out, x->rank)) return IOMX_ERR_INVALID;
+    const Matrix m = matrix_of(*x);
+    if (m.cols % 2 != 0) return IOMX_ERR_INVALID;
+    uint64_t last;
+    if (add_overflows(a, m.rows - 1, &last)) return IOMX_ERR_OVERFLOW;
+    if (last > (1ull << 24)) return IOMX_ERR_INVALID;   // positions stay exact in binary32
+    if (out->base == x->base) return IOMX_ERR_INVALID;
+    if (!(theta >= 1.0) || theta > 3.4028234663852886e38) return IOMX_ERR_INVALID;
+    if (!is_float_leaf(dtype)) return IOMX_ERR_UNSUPPORTED;
+    if (m.cols > 0xFFFFFFFFull) return IOMX_ERR_OVERFLOW;
+    RopeArgs k = {};
+    const iomx_view* v[2] = {x, out};
+    IOMX_TRY(walk_of<2>(v, x->dims, x->rank - 2, &k.walk));
+    k.x = static_cast<const uint8_t*>(x->base);
+    k.out = static_cast<uint8_t*>(out->base);
+    k.plane_bytes = m.plane_elems * bits / 8;
+    k.rows = (uint32_t)m.rows;
+    k.width = (uint32_t)m.cols;
+    k.half = k.width / 2;
+    k.tile_cols = (uint32_t)m.tile_cols;
+    const bool aligned = k.half % kTile == 0;
+    k.col_tiles = aligned ? k.half / kTile : k.tile_cols;
+    k.div_col_tiles = make_fast_div(k.col_tiles);
+    k.planes = (uint32_t)k.walk.planes;
+    k.a = (uint32_t)a;
+    k.theta = theta;
+    dim3 grid;
+    IOMX_TRY(plane_grid(m.tile_rows, k.col_tiles, k.walk.planes, &k.lanes_per_plane, &grid));
+    grid.y = planes_in_grid(k.lanes_per_plane, k.walk.planes);
+    const hipStream_t s = native(stream);
+    switch (dtype) {
+        case DT_F4_E2M1: launch_rope<DT_F4_E2M1, float>(k, aligned, grid, s); break;
+        case DT_F6_E2M3: launch_rope<DT_F6_E2M3, float>(k, aligned, grid, s); break;
+        case DT_F6_E3M2: launch_rope<DT_F6_E3M2, float>(k, aligned, grid, s); break;
+        case DT_F8_E4M3FN: launch_rope<DT_F8_E4M3FN, float>(k, aligned, grid, s); break;
+        case DT_F8_E5M2: launch_rope<DT_F8_E5M2, float>(k, aligned, grid, s); break;
+        case DT_F16: launch_rope<DT_F16, float>(k, aligned, grid, s); break;
+        case DT_BF16: launch_rope<DT_BF16, float>(k, aligned, grid, s); break;
+        case DT_F32: launch_rope<DT_F32, float>(k, aligned, grid, s); break;
+        default: launch_rope<DT_F64, double>(k, aligned, grid, s); break;
+    }
+    record_launch(aligned ? "rope_pairs" : "rope_general", grid.x, 256,
+                  (uint64_t)k.lanes_per_plane * k.planes);
+    IOMX_HIP(hipGetLastError());
+    return IOMX_OK;
+}
+
+}  // extern "C"

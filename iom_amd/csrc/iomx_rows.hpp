@@ -1,0 +1,324 @@
+// Tile-row helpers shared by the every-leaf kernels: leaf tables, a tile row of
+// sixteen packed elements as an array of 32-bit words, the little-endian bit
+// stream of the host format, and the per-element arithmetic of every leaf.
+#pragma once
+
+#include "iomx_common.hpp"
+
+namespace iomx {
+
+enum {
+    DT_BOOL = 0, DT_I2 = 1, DT_U2 = 2, DT_I4 = 3, DT_U4 = 4, DT_I8 = 5, DT_U8 = 6, DT_I16 = 7,
+    DT_U16 = 8, DT_I32 = 9, DT_U32 = 10, DT_I64 = 11, DT_U64 = 12, DT_F4_E2M1 = 13,
+    DT_F6_E2M3 = 14, DT_F6_E3M2 = 15, DT_F8_E4M3FN = 16, DT_F8_E5M2 = 17, DT_F8_E8M0 = 18,
+    DT_F16 = 19, DT_BF16 = 20, DT_F32 = 21, DT_F64 = 22
+};
+
+constexpr int bits_of(int dt) {
+    switch (dt) {
+        case DT_I2: case DT_U2: return 2;
+        case DT_I4: case DT_U4: case DT_F4_E2M1: return 4;
+        case DT_F6_E2M3: case DT_F6_E3M2: return 6;
+        case DT_BOOL: case DT_I8: case DT_U8: case DT_F8_E4M3FN: case DT_F8_E5M2:
+        case DT_F8_E8M0: return 8;
+        case DT_I16: case DT_U16: case DT_F16: case DT_BF16: return 16;
+        case DT_I32: case DT_U32: case DT_F32: return 32;
+        case DT_I64: case DT_U64: case DT_F64: return 64;
+        default: return 0;
+    }
+}
+
+constexpr bool is_float_leaf(int dt) { return dt >= DT_F4_E2M1 && dt != DT_F8_E8M0; }
+
+struct Fmt {
+    int ebits, fbits, bias;
+    bool finite_only, infs;
+};
+
+constexpr Fmt fmt_of(int dt) {
+    switch (dt) {
+        case DT_F4_E2M1: return {2, 1, 1, true, false};
+        case DT_F6_E2M3: return {2, 3, 1, true, false};
+        case DT_F6_E3M2: return {3, 2, 3, true, false};
+        case DT_F8_E4M3FN: return {4, 3, 7, true, false};
+        case DT_F8_E5M2: return {5, 2, 15, false, true};
+        case DT_F16: return {5, 10, 15, false, true};
+        case DT_BF16: return {8, 7, 127, false, true};
+        case DT_F32: return {8, 23, 127, false, true};
+        default: return {11, 52, 1023, false, true};
+    }
+}
+
+// The top exponent encodes infinity / NaN unless the leaf is finite-only with
+// fewer than four exponent bits.
+constexpr bool top_special(Fmt f) { return !f.finite_only || f.ebits >= 4; }
+
+// The packing helpers and the element arithmetic are plain C++ (usable from host
+// code as well), so they can be exercised without a device.
+#define IOMX_HD __host__ __device__ __forceinline__
+
+// ---------------------------------------------------------------------------
+// Tile rows as word arrays
+// ---------------------------------------------------------------------------
+
+template <int BITS>
+IOMX_HD void load_row(const uint8_t* p, uint32_t (&w)[BITS / 2]) {
+    constexpr int K = BITS / 2;
+    if constexpr (K == 1) {
+        w[0] = *reinterpret_cast<const uint32_t*>(p);
+    } else if constexpr (K == 2) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(p);
+        w[0] = v.x;
+        w[1] = v.y;
+    } else if constexpr (K == 3) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) w[j] = reinterpret_cast<const uint32_t*>(p)[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < K / 4; ++j) {
+            const u32x4 v = reinterpret_cast<const u32x4*>(p)[j];
+            w[4 * j] = v.x;
+            w[4 * j + 1] = v.y;
+            w[4 * j + 2] = v.z;
+            w[4 * j + 3] = v.w;
+        }
+    }
+}
+
+// Element i of a tile row (i is a compile-time constant after unrolling).
+template <int BITS>
+IOMX_HD uint64_t get(const uint32_t (&w)[BITS / 2], int i) {
+    if constexpr (BITS == 64) {
+        return (uint64_t)w[2 * i] | ((uint64_t)w[2 * i + 1] << 32);
+    } else if constexpr (32 % BITS == 0) {
+        constexpr int per = 32 / BITS;
+        const uint32_t v = w[i / per] >> ((i % per) * BITS);
+        return BITS == 32 ? v : (v & ((1u << (BITS & 31)) - 1u));
+    } else {
+        const int bit = i * BITS, j = bit >> 5, sh = bit & 31;
+        uint64_t v = w[j];
+        if (sh + BITS > 32) v |= (uint64_t)w[j + 1] << 32;
+        return (v >> sh) & ((1u << BITS) - 1u);
+    }
+}
+
+// ORs element i into a zero-initialised tile row.
+template <int BITS>
+IOMX_HD void put(uint32_t (&w)[BITS / 2], int i, uint64_t v) {
+    if constexpr (BITS == 64) {
+        w[2 * i] = (uint32_t)v;
+        w[2 * i + 1] = (uint32_t)(v >> 32);
+    } else if constexpr (32 % BITS == 0) {
+        constexpr int per = 32 / BITS;
+        w[i / per] |= (uint32_t)v << ((i % per) * BITS);
+    } else {
+        const int bit = i * BITS, j = bit >> 5, sh = bit & 31;
+        w[j] |= (uint32_t)v << sh;
+        if (sh + BITS > 32) w[j + 1] |= (uint32_t)v >> (32 - sh);
+    }
+}
+
+// Stores the first ncols elements of a tile row and nothing else: whole words
+// where they are covered, a read-modify-write of the one partly covered word.
+template <int BITS>
+IOMX_HD void store_row(uint8_t* p, const uint32_t (&w)[BITS / 2], uint32_t ncols) {
+    constexpr int K = BITS / 2;
+    if (ncols == kTile) {
+        if constexpr (K == 1) {
+            *reinterpret_cast<uint32_t*>(p) = w[0];
+        } else if constexpr (K == 2) {
+            *reinterpret_cast<u32x2*>(p) = u32x2{w[0], w[1]};
+        } else if constexpr (K == 3) {
+#pragma unroll
+            for (int j = 0; j < 3; ++j) reinterpret_cast<uint32_t*>(p)[j] = w[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < K / 4; ++j)
+                reinterpret_cast<u32x4*>(p)[j] = u32x4{w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]};
+        }
+        return;
+    }
+    const uint32_t nbits = ncols * BITS;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+        const uint32_t lo = j * 32u;
+        if (lo >= nbits) break;
+        uint32_t* dst = reinterpret_cast<uint32_t*>(p) + j;
+        if (lo + 32u <= nbits) {
+            *dst = w[j];
+        } else {
+            const uint32_t mask = (1u << (nbits - lo)) - 1u;
+            *dst = (*dst & ~mask) | (w[j] & mask);
+        }
+    }
+}
+
+// BITS bits of a little-endian bit stream held in 32-bit words.
+template <int BITS>
+IOMX_HD uint64_t read_bits(const uint32_t* words, uint64_t bit) {
+    if constexpr (BITS == 64) {
+        return read_bits<32>(words, bit) | (read_bits<32>(words, bit + 32) << 32);
+    } else {
+        const uint64_t j = bit >> 5;
+        const uint32_t sh = (uint32_t)bit & 31u;
+        uint32_t v = words[j] >> sh;
+        if (sh + BITS > 32) v |= words[j + 1] << (32u - sh);
+        return BITS == 32 ? v : (v & ((1u << (BITS & 31)) - 1u));
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Element arithmetic
+// ---------------------------------------------------------------------------
+
+IOMX_HD double as_f64(uint64_t b) { return __builtin_bit_cast(double, b); }
+IOMX_HD uint64_t as_u64(double d) { return __builtin_bit_cast(uint64_t, d); }
+
+constexpr uint64_t kQuietNanF64 = 0x7FF8000000000000ull;
+
+template <int DT>
+IOMX_HD double decode(uint64_t raw64) {
+    if constexpr (DT == DT_F64) {
+        return as_f64(raw64);
+    } else {
+        constexpr Fmt f = fmt_of(DT);
+        constexpr uint32_t emask = (1u << f.ebits) - 1u, fmask = (1u << f.fbits) - 1u;
+        const uint32_t raw = (uint32_t)raw64;
+        const uint32_t frac = raw & fmask, exp = (raw >> f.fbits) & emask;
+        double v;
+        if (top_special(f) && exp == emask) {
+            v = (f.infs && frac == 0) ? __builtin_inf() : __builtin_nan("");
+        } else {
+            const int m = exp ? (int)((1u << f.fbits) + frac) : (int)frac;
+            const int scale = (int)(exp ? exp : 1u) - f.bias - f.fbits;
+            v = ldexp((double)m, scale);
+        }
+        return ((raw >> (f.ebits + f.fbits)) & 1u) ? -v : v;
+    }
+}
+
+// One rounding of a binary64 value (zero, normal, infinite or NaN) onto the leaf.
+template <int DT>
+IOMX_HD uint64_t encode(double r) {
+    if constexpr (DT == DT_F64) {
+        return (r != r) ? kQuietNanF64 : as_u64(r);
+    } else {
+        constexpr Fmt f = fmt_of(DT);
+        constexpr uint32_t emask = (1u << f.ebits) - 1u, fmask = (1u << f.fbits) - 1u;
+        constexpr int shift = f.ebits + f.fbits;
+        constexpr uint32_t finite_emax = top_special(f) ? emask - 1u : emask;
+        constexpr uint32_t over = f.infs ? (emask << f.fbits) : ((finite_emax << f.fbits) | fmask);
+        constexpr uint32_t nan = !top_special(f) ? over
+                : (emask << f.fbits) | (f.finite_only ? fmask : 1u << (f.fbits - 1));
+        const uint64_t b = as_u64(r);
+        const uint32_t sign = (uint32_t)(b >> 63) << shift;
+        const uint64_t mag = b & 0x7FFFFFFFFFFFFFFFull;
+        if (mag > 0x7FF0000000000000ull) return nan;
+        if (mag == 0x7FF0000000000000ull) return sign | over;
+        if (mag == 0) return sign;
+        const int e = (int)(mag >> 52) - 1023;
+        const uint64_t m = (mag & 0xFFFFFFFFFFFFFull) | (1ull << 52);
+        constexpr int emin = 1 - f.bias;
+        const int drop = 52 - f.fbits + (e < emin ? emin - e : 0);
+        uint64_t q = 0, rest = 1, half = 2;  // far below half a unit unless set below
+        if (drop <= 62) {
+            q = m >> drop;
+            rest = m & ((1ull << drop) - 1ull);
+            half = 1ull << (drop - 1);
+        }
+        if (rest > half || (rest == half && (q & 1ull))) ++q;
+        // a normal q carries the implicit bit, which adds one to the exponent field; a
+        // subnormal q that reaches 2^fbits becomes the smallest normal the same way
+        const uint32_t field = e < emin ? (uint32_t)q
+                                        : ((uint32_t)(e + f.bias - 1) << f.fbits) + (uint32_t)q;
+        if ((field >> f.fbits) > finite_emax) return sign | over;
+        return sign | field;
+    }
+}
+
+template <int DT, int OP>
+IOMX_HD uint64_t leaf_binary(uint64_t a, uint64_t b) {
+    constexpr int BITS = bits_of(DT);
+    if constexpr (!is_float_leaf(DT)) {
+        if constexpr (BITS == 64) {
+            return OP == IOMX_OP_ADD ? a + b : (OP == IOMX_OP_MUL ? a * b : a - b);
+        } else {
+            const uint32_t x = (uint32_t)a, y = (uint32_t)b;
+            const uint32_t r = OP == IOMX_OP_ADD ? x + y : (OP == IOMX_OP_MUL ? x * y : x - y);
+            return BITS == 32 ? r : (r & ((1u << (BITS & 31)) - 1u));
+        }
+    } else {
+        // IEEE arithmetic supplies the special cases of the reference rule: opposite
+        // infinities and infinity times zero give NaN, an exact zero sum is +0 unless
+        // both operands are -0, NaN operands give NaN.
+        const double x = decode<DT>(a), y = decode<DT>(b);
+        const double r = OP == IOMX_OP_ADD ? x + y : (OP == IOMX_OP_MUL ? x * y : x - y);
+        return encode<DT>(r);
+    }
+}
+
+// x * sigmoid(x), two-branch form of src/shared/scalar_silu.hpp:69-97; one
+// exponential of a non-positive argument serves both branches.
+IOMX_HD float silu_carrier(float x) {
+    const bool pos = x >= 0.0f;
+    const float e = expf(pos ? -x : x * 0.5f);
+    const float xe = x * e;
+    float num = pos ? x : xe * e;
+    const float den = 1.0f + (pos ? e : e * e);
+    if (!pos && e == 0.0f) num = -0.0f;
+    return num / den;
+}
+IOMX_HD double silu_carrier(double x) {
+    const bool pos = x >= 0.0;
+    const double e = exp(pos ? -x : x * 0.5);
+    const double xe = x * e;
+    double num = pos ? x : xe * e;
+    const double den = 1.0 + (pos ? e : e * e);
+    if (!pos && e == 0.0) num = -0.0;
+    return num / den;
+}
+
+// Carrier: binary32 below F64, binary64 for F64 (src/cpu/queue.cpp:1769-1773).
+template <int DT>
+IOMX_HD uint64_t leaf_silu(uint64_t a) {
+    if constexpr (DT == DT_F64) return encode<DT>(silu_carrier(decode<DT>(a)));
+    else return encode<DT>((double)silu_carrier((float)decode<DT>(a)));
+}
+
+#if defined(__HIPCC__)
+
+struct TileRow {
+    uint32_t row, tc, ncols;
+    bool live;
+};
+
+__device__ __forceinline__ TileRow tile_row_of(uint32_t g, uint32_t rows_per_plane, uint32_t tile_cols,
+                                               FastDiv div, uint32_t rows, uint32_t cols) {
+    TileRow t;
+    const uint32_t r = g & 15u, q = g >> 4;
+    const uint32_t tr = tile_cols > 1 ? fast_div(q, div) : q;
+    t.tc = q - tr * tile_cols;
+    t.row = tr * kTile + r;
+    t.live = g < rows_per_plane && t.row < rows;
+    const uint32_t left = cols - t.tc * kTile;
+    t.ncols = left < kTile ? left : kTile;
+    return t;
+}
+
+#endif  // __HIPCC__
+
+// Grid of the kernels that give one lane to every padded tile row of a plane:
+// x covers one plane, y walks the planes.
+inline int plane_grid(uint64_t tile_rows, uint64_t tile_cols, uint64_t planes, uint32_t* rows_per_plane,
+                      dim3* grid) {
+    uint64_t per;
+    if (mul_overflows(tile_rows, tile_cols, &per) || mul_overflows(per, kTile, &per))
+        return IOMX_ERR_OVERFLOW;
+    if (per > 0xFFFFFF00ull || tile_cols > 0x0FFFFFFFull || planes > 0xFFFFFFFFull)
+        return IOMX_ERR_OVERFLOW;
+    *rows_per_plane = (uint32_t)per;
+    *grid = dim3((uint32_t)((per + 255) / 256), (uint32_t)(planes < 65535 ? planes : 65535));
+    return IOMX_OK;
+}
+
+}  // namespace iomx

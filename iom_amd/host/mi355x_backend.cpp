@@ -37,6 +37,7 @@
 #include <stdexcept>
 #include <string>
 #include <thread>
+#include <type_traits>
 #include <vector>
 
 #include "iom/alloc.hpp"
@@ -347,6 +348,12 @@ public:
                 events_.push_back(event);
                 free_events_.push_back(event);
             }
+            // one page-locked status word per completion event (the embedding lookup
+            // reports an invalid id through it,
+            // docs/BACKEND_CONTRACT/embedding-lookup.md:178-203)
+            void* cells = nullptr;
+            check(iomx_host_alloc(&cells, capacity * sizeof(std::uint32_t)), "status cells");
+            status_cells_ = static_cast<std::uint32_t*>(cells);
             check(iomx_stream_create(&stream_), "queue stream");
             completer_ = std::thread([this] { run_completer(); });
         } catch (...) {
@@ -377,11 +384,17 @@ public:
 private:
     using Finish = std::function<void(bool failed)>;
 
+    // After native completion: turns a data error the kernel reported into the
+    // operation's retained failure (null = none).
+    using Verify = std::function<std::exception_ptr(const std::uint32_t& status)>;
+
     struct InFlight {
         std::uint64_t sequence = 0;
         iomx_event_t event = nullptr;
+        std::uint32_t* status = nullptr;
         std::exception_ptr failure;
         Finish finish;
+        Verify verify;
     };
 
     static detail::FenceResult fence_pending(const detail::Fence&) noexcept {
@@ -399,13 +412,21 @@ private:
         free_events_.clear();
         if (stream_ != nullptr) (void)iomx_stream_destroy(stream_);
         stream_ = nullptr;
+        if (status_cells_ != nullptr) (void)iomx_host_free(status_cells_);
+        status_cells_ = nullptr;
+    }
+
+    [[nodiscard]] std::uint32_t* status_cell(iomx_event_t event) noexcept {
+        for (std::size_t i = 0; i < events_.size(); ++i)
+            if (events_[i] == event) return status_cells_ + i;
+        return nullptr;
     }
 
     // Runs inside the common admission dispatch: launch on the queue stream,
     // record the completion event, hand the rest to the completion thread.
     // Throws only before anything was launched.
     template <typename Launch>
-    void start(std::uint64_t sequence, Launch&& launch, Finish finish) {
+    void start(std::uint64_t sequence, Launch&& launch, Finish finish, Verify verify = {}) {
         iomx_event_t event = nullptr;
         {
             std::lock_guard<std::mutex> lock(mutex_);
@@ -418,8 +439,15 @@ private:
         item.sequence = sequence;
         item.event = event;
         item.finish = std::move(finish);
+        item.verify = std::move(verify);
+        item.status = status_cell(event);
         int status = iomx_set_device(device_.ordinal());
-        if (status == IOMX_OK) status = launch(stream_);
+        if (status == IOMX_OK) {
+            if constexpr (std::is_invocable_v<Launch&, iomx_stream_t, std::uint32_t*>)
+                status = launch(stream_, item.status);
+            else
+                status = launch(stream_);
+        }
         if (status == IOMX_OK) status = iomx_event_record(event, stream_);
         if (status != IOMX_OK) {
             try { throw_status(status, "MI355X kernel submission"); }
@@ -448,6 +476,9 @@ private:
                 if (status != IOMX_OK) {
                     try { throw_status(status, "MI355X kernel completion"); }
                     catch (...) { item.failure = std::current_exception(); }
+                } else if (item.verify) {
+                    // a native failure takes precedence over the status word
+                    item.failure = item.verify(*item.status);
                 }
             } else {
                 // the stream may still hold earlier work: keep completion in order
@@ -582,6 +613,146 @@ private:
                 });
     }
 
+    // ---- cache append / embedding / rope ----------------------------------------
+
+    template <typename Snapshot>
+    [[nodiscard]] static iomx_view snapshot_view(const Snapshot& s) {
+        return make_view(s.native_handle, s.shape_dimensions(), s.plane_offset,
+                         s.leading_plane_strides());
+    }
+
+    [[nodiscard]] WorkspaceRequirements cache_append_workspace_requirements(
+            const CacheAppendRequest&) override {
+        return {0, 1};
+    }
+
+    oid cache_append_impl(const CacheAppendRequest& request) override {
+        const int code = transfer_code(request.source.data_type);
+        if (code < 0) throw detail::UnsupportedOperation();
+        std::lock_guard<std::mutex> order(submission_mutex_);
+        return submit_cache_append(
+                request, device_.registry_state(), registry_queue_id_, pending_fence(),
+                [this, code](std::uint64_t sequence, const CacheAppendRequest& captured,
+                             detail::BinaryEntryRegistration entries) {
+                    auto& state = device_.registry_state();
+                    const detail::WorkspaceLease lease = captured.workspace_lease;
+                    try {
+                        start(sequence,
+                              [&captured, code](iomx_stream_t stream) {
+                                  const iomx_view source = snapshot_view(captured.source);
+                                  const iomx_view destination = snapshot_view(captured.destination);
+                                  return iomx_launch_cache_append(code, &source, &destination,
+                                                                  captured.a, stream);
+                              },
+                              [&state, entries, lease](bool failed) {
+                                  (void)detail::release_or_invalidate_binary_entries(
+                                          state.registry, entries, failed, true);
+                                  detail::complete_workspace_lease(state, lease, true);
+                              });
+                    } catch (...) {
+                        state.registry.remove_entries(std::span<const detail::EntryId>(
+                                entries.entries.data(), entries.count));
+                        detail::complete_workspace_lease(state, lease, true);
+                        throw;
+                    }
+                });
+    }
+
+    [[nodiscard]] WorkspaceRequirements rope_workspace_requirements(const RopeRequest& request) override {
+        if (float_code(request.x.data_type) < 0) throw detail::UnsupportedOperation();
+        return {0, 1};
+    }
+
+    oid rope_impl(const RopeRequest& request) override {
+        const int code = float_code(request.x.data_type);
+        if (code < 0) throw detail::UnsupportedOperation();
+        std::lock_guard<std::mutex> order(submission_mutex_);
+        return submit_rope(
+                request, device_.registry_state(), registry_queue_id_, pending_fence(),
+                [this, code](std::uint64_t sequence, const RopeRequest& captured,
+                             detail::BinaryEntryRegistration entries) {
+                    auto& registry = device_.registry_state().registry;
+                    try {
+                        start(sequence,
+                              [&captured, code](iomx_stream_t stream) {
+                                  const iomx_view x = snapshot_view(captured.x);
+                                  const iomx_view out = snapshot_view(captured.out);
+                                  return iomx_launch_rope(code, &x, &out, captured.a, captured.theta,
+                                                          stream);
+                              },
+                              [&registry, entries](bool failed) {
+                                  (void)detail::release_or_invalidate_binary_entries(
+                                          registry, entries, failed, true);
+                              });
+                    } catch (...) {
+                        registry.remove_entries(std::span<const detail::EntryId>(
+                                entries.entries.data(), entries.count));
+                        throw;
+                    }
+                });
+    }
+
+    // 32 bytes of caller-owned control scratch, 32-byte aligned: the first word is the
+    // bounds status (docs/BACKEND_CONTRACT/embedding-lookup.md:178-201).
+    [[nodiscard]] WorkspaceRequirements embedding_workspace_requirements_impl(
+            const TensorView& table, const TensorView& indices, const TensorView&) override {
+        if (transfer_code(table.spec().data_type) < 0) throw detail::UnsupportedOperation();
+        const int index = static_cast<int>(indices.spec().data_type);
+        if (index < static_cast<int>(DataType::I2) || index > static_cast<int>(DataType::U64))
+            throw detail::UnsupportedOperation();
+        return {32, 32};
+    }
+
+    oid embedding_impl(const EmbeddingRequest& request) override {
+        const int code = transfer_code(request.table.spec.data_type);
+        const int index_code = static_cast<int>(request.indices.spec.data_type);
+        if (code < 0) throw detail::UnsupportedOperation();
+        std::lock_guard<std::mutex> order(submission_mutex_);
+        return submit_embedding(
+                request, device_.registry_state(), registry_queue_id_, pending_fence(),
+                [this, code, index_code](std::uint64_t sequence, const EmbeddingRequest& captured,
+                                         detail::BinaryEntryRegistration entries) {
+                    auto& state = device_.registry_state();
+                    const detail::WorkspaceLease lease = captured.workspace_lease;
+                    try {
+                        auto* control = static_cast<std::uint32_t*>(
+                                detail::WorkspaceValidation::address(captured.workspace));
+                        start(sequence,
+                              [&captured, code, index_code, control](iomx_stream_t stream,
+                                                                    std::uint32_t* cell) {
+                                  const auto view_of = [](const CopyViewSnapshot& s) {
+                                      return make_view(s.native_handle, s.spec.shape.dimensions(),
+                                                       s.plane_offset, s.plane_strides);
+                                  };
+                                  const iomx_view table = view_of(captured.table);
+                                  const iomx_view indices = view_of(captured.indices);
+                                  const iomx_view out = view_of(captured.out);
+                                  // status reset, gather, then exactly four bytes back to the host
+                                  int status = iomx_launch_embedding(code, index_code, &table, &indices,
+                                                                     &out, control, stream);
+                                  if (status == IOMX_OK)
+                                      status = iomx_memcpy_d2h_async(cell, control, sizeof(*cell), stream);
+                                  return status;
+                              },
+                              [&state, entries, lease](bool failed) {
+                                  (void)detail::release_or_invalidate_binary_entries(
+                                          state.registry, entries, failed, true);
+                                  detail::complete_workspace_lease(state, lease, true);
+                              },
+                              [](const std::uint32_t& status) -> std::exception_ptr {
+                                  if (status == 0) return nullptr;
+                                  return std::make_exception_ptr(std::invalid_argument(
+                                          "MI355X embedding index is negative or out of range"));
+                              });
+                    } catch (...) {
+                        state.registry.remove_entries(std::span<const detail::EntryId>(
+                                entries.entries.data(), entries.count));
+                        detail::complete_workspace_lease(state, lease, true);
+                        throw;
+                    }
+                });
+    }
+
     [[nodiscard]] WorkspaceRequirements silu_workspace_requirements_impl(
             const SiLURequest& request) override {
         if (float_code(request.x.data_type) < 0) throw detail::UnsupportedOperation();
@@ -625,6 +796,7 @@ private:
     std::mutex submission_mutex_;
     iomx_stream_t stream_ = nullptr;
     std::vector<iomx_event_t> events_;
+    std::uint32_t* status_cells_ = nullptr;
     std::mutex mutex_;
     std::condition_variable cv_;
     std::vector<iomx_event_t> free_events_;

@@ -57,6 +57,7 @@ SYMBOLS = [
     "iomx_memcpy_d2d_async", "iomx_stream_create", "iomx_stream_destroy",
     "iomx_stream_synchronize", "iomx_event_create", "iomx_event_destroy", "iomx_event_record",
     "iomx_event_synchronize", "iomx_event_query", "iomx_event_elapsed_ms",
+    "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
     "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul",
     "iomx_launch_copy", "iomx_launch_scatter", "iomx_launch_gather", "iomx_launch_softmax",
     "iomx_last_launch", "iomx_selftest_bf16_convert",
@@ -144,6 +145,9 @@ def lib() -> C.CDLL:
         l.iomx_launch_silu.argtypes = [C.c_int, VP, VP, P]
         l.iomx_launch_silu_mul.argtypes = [C.c_int, VP, VP, VP, P]
         l.iomx_launch_copy.argtypes = [C.c_int, VP, VP, P]
+        l.iomx_launch_cache_append.argtypes = [C.c_int, VP, VP, C.c_uint64, P]
+        l.iomx_launch_embedding.argtypes = [C.c_int, C.c_int, VP, VP, VP, P, P]
+        l.iomx_launch_rope.argtypes = [C.c_int, VP, VP, C.c_uint64, C.c_double, P]
         l.iomx_launch_scatter.argtypes = [C.c_int, VP, P, P]
         l.iomx_launch_gather.argtypes = [C.c_int, VP, P, P]
         l.iomx_launch_softmax.argtypes = [C.POINTER(SoftmaxDesc), P]
@@ -420,6 +424,25 @@ def silu_mul(gate: DeviceView, up: DeviceView, y: DeviceView, stream=None) -> in
 def copy(src: DeviceView, dst: DeviceView, stream=None) -> int:
     a, o = src.cview(), dst.cview()
     return lib().iomx_launch_copy(dst.dtype, C.byref(a), C.byref(o), _h(stream))
+
+
+def cache_append(src: DeviceView, dst: DeviceView, a: int, stream: Optional[Stream] = None) -> int:
+    s_, d = src.cview(), dst.cview()
+    return lib().iomx_launch_cache_append(dst.dtype, C.byref(s_), C.byref(d), C.c_uint64(a), _h(stream))
+
+
+def embedding(table: DeviceView, indices: DeviceView, out: DeviceView, status: "Buffer",
+              stream: Optional[Stream] = None) -> int:
+    """`status` is a device buffer of at least 4 bytes; read word 0 after completion."""
+    t, i_, o = table.cview(), indices.cview(), out.cview()
+    return lib().iomx_launch_embedding(out.dtype, indices.dtype, C.byref(t), C.byref(i_), C.byref(o),
+                                       status.ptr, _h(stream))
+
+
+def rope(x: DeviceView, out: DeviceView, a: int, theta: float, stream: Optional[Stream] = None) -> int:
+    s_, o = x.cview(), out.cview()
+    return lib().iomx_launch_rope(out.dtype, C.byref(s_), C.byref(o), C.c_uint64(a), C.c_double(theta),
+                                  _h(stream))
 
 
 def dense_layout(heads: int, rows: int, cols: int) -> StageLayout:
