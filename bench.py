@@ -237,6 +237,64 @@ def wl_silu_mul(timer, steps, warmup, dims):
     return out
 
 
+def wl_layer_ops(timer, steps, warmup):
+    """The data-movement operations either side of the measured path, at TinyLlama-like
+    shapes: RoPE on [64,32,512,64], embedding of [64,1,512] ids from a [32000,2048] table,
+    and a 512-row cache append into [64,4,2048,64]."""
+    out = []
+    B, H, S, D = 64, 32, 512, 64
+    rot = 2
+    xs = [(device_tensor(BF16, (B, H, S, D), "normal", 71 + i), device_tensor(BF16, (B, H, S, D)))
+          for i in range(rot)]
+    n = B * H * S * D
+
+    def rope(i):
+        x, o = xs[i % rot]
+        check(iomx.rope(x.view(), o.view(), 0, 10000.0, timer.stream), "rope")
+
+    wall, ev = timer.run(rope, steps, warmup)
+    out.append(report("rope_bf16_[64,32,512,64]", 4 * n, n, wall, ev, iomx.last_launch().kernel.decode()))
+    for x, o in xs:
+        x.free()
+        o.free()
+
+    V, F = 32000, 2048
+    table = device_tensor(BF16, (V, F), "normal", 81)
+    ids = (datagen.pattern_bits(32, B * S, 82) % V).astype(np.uint32).reshape(B, 1, S)
+    idt = iomx.DeviceTensor(iomx.DT_I32, (B, 1, S))
+    idt.view().from_host(ids)
+    outs = [device_tensor(BF16, (B, S, F)) for _ in range(rot)]
+    status = iomx.Buffer(32)
+
+    def embed(i):
+        check(iomx.embedding(table.view(), idt.view(), outs[i % rot].view(), status, timer.stream), "embedding")
+
+    wall, ev = timer.run(embed, steps, warmup)
+    ne = B * S * F
+    out.append(report("embedding_bf16_[64,512]x[32000,2048]", 4 * ne + 4 * B * S, ne, wall, ev,
+                      iomx.last_launch().kernel.decode()))
+    assert int(status.download(np.uint32)[0]) == 0
+    for t in [table, idt] + outs:
+        t.free()
+    status.free()
+
+    KH, C = 4, 2048
+    src = device_tensor(BF16, (B, KH, S, D), "normal", 91)
+    caches = [device_tensor(BF16, (B, KH, C, D)) for _ in range(rot)]
+
+    def append(i):
+        check(iomx.cache_append(src.view(), caches[i % rot].view(), 1024, timer.stream), "cache_append")
+
+    wall, ev = timer.run(append, steps, warmup)
+    na = B * KH * S * D
+    out.append(report("cache_append_bf16_[64,4,512,64]->[64,4,2048,64]@1024", 4 * na, na, wall, ev,
+                      iomx.last_launch().kernel.decode()))
+    src.free()
+    for c in caches:
+        c.free()
+    return out
+
+
 def wl_softmax(timer, steps, warmup, planes, heads, rows, cols, causal_position):
     """F32 scores [planes,heads,rows,cols] with the strict upper triangle = -inf as data.
     causal_position=False: a = cols-1, every token is positionally visible (the mask
@@ -410,6 +468,7 @@ def main():
         "softmax": lambda: wl_softmax(timer, max(K // 20, 3), 2, 32, 32, 2048, 2048, False),
         "softmax_causal": lambda: wl_softmax(timer, max(K // 20, 3), 2, 32, 32, 2048, 2048, True),
         "chain": lambda: wl_chain(timer, max(K // 10, 5), max(W // 10, 2)),
+        "layer_ops": lambda: wl_layer_ops(timer, max(K // 4, 5), max(W // 4, 2)),
     }
 
     if args.only:
@@ -424,7 +483,7 @@ def main():
     if not args.no_detail:
         for key in ("bcast_mul_bf16", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "copy_bf16", "add_f32",
                     "add_i32", "rmsnorm_bf16", "rmsnorm_f32", "silu_mul", "softmax", "softmax_causal",
-                    "chain"):
+                    "chain", "layer_ops"):
             r = table[key]()
             detail.extend(r if isinstance(r, list) else [r])
     cpu = None if args.no_cpu else cpu_baseline()
