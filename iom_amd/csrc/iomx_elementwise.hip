@@ -169,14 +169,18 @@ struct FlatArgs {
     // one or two leading axes, as byte steps per coordinate (0 = broadcast)
     uint32_t n0, n1;
     uint64_t step0[3], step1[3];
+    FastDiv div_segments;
 };
 
 // FLAT    one dense range.
 // BANDS   one dense range cut into tile-row bands (row-vector operand).
 // AXIS1   one strided leading axis on blockIdx.z, segments on blockIdx.y.
 // AXIS2   two strided leading axes on blockIdx.z / blockIdx.y, one segment.
+// AXIS2B  two strided leading axes with bands: axis 0 on blockIdx.z, (axis 1, band) on
+//         blockIdx.y, split by one scalar multiply-shift division.
 // PLANES  anything else: the generic plane walk.
-enum { SHAPE_FLAT = 0, SHAPE_BANDS = 1, SHAPE_AXIS1 = 2, SHAPE_AXIS2 = 3, SHAPE_PLANES = 4 };
+enum { SHAPE_FLAT = 0, SHAPE_BANDS = 1, SHAPE_AXIS1 = 2, SHAPE_AXIS2 = 3, SHAPE_PLANES = 4,
+       SHAPE_AXIS2B = 5 };
 
 template <int DT, int OP, int LM, int RM>
 __device__ __forceinline__ void stream_chunk(const uint8_t* lbase, const uint8_t* rbase,
@@ -219,6 +223,17 @@ __global__ __launch_bounds__(kPlanesBlock) void elementwise_stream_kernel(const 
                 stream_chunk<DT, OP, LM, RM>(a.src[0] + z * a.step0[0], a.src[1] + z * a.step0[1],
                                              a.out + z * a.step0[2],
                                              ((uint64_t)y * a.seg_chunks + cb) * 16, voff);
+    } else if constexpr (SHAPE == SHAPE_AXIS2B) {
+        const uint64_t voff = rowvec_offset<DT>(cb);
+        for (uint32_t z = blockIdx.z; z < a.n0; z += gridDim.z)
+            for (uint32_t y = blockIdx.y; y < a.n1 * a.segments; y += gridDim.y) {
+                const uint32_t j = fast_div(y, a.div_segments);  // segments >= 2 here
+                const uint32_t seg = y - j * a.segments;
+                stream_chunk<DT, OP, LM, RM>(a.src[0] + z * a.step0[0] + j * a.step1[0],
+                                             a.src[1] + z * a.step0[1] + j * a.step1[1],
+                                             a.out + z * a.step0[2] + j * a.step1[2],
+                                             ((uint64_t)seg * a.seg_chunks + cb) * 16, voff);
+            }
     } else {
         for (uint32_t z = blockIdx.z; z < a.n0; z += gridDim.z)
             for (uint32_t y = blockIdx.y; y < a.n1; y += gridDim.y)
@@ -375,8 +390,8 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
                    pa.planes < 65535u ? pa.planes : 65535u);
         if (pa.planes == 1 && pa.walk.nlead == 0) {
             shape = pa.segments == 1 ? SHAPE_FLAT : SHAPE_BANDS;
-        } else if (pa.walk.nlead == 1 || (pa.walk.nlead == 2 && pa.segments == 1)) {
-            shape = pa.walk.nlead == 1 ? SHAPE_AXIS1 : SHAPE_AXIS2;
+        } else if (pa.walk.nlead == 1 || pa.walk.nlead == 2) {
+            shape = pa.walk.nlead == 1 ? SHAPE_AXIS1 : (pa.segments == 1 ? SHAPE_AXIS2 : SHAPE_AXIS2B);
             fa.n0 = pa.walk.dims[0];
             fa.n1 = pa.walk.nlead == 2 ? pa.walk.dims[1] : 1;
             fa.src[0] += pa.walk.offset[0] * pa.plane_bytes[0];
@@ -388,6 +403,13 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
             }
             if (shape == SHAPE_AXIS2) grid3 = dim3((uint32_t)gx, fa.n1 < 65535u ? fa.n1 : 65535u,
                                                    fa.n0 < 65535u ? fa.n0 : 65535u);
+            else if (shape == SHAPE_AXIS2B) {
+                const uint64_t ys = (uint64_t)fa.n1 * pa.segments;
+                fa.div_segments = make_fast_div(pa.segments);
+                grid3 = dim3((uint32_t)gx, (uint32_t)(ys < 65535u ? ys : 65535u),
+                             fa.n0 < 65535u ? fa.n0 : 65535u);
+                if (ys > 0xFFFFFFFFull) shape = SHAPE_PLANES;
+            }
             else grid3.z = fa.n0 < 65535u ? fa.n0 : 65535u;
         }
 #define IOMX_STREAM(LMV, RMV, SH)                                                               \
@@ -399,6 +421,7 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
         else if (shape == SHAPE_BANDS) IOMX_STREAM(LMV, RMV, SHAPE_BANDS);                      \
         else if (shape == SHAPE_AXIS1) IOMX_STREAM(LMV, RMV, SHAPE_AXIS1);                      \
         else if (shape == SHAPE_AXIS2) IOMX_STREAM(LMV, RMV, SHAPE_AXIS2);                      \
+        else if (shape == SHAPE_AXIS2B) IOMX_STREAM(LMV, RMV, SHAPE_AXIS2B);                    \
         else                                                                                    \
             hipLaunchKernelGGL((elementwise_planes_kernel<DT, OP, LMV, RMV>), grid3,            \
                                dim3(kPlanesBlock), 0, s, pa);                                   \
