@@ -295,6 +295,38 @@ def wl_layer_ops(timer, steps, warmup):
     return out
 
 
+def wl_other_leaves(timer, steps, warmup):
+    """The tile-row kernels that serve every leaf outside I32/U32/F32/BF16, on the headline
+    shape: correctness-first paths, measured so that their cost is known."""
+    out = []
+    dims, F = (64, 512, 2048), 2048
+    n = int(np.prod(dims))
+    for name, dtype in (("f16", iomx.DT_F16), ("u8", iomx.DT_U8), ("f8_e4m3fn", iomx.DT_F8_E4M3FN),
+                        ("u4", iomx.DT_U4), ("f64", iomx.DT_F64)):
+        bits = iomx.LEAF_BITS[dtype]
+        def owner(d, salt):
+            t = iomx.DeviceTensor(dtype, d, fill=None)
+            raw = datagen.pattern_bits(32, t.nbytes // 4, salt)
+            if dtype == iomx.DT_F64:     # moderate exponents
+                raw = raw.copy()
+                raw[1::2] = (raw[1::2] & 0x800FFFFF) | 0x3FE00000
+            elif dtype == iomx.DT_F16:
+                raw = (raw & 0xBBFFBBFF)
+            t.upload_raw(raw)
+            return t
+        lhs, rhs, o = owner(dims, 1), owner((1, F), 2), iomx.DeviceTensor(dtype, dims, fill=None)
+
+        def launch(i):
+            check(iomx.binary(ADD, lhs.view(), rhs.view(), o.view(), timer.stream), name)
+
+        wall, ev = timer.run(launch, steps, warmup)
+        out.append(report("bcast_add_%s_[64,512,2048]+[1,2048]" % name, (2 * n + F) * bits // 8, n, wall, ev,
+                          iomx.last_launch().kernel.decode()))
+        for t in (lhs, rhs, o):
+            t.free()
+    return out
+
+
 def wl_softmax(timer, steps, warmup, planes, heads, rows, cols, causal_position):
     """F32 scores [planes,heads,rows,cols] with the strict upper triangle = -inf as data.
     causal_position=False: a = cols-1, every token is positionally visible (the mask
@@ -469,6 +501,7 @@ def main():
         "softmax_causal": lambda: wl_softmax(timer, max(K // 20, 3), 2, 32, 32, 2048, 2048, True),
         "chain": lambda: wl_chain(timer, max(K // 10, 5), max(W // 10, 2)),
         "layer_ops": lambda: wl_layer_ops(timer, max(K // 4, 5), max(W // 4, 2)),
+        "other_leaves": lambda: wl_other_leaves(timer, max(K // 10, 5), max(W // 10, 2)),
     }
 
     if args.only:
