@@ -176,6 +176,89 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_band_kernel(const RmsArgs a) 
     }
 }
 
+// Wide rows: the band is cut into S parts of 16/S rows each, one workgroup per
+// part, so that a workgroup still holds only K chunks per lane (two workgroups
+// stay resident per compute unit) however large F is.  Inside a tile the rows
+// of one part are one contiguous run of kChunksPerTile/S chunks; a lane's chunk
+// index within its part maps to (tile, chunk in the run), and the lanes of a
+// wave that share a row differ in the position inside the row piece (low bits)
+// and in the tile (bits above the run).
+template <int DT, int K, int S>
+__global__ __launch_bounds__(1024) void rmsnorm_split_kernel(const RmsArgs a) {
+    using L = RLeaf<DT>;
+    constexpr int THREADS = 1024;
+    constexpr int kWaves = THREADS / 64;
+    constexpr uint32_t SUB = L::kChunksPerTile / S;   // chunks of one part in one tile
+    constexpr uint32_t RP = kTile / S;                // rows of one part
+    static_assert(SUB >= L::kChunksPerRow, "a part holds whole row pieces");
+    __shared__ __attribute__((aligned(16))) float partial[RP][kWaves];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t band = blockIdx.x / S, part = blockIdx.x % S;
+    const uint32_t w = tid % SUB;
+    const uint32_t row = w / L::kChunksPerRow;        // within the part
+    uint32_t p = 0, tr = band;
+    if (a.walk.nlead != 0) {
+        p = band / a.tile_rows;
+        tr = band - p * a.tile_rows;
+    }
+    uint64_t plane[2];
+    walk_planes(a.walk, p, plane);
+    const uint8_t* xb = a.x + plane[0] * a.plane_bytes + (uint64_t)tr * a.band_bytes;
+    uint8_t* ob = a.out + plane[1] * a.plane_bytes + (uint64_t)tr * a.band_bytes;
+    const uint32_t part_chunks = a.band_chunks / S;
+    uint32_t chunk[K];
+    u32x4 cur[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t c = tid + k * THREADS;
+        chunk[k] = (c / SUB) * L::kChunksPerTile + part * SUB + w;
+        cur[k] = u32x4{0, 0, 0, 0};
+        if (c < part_chunks)
+            cur[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xb + (uint64_t)chunk[k] * 16));
+    }
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        float f[L::kPerChunk];
+        unpack<DT>(cur[k], f);
+#pragma unroll
+        for (uint32_t e = 0; e < L::kPerChunk; ++e) acc = __builtin_fmaf(f[e], f[e], acc);
+    }
+    // lanes of the wave that hold the same row: every lane bit that is not a row bit
+    uint32_t shared_bits = 0;
+#pragma unroll
+    for (uint32_t bit = 1; bit < 64; bit <<= 1) {
+        if (bit < L::kChunksPerRow || bit >= SUB) {
+            acc += __shfl_xor(acc, (int)bit);
+            shared_bits |= bit;
+        }
+    }
+    if ((tid & shared_bits) == 0) partial[row][tid / 64] = acc;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < kWaves; ++wv) total = total + partial[row][wv];
+    const float inverse = inverse_rms(total, a.feats, a.eps);
+    if (tr * kTile + part * RP + row >= a.rows) return;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        if (tid + k * THREADS < part_chunks) {
+            const uint32_t c = chunk[k];
+            const uint32_t soff = ((c / L::kChunksPerTile) * L::kChunksPerTile
+                                   + (c % L::kChunksPerRow)) * 16;
+            float f[L::kPerChunk], sc[L::kPerChunk];
+            unpack<DT>(cur[k], f);
+            unpack<DT>(*reinterpret_cast<const u32x4*>(a.scale + soff), sc);
+#pragma unroll
+            for (uint32_t e = 0; e < L::kPerChunk; ++e) {
+                const float normalized = f[e] * inverse;
+                f[e] = normalized * sc[e];
+            }
+            __builtin_nontemporal_store(pack<DT>(f), reinterpret_cast<u32x4*>(ob + (uint64_t)c * 16));
+        }
+    }
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void rmsnorm_generic_kernel(const RmsArgs a) {
     using L = RLeaf<DT>;
@@ -252,10 +335,32 @@ void launch_band(const RmsArgs& a, hipStream_t s) {
     record_launch("rmsnorm_band", a.total_bands, THREADS, a.total_bands);
 }
 
+template <int DT, int K, int S>
+void launch_split(const RmsArgs& a, hipStream_t s) {
+    hipLaunchKernelGGL((rmsnorm_split_kernel<DT, K, S>), dim3(a.total_bands * S), dim3(1024), 0, s, a);
+    record_launch("rmsnorm_split", a.total_bands * S, 1024, (uint64_t)a.total_bands * S);
+}
+
+// Chunks one 1024-lane workgroup can hold in registers without spilling: K = 8 per
+// lane for BF16 (whose unpacked chunk is eight floats), 16 for F32.  Measured on
+// MI355X with rows of 4096..16384 features: the fewest, largest parts win (runs of
+// 256 bytes or more per tile), and sixteen parts (32-byte runs) lose even to the
+// two-pass kernel, so the split stops at eight.
+template <int DT>
+constexpr uint32_t kResidentChunks = (DT == IOMX_DT_BF16 ? 8u : 16u) * 1024u;
+
 template <int DT>
 int launch(const RmsArgs& a, bool band_ok, hipStream_t s) {
     const uint32_t n = a.band_chunks;
-    if (!band_ok || n > 16384 || a.total_bands > 0x7FFFFFFFu) {
+    constexpr int KS = DT == IOMX_DT_BF16 ? 8 : 16;
+    if (band_ok && n > kResidentChunks<DT> && n <= 8 * kResidentChunks<DT>
+        && (uint64_t)a.total_bands * 8 <= 0x7FFFFFFFull) {
+        if (n <= 2 * kResidentChunks<DT>) launch_split<DT, KS, 2>(a, s);
+        else if (n <= 4 * kResidentChunks<DT>) launch_split<DT, KS, 4>(a, s);
+        else launch_split<DT, KS, 8>(a, s);
+        return IOMX_OK;
+    }
+    if (!band_ok || n > kResidentChunks<DT> || a.total_bands > 0x7FFFFFFFu) {
         const uint32_t cap = 1u << 20;
         const uint32_t grid = a.total_bands < cap ? a.total_bands : cap;
         hipLaunchKernelGGL((rmsnorm_generic_kernel<DT>), dim3(grid), dim3(256), 0, s, a);
@@ -267,7 +372,7 @@ int launch(const RmsArgs& a, bool band_ok, hipStream_t s) {
     else if (n <= 2048) launch_band<DT, 2, 1024>(a, s);
     else if (n <= 4096) launch_band<DT, 4, 1024>(a, s);
     else if (n <= 8192) launch_band<DT, 8, 1024>(a, s);
-    else launch_band<DT, 16, 1024>(a, s);
+    else launch_band<DT, 16, 1024>(a, s);  // F32 only: BF16 bands this wide are split above
     return IOMX_OK;
 }
 
