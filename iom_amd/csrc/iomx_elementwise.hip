@@ -260,6 +260,68 @@ __global__ __launch_bounds__(kPlanesBlock) void elementwise_planes_kernel(const 
     }
 }
 
+// Tile padding (rows or columns that are not multiples of 16): the padded planes
+// are still whole contiguous bands, so the lanes keep the streaming kernel's chunk
+// mapping; a lane drops out where its chunk lies in the padding (columns: once per
+// launch; rows: in the last band of a plane) and stores element by element where a
+// chunk straddles the last logical column.  Padding is neither loaded nor stored.
+struct PaddedArgs {
+    BinaryArgs b;             // seg_chunks = chunks of one band, segments = bands walked per plane
+    uint32_t rows, cols;
+    uint32_t tile_rows;       // bands of one plane
+    FastDiv div_tile_rows;
+    uint32_t folded;          // segments run over several planes: band = segment mod tile_rows
+};
+
+template <int DT, int OP, int LM, int RM>
+__global__ __launch_bounds__(kPlanesBlock) void elementwise_padded_kernel(const PaddedArgs a) {
+    using L = Leaf<DT>;
+    constexpr int kInputs = Arity<OP>::kInputs;
+    const uint64_t cb = (uint64_t)blockIdx.x * kPlanesBlock + threadIdx.x;
+    if (cb >= a.b.seg_chunks) return;
+    const uint32_t in_tile = (uint32_t)cb & (L::kChunksPerTile - 1);
+    const uint32_t row = in_tile / L::kChunksPerRow;
+    const uint32_t col0 = (uint32_t)(cb / L::kChunksPerTile) * kTile + (in_tile & (L::kChunksPerRow - 1)) * L::kPerChunk;
+    if (col0 >= a.cols) return;
+    const uint32_t left = a.cols - col0;
+    const uint32_t valid = left < L::kPerChunk ? left : L::kPerChunk;
+    const uint64_t voff = rowvec_offset<DT>(cb);
+    for (uint32_t z = blockIdx.z; z < a.b.planes; z += gridDim.z) {
+        uint64_t plane[3];
+        walk_planes(a.b.walk, z, plane);
+        const uint8_t* lbase = a.b.src[0] + plane[0] * a.b.plane_bytes[0];
+        const uint8_t* rbase = a.b.src[1] + plane[1] * a.b.plane_bytes[1];
+        uint8_t* obase = a.b.out + plane[2] * a.b.plane_bytes[2];
+        for (uint32_t y = blockIdx.y; y < a.b.segments; y += gridDim.y) {
+            uint32_t tr = y;
+            if (a.folded && a.tile_rows > 1) tr = y - fast_div(y, a.div_tile_rows) * a.tile_rows;
+            else if (a.folded) tr = 0;
+            if (tr * kTile + row >= a.rows) continue;
+            const uint64_t off = ((uint64_t)y * a.b.seg_chunks + cb) * 16;
+            u32x4 va, vb = u32x4{0, 0, 0, 0};
+            if constexpr (LM == MODE_ROWVEC) va = *reinterpret_cast<const u32x4*>(lbase + voff);
+            else va = load_stream(lbase + off);
+            if constexpr (kInputs == 2) {
+                if constexpr (RM == MODE_ROWVEC) vb = *reinterpret_cast<const u32x4*>(rbase + voff);
+                else vb = load_stream(rbase + off);
+            }
+            const u32x4 r = op_chunk<DT, OP>(va, vb);
+            uint8_t* dst = obase + off;
+            if (valid == L::kPerChunk) {
+                store_stream(dst, r);
+            } else {
+                const uint32_t words[4] = {r.x, r.y, r.z, r.w};
+                for (uint32_t e = 0; e < valid; ++e) {
+                    if constexpr (L::kBytes == 2)
+                        reinterpret_cast<uint16_t*>(dst)[e] = (uint16_t)(words[e >> 1] >> ((e & 1) * 16));
+                    else
+                        reinterpret_cast<uint32_t*>(dst)[e] = words[e];
+                }
+            }
+        }
+    }
+}
+
 // One lane = one 16-byte piece (kPerChunk elements) of one logical result row.
 template <int DT, int OP>
 __global__ __launch_bounds__(kBlock) void elementwise_general_kernel(const GeneralArgs a) {
@@ -463,6 +525,44 @@ int dispatch(int op, bool planes, int lm, int rm, const BinaryArgs& pa, const Ge
     return IOMX_ERR_UNSUPPORTED;
 }
 
+template <int DT, int OP>
+int launch_padded(int lm, int rm, const PaddedArgs& pa, hipStream_t s) {
+    const uint64_t gx = (pa.b.seg_chunks + kPlanesBlock - 1) / kPlanesBlock;
+    if (gx > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
+    const dim3 grid((uint32_t)gx, pa.b.segments < 65535u ? pa.b.segments : 65535u,
+                    pa.b.planes < 65535u ? pa.b.planes : 65535u);
+#define IOMX_PADDED(LMV, RMV)                                                                  \
+    hipLaunchKernelGGL((elementwise_padded_kernel<DT, OP, LMV, RMV>), grid, dim3(kPlanesBlock), 0, s, pa)
+    if (lm == MODE_FULL && rm == MODE_FULL) IOMX_PADDED(MODE_FULL, MODE_FULL);
+    else if constexpr (OP <= IOMX_OP_SUB) {
+        if (lm == MODE_FULL) IOMX_PADDED(MODE_FULL, MODE_ROWVEC);
+        else IOMX_PADDED(MODE_ROWVEC, MODE_FULL);
+    } else {
+        return IOMX_ERR_INVALID;
+    }
+#undef IOMX_PADDED
+    const char* name = OP == OP_SILU ? "silu_padded" : OP == OP_COPY ? "copy_padded"
+            : OP == OP_SILU_MUL ? "silu_mul_padded" : "binary_padded";
+    record_launch(name, (uint32_t)gx, kPlanesBlock, gx * pa.b.segments * pa.b.planes);
+    return IOMX_OK;
+}
+
+template <int DT>
+int dispatch_padded(int op, int lm, int rm, const PaddedArgs& pa, hipStream_t s) {
+    switch (op) {
+        case IOMX_OP_ADD: return launch_padded<DT, IOMX_OP_ADD>(lm, rm, pa, s);
+        case IOMX_OP_MUL: return launch_padded<DT, IOMX_OP_MUL>(lm, rm, pa, s);
+        case IOMX_OP_SUB: return launch_padded<DT, IOMX_OP_SUB>(lm, rm, pa, s);
+        case OP_COPY: return launch_padded<DT, OP_COPY>(lm, rm, pa, s);
+        default: break;
+    }
+    if constexpr (DT != IOMX_DT_I32) {
+        if (op == OP_SILU) return launch_padded<DT, OP_SILU>(lm, rm, pa, s);
+        if (op == OP_SILU_MUL) return launch_padded<DT, OP_SILU_MUL>(lm, rm, pa, s);
+    }
+    return IOMX_ERR_UNSUPPORTED;
+}
+
 // Shared admission + planning of every elementwise operation.  `rhs` is null
 // for the one-input operations.
 enum AliasPolicy { ALIAS_NONE, ALIAS_EXACT, ALIAS_ANY };
@@ -513,7 +613,7 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
     const uint64_t rows = rdims[rank - 2], cols = rdims[rank - 1];
     const bool no_pad = rows % kTile == 0 && cols % kTile == 0;
     int mode[2] = {MODE_FULL, MODE_FULL};
-    bool planes_ok = no_pad;
+    bool planes_ok = true;   // operand modes the streaming kernels take (padding decided below)
     for (int k = 0; k < 2 && planes_ok; ++k) {
         if (!snap[k].brow && !snap[k].bcol) mode[k] = MODE_FULL;
         else if (snap[k].brow && !snap[k].bcol) mode[k] = MODE_ROWVEC;
@@ -522,6 +622,9 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
     if (planes_ok && mode[0] == MODE_ROWVEC && mode[1] == MODE_ROWVEC) planes_ok = false;
     if (planes_ok && op > IOMX_OP_SUB && (mode[0] != MODE_FULL || mode[1] != MODE_FULL))
         planes_ok = false;
+
+    const bool modes_ok = planes_ok;
+    planes_ok = modes_ok && no_pad;
 
     // A copy of whole planes is a move of bytes whatever the leaf.  Everything else
     // outside the four streaming leaves goes to the tile-row kernels.
@@ -541,6 +644,54 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
     }
     // byte counts below: exact for every width since a plane holds a multiple of 256 slots
     const uint64_t bytes8 = bits;  // bits per element; sizes are formed as elems * bits / 8
+
+    if (modes_ok && !no_pad && rows <= 0xFFFFFFFFull && cols <= 0xFFFFFFFFull) {
+        // padded planes: whole bands, chunk validity decided per lane
+        PaddedArgs pd = {};
+        BinaryArgs& b = pd.b;
+        b.src[0] = static_cast<const uint8_t*>(lhs->base);
+        b.src[1] = static_cast<const uint8_t*>(rhs->base);
+        b.out = static_cast<uint8_t*>(out->base);
+        b.walk = walk;
+        for (int k = 0; k < 3; ++k) b.plane_bytes[k] = m[k].plane_elems * bytes8 / 8;
+        b.seg_chunks = m[2].tile_cols * (kTileSlots * bytes8 / 128);
+        uint64_t planes = walk.planes, segments = m[2].tile_rows;
+        bool fold = walk.nlead <= 1;
+        for (int k = 0; k < 3 && fold; ++k) {
+            const bool vec = k < 2 && mode[k] == MODE_ROWVEC;
+            if (vec) fold = walk.nlead == 0 || walk.stride[k][0] == 0;
+            else fold = walk_is_dense(walk, k);
+        }
+        if (fold) {
+            b.src[0] += offsets[0] * b.plane_bytes[0];
+            b.src[1] += offsets[1] * b.plane_bytes[1];
+            b.out += offsets[2] * b.plane_bytes[2];
+            for (int k = 0; k < 3; ++k) b.walk.offset[k] = 0;
+            b.walk.nlead = 0;
+            if (mul_overflows(segments, planes, &segments)) return IOMX_ERR_OVERFLOW;
+            planes = 1;
+            pd.folded = 1;
+        }
+        if (segments > 0xFFFFFFFFull || planes > 0xFFFFFFFFull || m[2].tile_rows > 0xFFFFFFFFull)
+            return IOMX_ERR_OVERFLOW;
+        b.segments = (uint32_t)segments;
+        b.planes = (uint32_t)planes;
+        pd.rows = (uint32_t)rows;
+        pd.cols = (uint32_t)cols;
+        pd.tile_rows = (uint32_t)m[2].tile_rows;
+        pd.div_tile_rows = make_fast_div(pd.tile_rows);
+        const hipStream_t ps = native(stream);
+        int prc;
+        if (op == OP_COPY) {
+            prc = bits == 16 ? dispatch_padded<IOMX_DT_BF16>(op, mode[0], mode[1], pd, ps)
+                             : dispatch_padded<IOMX_DT_I32>(op, mode[0], mode[1], pd, ps);
+        } else if (dtype == IOMX_DT_BF16) prc = dispatch_padded<IOMX_DT_BF16>(op, mode[0], mode[1], pd, ps);
+        else if (dtype == IOMX_DT_F32) prc = dispatch_padded<IOMX_DT_F32>(op, mode[0], mode[1], pd, ps);
+        else prc = dispatch_padded<IOMX_DT_I32>(op, mode[0], mode[1], pd, ps);
+        IOMX_TRY(prc);
+        IOMX_HIP(hipGetLastError());
+        return IOMX_OK;
+    }
 
     BinaryArgs pa = {};
     GeneralArgs ga = {};

@@ -97,7 +97,7 @@ def test_copy_between_views(dtype, dims, family):
     if family == "copy_planes":
         assert kernel_name() == "copy_planes"
     else:
-        assert kernel_name() == ("copy_general" if LEAF_BITS[dtype] in (16, 32) else "rows_copy")
+        assert kernel_name() == ("copy_padded" if LEAF_BITS[dtype] in (16, 32) else "rows_copy")
     assert iomo.copy(src(hs), dst(hd)) == 0
     assert same_storage(dd, hd)
     ds.free()

@@ -104,14 +104,17 @@ def test_scatter_gather_match_the_closed_form_layout(dtype, dims, steps):
 
 BINARY_CASES = [
     # lhs owner dims, lhs steps, rhs owner dims, rhs steps, out owner dims, out steps, kernel family
-    ((2, 17, 33), [], (2, 17, 33), [], (2, 17, 33), [], "binary_general"),
-    ((1, 17, 33), [], (1, 17, 33), [], (1, 17, 33), [], "binary_general"),
+    ((2, 17, 33), [], (2, 17, 33), [], (2, 17, 33), [], "binary_padded"),
+    ((1, 17, 33), [], (1, 17, 33), [], (1, 17, 33), [], "binary_padded"),
     ((2, 1, 33), [], (1, 17, 1), [], (2, 17, 33), [], "binary_general"),
     ((3, 32, 48), [], (1, 48), [], (3, 32, 48), [], "binary_rowvec"),
     ((1, 48), [], (3, 32, 48), [], (3, 32, 48), [], "binary_rowvec"),
     ((3, 32, 48), [], (32, 1), [], (3, 32, 48), [], "binary_general"),
     ((1, 1), [], (2, 2, 16, 16), [], (2, 2, 16, 16), [], "binary_general"),
-    ((6, 20, 35), [("slice", (0, 1, 3, 2))], (3, 20, 35), [], (3, 20, 35), [], "binary_general"),
+    ((6, 20, 35), [("slice", (0, 1, 3, 2))], (3, 20, 35), [], (3, 20, 35), [], "binary_padded"),
+    ((3, 40, 4100), [], (1, 4100), [], (3, 40, 4100), [], "binary_padded"),
+    ((1, 52), [], (4, 3, 21, 52), [("permute", ([1, 0],))], (3, 4, 21, 52), [], "binary_padded"),
+    ((5, 500, 272), [], (5, 500, 272), [], (5, 500, 272), [], "binary_padded"),
     ((6, 32, 64), [("slice", (0, 1, 3, 2))], (3, 32, 64), [], (3, 32, 64), [], "binary_planes"),
     ((4, 3, 16, 32), [("permute", ([1, 0],))], (3, 4, 16, 32), [], (3, 4, 16, 32), [], "binary_planes"),
     ((4, 3, 16, 32), [("select", (0, 2))], (1, 16, 32), [], (5, 3, 16, 32), [("select", (0, 4))],
@@ -391,7 +394,7 @@ def test_rmsnorm_rejections():
 
 @pytest.mark.parametrize("dtype", [DT_BF16, DT_F32])
 @pytest.mark.parametrize("dims,steps,family", [
-    ((17, 33), [], "silu_general"), ((3, 16, 48), [], "silu_planes"),
+    ((17, 33), [], "silu_padded"), ((3, 16, 48), [], "silu_planes"),
     ((4, 2, 16, 16), [("permute", ([1, 0],))], "silu_planes"), ((64, 5632), [], "silu_planes"),
 ])
 @pytest.mark.parametrize("kind", ["normal", "bits"])
@@ -465,8 +468,8 @@ def test_fused_silu_mul_equals_the_two_operation_sequence(dtype, dims):
 
 @pytest.mark.parametrize("dtype", [DT_BF16, DT_F32, DT_I32])
 @pytest.mark.parametrize("sd,ss,dd,ds,family", [
-    ((2, 17, 33), [], (2, 17, 33), [], "copy_general"),
-    ((6, 20, 35), [("slice", (0, 1, 3, 2))], (3, 20, 35), [], "copy_general"),
+    ((2, 17, 33), [], (2, 17, 33), [], "copy_padded"),
+    ((6, 20, 35), [("slice", (0, 1, 3, 2))], (3, 20, 35), [], "copy_padded"),
     ((4, 3, 16, 32), [("permute", ([1, 0],))], (3, 4, 16, 32), [], "copy_planes"),
     ((3, 16, 16), [], (5, 3, 16, 16), [("select", (0, 1))], "copy_planes"),
     ((8, 64, 512), [], (8, 64, 512), [], "copy_planes"),
