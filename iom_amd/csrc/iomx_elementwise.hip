@@ -17,7 +17,9 @@
 
 namespace iomx {
 
-enum { MODE_FULL = 0, MODE_ROWVEC = 1 };
+// Operand shapes relative to the result plane: whole planes, a [.,1,F] row vector,
+// a [.,R,1] column vector, a [.,1,1] scalar (the last two on the padded kernel only).
+enum { MODE_FULL = 0, MODE_ROWVEC = 1, MODE_COLVEC = 2, MODE_SCALAR = 3 };
 
 // Internal operation codes: the three public binary operations keep their ABI
 // values; the rest are private to this file.
@@ -273,6 +275,31 @@ struct PaddedArgs {
     uint32_t folded;          // segments run over several planes: band = segment mod tile_rows
 };
 
+// One operand's chunk: streamed for whole planes; for the broadcast shapes the one
+// element a lane needs (row 0 of its tile column is a whole chunk; a column vector
+// holds element (row, 0) of tile (band, 0); a scalar is element 0 of its plane),
+// replicated across the chunk.
+template <int DT, int MODE>
+__device__ __forceinline__ u32x4 padded_operand(const uint8_t* base, uint64_t off, uint64_t voff,
+                                                uint32_t band, uint32_t row) {
+    using L = Leaf<DT>;
+    if constexpr (MODE == MODE_FULL) {
+        return load_stream(base + off);
+    } else if constexpr (MODE == MODE_ROWVEC) {
+        return *reinterpret_cast<const u32x4*>(base + voff);
+    } else {
+        const uint64_t slot = MODE == MODE_COLVEC ? (uint64_t)band * kTileSlots + row * kTile : 0;
+        uint32_t word;
+        if constexpr (L::kBytes == 2) {
+            const uint32_t e = *reinterpret_cast<const uint16_t*>(base + slot * 2);
+            word = e | (e << 16);
+        } else {
+            word = *reinterpret_cast<const uint32_t*>(base + slot * 4);
+        }
+        return u32x4{word, word, word, word};
+    }
+}
+
 template <int DT, int OP, int LM, int RM>
 __global__ __launch_bounds__(kPlanesBlock) void elementwise_padded_kernel(const PaddedArgs a) {
     using L = Leaf<DT>;
@@ -298,13 +325,9 @@ __global__ __launch_bounds__(kPlanesBlock) void elementwise_padded_kernel(const 
             else if (a.folded) tr = 0;
             if (tr * kTile + row >= a.rows) continue;
             const uint64_t off = ((uint64_t)y * a.b.seg_chunks + cb) * 16;
-            u32x4 va, vb = u32x4{0, 0, 0, 0};
-            if constexpr (LM == MODE_ROWVEC) va = *reinterpret_cast<const u32x4*>(lbase + voff);
-            else va = load_stream(lbase + off);
-            if constexpr (kInputs == 2) {
-                if constexpr (RM == MODE_ROWVEC) vb = *reinterpret_cast<const u32x4*>(rbase + voff);
-                else vb = load_stream(rbase + off);
-            }
+            const u32x4 va = padded_operand<DT, LM>(lbase, off, voff, tr, row);
+            u32x4 vb = u32x4{0, 0, 0, 0};
+            if constexpr (kInputs == 2) vb = padded_operand<DT, RM>(rbase, off, voff, tr, row);
             const u32x4 r = op_chunk<DT, OP>(va, vb);
             uint8_t* dst = obase + off;
             if (valid == L::kPerChunk) {
@@ -535,8 +558,13 @@ int launch_padded(int lm, int rm, const PaddedArgs& pa, hipStream_t s) {
     hipLaunchKernelGGL((elementwise_padded_kernel<DT, OP, LMV, RMV>), grid, dim3(kPlanesBlock), 0, s, pa)
     if (lm == MODE_FULL && rm == MODE_FULL) IOMX_PADDED(MODE_FULL, MODE_FULL);
     else if constexpr (OP <= IOMX_OP_SUB) {
-        if (lm == MODE_FULL) IOMX_PADDED(MODE_FULL, MODE_ROWVEC);
-        else IOMX_PADDED(MODE_ROWVEC, MODE_FULL);
+        if (lm == MODE_FULL && rm == MODE_ROWVEC) IOMX_PADDED(MODE_FULL, MODE_ROWVEC);
+        else if (lm == MODE_FULL && rm == MODE_COLVEC) IOMX_PADDED(MODE_FULL, MODE_COLVEC);
+        else if (lm == MODE_FULL && rm == MODE_SCALAR) IOMX_PADDED(MODE_FULL, MODE_SCALAR);
+        else if (lm == MODE_ROWVEC && rm == MODE_FULL) IOMX_PADDED(MODE_ROWVEC, MODE_FULL);
+        else if (lm == MODE_COLVEC && rm == MODE_FULL) IOMX_PADDED(MODE_COLVEC, MODE_FULL);
+        else if (lm == MODE_SCALAR && rm == MODE_FULL) IOMX_PADDED(MODE_SCALAR, MODE_FULL);
+        else return IOMX_ERR_INVALID;
     } else {
         return IOMX_ERR_INVALID;
     }
@@ -613,18 +641,17 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
     const uint64_t rows = rdims[rank - 2], cols = rdims[rank - 1];
     const bool no_pad = rows % kTile == 0 && cols % kTile == 0;
     int mode[2] = {MODE_FULL, MODE_FULL};
-    bool planes_ok = true;   // operand modes the streaming kernels take (padding decided below)
-    for (int k = 0; k < 2 && planes_ok; ++k) {
+    for (int k = 0; k < 2; ++k) {
         if (!snap[k].brow && !snap[k].bcol) mode[k] = MODE_FULL;
         else if (snap[k].brow && !snap[k].bcol) mode[k] = MODE_ROWVEC;
-        else planes_ok = false;
+        else if (!snap[k].brow && snap[k].bcol) mode[k] = MODE_COLVEC;
+        else mode[k] = MODE_SCALAR;
     }
-    if (planes_ok && mode[0] == MODE_ROWVEC && mode[1] == MODE_ROWVEC) planes_ok = false;
-    if (planes_ok && op > IOMX_OP_SUB && (mode[0] != MODE_FULL || mode[1] != MODE_FULL))
-        planes_ok = false;
-
-    const bool modes_ok = planes_ok;
-    planes_ok = modes_ok && no_pad;
+    // the chunk-mapped kernels take at most one operand that is not whole planes
+    bool modes_ok = mode[0] == MODE_FULL || mode[1] == MODE_FULL;
+    if (op > IOMX_OP_SUB && (mode[0] != MODE_FULL || mode[1] != MODE_FULL)) modes_ok = false;
+    const bool lean_modes = mode[0] <= MODE_ROWVEC && mode[1] <= MODE_ROWVEC;
+    bool planes_ok = modes_ok && lean_modes && no_pad;
 
     // A copy of whole planes is a move of bytes whatever the leaf.  Everything else
     // outside the four streaming leaves goes to the tile-row kernels.
@@ -645,8 +672,8 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
     // byte counts below: exact for every width since a plane holds a multiple of 256 slots
     const uint64_t bytes8 = bits;  // bits per element; sizes are formed as elems * bits / 8
 
-    if (modes_ok && !no_pad && rows <= 0xFFFFFFFFull && cols <= 0xFFFFFFFFull) {
-        // padded planes: whole bands, chunk validity decided per lane
+    if (modes_ok && (!no_pad || !lean_modes) && rows <= 0xFFFFFFFFull && cols <= 0xFFFFFFFFull) {
+        // padded planes, column vectors, scalars: whole bands, chunk validity decided per lane
         PaddedArgs pd = {};
         BinaryArgs& b = pd.b;
         b.src[0] = static_cast<const uint8_t*>(lhs->base);
@@ -658,7 +685,7 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
         uint64_t planes = walk.planes, segments = m[2].tile_rows;
         bool fold = walk.nlead <= 1;
         for (int k = 0; k < 3 && fold; ++k) {
-            const bool vec = k < 2 && mode[k] == MODE_ROWVEC;
+            const bool vec = k < 2 && mode[k] != MODE_FULL;
             if (vec) fold = walk.nlead == 0 || walk.stride[k][0] == 0;
             else fold = walk_is_dense(walk, k);
         }

@@ -109,8 +109,11 @@ BINARY_CASES = [
     ((2, 1, 33), [], (1, 17, 1), [], (2, 17, 33), [], "binary_general"),
     ((3, 32, 48), [], (1, 48), [], (3, 32, 48), [], "binary_rowvec"),
     ((1, 48), [], (3, 32, 48), [], (3, 32, 48), [], "binary_rowvec"),
-    ((3, 32, 48), [], (32, 1), [], (3, 32, 48), [], "binary_general"),
-    ((1, 1), [], (2, 2, 16, 16), [], (2, 2, 16, 16), [], "binary_general"),
+    ((3, 32, 48), [], (32, 1), [], (3, 32, 48), [], "binary_padded"),
+    ((3, 1), [], (5, 3, 19), [], (5, 3, 19), [], "binary_padded"),
+    ((4, 3, 35, 1), [("permute", ([1, 0],))], (3, 4, 35, 50), [], (3, 4, 35, 50), [], "binary_padded"),
+    ((2, 40, 64), [], (2, 1, 1), [], (2, 40, 64), [], "binary_padded"),
+    ((1, 1), [], (2, 2, 16, 16), [], (2, 2, 16, 16), [], "binary_padded"),
     ((6, 20, 35), [("slice", (0, 1, 3, 2))], (3, 20, 35), [], (3, 20, 35), [], "binary_padded"),
     ((3, 40, 4100), [], (1, 4100), [], (3, 40, 4100), [], "binary_padded"),
     ((1, 52), [], (4, 3, 21, 52), [("permute", ([1, 0],))], (3, 4, 21, 52), [], "binary_padded"),
