@@ -159,6 +159,14 @@ int iomc_device_backend_kind(const iomc_device* device) {
     return static_cast<int>(device->device->backend_kind());
 }
 
+// Device::supported_data_types() (include/iom/device.hpp:57-131): writes up to
+// `capacity` leaf codes in the advertised order and returns the full count.
+std::uint32_t iomc_device_supported_types(const iomc_device* device, int* codes, std::uint32_t capacity) {
+    const auto types = device->device->supported_data_types();
+    for (std::uint32_t i = 0; i < types.size() && i < capacity; ++i) codes[i] = static_cast<int>(types[i]);
+    return static_cast<std::uint32_t>(types.size());
+}
+
 iomc_tensor* iomc_tensor_create(
         iomc_device* device, int dtype, std::uint32_t rank,
         const std::uint64_t* dims) {

@@ -404,6 +404,8 @@ def bind_iomc(l: C.CDLL) -> C.CDLL:
         l.iomc_mi355x_device_create.argtypes = [C.c_uint32, C.c_size_t, C.c_size_t]
     l.iomc_device_destroy.argtypes = [P]
     l.iomc_device_backend_kind.argtypes = [P]
+    l.iomc_device_supported_types.restype = C.c_uint32
+    l.iomc_device_supported_types.argtypes = [P, C.POINTER(C.c_int), C.c_uint32]
     l.iomc_tensor_create.restype = P
     l.iomc_tensor_create.argtypes = [P, C.c_int, C.c_uint32, U64P]
     l.iomc_tensor_destroy.argtypes = [P]
@@ -555,6 +557,21 @@ class IomBackend:
     def tensor(self, dtype, dims) -> IomTensor:
         return IomTensor(self, dtype, dims)
 
+    def supported_types(self):
+        codes = (C.c_int * 64)()
+        n = self.l.iomc_device_supported_types(self.dev, codes, 64)
+        return list(codes[:n])
+
+    def second_queue(self) -> "IomBackend":
+        """Another queue of the same device (shares the device handle; close() it first)."""
+        other = object.__new__(IomBackend)
+        other.l, other.dev = self.l, self.dev
+        other.queue = self.l.iomc_queue_create(self.dev)
+        if not other.queue:
+            raise RuntimeError(self.error())
+        other.borrowed = True
+        return other
+
     def wait(self, token: int) -> int:
         return self.l.iomc_wait(self.queue, token)
 
@@ -597,6 +614,8 @@ class IomBackend:
         if self.queue:
             self.l.iomc_queue_destroy(self.queue)
             self.queue = None
+        if getattr(self, "borrowed", False):
+            self.dev = None
         if self.dev:
             self.l.iomc_device_destroy(self.dev)
             self.dev = None

@@ -123,6 +123,7 @@ def test_every_standard_leaf_is_advertised_in_order(devices):
     """23 leaves in the published order (src/shared/standard_tiled_copy.hpp:17-31); the
     conformance drivers iterate exactly this list (test/rocm/test_rocm_conformance.cpp:225-240)."""
     cpu, gpu = devices
+    assert gpu.supported_types() == list(ALL_LEAVES) == cpu.supported_types()
     for dtype in ALL_LEAVES:                     # creation is refused for an unadvertised leaf
         t = gpu.tensor(dtype, (3, 5))
         t.close()
@@ -253,6 +254,38 @@ def test_in_order_queue_with_more_submissions_than_credits(devices):
     assert gpu.wait(last) == 0                      # repeat-waitable
     assert np.all(acc_g.view().to_host() == 64)
     close(acc_c, acc_g, one_c, one_g)
+
+
+def test_two_queues_and_an_owner_released_while_its_work_is_in_flight(devices):
+    """Queues of one device run independently and keep their own token spaces; an owner
+    destroyed right after submission is kept alive by the queue until completion
+    (docs/BACKEND_CONTRACT/queue-and-token-contract.md)."""
+    cpu, gpu = devices
+    q2 = gpu.second_queue()
+    dims = (8, 64, 256)
+    a = gpu.tensor(DT_F32, dims); b = gpu.tensor(DT_F32, dims)
+    o1 = gpu.tensor(DT_F32, dims); o2 = gpu.tensor(DT_F32, dims)
+    va = datagen.uniform_f32(int(np.prod(dims)), -1, 1, 1).view(np.uint32).reshape(dims)
+    vb = datagen.uniform_f32(int(np.prod(dims)), -1, 1, 2).view(np.uint32).reshape(dims)
+    a.view().from_host(va); b.view().from_host(vb)
+    t1 = gpu.l.iomc_binary(gpu.queue, OP_ADD, a.view().h, b.view().h, o1.view().h)
+    t2 = q2.l.iomc_binary(q2.queue, OP_MUL, a.view().h, b.view().h, o2.view().h)
+    assert t1 > 0 and t2 > 0
+    assert (t1 >> 55) != (t2 >> 55)                       # different queue ids in the tokens
+    assert gpu.wait(t2) != 0                              # a token of the other queue is refused
+    assert q2.wait(t2) == 0 and gpu.wait(t1) == 0
+    fa, fb = va.view(np.float32), vb.view(np.float32)
+    assert np.array_equal(o1.view().to_host().view(np.float32), fa + fb)
+    assert np.array_equal(o2.view().to_host().view(np.float32), fa * fb)
+    # release the inputs immediately after submitting
+    tmp = gpu.tensor(DT_F32, dims)
+    tmp.view().from_host(va)
+    t3 = gpu.l.iomc_binary(gpu.queue, OP_SUB, tmp.view().h, b.view().h, o1.view().h)
+    tmp.close()
+    assert t3 > 0 and gpu.wait(t3) == 0
+    assert np.array_equal(o1.view().to_host().view(np.float32), fa - fb)
+    q2.close()
+    close(a, b, o1, o2)
 
 
 def test_arena_exhaustion_and_reuse(devices):
