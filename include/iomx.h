@@ -279,6 +279,12 @@ int iomx_last_launch(iomx_launch_info* info);
  * even rule over all 2^32 binary32 encodings; *mismatches receives the count. */
 int iomx_selftest_bf16_convert(uint64_t* mismatches, iomx_stream_t stream);
 
+/* Compares the packed F16 arithmetic of the streaming kernels (hardware F16 <->
+ * binary32 conversions around one binary32 operation) with the integer-rounded
+ * binary64 rule for all 2^32 operand pairs and ADD, MUL, SUB; *mismatches receives
+ * the count. */
+int iomx_selftest_f16_binary(uint64_t* mismatches, iomx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

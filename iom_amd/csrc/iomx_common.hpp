@@ -42,10 +42,17 @@ inline uint32_t leaf_bits(int dtype) {
     return (dtype >= 0 && dtype < 23) ? kBits[dtype] : 0;
 }
 
-// The leaves whose arithmetic runs on the streaming kernels.
+// The leaves whose arithmetic runs on the streaming kernels: the integers of 8 to
+// 64 bits, F16, BF16, F32 and F64.
 inline bool streaming_leaf(int dtype) {
-    return dtype == IOMX_DT_I32 || dtype == IOMX_DT_U32 || dtype == IOMX_DT_F32
-            || dtype == IOMX_DT_BF16;
+    switch (dtype) {
+        case IOMX_DT_I8: case IOMX_DT_U8: case IOMX_DT_I16: case IOMX_DT_U16:
+        case IOMX_DT_I32: case IOMX_DT_U32: case IOMX_DT_I64: case IOMX_DT_U64:
+        case IOMX_DT_F16: case IOMX_DT_BF16: case IOMX_DT_F32: case IOMX_DT_F64:
+            return true;
+        default:
+            return false;
+    }
 }
 
 inline uint32_t leaf_bytes(int dtype) {

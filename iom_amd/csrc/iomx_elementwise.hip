@@ -1,6 +1,8 @@
 // Elementwise operations on tiled, plane-strided, broadcast views:
-// ADD / SUB / MUL over I32, U32, F32, BF16; SiLU and SiLU*up over F32, BF16;
-// same-spec copy.  Two kernel families, selected on the host:
+// ADD / SUB / MUL over the integers of 8 to 64 bits, F16, BF16, F32 and F64; SiLU
+// and SiLU*up over the four floating ones; same-spec copy.  (The 2/4/6-bit leaves
+// and the 8-bit floats run on the tile-row kernels.)  Kernel families, selected on
+// the host:
 //
 //   *_planes        every operand either covers whole 16x16-tiled planes
 //                   (FULL) or is a [.,1,F] row vector broadcast over rows
@@ -14,6 +16,7 @@
 // Both read every input of a chunk before storing it, so an input that is the
 // exact alias of the output is safe without staging.
 #include "iomx_leaves.hpp"
+#include "iomx_rows.hpp"
 
 namespace iomx {
 
@@ -85,19 +88,47 @@ struct GeneralArgs {
     uint32_t brow[2], bcol[2];
 };
 
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// Leaf classes of the chunk kernels: signed and unsigned integers of one width
+// share a class (two's-complement wrap does not see the sign).
+constexpr bool is_float_class(int dt) {
+    return dt == IOMX_DT_F16 || dt == IOMX_DT_BF16 || dt == IOMX_DT_F32 || dt == IOMX_DT_F64;
+}
+
+// Two F16 values of one word as binary32 and back.  The widening is exact; the
+// narrowing is the hardware's round-to-nearest-even with gradual underflow, and
+// one binary32 operation between them rounds innocuously (24 >= 2*11 + 2), so
+// the pair equals one correctly rounded binary16 operation.  NaN results are
+// made canonical (0x7E00) before the narrowing.
+__device__ __forceinline__ f32x2 f16_pair(uint32_t w) {
+    return __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+}
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+    const f32x2 v = {canonical(lo), canonical(hi)};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+
 template <int DT, int OP>
 __device__ __forceinline__ uint32_t op_word(uint32_t a, uint32_t b) {
     if constexpr (OP == OP_COPY) {
         return a;
     } else if constexpr (OP == OP_SILU) {
         if constexpr (DT == IOMX_DT_F32) return as_u32(canonical(silu_f32(as_f32(a))));
-        else return pack_bf16(silu_for_bf16(bf16_lo(a)), silu_for_bf16(bf16_hi(a)));
+        else if constexpr (DT == IOMX_DT_F16) {
+            const f32x2 x = f16_pair(a);
+            return pack_f16(silu_for_bf16(x.x), silu_for_bf16(x.y));
+        } else return pack_bf16(silu_for_bf16(bf16_lo(a)), silu_for_bf16(bf16_hi(a)));
     } else if constexpr (OP == OP_SILU_MUL) {
         // the activation is rounded to the leaf before the product, exactly as
         // the stored intermediate of the two-operation sequence
         if constexpr (DT == IOMX_DT_F32) {
             const float act = canonical(silu_f32(as_f32(a)));
             return as_u32(canonical(act * as_f32(b)));
+        } else if constexpr (DT == IOMX_DT_F16) {
+            const f32x2 x = f16_pair(a);
+            const f32x2 act = f16_pair(pack_f16(silu_for_bf16(x.x), silu_for_bf16(x.y))), y = f16_pair(b);
+            return pack_f16(act.x * y.x, act.y * y.y);
         } else {
             const uint32_t act = pack_bf16(silu_for_bf16(bf16_lo(a)), silu_for_bf16(bf16_hi(a)));
             return pack_bf16(bf16_lo(act) * bf16_lo(b), bf16_hi(act) * bf16_hi(b));
@@ -106,6 +137,23 @@ __device__ __forceinline__ uint32_t op_word(uint32_t a, uint32_t b) {
         if constexpr (OP == IOMX_OP_ADD) return a + b;
         else if constexpr (OP == IOMX_OP_MUL) return a * b;
         else return a - b;
+    } else if constexpr (DT == IOMX_DT_I16) {
+        // two 16-bit lanes: carries are kept out of the neighbour's top bit
+        constexpr uint32_t H = 0x80008000u, L7 = 0x7FFF7FFFu;
+        if constexpr (OP == IOMX_OP_ADD) return ((a & L7) + (b & L7)) ^ ((a ^ b) & H);
+        else if constexpr (OP == IOMX_OP_SUB) return ((a | H) - (b & L7)) ^ ((a ^ ~b) & H);
+        else return ((a & 0xFFFFu) * (b & 0xFFFFu) & 0xFFFFu) | ((a >> 16) * (b >> 16) << 16);
+    } else if constexpr (DT == IOMX_DT_I8) {
+        constexpr uint32_t H = 0x80808080u, L7 = 0x7F7F7F7Fu;
+        if constexpr (OP == IOMX_OP_ADD) return ((a & L7) + (b & L7)) ^ ((a ^ b) & H);
+        else if constexpr (OP == IOMX_OP_SUB) return ((a | H) - (b & L7)) ^ ((a ^ ~b) & H);
+        else {
+            uint32_t r = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                r |= ((((a >> (8 * i)) & 0xFFu) * ((b >> (8 * i)) & 0xFFu)) & 0xFFu) << (8 * i);
+            return r;
+        }
     } else if constexpr (DT == IOMX_DT_F32) {
         const float x = as_f32(a), y = as_f32(b);
         float r;
@@ -113,6 +161,13 @@ __device__ __forceinline__ uint32_t op_word(uint32_t a, uint32_t b) {
         else if constexpr (OP == IOMX_OP_MUL) r = x * y;
         else r = x - y;
         return as_u32(canonical(r));
+    } else if constexpr (DT == IOMX_DT_F16) {
+        const f32x2 x = f16_pair(a), y = f16_pair(b);
+        f32x2 r;
+        if constexpr (OP == IOMX_OP_ADD) r = x + y;
+        else if constexpr (OP == IOMX_OP_MUL) r = x * y;
+        else r = x - y;
+        return pack_f16(r.x, r.y);
     } else {
         // BF16 pair.  The binary32 result of one operation on two BF16 values
         // is exact or correctly rounded with enough guard bits that the single
@@ -127,19 +182,80 @@ __device__ __forceinline__ uint32_t op_word(uint32_t a, uint32_t b) {
     }
 }
 
+// One 64-bit element (two words of a chunk).
+template <int DT, int OP>
+__device__ __forceinline__ uint64_t op_wide(uint64_t a, uint64_t b) {
+    if constexpr (OP == OP_COPY) {
+        return a;
+    } else if constexpr (DT == IOMX_DT_I64) {
+        if constexpr (OP == IOMX_OP_ADD) return a + b;
+        else if constexpr (OP == IOMX_OP_MUL) return a * b;
+        else return a - b;
+    } else {
+        const double x = as_f64(a), y = as_f64(b);
+        double r;
+        if constexpr (OP == OP_SILU) r = silu_carrier(x);
+        else if constexpr (OP == OP_SILU_MUL) {
+            const double act = silu_carrier(x);
+            r = ((act != act) ? as_f64(kQuietNanF64) : act) * y;
+        } else if constexpr (OP == IOMX_OP_ADD) r = x + y;
+        else if constexpr (OP == IOMX_OP_MUL) r = x * y;
+        else r = x - y;
+        return (r != r) ? kQuietNanF64 : as_u64(r);
+    }
+}
+
 template <int DT, int OP>
 __device__ __forceinline__ u32x4 op_chunk(u32x4 a, u32x4 b) {
     u32x4 r;
-    r.x = op_word<DT, OP>(a.x, b.x);
-    r.y = op_word<DT, OP>(a.y, b.y);
-    r.z = op_word<DT, OP>(a.z, b.z);
-    r.w = op_word<DT, OP>(a.w, b.w);
+    if constexpr (DT == IOMX_DT_I64 || DT == IOMX_DT_F64) {
+        const uint64_t lo = op_wide<DT, OP>((uint64_t)a.x | ((uint64_t)a.y << 32), (uint64_t)b.x | ((uint64_t)b.y << 32));
+        const uint64_t hi = op_wide<DT, OP>((uint64_t)a.z | ((uint64_t)a.w << 32), (uint64_t)b.z | ((uint64_t)b.w << 32));
+        r.x = (uint32_t)lo; r.y = (uint32_t)(lo >> 32); r.z = (uint32_t)hi; r.w = (uint32_t)(hi >> 32);
+    } else {
+        r.x = op_word<DT, OP>(a.x, b.x);
+        r.y = op_word<DT, OP>(a.y, b.y);
+        r.z = op_word<DT, OP>(a.z, b.z);
+        r.w = op_word<DT, OP>(a.w, b.w);
+    }
     return r;
+}
+
+constexpr uint32_t class_bytes(int dt) {
+    return dt == IOMX_DT_I8 ? 1 : (dt == IOMX_DT_I16 || dt == IOMX_DT_F16 || dt == IOMX_DT_BF16) ? 2
+            : (dt == IOMX_DT_I64 || dt == IOMX_DT_F64) ? 8 : 4;
+}
+
+// One element replicated over a chunk, and the first `valid` elements of a chunk
+// stored one by one.
+template <int BYTES>
+__device__ __forceinline__ u32x4 splat_element(const uint8_t* p) {
+    if constexpr (BYTES == 8) {
+        const u32x2 e = *reinterpret_cast<const u32x2*>(p);
+        return u32x4{e.x, e.y, e.x, e.y};
+    } else {
+        uint32_t word;
+        if constexpr (BYTES == 1) word = *p * 0x01010101u;
+        else if constexpr (BYTES == 2) word = *reinterpret_cast<const uint16_t*>(p) * 0x00010001u;
+        else word = *reinterpret_cast<const uint32_t*>(p);
+        return u32x4{word, word, word, word};
+    }
+}
+
+template <int BYTES>
+__device__ __forceinline__ void store_elements(uint8_t* dst, u32x4 r, uint32_t valid) {
+    const uint32_t words[4] = {r.x, r.y, r.z, r.w};
+    for (uint32_t e = 0; e < valid; ++e) {
+        if constexpr (BYTES == 1) dst[e] = (uint8_t)(words[e >> 2] >> ((e & 3) * 8));
+        else if constexpr (BYTES == 2) reinterpret_cast<uint16_t*>(dst)[e] = (uint16_t)(words[e >> 1] >> ((e & 1) * 16));
+        else if constexpr (BYTES == 4) reinterpret_cast<uint32_t*>(dst)[e] = words[e];
+        else *reinterpret_cast<u32x2*>(dst + e * 8) = u32x2{words[2 * e], words[2 * e + 1]};
+    }
 }
 
 template <int DT>
 struct Leaf {
-    static constexpr uint32_t kBytes = (DT == IOMX_DT_BF16) ? 2 : 4;
+    static constexpr uint32_t kBytes = class_bytes(DT);
     static constexpr uint32_t kPerChunk = 16 / kBytes;          // elements per 16 bytes
     static constexpr uint32_t kChunksPerRow = kTile / kPerChunk; // per tile row
     static constexpr uint32_t kChunksPerTile = kTileSlots / kPerChunk;
@@ -289,14 +405,7 @@ __device__ __forceinline__ u32x4 padded_operand(const uint8_t* base, uint64_t of
         return *reinterpret_cast<const u32x4*>(base + voff);
     } else {
         const uint64_t slot = MODE == MODE_COLVEC ? (uint64_t)band * kTileSlots + row * kTile : 0;
-        uint32_t word;
-        if constexpr (L::kBytes == 2) {
-            const uint32_t e = *reinterpret_cast<const uint16_t*>(base + slot * 2);
-            word = e | (e << 16);
-        } else {
-            word = *reinterpret_cast<const uint32_t*>(base + slot * 4);
-        }
-        return u32x4{word, word, word, word};
+        return splat_element<L::kBytes>(base + slot * L::kBytes);
     }
 }
 
@@ -333,13 +442,7 @@ __global__ __launch_bounds__(kPlanesBlock) void elementwise_padded_kernel(const 
             if (valid == L::kPerChunk) {
                 store_stream(dst, r);
             } else {
-                const uint32_t words[4] = {r.x, r.y, r.z, r.w};
-                for (uint32_t e = 0; e < valid; ++e) {
-                    if constexpr (L::kBytes == 2)
-                        reinterpret_cast<uint16_t*>(dst)[e] = (uint16_t)(words[e >> 1] >> ((e & 1) * 16));
-                    else
-                        reinterpret_cast<uint32_t*>(dst)[e] = words[e];
-                }
+                store_elements<L::kBytes>(dst, r, valid);
             }
         }
     }
@@ -370,14 +473,7 @@ __global__ __launch_bounds__(kBlock) void elementwise_general_kernel(const Gener
                     + ((r / kTile) * a.tile_cols[k] + c / kTile) * kTileSlots
                     + (r % kTile) * kTile + c % kTile;
             if (a.bcol[k]) {
-                uint32_t word;
-                if constexpr (L::kBytes == 2) {
-                    const uint32_t e = *reinterpret_cast<const uint16_t*>(a.src[k] + slot * 2);
-                    word = e | (e << 16);
-                } else {
-                    word = *reinterpret_cast<const uint32_t*>(a.src[k] + slot * 4);
-                }
-                v[k] = u32x4{word, word, word, word};
+                v[k] = splat_element<L::kBytes>(a.src[k] + slot * L::kBytes);
             } else {
                 v[k] = *reinterpret_cast<const u32x4*>(a.src[k] + slot * L::kBytes);
             }
@@ -390,17 +486,33 @@ __global__ __launch_bounds__(kBlock) void elementwise_general_kernel(const Gener
         if (valid == L::kPerChunk) {
             *reinterpret_cast<u32x4*>(dst) = r;
         } else {
-            const uint32_t words[4] = {r.x, r.y, r.z, r.w};
-            for (uint32_t e = 0; e < valid; ++e) {
-                if constexpr (L::kBytes == 2) {
-                    reinterpret_cast<uint16_t*>(dst)[e] =
-                            (uint16_t)(words[e >> 1] >> ((e & 1) * 16));
-                } else {
-                    reinterpret_cast<uint32_t*>(dst)[e] = words[e];
-                }
-            }
+            store_elements<L::kBytes>(dst, r, valid);
         }
     }
+}
+
+// Self test: the packed F16 arithmetic of the streaming kernels (hardware
+// conversions around one binary32 operation) against the integer-rounded binary64
+// rule of the tile-row kernels, for every pair of binary16 encodings and the three
+// operations.
+__global__ __launch_bounds__(256) void f16_binary_selftest_kernel(unsigned long long* mismatches) {
+    unsigned long long bad = 0;
+    for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < (1ull << 31); i += (uint64_t)gridDim.x * 256) {
+        const uint64_t p0 = 2 * i, p1 = 2 * i + 1;   // pair index = a * 65536 + b
+        const uint32_t a0 = (uint32_t)(p0 >> 16), b0 = (uint32_t)(p0 & 0xFFFFu);
+        const uint32_t a1 = (uint32_t)(p1 >> 16), b1 = (uint32_t)(p1 & 0xFFFFu);
+        const uint32_t wa = a0 | (a1 << 16), wb = b0 | (b1 << 16);
+        const uint32_t add = op_word<IOMX_DT_F16, IOMX_OP_ADD>(wa, wb);
+        const uint32_t mul = op_word<IOMX_DT_F16, IOMX_OP_MUL>(wa, wb);
+        const uint32_t sub = op_word<IOMX_DT_F16, IOMX_OP_SUB>(wa, wb);
+        bad += (add & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_ADD>(a0, b0);
+        bad += (add >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_ADD>(a1, b1);
+        bad += (mul & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_MUL>(a0, b0);
+        bad += (mul >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_MUL>(a1, b1);
+        bad += (sub & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_SUB>(a0, b0);
+        bad += (sub >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_SUB>(a1, b1);
+    }
+    if (bad) atomicAdd(mismatches, bad);
 }
 
 // ---------------------------------------------------------------------------
@@ -541,7 +653,7 @@ int dispatch(int op, bool planes, int lm, int rm, const BinaryArgs& pa, const Ge
         case OP_COPY: return launch<DT, OP_COPY>(planes, lm, rm, pa, ga, s);
         default: break;
     }
-    if constexpr (DT != IOMX_DT_I32) {
+    if constexpr (is_float_class(DT)) {
         if (op == OP_SILU) return launch<DT, OP_SILU>(planes, lm, rm, pa, ga, s);
         if (op == OP_SILU_MUL) return launch<DT, OP_SILU_MUL>(planes, lm, rm, pa, ga, s);
     }
@@ -584,7 +696,7 @@ int dispatch_padded(int op, int lm, int rm, const PaddedArgs& pa, hipStream_t s)
         case OP_COPY: return launch_padded<DT, OP_COPY>(lm, rm, pa, s);
         default: break;
     }
-    if constexpr (DT != IOMX_DT_I32) {
+    if constexpr (is_float_class(DT)) {
         if (op == OP_SILU) return launch_padded<DT, OP_SILU>(lm, rm, pa, s);
         if (op == OP_SILU_MUL) return launch_padded<DT, OP_SILU_MUL>(lm, rm, pa, s);
     }
@@ -656,7 +768,22 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
     // A copy of whole planes is a move of bytes whatever the leaf.  Everything else
     // outside the four streaming leaves goes to the tile-row kernels.
     const bool byte_copy = op == OP_COPY && planes_ok;
-    const bool streaming = streaming_leaf(dtype) || (op == OP_COPY && (bits == 16 || bits == 32));
+    // kernel class: integers by width, floats by leaf; a copy moves raw bits of its width
+    int cls;
+    if (op == OP_COPY) {
+        cls = bits == 8 ? IOMX_DT_I8 : bits == 16 ? IOMX_DT_I16 : bits == 32 ? IOMX_DT_I32
+                : bits == 64 ? IOMX_DT_I64 : -1;
+    } else {
+        switch (dtype) {
+            case IOMX_DT_I8: case IOMX_DT_U8: cls = IOMX_DT_I8; break;
+            case IOMX_DT_I16: case IOMX_DT_U16: cls = IOMX_DT_I16; break;
+            case IOMX_DT_I32: case IOMX_DT_U32: cls = IOMX_DT_I32; break;
+            case IOMX_DT_I64: case IOMX_DT_U64: cls = IOMX_DT_I64; break;
+            case IOMX_DT_F16: case IOMX_DT_BF16: case IOMX_DT_F32: case IOMX_DT_F64: cls = dtype; break;
+            default: cls = -1; break;
+        }
+    }
+    const bool streaming = cls >= 0;
     if (!byte_copy && !streaming) {
         RowsRequest r = {};
         r.src[0] = static_cast<const uint8_t*>(lhs->base);
@@ -708,13 +835,17 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
         pd.tile_rows = (uint32_t)m[2].tile_rows;
         pd.div_tile_rows = make_fast_div(pd.tile_rows);
         const hipStream_t ps = native(stream);
-        int prc;
-        if (op == OP_COPY) {
-            prc = bits == 16 ? dispatch_padded<IOMX_DT_BF16>(op, mode[0], mode[1], pd, ps)
-                             : dispatch_padded<IOMX_DT_I32>(op, mode[0], mode[1], pd, ps);
-        } else if (dtype == IOMX_DT_BF16) prc = dispatch_padded<IOMX_DT_BF16>(op, mode[0], mode[1], pd, ps);
-        else if (dtype == IOMX_DT_F32) prc = dispatch_padded<IOMX_DT_F32>(op, mode[0], mode[1], pd, ps);
-        else prc = dispatch_padded<IOMX_DT_I32>(op, mode[0], mode[1], pd, ps);
+        int prc = IOMX_ERR_UNSUPPORTED;
+        switch (cls) {
+            case IOMX_DT_I8: prc = dispatch_padded<IOMX_DT_I8>(op, mode[0], mode[1], pd, ps); break;
+            case IOMX_DT_I16: prc = dispatch_padded<IOMX_DT_I16>(op, mode[0], mode[1], pd, ps); break;
+            case IOMX_DT_I32: prc = dispatch_padded<IOMX_DT_I32>(op, mode[0], mode[1], pd, ps); break;
+            case IOMX_DT_I64: prc = dispatch_padded<IOMX_DT_I64>(op, mode[0], mode[1], pd, ps); break;
+            case IOMX_DT_F16: prc = dispatch_padded<IOMX_DT_F16>(op, mode[0], mode[1], pd, ps); break;
+            case IOMX_DT_BF16: prc = dispatch_padded<IOMX_DT_BF16>(op, mode[0], mode[1], pd, ps); break;
+            case IOMX_DT_F32: prc = dispatch_padded<IOMX_DT_F32>(op, mode[0], mode[1], pd, ps); break;
+            default: prc = dispatch_padded<IOMX_DT_F64>(op, mode[0], mode[1], pd, ps); break;
+        }
         IOMX_TRY(prc);
         IOMX_HIP(hipGetLastError());
         return IOMX_OK;
@@ -775,13 +906,18 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
 
     const hipStream_t s = native(stream);
     int rc;
-    if (op == OP_COPY) {
-        // raw bits: the 16-bit kernels serve the padded 16-bit case, the 32-bit ones the rest
-        if (!planes_ok && bits == 16) rc = dispatch<IOMX_DT_BF16>(op, planes_ok, mode[0], mode[1], pa, ga, s);
-        else rc = dispatch<IOMX_DT_I32>(op, planes_ok, mode[0], mode[1], pa, ga, s);
-    } else if (dtype == IOMX_DT_BF16) rc = dispatch<IOMX_DT_BF16>(op, planes_ok, mode[0], mode[1], pa, ga, s);
-    else if (dtype == IOMX_DT_F32) rc = dispatch<IOMX_DT_F32>(op, planes_ok, mode[0], mode[1], pa, ga, s);
-    else rc = dispatch<IOMX_DT_I32>(op, planes_ok, mode[0], mode[1], pa, ga, s);
+    // whole planes of any width move as 32-bit words
+    if (byte_copy) cls = IOMX_DT_I32;
+    switch (cls) {
+        case IOMX_DT_I8: rc = dispatch<IOMX_DT_I8>(op, planes_ok, mode[0], mode[1], pa, ga, s); break;
+        case IOMX_DT_I16: rc = dispatch<IOMX_DT_I16>(op, planes_ok, mode[0], mode[1], pa, ga, s); break;
+        case IOMX_DT_I32: rc = dispatch<IOMX_DT_I32>(op, planes_ok, mode[0], mode[1], pa, ga, s); break;
+        case IOMX_DT_I64: rc = dispatch<IOMX_DT_I64>(op, planes_ok, mode[0], mode[1], pa, ga, s); break;
+        case IOMX_DT_F16: rc = dispatch<IOMX_DT_F16>(op, planes_ok, mode[0], mode[1], pa, ga, s); break;
+        case IOMX_DT_BF16: rc = dispatch<IOMX_DT_BF16>(op, planes_ok, mode[0], mode[1], pa, ga, s); break;
+        case IOMX_DT_F32: rc = dispatch<IOMX_DT_F32>(op, planes_ok, mode[0], mode[1], pa, ga, s); break;
+        default: rc = dispatch<IOMX_DT_F64>(op, planes_ok, mode[0], mode[1], pa, ga, s); break;
+    }
     IOMX_TRY(rc);
     IOMX_HIP(hipGetLastError());
     return IOMX_OK;
@@ -799,6 +935,26 @@ bool same_shape(const iomx_view* a, const iomx_view* b) {
 using namespace iomx;
 
 extern "C" {
+
+int iomx_selftest_f16_binary(uint64_t* mismatches, iomx_stream_t stream) {
+    if (!mismatches) return IOMX_ERR_INVALID;
+    unsigned long long* counter = nullptr;
+    IOMX_HIP(hipMalloc(reinterpret_cast<void**>(&counter), sizeof(*counter)));
+    const hipStream_t s = native(stream);
+    int rc = IOMX_OK;
+    hipError_t e = hipMemsetAsync(counter, 0, sizeof(*counter), s);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(f16_binary_selftest_kernel, dim3(8192), dim3(256), 0, s, counter);
+        e = hipGetLastError();
+    }
+    unsigned long long host = 0;
+    if (e == hipSuccess) e = hipMemcpyAsync(&host, counter, sizeof(host), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) rc = (int)e;
+    (void)hipFree(counter);
+    *mismatches = host;
+    return rc;
+}
 
 int iomx_launch_binary(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs,
                        const iomx_view* out, iomx_stream_t stream) {
@@ -818,7 +974,8 @@ int iomx_launch_silu(int dtype, const iomx_view* x, const iomx_view* y, iomx_str
 
 int iomx_launch_silu_mul(int dtype, const iomx_view* gate, const iomx_view* up,
                          const iomx_view* y, iomx_stream_t stream) {
-    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32) return IOMX_ERR_UNSUPPORTED;
+    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32 && dtype != IOMX_DT_F16 && dtype != IOMX_DT_F64)
+        return IOMX_ERR_UNSUPPORTED;
     if (!same_shape(gate, y) || !same_shape(up, y)) return IOMX_ERR_INVALID;
     return run(OP_SILU_MUL, dtype, gate, up, y, ALIAS_EXACT, stream);
 }

@@ -60,7 +60,7 @@ SYMBOLS = [
     "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
     "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul",
     "iomx_launch_copy", "iomx_launch_scatter", "iomx_launch_gather", "iomx_launch_softmax",
-    "iomx_last_launch", "iomx_selftest_bf16_convert",
+    "iomx_last_launch", "iomx_selftest_bf16_convert", "iomx_selftest_f16_binary",
 ]
 
 
@@ -153,6 +153,7 @@ def lib() -> C.CDLL:
         l.iomx_launch_softmax.argtypes = [C.POINTER(SoftmaxDesc), P]
         l.iomx_last_launch.argtypes = [C.POINTER(LaunchInfo)]
         l.iomx_selftest_bf16_convert.argtypes = [C.POINTER(C.c_uint64), P]
+        l.iomx_selftest_f16_binary.argtypes = [C.POINTER(C.c_uint64), P]
         _lib = l
     return _lib
 

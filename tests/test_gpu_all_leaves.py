@@ -20,9 +20,15 @@ from iomo import (ALL_LEAVES, DT_BOOL, DT_F16, DT_F64, DT_F8_E8M0, DT_I16, DT_I6
 
 pytestmark = pytest.mark.gpu
 
-STREAMING = (iomo.DT_I32, iomo.DT_U32, iomo.DT_F32, iomo.DT_BF16)
+STREAMING = (iomo.DT_I32, iomo.DT_U32, iomo.DT_F32, iomo.DT_BF16)          # covered by test_gpu_parity
+# leaves that also run on the chunk-mapped kernels; the rest run on the tile-row kernels
+CHUNKED = STREAMING + (iomo.DT_I8, iomo.DT_U8, DT_I16, DT_U16, DT_I64, DT_U64, DT_F16, DT_F64)
 ROWS_NUMERIC = [d for d in NUMERIC_LEAVES if d not in STREAMING]
 ROWS_FLOAT = [d for d in FLOAT_LEAVES if d not in STREAMING]
+
+
+def on_rows(dtype):
+    return dtype not in CHUNKED
 NARROW = [d for d in ROWS_NUMERIC if LEAF_BITS[d] <= 8]
 names = lambda ds: [LEAF_NAME[d] for d in ds]
 
@@ -97,7 +103,7 @@ def test_copy_between_views(dtype, dims, family):
     if family == "copy_planes":
         assert kernel_name() == "copy_planes"
     else:
-        assert kernel_name() == ("copy_padded" if LEAF_BITS[dtype] in (16, 32) else "rows_copy")
+        assert kernel_name() == ("copy_padded" if LEAF_BITS[dtype] in (8, 16, 32, 64) else "rows_copy")
     assert iomo.copy(src(hs), dst(hd)) == 0
     assert same_storage(dd, hd)
     ds.free()
@@ -115,11 +121,59 @@ def test_binary_every_pair_of_a_narrow_leaf(dtype, op):
     dr, hr = pair(dtype, (1, n), values=every.reshape(1, n))
     do, ho = pair(dtype, (n, n))
     assert iomx.binary(op, dl.view(), dr.view(), do.view()) == 0
-    assert kernel_name() == "rows_binary"
+    assert kernel_name() == ("rows_binary" if on_rows(dtype) else "binary_general")
     assert iomo.binary(op, hl.view(), hr.view(), ho.view()) == 0          # the codec itself
     assert same_storage(do, ho)
     for t in (dl, dr, do):
         t.free()
+
+
+@pytest.mark.parametrize("dtype", [iomo.DT_I8, iomo.DT_U8], ids=["I8", "U8"])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+def test_binary_every_8bit_pair_on_whole_planes(dtype, op):
+    """Both operands materialised as [256,256], so the packed-lane arithmetic of the
+    streaming kernel sees every operand pair."""
+    every = np.arange(256, dtype=np.uint8)
+    a = np.repeat(every.reshape(256, 1), 256, axis=1)
+    b = np.repeat(every.reshape(1, 256), 256, axis=0)
+    dl, hl = pair(dtype, (256, 256), values=a)
+    dr, hr = pair(dtype, (256, 256), values=b)
+    do, ho = pair(dtype, (256, 256))
+    assert iomx.binary(op, dl.view(), dr.view(), do.view()) == 0
+    assert kernel_name() == "binary_planes"
+    assert iomo.binary(op, hl.view(), hr.view(), ho.view()) == 0
+    assert same_storage(do, ho)
+    for t in (dl, dr, do):
+        t.free()
+
+
+@pytest.mark.parametrize("dtype", [DT_I16, DT_U16, DT_F16], ids=["I16", "U16", "F16"])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+def test_binary_16bit_pairs_on_whole_planes(dtype, op):
+    """4 million operand pairs (specials against everything) as whole planes: the packed
+    two-lane integer arithmetic and the hardware F16 conversions, against the codec."""
+    n = 2048
+    spec = half_specials()
+    vals = np.concatenate([spec, datagen.pattern_bits(16, n - spec.size, 141)])
+    other = np.concatenate([datagen.pattern_bits(16, n - spec.size, 142), spec])
+    a = np.repeat(vals.reshape(n, 1), n, axis=1)
+    b = np.repeat(other.reshape(1, n), n, axis=0)
+    dl, hl = pair(dtype, (n, n), values=a)
+    dr, hr = pair(dtype, (n, n), values=b)
+    do, ho = pair(dtype, (n, n))
+    assert iomx.binary(op, dl.view(), dr.view(), do.view()) == 0
+    assert kernel_name() == "binary_planes"
+    assert iomo.binary(op, hl.view(), hr.view(), ho.view(), ieee=True) == 0
+    assert same_storage(do, ho)
+    for t in (dl, dr, do):
+        t.free()
+
+
+def test_f16_streaming_arithmetic_equals_the_codec_rule_for_every_pair():
+    import ctypes as C
+    bad = C.c_uint64(123)
+    iomx.check(iomx.lib().iomx_selftest_f16_binary(C.byref(bad), None))
+    assert bad.value == 0
 
 
 ROWS_CASES = [
@@ -148,7 +202,7 @@ def test_binary_views_and_broadcasts(dtype, case):
     do, ho = pair(dtype, od, salt=0x300 + case)
     rc = iomx.binary(op, apply(dl.view(), ls), apply(dr.view(), rs), apply(do.view(), os_))
     assert rc == 0, iomx.lib().iomx_error_string(rc)
-    assert kernel_name() == "rows_binary"
+    assert kernel_name().startswith("rows_") == on_rows(dtype)
     assert iomo.binary(op, apply(hl.view(), ls), apply(hr.view(), rs), apply(ho.view(), os_),
                        ieee=True) == 0
     assert same_storage(do, ho)
@@ -273,7 +327,7 @@ def test_silu_every_encoding(dtype):
     dx, hx = pair(dtype, dims, values=vals.reshape(dims))
     do, ho = pair(dtype, dims)
     assert iomx.silu(dx.view(), do.view()) == 0
-    assert kernel_name() == "rows_silu"
+    assert kernel_name().startswith("rows_") == on_rows(dtype)
     assert iomo.silu(hx.view(), ho.view()) == 0
     got, want = do.view().to_host().reshape(-1), ho.view().to_logical().reshape(-1)
     nan = is_nan(want, dtype)
