@@ -233,6 +233,21 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// Two F16 values of one word as binary32 and back.  The widening is exact; the
+// narrowing is the hardware's round-to-nearest-even with gradual underflow, and
+// one binary32 operation between them rounds innocuously (24 >= 2*11 + 2), so
+// the pair equals one correctly rounded binary16 operation.  NaN results are
+// made canonical (0x7E00) before the narrowing.
+__device__ __forceinline__ f32x2 f16_pair(uint32_t w) {
+    return __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+}
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+    const f32x2 v = {canonical(lo), canonical(hi)};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return as_f32(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return as_f32(w & 0xFFFF0000u); }
 

@@ -32,7 +32,7 @@ struct RmsArgs {
 
 template <int DT>
 struct RLeaf {
-    static constexpr uint32_t kBytes = (DT == IOMX_DT_BF16) ? 2 : 4;
+    static constexpr uint32_t kBytes = (DT == IOMX_DT_BF16 || DT == IOMX_DT_F16) ? 2 : 4;
     static constexpr uint32_t kPerChunk = 16 / kBytes;
     static constexpr uint32_t kChunksPerRow = kTile / kPerChunk;     // 2 | 4
     static constexpr uint32_t kChunksPerTile = kTileSlots / kPerChunk; // 32 | 64
@@ -43,6 +43,9 @@ __device__ __forceinline__ void unpack(const u32x4& v, float* f) {
     if constexpr (DT == IOMX_DT_BF16) {
         f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
         f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z); f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+    } else if constexpr (DT == IOMX_DT_F16) {
+        const f32x2 a = f16_pair(v.x), b = f16_pair(v.y), c = f16_pair(v.z), d = f16_pair(v.w);
+        f[0] = a.x; f[1] = a.y; f[2] = b.x; f[3] = b.y; f[4] = c.x; f[5] = c.y; f[6] = d.x; f[7] = d.y;
     } else {
         f[0] = as_f32(v.x); f[1] = as_f32(v.y); f[2] = as_f32(v.z); f[3] = as_f32(v.w);
     }
@@ -54,6 +57,9 @@ __device__ __forceinline__ u32x4 pack(const float* f) {
     if constexpr (DT == IOMX_DT_BF16) {
         r.x = pack_bf16(f[0], f[1]); r.y = pack_bf16(f[2], f[3]);
         r.z = pack_bf16(f[4], f[5]); r.w = pack_bf16(f[6], f[7]);
+    } else if constexpr (DT == IOMX_DT_F16) {
+        r.x = pack_f16(f[0], f[1]); r.y = pack_f16(f[2], f[3]);
+        r.z = pack_f16(f[4], f[5]); r.w = pack_f16(f[6], f[7]);
     } else {
         r.x = as_u32(canonical(f[0])); r.y = as_u32(canonical(f[1]));
         r.z = as_u32(canonical(f[2])); r.w = as_u32(canonical(f[3]));
@@ -65,13 +71,13 @@ __device__ __forceinline__ u32x4 pack(const float* f) {
 // the lanes of one wave that share a row.
 template <int DT>
 __device__ __forceinline__ uint32_t lane_row(uint32_t tid) {
-    if constexpr (DT == IOMX_DT_BF16) return (tid & 31u) >> 1;
+    if constexpr (RLeaf<DT>::kBytes == 2) return (tid & 31u) >> 1;
     else return (tid & 63u) >> 2;
 }
 
 template <int DT>
 __device__ __forceinline__ float row_sum_in_wave(float acc) {
-    if constexpr (DT == IOMX_DT_BF16) {
+    if constexpr (RLeaf<DT>::kBytes == 2) {
         acc += __shfl_xor(acc, 1);
         acc += __shfl_xor(acc, 32);
     } else {
@@ -83,7 +89,7 @@ __device__ __forceinline__ float row_sum_in_wave(float acc) {
 
 template <int DT>
 __device__ __forceinline__ bool row_leader(uint32_t tid) {
-    if constexpr (DT == IOMX_DT_BF16) return (tid & 33u) == 0;
+    if constexpr (RLeaf<DT>::kBytes == 2) return (tid & 33u) == 0;
     else return (tid & 3u) == 0;
 }
 
@@ -347,12 +353,12 @@ void launch_split(const RmsArgs& a, hipStream_t s) {
 // 256 bytes or more per tile), and sixteen parts (32-byte runs) lose even to the
 // two-pass kernel, so the split stops at eight.
 template <int DT>
-constexpr uint32_t kResidentChunks = (DT == IOMX_DT_BF16 ? 8u : 16u) * 1024u;
+constexpr uint32_t kResidentChunks = (RLeaf<DT>::kBytes == 2 ? 8u : 16u) * 1024u;
 
 template <int DT>
 int launch(const RmsArgs& a, bool band_ok, hipStream_t s) {
     const uint32_t n = a.band_chunks;
-    constexpr int KS = DT == IOMX_DT_BF16 ? 8 : 16;
+    constexpr int KS = RLeaf<DT>::kBytes == 2 ? 8 : 16;
     if (band_ok && n > kResidentChunks<DT> && n <= 8 * kResidentChunks<DT>
         && (uint64_t)a.total_bands * 8 <= 0x7FFFFFFFull) {
         if (n <= 2 * kResidentChunks<DT>) launch_split<DT, KS, 2>(a, s);
@@ -397,7 +403,7 @@ extern "C" int iomx_launch_rmsnorm(int dtype, const iomx_view* x, const iomx_vie
     if (scale->rank != 2 || scale->dims[0] != 1 || scale->dims[1] != m.cols) return IOMX_ERR_INVALID;
     if (out->base == x->base || out->base == scale->base) return IOMX_ERR_INVALID;
     if (!(eps >= 0.0f) || eps > 3.4028234e38f) return IOMX_ERR_INVALID;
-    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32) {
+    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32 && dtype != IOMX_DT_F16) {
         // the other floating leaves: one workgroup per row on packed tile rows
         RowsRmsnormRequest r = {};
         uint64_t rstrides[2][kMaxLead] = {};
@@ -457,6 +463,7 @@ extern "C" int iomx_launch_rmsnorm(int dtype, const iomx_view* x, const iomx_vie
     const bool band_ok = m.cols % kTile == 0;
     const hipStream_t s = native(stream);
     if (dtype == IOMX_DT_BF16) IOMX_TRY(launch<IOMX_DT_BF16>(a, band_ok, s));
+    else if (dtype == IOMX_DT_F16) IOMX_TRY(launch<IOMX_DT_F16>(a, band_ok, s));
     else IOMX_TRY(launch<IOMX_DT_F32>(a, band_ok, s));
     IOMX_HIP(hipGetLastError());
     return IOMX_OK;

@@ -359,7 +359,7 @@ def finite_values(dtype, count, salt):
 
 @pytest.mark.parametrize("dtype", ROWS_FLOAT, ids=names(ROWS_FLOAT))
 @pytest.mark.parametrize("dims,steps", [((2, 5, 40), []), ((3, 17, 33), []), ((4, 16, 4112), [("slice", (0, 0, 2, 2))]),
-                                        ((1, 1), [])])
+                                        ((1, 1), []), ((40, 2048), []), ((2, 33, 256), [])])
 def test_rmsnorm_float_leaves(dtype, dims, steps):
     F = dims[-1]
     dx, hx = pair(dtype, dims, values=finite_values(dtype, int(np.prod(dims)), 81).reshape(dims))
@@ -367,7 +367,7 @@ def test_rmsnorm_float_leaves(dtype, dims, steps):
     do, ho = pair(dtype, dims, salt=83)
     rc = iomx.rmsnorm(apply(dx.view(), steps), dw.view(), apply(do.view(), steps), 1e-5)
     assert rc == 0, iomx.lib().iomx_error_string(rc)
-    assert kernel_name() == "rows_rmsnorm"
+    assert (kernel_name() == "rows_rmsnorm") == (dtype != DT_F16)
     assert iomo.rmsnorm(apply(hx.view(), steps), hw.view(), apply(ho.view(), steps), 1e-5) == 0
     got, want = do.view().to_host().reshape(-1), ho.view().to_logical().reshape(-1)
     nan = is_nan(want, dtype)
