@@ -122,14 +122,14 @@ template <int DT, typename T>
 __device__ __forceinline__ T rope_decode(uint64_t raw) {
     if constexpr (DT == DT_BF16) return (T)as_f32((uint32_t)raw << 16);
     else if constexpr (DT == DT_F32) return (T)as_f32((uint32_t)raw);
-    else return (T)decode<DT>(raw);
+    else return decode_as<DT, T>(raw);
 }
 
 template <int DT, typename T>
 __device__ __forceinline__ uint64_t rope_encode(T v) {
     if constexpr (DT == DT_BF16) return bf16_rne_sw(as_u32((float)v));
     else if constexpr (DT == DT_F32) return as_u32(canonical((float)v));
-    else return encode<DT>((double)v);
+    else return encode_from<DT, T>(v);
 }
 
 __device__ __forceinline__ void rope_angle(uint32_t column, uint32_t width, uint32_t position,

@@ -141,7 +141,7 @@ __global__ __launch_bounds__(256) void rows_rmsnorm_kernel(const RowsRmsArgs a) 
 #pragma unroll
             for (int i = 0; i < (int)kTile; ++i) {
                 if ((uint32_t)i < left) {
-                    const T v = (T)decode<DT>(get<BITS>(w, i));
+                    const T v = decode_as<DT, T>(get<BITS>(w, i));
                     acc = acc + v * v;
                 }
             }
@@ -162,11 +162,11 @@ __global__ __launch_bounds__(256) void rows_rmsnorm_kernel(const RowsRmsArgs a) 
             for (int j = 0; j < K; ++j) res[j] = 0;
 #pragma unroll
             for (int i = 0; i < (int)kTile; ++i) {
-                const T v = (T)decode<DT>(get<BITS>(w, i));
-                const T g = (T)decode<DT>(get<BITS>(s, i));
+                const T v = decode_as<DT, T>(get<BITS>(w, i));
+                const T g = decode_as<DT, T>(get<BITS>(s, i));
                 const T normalized = v * inverse;
                 const T y = normalized * g;
-                put<BITS>(res, i, encode<DT>((double)y));
+                put<BITS>(res, i, encode_from<DT, T>(y));
             }
             const uint32_t left = a.feats - tc * kTile;
             store_row<BITS>(orow + (uint64_t)tc * kTileBytes, res, left < kTile ? left : kTile);

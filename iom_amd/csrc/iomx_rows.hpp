@@ -236,6 +236,62 @@ IOMX_HD uint64_t encode(double r) {
     }
 }
 
+// The same two steps in binary32, for the leaves of at most 8 bits.  Their values are
+// exact in binary32; a product of two is exact (at most 8 significand bits), and a
+// sum or difference is exact or rounded with so many guard bits (24 >= 2*4 + 2)
+// that the rounding below still equals one rounding of the exact result.  The
+// binary32 path equals the binary64 one for every operand pair (checked
+// exhaustively on the host and on the device).
+IOMX_HD float as_f32_hd(uint32_t b) { return __builtin_bit_cast(float, b); }
+IOMX_HD uint32_t as_u32_hd(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+template <int DT>
+IOMX_HD float decode_f32(uint32_t raw) {
+    constexpr Fmt f = fmt_of(DT);
+    constexpr uint32_t emask = (1u << f.ebits) - 1u, fmask = (1u << f.fbits) - 1u;
+    const uint32_t frac = raw & fmask, exp = (raw >> f.fbits) & emask;
+    float v;
+    if (top_special(f) && exp == emask) {
+        v = (f.infs && frac == 0) ? __builtin_inff() : __builtin_nanf("");
+    } else {
+        const int m = exp ? (int)((1u << f.fbits) + frac) : (int)frac;
+        const int scale = (int)(exp ? exp : 1u) - f.bias - f.fbits;
+        v = ldexpf((float)m, scale);
+    }
+    return ((raw >> (f.ebits + f.fbits)) & 1u) ? -v : v;
+}
+
+template <int DT>
+IOMX_HD uint32_t encode_f32(float r) {
+    constexpr Fmt f = fmt_of(DT);
+    constexpr uint32_t emask = (1u << f.ebits) - 1u, fmask = (1u << f.fbits) - 1u;
+    constexpr int shift = f.ebits + f.fbits;
+    constexpr uint32_t finite_emax = top_special(f) ? emask - 1u : emask;
+    constexpr uint32_t over = f.infs ? (emask << f.fbits) : ((finite_emax << f.fbits) | fmask);
+    constexpr uint32_t nan = !top_special(f) ? over
+            : (emask << f.fbits) | (f.finite_only ? fmask : 1u << (f.fbits - 1));
+    const uint32_t b = as_u32_hd(r);
+    const uint32_t sign = (b >> 31) << shift;
+    const uint32_t mag = b & 0x7FFFFFFFu;
+    if (mag > 0x7F800000u) return nan;
+    if (mag == 0x7F800000u) return sign | over;
+    if (mag < 0x00800000u) return sign;   // zero, or below 2^-126: far under half the smallest step
+    const int e = (int)(mag >> 23) - 127;
+    const uint32_t m = (mag & 0x7FFFFFu) | 0x800000u;
+    constexpr int emin = 1 - f.bias;
+    const int drop = 23 - f.fbits + (e < emin ? emin - e : 0);
+    uint32_t q = 0, rest = 1, half = 2;
+    if (drop <= 30) {
+        q = m >> drop;
+        rest = m & ((1u << drop) - 1u);
+        half = 1u << (drop - 1);
+    }
+    if (rest > half || (rest == half && (q & 1u))) ++q;
+    const uint32_t field = e < emin ? q : ((uint32_t)(e + f.bias - 1) << f.fbits) + q;
+    if ((field >> f.fbits) > finite_emax) return sign | over;
+    return sign | field;
+}
+
 template <int DT, int OP>
 IOMX_HD uint64_t leaf_binary(uint64_t a, uint64_t b) {
     constexpr int BITS = bits_of(DT);
@@ -251,6 +307,11 @@ IOMX_HD uint64_t leaf_binary(uint64_t a, uint64_t b) {
         // IEEE arithmetic supplies the special cases of the reference rule: opposite
         // infinities and infinity times zero give NaN, an exact zero sum is +0 unless
         // both operands are -0, NaN operands give NaN.
+        if constexpr (BITS <= 8) {
+            const float x = decode_f32<DT>((uint32_t)a), y = decode_f32<DT>((uint32_t)b);
+            const float r = OP == IOMX_OP_ADD ? x + y : (OP == IOMX_OP_MUL ? x * y : x - y);
+            return encode_f32<DT>(r);
+        }
         const double x = decode<DT>(a), y = decode<DT>(b);
         const double r = OP == IOMX_OP_ADD ? x + y : (OP == IOMX_OP_MUL ? x * y : x - y);
         return encode<DT>(r);
@@ -282,7 +343,20 @@ IOMX_HD double silu_carrier(double x) {
 template <int DT>
 IOMX_HD uint64_t leaf_silu(uint64_t a) {
     if constexpr (DT == DT_F64) return encode<DT>(silu_carrier(decode<DT>(a)));
+    else if constexpr (bits_of(DT) <= 8) return encode_f32<DT>(silu_carrier(decode_f32<DT>((uint32_t)a)));
     else return encode<DT>((double)silu_carrier((float)decode<DT>(a)));
+}
+
+// A leaf value in the carrier T (float or double) and back, by the cheaper route.
+template <int DT, typename T>
+IOMX_HD T decode_as(uint64_t raw) {
+    if constexpr (bits_of(DT) <= 8) return (T)decode_f32<DT>((uint32_t)raw);
+    else return (T)decode<DT>(raw);
+}
+template <int DT, typename T>
+IOMX_HD uint64_t encode_from(T v) {
+    if constexpr (bits_of(DT) <= 8) return encode_f32<DT>((float)v);
+    else return encode<DT>((double)v);
 }
 
 #if defined(__HIPCC__)
