@@ -868,6 +868,84 @@ int iomo_rope(int dtype, const iomo_view* x, const iomo_view* out, uint64_t a, d
 }
 
 /* ------------------------------------------------------------------ */
+/* Linear projection (src/cpu/queue.cpp:1905-2051)                      */
+/* ------------------------------------------------------------------ */
+
+/* out[b,r,o] = sum_i x[b,s+r,i] * w[o,i] (ordinary, H = 1, D = O) or
+ * out[b,h,r,d] = sum_i x[b,s+r,i] * w[h*D+d,i] (head planar, O = H*D): integers
+ * modulo 2^N; floating leaves start at +0 and take one correctly rounded fused
+ * multiply-add per increasing i in binary32 (binary64 for F64), encoded once.
+ * Admission of docs/BACKEND_CONTRACT/linear-projections.md:86-112 as far as it can
+ * be checked without owner identities. */
+int iomo_linear(int dtype, const iomo_view* x, const iomo_view* w, const iomo_view* out,
+                uint64_t s, uint64_t R, int head_planar, uint64_t H, uint64_t D) {
+    const unsigned bits = iomo_leaf_bits(dtype);
+    fmt_t f;
+    if (!view_ok(x) || !view_ok(w) || !view_ok(out)) return IOMO_ERR_INVALID;
+    if (w->rank != 2) return IOMO_ERR_INVALID;
+    const uint64_t T = view_rows(x), I = view_cols(x), O = w->dims[0];
+    if (w->dims[1] != I) return IOMO_ERR_INVALID;
+    if (R == 0 || s > T || R > T - s) return IOMO_ERR_INVALID;
+    if (head_planar) {
+        if (H == 0 || D == 0 || H * D != O) return IOMO_ERR_INVALID;
+        if (out->rank != x->rank + 1 || out->rank > 8) return IOMO_ERR_INVALID;
+    } else {
+        if (H != 1 || D != O) return IOMO_ERR_INVALID;
+        if (out->rank != x->rank) return IOMO_ERR_INVALID;
+    }
+    const uint32_t leading = x->rank - 2;
+    for (uint32_t i = 0; i < leading; ++i)
+        if (x->dims[i] != out->dims[i]) return IOMO_ERR_INVALID;
+    if (head_planar && out->dims[leading] != H) return IOMO_ERR_INVALID;
+    if (view_rows(out) != R || view_cols(out) != D) return IOMO_ERR_INVALID;
+    if (out->base == x->base || out->base == w->base) return IOMO_ERR_INVALID;
+    const unsigned width = integer_width(dtype);
+    if (!bits || (!width && !float_format(dtype, &f))) return IOMO_ERR_UNSUPPORTED;
+    const uint64_t mask = width == 64 ? ~0ull : (1ull << width) - 1;
+    const uint64_t heads = head_planar ? H : 1;
+    const uint64_t head_stride = head_planar ? out->plane_strides[leading] : 0;
+    uint64_t coord[8] = {0};
+    do {
+        uint64_t xp = x->plane_offset, op = out->plane_offset;
+        for (uint32_t a = 0; a < leading; ++a) {
+            xp += coord[a] * x->plane_strides[a];
+            op += coord[a] * out->plane_strides[a];
+        }
+        for (uint64_t r = 0; r < R; ++r)
+        for (uint64_t h = 0; h < heads; ++h)
+        for (uint64_t d = 0; d < D; ++d) {
+            const uint64_t o = h * D + d;
+            uint64_t raw;
+            if (width) {
+                uint64_t acc = 0;
+                for (uint64_t i = 0; i < I; ++i) {
+                    const uint64_t a = load_leaf(x->base, iomo_plane_slot(T, I, xp, s + r, i), bits) & mask;
+                    const uint64_t b = load_leaf(w->base, iomo_plane_slot(O, I, w->plane_offset, o, i), bits) & mask;
+                    acc = (acc + a * b) & mask;
+                }
+                raw = acc;
+            } else if (dtype == IOMO_DT_F64) {
+                double acc = 0.0;
+                for (uint64_t i = 0; i < I; ++i)
+                    acc = fma((double)codec_decode(load_leaf(x->base, iomo_plane_slot(T, I, xp, s + r, i), bits), f),
+                              (double)codec_decode(load_leaf(w->base, iomo_plane_slot(O, I, w->plane_offset, o, i), bits), f),
+                              acc);
+                raw = codec_encode(acc != acc ? positive_nan() : (long double)acc, f);
+            } else {
+                float acc = 0.0f;
+                for (uint64_t i = 0; i < I; ++i)
+                    acc = fmaf((float)codec_decode(load_leaf(x->base, iomo_plane_slot(T, I, xp, s + r, i), bits), f),
+                               (float)codec_decode(load_leaf(w->base, iomo_plane_slot(O, I, w->plane_offset, o, i), bits), f),
+                               acc);
+                raw = codec_encode(acc != acc ? positive_nan() : (long double)acc, f);
+            }
+            store_leaf(out->base, iomo_plane_slot(R, D, op + h * head_stride, r, d), bits, raw);
+        }
+    } while (next_coord(coord, x->dims, leading));
+    return IOMO_OK;
+}
+
+/* ------------------------------------------------------------------ */
 /* Softmax stage (src/cpu/sdpa.cpp:214-309)                             */
 /* ------------------------------------------------------------------ */
 

@@ -128,6 +128,14 @@ int iomo_embedding(int dtype, int index_dtype, const iomo_view* table,
  * src/device_ops_neural.cpp:241-362). */
 int iomo_rope(int dtype, const iomo_view* x, const iomo_view* out, uint64_t a, double theta);
 
+/* Linear projection out[b,r,o] = sum_i x[b,s+r,i] * w[o,i] and its head-planar
+ * form (src/cpu/queue.cpp:1905-2051, docs/BACKEND_CONTRACT/linear-projections.md):
+ * one fused multiply-add per increasing i in binary32 (binary64 for F64), integers
+ * modulo 2^N, one encode.  NaN results are stored positive (NaN signs are outside
+ * the contract). */
+int iomo_linear(int dtype, const iomo_view* x, const iomo_view* w, const iomo_view* out,
+                uint64_t s, uint64_t R, int head_planar, uint64_t H, uint64_t D);
+
 /*
  * Softmax stage.  Request shape follows src/rocm/sdpa_softmax.hpp:14-62
  * (strides in elements); arithmetic follows src/cpu/sdpa.cpp:214-309 with

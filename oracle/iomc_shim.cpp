@@ -343,6 +343,17 @@ std::int64_t iomc_sdpa(
     }
 }
 
+// out[b,r,o] = sum_i x[b,s+r,i] * w[o,i], ordinary or head planar
+// (docs/BACKEND_CONTRACT/linear-projections.md:20-31).
+std::int64_t iomc_linear(
+        iomc_queue* queue, const iomc_view* x, const iomc_view* w, iomc_view* out, std::size_t s,
+        std::size_t R, int head_planar, std::size_t H, std::size_t D) {
+    return queue->ops->linear(
+            x->view, w->view, out->view, s, R,
+            head_planar ? iom::LinearOutputLayout::head_planar : iom::LinearOutputLayout::ordinary,
+            H, D);
+}
+
 // destination[..., h, a + r, d] = source[..., h, r, d] (include/iom/iom.hpp:171-182).
 std::int64_t iomc_cache_append(
         iomc_queue* queue, const iomc_view* source, iomc_view* destination, std::size_t a) {

@@ -135,6 +135,7 @@ def lib() -> C.CDLL:
         l.iomo_cache_append.argtypes = [C.c_int, VP, VP, C.c_uint64]
         l.iomo_embedding.argtypes = [C.c_int, C.c_int, VP, VP, VP]
         l.iomo_rope.argtypes = [C.c_int, VP, VP, C.c_uint64, C.c_double]
+        l.iomo_linear.argtypes = [C.c_int, VP, VP, VP, C.c_uint64, C.c_uint64, C.c_int, C.c_uint64, C.c_uint64]
         _lib = l
     return _lib
 
@@ -338,6 +339,11 @@ def rope(x: HostView, out: HostView, a: int, theta: float) -> int:
     return lib().iomo_rope(out.dtype, C.byref(s), C.byref(o), a, theta)
 
 
+def linear(x: HostView, w: HostView, out: HostView, s: int, R: int, head_planar: bool, H: int, D: int) -> int:
+    a, b, o = x.cview(), w.cview(), out.cview()
+    return lib().iomo_linear(out.dtype, C.byref(a), C.byref(b), C.byref(o), s, R, int(head_planar), H, D)
+
+
 def dense_layout(heads: int, rows: int, cols: int) -> StageLayout:
     l = StageLayout()
     l.plane_offset = 0
@@ -445,6 +451,8 @@ def bind_iomc(l: C.CDLL) -> C.CDLL:
     l.iomc_sdpa.restype = C.c_int64
     l.iomc_sdpa.argtypes = [P, P, P, P, P, P, C.c_size_t, C.c_size_t]
     l.iomc_wait.argtypes = [P, C.c_int64]
+    l.iomc_linear.restype = C.c_int64
+    l.iomc_linear.argtypes = [P, P, P, P, C.c_size_t, C.c_size_t, C.c_int, C.c_size_t, C.c_size_t]
     l.iomc_cache_append.restype = C.c_int64
     l.iomc_cache_append.argtypes = [P, P, P, C.c_size_t]
     l.iomc_rope.restype = C.c_int64
@@ -594,6 +602,9 @@ class IomBackend:
 
     def silu(self, x, y) -> int:
         return self.run(self.l.iomc_silu(self.queue, x.h, y.h))
+
+    def linear(self, x, w, out, s, R, head_planar, H, D) -> int:
+        return self.run(self.l.iomc_linear(self.queue, x.h, w.h, out.h, s, R, int(head_planar), H, D))
 
     def cache_append(self, src, dst, a) -> int:
         return self.run(self.l.iomc_cache_append(self.queue, src.h, dst.h, a))
