@@ -236,6 +236,23 @@ int iomx_launch_embedding(int dtype, int index_dtype, const iomx_view* table,
 int iomx_launch_rope(int dtype, const iomx_view* x, const iomx_view* out, uint64_t a, double theta,
                      iomx_stream_t stream);
 
+/*
+ * out[b,r,o] = sum_i x[b,s+r,i] * w[o,i] (ordinary: H = 1, D = O, out [...,R,O]) or
+ * out[b,h,r,d] = sum_i x[b,s+r,i] * w[h*D+d,i] (head planar: O = H*D, out
+ * [...,H,R,D]); w is rank two in the [out,in] orientation and is never transposed.
+ * Replaces the linear kernels of the standard tiled backends behind
+ * DeviceOps::linear_impl; contract docs/BACKEND_CONTRACT/linear-projections.md,
+ * arithmetic of src/cpu/queue.cpp:1905-2003: integers modulo 2^N; floating leaves
+ * one fused multiply-add per increasing i in F32 (F64 for F64) from +0 and one
+ * encode.  path 0 lets BF16 run on the matrix cores (exact products, F32
+ * accumulation in the hardware's order, one round-to-nearest-even store: the
+ * "native BF16" allowance of linear-projections.md:213-218); path 1 forces the
+ * scalar recurrence for every leaf.
+ */
+int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const iomx_view* out,
+                       uint64_t s, uint64_t R, int head_planar, uint64_t H, uint64_t D, int path,
+                       iomx_stream_t stream);
+
 /* Element strides of one softmax-stage buffer (src/rocm/sdpa_softmax.hpp:14-22). */
 typedef struct iomx_stage_layout {
     uint64_t plane_offset, plane_stride, head_stride, row_stride, column_stride;

@@ -26,6 +26,7 @@ SOURCES = [
     "iomx_transfer.hip",
     "iomx_leaves.hip",
     "iomx_layer.hip",
+    "iomx_linear.hip",
 ]
 
 # -ffp-contract=off: no fused multiply-add may replace the reference's two

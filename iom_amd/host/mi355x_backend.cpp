@@ -613,6 +613,56 @@ private:
                 });
     }
 
+    // ---- linear projection --------------------------------------------------------
+
+    [[nodiscard]] WorkspaceRequirements linear_workspace_requirements_impl(
+            const TensorView& x, const TensorView&, const TensorView&, std::size_t, std::size_t,
+            LinearOutputLayout, std::size_t, std::size_t) override {
+        if (binary_code(x.spec().data_type) < 0) throw detail::UnsupportedOperation();
+        return {0, 1};
+    }
+
+    oid linear_impl(const LinearRequest& request) override {
+        const int code = binary_code(request.x.spec.data_type);
+        if (code < 0) throw detail::UnsupportedOperation();
+        if (!request.workspace.empty())
+            throw std::invalid_argument("MI355X linear projection consumes no raw workspace");
+        std::lock_guard<std::mutex> order(submission_mutex_);
+        return submit_linear(
+                request, device_.registry_state(), registry_queue_id_, pending_fence(),
+                [this, code](std::uint64_t sequence, const LinearRequest& captured,
+                             detail::BinaryEntryRegistration entries) {
+                    auto& state = device_.registry_state();
+                    const detail::WorkspaceLease lease = captured.workspace_lease;
+                    try {
+                        start(sequence,
+                              [&captured, code](iomx_stream_t stream) {
+                                  const auto view_of = [](const LinearViewSnapshot& s) {
+                                      return make_view(s.native_handle, s.spec.shape.dimensions(),
+                                                       s.plane_offset, s.plane_strides);
+                                  };
+                                  const iomx_view x = view_of(captured.x);
+                                  const iomx_view w = view_of(captured.w);
+                                  const iomx_view out = view_of(captured.out);
+                                  const bool planar = captured.layout == LinearOutputLayout::head_planar;
+                                  return iomx_launch_linear(code, &x, &w, &out, captured.start_row,
+                                                            captured.rows, planar ? 1 : 0, captured.heads,
+                                                            captured.head_dim, 0, stream);
+                              },
+                              [&state, entries, lease](bool failed) {
+                                  (void)detail::release_or_invalidate_binary_entries(
+                                          state.registry, entries, failed, true);
+                                  detail::complete_workspace_lease(state, lease, true);
+                              });
+                    } catch (...) {
+                        state.registry.remove_entries(std::span<const detail::EntryId>(
+                                entries.entries.data(), entries.count));
+                        detail::complete_workspace_lease(state, lease, true);
+                        throw;
+                    }
+                });
+    }
+
     // ---- cache append / embedding / rope ----------------------------------------
 
     template <typename Snapshot>

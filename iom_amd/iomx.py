@@ -57,7 +57,7 @@ SYMBOLS = [
     "iomx_memcpy_d2d_async", "iomx_stream_create", "iomx_stream_destroy",
     "iomx_stream_synchronize", "iomx_event_create", "iomx_event_destroy", "iomx_event_record",
     "iomx_event_synchronize", "iomx_event_query", "iomx_event_elapsed_ms",
-    "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
+    "iomx_launch_linear", "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
     "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul",
     "iomx_launch_copy", "iomx_launch_scatter", "iomx_launch_gather", "iomx_launch_softmax",
     "iomx_last_launch", "iomx_selftest_bf16_convert", "iomx_selftest_f16_binary",
@@ -146,6 +146,8 @@ def lib() -> C.CDLL:
         l.iomx_launch_silu_mul.argtypes = [C.c_int, VP, VP, VP, P]
         l.iomx_launch_copy.argtypes = [C.c_int, VP, VP, P]
         l.iomx_launch_cache_append.argtypes = [C.c_int, VP, VP, C.c_uint64, P]
+        l.iomx_launch_linear.argtypes = [C.c_int, VP, VP, VP, C.c_uint64, C.c_uint64, C.c_int, C.c_uint64,
+                                         C.c_uint64, C.c_int, P]
         l.iomx_launch_embedding.argtypes = [C.c_int, C.c_int, VP, VP, VP, P, P]
         l.iomx_launch_rope.argtypes = [C.c_int, VP, VP, C.c_uint64, C.c_double, P]
         l.iomx_launch_scatter.argtypes = [C.c_int, VP, P, P]
@@ -425,6 +427,13 @@ def silu_mul(gate: DeviceView, up: DeviceView, y: DeviceView, stream=None) -> in
 def copy(src: DeviceView, dst: DeviceView, stream=None) -> int:
     a, o = src.cview(), dst.cview()
     return lib().iomx_launch_copy(dst.dtype, C.byref(a), C.byref(o), _h(stream))
+
+
+def linear(x: DeviceView, w: DeviceView, out: DeviceView, s: int, R: int, head_planar: bool, H: int, D: int,
+           path: int = 0, stream: Optional[Stream] = None) -> int:
+    a, b, o = x.cview(), w.cview(), out.cview()
+    return lib().iomx_launch_linear(out.dtype, C.byref(a), C.byref(b), C.byref(o), s, R, int(head_planar),
+                                    H, D, path, _h(stream))
 
 
 def cache_append(src: DeviceView, dst: DeviceView, a: int, stream: Optional[Stream] = None) -> int:
