@@ -327,6 +327,45 @@ def wl_other_leaves(timer, steps, warmup):
     return out
 
 
+def wl_linear(timer, steps, warmup):
+    """BF16 projections of a TinyLlama-sized layer on the matrix cores: prefill
+    ([64,512,2048] rows) and decode (one row per sequence)."""
+    out = []
+    B, S, I = 64, 512, 2048
+    x = device_tensor(BF16, (B, S, I), "normal", 101)
+    for O, name in ((2048, "o_proj"), (5632, "gate_proj")):
+        w = device_tensor(BF16, (O, I), "normal_0p02", 102)
+        o = device_tensor(BF16, (B, S, O))
+
+        def launch(i):
+            check(iomx.linear(x.view(), w.view(), o.view(), 0, S, False, 1, O, 0, timer.stream), "linear")
+
+        wall, ev = timer.run(launch, steps, warmup)
+        flops = 2.0 * B * S * I * O
+        r = report("linear_bf16_%s_[64,512,2048]x[%d,2048]" % (name, O), 2 * (B * S * I + O * I + B * S * O),
+                   B * S * O, wall, ev, iomx.last_launch().kernel.decode())
+        r["TFLOP_per_s"] = round(flops / (ev * 1e-3) / 1e12, 1)
+        r["mfma_frac_of_2500"] = round(r["TFLOP_per_s"] / 2500.0, 4)
+        out.append(r)
+        w.free()
+        o.free()
+    # decode: the last row of every sequence through the 5632-wide projection
+    w = device_tensor(BF16, (5632, I), "normal_0p02", 103)
+    o = device_tensor(BF16, (B, 1, 5632))
+
+    def decode(i):
+        check(iomx.linear(x.view(), w.view(), o.view(), S - 1, 1, False, 1, 5632, 0, timer.stream), "linear")
+
+    wall, ev = timer.run(decode, steps, warmup)
+    r = report("linear_bf16_decode_[64,1,2048]x[5632,2048]", 2 * (B * I + 5632 * I + B * 5632), B * 5632, wall, ev,
+               iomx.last_launch().kernel.decode())
+    r["TFLOP_per_s"] = round(2.0 * B * I * 5632 / (ev * 1e-3) / 1e12, 2)
+    out.append(r)
+    for t in (x, w, o):
+        t.free()
+    return out
+
+
 def wl_softmax(timer, steps, warmup, planes, heads, rows, cols, causal_position):
     """F32 scores [planes,heads,rows,cols] with the strict upper triangle = -inf as data.
     causal_position=False: a = cols-1, every token is positionally visible (the mask
@@ -501,6 +540,7 @@ def main():
         "softmax_causal": lambda: wl_softmax(timer, max(K // 20, 3), 2, 32, 32, 2048, 2048, True),
         "chain": lambda: wl_chain(timer, max(K // 10, 5), max(W // 10, 2)),
         "layer_ops": lambda: wl_layer_ops(timer, max(K // 4, 5), max(W // 4, 2)),
+        "linear": lambda: wl_linear(timer, max(K // 20, 5), 2),
         "other_leaves": lambda: wl_other_leaves(timer, max(K // 10, 5), max(W // 10, 2)),
     }
 
