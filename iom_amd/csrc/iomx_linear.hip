@@ -6,14 +6,15 @@
 //                    increasing i in binary32 (binary64 for F64) from +0, one
 //                    encode.  A lane owns one output tile row (16 outputs of one
 //                    row) and walks the inner axis tile by tile.
-//   linear_mfma      BF16 on the matrix cores (v_mfma_f32_16x16x16_bf16): products
+//   linear_mfma      BF16 on the matrix cores (v_mfma_f32_16x16x32_bf16): products
 //                    exact, binary32 accumulation, one round-to-nearest-even
-//                    store.  A 16x16 tile of either operand is one MFMA operand as
-//                    it lies in memory: lane l reads four consecutive inner
-//                    elements of tile row l%16, so no staging or transposition is
-//                    needed; the weight tile is the A operand so that a lane ends
-//                    up with four consecutive outputs of one row.
+//                    store.  Two neighbouring 16x16 tiles of either operand are one
+//                    MFMA operand as they lie in memory: lane l reads eight
+//                    consecutive inner elements (16 bytes) of tile row l%16, so no
+//                    transposition is needed; the weight tile is the A operand so
+//                    that a lane ends up with four consecutive outputs of one row.
 #include "iomx_rows.hpp"
+#include <cstdlib>
 
 namespace iomx {
 
@@ -150,99 +151,279 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(const LinearArgs a) {
 // BF16 on the matrix cores
 // ---------------------------------------------------------------------------
 
-typedef short bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-// Four consecutive BF16 of one tile row, columns c0..c0+3 of inner tile ti, zero
-// where the inner index is past I (tile padding is never an operand).
-__device__ __forceinline__ bf16x4_t load_k4(const uint8_t* tile_row, uint32_t c0, uint32_t i0, uint32_t I) {
-    bf16x4_t v = {0, 0, 0, 0};
-    if (i0 + 4 <= I) {
-        v = *reinterpret_cast<const bf16x4_t*>(tile_row + c0 * 2);
-    } else {
+// Eight consecutive BF16 of one tile row starting at column c0 (0 or 8), inner
+// indices i0..i0+7, zero where the inner index is past I (tile padding is never
+// an operand).
+__device__ __forceinline__ bf16x8_t load_k8(const uint8_t* tile_row, uint32_t c0, uint32_t i0, uint32_t I) {
+    u32x4 v = {0, 0, 0, 0};
+    if (i0 + 8 <= I) {
+        v = *reinterpret_cast<const u32x4*>(tile_row + c0 * 2);
+    } else if (i0 < I) {
+        uint32_t h[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (i0 + j < I) v[j] = *reinterpret_cast<const short*>(tile_row + (c0 + j) * 2);
+        for (int j = 0; j < 8; ++j)
+            h[j] = (i0 + j < I) ? *reinterpret_cast<const uint16_t*>(tile_row + (c0 + j) * 2) : 0u;
+        v = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
     }
-    return v;
+    return __builtin_bit_cast(bf16x8_t, v);
 }
 
-// One wave = MT row tiles x NT output tiles; a workgroup = 2 x 2 waves.
+// The rows of every plane form one row axis (row index = plane * R + r), so a
+// decode step of many sequences fills whole row tiles and reads the weight once.
+// One wave = MT row tiles x NT output tiles, one v_mfma_f32_16x16x32_bf16 per pair
+// and per 32 inner elements (two inner tiles); a workgroup = 2 x 2 waves.
 template <int MT, int NT>
 __global__ __launch_bounds__(256) void linear_mfma_bf16_kernel(const LinearArgs a) {
     constexpr uint32_t kTileBytes = 512, kRowBytes = 32;
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const uint32_t l16 = lane & 15u, kg = lane >> 4;          // tile row, inner group of four
-    const uint32_t rt0 = (blockIdx.x * 2 + (wave & 1u)) * MT;  // first row tile of this wave
-    const uint32_t ot0 = (blockIdx.y * 2 + (wave >> 1)) * NT;  // first output tile (over O = H*D)
+    const uint32_t l16 = lane & 15u, kg = lane >> 4;          // tile row, group of eight inner elements
+    const uint32_t total_rows = a.planes * a.R;
+    const uint32_t row_tiles = (total_rows + kTile - 1) / kTile;
     const uint32_t o_tiles = (a.O + kTile - 1) / kTile;
-    if (rt0 >= a.row_tiles || ot0 >= o_tiles) return;
-    for (uint32_t p = blockIdx.z; p < a.planes; p += gridDim.z) {
+    const uint32_t rt0 = (blockIdx.x * 2 + (wave & 1u)) * MT;
+    const uint32_t ot0 = (blockIdx.y * 2 + (wave >> 1)) * NT;
+    if (rt0 >= row_tiles || ot0 >= o_tiles) return;
+    // per-lane operand rows
+    const uint8_t* xrow[MT];
+    uint8_t* orow[MT];     // output plane of the lane's row (head 0), advanced per head below
+    uint32_t orow_r[MT];
+    bool xok[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const uint32_t idx = (rt0 + m) * kTile + l16;
+        xok[m] = idx < total_rows;
+        const uint32_t p = xok[m] ? idx / a.R : 0;
+        const uint32_t r = xok[m] ? idx - p * a.R : 0;
         uint64_t plane[2];
         walk_planes(a.walk, p, plane);
-        const uint8_t* xb = a.x + plane[0] * a.x_plane_bytes;
-        // per-lane operand rows: x row for each row tile, w row for each output tile
-        const uint8_t* xrow[MT];
-        bool xok[MT];
+        const uint32_t srow = a.s + r;
+        xrow[m] = a.x + plane[0] * a.x_plane_bytes
+                + (uint64_t)(srow >> 4) * a.x_tile_cols * kTileBytes + (srow & 15u) * kRowBytes;
+        orow[m] = a.out + plane[1] * a.out_plane_bytes
+                + (uint64_t)(r >> 4) * a.out_tile_cols * kTileBytes + (r & 15u) * kRowBytes;
+        orow_r[m] = r;
+    }
+    const uint8_t* wrow[NT];
+    bool wok[NT];
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            const uint32_t r = (rt0 + m) * kTile + l16;
-            xok[m] = r < a.R;
-            const uint32_t srow = a.s + (xok[m] ? r : 0);
-            xrow[m] = xb + (uint64_t)(srow >> 4) * a.x_tile_cols * kTileBytes + (srow & 15u) * kRowBytes;
-        }
-        const uint8_t* wrow[NT];
-        bool wok[NT];
+    for (int n = 0; n < NT; ++n) {
+        const uint32_t o = (ot0 + n) * kTile + l16;
+        wok[n] = o < a.O;
+        const uint32_t oo = wok[n] ? o : 0;
+        wrow[n] = a.w + (uint64_t)(oo >> 4) * a.w_tile_cols * kTileBytes + (oo & 15u) * kRowBytes;
+    }
+    f32x4_t acc[MT][NT];
 #pragma unroll
-        for (int n = 0; n < NT; ++n) {
-            const uint32_t o = (ot0 + n) * kTile + l16;
-            wok[n] = o < a.O;
-            const uint32_t oo = wok[n] ? o : 0;
-            wrow[n] = a.w + (uint64_t)(oo >> 4) * a.w_tile_cols * kTileBytes + (oo & 15u) * kRowBytes;
-        }
-        f32x4_t acc[MT][NT];
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[m][n] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t tile_off = (kg >> 1) * kTileBytes, c0 = (kg & 1u) * 8u;
+    // Rows and outputs past the end read row 0 / output 0 instead (valid memory):
+    // an MFMA column only ever feeds its own outputs, which are not stored.  Only the
+    // inner tail needs zeros.
+    const uint32_t lane_off = tile_off + c0 * 2;
+    const uint32_t full_steps = a.I >> 5;
+#pragma unroll 1
+    for (uint32_t step = 0; step < full_steps; ++step) {
+        const uint64_t off = (uint64_t)step * (2 * kTileBytes) + lane_off;
+        bf16x8_t xf[MT], wf[NT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            xf[m] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(xrow[m] + off));
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+            wf[n] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(wrow[n] + off));
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
-            for (int n = 0; n < NT; ++n) acc[m][n] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        for (uint32_t ti = 0; ti < a.x_tile_cols; ++ti) {
-            const uint32_t i0 = ti * kTile + kg * 4;
-            bf16x4_t xf[MT], wf[NT];
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                xf[m] = bf16x4_t{0, 0, 0, 0};
-                if (xok[m]) xf[m] = load_k4(xrow[m] + (uint64_t)ti * kTileBytes, kg * 4, i0, a.I);
-            }
-#pragma unroll
-            for (int n = 0; n < NT; ++n) {
-                wf[n] = bf16x4_t{0, 0, 0, 0};
-                if (wok[n]) wf[n] = load_k4(wrow[n] + (uint64_t)ti * kTileBytes, kg * 4, i0, a.I);
-            }
-#pragma unroll
-            for (int m = 0; m < MT; ++m)
-#pragma unroll
-                for (int n = 0; n < NT; ++n)
-                    acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(wf[n], xf[m], acc[m][n], 0, 0, 0);
-        }
-        // lane holds outputs o = tile*16 + 4*kg + j (j < 4) of row r = tile*16 + l16
+            for (int n = 0; n < NT; ++n)
+                acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[n], xf[m], acc[m][n], 0, 0, 0);
+    }
+    if ((a.I & 31u) != 0) {
+        const uint32_t i0 = full_steps * 32 + kg * 8;
+        const uint64_t off = (uint64_t)full_steps * (2 * kTileBytes) + tile_off;
+        bf16x8_t xf[MT], wf[NT];
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-            const uint32_t r = (rt0 + m) * kTile + l16;
-            if (r >= a.R) continue;
+            xf[m] = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
+            if (i0 < a.I) xf[m] = load_k8(xrow[m] + off, c0, i0, a.I);
+        }
 #pragma unroll
-            for (int n = 0; n < NT; ++n) {
-                const uint32_t o = (ot0 + n) * kTile + kg * 4;
+        for (int n = 0; n < NT; ++n) {
+            wf[n] = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
+            if (i0 < a.I) wf[n] = load_k8(wrow[n] + off, c0, i0, a.I);
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[n], xf[m], acc[m][n], 0, 0, 0);
+    }
+    // lane holds outputs o = tile*16 + 4*(lane/16) + j (j < 4) of its row
+    const uint32_t og = (lane >> 4) * 4;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        if (!xok[m]) continue;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+            const uint32_t o = (ot0 + n) * kTile + og;
+            if (o >= a.O) continue;
+            if ((a.D & 15u) == 0) {
+                // heads and output tiles are aligned: the four outputs are contiguous
+                const uint32_t h = o / a.D, d = o - h * a.D;
+                uint8_t* dst = orow[m] + (uint64_t)h * a.head_stride * a.out_plane_bytes
+                        + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2;
+                *reinterpret_cast<u32x2*>(dst) = u32x2{pack_bf16(acc[m][n][0], acc[m][n][1]),
+                                                      pack_bf16(acc[m][n][2], acc[m][n][3])};
+            } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t oj = o + j;
                     if (oj >= a.O) continue;
                     const uint32_t h = oj / a.D, d = oj - h * a.D;
-                    uint8_t* dst = a.out + (plane[1] + (uint64_t)h * a.head_stride) * a.out_plane_bytes
-                            + ((uint64_t)(r >> 4) * a.out_tile_cols + (d >> 4)) * kTileBytes
-                            + (r & 15u) * kRowBytes + (d & 15u) * 2;
+                    uint8_t* dst = orow[m] + (uint64_t)h * a.head_stride * a.out_plane_bytes
+                            + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2;
                     *reinterpret_cast<uint16_t*>(dst) = (uint16_t)bf16_rne_sw(as_u32(acc[m][n][j]));
                 }
             }
+        }
+    }
+    (void)orow_r;
+}
+
+// ---------------------------------------------------------------------------
+// BF16 on the matrix cores, operands staged through LDS
+// ---------------------------------------------------------------------------
+//
+// A workgroup of eight waves owns 256 rows x 256 outputs; a wave owns 128 rows x
+// 64 outputs (8 x 4 MFMA tiles, 128 accumulator registers).  The inner axis is
+// walked in stages of 32*KS elements.  One "fragment" is the pair of neighbouring
+// 16x16 tiles (1 KiB, contiguous in memory) that feeds one MFMA operand; a stage
+// holds 16 row-tile and 16 output-tile fragments per 32 inner elements.  Fragments
+// go from global memory to LDS with the direct loader (global_load_lds, 16 bytes a
+// lane, no registers) into the other half of a double buffer while the matrix
+// cores work on this half, so every operand crosses L2->CU once per workgroup
+// instead of once per wave.
+//
+// The direct loader puts lane i's 16 bytes at fragment + 16*i, so the LDS order is
+// chosen by which global chunk lane i asks for: chunk (tile t, row r, half h) is
+// placed at position 32*t + 2*r + (h ^ (r >> 3)).  A 16-lane group of an operand
+// read (same t and h, rows 0..15) then touches 16 different 16-byte bank groups.
+
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+template <int KS>
+__global__ __launch_bounds__(512) void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
+    constexpr int WM = 8, WN = 4;                 // wave tile, in 16x16 tiles
+    constexpr uint32_t BM = 16, BN = 16;          // workgroup tile, in 16x16 tiles
+    constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
+    constexpr uint32_t kStageFrags = (BM + BN) * KS, kStageBytes = kStageFrags * kFrag;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t l16 = lane & 15u, kg = lane >> 4;
+    const uint32_t total_rows = a.planes * a.R;
+    const uint32_t bm0 = blockIdx.x * BM, bn0 = blockIdx.y * BN;   // first row tile / output tile
+    const uint32_t wm = wave & 1u, wn = wave >> 1;
+
+    // loader role: this wave brings in fragments wave, wave+8 (rows) and wave+16,
+    // wave+24 (outputs) of every 32-element slice; lane i fetches the chunk whose
+    // LDS position is i
+    const uint32_t ld_tile = lane >> 5, ld_q = lane & 31u, ld_row = ld_q >> 1;
+    const uint32_t ld_half = (ld_q & 1u) ^ (ld_row >> 3);
+    const uint32_t ld_off = ld_tile * kTileBytes + ld_half * 16;
+    const uint8_t* src[4];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        uint32_t idx = (bm0 + wave + 8 * j) * kTile + ld_row;
+        if (idx >= total_rows) idx = 0;            // valid memory; its results are not stored
+        const uint32_t p = idx / a.R, r = idx - p * a.R;
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        const uint32_t srow = a.s + r;
+        src[j] = a.x + plane[0] * a.x_plane_bytes + (uint64_t)(srow >> 4) * a.x_tile_cols * kTileBytes
+                + (srow & 15u) * kRowBytes + ld_off;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        uint32_t o = (bn0 + wave + 8 * j) * kTile + ld_row;
+        if (o >= a.O) o = 0;
+        src[2 + j] = a.w + (uint64_t)(o >> 4) * a.w_tile_cols * kTileBytes + (o & 15u) * kRowBytes + ld_off;
+    }
+    auto issue = [&](uint32_t stage, uint32_t buf) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint64_t goff = (uint64_t)(stage * KS + ks) * kFrag;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t frag = ks * (BM + BN) + wave + 8 * j;
+                __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + goff),
+                                                 (lptr_t)(lds + buf * kStageBytes + frag * kFrag), 16, 0, 0);
+            }
+        }
+    };
+
+    f32x4_t acc[WM][WN];
+#pragma unroll
+    for (int m = 0; m < WM; ++m)
+#pragma unroll
+        for (int n = 0; n < WN; ++n) acc[m][n] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // reader role: position of the lane's eight inner elements inside a fragment
+    const uint32_t rd_off = ((kg >> 1) * 32 + l16 * 2 + ((kg & 1u) ^ (l16 >> 3))) * 16;
+    const uint32_t stages = a.I / (32 * KS);
+    issue(0, 0);
+    for (uint32_t st = 0; st < stages; ++st) {
+        const uint32_t buf = st & 1u;
+        // my fragments of this stage have landed; after the barrier everyone's have,
+        // and everyone has finished reading the other half
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        if (st + 1 < stages) issue(st + 1, buf ^ 1u);
+        const uint8_t* base = lds + buf * kStageBytes + rd_off;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            bf16x8_t xf[WM], wf[WN];
+#pragma unroll
+            for (int n = 0; n < WN; ++n)
+                wf[n] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(
+                        base + (ks * (BM + BN) + BM + wn * WN + n) * kFrag));
+#pragma unroll
+            for (int m = 0; m < WM; ++m)
+                xf[m] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(
+                        base + (ks * (BM + BN) + wm * WM + m) * kFrag));
+#pragma unroll
+            for (int m = 0; m < WM; ++m)
+#pragma unroll
+                for (int n = 0; n < WN; ++n)
+                    acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[n], xf[m], acc[m][n], 0, 0, 0);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+
+    // lane holds outputs o = tile*16 + 4*(lane/16) + j (j < 4) of row l16 of its row tiles
+    const uint32_t og = kg * 4;
+#pragma unroll
+    for (int m = 0; m < WM; ++m) {
+        const uint32_t idx = (bm0 + wm * WM + m) * kTile + l16;
+        if (idx >= total_rows) continue;
+        const uint32_t p = idx / a.R, r = idx - p * a.R;
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        uint8_t* orow = a.out + plane[1] * a.out_plane_bytes
+                + (uint64_t)(r >> 4) * a.out_tile_cols * kTileBytes + (r & 15u) * kRowBytes;
+#pragma unroll
+        for (int n = 0; n < WN; ++n) {
+            const uint32_t o = (bn0 + wn * WN + n) * kTile + og;
+            if (o >= a.O) continue;
+            const uint32_t h = o / a.D, d = o - h * a.D;      // D % 16 == 0 on this path
+            uint8_t* dst = orow + (uint64_t)h * a.head_stride * a.out_plane_bytes
+                    + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2;
+            *reinterpret_cast<u32x2*>(dst) = u32x2{pack_bf16(acc[m][n][0], acc[m][n][1]),
+                                                  pack_bf16(acc[m][n][2], acc[m][n][3])};
         }
     }
 }
@@ -331,19 +512,31 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
     const hipStream_t st = native(stream);
     const uint32_t gy = a.planes < 65535u ? a.planes : 65535u;
 
-    if (dtype == DT_BF16 && path == 0) {
+    if (dtype == DT_BF16 && (path == 0 || path == 2)) {
+        const uint64_t total_rows = (uint64_t)a.planes * a.R;
         const uint32_t o_tiles = (a.O + kTile - 1) / kTile;
-        if (a.row_tiles <= 2) {
-            // few rows (decode, last-row logits): one row tile per wave, more output tiles
-            const dim3 grid((a.row_tiles + 1) / 2, (o_tiles + 15) / 16, gy);
-            hipLaunchKernelGGL((linear_mfma_bf16_kernel<1, 8>), grid, dim3(256), 0, st, a);
-        } else {
-            const dim3 grid((a.row_tiles + 3) / 4, (o_tiles + 7) / 8, gy);
-            hipLaunchKernelGGL((linear_mfma_bf16_kernel<2, 4>), grid, dim3(256), 0, st, a);
+        if (total_rows <= 0x7FFFFFFFull && o_tiles <= 65535u * 8u) {
+            const uint32_t row_tiles = (uint32_t)((total_rows + kTile - 1) / kTile);
+            static const int lds_ks = getenv("IOMX_LT") ? atoi(getenv("IOMX_LT")) : 2;
+            if (path == 0 && lds_ks > 0 && row_tiles >= 16 && (a.I % 64) == 0 && (a.D & 15u) == 0) {
+                // enough rows to fill 256-row workgroup tiles: operands staged through LDS
+                const dim3 grid((row_tiles + 15) / 16, (o_tiles + 15) / 16);
+                if (lds_ks == 1) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<1>), grid, dim3(512), 0, st, a);
+                else hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<2>), grid, dim3(512), 0, st, a);
+                record_launch("linear_mfma_lds", grid.x * grid.y, 512, (uint64_t)row_tiles * o_tiles);
+            } else if (row_tiles <= 4) {
+                // few rows (decode, last-row logits): one row tile per wave, more output tiles
+                const dim3 grid((row_tiles + 1) / 2, (o_tiles + 15) / 16);
+                hipLaunchKernelGGL((linear_mfma_bf16_kernel<1, 8>), grid, dim3(256), 0, st, a);
+                record_launch("linear_mfma", grid.x * grid.y, 256, (uint64_t)row_tiles * o_tiles);
+            } else {
+                const dim3 grid((row_tiles + 7) / 8, (o_tiles + 7) / 8);
+                hipLaunchKernelGGL((linear_mfma_bf16_kernel<4, 4>), grid, dim3(256), 0, st, a);
+                record_launch("linear_mfma", grid.x * grid.y, 256, (uint64_t)row_tiles * o_tiles);
+            }
+            IOMX_HIP(hipGetLastError());
+            return IOMX_OK;
         }
-        record_launch("linear_mfma", (a.row_tiles + 3) / 4, 256, (uint64_t)a.row_tiles * o_tiles * a.planes);
-        IOMX_HIP(hipGetLastError());
-        return IOMX_OK;
     }
 
     const dim3 grid((a.lanes_per_plane + 255) / 256, gy);

@@ -207,3 +207,34 @@ def test_backend_linear_next_to_the_reference_cpu_backend(devices, dtype):
         assert (np.abs(a - b) <= np.maximum(2.0 ** -7, 2.0 ** -6 * np.abs(a))).all()
     else:
         assert np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("hp", [False, True], ids=["ordinary", "head_planar"])
+@pytest.mark.parametrize("window", [(0, 200), (5, 190)], ids=["all_rows", "window"])
+def test_bf16_matrix_cores_staged_through_lds(hp, window):
+    """Many rows: the workgroup-tiled kernel.  Rows of different planes share row tiles
+    (R is not a multiple of 16), the last workgroup column is mostly past O."""
+    s, R = window
+    xd, wd, H, D = (3, 200, 128), (272, 128), 17, 16
+    xv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(xd)), 0, 1, 31)).reshape(xd)
+    wv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(wd)), 0, 0.1, 32)).reshape(wd)
+    dx, hx = pair(DT_BF16, xd, values=xv)
+    dw, hw = pair(DT_BF16, wd, values=wv)
+    od = (3, H, R, D) if hp else (3, R, H * D)
+    do, ho = pair(DT_BF16, od, salt=33)
+    args = (s, R, hp, H if hp else 1, D if hp else H * D)
+    assert iomx.linear(dx.view(), dw.view(), do.view(), *args) == 0
+    assert iomx.last_launch().kernel.decode() == "linear_mfma_lds"
+    got = do.view().to_host()
+    g3 = got.transpose(0, 2, 1, 3).reshape(3, R, H * D) if hp else got
+    for b in range(3):
+        assert bf16_bound(g3[b], xv[b, s:s + R], wv).all()
+    mask = iomo.tile_plane(np.ones(od, np.uint16)) == 0
+    assert np.array_equal(do.raw()[mask], ho.storage[mask])
+    # the direct-from-global kernel adds the same products in the same order
+    d2, _ = pair(DT_BF16, od, salt=33)
+    assert iomx.linear(dx.view(), dw.view(), d2.view(), *args, path=2) == 0
+    assert iomx.last_launch().kernel.decode() == "linear_mfma"
+    assert np.array_equal(d2.raw(), do.raw())
+    for t in (dx, dw, do, d2):
+        t.free()
