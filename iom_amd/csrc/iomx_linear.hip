@@ -15,6 +15,7 @@
 //                    that a lane ends up with four consecutive outputs of one row.
 #include "iomx_rows.hpp"
 #include <cstdlib>
+#include <type_traits>
 
 namespace iomx {
 
@@ -32,6 +33,7 @@ struct LinearArgs {
     uint32_t row_tiles;       // ceil(R / 16)
     uint32_t lanes_per_plane; // row_tiles * 16 * H * out_tile_cols
     uint32_t planes;
+    uint32_t row_blocks, out_blocks, super_y;   // workgroup-tiled kernel: 256-row / 256-output blocks
 };
 
 // ---------------------------------------------------------------------------
@@ -308,33 +310,42 @@ __global__ __launch_bounds__(256) void linear_mfma_bf16_kernel(const LinearArgs 
 // cores work on this half, so every operand crosses L2->CU once per workgroup
 // instead of once per wave.
 //
-// The direct loader puts lane i's 16 bytes at fragment + 16*i, so the LDS order is
-// chosen by which global chunk lane i asks for: chunk (tile t, row r, half h) is
-// placed at position 32*t + 2*r + (h ^ (r >> 3)).  A 16-lane group of an operand
-// read (same t and h, rows 0..15) then touches 16 different 16-byte bank groups.
+// The direct loader puts lane i's 16 bytes at fragment + 16*i, so a fragment lies in
+// LDS as it lies in memory.  ds_read_b128 serves the lanes {0-3, 12-15, 20-23, 24-27},
+// {4-7, 8-11, 16-19, 28-31} (and the same +32) together; with lane l reading row l%16,
+// inner elements 8*(l/16).., of the plain tiled fragment each such group touches 16
+// different 16-byte bank groups, so the operand reads are conflict-free as stored.
+//
+// Workgroups are numbered so that the 32 that run together on one XCD (ids equal
+// modulo 8) cover 8 row blocks x 4 output blocks: the XCD's L2 then serves every
+// operand slice to 4 or 8 workgroups for one fetch from HBM.
 
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-template <int KS>
-__global__ __launch_bounds__(512) void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
+template <int KS, int DEPTH>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     constexpr int WM = 8, WN = 4;                 // wave tile, in 16x16 tiles
     constexpr uint32_t BM = 16, BN = 16;          // workgroup tile, in 16x16 tiles
     constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
     constexpr uint32_t kStageFrags = (BM + BN) * KS, kStageBytes = kStageFrags * kFrag;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kStageBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[DEPTH * kStageBytes];
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     const uint32_t total_rows = a.planes * a.R;
-    const uint32_t bm0 = blockIdx.x * BM, bn0 = blockIdx.y * BN;   // first row tile / output tile
+    // blockIdx.x -> (row block, output block): XCD = id % 8, 32 consecutive slots of an
+    // XCD = 8 x 4 blocks, eight XCDs stacked along the rows, super-blocks output-major
+    const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+    const uint32_t sb = slot >> 5, jx = slot & 7u, jy = (slot >> 3) & 3u;
+    const uint32_t bx = (sb / a.super_y) * 64 + xcd * 8 + jx, by = (sb % a.super_y) * 4 + jy;
+    if (bx >= a.row_blocks || by >= a.out_blocks) return;
+    const uint32_t bm0 = bx * BM, bn0 = by * BN;   // first row tile / output tile
     const uint32_t wm = wave & 1u, wn = wave >> 1;
 
     // loader role: this wave brings in fragments wave, wave+8 (rows) and wave+16,
-    // wave+24 (outputs) of every 32-element slice; lane i fetches the chunk whose
-    // LDS position is i
-    const uint32_t ld_tile = lane >> 5, ld_q = lane & 31u, ld_row = ld_q >> 1;
-    const uint32_t ld_half = (ld_q & 1u) ^ (ld_row >> 3);
-    const uint32_t ld_off = ld_tile * kTileBytes + ld_half * 16;
+    // wave+24 (outputs) of every 32-element slice; lane i fetches 16-byte chunk i
+    const uint32_t ld_tile = lane >> 5, ld_row = (lane & 31u) >> 1;
+    const uint32_t ld_off = ld_tile * kTileBytes + (lane & 1u) * 16;
     const uint8_t* src[4];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -373,36 +384,82 @@ __global__ __launch_bounds__(512) void linear_mfma_lds_bf16_kernel(const LinearA
         for (int n = 0; n < WN; ++n) acc[m][n] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     // reader role: position of the lane's eight inner elements inside a fragment
-    const uint32_t rd_off = ((kg >> 1) * 32 + l16 * 2 + ((kg & 1u) ^ (l16 >> 3))) * 16;
-    const uint32_t stages = a.I / (32 * KS);
-    issue(0, 0);
-    for (uint32_t st = 0; st < stages; ++st) {
-        const uint32_t buf = st & 1u;
-        // my fragments of this stage have landed; after the barrier everyone's have,
-        // and everyone has finished reading the other half
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        if (st + 1 < stages) issue(st + 1, buf ^ 1u);
-        const uint8_t* base = lds + buf * kStageBytes + rd_off;
+    const uint32_t rd_off = (kg >> 1) * kTileBytes + l16 * kRowBytes + (kg & 1u) * 16;
+    const uint32_t stages = a.I / 32;
+    // A ring of four stage buffers (one stage = 32 inner elements).  In the middle of
+    // stage st every wave waits for its own loads of stage st+1 and meets the others
+    // at the barrier: from there on stage st+1 is complete in LDS and nobody reads
+    // stage st-1 any more, so the second half of the stage (a) requests stage st+3
+    // into the buffer of st-1, one direct load after every four MFMAs -- a direct load
+    // holds its wave at issue until the memory pipeline takes it, and the matrix
+    // instructions issued before it keep the matrix core busy meanwhile -- and (b)
+    // already reads the first operands of stage st+1, so the matrix core does not
+    // drain at the stage boundary.
+    static_assert(KS == 1 && DEPTH == 4, "the schedule below is written for four 32-element stages");
+    const uint32_t last = stages - 1;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            bf16x8_t xf[WM], wf[WN];
+    for (uint32_t d = 0; d < 3; ++d) issue(d < stages ? d : last, d);
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    bf16x8_t wf[2][WN], xf[4];
+    auto rd = [&](uint32_t ring, uint32_t frag) {
+        return __builtin_bit_cast(bf16x8_t,
+                *reinterpret_cast<const u32x4*>(lds + ring * kStageBytes + rd_off + frag * kFrag));
+    };
+#pragma unroll
+    for (int n = 0; n < WN; ++n) wf[0][n] = rd(0, BM + wn * WN + n);
+    xf[0] = rd(0, wm * WM);
+    xf[1] = rd(0, wm * WM + 1);
+    // one stage; P = parity of the stage (which half of wf holds its output fragments)
+    auto stage = [&](auto parity, uint32_t st) {
+        constexpr int P = decltype(parity)::value;
+        const uint32_t ring = st & 3u, ring1 = (st + 1) & 3u, ring3 = (st + 3) & 3u;
+        const uint64_t gnext = (uint64_t)(st + 3 < stages ? st + 3 : last) * kFrag;
+#pragma unroll
+        for (int step = 0; step < 4; ++step) {
+            xf[(step + 2) & 3] = rd(ring, wm * WM + step + 2);
 #pragma unroll
             for (int n = 0; n < WN; ++n)
-                wf[n] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(
-                        base + (ks * (BM + BN) + BM + wn * WN + n) * kFrag));
-#pragma unroll
-            for (int m = 0; m < WM; ++m)
-                xf[m] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(
-                        base + (ks * (BM + BN) + wm * WM + m) * kFrag));
-#pragma unroll
-            for (int m = 0; m < WM; ++m)
-#pragma unroll
-                for (int n = 0; n < WN; ++n)
-                    acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[n], xf[m], acc[m][n], 0, 0, 0);
+                acc[step][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[P][n], xf[step & 3], acc[step][n], 0, 0, 0);
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int step = 0; step < 4; ++step) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, WN, 0);
+        }
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int step = 4; step < 8; ++step) {
+            if (step < 6) xf[(step + 2) & 3] = rd(ring, wm * WM + step + 2);
+            else xf[(step + 2) & 3] = rd(ring1, wm * WM + step - 6);
+            if (step == 5) {
+#pragma unroll
+                for (int n = 0; n < WN; ++n) wf[P ^ 1][n] = rd(ring1, BM + wn * WN + n);
+            }
+#pragma unroll
+            for (int n = 0; n < WN; ++n)
+                acc[step][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[P][n], xf[step & 3], acc[step][n], 0, 0, 0);
+            const int j = step - 4;
+            __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + gnext),
+                                             (lptr_t)(lds + ring3 * kStageBytes + (wave + 8 * j) * kFrag), 16, 0, 0);
+        }
+#pragma unroll
+        for (int step = 4; step < 8; ++step) {
+            if (step == 5) __builtin_amdgcn_sched_group_barrier(0x100, WN + 1, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, WN, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+    };
+    uint32_t st = 0;
+    for (; st + 1 < stages; st += 2) {
+        stage(std::integral_constant<int, 0>{}, st);
+        stage(std::integral_constant<int, 1>{}, st + 1);
     }
+    if (st < stages) stage(std::integral_constant<int, 0>{}, st);
+    // nothing may still be landing in LDS when the workgroup gives it back
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // lane holds outputs o = tile*16 + 4*(lane/16) + j (j < 4) of row l16 of its row tiles
     const uint32_t og = kg * 4;
@@ -518,12 +575,16 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
         if (total_rows <= 0x7FFFFFFFull && o_tiles <= 65535u * 8u) {
             const uint32_t row_tiles = (uint32_t)((total_rows + kTile - 1) / kTile);
             static const int lds_ks = getenv("IOMX_LT") ? atoi(getenv("IOMX_LT")) : 2;
-            if (path == 0 && lds_ks > 0 && row_tiles >= 16 && (a.I % 64) == 0 && (a.D & 15u) == 0) {
+            if (path == 0 && lds_ks > 0 && row_tiles >= 16 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
                 // enough rows to fill 256-row workgroup tiles: operands staged through LDS
-                const dim3 grid((row_tiles + 15) / 16, (o_tiles + 15) / 16);
-                if (lds_ks == 1) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<1>), grid, dim3(512), 0, st, a);
-                else hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<2>), grid, dim3(512), 0, st, a);
-                record_launch("linear_mfma_lds", grid.x * grid.y, 512, (uint64_t)row_tiles * o_tiles);
+                a.row_blocks = (row_tiles + 15) / 16;
+                a.out_blocks = (o_tiles + 15) / 16;
+                a.super_y = (a.out_blocks + 3) / 4;
+                const uint64_t wgs = (uint64_t)((a.row_blocks + 63) / 64) * a.super_y * 256;
+                if (wgs > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
+                const dim3 grid((uint32_t)wgs);
+                hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<1, 4>), grid, dim3(512), 0, st, a);
+                record_launch("linear_mfma_lds", grid.x, 512, (uint64_t)row_tiles * o_tiles);
             } else if (row_tiles <= 4) {
                 // few rows (decode, last-row logits): one row tile per wave, more output tiles
                 const dim3 grid((row_tiles + 1) / 2, (o_tiles + 15) / 16);
