@@ -246,8 +246,13 @@ int iomx_launch_rope(int dtype, const iomx_view* x, const iomx_view* out, uint64
  * one fused multiply-add per increasing i in F32 (F64 for F64) from +0 and one
  * encode.  path 0 lets BF16 run on the matrix cores (exact products, F32
  * accumulation in the hardware's order, one round-to-nearest-even store: the
- * "native BF16" allowance of linear-projections.md:213-218); path 1 forces the
- * scalar recurrence for every leaf.
+ * "native BF16" allowance of linear-projections.md:213-218) and picks the kernel by
+ * the number of rows (rows of all planes count as one row axis): 256 rows or more
+ * with I % 32 == 0 and D % 16 == 0 take the workgroup-tiled kernel that stages
+ * operands through LDS, fewer rows the kernel that splits the inner axis over the
+ * waves of a workgroup; path 1 forces the scalar recurrence for every leaf; path 2
+ * forces the BF16 matrix-core kernel that loads operands straight from global
+ * memory (any shape; the fallback of path 0 and the cross-check of the other two).
  */
 int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const iomx_view* out,
                        uint64_t s, uint64_t R, int head_planar, uint64_t H, uint64_t D, int path,

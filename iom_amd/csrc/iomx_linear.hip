@@ -13,8 +13,13 @@
 //                    consecutive inner elements (16 bytes) of tile row l%16, so no
 //                    transposition is needed; the weight tile is the A operand so
 //                    that a lane ends up with four consecutive outputs of one row.
+//                    The rows of all planes form one row axis.  Three kernels share
+//                    this operand mapping: linear_mfma (operands straight from
+//                    global memory, any shape), linear_mfma_splitk (few rows: the
+//                    inner axis split over the waves of a workgroup so that every
+//                    CU streams weights) and linear_mfma_lds (256 rows or more:
+//                    256x256 workgroup tiles staged through LDS).
 #include "iomx_rows.hpp"
-#include <cstdlib>
 #include <type_traits>
 
 namespace iomx {
@@ -296,6 +301,155 @@ __global__ __launch_bounds__(256) void linear_mfma_bf16_kernel(const LinearArgs 
     (void)orow_r;
 }
 
+// Few rows (a decode step, last-row logits): the weight is the traffic, read once,
+// and the job is to have every CU streaming it.  One workgroup = NT output tiles
+// against MT row tiles; its four waves take every fourth 32-element slice of the
+// inner axis, so together they read each tile's weight rows as one contiguous
+// stream, and their partial sums meet in LDS (added in wave order, so the result
+// does not depend on timing).  When each row is the only row of its plane (one
+// token per sequence) a 128-byte line of x holds 32 useful bytes, so x costs MT x
+// 4 bytes of line traffic per weight byte-row it meets: the launch picks MT = 1 and
+// lets NT output tiles share each x fragment.
+template <int MT, int NT>
+__global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const LinearArgs a) {
+    constexpr uint32_t kTileBytes = 512, kRowBytes = 32;
+    __shared__ f32x4_t partial[3][MT][NT][64];
+    const uint32_t lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t l16 = lane & 15u, kg = lane >> 4;
+    const uint32_t total_rows = a.planes * a.R;
+    const uint32_t ot0 = blockIdx.x * NT, rt0 = blockIdx.y * MT;
+    const uint8_t* xrow[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        uint32_t idx = (rt0 + m) * kTile + l16;
+        if (idx >= total_rows) idx = 0;            // valid memory; its results are not stored
+        const uint32_t p = idx / a.R, r = idx - p * a.R;
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        const uint32_t srow = a.s + r;
+        xrow[m] = a.x + plane[0] * a.x_plane_bytes
+                + (uint64_t)(srow >> 4) * a.x_tile_cols * kTileBytes + (srow & 15u) * kRowBytes;
+    }
+    const uint8_t* wrow[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+        uint32_t o_row = (ot0 + n) * kTile + l16;
+        if (o_row >= a.O) o_row = 0;
+        wrow[n] = a.w + (uint64_t)(o_row >> 4) * a.w_tile_cols * kTileBytes + (o_row & 15u) * kRowBytes;
+    }
+    f32x4_t acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) acc[m][n] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t tile_off = (kg >> 1) * kTileBytes, c0 = (kg & 1u) * 8u;
+    const uint32_t lane_off = tile_off + c0 * 2;
+    const uint32_t full_steps = a.I >> 5;
+    // kBatch slices a wave are requested before the first is multiplied: a wave has
+    // only a few slices, and what it waits for is memory latency
+    constexpr uint32_t kBatch = (MT + NT) <= 5 ? 8 : 4;
+    uint32_t step = wave;
+    for (; step + 4 * (kBatch - 1) < full_steps; step += 4 * kBatch) {
+        bf16x8_t wf[kBatch][NT], xf[kBatch][MT];
+#pragma unroll
+        for (uint32_t u = 0; u < kBatch; ++u) {
+            const uint64_t off = (uint64_t)(step + 4 * u) * (2 * kTileBytes) + lane_off;
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                wf[u][n] = __builtin_bit_cast(bf16x8_t, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[n] + off)));
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+                xf[u][m] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(xrow[m] + off));
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < kBatch; ++u)
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+#pragma unroll
+                for (int n = 0; n < NT; ++n)
+                    acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][n], xf[u][m], acc[m][n], 0, 0, 0);
+    }
+    for (; step < full_steps; step += 4) {
+        const uint64_t off = (uint64_t)step * (2 * kTileBytes) + lane_off;
+        bf16x8_t wf[NT], xf[MT];
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+            wf[n] = __builtin_bit_cast(bf16x8_t, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[n] + off)));
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            xf[m] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(xrow[m] + off));
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[n], xf[m], acc[m][n], 0, 0, 0);
+    }
+    if ((a.I & 31u) != 0 && (full_steps & 3u) == wave) {
+        const uint32_t i0 = full_steps * 32 + kg * 8;
+        const uint64_t off = (uint64_t)full_steps * (2 * kTileBytes) + tile_off;
+        bf16x8_t wf[NT], xf[MT];
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+            wf[n] = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
+            if (i0 < a.I) wf[n] = load_k8(wrow[n] + off, c0, i0, a.I);
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            xf[m] = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
+            if (i0 < a.I) xf[m] = load_k8(xrow[m] + off, c0, i0, a.I);
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[n], xf[m], acc[m][n], 0, 0, 0);
+    }
+    if (wave != 0) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n) partial[wave - 1][m][n][lane] = acc[m][n];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // lane holds outputs o = tile*16 + 4*(lane/16) + j (j < 4) of row l16 of its row tiles
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const uint32_t idx = (rt0 + m) * kTile + l16;
+        if (idx >= total_rows) continue;
+        const uint32_t p = idx / a.R, r = idx - p * a.R;
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        uint8_t* orow = a.out + plane[1] * a.out_plane_bytes
+                + (uint64_t)(r >> 4) * a.out_tile_cols * kTileBytes + (r & 15u) * kRowBytes;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+            const uint32_t o = (ot0 + n) * kTile + kg * 4;
+            if (o >= a.O) continue;
+            f32x4_t v = acc[m][n];
+#pragma unroll
+            for (int k = 0; k < 3; ++k) v += partial[k][m][n][lane];
+            if ((a.D & 3u) == 0 && o + 4 <= a.O) {
+                // the four outputs lie in one head and one tile row
+                const uint32_t h = o / a.D, d = o - h * a.D;
+                uint8_t* dst = orow + (uint64_t)h * a.head_stride * a.out_plane_bytes
+                        + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2;
+                *reinterpret_cast<u32x2*>(dst) = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+                continue;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t oj = o + j;
+                if (oj >= a.O) continue;
+                const uint32_t h = oj / a.D, d = oj - h * a.D;
+                uint8_t* dst = orow + (uint64_t)h * a.head_stride * a.out_plane_bytes
+                        + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2;
+                *reinterpret_cast<uint16_t*>(dst) = (uint16_t)bf16_rne_sw(as_u32(v[j]));
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // BF16 on the matrix cores, operands staged through LDS
 // ---------------------------------------------------------------------------
@@ -461,8 +615,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // nothing may still be landing in LDS when the workgroup gives it back
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // lane holds outputs o = tile*16 + 4*(lane/16) + j (j < 4) of row l16 of its row tiles
-    const uint32_t og = kg * 4;
+    // lane holds outputs o = tile*16 + 4*(lane/16) + j (j < 4) of row l16 of its row tiles.
+    // Heads are whole tiles wide here, so head and tile of an output tile are the same
+    // for the whole wave.
+    const uint32_t d_tiles = a.D >> 4;
+    uint64_t col_off[WN];
+    bool col_ok[WN];
+#pragma unroll
+    for (int n = 0; n < WN; ++n) {
+        const uint32_t ot = bn0 + wn * WN + n;
+        col_ok[n] = ot * kTile < a.O;
+        const uint32_t h = ot / d_tiles, dt = ot - h * d_tiles;
+        col_off[n] = (uint64_t)h * a.head_stride * a.out_plane_bytes + (uint64_t)dt * kTileBytes + kg * 8;
+    }
 #pragma unroll
     for (int m = 0; m < WM; ++m) {
         const uint32_t idx = (bm0 + wm * WM + m) * kTile + l16;
@@ -474,13 +639,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 + (uint64_t)(r >> 4) * a.out_tile_cols * kTileBytes + (r & 15u) * kRowBytes;
 #pragma unroll
         for (int n = 0; n < WN; ++n) {
-            const uint32_t o = (bn0 + wn * WN + n) * kTile + og;
-            if (o >= a.O) continue;
-            const uint32_t h = o / a.D, d = o - h * a.D;      // D % 16 == 0 on this path
-            uint8_t* dst = orow + (uint64_t)h * a.head_stride * a.out_plane_bytes
-                    + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2;
-            *reinterpret_cast<u32x2*>(dst) = u32x2{pack_bf16(acc[m][n][0], acc[m][n][1]),
-                                                  pack_bf16(acc[m][n][2], acc[m][n][3])};
+            if (!col_ok[n]) continue;
+            *reinterpret_cast<u32x2*>(orow + col_off[n]) = u32x2{pack_bf16(acc[m][n][0], acc[m][n][1]),
+                                                                 pack_bf16(acc[m][n][2], acc[m][n][3])};
         }
     }
 }
@@ -574,8 +735,7 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
         const uint32_t o_tiles = (a.O + kTile - 1) / kTile;
         if (total_rows <= 0x7FFFFFFFull && o_tiles <= 65535u * 8u) {
             const uint32_t row_tiles = (uint32_t)((total_rows + kTile - 1) / kTile);
-            static const int lds_ks = getenv("IOMX_LT") ? atoi(getenv("IOMX_LT")) : 2;
-            if (path == 0 && lds_ks > 0 && row_tiles >= 16 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
+            if (path == 0 && row_tiles >= 16 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
                 // enough rows to fill 256-row workgroup tiles: operands staged through LDS
                 a.row_blocks = (row_tiles + 15) / 16;
                 a.out_blocks = (o_tiles + 15) / 16;
@@ -585,8 +745,23 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                 const dim3 grid((uint32_t)wgs);
                 hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<1, 4>), grid, dim3(512), 0, st, a);
                 record_launch("linear_mfma_lds", grid.x, 512, (uint64_t)row_tiles * o_tiles);
+            } else if (path == 0 && row_tiles < 16 && o_tiles <= 0x7FFFFFFFu) {
+                // few rows (decode, last-row logits): one output tile per workgroup, the
+                // inner axis split over its waves
+                // rows that are alone in their plane (R == 1 of many planes) make x the
+                // expensive operand: then one row tile against four output tiles;
+                // otherwise up to four row tiles against one or two
+                const bool sparse_rows = a.R < kTile && a.planes > 1;
+                uint32_t mt, nt;
+                if (sparse_rows) { mt = 1; nt = 4; }
+                else { mt = row_tiles == 1 ? 1 : row_tiles == 2 ? 2 : 4; nt = mt == 1 ? 2 : 1; }
+                const dim3 grid((o_tiles + nt - 1) / nt, (row_tiles + mt - 1) / mt);
+#define IOMX_SPLITK(M, N) \
+    if (mt == M && nt == N) hipLaunchKernelGGL((linear_mfma_splitk_bf16_kernel<M, N>), grid, dim3(256), 0, st, a)
+                IOMX_SPLITK(1, 2); IOMX_SPLITK(1, 4); IOMX_SPLITK(2, 1); IOMX_SPLITK(4, 1);
+#undef IOMX_SPLITK
+                record_launch("linear_mfma_splitk", grid.x * grid.y, 256, (uint64_t)row_tiles * o_tiles);
             } else if (row_tiles <= 4) {
-                // few rows (decode, last-row logits): one row tile per wave, more output tiles
                 const dim3 grid((row_tiles + 1) / 2, (o_tiles + 15) / 16);
                 hipLaunchKernelGGL((linear_mfma_bf16_kernel<1, 8>), grid, dim3(256), 0, st, a);
                 record_launch("linear_mfma", grid.x * grid.y, 256, (uint64_t)row_tiles * o_tiles);

@@ -90,8 +90,9 @@ def bf16_bound(g_raw, x_raw, w_raw):
     return np.abs(g - q) <= np.maximum(np.maximum(ulp, 2.0 ** -7), 2.0 ** -6 * np.abs(q))
 
 
+@pytest.mark.parametrize("path,kernel", [(0, "linear_mfma_splitk"), (2, "linear_mfma")], ids=["split_inner", "direct"])
 @pytest.mark.parametrize("case", range(len(FIXTURES)))
-def test_bf16_matrix_cores_on_the_fixtures(case):
+def test_bf16_matrix_cores_on_the_fixtures(case, path, kernel):
     xd, wd, s, R, hp, H, D = FIXTURES[case]
     xv = small_values(DT_BF16, int(np.prod(xd)), 1 + case).reshape(xd)
     wv = small_values(DT_BF16, int(np.prod(wd)), 11 + case).reshape(wd)
@@ -99,8 +100,8 @@ def test_bf16_matrix_cores_on_the_fixtures(case):
     dw, hw = pair(DT_BF16, wd, values=wv)
     od = xd[:-2] + ((H, R, D) if hp else (R, D))
     do, ho = pair(DT_BF16, od, salt=21 + case)
-    assert iomx.linear(dx.view(), dw.view(), do.view(), s, R, hp, H, D) == 0
-    assert iomx.last_launch().kernel.decode() == "linear_mfma"
+    assert iomx.linear(dx.view(), dw.view(), do.view(), s, R, hp, H, D, path=path) == 0
+    assert iomx.last_launch().kernel.decode() == kernel
     assert iomo.linear(hx.view(), hw.view(), ho.view(), s, R, hp, H, D) == 0
     got = do.view().to_host()
     lead = int(np.prod(xd[:-2])) if len(xd) > 2 else 1
