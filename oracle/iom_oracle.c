@@ -9,6 +9,7 @@
 #include "iom_oracle.h"
 
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 #define TILE 16u
@@ -942,6 +943,131 @@ int iomo_linear(int dtype, const iomo_view* x, const iomo_view* w, const iomo_vi
             store_leaf(out->base, iomo_plane_slot(R, D, op + h * head_stride, r, d), bits, raw);
         }
     } while (next_coord(coord, x->dims, leading));
+    return IOMO_OK;
+}
+
+/* ------------------------------------------------------------------ */
+/* Scaled dot-product attention (src/cpu/sdpa.cpp:132-336)              */
+/* ------------------------------------------------------------------ */
+
+/* The matrix-operand flush of src/cpu/sdpa.cpp:57-60: a nonzero magnitude below the
+ * smallest normal becomes a zero of the same sign. */
+static float matrix_daz(float v) {
+    return (v != 0.0f && fabsf(v) < 0x1p-126f) ? copysignf(0.0f, v) : v;
+}
+
+static float bf16_value(const iomo_view* v, uint64_t rows, uint64_t cols, uint64_t plane,
+                        uint64_t row, uint64_t col) {
+    const uint32_t bits = (uint32_t)load_leaf(v->base, iomo_plane_slot(rows, cols, plane, row, col), 16);
+    return f32_from_bits(bits << 16);
+}
+
+/* q [B..,Hq,R,D], k and v [B..,Hkv,C,D], out [B..,R,Hq*D]; BF16 only.  Per head and
+ * row, over the visible tokens t < min(L, a+r+1): score = (sum_d q*k in binary32,
+ * one product and one sum per increasing d) / sqrtf(D); the special rows and the
+ * max-subtracted softmax of src/cpu/sdpa.cpp:214-309 with the probability rounded
+ * once to BF16; out = sum_t P*V in binary32 per increasing t, -0 stored as +0, one
+ * BF16 rounding (src/cpu/sdpa.cpp:317-336).  Admission follows
+ * docs/BACKEND_CONTRACT/scaled-dot-product-attention.md:28-57 as far as it can be
+ * checked without owner identities. */
+int iomo_sdpa(int dtype, const iomo_view* q, const iomo_view* k, const iomo_view* v,
+              const iomo_view* out, uint64_t a, uint64_t L) {
+    if (!view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(out)) return IOMO_ERR_INVALID;
+    if (q->rank < 3 || k->rank != q->rank || v->rank != q->rank || out->rank != q->rank - 1)
+        return IOMO_ERR_INVALID;
+    const uint32_t leading = q->rank - 3;
+    const uint64_t Hq = q->dims[leading], R = view_rows(q), D = view_cols(q);
+    const uint64_t Hkv = k->dims[leading], C = view_rows(k);
+    if (view_cols(k) != D || v->dims[leading] != Hkv || view_rows(v) != C || view_cols(v) != D)
+        return IOMO_ERR_INVALID;
+    if (Hq == 0 || Hkv == 0 || Hq % Hkv != 0) return IOMO_ERR_INVALID;
+    if (view_rows(out) != R || view_cols(out) != Hq * D) return IOMO_ERR_INVALID;
+    for (uint32_t i = 0; i < leading; ++i)
+        if (k->dims[i] != q->dims[i] || v->dims[i] != q->dims[i] || out->dims[i] != q->dims[i])
+            return IOMO_ERR_INVALID;
+    if (L == 0 || L > C || a >= C || R > C - a) return IOMO_ERR_INVALID;
+    if (out->base == q->base || out->base == k->base || out->base == v->base) return IOMO_ERR_INVALID;
+    if (dtype != IOMO_DT_BF16) return IOMO_ERR_UNSUPPORTED;
+    const uint64_t grouping = Hq / Hkv;
+    const float scale = sqrtf((float)D);
+    float* score = (float*)malloc((size_t)L * sizeof(float));
+    uint16_t* prob = (uint16_t*)malloc((size_t)L * sizeof(uint16_t));
+    if (!score || !prob) { free(score); free(prob); return IOMO_ERR_INVALID; }
+    uint64_t coord[8] = {0};
+    do {
+        uint64_t qp = q->plane_offset, kp = k->plane_offset, vp = v->plane_offset, op = out->plane_offset;
+        for (uint32_t i = 0; i < leading; ++i) {
+            qp += coord[i] * q->plane_strides[i];
+            kp += coord[i] * k->plane_strides[i];
+            vp += coord[i] * v->plane_strides[i];
+            op += coord[i] * out->plane_strides[i];
+        }
+        for (uint64_t head = 0; head < Hq; ++head) {
+            const uint64_t qh = qp + head * q->plane_strides[leading];
+            const uint64_t kh = kp + (head / grouping) * k->plane_strides[leading];
+            const uint64_t vh = vp + (head / grouping) * v->plane_strides[leading];
+            for (uint64_t row = 0; row < R; ++row) {
+                const uint64_t visible = L < a + row + 1 ? L : a + row + 1;
+                int has_nan = 0, all_ninf = 1;
+                uint64_t pinf = 0;
+                for (uint64_t t = 0; t < visible; ++t) {
+                    float dot = 0.0f;
+                    for (uint64_t d = 0; d < D; ++d) {
+                        const volatile float product = matrix_daz(bf16_value(q, R, D, qh, row, d))
+                                * matrix_daz(bf16_value(k, C, D, kh, t, d));
+                        const volatile float next = dot + product;
+                        dot = next;
+                    }
+                    const volatile float scaled = dot / scale;
+                    score[t] = scaled;
+                    has_nan = has_nan || isnan(scaled);
+                    pinf += (scaled == INFINITY) ? 1 : 0;
+                    all_ninf = all_ninf && isinf(scaled) && signbit(scaled);
+                }
+                if (has_nan || all_ninf) {
+                    for (uint64_t f = 0; f < D; ++f)
+                        store_leaf(out->base, iomo_plane_slot(R, Hq * D, op, row, head * D + f), 16, 0x7FC0u);
+                    continue;
+                }
+                if (pinf != 0) {
+                    const volatile float p = 1.0f / (float)pinf;
+                    for (uint64_t t = 0; t < visible; ++t)
+                        prob[t] = iomo_encode_bf16(score[t] == INFINITY ? p : 0.0f);
+                } else {
+                    float maximum = -INFINITY;
+                    for (uint64_t t = 0; t < visible; ++t)
+                        if (score[t] > maximum) maximum = score[t];
+                    float sum = 0.0f;
+                    for (uint64_t t = 0; t < visible; ++t) {
+                        if (isinf(score[t]) && signbit(score[t])) { score[t] = 0.0f; continue; }
+                        const volatile float shifted = score[t] - maximum;
+                        const volatile float e = expf(shifted);
+                        const volatile float next = sum + e;
+                        sum = next;
+                        score[t] = e;
+                    }
+                    for (uint64_t t = 0; t < visible; ++t) {
+                        const volatile float normalized = score[t] / sum;
+                        prob[t] = iomo_encode_bf16(normalized);
+                    }
+                }
+                for (uint64_t f = 0; f < D; ++f) {
+                    float result = 0.0f;
+                    for (uint64_t t = 0; t < visible; ++t) {
+                        const volatile float product = matrix_daz(f32_from_bits((uint32_t)prob[t] << 16))
+                                * matrix_daz(bf16_value(v, C, D, vh, t, f));
+                        const volatile float next = result + product;
+                        result = next;
+                    }
+                    if (result == 0.0f) result = 0.0f;   /* -0 is stored as +0 */
+                    store_leaf(out->base, iomo_plane_slot(R, Hq * D, op, row, head * D + f), 16,
+                               iomo_encode_bf16(result));
+                }
+            }
+        }
+    } while (next_coord(coord, q->dims, leading));
+    free(score);
+    free(prob);
     return IOMO_OK;
 }
 

@@ -137,6 +137,13 @@ int iomo_linear(int dtype, const iomo_view* x, const iomo_view* w, const iomo_vi
                 uint64_t s, uint64_t R, int head_planar, uint64_t H, uint64_t D);
 
 /*
+ * Causal grouped-query attention, BF16 (src/cpu/sdpa.cpp:132-336): q [B..,Hq,R,D],
+ * k and v [B..,Hkv,C,D], out [B..,R,Hq*D]; row r sees tokens t < min(L, a+r+1).
+ */
+int iomo_sdpa(int dtype, const iomo_view* q, const iomo_view* k, const iomo_view* v,
+              const iomo_view* out, uint64_t a, uint64_t L);
+
+/*
  * Softmax stage.  Request shape follows src/rocm/sdpa_softmax.hpp:14-62
  * (strides in elements); arithmetic follows src/cpu/sdpa.cpp:214-309 with
  * scaled = score * scale as in src/rocm/sdpa_softmax.hip:131-132.

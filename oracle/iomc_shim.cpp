@@ -30,6 +30,10 @@
 #include "iom/iom.hpp"
 #include "iom/tensor.hpp"
 #include "src/iom_internal.hpp"  // iom::detail::UnsupportedOperation
+#ifndef IOMC_WITH_MI355X
+// The reference's own backend-free attention reference and fixture corpus.
+#include "test/backend/backend_conformance_sdpa_reference.hpp"
+#endif
 #ifdef IOMC_WITH_MI355X
 #include "iom/rocm/device.hpp"
 #endif
@@ -399,6 +403,71 @@ std::int64_t iomc_embedding(
         return classify(std::current_exception());
     }
 }
+
+#ifndef IOMC_WITH_MI355X
+// The fixed attention fixtures of test/backend/backend_conformance_sdpa_reference.hpp
+// (sdpa_reference_cases, :1267-1299), their expected values (evaluate, :988) and the
+// comparison rule (matches, :1232-1259), for writing golden vectors.
+namespace {
+const std::vector<iom_conformance::SdpaReferenceCase>& sdpa_cases() {
+    static const std::vector<iom_conformance::SdpaReferenceCase> cases =
+            iom_conformance::sdpa_reference_cases(iom::DataType::BF16);
+    return cases;
+}
+}  // namespace
+
+int iomc_sdpa_case_count() { return static_cast<int>(sdpa_cases().size()); }
+
+// info: kind, leading rank, 4 leading dimensions, Hq, Hkv, R, D, C, a, L, padding salt
+int iomc_sdpa_case_info(int index, std::uint64_t* info, char* label, std::size_t label_size) {
+    if (index < 0 || index >= iomc_sdpa_case_count()) return -1;
+    const auto& c = sdpa_cases()[static_cast<std::size_t>(index)];
+    if (c.leading_dimensions.size() > 4) return -1;
+    info[0] = static_cast<std::uint64_t>(c.kind);
+    info[1] = c.leading_dimensions.size();
+    for (std::size_t i = 0; i < 4; ++i) info[2 + i] = i < c.leading_dimensions.size() ? c.leading_dimensions[i] : 1;
+    info[6] = c.hq; info[7] = c.hkv; info[8] = c.rows; info[9] = c.head_dim;
+    info[10] = c.capacity; info[11] = c.position; info[12] = c.length;
+    info[13] = c.physical_padding_salt;
+    info[14] = c.q_bits.size(); info[15] = c.k_bits.size(); info[16] = c.v_bits.size();
+    const std::string text = iom_conformance::sdpa_reference_case_label(c);
+    std::strncpy(label, text.c_str(), label_size - 1);
+    label[label_size - 1] = 0;
+    return 0;
+}
+
+int iomc_sdpa_case_data(int index, std::uint16_t* q, std::uint16_t* k, std::uint16_t* v) {
+    if (index < 0 || index >= iomc_sdpa_case_count()) return -1;
+    const auto& c = sdpa_cases()[static_cast<std::size_t>(index)];
+    for (std::size_t i = 0; i < c.q_bits.size(); ++i) q[i] = static_cast<std::uint16_t>(c.q_bits[i]);
+    for (std::size_t i = 0; i < c.k_bits.size(); ++i) k[i] = static_cast<std::uint16_t>(c.k_bits[i]);
+    for (std::size_t i = 0; i < c.v_bits.size(); ++i) v[i] = static_cast<std::uint16_t>(c.v_bits[i]);
+    return 0;
+}
+
+// Expected output [B..., R, Hq*D] row-major: raw bits and value class per element.
+std::int64_t iomc_sdpa_case_expected(int index, std::uint16_t* bits, std::uint8_t* classes, std::size_t capacity) {
+    if (index < 0 || index >= iomc_sdpa_case_count()) return -1;
+    try {
+        const auto values = iom_conformance::evaluate(sdpa_cases()[static_cast<std::size_t>(index)]);
+        if (values.size() > capacity) return -static_cast<std::int64_t>(values.size());
+        for (std::size_t i = 0; i < values.size(); ++i) {
+            bits[i] = static_cast<std::uint16_t>(values[i].bits);
+            classes[i] = static_cast<std::uint8_t>(values[i].value_class);
+        }
+        return static_cast<std::int64_t>(values.size());
+    } catch (...) {
+        return classify(std::current_exception());
+    }
+}
+
+int iomc_sdpa_matches(std::uint16_t actual, std::uint16_t expected_bits, std::uint8_t expected_class) {
+    iom_conformance::SdpaReferenceValue expected;
+    expected.bits = expected_bits;
+    expected.value_class = static_cast<iom_conformance::SdpaReferenceClass>(expected_class);
+    return iom_conformance::matches(iom::DataType::BF16, static_cast<std::uint64_t>(actual), expected) ? 1 : 0;
+}
+#endif
 
 int iomc_wait(iomc_queue* queue, std::int64_t token) {
     return guarded_status([&] { queue->ops->wait(token); });

@@ -136,6 +136,7 @@ def lib() -> C.CDLL:
         l.iomo_embedding.argtypes = [C.c_int, C.c_int, VP, VP, VP]
         l.iomo_rope.argtypes = [C.c_int, VP, VP, C.c_uint64, C.c_double]
         l.iomo_linear.argtypes = [C.c_int, VP, VP, VP, C.c_uint64, C.c_uint64, C.c_int, C.c_uint64, C.c_uint64]
+        l.iomo_sdpa.argtypes = [C.c_int, VP, VP, VP, VP, C.c_uint64, C.c_uint64]
         _lib = l
     return _lib
 
@@ -344,6 +345,11 @@ def linear(x: HostView, w: HostView, out: HostView, s: int, R: int, head_planar:
     return lib().iomo_linear(out.dtype, C.byref(a), C.byref(b), C.byref(o), s, R, int(head_planar), H, D)
 
 
+def sdpa(q: HostView, k: HostView, v: HostView, out: HostView, a: int, L: int) -> int:
+    cq, ck, cv, co = q.cview(), k.cview(), v.cview(), out.cview()
+    return lib().iomo_sdpa(out.dtype, C.byref(cq), C.byref(ck), C.byref(cv), C.byref(co), a, L)
+
+
 def dense_layout(heads: int, rows: int, cols: int) -> StageLayout:
     l = StageLayout()
     l.plane_offset = 0
@@ -448,6 +454,13 @@ def bind_iomc(l: C.CDLL) -> C.CDLL:
     l.iomc_rmsnorm.argtypes = [P, P, P, P, C.c_float]
     l.iomc_silu.restype = C.c_int64
     l.iomc_silu.argtypes = [P, P, P]
+    if hasattr(l, "iomc_sdpa_case_count"):
+        U16P, U8P = C.POINTER(C.c_uint16), C.POINTER(C.c_uint8)
+        l.iomc_sdpa_case_info.argtypes = [C.c_int, U64P, C.c_char_p, C.c_size_t]
+        l.iomc_sdpa_case_data.argtypes = [C.c_int, U16P, U16P, U16P]
+        l.iomc_sdpa_case_expected.restype = C.c_int64
+        l.iomc_sdpa_case_expected.argtypes = [C.c_int, U16P, U8P, C.c_size_t]
+        l.iomc_sdpa_matches.argtypes = [C.c_uint16, C.c_uint16, C.c_uint8]
     l.iomc_sdpa.restype = C.c_int64
     l.iomc_sdpa.argtypes = [P, P, P, P, P, P, C.c_size_t, C.c_size_t]
     l.iomc_wait.argtypes = [P, C.c_int64]
