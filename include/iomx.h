@@ -258,6 +258,34 @@ int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const 
                        uint64_t s, uint64_t R, int head_planar, uint64_t H, uint64_t D, int path,
                        iomx_stream_t stream);
 
+/*
+ * Causal grouped-query attention: q [B..,Hq,R,D], k and v [B..,Hkv,C,D] (Hq % Hkv
+ * == 0, kv head of h = h / (Hq/Hkv)), out [B..,R,Hq*D]; row r attends to the
+ * tokens t < min(L, a+r+1) of the initialised prefix L <= C.  Replaces the attention
+ * kernels behind DeviceOps::sdpa_impl (include/iom/iom.hpp:368-373,913-922; the
+ * reference's ROCm chain src/rocm/sdpa*.hip is wave32 WMMA for gfx12 only).
+ * Contract docs/BACKEND_CONTRACT/scaled-dot-product-attention.md, arithmetic of
+ * src/cpu/sdpa.cpp:186-336: BF16 only (any other leaf -2); scores in F32 divided by
+ * sqrtf(D); NaN / +inf / all -inf rows by the special-row rules; the normalised
+ * probability rounded once to BF16; P x V in F32, -0 stored as +0, one BF16
+ * rounding; subnormal Q, K, P and V operands flushed to signed zero; the cache
+ * tail [L,C), future tokens and tile padding are never read.
+ *
+ * iomx_sdpa_workspace is the pure requirement query (sdpa_workspace_requirements):
+ * the bytes and alignment of caller workspace iomx_launch_sdpa needs for these
+ * operands (the transposed copy of the visible V prefix and one flag word; 0 when D
+ * exceeds what the matrix-core kernel covers).  path 0 runs the matrix-core kernel
+ * (D <= 128) followed by the reference-order kernel, which returns at once unless V
+ * holds an infinity or NaN; path 1 runs the reference-order kernel alone (D <= 256,
+ * no workspace).
+ */
+int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
+                        const iomx_view* out, uint64_t a, uint64_t L, uint64_t* bytes,
+                        uint64_t* alignment);
+int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
+                     const iomx_view* out, uint64_t a, uint64_t L, void* workspace,
+                     uint64_t workspace_bytes, int path, iomx_stream_t stream);
+
 /* Element strides of one softmax-stage buffer (src/rocm/sdpa_softmax.hpp:14-22). */
 typedef struct iomx_stage_layout {
     uint64_t plane_offset, plane_stride, head_stride, row_stride, column_stride;

@@ -27,6 +27,7 @@ SOURCES = [
     "iomx_leaves.hip",
     "iomx_layer.hip",
     "iomx_linear.hip",
+    "iomx_sdpa.hip",
 ]
 
 # -ffp-contract=off: no fused multiply-add may replace the reference's two

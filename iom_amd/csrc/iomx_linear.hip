@@ -20,6 +20,7 @@
 //                    CU streams weights) and linear_mfma_lds (256 rows or more:
 //                    256x256 workgroup tiles staged through LDS).
 #include "iomx_rows.hpp"
+#include "iomx_mfma.hpp"
 #include <type_traits>
 
 namespace iomx {
@@ -157,26 +158,6 @@ __global__ __launch_bounds__(256) void linear_rows_kernel(const LinearArgs a) {
 // ---------------------------------------------------------------------------
 // BF16 on the matrix cores
 // ---------------------------------------------------------------------------
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-
-// Eight consecutive BF16 of one tile row starting at column c0 (0 or 8), inner
-// indices i0..i0+7, zero where the inner index is past I (tile padding is never
-// an operand).
-__device__ __forceinline__ bf16x8_t load_k8(const uint8_t* tile_row, uint32_t c0, uint32_t i0, uint32_t I) {
-    u32x4 v = {0, 0, 0, 0};
-    if (i0 + 8 <= I) {
-        v = *reinterpret_cast<const u32x4*>(tile_row + c0 * 2);
-    } else if (i0 < I) {
-        uint32_t h[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            h[j] = (i0 + j < I) ? *reinterpret_cast<const uint16_t*>(tile_row + (c0 + j) * 2) : 0u;
-        v = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
-    }
-    return __builtin_bit_cast(bf16x8_t, v);
-}
 
 // The rows of every plane form one row axis (row index = plane * R + r), so a
 // decode step of many sequences fills whole row tiles and reads the weight once.

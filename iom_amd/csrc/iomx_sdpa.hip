@@ -1,0 +1,509 @@
+// Causal grouped-query attention, BF16: q [B..,Hq,R,D], k and v [B..,Hkv,C,D],
+// out [B..,R,Hq*D]; row r sees tokens t < min(L, a+r+1).
+//
+//   sdpa_pack_v     V of the visible prefix, transposed into matrix-core operand
+//                   fragments in the caller's workspace (subnormals flushed to signed
+//                   zero, zeros past L and past D), and a flag raised when a V value
+//                   of the prefix is infinite or NaN.
+//   sdpa_mfma       one wave = one head x 16 rows.  Pass 1 forms the scores
+//                   (K tile x Q tile on the matrix cores, binary32) and the row's
+//                   maximum and sum of exponentials; pass 2 forms them again, turns
+//                   them into the normalised probability rounded once to BF16, and
+//                   multiplies by the packed V fragments (binary32 accumulation),
+//                   one BF16 rounding at the store.  Scores never leave registers.
+//   sdpa_rows       the scalar recurrence in the reference's order (one wave per
+//                   row: sequential sums over features and over tokens).  It runs
+//                   after sdpa_mfma and returns at once unless the flag is up: a
+//                   masked probability is +0, and +0 times an infinite V of a token
+//                   the row must not see would poison the row on the matrix cores.
+//                   It is also the path for head sizes the fragments do not cover.
+#include "iomx_mfma.hpp"
+
+namespace iomx {
+
+struct SdpaArgs {
+    const uint8_t* q;
+    const uint8_t* k;
+    const uint8_t* v;
+    uint8_t* out;
+    PlaneWalk<4> walk;          // 0 q, 1 k, 2 v, 3 out: the shared leading tuple
+    uint64_t q_plane_bytes, kv_plane_bytes, out_plane_bytes;
+    uint64_t q_head_stride, k_head_stride, v_head_stride;   // owner planes per head
+    uint32_t Hq, Hkv, grouping, R, C, D, a, L;
+    uint32_t d_tiles, out_tile_cols, kv_tile_rows;
+    uint32_t planes, groups;    // leading planes; 32-token groups of the prefix
+    uint8_t* packed_v;          // [plane][kv head][group][d tile] fragments of 1 KiB
+    uint32_t* flag;             // nonzero: the prefix of V holds an infinity or NaN
+    uint32_t guarded;           // sdpa_rows: return unless the flag is up
+    float scale;                // sqrtf(D)
+};
+
+constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
+
+__global__ void sdpa_clear_flag_kernel(uint32_t* flag) { *flag = 0u; }
+
+// Subnormal operands of the matrix stages become zeros of the same sign
+// (src/cpu/sdpa.cpp:57-60), two BF16 per word.
+__device__ __forceinline__ uint32_t daz2(uint32_t w) {
+    const uint32_t lo = (w & 0x00007F80u) ? 0x0000FFFFu : 0x00008000u;
+    const uint32_t hi = (w & 0x7F800000u) ? 0xFFFF0000u : 0x80000000u;
+    return w & (lo | hi);
+}
+__device__ __forceinline__ bf16x8_t daz8(u32x4 v) {
+    return __builtin_bit_cast(bf16x8_t, u32x4{daz2(v[0]), daz2(v[1]), daz2(v[2]), daz2(v[3])});
+}
+__device__ __forceinline__ float daz_bf16(uint32_t h) {
+    return as_f32(((h & 0x7F80u) ? h : (h & 0x8000u)) << 16);
+}
+
+// Fragment (group g, d tile dt) holds, for lane (d = l%16, kg = l/16), the eight
+// values V[32g + 4kg + j][16dt + d] (j < 4) and V[32g + 16 + 4kg + j][16dt + d]:
+// the token order in which a lane of sdpa_mfma holds its probabilities.
+__global__ __launch_bounds__(256) void sdpa_pack_v_kernel(const SdpaArgs a) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t frag = blockIdx.x * 4 + wave;
+    if (frag >= a.groups * a.d_tiles) return;
+    const uint32_t g = frag / a.d_tiles, dt = frag - g * a.d_tiles;
+    const uint32_t l16 = lane & 15u, kg = lane >> 4;
+    const uint32_t d = dt * kTile + l16;
+    const uint32_t hkv = blockIdx.y;
+    for (uint32_t p = blockIdx.z; p < a.planes; p += gridDim.z) {
+        uint64_t plane[4];
+        walk_planes(a.walk, p, plane);
+        const uint8_t* vb = a.v + (plane[2] + (uint64_t)hkv * a.v_head_stride) * a.kv_plane_bytes;
+        uint32_t h[8];
+        bool special = false;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t token = 32 * g + (j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4));
+            uint32_t bits = 0;
+            if (token < a.L && d < a.D) {
+                bits = *reinterpret_cast<const uint16_t*>(
+                        vb + ((uint64_t)(token >> 4) * a.d_tiles + dt) * kTileBytes + (token & 15u) * kRowBytes + l16 * 2);
+                special = special || (bits & 0x7F80u) == 0x7F80u;
+                if ((bits & 0x7F80u) == 0) bits &= 0x8000u;
+            }
+            h[j] = bits;
+        }
+        uint8_t* dst = a.packed_v + ((((uint64_t)p * a.Hkv + hkv) * a.groups + g) * a.d_tiles + dt) * kFrag + lane * 16;
+        *reinterpret_cast<u32x4*>(dst) = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16),
+                                               h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+        if (special) atomicOr(a.flag, 1u);
+    }
+}
+
+// Running maximum and sum of exp(score - maximum) over the finite scores of a row,
+// and what the special rows need (docs/BACKEND_CONTRACT/scaled-dot-product-attention.md:
+// "Formed-score special values").
+struct RowStats {
+    float m, sum;
+    uint32_t pinf;
+    bool nan, finite;
+    __device__ __forceinline__ void add(float s) {
+        if (s != s) nan = true;
+        else if (s == __builtin_inff()) ++pinf;
+        else if (s != -__builtin_inff()) {
+            finite = true;
+            if (s > m) { sum *= expf(m - s); m = s; }
+            sum += expf(s - m);
+        }
+    }
+    __device__ __forceinline__ void merge(float m2, float sum2, uint32_t pinf2, bool nan2, bool finite2) {
+        const float mm = m > m2 ? m : m2;
+        if (mm == -__builtin_inff()) sum = 0.0f;
+        else sum = sum * expf(m - mm) + sum2 * expf(m2 - mm);
+        m = mm;
+        pinf += pinf2;
+        nan = nan || nan2;
+        finite = finite || finite2;
+    }
+};
+
+template <int DT16>
+__global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
+    constexpr int D32 = (DT16 + 1) / 2;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t l16 = lane & 15u, kg = lane >> 4;
+    const uint32_t head = blockIdx.y * 4 + wave;
+    if (head >= a.Hq) return;
+    const uint32_t hkv = head / a.grouping;
+    const uint32_t r0 = blockIdx.x * kTile;
+    const uint32_t row = r0 + l16;
+    const bool row_ok = row < a.R;
+    const uint32_t qrow = row_ok ? row : a.R - 1;
+    const uint32_t last_row = r0 + 15 < a.R ? r0 + 15 : a.R - 1;
+    const uint32_t reach = a.a + row + 1, reach_max = a.a + last_row + 1;
+    const uint32_t vis = row_ok ? (reach < a.L ? reach : a.L) : 0;     // tokens this lane's row sees
+    const uint32_t vis_max = reach_max < a.L ? reach_max : a.L;        // ... and the wave's last row
+    const uint32_t groups = (vis_max + 31) / 32;
+    const uint32_t c0 = (kg & 1u) * 8u;
+    const float inf = __builtin_inff();
+    for (uint32_t p = blockIdx.z; p < a.planes; p += gridDim.z) {
+        uint64_t plane[4];
+        walk_planes(a.walk, p, plane);
+        const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
+        const uint8_t* kb = a.k + (plane[1] + (uint64_t)hkv * a.k_head_stride) * a.kv_plane_bytes;
+        const uint8_t* vf = a.packed_v + (((uint64_t)p * a.Hkv + hkv) * a.groups) * a.d_tiles * kFrag + lane * 16;
+        // the row tile of Q, flushed, as the B operand of every score tile
+        bf16x8_t qf[D32];
+#pragma unroll
+        for (int c = 0; c < D32; ++c) {
+            const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
+            qf[c] = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
+            if (i0 < a.D)
+                qf[c] = daz8(load_k8_bits(qb + ((uint64_t)(qrow >> 4) * a.d_tiles + tile) * kTileBytes
+                                                  + (qrow & 15u) * kRowBytes, c0, i0, a.D));
+        }
+        // scores of the 16 tokens from t0 against the 16 rows: lane gets token
+        // t0 + 4*kg + j (j < 4) of row l16.  Tokens past the prefix read its last
+        // token instead (the cache tail is never touched); their scores are dropped.
+        auto scores = [&](uint32_t t0) {
+            uint32_t token = t0 + l16;
+            if (token >= a.L) token = a.L - 1;
+            const uint8_t* krow = kb + (uint64_t)(token >> 4) * a.d_tiles * kTileBytes + (token & 15u) * kRowBytes;
+            f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int c = 0; c < D32; ++c) {
+                const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
+                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
+                if (i0 < a.D) kf = daz8(load_k8_bits(krow + (uint64_t)tile * kTileBytes, c0, i0, a.D));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = acc[j] / a.scale;
+            return acc;
+        };
+        // pass 1: the row's statistics
+        RowStats st = {-inf, 0.0f, 0u, false, false};
+        for (uint32_t g = 0; g < groups; ++g) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const uint32_t t0 = 32 * g + 16 * half;
+                if (t0 >= vis_max) continue;
+                const f32x4_t s = scores(t0);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (t0 + 4 * kg + j < vis) st.add(s[j]);
+            }
+        }
+#pragma unroll
+        for (int off = 16; off <= 32; off *= 2) {
+            const float m2 = __shfl_xor(st.m, off), s2 = __shfl_xor(st.sum, off);
+            const uint32_t p2 = __shfl_xor(st.pinf, off);
+            const int n2 = __shfl_xor((int)st.nan, off), f2 = __shfl_xor((int)st.finite, off);
+            st.merge(m2, s2, p2, n2 != 0, f2 != 0);
+        }
+        const bool nan_row = st.nan || (st.pinf == 0 && !st.finite);      // NaN score or all -inf
+        const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
+        // pass 2: probabilities, rounded once to BF16, times V
+        f32x4_t o[DT16];
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (uint32_t g = 0; g < groups; ++g) {
+            uint32_t pb[8];
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const uint32_t t0 = 32 * g + 16 * half;
+                f32x4_t s = {-inf, -inf, -inf, -inf};
+                if (t0 < vis_max) s = scores(t0);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float pr = 0.0f;
+                    if (t0 + 4 * kg + j < vis && !nan_row) {
+                        if (st.pinf) pr = s[j] == inf ? pinf_p : 0.0f;
+                        else if (s[j] != -inf) pr = expf(s[j] - st.m) / st.sum;
+                    }
+                    uint32_t h = bf16_rne_sw(as_u32(pr));
+                    if ((h & 0x7F80u) == 0) h = 0;                  // flushed before the product; p >= 0
+                    pb[half * 4 + j] = h;
+                }
+            }
+            const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, u32x4{pb[0] | (pb[1] << 16), pb[2] | (pb[3] << 16),
+                                                                   pb[4] | (pb[5] << 16), pb[6] | (pb[7] << 16)});
+#pragma unroll
+            for (int dt = 0; dt < DT16; ++dt) {
+                const bf16x8_t vfr = __builtin_bit_cast(bf16x8_t,
+                        *reinterpret_cast<const u32x4*>(vf + ((uint64_t)g * a.d_tiles + dt) * kFrag));
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfr, pf, o[dt], 0, 0, 0);
+            }
+        }
+        // lane holds out[row][head*D + 16*dt + 4*kg + j]
+        if (!row_ok) continue;
+        uint8_t* ob = a.out + plane[3] * a.out_plane_bytes
+                + (uint64_t)(row >> 4) * a.out_tile_cols * kTileBytes + (row & 15u) * kRowBytes;
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t d = dt * kTile + 4 * kg + j;
+                if (d >= a.D) continue;
+                float val = o[dt][j];
+                if (val == 0.0f) val = 0.0f;                          // -0 is stored as +0
+                const uint32_t bits = nan_row ? 0x7FC0u : bf16_rne_sw(as_u32(val));
+                const uint32_t col = head * a.D + d;
+                *reinterpret_cast<uint16_t*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) = (uint16_t)bits;
+            }
+        }
+    }
+}
+
+// One wave per (row, head, plane), the arithmetic and the order of
+// src/cpu/sdpa.cpp:186-336: every score a sequential sum over the features, the sum
+// of exponentials sequential over the tokens, every output a sequential sum over
+// the tokens; lanes only divide the tokens (scores) or the features (outputs).
+__global__ __launch_bounds__(64) void sdpa_rows_kernel(const SdpaArgs a) {
+    __shared__ float pbuf[64];
+    if (a.guarded && *a.flag == 0u) return;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t row = blockIdx.x, head = blockIdx.y;
+    const uint32_t hkv = head / a.grouping;
+    const uint32_t reach = a.a + row + 1;
+    const uint32_t vis = reach < a.L ? reach : a.L;
+    const float inf = __builtin_inff();
+    for (uint32_t p = blockIdx.z; p < a.planes; p += gridDim.z) {
+        uint64_t plane[4];
+        walk_planes(a.walk, p, plane);
+        const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes
+                + (uint64_t)(row >> 4) * a.d_tiles * kTileBytes + (row & 15u) * kRowBytes;
+        const uint8_t* kb = a.k + (plane[1] + (uint64_t)hkv * a.k_head_stride) * a.kv_plane_bytes;
+        const uint8_t* vb = a.v + (plane[2] + (uint64_t)hkv * a.v_head_stride) * a.kv_plane_bytes;
+        auto element = [&](const uint8_t* row_base, uint32_t d) {
+            return daz_bf16(*reinterpret_cast<const uint16_t*>(row_base + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2));
+        };
+        auto score = [&](uint32_t t) {
+            const uint8_t* kr = kb + (uint64_t)(t >> 4) * a.d_tiles * kTileBytes + (t & 15u) * kRowBytes;
+            float dot = 0.0f;
+            for (uint32_t d = 0; d < a.D; ++d) dot = dot + element(qb, d) * element(kr, d);   // products are exact
+            return dot / a.scale;
+        };
+        // classes and maximum
+        float m = -inf;
+        uint32_t pinf = 0;
+        bool nan = false, not_ninf = false;
+        for (uint32_t t = lane; t < vis; t += 64) {
+            const float s = score(t);
+            nan = nan || s != s;
+            pinf += s == inf ? 1u : 0u;
+            not_ninf = not_ninf || s != -inf;
+            if (s > m) m = s;
+        }
+#pragma unroll
+        for (int off = 1; off < 64; off *= 2) {
+            // every lane takes part in every exchange (no short-circuit around a shuffle)
+            const float m2 = __shfl_xor(m, off);
+            const uint32_t p2 = __shfl_xor(pinf, off);
+            const int n2 = __shfl_xor((int)nan, off), f2 = __shfl_xor((int)not_ninf, off);
+            m = m2 > m ? m2 : m;
+            pinf += p2;
+            nan = nan || n2 != 0;
+            not_ninf = not_ninf || f2 != 0;
+        }
+        uint8_t* ob = a.out + plane[3] * a.out_plane_bytes
+                + (uint64_t)(row >> 4) * a.out_tile_cols * kTileBytes + (row & 15u) * kRowBytes;
+        auto store = [&](uint32_t d, uint32_t bits) {
+            const uint32_t col = head * a.D + d;
+            *reinterpret_cast<uint16_t*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) = (uint16_t)bits;
+        };
+        if (nan || !not_ninf) {
+            for (uint32_t d = lane; d < a.D; d += 64) store(d, 0x7FC0u);
+            continue;
+        }
+        // sum of exponentials in token order
+        float sum = 0.0f;
+        if (pinf == 0) {
+            for (uint32_t t0 = 0; t0 < vis; t0 += 64) {
+                const uint32_t t = t0 + lane;
+                float e = 0.0f;
+                if (t < vis) {
+                    const float s = score(t);
+                    if (s != -inf) e = expf(s - m);
+                }
+                for (int i = 0; i < 64; ++i) sum = sum + __shfl(e, i);     // adding +0 changes nothing
+            }
+        }
+        const float pinf_p = pinf ? 1.0f / (float)pinf : 0.0f;
+        // out = sum over tokens of P * V, features over lanes (up to 256)
+        float result[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (uint32_t t0 = 0; t0 < vis; t0 += 64) {
+            const uint32_t t = t0 + lane;
+            float pr = 0.0f;
+            if (t < vis) {
+                const float s = score(t);
+                if (pinf) pr = s == inf ? pinf_p : 0.0f;
+                else if (s != -inf) pr = expf(s - m) / sum;
+            }
+            __syncthreads();
+            pbuf[lane] = daz_bf16(bf16_rne_sw(as_u32(pr)));
+            __syncthreads();
+            const uint32_t n = vis - t0 < 64 ? vis - t0 : 64;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t d = lane + 64 * c;
+                if (d >= a.D) continue;
+                for (uint32_t i = 0; i < n; ++i) {
+                    const uint32_t tt = t0 + i;
+                    const uint8_t* vr = vb + (uint64_t)(tt >> 4) * a.d_tiles * kTileBytes + (tt & 15u) * kRowBytes;
+                    result[c] = result[c] + pbuf[i] * element(vr, d);             // products are exact
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t d = lane + 64 * c;
+            if (d >= a.D) continue;
+            float val = result[c];
+            if (val == 0.0f) val = 0.0f;
+            store(d, bf16_rne_sw(as_u32(val)));
+        }
+    }
+}
+
+namespace {
+
+struct SdpaShape {
+    uint64_t Hq, Hkv, R, C, D, planes;
+    uint32_t leading;
+};
+
+int sdpa_shape(const iomx_view* q, const iomx_view* k, const iomx_view* v, const iomx_view* out,
+               uint64_t a, uint64_t L, SdpaShape* s) {
+    IOMX_TRY(check_view(q, 16));
+    IOMX_TRY(check_view(k, 16));
+    IOMX_TRY(check_view(v, 16));
+    IOMX_TRY(check_view(out, 16));
+    if (q->rank < 3 || k->rank != q->rank || v->rank != q->rank || out->rank != q->rank - 1) return IOMX_ERR_INVALID;
+    const uint32_t leading = q->rank - 3;
+    const Matrix qm = matrix_of(*q), km = matrix_of(*k), vm = matrix_of(*v), om = matrix_of(*out);
+    s->leading = leading;
+    s->Hq = q->dims[leading];
+    s->Hkv = k->dims[leading];
+    s->R = qm.rows;
+    s->D = qm.cols;
+    s->C = km.rows;
+    if (km.cols != s->D || v->dims[leading] != s->Hkv || vm.rows != s->C || vm.cols != s->D) return IOMX_ERR_INVALID;
+    if (s->Hq == 0 || s->Hkv == 0 || s->Hq % s->Hkv != 0) return IOMX_ERR_INVALID;
+    uint64_t width;
+    if (mul_overflows(s->Hq, s->D, &width) || om.rows != s->R || om.cols != width) return IOMX_ERR_INVALID;
+    s->planes = 1;
+    for (uint32_t i = 0; i < leading; ++i) {
+        if (k->dims[i] != q->dims[i] || v->dims[i] != q->dims[i] || out->dims[i] != q->dims[i]) return IOMX_ERR_INVALID;
+        if (mul_overflows(s->planes, q->dims[i], &s->planes)) return IOMX_ERR_OVERFLOW;
+    }
+    if (L == 0 || L > s->C || a >= s->C || s->R > s->C - a) return IOMX_ERR_INVALID;
+    if (out->base == q->base || out->base == k->base || out->base == v->base) return IOMX_ERR_INVALID;
+    if (s->C > 0x7FFFFFF0ull || width > 0x7FFFFFF0ull || s->planes > 0x7FFFFFF0ull) return IOMX_ERR_OVERFLOW;
+    return IOMX_OK;
+}
+
+constexpr uint64_t kSdpaHeader = 256;   // the flag word, padded so that the fragments stay aligned
+constexpr uint64_t kMaxMfmaHeadDim = 128;
+
+int sdpa_packed_bytes(const SdpaShape& s, uint64_t L, uint64_t* bytes) {
+    uint64_t n = s.planes;
+    if (mul_overflows(n, s.Hkv, &n) || mul_overflows(n, (L + 31) / 32, &n)
+        || mul_overflows(n, (s.D + 15) / 16, &n) || mul_overflows(n, (uint64_t)kFrag, &n)
+        || n > ~0ull - kSdpaHeader)
+        return IOMX_ERR_OVERFLOW;
+    *bytes = n + kSdpaHeader;
+    return IOMX_OK;
+}
+
+}  // namespace
+
+}  // namespace iomx
+
+using namespace iomx;
+
+extern "C" int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
+                                   const iomx_view* out, uint64_t a, uint64_t L, uint64_t* bytes,
+                                   uint64_t* alignment) {
+    if (!bytes || !alignment) return IOMX_ERR_INVALID;
+    SdpaShape s;
+    IOMX_TRY(sdpa_shape(q, k, v, out, a, L, &s));
+    if (dtype != IOMX_DT_BF16) return IOMX_ERR_UNSUPPORTED;
+    *alignment = 256;
+    if (s.D > kMaxMfmaHeadDim) { *bytes = 0; *alignment = 1; return IOMX_OK; }
+    return sdpa_packed_bytes(s, L, bytes);
+}
+
+extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
+                                const iomx_view* out, uint64_t a, uint64_t L, void* workspace,
+                                uint64_t workspace_bytes, int path, iomx_stream_t stream) {
+    SdpaShape s;
+    IOMX_TRY(sdpa_shape(q, k, v, out, a, L, &s));
+    if (dtype != IOMX_DT_BF16) return IOMX_ERR_UNSUPPORTED;
+    if (s.D > 256) return IOMX_ERR_UNSUPPORTED;
+    const Matrix qm = matrix_of(*q), km = matrix_of(*k), om = matrix_of(*out);
+    SdpaArgs g = {};
+    uint64_t strides[4][kMaxLead] = {};
+    uint64_t offsets[4] = {q->plane_offset, k->plane_offset, v->plane_offset, out->plane_offset};
+    for (uint32_t i = 0; i < s.leading; ++i) {
+        strides[0][i] = q->plane_strides[i];
+        strides[1][i] = k->plane_strides[i];
+        strides[2][i] = v->plane_strides[i];
+        strides[3][i] = out->plane_strides[i];
+    }
+    IOMX_TRY(build_walk<4>(s.leading, q->dims, strides, offsets, &g.walk));
+    g.q = static_cast<const uint8_t*>(q->base);
+    g.k = static_cast<const uint8_t*>(k->base);
+    g.v = static_cast<const uint8_t*>(v->base);
+    g.out = static_cast<uint8_t*>(out->base);
+    g.q_plane_bytes = qm.plane_elems * 2;
+    g.kv_plane_bytes = km.plane_elems * 2;
+    g.out_plane_bytes = om.plane_elems * 2;
+    g.q_head_stride = q->plane_strides[s.leading];
+    g.k_head_stride = k->plane_strides[s.leading];
+    g.v_head_stride = v->plane_strides[s.leading];
+    g.Hq = (uint32_t)s.Hq;
+    g.Hkv = (uint32_t)s.Hkv;
+    g.grouping = (uint32_t)(s.Hq / s.Hkv);
+    g.R = (uint32_t)s.R;
+    g.C = (uint32_t)s.C;
+    g.D = (uint32_t)s.D;
+    g.a = (uint32_t)a;
+    g.L = (uint32_t)L;
+    g.d_tiles = (uint32_t)qm.tile_cols;
+    g.out_tile_cols = (uint32_t)om.tile_cols;
+    g.kv_tile_rows = (uint32_t)km.tile_rows;
+    g.planes = (uint32_t)g.walk.planes;
+    g.groups = (uint32_t)((L + 31) / 32);
+    g.scale = sqrtf((float)s.D);
+    if (s.Hq > 65535u || s.R > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
+    const hipStream_t st = native(stream);
+    const uint32_t gz = g.planes < 65535u ? g.planes : 65535u;
+
+    bool matrix_cores = path == 0 && s.D <= kMaxMfmaHeadDim;
+    if (matrix_cores) {
+        uint64_t need;
+        IOMX_TRY(sdpa_packed_bytes(s, L, &need));
+        if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+            return IOMX_ERR_INVALID;
+        if (s.Hkv > 65535u) matrix_cores = false;
+    }
+    if (matrix_cores) {
+        g.flag = static_cast<uint32_t*>(workspace);
+        g.packed_v = static_cast<uint8_t*>(workspace) + kSdpaHeader;
+        hipLaunchKernelGGL(sdpa_clear_flag_kernel, dim3(1), dim3(1), 0, st, g.flag);
+        const uint32_t frags = g.groups * g.d_tiles;
+        hipLaunchKernelGGL(sdpa_pack_v_kernel, dim3((frags + 3) / 4, g.Hkv, gz), dim3(256), 0, st, g);
+        const dim3 grid((g.R + kTile - 1) / kTile, (g.Hq + 3) / 4, gz);
+        switch (g.d_tiles) {
+            case 1: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<1>), grid, dim3(256), 0, st, g); break;
+            case 2: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<2>), grid, dim3(256), 0, st, g); break;
+            case 3: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<3>), grid, dim3(256), 0, st, g); break;
+            case 4: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<4>), grid, dim3(256), 0, st, g); break;
+            case 5: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<5>), grid, dim3(256), 0, st, g); break;
+            case 6: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<6>), grid, dim3(256), 0, st, g); break;
+            case 7: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<7>), grid, dim3(256), 0, st, g); break;
+            default: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<8>), grid, dim3(256), 0, st, g); break;
+        }
+        record_launch("sdpa_mfma", grid.x * grid.y * grid.z, 256, (uint64_t)g.planes * g.Hq * g.R);
+        g.guarded = 1;
+    }
+    const dim3 rows_grid(g.R, g.Hq, gz);
+    hipLaunchKernelGGL(sdpa_rows_kernel, rows_grid, dim3(64), 0, st, g);
+    if (!matrix_cores) record_launch("sdpa_rows", rows_grid.x * rows_grid.y * rows_grid.z, 64, (uint64_t)g.planes * g.Hq * g.R);
+    IOMX_HIP(hipGetLastError());
+    return IOMX_OK;
+}

@@ -57,7 +57,7 @@ SYMBOLS = [
     "iomx_memcpy_d2d_async", "iomx_stream_create", "iomx_stream_destroy",
     "iomx_stream_synchronize", "iomx_event_create", "iomx_event_destroy", "iomx_event_record",
     "iomx_event_synchronize", "iomx_event_query", "iomx_event_elapsed_ms",
-    "iomx_launch_linear", "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
+    "iomx_launch_linear", "iomx_sdpa_workspace", "iomx_launch_sdpa", "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
     "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul",
     "iomx_launch_copy", "iomx_launch_scatter", "iomx_launch_gather", "iomx_launch_softmax",
     "iomx_last_launch", "iomx_selftest_bf16_convert", "iomx_selftest_f16_binary",
@@ -148,6 +148,10 @@ def lib() -> C.CDLL:
         l.iomx_launch_cache_append.argtypes = [C.c_int, VP, VP, C.c_uint64, P]
         l.iomx_launch_linear.argtypes = [C.c_int, VP, VP, VP, C.c_uint64, C.c_uint64, C.c_int, C.c_uint64,
                                          C.c_uint64, C.c_int, P]
+        l.iomx_sdpa_workspace.argtypes = [C.c_int, VP, VP, VP, VP, C.c_uint64, C.c_uint64,
+                                          C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
+        l.iomx_launch_sdpa.argtypes = [C.c_int, VP, VP, VP, VP, C.c_uint64, C.c_uint64, C.c_void_p,
+                                       C.c_uint64, C.c_int, C.c_void_p]
         l.iomx_launch_embedding.argtypes = [C.c_int, C.c_int, VP, VP, VP, P, P]
         l.iomx_launch_rope.argtypes = [C.c_int, VP, VP, C.c_uint64, C.c_double, P]
         l.iomx_launch_scatter.argtypes = [C.c_int, VP, P, P]
@@ -434,6 +438,23 @@ def linear(x: DeviceView, w: DeviceView, out: DeviceView, s: int, R: int, head_p
     a, b, o = x.cview(), w.cview(), out.cview()
     return lib().iomx_launch_linear(out.dtype, C.byref(a), C.byref(b), C.byref(o), s, R, int(head_planar),
                                     H, D, path, _h(stream))
+
+
+def sdpa_workspace(q: DeviceView, k: DeviceView, v: DeviceView, out: DeviceView, a: int, L: int):
+    """(status, bytes, alignment) of the caller workspace sdpa needs for these operands."""
+    cq, ck, cv, co = q.cview(), k.cview(), v.cview(), out.cview()
+    nbytes, align = C.c_uint64(0), C.c_uint64(0)
+    rc = lib().iomx_sdpa_workspace(out.dtype, C.byref(cq), C.byref(ck), C.byref(cv), C.byref(co), a, L,
+                                   C.byref(nbytes), C.byref(align))
+    return rc, nbytes.value, align.value
+
+
+def sdpa(q: DeviceView, k: DeviceView, v: DeviceView, out: DeviceView, a: int, L: int,
+         workspace: Optional["Buffer"] = None, path: int = 0, stream: Optional[Stream] = None) -> int:
+    cq, ck, cv, co = q.cview(), k.cview(), v.cview(), out.cview()
+    return lib().iomx_launch_sdpa(out.dtype, C.byref(cq), C.byref(ck), C.byref(cv), C.byref(co), a, L,
+                                  workspace.ptr if workspace is not None else None,
+                                  workspace.nbytes if workspace is not None else 0, path, _h(stream))
 
 
 def cache_append(src: DeviceView, dst: DeviceView, a: int, stream: Optional[Stream] = None) -> int:

@@ -1,0 +1,216 @@
+"""GPU parity of causal grouped-query attention, through the C ABI.
+
+Checked against the reference's fixed fixtures and their expected values
+(tests/golden/sdpa_reference_cases.json, acceptance rule of
+test/backend/backend_conformance_sdpa_reference.hpp:1232-1259: same value class, and for
+finite values at most two BF16 steps or 2^-10 absolute) and against the CPU oracle
+(the reference CPU backend's arithmetic) on seeded shapes with the same rule.
+"""
+import numpy as np
+import pytest
+
+import datagen
+import iomo
+from iom_amd import iomx
+from iomo import DT_BF16, DT_F32
+from test_oracle_sdpa import CASES, all_match, matches, random_case, shapes
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    assert iomx.device_count() >= 1
+    iomx.check(iomx.lib().iomx_set_device(0))
+    yield
+
+
+def device_operands(case, fill=0x5A):
+    qd, kd, od = shapes(case)
+    t = [iomx.DeviceTensor(DT_BF16, d, fill=fill) for d in (qd, kd, kd, od)]
+    t[0].view().from_host(np.array(case["q"], np.uint16).reshape(qd))
+    t[1].view().from_host(np.array(case["k"], np.uint16).reshape(kd))
+    t[2].view().from_host(np.array(case["v"], np.uint16).reshape(kd))
+    return t
+
+
+def run(case, path, fill=0x5A, expect_kernel=None):
+    q, k, v, o = device_operands(case, fill)
+    before = o.raw().copy()
+    ws = None
+    if path == 0:
+        rc, nbytes, align = iomx.sdpa_workspace(q.view(), k.view(), v.view(), o.view(), case["a"], case["L"])
+        assert rc == 0 and align in (1, 256)
+        ws = iomx.Buffer(nbytes) if nbytes else None
+        if ws:
+            ws.fill(0xEE)
+    rc = iomx.sdpa(q.view(), k.view(), v.view(), o.view(), case["a"], case["L"], ws, path)
+    assert rc == 0, iomx.lib().iomx_error_string(rc)
+    iomx.synchronize()
+    if expect_kernel:
+        assert iomx.last_launch().kernel.decode() == expect_kernel
+    got = o.view().to_host()
+    # nothing outside the logical output is written
+    mask = iomo.tile_plane(np.ones(o.dims, np.uint16)) == 0
+    assert np.array_equal(o.raw()[mask], before[mask])
+    for t in (q, k, v, o):
+        t.free()
+    if ws:
+        ws.free()
+    return got
+
+
+def oracle(case, fill=0x5A):
+    from test_oracle_sdpa import host_operands
+    q, k, v, o = host_operands(case, fill)
+    assert iomo.sdpa(q.view(), k.view(), v.view(), o.view(), case["a"], case["L"]) == 0
+    return o.view().to_logical()
+
+
+def close_to_oracle(got, want):
+    got, want = got.reshape(-1), want.reshape(-1)
+    from test_oracle_sdpa import bf16_class
+    return [i for i, (g, w) in enumerate(zip(got, want)) if not matches(int(g), int(w), bf16_class(int(w)))]
+
+
+@pytest.mark.parametrize("path,kernel", [(0, "sdpa_mfma"), (1, "sdpa_rows")], ids=["matrix_cores", "reference_order"])
+@pytest.mark.parametrize("index", range(len(CASES)), ids=[c["label"].replace(" ", "_") for c in CASES])
+def test_reference_fixtures(index, path, kernel):
+    case = CASES[index]
+    for fill in (0x5A, 0xFF):          # 0xFF: NaN patterns in tile padding
+        got = run(case, path, fill, kernel)
+        assert all_match(got, case) == [], case["label"]
+
+
+SEEDED = [((), 2, 1, 5, 8, 12, 3, 9), ((2,), 4, 2, 17, 16, 40, 20, 37), ((2, 2), 4, 1, 3, 33, 20, 0, 2),
+          ((), 8, 2, 1, 64, 70, 69, 70), ((3,), 2, 2, 16, 5, 16, 0, 16), ((2,), 8, 2, 40, 64, 100, 50, 90),
+          ((), 4, 4, 33, 128, 64, 10, 43), ((), 2, 1, 70, 48, 200, 100, 170)]
+
+
+def float64_attention(case):
+    """Attention in float64 on the flushed operands, and per output the budget of the BF16
+    probability: every P is rounded once to BF16 (2^-9 relative) and a score that differs in
+    its last binary32 bits can move it one more step, so |error| <= 2^-8 * sum_t P|V|, plus the
+    final BF16 rounding."""
+    lead, Hq, Hkv, R, D, C, a, L = (case[k] for k in ("leading", "Hq", "Hkv", "R", "D", "C", "a", "L"))
+    n = int(np.prod(lead)) if lead else 1
+
+    def values(name, shape):
+        bits = np.array(case[name], np.uint16).reshape(shape).copy()
+        bits[(bits & 0x7F80) == 0] &= 0x8000
+        return datagen.bf16_to_f32(bits.reshape(-1)).astype(np.float64).reshape(shape)
+    q, k, v = values("q", (n, Hq, R, D)), values("k", (n, Hkv, C, D)), values("v", (n, Hkv, C, D))
+    out = np.zeros((n, R, Hq * D))
+    budget = np.zeros((n, R, Hq * D))
+    for b in range(n):
+        for h in range(Hq):
+            g = h // (Hq // Hkv)
+            s = q[b, h] @ k[b, g, :L].T / np.sqrt(np.float32(D)).astype(np.float64)
+            t = np.arange(L)[None, :]
+            s = np.where(t <= a + np.arange(R)[:, None], s, -np.inf)
+            e = np.exp(s - s.max(axis=1, keepdims=True))
+            pr = e / e.sum(axis=1, keepdims=True)
+            out[b, :, h * D:(h + 1) * D] = pr @ v[b, g, :L]
+            budget[b, :, h * D:(h + 1) * D] = 2.0 ** -8 * (pr @ np.abs(v[b, g, :L]))
+    return out, budget + 2.0 ** -8 * np.abs(out) + 2.0 ** -126
+
+
+@pytest.mark.parametrize("path", [0, 1], ids=["matrix_cores", "reference_order"])
+@pytest.mark.parametrize("spec", SEEDED, ids=[str(i) for i in range(len(SEEDED))])
+def test_seeded_shapes_against_the_oracle(spec, path):
+    lead, Hq, Hkv, R, D, C, a, L = spec
+    case = random_case(41 + R, lead, Hq, Hkv, R, D, C, a, L)
+    kk = np.array(case["k"], np.uint16)
+    kk[1], kk[2] = 0x0040, 0x8001         # subnormal operands: flushed
+    case["k"] = kk.tolist()
+    got = run(case, path, fill=0xFF)
+    want = oracle(case)
+    exact = int(np.sum(got.reshape(-1) == want.reshape(-1)))
+    outside = close_to_oracle(got, want)
+    print(spec, "path", path, "bit-equal to the oracle:", exact, "of", got.size,
+          "outside the fixture rule:", len(outside), flush=True)
+    ref64, budget = float64_attention(case)
+    g = datagen.bf16_to_f32(got.reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    assert np.all(np.abs(g - ref64) <= budget)
+    # the oracle itself sits inside the same budget, so the budget is not a loose one
+    w = datagen.bf16_to_f32(want.reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    assert np.all(np.abs(w - ref64) <= budget)
+    if path == 1:
+        assert outside == [] and exact >= 0.98 * got.size     # same order of operations; only expf may differ
+    else:
+        assert len(outside) <= 0.001 * got.size                # the fixture rule is not a cancellation bound
+
+
+def test_tail_future_tokens_and_special_v():
+    """The cache tail and tokens no row may see hold infinities and NaN: results are the
+    same bits as with finite values there.  An infinity in a V row that some rows see and
+    others do not reaches exactly the rows that see it."""
+    case = random_case(5, (2,), 4, 2, 6, 16, 24, 4, 8)
+    base = run(case, 0)
+    k = np.array(case["k"], np.uint16).reshape(2, 2, 24, 16).copy()
+    v = np.array(case["v"], np.uint16).reshape(2, 2, 24, 16).copy()
+    k[:, :, 8:, :] = 0x7FC0
+    v[:, :, 8:, :] = 0x7F80
+    tail = dict(case, k=k.reshape(-1).tolist(), v=v.reshape(-1).tolist())
+    assert np.array_equal(run(tail, 0, fill=0xFF), base)
+    assert np.array_equal(run(tail, 1, fill=0xFF), run(case, 1))
+    # token 6 is visible to rows r >= 2 (a + r + 1 > 6) only
+    v2 = np.array(case["v"], np.uint16).reshape(2, 2, 24, 16).copy()
+    v2[0, 1, 6, 3] = 0x7F80
+    part = dict(case, v=v2.reshape(-1).tolist())
+    got = run(part, 0)
+    want = oracle(part)
+    assert close_to_oracle(got, want) == []
+    g = got.reshape(2, 6, 4, 16)
+    assert np.all(g[0, 2:, 2:, 3] == 0x7F80) and np.all((g[0, :2, :, :] & 0x7F80) != 0x7F80)
+    assert np.array_equal(g[1], base.reshape(2, 6, 4, 16)[1])
+
+
+def test_incremental_rows_equal_the_prefill():
+    case = random_case(9, (), 4, 2, 7, 8, 7, 0, 7)
+    full = run(case, 0)
+    for r in range(7):
+        c = dict(case, R=1, q=np.array(case["q"], np.uint16).reshape(4, 7, 8)[:, r:r + 1].reshape(-1).tolist())
+        c["a"], c["L"] = r, r + 1
+        one = run(c, 0)
+        assert close_to_oracle(one[0], full[r]) == []
+
+
+def test_views_and_rejections():
+    # q, k, v as windows of larger owners; out a plane of a larger owner
+    Hq, Hkv, R, D, C, a, L = 4, 2, 5, 16, 12, 3, 8
+    case = random_case(77, (2,), Hq, Hkv, R, D, C, a, L)
+    want = oracle(case)
+    qo = iomx.DeviceTensor(DT_BF16, (3, Hq, R, D), fill=0x11)
+    ko = iomx.DeviceTensor(DT_BF16, (2, Hkv + 1, C, D), fill=0x11)
+    vo = iomx.DeviceTensor(DT_BF16, (2, Hkv, C, D), fill=0x11)
+    oo = iomx.DeviceTensor(DT_BF16, (4, R, Hq * D), fill=0x11)
+    qv = qo.view().slice(0, 1, 2, 1)
+    kv = ko.view().slice(1, 1, Hkv, 1)
+    ov = oo.view().slice(0, 0, 2, 2)
+    qv.from_host(np.array(case["q"], np.uint16).reshape(2, Hq, R, D))
+    kv.from_host(np.array(case["k"], np.uint16).reshape(2, Hkv, C, D))
+    vo.view().from_host(np.array(case["v"], np.uint16).reshape(2, Hkv, C, D))
+    rc, nbytes, _ = iomx.sdpa_workspace(qv, kv, vo.view(), ov, a, L)
+    assert rc == 0 and nbytes > 0
+    ws = iomx.Buffer(nbytes)
+    assert iomx.sdpa(qv, kv, vo.view(), ov, a, L, ws) == 0
+    iomx.synchronize()
+    assert close_to_oracle(ov.to_host(), want) == []
+    assert np.all(oo.view().to_host()[[1, 3]] == 0x1111)
+    # admission
+    q, k, v, o = qo.view().slice(0, 0, 2, 1), ko.view().slice(1, 0, Hkv, 1), vo.view(), oo.view().slice(0, 0, 2, 1)
+    for bad_a, bad_L in ((3, 0), (3, 13), (12, 8), (8, 8)):
+        assert iomx.sdpa(q, k, v, o, bad_a, bad_L, ws) == -1
+    assert iomx.sdpa(q, k, v, o, a, L, None) == -1                  # the matrix-core path needs its workspace
+    assert iomx.sdpa(q, k, v, o, a, L, None, 1) == 0                # the reference-order path does not
+    small = iomx.Buffer(512)
+    assert iomx.sdpa(q, k, v, o, a, L, small) == -1
+    assert iomx.sdpa(q, ko.view(), v, o, a, L, ws) == -1            # Hq % Hkv != 0
+    f = [iomx.DeviceTensor(DT_F32, d) for d in ((4, 3, 8), (2, 10, 8), (3, 32))]
+    assert iomx.sdpa(f[0].view(), f[1].view(), f[1].view(), f[2].view(), 2, 5, ws) == -2
+    iomx.synchronize()
+    for t in (qo, ko, vo, oo, *f):
+        t.free()
+    ws.free()
+    small.free()
