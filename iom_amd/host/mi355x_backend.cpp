@@ -663,6 +663,63 @@ private:
                 });
     }
 
+    // ---- attention ----------------------------------------------------------------
+
+    // BF16 only (docs/BACKEND_CONTRACT/scaled-dot-product-attention.md "Current capability
+    // matrix"); every other leaf is an explicit rejection after structural validation.
+    [[nodiscard]] WorkspaceRequirements sdpa_workspace_requirements_impl(
+            const SdpaRequest& request) override {
+        if (request.q.data_type != DataType::BF16) throw detail::UnsupportedOperation();
+        const iomx_view q = snapshot_view(request.q), k = snapshot_view(request.k);
+        const iomx_view v = snapshot_view(request.v), out = snapshot_view(request.out);
+        std::uint64_t bytes = 0, alignment = 1;
+        const int status = iomx_sdpa_workspace(IOMX_DT_BF16, &q, &k, &v, &out, request.a, request.L,
+                                               &bytes, &alignment);
+        if (status == IOMX_ERR_UNSUPPORTED) throw detail::UnsupportedOperation();
+        if (status != IOMX_OK) throw std::length_error("MI355X SDPA workspace size overflows");
+        return {static_cast<std::size_t>(bytes), static_cast<std::size_t>(alignment)};
+    }
+
+    oid sdpa_impl(const SdpaRequest& request) override {
+        if (request.q.data_type != DataType::BF16) throw detail::UnsupportedOperation();
+        std::lock_guard<std::mutex> order(submission_mutex_);
+        return submit_sdpa(
+                request, device_.registry_state(), registry_queue_id_, pending_fence(),
+                [this](std::uint64_t sequence, const SdpaRequest& captured,
+                       detail::SdpaEntryRegistration entries) {
+                    auto& state = device_.registry_state();
+                    const detail::WorkspaceLease lease = captured.workspace_lease;
+                    try {
+                        void* scratch = captured.workspace.empty()
+                                ? nullptr : detail::WorkspaceValidation::address(captured.workspace);
+                        const std::uint64_t scratch_bytes = captured.workspace.byte_size();
+                        start(sequence,
+                              [&captured, scratch, scratch_bytes](iomx_stream_t stream) {
+                                  const iomx_view q = snapshot_view(captured.q);
+                                  const iomx_view k = snapshot_view(captured.k);
+                                  const iomx_view v = snapshot_view(captured.v);
+                                  const iomx_view out = snapshot_view(captured.out);
+                                  // no workspace was asked for: the head is wider than the
+                                  // matrix-core fragments cover, the reference-order kernel runs
+                                  return iomx_launch_sdpa(IOMX_DT_BF16, &q, &k, &v, &out, captured.a,
+                                                          captured.L, scratch, scratch_bytes,
+                                                          captured.workspace_requirements.bytes ? 0 : 1,
+                                                          stream);
+                              },
+                              [&state, entries, lease](bool failed) {
+                                  (void)detail::release_or_invalidate_sdpa_entries(
+                                          state.registry, entries, failed, true);
+                                  detail::complete_workspace_lease(state, lease, true);
+                              });
+                    } catch (...) {
+                        state.registry.remove_entries(std::span<const detail::EntryId>(
+                                entries.entries.data(), entries.count));
+                        detail::complete_workspace_lease(state, lease, true);
+                        throw;
+                    }
+                });
+    }
+
     // ---- cache append / embedding / rope ----------------------------------------
 
     template <typename Snapshot>

@@ -214,3 +214,61 @@ def test_views_and_rejections():
         t.free()
     ws.free()
     small.free()
+
+
+# -- through the C++ backend, next to the reference CPU backend ---------------------------
+
+@pytest.fixture(scope="module")
+def devices():
+    if not iomo.mi355x_available():
+        pytest.skip("oracle/_ref/libiom_mi355x_shim.so not built (needs the reference headers)")
+    gpu = iomo.mi355x_backend(arena_bytes=1 << 28, max_in_flight=4)
+    cpu = iomo.cpu_backend_beside_mi355x()
+    yield cpu, gpu
+    gpu.close()
+    cpu.close()
+
+
+def backend_run(dev, case):
+    qd, kd, od = shapes(case)
+    t = [dev.tensor(DT_BF16, d) for d in (qd, kd, kd, od)]
+    t[0].view().from_host(np.array(case["q"], np.uint16).reshape(qd))
+    t[1].view().from_host(np.array(case["k"], np.uint16).reshape(kd))
+    t[2].view().from_host(np.array(case["v"], np.uint16).reshape(kd))
+    token = dev.sdpa(t[0].view(), t[1].view(), t[2].view(), t[3].view(), case["a"], case["L"])
+    got = t[3].view().to_host() if token > 0 else None
+    for x in t:
+        x.close()
+    return token, got
+
+
+@pytest.mark.parametrize("index", range(len(CASES)), ids=[c["label"].replace(" ", "_") for c in CASES])
+def test_backend_on_the_reference_fixtures(devices, index):
+    cpu, gpu = devices
+    case = CASES[index]
+    token, got = backend_run(gpu, case)
+    assert token > 0, gpu.error()
+    assert all_match(got, case) == []
+    token, want = backend_run(cpu, case)
+    assert token > 0, cpu.error()
+    assert close_to_oracle(got, want) == []
+
+
+def test_backend_prefill_then_decode_and_rejections(devices):
+    cpu, gpu = devices
+    case = random_case(91, (2,), 8, 2, 24, 64, 48, 0, 24)
+    outs = [backend_run(dev, case) for dev in (cpu, gpu)]
+    assert outs[0][0] > 0 and outs[1][0] > 0
+    assert len(close_to_oracle(outs[1][1], outs[0][1])) <= 0.001 * outs[0][1].size
+    step = dict(case, R=1, a=24, L=25,
+                q=np.array(case["q"], np.uint16).reshape(2, 8, 24, 64)[:, :, :1].reshape(-1).tolist())
+    outs = [backend_run(dev, step) for dev in (cpu, gpu)]
+    assert close_to_oracle(outs[1][1], outs[0][1]) == []
+    # admission and capability answers are the reference's own
+    for bad in (dict(case, L=0), dict(case, L=49), dict(case, a=48), dict(case, a=30)):
+        assert backend_run(cpu, bad)[0] == backend_run(gpu, bad)[0] < 0
+    for dev in (cpu, gpu):
+        f = [dev.tensor(DT_F32, d) for d in ((4, 3, 8), (2, 10, 8), (3, 32))]
+        assert dev.sdpa(f[0].view(), f[1].view(), f[1].view(), f[2].view(), 2, 5) < 0
+        for x in f:
+            x.close()
