@@ -366,6 +366,39 @@ def wl_linear(timer, steps, warmup):
     return out
 
 
+def wl_sdpa(timer, steps, warmup):
+    """BF16 causal grouped-query attention at TinyLlama's head shape (32 query heads, 4 KV
+    heads, D = 64): a 512-token prefill of 8 sequences and a decode step of 64 sequences
+    against a 512-token cache.  Algorithmic bytes: q, the visible K and V prefix and out,
+    once each; flops: 4 * D per (row, visible token, head)."""
+    out = []
+    Hq, Hkv, D, C = 32, 4, 64, 512
+    for name, B, R, a, L in (("prefill", 8, 512, 0, 512), ("decode", 64, 1, 511, 512)):
+        q = device_tensor(BF16, (B, Hq, R, D), "normal", 111)
+        k = device_tensor(BF16, (B, Hkv, C, D), "normal", 112)
+        v = device_tensor(BF16, (B, Hkv, C, D), "normal", 113)
+        o = device_tensor(BF16, (B, R, Hq * D))
+        qv, ov = q.view(), o.view()
+        rc, nbytes, _ = iomx.sdpa_workspace(qv, k.view(), v.view(), ov, a, L)
+        check(rc, "sdpa_workspace")
+        ws = iomx.Buffer(nbytes)
+
+        def launch(i):
+            check(iomx.sdpa(qv, k.view(), v.view(), ov, a, L, ws, 0, timer.stream), "sdpa")
+
+        wall, ev = timer.run(launch, steps, warmup)
+        visible = sum(min(L, a + r + 1) for r in range(R))
+        flops = 4.0 * B * Hq * D * visible
+        r = report("sdpa_bf16_%s_B%d_Hq32_Hkv4_R%d_L%d_D64" % (name, B, R, L),
+                   2 * (B * Hq * R * D * 2 + 2 * B * Hkv * L * D), B * Hq * R * D, wall, ev, "sdpa_mfma")
+        r["TFLOP_per_s"] = round(flops / (ev * 1e-3) / 1e12, 2)
+        r["launches"] = "clear_flag + pack_v + sdpa_mfma + sdpa_rows (guard)"
+        out.append(r)
+        for t in (q, k, v, o, ws):
+            t.free()
+    return out
+
+
 def wl_softmax(timer, steps, warmup, planes, heads, rows, cols, causal_position):
     """F32 scores [planes,heads,rows,cols] with the strict upper triangle = -inf as data.
     causal_position=False: a = cols-1, every token is positionally visible (the mask
@@ -541,6 +574,7 @@ def main():
         "chain": lambda: wl_chain(timer, max(K // 10, 5), max(W // 10, 2)),
         "layer_ops": lambda: wl_layer_ops(timer, max(K // 4, 5), max(W // 4, 2)),
         "linear": lambda: wl_linear(timer, max(K // 20, 5), 2),
+        "sdpa": lambda: wl_sdpa(timer, max(K // 20, 5), 2),
         "other_leaves": lambda: wl_other_leaves(timer, max(K // 10, 5), max(W // 10, 2)),
     }
 

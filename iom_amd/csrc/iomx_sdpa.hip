@@ -33,14 +33,16 @@ struct SdpaArgs {
     uint32_t d_tiles, out_tile_cols, kv_tile_rows;
     uint32_t planes, groups;    // leading planes; 32-token groups of the prefix
     uint8_t* packed_v;          // [plane][kv head][group][d tile] fragments of 1 KiB
-    uint32_t* flag;             // nonzero: the prefix of V holds an infinity or NaN
-    uint32_t guarded;           // sdpa_rows: return unless the flag is up
+    uint8_t* packed_k;          // [plane][kv head][token tile][d tile] flushed tiles (null: not packed)
+    uint32_t* flags;            // [plane][kv head][pack split]: nonzero = that part of the V prefix
+                                // holds an infinity or NaN
+    uint32_t pack_splits;       // workgroups sharing the fragments of one KV head
+    uint32_t guarded;           // sdpa_rows: skip the rows whose KV head has no flag up
     float scale;                // sqrtf(D)
+    float inv_scale;            // 1 / scale when that is a power of two (the product is then the quotient), else 0
 };
 
 constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
-
-__global__ void sdpa_clear_flag_kernel(uint32_t* flag) { *flag = 0u; }
 
 // Subnormal operands of the matrix stages become zeros of the same sign
 // (src/cpu/sdpa.cpp:57-60), two BF16 per word.
@@ -56,39 +58,61 @@ __device__ __forceinline__ float daz_bf16(uint32_t h) {
     return as_f32(((h & 0x7F80u) ? h : (h & 0x8000u)) << 16);
 }
 
-// Fragment (group g, d tile dt) holds, for lane (d = l%16, kg = l/16), the eight
-// values V[32g + 4kg + j][16dt + d] (j < 4) and V[32g + 16 + 4kg + j][16dt + d]:
-// the token order in which a lane of sdpa_mfma holds its probabilities.
-__global__ __launch_bounds__(256) void sdpa_pack_v_kernel(const SdpaArgs a) {
+// One workgroup packs a share of the fragments of one KV head of one plane and writes
+// that share's flag word (every word is written on every call, so the workspace needs
+// no clearing).
+//
+// V fragment (group g, d tile dt) holds, for lane (d = l%16, kg = l/16), the eight
+// values V[32g + 4kg + j][16dt + d] (j < 4) and V[32g + 16 + 4kg + j][16dt + d]: the
+// token order in which a lane of sdpa_mfma holds its probabilities.  K is copied tile
+// for tile (token tiles 2g and 2g+1, d tile dt) with the same flush, rows past the
+// prefix and columns past D as zeros, so that the many waves that meet a K tile do not
+// each flush it again.
+__global__ __launch_bounds__(256) void sdpa_pack_kernel(const SdpaArgs a) {
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const uint32_t frag = blockIdx.x * 4 + wave;
-    if (frag >= a.groups * a.d_tiles) return;
-    const uint32_t g = frag / a.d_tiles, dt = frag - g * a.d_tiles;
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
-    const uint32_t d = dt * kTile + l16;
-    const uint32_t hkv = blockIdx.y;
-    for (uint32_t p = blockIdx.z; p < a.planes; p += gridDim.z) {
+    const uint32_t hkv = blockIdx.x / a.pack_splits, split = blockIdx.x - hkv * a.pack_splits;
+    const uint32_t frags = a.groups * a.d_tiles;
+    for (uint32_t p = blockIdx.y; p < a.planes; p += gridDim.y) {
         uint64_t plane[4];
         walk_planes(a.walk, p, plane);
         const uint8_t* vb = a.v + (plane[2] + (uint64_t)hkv * a.v_head_stride) * a.kv_plane_bytes;
-        uint32_t h[8];
+        const uint8_t* kb = a.k + (plane[1] + (uint64_t)hkv * a.k_head_stride) * a.kv_plane_bytes;
+        const uint64_t head_frags = ((uint64_t)p * a.Hkv + hkv) * frags;
         bool special = false;
+        for (uint32_t frag = split * 4 + wave; frag < frags; frag += 4 * a.pack_splits) {
+            const uint32_t g = frag / a.d_tiles, dt = frag - g * a.d_tiles;
+            const uint32_t d = dt * kTile + l16;
+            uint32_t h[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const uint32_t token = 32 * g + (j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4));
-            uint32_t bits = 0;
-            if (token < a.L && d < a.D) {
-                bits = *reinterpret_cast<const uint16_t*>(
-                        vb + ((uint64_t)(token >> 4) * a.d_tiles + dt) * kTileBytes + (token & 15u) * kRowBytes + l16 * 2);
-                special = special || (bits & 0x7F80u) == 0x7F80u;
-                if ((bits & 0x7F80u) == 0) bits &= 0x8000u;
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t token = 32 * g + (j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4));
+                uint32_t bits = 0;
+                if (token < a.L && d < a.D) {
+                    bits = *reinterpret_cast<const uint16_t*>(
+                            vb + ((uint64_t)(token >> 4) * a.d_tiles + dt) * kTileBytes + (token & 15u) * kRowBytes + l16 * 2);
+                    special = special || (bits & 0x7F80u) == 0x7F80u;
+                    if ((bits & 0x7F80u) == 0) bits &= 0x8000u;
+                }
+                h[j] = bits;
             }
-            h[j] = bits;
+            *reinterpret_cast<u32x4*>(a.packed_v + (head_frags + frag) * kFrag + lane * 16) =
+                    u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+            if (a.packed_k) {
+                // lane = 16-byte chunk of the two tiles: tile lane/32, row (lane%32)/2, half lane%2
+                const uint32_t tt = 2 * g + (lane >> 5), r = (lane & 31u) >> 1, half = lane & 1u;
+                const uint32_t token = tt * kTile + r;
+                u32x4 w = {0, 0, 0, 0};
+                if (token < a.L)
+                    w = load_k8_bits(kb + ((uint64_t)tt * a.d_tiles + dt) * kTileBytes + r * kRowBytes,
+                                     half * 8, dt * kTile + half * 8, a.D);
+                w = u32x4{daz2(w[0]), daz2(w[1]), daz2(w[2]), daz2(w[3])};
+                *reinterpret_cast<u32x4*>(a.packed_k + ((head_frags * 2 + (uint64_t)tt * a.d_tiles + dt) * kTileBytes)
+                                          + (lane & 31u) * 16) = w;
+            }
         }
-        uint8_t* dst = a.packed_v + ((((uint64_t)p * a.Hkv + hkv) * a.groups + g) * a.d_tiles + dt) * kFrag + lane * 16;
-        *reinterpret_cast<u32x4*>(dst) = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16),
-                                               h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
-        if (special) atomicOr(a.flag, 1u);
+        const int any = __syncthreads_or(special ? 1 : 0);
+        if (threadIdx.x == 0) a.flags[((uint64_t)p * a.Hkv + hkv) * a.pack_splits + split] = any ? 1u : 0u;
     }
 }
 
@@ -99,19 +123,10 @@ struct RowStats {
     float m, sum;
     uint32_t pinf;
     bool nan, finite;
-    __device__ __forceinline__ void add(float s) {
-        if (s != s) nan = true;
-        else if (s == __builtin_inff()) ++pinf;
-        else if (s != -__builtin_inff()) {
-            finite = true;
-            if (s > m) { sum *= expf(m - s); m = s; }
-            sum += expf(s - m);
-        }
-    }
     __device__ __forceinline__ void merge(float m2, float sum2, uint32_t pinf2, bool nan2, bool finite2) {
         const float mm = m > m2 ? m : m2;
         if (mm == -__builtin_inff()) sum = 0.0f;
-        else sum = sum * expf(m - mm) + sum2 * expf(m2 - mm);
+        else sum = sum * __expf(m - mm) + sum2 * __expf(m2 - mm);
         m = mm;
         pinf += pinf2;
         nan = nan || nan2;
@@ -119,24 +134,44 @@ struct RowStats {
     }
 };
 
-template <int DT16>
+// One workgroup = four waves.  MODE 0: four heads of one row tile, each wave walks
+// all visible tokens (prefill: many row tiles, K and V shared through the caches).
+// MODE 1: one head, the waves take every fourth 32-token group and meet in LDS (few
+// rows against a long prefix would otherwise be one wave's chain of dependent
+// loads).  MODE 2: the same split, and the 16 rows of the tile are the rows of all
+// query heads that share one KV head (grouping * R <= 16: a decode step reads K and
+// V once per KV head instead of once per query head).  In every mode the K
+// fragments of the next group are requested before the current group is multiplied.
+template <int DT16, int MODE>
 __global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
+    constexpr bool SPLIT = MODE != 0;
     constexpr int D32 = (DT16 + 1) / 2;
+    __shared__ float wave_stats[4][16][5];
+    __shared__ f32x4_t wave_out[SPLIT ? 3 : 1][SPLIT ? DT16 : 1][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
-    const uint32_t head = blockIdx.y * 4 + wave;
-    if (head >= a.Hq) return;
-    const uint32_t hkv = head / a.grouping;
-    const uint32_t r0 = blockIdx.x * kTile;
-    const uint32_t row = r0 + l16;
+    // which (head, row) the lane's tile row is
+    uint32_t hkv, head, row, last_row;
+    if (MODE == 2) {
+        hkv = blockIdx.y;
+        row = l16 / a.grouping;
+        head = hkv * a.grouping + (l16 - row * a.grouping);
+        last_row = a.R - 1;
+    } else {
+        head = MODE == 1 ? blockIdx.y : blockIdx.y * 4 + wave;
+        if (MODE == 0 && head >= a.Hq) return;          // no barrier on this path
+        hkv = head / a.grouping;
+        row = blockIdx.x * kTile + l16;
+        last_row = blockIdx.x * kTile + 15 < a.R ? blockIdx.x * kTile + 15 : a.R - 1;
+    }
     const bool row_ok = row < a.R;
     const uint32_t qrow = row_ok ? row : a.R - 1;
-    const uint32_t last_row = r0 + 15 < a.R ? r0 + 15 : a.R - 1;
     const uint32_t reach = a.a + row + 1, reach_max = a.a + last_row + 1;
     const uint32_t vis = row_ok ? (reach < a.L ? reach : a.L) : 0;     // tokens this lane's row sees
-    const uint32_t vis_max = reach_max < a.L ? reach_max : a.L;        // ... and the wave's last row
+    const uint32_t vis_max = reach_max < a.L ? reach_max : a.L;        // ... and the tile's last row
     const uint32_t groups = (vis_max + 31) / 32;
+    const uint32_t g_first = SPLIT ? wave : 0, g_step = SPLIT ? 4 : 1;
     const uint32_t c0 = (kg & 1u) * 8u;
     const float inf = __builtin_inff();
     for (uint32_t p = blockIdx.z; p < a.planes; p += gridDim.z) {
@@ -155,36 +190,97 @@ __global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 qf[c] = daz8(load_k8_bits(qb + ((uint64_t)(qrow >> 4) * a.d_tiles + tile) * kTileBytes
                                                   + (qrow & 15u) * kRowBytes, c0, i0, a.D));
         }
-        // scores of the 16 tokens from t0 against the 16 rows: lane gets token
-        // t0 + 4*kg + j (j < 4) of row l16.  Tokens past the prefix read its last
-        // token instead (the cache tail is never touched); their scores are dropped.
-        auto scores = [&](uint32_t t0) {
-            uint32_t token = t0 + l16;
-            if (token >= a.L) token = a.L - 1;
-            const uint8_t* krow = kb + (uint64_t)(token >> 4) * a.d_tiles * kTileBytes + (token & 15u) * kRowBytes;
-            f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        // K of the 32 tokens of group g: two 16-token tiles, lane (token l16, features
+        // 8*kg..).  Tokens past the prefix read its last token instead (the cache tail
+        // is never touched); their scores are dropped.
+        struct KGroup { u32x4 w[2][D32]; };
+        constexpr bool KPACK = MODE != 2;      // the flushed copy pays when many waves meet each tile
+        const uint8_t* kp = KPACK ? a.packed_k + (((uint64_t)p * a.Hkv + hkv) * a.groups * 2) * a.d_tiles * kTileBytes
+                                           + l16 * kRowBytes + c0 * 2
+                                  : nullptr;
+        auto load_k = [&](uint32_t g, KGroup& kgp) {
 #pragma unroll
-            for (int c = 0; c < D32; ++c) {
-                const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
-                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
-                if (i0 < a.D) kf = daz8(load_k8_bits(krow + (uint64_t)tile * kTileBytes, c0, i0, a.D));
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], acc, 0, 0, 0);
+            for (int half = 0; half < 2; ++half) {
+                if (KPACK) {
+#pragma unroll
+                    for (int c = 0; c < D32; ++c) {
+                        const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
+                        kgp.w[half][c] = u32x4{0, 0, 0, 0};
+                        if (i0 < a.D)
+                            kgp.w[half][c] = *reinterpret_cast<const u32x4*>(
+                                    kp + ((uint64_t)(2 * g + half) * a.d_tiles + tile) * kTileBytes);
+                    }
+                    continue;
+                }
+                uint32_t token = 32 * g + 16 * half + l16;
+                if (token >= a.L) token = a.L - 1;
+                const uint8_t* krow = kb + (uint64_t)(token >> 4) * a.d_tiles * kTileBytes + (token & 15u) * kRowBytes;
+#pragma unroll
+                for (int c = 0; c < D32; ++c) {
+                    const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
+                    kgp.w[half][c] = u32x4{0, 0, 0, 0};
+                    if (i0 < a.D) {
+                        const u32x4 w = load_k8_bits(krow + (uint64_t)tile * kTileBytes, c0, i0, a.D);
+                        kgp.w[half][c] = u32x4{daz2(w[0]), daz2(w[1]), daz2(w[2]), daz2(w[3])};
+                    }
+                }
             }
+        };
+        // scores: lane gets tokens 32g + 16*half + 4*kg + j (j < 4) of row l16
+        auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2]) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = acc[j] / a.scale;
-            return acc;
+            for (int half = 0; half < 2; ++half) {
+                f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int c = 0; c < D32; ++c)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kgp.w[half][c]), qf[c], acc, 0, 0, 0);
+                if (a.inv_scale != 0.0f) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[j] = acc[j] * a.inv_scale;   // sqrt(D) is a power of two
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[j] = acc[j] / a.scale;
+                }
+                s[half] = acc;
+            }
         };
         // pass 1: the row's statistics
         RowStats st = {-inf, 0.0f, 0u, false, false};
-        for (uint32_t g = 0; g < groups; ++g) {
+        {
+            KGroup cur, nxt;
+            if (g_first < groups) load_k(g_first, cur);
+            for (uint32_t g = g_first; g < groups; g += g_step) {
+                if (g + g_step < groups) load_k(g + g_step, nxt);     // the next group is in flight meanwhile
+                f32x4_t s[2];
+                scores(cur, s);
+                // the finite maximum of the lane's eight scores first, then one rescale
+                float local = -inf;
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const uint32_t t0 = 32 * g + 16 * half;
-                if (t0 >= vis_max) continue;
-                const f32x4_t s = scores(t0);
+                for (int half = 0; half < 2; ++half)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (t0 + 4 * kg + j < vis) st.add(s[j]);
+                    for (int j = 0; j < 4; ++j) {
+                        const bool seen = 32 * g + 16 * half + 4 * kg + j < vis;
+                        const float v = s[half][j];
+                        if (seen) {
+                            st.nan = st.nan || v != v;
+                            st.pinf += v == inf ? 1u : 0u;
+                        }
+                        // masked, NaN and infinite scores take no part in the sum
+                        s[half][j] = (seen && v - v == 0.0f) ? v : -inf;
+                        local = s[half][j] > local ? s[half][j] : local;
+                    }
+                if (local > st.m) {
+                    st.sum *= __expf(st.m - local);
+                    st.m = local;
+                    st.finite = true;
+                }
+                if (st.finite) {
+#pragma unroll
+                    for (int half = 0; half < 2; ++half)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) st.sum += __expf(s[half][j] - st.m);   // exp(-inf) = 0
+                }
+                cur = nxt;
             }
         }
 #pragma unroll
@@ -194,39 +290,74 @@ __global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             const int n2 = __shfl_xor((int)st.nan, off), f2 = __shfl_xor((int)st.finite, off);
             st.merge(m2, s2, p2, n2 != 0, f2 != 0);
         }
+        if (SPLIT) {
+            __syncthreads();                       // the previous plane's readers are done
+            if (kg == 0) {
+                wave_stats[wave][l16][0] = st.m;
+                wave_stats[wave][l16][1] = st.sum;
+                wave_stats[wave][l16][2] = as_f32(st.pinf);
+                wave_stats[wave][l16][3] = st.nan ? 1.0f : 0.0f;
+                wave_stats[wave][l16][4] = st.finite ? 1.0f : 0.0f;
+            }
+            __syncthreads();
+            st = RowStats{-inf, 0.0f, 0u, false, false};
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+                st.merge(wave_stats[w][l16][0], wave_stats[w][l16][1], as_u32(wave_stats[w][l16][2]),
+                         wave_stats[w][l16][3] != 0.0f, wave_stats[w][l16][4] != 0.0f);
+        }
         const bool nan_row = st.nan || (st.pinf == 0 && !st.finite);      // NaN score or all -inf
         const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
+        const float inv_sum = 1.0f / st.sum;
         // pass 2: probabilities, rounded once to BF16, times V
         f32x4_t o[DT16];
 #pragma unroll
         for (int dt = 0; dt < DT16; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        for (uint32_t g = 0; g < groups; ++g) {
-            uint32_t pb[8];
+        {
+            KGroup cur, nxt;
+            if (g_first < groups) load_k(g_first, cur);
+            for (uint32_t g = g_first; g < groups; g += g_step) {
+                if (g + g_step < groups) load_k(g + g_step, nxt);
+                u32x4 vfr[DT16];
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const uint32_t t0 = 32 * g + 16 * half;
-                f32x4_t s = {-inf, -inf, -inf, -inf};
-                if (t0 < vis_max) s = scores(t0);
+                for (int dt = 0; dt < DT16; ++dt)
+                    vfr[dt] = *reinterpret_cast<const u32x4*>(vf + ((uint64_t)g * a.d_tiles + dt) * kFrag);
+                f32x4_t s[2];
+                scores(cur, s);
+                float pr[8];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float pr = 0.0f;
-                    if (t0 + 4 * kg + j < vis && !nan_row) {
-                        if (st.pinf) pr = s[j] == inf ? pinf_p : 0.0f;
-                        else if (s[j] != -inf) pr = expf(s[j] - st.m) / st.sum;
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float v = s[half][j];
+                        float e = 0.0f;
+                        if (32 * g + 16 * half + 4 * kg + j < vis && !nan_row) {
+                            if (st.pinf) e = v == inf ? pinf_p : 0.0f;
+                            else if (v != -inf) e = __expf(v - st.m) * inv_sum;
+                        }
+                        pr[half * 4 + j] = e;
                     }
-                    uint32_t h = bf16_rne_sw(as_u32(pr));
-                    if ((h & 0x7F80u) == 0) h = 0;                  // flushed before the product; p >= 0
-                    pb[half * 4 + j] = h;
-                }
-            }
-            const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, u32x4{pb[0] | (pb[1] << 16), pb[2] | (pb[3] << 16),
-                                                                   pb[4] | (pb[5] << 16), pb[6] | (pb[7] << 16)});
+                // one rounding to BF16, then flushed like every matrix operand (p >= 0)
+                const bf16x8_t pf = __builtin_bit_cast(bf16x8_t,
+                        u32x4{daz2(pack_bf16(pr[0], pr[1])), daz2(pack_bf16(pr[2], pr[3])),
+                              daz2(pack_bf16(pr[4], pr[5])), daz2(pack_bf16(pr[6], pr[7]))});
 #pragma unroll
-            for (int dt = 0; dt < DT16; ++dt) {
-                const bf16x8_t vfr = __builtin_bit_cast(bf16x8_t,
-                        *reinterpret_cast<const u32x4*>(vf + ((uint64_t)g * a.d_tiles + dt) * kFrag));
-                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfr, pf, o[dt], 0, 0, 0);
+                for (int dt = 0; dt < DT16; ++dt)
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vfr[dt]), pf, o[dt], 0, 0, 0);
+                cur = nxt;
             }
+        }
+        if (SPLIT) {
+            if (wave != 0) {
+#pragma unroll
+                for (int dt = 0; dt < DT16; ++dt) wave_out[wave - 1][dt][lane] = o[dt];
+            }
+            __syncthreads();
+            if (wave != 0) continue;
+#pragma unroll
+            for (int w = 0; w < 3; ++w)
+#pragma unroll
+                for (int dt = 0; dt < DT16; ++dt) o[dt] += wave_out[w][dt][lane];
         }
         // lane holds out[row][head*D + 16*dt + 4*kg + j]
         if (!row_ok) continue;
@@ -234,15 +365,27 @@ __global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 + (uint64_t)(row >> 4) * a.out_tile_cols * kTileBytes + (row & 15u) * kRowBytes;
 #pragma unroll
         for (int dt = 0; dt < DT16; ++dt) {
+            float val[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const uint32_t d = dt * kTile + 4 * kg + j;
+                val[j] = o[dt][j];
+                if (val[j] == 0.0f) val[j] = 0.0f;                    // -0 is stored as +0
+            }
+            const uint32_t d = dt * kTile + 4 * kg, col = head * a.D + d;
+            if ((a.D & 3u) == 0) {
+                // the four outputs lie in one tile row of out
                 if (d >= a.D) continue;
-                float val = o[dt][j];
-                if (val == 0.0f) val = 0.0f;                          // -0 is stored as +0
-                const uint32_t bits = nan_row ? 0x7FC0u : bf16_rne_sw(as_u32(val));
-                const uint32_t col = head * a.D + d;
-                *reinterpret_cast<uint16_t*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) = (uint16_t)bits;
+                const u32x2 bits = nan_row ? u32x2{0x7FC07FC0u, 0x7FC07FC0u}
+                                           : u32x2{pack_bf16(val[0], val[1]), pack_bf16(val[2], val[3])};
+                *reinterpret_cast<u32x2*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) = bits;
+                continue;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (d + j >= a.D) continue;
+                const uint32_t bits = nan_row ? 0x7FC0u : bf16_rne_sw(as_u32(val[j]));
+                const uint32_t cj = col + j;
+                *reinterpret_cast<uint16_t*>(ob + (uint64_t)(cj >> 4) * kTileBytes + (cj & 15u) * 2) = (uint16_t)bits;
             }
         }
     }
@@ -254,14 +397,23 @@ __global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 // the tokens; lanes only divide the tokens (scores) or the features (outputs).
 __global__ __launch_bounds__(64) void sdpa_rows_kernel(const SdpaArgs a) {
     __shared__ float pbuf[64];
-    if (a.guarded && *a.flag == 0u) return;
     const uint32_t lane = threadIdx.x;
-    const uint32_t row = blockIdx.x, head = blockIdx.y;
-    const uint32_t hkv = head / a.grouping;
-    const uint32_t reach = a.a + row + 1;
-    const uint32_t vis = reach < a.L ? reach : a.L;
     const float inf = __builtin_inff();
-    for (uint32_t p = blockIdx.z; p < a.planes; p += gridDim.z) {
+    // blockIdx.y walks the (plane, KV head) pairs, blockIdx.x the rows of the pair's
+    // query heads; a guarded launch leaves a pair whose flags are all down at once
+    const uint32_t pairs = a.planes * a.Hkv, per_pair = a.grouping * a.R;
+    for (uint32_t pair = blockIdx.y; pair < pairs; pair += gridDim.y) {
+      const uint32_t p = pair / a.Hkv, hkv = pair - p * a.Hkv;
+      if (a.guarded) {
+          uint32_t up = 0;
+          for (uint32_t i = 0; i < a.pack_splits; ++i) up |= a.flags[(uint64_t)pair * a.pack_splits + i];
+          if (up == 0) continue;            // uniform: every lane reads the same words
+      }
+      for (uint32_t it = blockIdx.x; it < per_pair; it += gridDim.x) {
+        const uint32_t hg = it / a.R, row = it - hg * a.R;
+        const uint32_t head = hkv * a.grouping + hg;
+        const uint32_t reach = a.a + row + 1;
+        const uint32_t vis = reach < a.L ? reach : a.L;
         uint64_t plane[4];
         walk_planes(a.walk, p, plane);
         const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes
@@ -356,6 +508,7 @@ __global__ __launch_bounds__(64) void sdpa_rows_kernel(const SdpaArgs a) {
             if (val == 0.0f) val = 0.0f;
             store(d, bf16_rne_sw(as_u32(val)));
         }
+      }
     }
 }
 
@@ -396,16 +549,34 @@ int sdpa_shape(const iomx_view* q, const iomx_view* k, const iomx_view* v, const
     return IOMX_OK;
 }
 
-constexpr uint64_t kSdpaHeader = 256;   // the flag word, padded so that the fragments stay aligned
 constexpr uint64_t kMaxMfmaHeadDim = 128;
 
-int sdpa_packed_bytes(const SdpaShape& s, uint64_t L, uint64_t* bytes) {
-    uint64_t n = s.planes;
-    if (mul_overflows(n, s.Hkv, &n) || mul_overflows(n, (L + 31) / 32, &n)
-        || mul_overflows(n, (s.D + 15) / 16, &n) || mul_overflows(n, (uint64_t)kFrag, &n)
-        || n > ~0ull - kSdpaHeader)
+// Workgroups that share the packing of one KV head: enough of them to occupy the
+// chip when planes * Hkv alone would not.
+uint32_t sdpa_pack_splits(const SdpaShape& s, uint64_t L) {
+    const uint64_t frags = ((L + 31) / 32) * ((s.D + 15) / 16);
+    const uint64_t heads = s.planes * s.Hkv;
+    uint64_t splits = heads >= 4096 ? 1 : (4096 + heads - 1) / heads;
+    const uint64_t most = (frags + 3) / 4;
+    if (splits > most) splits = most;
+    if (splits > 64) splits = 64;
+    return (uint32_t)(splits ? splits : 1);
+}
+
+// header (one flag word per plane, KV head and pack split, rounded up to 256 bytes),
+// the V fragments, then the flushed K tiles (the same number of bytes)
+int sdpa_layout(const SdpaShape& s, uint64_t L, uint64_t* header, uint64_t* region, uint64_t* bytes) {
+    uint64_t heads = s.planes, n, h, total;
+    if (mul_overflows(heads, s.Hkv, &heads)) return IOMX_ERR_OVERFLOW;
+    if (mul_overflows(heads, (uint64_t)sdpa_pack_splits(s, L) * 4, &h) || h > ~0ull - 255) return IOMX_ERR_OVERFLOW;
+    h = (h + 255) & ~255ull;
+    if (mul_overflows(heads, (L + 31) / 32, &n) || mul_overflows(n, (s.D + 15) / 16, &n)
+        || mul_overflows(n, (uint64_t)kFrag, &n) || mul_overflows(n, (uint64_t)2, &total)
+        || total > ~0ull - h)
         return IOMX_ERR_OVERFLOW;
-    *bytes = n + kSdpaHeader;
+    *header = h;
+    *region = n;
+    *bytes = total + h;
     return IOMX_OK;
 }
 
@@ -424,7 +595,8 @@ extern "C" int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_vie
     if (dtype != IOMX_DT_BF16) return IOMX_ERR_UNSUPPORTED;
     *alignment = 256;
     if (s.D > kMaxMfmaHeadDim) { *bytes = 0; *alignment = 1; return IOMX_OK; }
-    return sdpa_packed_bytes(s, L, bytes);
+    uint64_t header, region;
+    return sdpa_layout(s, L, &header, &region, bytes);
 }
 
 extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
@@ -469,41 +641,62 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
     g.planes = (uint32_t)g.walk.planes;
     g.groups = (uint32_t)((L + 31) / 32);
     g.scale = sqrtf((float)s.D);
+    {
+        int e = 0;
+        g.inv_scale = frexpf(g.scale, &e) == 0.5f ? 1.0f / g.scale : 0.0f;
+    }
     if (s.Hq > 65535u || s.R > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
     const hipStream_t st = native(stream);
     const uint32_t gz = g.planes < 65535u ? g.planes : 65535u;
 
     bool matrix_cores = path == 0 && s.D <= kMaxMfmaHeadDim;
+    uint64_t header = 0, region = 0;
     if (matrix_cores) {
         uint64_t need;
-        IOMX_TRY(sdpa_packed_bytes(s, L, &need));
+        IOMX_TRY(sdpa_layout(s, L, &header, &region, &need));
         if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
             return IOMX_ERR_INVALID;
         if (s.Hkv > 65535u) matrix_cores = false;
     }
     if (matrix_cores) {
-        g.flag = static_cast<uint32_t*>(workspace);
-        g.packed_v = static_cast<uint8_t*>(workspace) + kSdpaHeader;
-        hipLaunchKernelGGL(sdpa_clear_flag_kernel, dim3(1), dim3(1), 0, st, g.flag);
-        const uint32_t frags = g.groups * g.d_tiles;
-        hipLaunchKernelGGL(sdpa_pack_v_kernel, dim3((frags + 3) / 4, g.Hkv, gz), dim3(256), 0, st, g);
-        const dim3 grid((g.R + kTile - 1) / kTile, (g.Hq + 3) / 4, gz);
+        // few row tiles against a long prefix: the waves of a workgroup split the tokens,
+        // and when all rows of a KV head's query heads fit one tile they share it
+        const uint32_t row_tiles = (g.R + kTile - 1) / kTile;
+        int mode = 0;
+        if ((uint64_t)g.grouping * g.R <= kTile && g.grouping > 1) mode = 2;
+        else if ((uint64_t)row_tiles * g.Hq * g.planes < 4096 && g.groups >= 8) mode = 1;
+        g.flags = static_cast<uint32_t*>(workspace);
+        g.packed_v = static_cast<uint8_t*>(workspace) + header;
+        g.packed_k = mode == 2 ? nullptr : g.packed_v + region;
+        g.pack_splits = sdpa_pack_splits(s, L);
+        hipLaunchKernelGGL(sdpa_pack_kernel, dim3(g.Hkv * g.pack_splits, gz), dim3(256), 0, st, g);
+        const dim3 grid(mode == 2 ? 1 : row_tiles, mode == 2 ? g.Hkv : mode == 1 ? g.Hq : (g.Hq + 3) / 4, gz);
+#define IOMX_SDPA(N) \
+    case N: \
+        if (mode == 2) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 2>), grid, dim3(256), 0, st, g); \
+        else if (mode == 1) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 1>), grid, dim3(256), 0, st, g); \
+        else hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 0>), grid, dim3(256), 0, st, g); \
+        break;
         switch (g.d_tiles) {
-            case 1: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<1>), grid, dim3(256), 0, st, g); break;
-            case 2: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<2>), grid, dim3(256), 0, st, g); break;
-            case 3: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<3>), grid, dim3(256), 0, st, g); break;
-            case 4: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<4>), grid, dim3(256), 0, st, g); break;
-            case 5: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<5>), grid, dim3(256), 0, st, g); break;
-            case 6: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<6>), grid, dim3(256), 0, st, g); break;
-            case 7: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<7>), grid, dim3(256), 0, st, g); break;
-            default: hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<8>), grid, dim3(256), 0, st, g); break;
+            IOMX_SDPA(1) IOMX_SDPA(2) IOMX_SDPA(3) IOMX_SDPA(4)
+            IOMX_SDPA(5) IOMX_SDPA(6) IOMX_SDPA(7)
+            default: IOMX_SDPA(8)
         }
+#undef IOMX_SDPA
         record_launch("sdpa_mfma", grid.x * grid.y * grid.z, 256, (uint64_t)g.planes * g.Hq * g.R);
         g.guarded = 1;
     }
-    const dim3 rows_grid(g.R, g.Hq, gz);
+    // one grid row per (plane, KV head) pair: when it only has to look at the flags it is
+    // gone in a few microseconds
+    const uint64_t pairs = (uint64_t)g.planes * g.Hkv, per_pair = (uint64_t)g.grouping * g.R;
+    if (pairs > 0x7FFFFFFFull || per_pair > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
+    const uint32_t gy = (uint32_t)(pairs < 65535 ? pairs : 65535);
+    uint64_t gx = matrix_cores ? (8192 + gy - 1) / gy : per_pair;     // guarded: a modest grid
+    if (gx > per_pair) gx = per_pair;
+    if (gx > 65535) gx = 65535;
+    const dim3 rows_grid((uint32_t)gx, gy);
     hipLaunchKernelGGL(sdpa_rows_kernel, rows_grid, dim3(64), 0, st, g);
-    if (!matrix_cores) record_launch("sdpa_rows", rows_grid.x * rows_grid.y * rows_grid.z, 64, (uint64_t)g.planes * g.Hq * g.R);
+    if (!matrix_cores) record_launch("sdpa_rows", rows_grid.x * rows_grid.y, 64, pairs * per_pair);
     IOMX_HIP(hipGetLastError());
     return IOMX_OK;
 }
