@@ -392,7 +392,7 @@ def wl_sdpa(timer, steps, warmup):
         r = report("sdpa_bf16_%s_B%d_Hq32_Hkv4_R%d_L%d_D64" % (name, B, R, L),
                    2 * (B * Hq * R * D * 2 + 2 * B * Hkv * L * D), B * Hq * R * D, wall, ev, "sdpa_mfma")
         r["TFLOP_per_s"] = round(flops / (ev * 1e-3) / 1e12, 2)
-        r["launches"] = "clear_flag + pack_v + sdpa_mfma + sdpa_rows (guard)"
+        r["launches"] = "sdpa_pack + sdpa_mfma + sdpa_rows (guarded)"
         out.append(r)
         for t in (q, k, v, o, ws):
             t.free()
@@ -590,7 +590,7 @@ def main():
     if not args.no_detail:
         for key in ("bcast_mul_bf16", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "copy_bf16", "add_f32",
                     "add_i32", "rmsnorm_bf16", "rmsnorm_f32", "silu_mul", "softmax", "softmax_causal",
-                    "chain", "layer_ops"):
+                    "chain", "layer_ops", "linear", "sdpa"):
             r = table[key]()
             detail.extend(r if isinstance(r, list) else [r])
     cpu = None if args.no_cpu else cpu_baseline()

@@ -134,20 +134,24 @@ struct RowStats {
     }
 };
 
-// One workgroup = four waves.  MODE 0: four heads of one row tile, each wave walks
+// MODE 0: a workgroup of four waves = four heads of one row tile, each wave walks
 // all visible tokens (prefill: many row tiles, K and V shared through the caches).
-// MODE 1: one head, the waves take every fourth 32-token group and meet in LDS (few
+// MODE 1: one head, the 4 or 8 waves share out the 32-token groups and meet in LDS (few
 // rows against a long prefix would otherwise be one wave's chain of dependent
 // loads).  MODE 2: the same split, and the 16 rows of the tile are the rows of all
 // query heads that share one KV head (grouping * R <= 16: a decode step reads K and
 // V once per KV head instead of once per query head).  In every mode the K
 // fragments of the next group are requested before the current group is multiplied.
+// waves of a workgroup: four heads, or as many token shares as LDS holds partial outputs for
+constexpr int sdpa_waves(int dt16, int mode) { return mode == 0 ? 4 : dt16 <= 4 ? 8 : 4; }
+
 template <int DT16, int MODE>
-__global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
+__global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     constexpr bool SPLIT = MODE != 0;
+    constexpr int NW = sdpa_waves(DT16, MODE);
     constexpr int D32 = (DT16 + 1) / 2;
-    __shared__ float wave_stats[4][16][5];
-    __shared__ f32x4_t wave_out[SPLIT ? 3 : 1][SPLIT ? DT16 : 1][64];
+    __shared__ float wave_stats[NW][16][5];
+    __shared__ f32x4_t wave_out[SPLIT ? NW - 1 : 1][SPLIT ? DT16 : 1][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
@@ -171,7 +175,7 @@ __global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     const uint32_t vis = row_ok ? (reach < a.L ? reach : a.L) : 0;     // tokens this lane's row sees
     const uint32_t vis_max = reach_max < a.L ? reach_max : a.L;        // ... and the tile's last row
     const uint32_t groups = (vis_max + 31) / 32;
-    const uint32_t g_first = SPLIT ? wave : 0, g_step = SPLIT ? 4 : 1;
+    const uint32_t g_first = SPLIT ? wave : 0, g_step = SPLIT ? NW : 1;
     const uint32_t c0 = (kg & 1u) * 8u;
     const float inf = __builtin_inff();
     for (uint32_t p = blockIdx.z; p < a.planes; p += gridDim.z) {
@@ -302,7 +306,7 @@ __global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             __syncthreads();
             st = RowStats{-inf, 0.0f, 0u, false, false};
 #pragma unroll
-            for (int w = 0; w < 4; ++w)
+            for (int w = 0; w < NW; ++w)
                 st.merge(wave_stats[w][l16][0], wave_stats[w][l16][1], as_u32(wave_stats[w][l16][2]),
                          wave_stats[w][l16][3] != 0.0f, wave_stats[w][l16][4] != 0.0f);
         }
@@ -354,8 +358,10 @@ __global__ __launch_bounds__(256) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             }
             __syncthreads();
             if (wave != 0) continue;
-#pragma unroll
-            for (int w = 0; w < 3; ++w)
+            // one wave's partial at a time (unrolled, the loads of all of them would be
+            // hoisted and would not fit the register file)
+#pragma unroll 1
+            for (int w = 0; w < NW - 1; ++w)
 #pragma unroll
                 for (int dt = 0; dt < DT16; ++dt) o[dt] += wave_out[w][dt][lane];
         }
@@ -673,8 +679,8 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         const dim3 grid(mode == 2 ? 1 : row_tiles, mode == 2 ? g.Hkv : mode == 1 ? g.Hq : (g.Hq + 3) / 4, gz);
 #define IOMX_SDPA(N) \
     case N: \
-        if (mode == 2) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 2>), grid, dim3(256), 0, st, g); \
-        else if (mode == 1) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 1>), grid, dim3(256), 0, st, g); \
+        if (mode == 2) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 2>), grid, dim3(sdpa_waves(N, 2) * 64), 0, st, g); \
+        else if (mode == 1) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 1>), grid, dim3(sdpa_waves(N, 1) * 64), 0, st, g); \
         else hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 0>), grid, dim3(256), 0, st, g); \
         break;
         switch (g.d_tiles) {
