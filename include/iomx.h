@@ -273,8 +273,9 @@ int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const 
  *
  * iomx_sdpa_workspace is the pure requirement query (sdpa_workspace_requirements):
  * the bytes and alignment of caller workspace iomx_launch_sdpa needs for these
- * operands (the transposed copy of the visible V prefix and one flag word; 0 when D
- * exceeds what the matrix-core kernel covers).  path 0 runs the matrix-core kernel
+ * operands (the packed V fragments and flushed K tiles of the visible prefix and one
+ * flag word per plane, KV head and pack share; 0 when D exceeds what the matrix-core
+ * kernel covers).  The workspace needs no initialisation and must be 256-byte aligned.  path 0 runs the matrix-core kernel
  * (D <= 128) followed by the reference-order kernel, which returns at once unless V
  * holds an infinity or NaN; path 1 runs the reference-order kernel alone (D <= 256,
  * no workspace).
