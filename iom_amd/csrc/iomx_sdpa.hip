@@ -39,7 +39,8 @@ struct SdpaArgs {
     uint32_t pack_splits;       // workgroups sharing the fragments of one KV head
     uint32_t guarded;           // sdpa_rows: skip the rows whose KV head has no flag up
     float scale;                // sqrtf(D)
-    float inv_scale;            // 1 / scale when that is a power of two (the product is then the quotient), else 0
+    float inv_scale;            // 1 / scale, rounded
+    uint32_t scale_pow2;        // scale is a power of two: the product with inv_scale is the quotient
 };
 
 constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
@@ -142,10 +143,11 @@ struct RowStats {
 // query heads that share one KV head (grouping * R <= 16: a decode step reads K and
 // V once per KV head instead of once per query head).  In every mode the K
 // fragments of the next group are requested before the current group is multiplied.
+// FULLD: D is a multiple of 32, no operand load needs a guard against the columns past D.
 // waves of a workgroup: four heads, or as many token shares as LDS holds partial outputs for
 constexpr int sdpa_waves(int dt16, int mode) { return mode == 0 ? 4 : dt16 <= 4 ? 8 : 4; }
 
-template <int DT16, int MODE>
+template <int DT16, int MODE, bool FULLD>
 __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     constexpr bool SPLIT = MODE != 0;
     constexpr int NW = sdpa_waves(DT16, MODE);
@@ -183,14 +185,17 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
         walk_planes(a.walk, p, plane);
         const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
         const uint8_t* kb = a.k + (plane[1] + (uint64_t)hkv * a.k_head_stride) * a.kv_plane_bytes;
-        const uint8_t* vf = a.packed_v + (((uint64_t)p * a.Hkv + hkv) * a.groups) * a.d_tiles * kFrag + lane * 16;
+        // wave-uniform bases and 32-bit lane offsets: the packed region of one KV head is far
+        // below 4 GiB, and 64-bit addresses per load would cost the registers of a whole wave slot
+        const uint8_t* vf = a.packed_v + (((uint64_t)p * a.Hkv + hkv) * a.groups) * a.d_tiles * kFrag;
+        const uint32_t vf_lane = lane * 16;
         // the row tile of Q, flushed, as the B operand of every score tile
         bf16x8_t qf[D32];
 #pragma unroll
         for (int c = 0; c < D32; ++c) {
             const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
             qf[c] = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
-            if (i0 < a.D)
+            if (FULLD || i0 < a.D)
                 qf[c] = daz8(load_k8_bits(qb + ((uint64_t)(qrow >> 4) * a.d_tiles + tile) * kTileBytes
                                                   + (qrow & 15u) * kRowBytes, c0, i0, a.D));
         }
@@ -200,8 +205,8 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
         struct KGroup { u32x4 w[2][D32]; };
         constexpr bool KPACK = MODE != 2;      // the flushed copy pays when many waves meet each tile
         const uint8_t* kp = KPACK ? a.packed_k + (((uint64_t)p * a.Hkv + hkv) * a.groups * 2) * a.d_tiles * kTileBytes
-                                           + l16 * kRowBytes + c0 * 2
                                   : nullptr;
+        const uint32_t kp_lane = l16 * kRowBytes + c0 * 2;
         auto load_k = [&](uint32_t g, KGroup& kgp) {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
@@ -210,9 +215,9 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
                     for (int c = 0; c < D32; ++c) {
                         const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
                         kgp.w[half][c] = u32x4{0, 0, 0, 0};
-                        if (i0 < a.D)
+                        if (FULLD || i0 < a.D)
                             kgp.w[half][c] = *reinterpret_cast<const u32x4*>(
-                                    kp + ((uint64_t)(2 * g + half) * a.d_tiles + tile) * kTileBytes);
+                                    kp + (((2 * g + half) * a.d_tiles + tile) * kTileBytes + kp_lane));
                     }
                     continue;
                 }
@@ -223,8 +228,9 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
                 for (int c = 0; c < D32; ++c) {
                     const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
                     kgp.w[half][c] = u32x4{0, 0, 0, 0};
-                    if (i0 < a.D) {
-                        const u32x4 w = load_k8_bits(krow + (uint64_t)tile * kTileBytes, c0, i0, a.D);
+                    if (FULLD || i0 < a.D) {
+                        const u32x4 w = FULLD ? *reinterpret_cast<const u32x4*>(krow + (uint64_t)tile * kTileBytes + c0 * 2)
+                                              : load_k8_bits(krow + (uint64_t)tile * kTileBytes, c0, i0, a.D);
                         kgp.w[half][c] = u32x4{daz2(w[0]), daz2(w[1]), daz2(w[2]), daz2(w[3])};
                     }
                 }
@@ -238,14 +244,18 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
 #pragma unroll
                 for (int c = 0; c < D32; ++c)
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kgp.w[half][c]), qf[c], acc, 0, 0, 0);
-                if (a.inv_scale != 0.0f) {
+                // dot / sqrt(D): the product with the reciprocal is the quotient when sqrt(D) is
+                // a power of two; otherwise one correction step of the remainder makes it the
+                // correctly rounded quotient in all but halfway cases of the last bit
+                f32x4_t q = acc * a.inv_scale;
+                if (!a.scale_pow2) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[j] = acc[j] * a.inv_scale;   // sqrt(D) is a power of two
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[j] = acc[j] / a.scale;
+                    for (int j = 0; j < 4; ++j) {
+                        const float refined = __builtin_fmaf(__builtin_fmaf(-q[j], a.scale, acc[j]), a.inv_scale, q[j]);
+                        q[j] = __builtin_fabsf(q[j]) < __builtin_inff() ? refined : q[j];   // inf - inf is not a remainder
+                    }
                 }
-                s[half] = acc;
+                s[half] = q;
             }
         };
         // pass 1: the row's statistics
@@ -253,11 +263,13 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
         {
             KGroup cur, nxt;
             if (g_first < groups) load_k(g_first, cur);
+#pragma unroll 1
             for (uint32_t g = g_first; g < groups; g += g_step) {
                 if (g + g_step < groups) load_k(g + g_step, nxt);     // the next group is in flight meanwhile
                 f32x4_t s[2];
                 scores(cur, s);
-                // the finite maximum of the lane's eight scores first, then one rescale
+                // the finite maximum of the lane's eight scores first, then one rescale; written
+                // with selects only (a branch per element would cost more than the arithmetic)
                 float local = -inf;
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
@@ -265,25 +277,21 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
                     for (int j = 0; j < 4; ++j) {
                         const bool seen = 32 * g + 16 * half + 4 * kg + j < vis;
                         const float v = s[half][j];
-                        if (seen) {
-                            st.nan = st.nan || v != v;
-                            st.pinf += v == inf ? 1u : 0u;
-                        }
+                        st.nan = st.nan | (seen & (v != v));
+                        st.pinf += (seen & (v == inf)) ? 1u : 0u;
                         // masked, NaN and infinite scores take no part in the sum
-                        s[half][j] = (seen && v - v == 0.0f) ? v : -inf;
-                        local = s[half][j] > local ? s[half][j] : local;
+                        s[half][j] = (seen & (__builtin_fabsf(v) < inf)) ? v : -inf;
+                        local = __builtin_fmaxf(local, s[half][j]);
                     }
-                if (local > st.m) {
-                    st.sum *= __expf(st.m - local);
-                    st.m = local;
-                    st.finite = true;
-                }
-                if (st.finite) {
+                const float newm = __builtin_fmaxf(st.m, local);
+                st.sum = newm == st.m ? st.sum : st.sum * __expf(st.m - newm);   // exp(-inf) = 0
+                st.m = newm;
+                st.finite = st.finite | (local > -inf);
 #pragma unroll
-                    for (int half = 0; half < 2; ++half)
+                for (int half = 0; half < 2; ++half)
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) st.sum += __expf(s[half][j] - st.m);   // exp(-inf) = 0
-                }
+                    for (int j = 0; j < 4; ++j)
+                        st.sum += s[half][j] == -inf ? 0.0f : __expf(s[half][j] - newm);
                 cur = nxt;
             }
         }
@@ -320,12 +328,13 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
         {
             KGroup cur, nxt;
             if (g_first < groups) load_k(g_first, cur);
+#pragma unroll 1
             for (uint32_t g = g_first; g < groups; g += g_step) {
                 if (g + g_step < groups) load_k(g + g_step, nxt);
                 u32x4 vfr[DT16];
 #pragma unroll
                 for (int dt = 0; dt < DT16; ++dt)
-                    vfr[dt] = *reinterpret_cast<const u32x4*>(vf + ((uint64_t)g * a.d_tiles + dt) * kFrag);
+                    vfr[dt] = *reinterpret_cast<const u32x4*>(vf + ((g * a.d_tiles + dt) * kFrag + vf_lane));
                 f32x4_t s[2];
                 scores(cur, s);
                 float pr[8];
@@ -334,12 +343,10 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float v = s[half][j];
-                        float e = 0.0f;
-                        if (32 * g + 16 * half + 4 * kg + j < vis && !nan_row) {
-                            if (st.pinf) e = v == inf ? pinf_p : 0.0f;
-                            else if (v != -inf) e = __expf(v - st.m) * inv_sum;
-                        }
-                        pr[half * 4 + j] = e;
+                        const bool seen = (32 * g + 16 * half + 4 * kg + j < vis) & !nan_row;
+                        const float regular = v == -inf ? 0.0f : __expf(v - st.m) * inv_sum;
+                        const float special = v == inf ? pinf_p : 0.0f;
+                        pr[half * 4 + j] = seen ? (st.pinf ? special : regular) : 0.0f;
                     }
                 // one rounding to BF16, then flushed like every matrix operand (p >= 0)
                 const bf16x8_t pf = __builtin_bit_cast(bf16x8_t,
@@ -649,7 +656,8 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
     g.scale = sqrtf((float)s.D);
     {
         int e = 0;
-        g.inv_scale = frexpf(g.scale, &e) == 0.5f ? 1.0f / g.scale : 0.0f;
+        g.scale_pow2 = frexpf(g.scale, &e) == 0.5f ? 1u : 0u;
+        g.inv_scale = 1.0f / g.scale;
     }
     if (s.Hq > 65535u || s.R > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
     const hipStream_t st = native(stream);
@@ -677,17 +685,22 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         g.pack_splits = sdpa_pack_splits(s, L);
         hipLaunchKernelGGL(sdpa_pack_kernel, dim3(g.Hkv * g.pack_splits, gz), dim3(256), 0, st, g);
         const dim3 grid(mode == 2 ? 1 : row_tiles, mode == 2 ? g.Hkv : mode == 1 ? g.Hq : (g.Hq + 3) / 4, gz);
+        const bool full_d = (g.D & 31u) == 0;
+#define IOMX_SDPA_MODE(N, M) \
+    if (full_d) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, M, true>), grid, dim3(sdpa_waves(N, M) * 64), 0, st, g); \
+    else hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, M, false>), grid, dim3(sdpa_waves(N, M) * 64), 0, st, g)
 #define IOMX_SDPA(N) \
     case N: \
-        if (mode == 2) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 2>), grid, dim3(sdpa_waves(N, 2) * 64), 0, st, g); \
-        else if (mode == 1) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 1>), grid, dim3(sdpa_waves(N, 1) * 64), 0, st, g); \
-        else hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, 0>), grid, dim3(256), 0, st, g); \
+        if (mode == 2) { IOMX_SDPA_MODE(N, 2); } \
+        else if (mode == 1) { IOMX_SDPA_MODE(N, 1); } \
+        else { IOMX_SDPA_MODE(N, 0); } \
         break;
         switch (g.d_tiles) {
             IOMX_SDPA(1) IOMX_SDPA(2) IOMX_SDPA(3) IOMX_SDPA(4)
             IOMX_SDPA(5) IOMX_SDPA(6) IOMX_SDPA(7)
             default: IOMX_SDPA(8)
         }
+#undef IOMX_SDPA_MODE
 #undef IOMX_SDPA
         record_launch("sdpa_mfma", grid.x * grid.y * grid.z, 256, (uint64_t)g.planes * g.Hq * g.R);
         g.guarded = 1;
