@@ -9,6 +9,10 @@ oracle on sampled planes / rows, and through size-independent properties.
   config 4  softmax F32->BF16 [8,8,2048,2048] (1/16 of the planes of the benchmark
             shape; rows are independent) and SiLU then MUL BF16 [32768,5632]
   config 5  the six-operation layer chain over [64,512,.]   end to end
+  linear    [64,512,2048] x [2048,2048] BF16                exact one-hot / scaling properties,
+                                                            sampled rows within the native bound
+  attention 8 x 32/4 heads, R = L = 512, D = 64 BF16        uniform-score closed form, sampled
+                                                            rows against the oracle
 """
 import numpy as np
 import pytest
@@ -304,4 +308,91 @@ def test_config5_layer_chain_end_to_end():
     # prod multiplies an activation that may differ by one ulp: at most one product ulp more
     assert stats["prod"][0] <= 2
     for t in (x, attn, down, gate, up, w1, w2, n1, x2, n2, nxt, act, prod):
+        t.free()
+
+
+# ---- the matrix-core workloads of bench.py at their full sizes ----------------------------
+
+def test_linear_full_size_by_linearity_and_sampled_rows():
+    """[64,512,2048] x [2048,2048] on the workgroup-tiled kernel.  Properties that do not
+    depend on the size: a one-hot input row returns a weight column exactly (one product,
+    no rounding), a row scaled by a power of two returns the scaled result exactly, and
+    sampled rows meet the contract's BF16 bound against float64."""
+    B, S, I, O = 64, 512, 2048, 2048
+    rng = np.random.default_rng(7)
+    x = datagen.bf16_rne(datagen.normal_f32(B * S * I, 0, 1, 201)).reshape(B, S, I)
+    w = datagen.bf16_rne(datagen.normal_f32(O * I, 0, 0.02, 202)).reshape(O, I)
+    hot = [(0, 0, 5), (17, 300, 2047), (63, 511, 1024)]
+    for b, r, i in hot:
+        x[b, r, :] = 0
+        x[b, r, i] = 0x3F80                      # 1.0
+    x[5, 7] = x[4, 7]
+    x[5, 7] = np.where((x[5, 7] & 0x7F80) < 0x7E00, x[5, 7] + 0x0100, x[5, 7])   # times 4 (exponent + 2)
+    dx = iomx.DeviceTensor(DT_BF16, (B, S, I)); dx.view().from_host(x)
+    dw = iomx.DeviceTensor(DT_BF16, (O, I)); dw.view().from_host(w)
+    do = iomx.DeviceTensor(DT_BF16, (B, S, O))
+    assert iomx.linear(dx.view(), dw.view(), do.view(), 0, S, False, 1, O) == 0
+    assert iomx.last_launch().kernel.decode() == "linear_mfma_lds"
+    got = do.view().to_host()
+    for b, r, i in hot:
+        assert np.array_equal(got[b, r], w[:, i])
+    scaled = (x[5, 7] & 0x7F80) != (x[4, 7] & 0x7F80)
+    assert scaled.all()
+    a4 = datagen.bf16_to_f32(got[4, 7]).astype(np.float64) * 4
+    a5 = datagen.bf16_to_f32(got[5, 7]).astype(np.float64)
+    assert np.array_equal(a4, a5)
+    w64 = datagen.bf16_to_f32(w.reshape(-1)).astype(np.float64).reshape(O, I)
+    for b, r in [(0, 1), (31, 255), (63, 510)] + [tuple(rng.integers(0, [B, S])) for _ in range(5)]:
+        ref = datagen.bf16_to_f32(x[b, r]).astype(np.float64) @ w64.T
+        q = datagen.bf16_to_f32(datagen.bf16_rne(ref.astype(np.float32))).astype(np.float64)
+        g = datagen.bf16_to_f32(got[b, r]).astype(np.float64)
+        ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(q), 1e-30))) - 7)
+        assert (np.abs(g - q) <= np.maximum(np.maximum(ulp, 2.0 ** -7), 2.0 ** -6 * np.abs(q))).all()
+    for t in (dx, dw, do):
+        t.free()
+
+
+def test_attention_full_size_by_uniform_scores_and_sampled_rows():
+    """Prefill of the benchmark shape (8 sequences, 32 query / 4 KV heads, R = L = 512,
+    D = 64).  Heads whose queries are zero give every visible token the same probability:
+    the output row r is the running mean of V, computed here as the binary32 sum of
+    bf16(1/(r+1)) * v in float64 with the probability-rounding budget.  Sampled rows of
+    the other heads are compared with the CPU oracle under the reference's acceptance
+    rule."""
+    B, Hq, Hkv, R, D = 8, 32, 4, 512, 64
+    q = datagen.bf16_rne(datagen.normal_f32(B * Hq * R * D, 0, 1, 211)).reshape(B, Hq, R, D)
+    k = datagen.bf16_rne(datagen.normal_f32(B * Hkv * R * D, 0, 1, 212)).reshape(B, Hkv, R, D)
+    v = datagen.bf16_rne(datagen.normal_f32(B * Hkv * R * D, 0, 1, 213)).reshape(B, Hkv, R, D)
+    q[:, 3] = 0
+    q[:, 20] = 0
+    dq = iomx.DeviceTensor(DT_BF16, (B, Hq, R, D)); dq.view().from_host(q)
+    dk = iomx.DeviceTensor(DT_BF16, (B, Hkv, R, D)); dk.view().from_host(k)
+    dv = iomx.DeviceTensor(DT_BF16, (B, Hkv, R, D)); dv.view().from_host(v)
+    do = iomx.DeviceTensor(DT_BF16, (B, R, Hq * D))
+    rc, nbytes, _ = iomx.sdpa_workspace(dq.view(), dk.view(), dv.view(), do.view(), 0, R)
+    assert rc == 0
+    ws = iomx.Buffer(nbytes)
+    assert iomx.sdpa(dq.view(), dk.view(), dv.view(), do.view(), 0, R, ws) == 0
+    iomx.synchronize()
+    got = do.view().to_host()
+    for b, h in ((0, 3), (7, 20)):
+        vv = datagen.bf16_to_f32(v[b, h // 8].reshape(-1)).astype(np.float64).reshape(R, D)
+        n = np.arange(1, R + 1, dtype=np.float32)
+        p = datagen.bf16_to_f32(datagen.bf16_rne((np.float32(1) / n).astype(np.float32))).astype(np.float64)
+        want = np.cumsum(vv, axis=0) * p[:, None]
+        budget = 2.0 ** -8 * (np.cumsum(np.abs(vv), axis=0) * p[:, None]) + 2.0 ** -8 * np.abs(want) + 2.0 ** -20
+        g = datagen.bf16_to_f32(got[b, :, h * D:(h + 1) * D].reshape(-1)).astype(np.float64).reshape(R, D)
+        assert (np.abs(g - want) <= budget).all()
+    # sampled rows against the oracle: a one-row attention at position r over r+1 tokens
+    from test_oracle_sdpa import bf16_class, matches
+    for b, r in ((0, 0), (2, 17), (5, 255), (7, 511)):
+        hq = iomo.HostTensor(DT_BF16, (Hq, 1, D)); hq.view().from_logical(q[b, :, r:r + 1])
+        hk = iomo.HostTensor(DT_BF16, (Hkv, R, D)); hk.view().from_logical(k[b])
+        hv = iomo.HostTensor(DT_BF16, (Hkv, R, D)); hv.view().from_logical(v[b])
+        ho = iomo.HostTensor(DT_BF16, (1, Hq * D))
+        assert iomo.sdpa(hq.view(), hk.view(), hv.view(), ho.view(), r, r + 1) == 0
+        want = ho.view().to_logical().reshape(-1)
+        bad = [i for i, (g, w) in enumerate(zip(got[b, r], want)) if not matches(int(g), int(w), bf16_class(int(w)))]
+        assert len(bad) <= 2, (b, r, bad[:5])          # the fixture rule is not a cancellation bound
+    for t in (dq, dk, dv, do, ws):
         t.free()
