@@ -399,6 +399,76 @@ def wl_sdpa(timer, steps, warmup):
     return out
 
 
+def wl_decoder_layer(timer, steps, warmup):
+    """Every operation of one TinyLlama-1.1B decoder layer (hidden 2048, 32 query / 4 KV heads
+    of 64, FFN 5632), BF16, in the order of the reference session: rmsnorm, q/k/v
+    projections (head planar), rope on q and k, cache append of k and v, attention, output
+    projection, residual add, rmsnorm, gate / up projections, silu * up, down projection,
+    residual add.  Prefill: 8 sequences of 512 tokens into an empty 512-token cache; decode:
+    one token for 64 sequences at position 511.  Each operation is also timed alone."""
+    out = []
+    H, Hq, Hkv, D, FF, C = 2048, 32, 4, 64, 5632, 512
+    st = timer.stream
+    for name, B, S, a in (("prefill", 8, 512, 0), ("decode", 64, 1, 511)):
+        L = a + S
+        x = device_tensor(BF16, (B, S, H), "normal", 121)
+        w_n1, w_n2 = (device_tensor(BF16, (1, H), "uniform_half_3half", s) for s in (122, 123))
+        wq, wo = (device_tensor(BF16, (H, H), "normal_0p02", s) for s in (124, 125))
+        wk, wv = (device_tensor(BF16, (Hkv * D, H), "normal_0p02", s) for s in (126, 127))
+        wg, wu = (device_tensor(BF16, (FF, H), "normal_0p02", s) for s in (128, 129))
+        wd = device_tensor(BF16, (H, FF), "normal_0p02", 130)
+        kc, vc = (device_tensor(BF16, (B, Hkv, C, D), "normal", s) for s in (131, 132))
+        n1, x1, n2, x2, attn, proj = (device_tensor(BF16, (B, S, H)) for _ in range(6))
+        q, qr = (device_tensor(BF16, (B, Hq, S, D)) for _ in range(2))
+        k, kr, v = (device_tensor(BF16, (B, Hkv, S, D)) for _ in range(3))
+        gate, up, act = (device_tensor(BF16, (B, S, FF)) for _ in range(3))
+        rc, nbytes, _ = iomx.sdpa_workspace(qr.view(), kc.view(), vc.view(), attn.view(), a, L)
+        check(rc, "sdpa_workspace")
+        ws = iomx.Buffer(nbytes)
+        ops = [
+            ("rmsnorm", lambda: iomx.rmsnorm(x.view(), w_n1.view(), n1.view(), 1e-5, st)),
+            ("linear_q", lambda: iomx.linear(n1.view(), wq.view(), q.view(), 0, S, True, Hq, D, 0, st)),
+            ("linear_k", lambda: iomx.linear(n1.view(), wk.view(), k.view(), 0, S, True, Hkv, D, 0, st)),
+            ("linear_v", lambda: iomx.linear(n1.view(), wv.view(), v.view(), 0, S, True, Hkv, D, 0, st)),
+            ("rope_q", lambda: iomx.rope(q.view(), qr.view(), a, 10000.0, st)),
+            ("rope_k", lambda: iomx.rope(k.view(), kr.view(), a, 10000.0, st)),
+            ("append_k", lambda: iomx.cache_append(kr.view(), kc.view(), a, st)),
+            ("append_v", lambda: iomx.cache_append(v.view(), vc.view(), a, st)),
+            ("sdpa", lambda: iomx.sdpa(qr.view(), kc.view(), vc.view(), attn.view(), a, L, ws, 0, st)),
+            ("linear_o", lambda: iomx.linear(attn.view(), wo.view(), proj.view(), 0, S, False, 1, H, 0, st)),
+            ("add_attn", lambda: iomx.binary(ADD, x.view(), proj.view(), x1.view(), st)),
+            ("rmsnorm_ffn", lambda: iomx.rmsnorm(x1.view(), w_n2.view(), n2.view(), 1e-5, st)),
+            ("linear_gate", lambda: iomx.linear(n2.view(), wg.view(), gate.view(), 0, S, False, 1, FF, 0, st)),
+            ("linear_up", lambda: iomx.linear(n2.view(), wu.view(), up.view(), 0, S, False, 1, FF, 0, st)),
+            ("silu_mul", lambda: iomx.silu_mul(gate.view(), up.view(), act.view(), st)),
+            ("linear_down", lambda: iomx.linear(act.view(), wd.view(), proj.view(), 0, S, False, 1, H, 0, st)),
+            ("add_ffn", lambda: iomx.binary(ADD, x1.view(), proj.view(), x2.view(), st)),
+        ]
+
+        def layer(i):
+            for label, op in ops:
+                check(op(), label)
+
+        wall, ev = timer.run(layer, steps, warmup)
+        each = {}
+        for label, op in ops:
+            _, e = timer.run(lambda i: check(op(), label), steps, 1)
+            each[label] = round(e * 1e3, 1)
+        tokens = B * S
+        weights = 2 * (2 * H * H + 2 * Hkv * D * H + 3 * FF * H)
+        flops = 2.0 * tokens * (weights / 2) + 4.0 * B * Hq * D * sum(min(L, a + r + 1) for r in range(S))
+        r = report("tinyllama_decoder_layer_bf16_%s_B%d_S%d" % (name, B, S), weights, tokens, wall, ev,
+                   "%d launches" % (len(ops) + 2))
+        r["TFLOP_per_s"] = round(flops / (ev * 1e-3) / 1e12, 1)
+        r["tokens_per_s_22_layers"] = round(tokens / (ev * 1e-3 * 22), 0)
+        r["us_per_op_alone"] = each
+        out.append(r)
+        for t in (x, w_n1, w_n2, wq, wo, wk, wv, wg, wu, wd, kc, vc, n1, x1, n2, x2, attn, proj, q, qr, k, kr, v,
+                  gate, up, act, ws):
+            t.free()
+    return out
+
+
 def wl_softmax(timer, steps, warmup, planes, heads, rows, cols, causal_position):
     """F32 scores [planes,heads,rows,cols] with the strict upper triangle = -inf as data.
     causal_position=False: a = cols-1, every token is positionally visible (the mask
@@ -575,6 +645,7 @@ def main():
         "layer_ops": lambda: wl_layer_ops(timer, max(K // 4, 5), max(W // 4, 2)),
         "linear": lambda: wl_linear(timer, max(K // 20, 5), 2),
         "sdpa": lambda: wl_sdpa(timer, max(K // 20, 5), 2),
+        "decoder_layer": lambda: wl_decoder_layer(timer, max(K // 20, 5), 2),
         "other_leaves": lambda: wl_other_leaves(timer, max(K // 10, 5), max(W // 10, 2)),
     }
 
@@ -590,7 +661,7 @@ def main():
     if not args.no_detail:
         for key in ("bcast_mul_bf16", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "copy_bf16", "add_f32",
                     "add_i32", "rmsnorm_bf16", "rmsnorm_f32", "silu_mul", "softmax", "softmax_causal",
-                    "chain", "layer_ops", "linear", "sdpa"):
+                    "chain", "layer_ops", "linear", "sdpa", "decoder_layer"):
             r = table[key]()
             detail.extend(r if isinstance(r, list) else [r])
     cpu = None if args.no_cpu else cpu_baseline()

@@ -458,10 +458,16 @@ __global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const Line
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-template <int KS, int DEPTH>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
-    constexpr int WM = 8, WN = 4;                 // wave tile, in 16x16 tiles
-    constexpr uint32_t BM = 16, BN = 16;          // workgroup tile, in 16x16 tiles
+template <int WM, int WVM, int WVN>
+__global__ __launch_bounds__(WVM * WVN * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
+    constexpr int WN = 4;                                   // wave tile WM x WN, in 16x16 tiles
+    constexpr int NW = WVM * WVN;                           // waves, WVM along the rows
+    constexpr uint32_t BM = WM * WVM, BN = WN * WVN;        // workgroup tile, in 16x16 tiles
+    constexpr int KS = 1, DEPTH = 4, HALF = WM / 2;
+    constexpr int LPS = (BM + BN) / NW;                     // direct loads per wave and stage
+    static_assert(LPS == 4 && BM == 2 * NW && BN == 2 * NW, "two row and two output fragments per wave");
+    static_assert(WM >= 4 && WM % 2 == 0 && LPS % HALF == 0, "loads spread over the second half of a stage");
     constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
     constexpr uint32_t kStageFrags = (BM + BN) * KS, kStageBytes = kStageFrags * kFrag;
     __shared__ __attribute__((aligned(16))) uint8_t lds[DEPTH * kStageBytes];
@@ -475,16 +481,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t bx = (sb / a.super_y) * 64 + xcd * 8 + jx, by = (sb % a.super_y) * 4 + jy;
     if (bx >= a.row_blocks || by >= a.out_blocks) return;
     const uint32_t bm0 = bx * BM, bn0 = by * BN;   // first row tile / output tile
-    const uint32_t wm = wave & 1u, wn = wave >> 1;
+    const uint32_t wm = wave % WVM, wn = wave / WVM;
 
-    // loader role: this wave brings in fragments wave, wave+8 (rows) and wave+16,
-    // wave+24 (outputs) of every 32-element slice; lane i fetches 16-byte chunk i
+    // loader role: this wave brings in row fragments wave, wave+NW and output fragments
+    // wave, wave+NW of every 32-element slice; lane i fetches 16-byte chunk i
     const uint32_t ld_tile = lane >> 5, ld_row = (lane & 31u) >> 1;
     const uint32_t ld_off = ld_tile * kTileBytes + (lane & 1u) * 16;
     const uint8_t* src[4];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        uint32_t idx = (bm0 + wave + 8 * j) * kTile + ld_row;
+        uint32_t idx = (bm0 + wave + NW * j) * kTile + ld_row;
         if (idx >= total_rows) idx = 0;            // valid memory; its results are not stored
         const uint32_t p = idx / a.R, r = idx - p * a.R;
         uint64_t plane[2];
@@ -495,7 +501,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        uint32_t o = (bn0 + wave + 8 * j) * kTile + ld_row;
+        uint32_t o = (bn0 + wave + NW * j) * kTile + ld_row;
         if (o >= a.O) o = 0;
         src[2 + j] = a.w + (uint64_t)(o >> 4) * a.w_tile_cols * kTileBytes + (o & 15u) * kRowBytes + ld_off;
     }
@@ -505,7 +511,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             const uint64_t goff = (uint64_t)(stage * KS + ks) * kFrag;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const uint32_t frag = ks * (BM + BN) + wave + 8 * j;
+                const uint32_t frag = ks * (BM + BN) + (j < 2 ? wave + NW * j : BM + wave + NW * (j - 2));
                 __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + goff),
                                                  (lptr_t)(lds + buf * kStageBytes + frag * kFrag), 16, 0, 0);
             }
@@ -525,16 +531,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // stage st every wave waits for its own loads of stage st+1 and meets the others
     // at the barrier: from there on stage st+1 is complete in LDS and nobody reads
     // stage st-1 any more, so the second half of the stage (a) requests stage st+3
-    // into the buffer of st-1, one direct load after every four MFMAs -- a direct load
+    // into the buffer of st-1, direct loads between the groups of four MFMAs -- a direct load
     // holds its wave at issue until the memory pipeline takes it, and the matrix
     // instructions issued before it keep the matrix core busy meanwhile -- and (b)
     // already reads the first operands of stage st+1, so the matrix core does not
     // drain at the stage boundary.
-    static_assert(KS == 1 && DEPTH == 4, "the schedule below is written for four 32-element stages");
     const uint32_t last = stages - 1;
 #pragma unroll
     for (uint32_t d = 0; d < 3; ++d) issue(d < stages ? d : last, d);
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPS) : "memory");
     __builtin_amdgcn_s_barrier();
     bf16x8_t wf[2][WN], xf[4];
     auto rd = [&](uint32_t ring, uint32_t frag) {
@@ -545,46 +550,51 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int n = 0; n < WN; ++n) wf[0][n] = rd(0, BM + wn * WN + n);
     xf[0] = rd(0, wm * WM);
     xf[1] = rd(0, wm * WM + 1);
-    // one stage; P = parity of the stage (which half of wf holds its output fragments)
+    // one stage = WM steps (one row fragment against the WN output fragments);
+    // P = parity of the stage (which half of wf holds its output fragments)
     auto stage = [&](auto parity, uint32_t st) {
         constexpr int P = decltype(parity)::value;
         const uint32_t ring = st & 3u, ring1 = (st + 1) & 3u, ring3 = (st + 3) & 3u;
         const uint64_t gnext = (uint64_t)(st + 3 < stages ? st + 3 : last) * kFrag;
 #pragma unroll
-        for (int step = 0; step < 4; ++step) {
-            xf[(step + 2) & 3] = rd(ring, wm * WM + step + 2);
+        for (int step = 0; step < HALF; ++step) {
+            xf[(step + 2) & 3] = rd(ring, wm * WM + step + 2);          // step + 2 < WM in this half
 #pragma unroll
             for (int n = 0; n < WN; ++n)
                 acc[step][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[P][n], xf[step & 3], acc[step][n], 0, 0, 0);
         }
 #pragma unroll
-        for (int step = 0; step < 4; ++step) {
+        for (int step = 0; step < HALF; ++step) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, WN, 0);
         }
-        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPS) : "memory");
         __builtin_amdgcn_s_barrier();
 #pragma unroll
-        for (int step = 4; step < 8; ++step) {
-            if (step < 6) xf[(step + 2) & 3] = rd(ring, wm * WM + step + 2);
-            else xf[(step + 2) & 3] = rd(ring1, wm * WM + step - 6);
-            if (step == 5) {
+        for (int step = HALF; step < WM; ++step) {
+            if (step + 2 < WM) xf[(step + 2) & 3] = rd(ring, wm * WM + step + 2);
+            else xf[(step + 2) & 3] = rd(ring1, wm * WM + step + 2 - WM);
+            if (step == HALF + 1) {
 #pragma unroll
                 for (int n = 0; n < WN; ++n) wf[P ^ 1][n] = rd(ring1, BM + wn * WN + n);
             }
 #pragma unroll
             for (int n = 0; n < WN; ++n)
                 acc[step][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[P][n], xf[step & 3], acc[step][n], 0, 0, 0);
-            const int j = step - 4;
-            __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + gnext),
-                                             (lptr_t)(lds + ring3 * kStageBytes + (wave + 8 * j) * kFrag), 16, 0, 0);
+#pragma unroll
+            for (int i = 0; i < LPS / HALF; ++i) {
+                const int j = (step - HALF) * (LPS / HALF) + i;
+                const uint32_t frag = j < 2 ? wave + NW * j : BM + wave + NW * (j - 2);
+                __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + gnext),
+                                                 (lptr_t)(lds + ring3 * kStageBytes + frag * kFrag), 16, 0, 0);
+            }
         }
 #pragma unroll
-        for (int step = 4; step < 8; ++step) {
-            if (step == 5) __builtin_amdgcn_sched_group_barrier(0x100, WN + 1, 0);
+        for (int step = HALF; step < WM; ++step) {
+            if (step == HALF + 1) __builtin_amdgcn_sched_group_barrier(0x100, WN + 1, 0);
             else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, WN, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, LPS / HALF, 0);
         }
     };
     uint32_t st = 0;
@@ -716,16 +726,21 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
         const uint32_t o_tiles = (a.O + kTile - 1) / kTile;
         if (total_rows <= 0x7FFFFFFFull && o_tiles <= 65535u * 8u) {
             const uint32_t row_tiles = (uint32_t)((total_rows + kTile - 1) / kTile);
-            if (path == 0 && row_tiles >= 16 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
-                // enough rows to fill 256-row workgroup tiles: operands staged through LDS
-                a.row_blocks = (row_tiles + 15) / 16;
-                a.out_blocks = (o_tiles + 15) / 16;
+            if (path == 0 && row_tiles >= 8 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
+                // enough rows for workgroup tiles: operands staged through LDS.  256 x 256
+                // outputs per workgroup when that still gives every CU two workgroups,
+                // 128 x 128 otherwise
+                const uint64_t big = (uint64_t)((row_tiles + 15) / 16) * ((o_tiles + 15) / 16);
+                const uint32_t bt = big >= 512 ? 16 : 8;
+                a.row_blocks = (row_tiles + bt - 1) / bt;
+                a.out_blocks = (o_tiles + bt - 1) / bt;
                 a.super_y = (a.out_blocks + 3) / 4;
                 const uint64_t wgs = (uint64_t)((a.row_blocks + 63) / 64) * a.super_y * 256;
                 if (wgs > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
                 const dim3 grid((uint32_t)wgs);
-                hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<1, 4>), grid, dim3(512), 0, st, a);
-                record_launch("linear_mfma_lds", grid.x, 512, (uint64_t)row_tiles * o_tiles);
+                if (bt == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4>), grid, dim3(512), 0, st, a);
+                else hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2>), grid, dim3(256), 0, st, a);
+                record_launch("linear_mfma_lds", grid.x, bt == 16 ? 512 : 256, (uint64_t)row_tiles * o_tiles);
             } else if (path == 0 && row_tiles < 16 && o_tiles <= 0x7FFFFFFFu) {
                 // few rows (decode, last-row logits): one output tile per workgroup, the
                 // inner axis split over its waves
