@@ -199,6 +199,60 @@ __global__ __launch_bounds__(256) void rope_pairs_kernel(const RopeArgs a) {
     }
 }
 
+// One row per plane (a decode step): every plane has the same position, so the 16
+// lanes of a group evaluate one angle each, exchange them, and then rotate the row
+// of 16 different planes: no lane repeats the powf / sincos work of another.
+template <int DT, typename T>
+__global__ __launch_bounds__(256) void rope_row_kernel(const RopeArgs a) {
+    constexpr int BITS = bits_of(DT);
+    constexpr int K = BITS / 2;
+    constexpr uint32_t kTileBytes = 32 * BITS;
+    const uint32_t g = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t r = g & 15u, q = g >> 4;
+    const uint32_t pg = a.col_tiles > 1 ? fast_div(q, a.div_col_tiles) : q;   // group of 16 planes
+    const uint32_t ptc = q - pg * a.col_tiles;
+    const uint32_t position = a.a;
+    T my_sine = (T)0, my_cosine = (T)1;
+    if (position != 0) rope_angle(ptc * kTile + r, a.width, position, (T)a.theta, &my_sine, &my_cosine);
+    T sine[kTile], cosine[kTile];
+    const int base = (int)(threadIdx.x & 63u & ~15u);
+#pragma unroll
+    for (int i = 0; i < (int)kTile; ++i) {          // every lane of the wave takes part
+        sine[i] = __shfl(my_sine, base + i);
+        cosine[i] = __shfl(my_cosine, base + i);
+    }
+    const uint64_t p = (uint64_t)pg * kTile + r;
+    if (p >= a.planes) return;
+    const uint64_t off0 = (uint64_t)ptc * kTileBytes;                 // row 0 of the first tile row
+    const uint64_t off1 = off0 + (uint64_t)(a.half >> 4) * kTileBytes;
+    uint64_t plane[2];
+    walk_planes(a.walk, (uint32_t)p, plane);
+    const uint8_t* xb = a.x + plane[0] * a.plane_bytes;
+    uint8_t* ob = a.out + plane[1] * a.plane_bytes;
+    uint32_t w0[K], w1[K];
+    load_row<BITS>(xb + off0, w0);
+    load_row<BITS>(xb + off1, w1);
+    if (position != 0) {
+        uint32_t r0[K], r1[K];
+#pragma unroll
+        for (int j = 0; j < K; ++j) { r0[j] = 0; r1[j] = 0; }
+#pragma unroll
+        for (int i = 0; i < (int)kTile; ++i) {
+            const T first = rope_decode<DT, T>(get<BITS>(w0, i));
+            const T second = rope_decode<DT, T>(get<BITS>(w1, i));
+            const T fc = first * cosine[i], ss = second * sine[i];
+            const T sc = second * cosine[i], fs = first * sine[i];
+            put<BITS>(r0, i, rope_encode<DT, T>(fc - ss));
+            put<BITS>(r1, i, rope_encode<DT, T>(sc + fs));
+        }
+        store_row<BITS>(ob + off0, r0, kTile);
+        store_row<BITS>(ob + off1, r1, kTile);
+    } else {
+        store_row<BITS>(ob + off0, w0, kTile);
+        store_row<BITS>(ob + off1, w1, kTile);
+    }
+}
+
 // Any even D: a lane owns one output tile row and fetches each partner element
 // from wherever the other half puts it.
 template <int DT, typename T>
@@ -296,7 +350,8 @@ uint32_t planes_in_grid(uint64_t lanes_per_plane, uint64_t planes) {
 
 template <int DT, typename T>
 void launch_rope(const RopeArgs& a, bool aligned, dim3 grid, hipStream_t s) {
-    if (aligned) hipLaunchKernelGGL((rope_pairs_kernel<DT, T>), grid, dim3(256), 0, s, a);
+    if (aligned && a.rows == 1) hipLaunchKernelGGL((rope_row_kernel<DT, T>), grid, dim3(256), 0, s, a);
+    else if (aligned) hipLaunchKernelGGL((rope_pairs_kernel<DT, T>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((rope_general_kernel<DT, T>), grid, dim3(256), 0, s, a);
 }
 
@@ -455,6 +510,13 @@ int iomx_launch_rope(int dtype, const iomx_view* x, const iomx_view* out, uint64
     dim3 grid;
     IOMX_TRY(plane_grid(m.tile_rows, k.col_tiles, k.walk.planes, &k.lanes_per_plane, &grid));
     grid.y = planes_in_grid(k.lanes_per_plane, k.walk.planes);
+    const bool single_row = aligned && k.rows == 1;
+    if (single_row) {
+        // 16 lanes = 16 planes of one pair tile
+        const uint64_t lanes = ((k.walk.planes + kTile - 1) / kTile) * k.col_tiles * kTile;
+        if (lanes > 0x7FFFFF00ull * 256) return IOMX_ERR_OVERFLOW;
+        grid = dim3((uint32_t)((lanes + 255) / 256), 1, 1);
+    }
     const hipStream_t s = native(stream);
     switch (dtype) {
         case DT_F4_E2M1: launch_rope<DT_F4_E2M1, float>(k, aligned, grid, s); break;
@@ -467,7 +529,7 @@ int iomx_launch_rope(int dtype, const iomx_view* x, const iomx_view* out, uint64
         case DT_F32: launch_rope<DT_F32, float>(k, aligned, grid, s); break;
         default: launch_rope<DT_F64, double>(k, aligned, grid, s); break;
     }
-    record_launch(aligned ? "rope_pairs" : "rope_general", grid.x, 256,
+    record_launch(single_row ? "rope_row" : aligned ? "rope_pairs" : "rope_general", grid.x, 256,
                   (uint64_t)k.lanes_per_plane * k.planes);
     IOMX_HIP(hipGetLastError());
     return IOMX_OK;

@@ -749,12 +749,19 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                 // otherwise up to four row tiles against one or two
                 const bool sparse_rows = a.R < kTile && a.planes > 1;
                 uint32_t mt, nt;
-                if (sparse_rows) { mt = 1; nt = 4; }
-                else { mt = row_tiles == 1 ? 1 : row_tiles == 2 ? 2 : 4; nt = mt == 1 ? 2 : 1; }
+                if (sparse_rows) {
+                    // ... as long as that still leaves a workgroup for every CU
+                    mt = 1;
+                    nt = 4;
+                    while (nt > 1 && (uint64_t)((o_tiles + nt - 1) / nt) * row_tiles < 256) nt /= 2;
+                } else {
+                    mt = row_tiles == 1 ? 1 : row_tiles == 2 ? 2 : 4;
+                    nt = mt == 1 ? 2 : 1;
+                }
                 const dim3 grid((o_tiles + nt - 1) / nt, (row_tiles + mt - 1) / mt);
 #define IOMX_SPLITK(M, N) \
     if (mt == M && nt == N) hipLaunchKernelGGL((linear_mfma_splitk_bf16_kernel<M, N>), grid, dim3(256), 0, st, a)
-                IOMX_SPLITK(1, 2); IOMX_SPLITK(1, 4); IOMX_SPLITK(2, 1); IOMX_SPLITK(4, 1);
+                IOMX_SPLITK(1, 1); IOMX_SPLITK(1, 2); IOMX_SPLITK(1, 4); IOMX_SPLITK(2, 1); IOMX_SPLITK(4, 1);
 #undef IOMX_SPLITK
                 record_launch("linear_mfma_splitk", grid.x * grid.y, 256, (uint64_t)row_tiles * o_tiles);
             } else if (row_tiles <= 4) {

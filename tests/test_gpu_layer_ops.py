@@ -237,7 +237,9 @@ def rope64(x, a, theta):
 @pytest.mark.parametrize("dtype", FLOAT_LEAVES, ids=names(FLOAT_LEAVES))
 @pytest.mark.parametrize("dims,a,family", [((2, 3, 5, 40), 1, "rope_general"), ((2, 3, 5, 40), 0, "rope_general"),
                                            ((2, 2, 33, 64), 0, "rope_pairs"), ((3, 4, 16, 128), 500, "rope_pairs"),
-                                           ((1, 1, 2, 2), 7, "rope_general")])
+                                           ((1, 1, 2, 2), 7, "rope_general"),
+                                           ((5, 7, 1, 64), 37, "rope_row"), ((3, 1, 32), 0, "rope_row"),
+                                           ((2, 40, 1, 128), 1023, "rope_row")])
 def test_rope_float_leaves(dtype, dims, a, family):
     theta = 10000.0
     vals = finite_values(dtype, int(np.prod(dims)), 41).reshape(dims)
@@ -274,6 +276,24 @@ def test_rope_float_leaves(dtype, dims, a, family):
     # tile padding of the output untouched: compare raw storage where every element agrees
     if equal == 1.0:
         assert same_storage(do, ho)
+    dx.free(); do.free()
+
+
+def test_rope_single_row_planes_through_views():
+    """A decode step: one row per plane, the planes reached through a permuted and sliced view."""
+    dims = (6, 9, 1, 64)
+    vals = finite_values(DT_BF16, int(np.prod(dims)), 45).reshape(dims)
+    dx, hx = pair(DT_BF16, dims, values=vals)
+    do, ho = pair(DT_BF16, (9, 3, 1, 64), salt=46)
+    xv = lambda t: t.view().permute([1, 0]).slice(1, 1, 3, 2)
+    assert iomx.rope(xv(dx), do.view(), 123, 10000.0) == 0
+    assert kernel_name() == "rope_row"
+    assert iomo.rope(xv(hx), ho.view(), 123, 10000.0) == 0
+    got, want = do.view().to_host(), ho.view().to_logical()
+    assert (np.abs(got.astype(np.int64) - want.astype(np.int64)) <= 1).all()
+    assert float((got == want).mean()) > 0.9
+    mask = iomo.tile_plane(np.ones((9, 3, 1, 64), np.uint16)) == 0
+    assert np.array_equal(do.raw()[mask], ho.storage[mask])      # the 15 padding rows of every tile untouched
     dx.free(); do.free()
 
 
