@@ -454,6 +454,12 @@ def wl_decoder_layer(timer, steps, warmup):
         for label, op in ops:
             _, e = timer.run(lambda i: check(op(), label), steps, 1)
             each[label] = round(e * 1e3, 1)
+        # the same sequence recorded once and replayed with one submission
+        st.begin_capture()
+        layer(0)
+        graph = st.end_capture()
+        _, ev_graph = timer.run(lambda i: graph.launch(st), steps, warmup)
+        graph.close()
         tokens = B * S
         weights = 2 * (2 * H * H + 2 * Hkv * D * H + 3 * FF * H)
         flops = 2.0 * tokens * (weights / 2) + 4.0 * B * Hq * D * sum(min(L, a + r + 1) for r in range(S))
@@ -461,6 +467,7 @@ def wl_decoder_layer(timer, steps, warmup):
                    "%d launches" % (len(ops) + 2))
         r["TFLOP_per_s"] = round(flops / (ev * 1e-3) / 1e12, 1)
         r["tokens_per_s_22_layers"] = round(tokens / (ev * 1e-3 * 22), 0)
+        r["ms_per_layer_replayed_graph"] = round(ev_graph, 5)
         r["us_per_op_alone"] = each
         out.append(r)
         for t in (x, w_n1, w_n2, wq, wo, wk, wv, wg, wu, wd, kc, vc, n1, x1, n2, x2, attn, proj, q, qr, k, kr, v,

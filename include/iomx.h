@@ -122,6 +122,22 @@ int iomx_event_synchronize(iomx_event_t event);
 int iomx_event_query(iomx_event_t event, int* done);
 int iomx_event_elapsed_ms(iomx_event_t start, iomx_event_t stop, float* ms);
 
+/*
+ * Recording and replay of a fixed sequence of launches (HIP graph).  No counterpart in
+ * the reference, which submits every operation separately: a caller that repeats the
+ * same sequence on the same buffers (a decode step is ~20 launches of a few
+ * microseconds each) records it once between begin and end on a stream created here
+ * and replays it with one submission.  Every iomx_launch_* entry point may be recorded
+ * (none allocates or clears memory with a memset node); host transfers and
+ * synchronisation calls may not.  Views, sizes and pointers are frozen into the
+ * recording.
+ */
+typedef struct iomx_graph_s* iomx_graph_t;
+int iomx_stream_begin_capture(iomx_stream_t stream);
+int iomx_stream_end_capture(iomx_stream_t stream, iomx_graph_t* graph);
+int iomx_graph_launch(iomx_graph_t graph, iomx_stream_t stream);
+int iomx_graph_destroy(iomx_graph_t graph);
+
 /* ---- operations ---------------------------------------------------------- */
 
 /*

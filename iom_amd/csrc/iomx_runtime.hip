@@ -184,6 +184,35 @@ int iomx_stream_synchronize(iomx_stream_t stream) {
     return IOMX_OK;
 }
 
+int iomx_stream_begin_capture(iomx_stream_t stream) {
+    if (!stream) return IOMX_ERR_INVALID;          // the null stream cannot be captured
+    IOMX_HIP(hipStreamBeginCapture(native(stream), hipStreamCaptureModeThreadLocal));
+    return IOMX_OK;
+}
+
+int iomx_stream_end_capture(iomx_stream_t stream, iomx_graph_t* graph) {
+    if (!stream || !graph) return IOMX_ERR_INVALID;
+    hipGraph_t recorded = nullptr;
+    IOMX_HIP(hipStreamEndCapture(native(stream), &recorded));
+    hipGraphExec_t exec = nullptr;
+    const hipError_t status = hipGraphInstantiate(&exec, recorded, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(recorded);
+    IOMX_HIP(status);
+    *graph = reinterpret_cast<iomx_graph_t>(exec);
+    return IOMX_OK;
+}
+
+int iomx_graph_launch(iomx_graph_t graph, iomx_stream_t stream) {
+    if (!graph) return IOMX_ERR_INVALID;
+    IOMX_HIP(hipGraphLaunch(reinterpret_cast<hipGraphExec_t>(graph), native(stream)));
+    return IOMX_OK;
+}
+
+int iomx_graph_destroy(iomx_graph_t graph) {
+    if (graph) IOMX_HIP(hipGraphExecDestroy(reinterpret_cast<hipGraphExec_t>(graph)));
+    return IOMX_OK;
+}
+
 int iomx_event_create(iomx_event_t* event, int enable_timing) {
     if (!event) return IOMX_ERR_INVALID;
     hipEvent_t e = nullptr;

@@ -57,6 +57,7 @@ SYMBOLS = [
     "iomx_memcpy_d2d_async", "iomx_stream_create", "iomx_stream_destroy",
     "iomx_stream_synchronize", "iomx_event_create", "iomx_event_destroy", "iomx_event_record",
     "iomx_event_synchronize", "iomx_event_query", "iomx_event_elapsed_ms",
+    "iomx_stream_begin_capture", "iomx_stream_end_capture", "iomx_graph_launch", "iomx_graph_destroy",
     "iomx_launch_linear", "iomx_sdpa_workspace", "iomx_launch_sdpa", "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
     "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul",
     "iomx_launch_copy", "iomx_launch_scatter", "iomx_launch_gather", "iomx_launch_softmax",
@@ -142,6 +143,10 @@ def lib() -> C.CDLL:
         l.iomx_event_elapsed_ms.argtypes = [P, P, C.POINTER(C.c_float)]
         l.iomx_launch_binary.argtypes = [C.c_int, C.c_int, VP, VP, VP, P]
         l.iomx_launch_rmsnorm.argtypes = [C.c_int, VP, VP, VP, C.c_float, P]
+        l.iomx_stream_begin_capture.argtypes = [P]
+        l.iomx_stream_end_capture.argtypes = [P, C.POINTER(C.c_void_p)]
+        l.iomx_graph_launch.argtypes = [P, P]
+        l.iomx_graph_destroy.argtypes = [P]
         l.iomx_launch_silu.argtypes = [C.c_int, VP, VP, P]
         l.iomx_launch_silu_mul.argtypes = [C.c_int, VP, VP, VP, P]
         l.iomx_launch_copy.argtypes = [C.c_int, VP, VP, P]
@@ -202,6 +207,29 @@ class Stream:
     def close(self):
         if self.h:
             lib().iomx_stream_destroy(self.h)
+            self.h = C.c_void_p()
+
+    def begin_capture(self):
+        check(lib().iomx_stream_begin_capture(self.h), "begin_capture")
+
+    def end_capture(self) -> "Graph":
+        g = C.c_void_p()
+        check(lib().iomx_stream_end_capture(self.h, C.byref(g)), "end_capture")
+        return Graph(g)
+
+
+class Graph:
+    """A recorded sequence of launches, replayed with one submission."""
+
+    def __init__(self, handle):
+        self.h = handle
+
+    def launch(self, stream: "Stream"):
+        check(lib().iomx_graph_launch(self.h, stream.h), "graph_launch")
+
+    def close(self):
+        if self.h:
+            lib().iomx_graph_destroy(self.h)
             self.h = C.c_void_p()
 
 
