@@ -381,7 +381,7 @@ def wl_sdpa(timer, steps, warmup):
         qv, ov = q.view(), o.view()
         rc, nbytes, _ = iomx.sdpa_workspace(qv, k.view(), v.view(), ov, a, L)
         check(rc, "sdpa_workspace")
-        ws = iomx.Buffer(nbytes)
+        ws = iomx.Buffer(nbytes) if nbytes else None
 
         def launch(i):
             check(iomx.sdpa(qv, k.view(), v.view(), ov, a, L, ws, 0, timer.stream), "sdpa")
@@ -390,11 +390,12 @@ def wl_sdpa(timer, steps, warmup):
         visible = sum(min(L, a + r + 1) for r in range(R))
         flops = 4.0 * B * Hq * D * visible
         r = report("sdpa_bf16_%s_B%d_Hq32_Hkv4_R%d_L%d_D64" % (name, B, R, L),
-                   2 * (B * Hq * R * D * 2 + 2 * B * Hkv * L * D), B * Hq * R * D, wall, ev, "sdpa_mfma")
+                   2 * (B * Hq * R * D * 2 + 2 * B * Hkv * L * D), B * Hq * R * D, wall, ev,
+                   iomx.last_launch().kernel.decode())
         r["TFLOP_per_s"] = round(flops / (ev * 1e-3) / 1e12, 2)
-        r["launches"] = "sdpa_pack + sdpa_mfma + sdpa_rows (guarded)"
+        r["launches"] = "sdpa_decode" if nbytes == 0 else "sdpa_pack + sdpa_mfma + sdpa_rows (guarded)"
         out.append(r)
-        for t in (q, k, v, o, ws):
+        for t in (q, k, v, o) + ((ws,) if ws else ()):
             t.free()
     return out
 

@@ -404,6 +404,278 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
     }
 }
 
+// Few rows per KV head (grouping * R <= 16: a decode step): one workgroup of eight waves
+// = one KV head of one plane, the 16 rows of its tile = the rows of all query heads of
+// that KV head, the waves share out the 32-token groups.  Scores come from the matrix
+// cores as in sdpa_mfma (K read from the cache as it lies, flushed in registers); the
+// product with V runs on the vector units straight from the cache -- lane = feature,
+// the probabilities of a group broadcast from LDS -- so nothing is packed or
+// transposed, no workspace is used, and a token a row must not see is left out of that
+// row's sum by a select (an infinite V there cannot reach it).
+template <int DT16>
+__global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a) {
+    constexpr int D32 = (DT16 + 1) / 2;
+    constexpr int NW = 8;
+    constexpr int DL = (DT16 + 3) / 4;                 // features per lane (lane, lane + 64)
+    __shared__ float wave_stats[NW][16][5];
+    __shared__ __attribute__((aligned(16))) float p_tile[NW][16][32];
+    __shared__ float o_part[NW][16][DL * 64];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t l16 = lane & 15u, kg = lane >> 4;
+    const uint32_t hkv = blockIdx.x;
+    const uint32_t row = l16 / a.grouping;                            // the lane's tile row: (row, query head)
+    const uint32_t head = hkv * a.grouping + (l16 - row * a.grouping);
+    const bool row_ok = row < a.R;
+    const uint32_t qrow = row_ok ? row : a.R - 1;
+    const uint32_t nrows = a.grouping * a.R;                          // tile rows in use
+    const uint32_t reach = a.a + row + 1, reach_max = a.a + a.R;
+    const uint32_t vis = row_ok ? (reach < a.L ? reach : a.L) : 0;
+    const uint32_t vis_max = reach_max < a.L ? reach_max : a.L;
+    const uint32_t groups = (vis_max + 31) / 32;
+    const uint32_t c0 = (kg & 1u) * 8u;
+    const float inf = __builtin_inff();
+    for (uint32_t p = blockIdx.y; p < a.planes; p += gridDim.y) {
+        uint64_t plane[4];
+        walk_planes(a.walk, p, plane);
+        const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
+        const uint8_t* kb = a.k + (plane[1] + (uint64_t)hkv * a.k_head_stride) * a.kv_plane_bytes;
+        const uint8_t* vb = a.v + (plane[2] + (uint64_t)hkv * a.v_head_stride) * a.kv_plane_bytes;
+        bf16x8_t qf[D32];
+#pragma unroll
+        for (int c = 0; c < D32; ++c) {
+            const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
+            qf[c] = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
+            if (i0 < a.D)
+                qf[c] = daz8(load_k8_bits(qb + ((uint64_t)(qrow >> 4) * a.d_tiles + tile) * kTileBytes
+                                                  + (qrow & 15u) * kRowBytes, c0, i0, a.D));
+        }
+        // K of group g (two 16-token tiles), requested one group ahead of its use
+        struct KGroup { u32x4 w[2][D32]; };
+        auto load_k = [&](uint32_t g, KGroup& kgp) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                uint32_t token = 32 * g + 16 * half + l16;
+                if (token >= a.L) token = a.L - 1;                    // the cache tail is never touched
+                const uint8_t* krow = kb + (uint64_t)(token >> 4) * a.d_tiles * kTileBytes + (token & 15u) * kRowBytes;
+#pragma unroll
+                for (int c = 0; c < D32; ++c) {
+                    const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
+                    kgp.w[half][c] = u32x4{0, 0, 0, 0};
+                    if (i0 < a.D) kgp.w[half][c] = load_k8_bits(krow + (uint64_t)tile * kTileBytes, c0, i0, a.D);
+                }
+            }
+        };
+        // scores: lane gets tokens 32g + 16*half + 4*kg + j (j < 4) of tile row l16
+        auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2]) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int c = 0; c < D32; ++c)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(daz8(kgp.w[half][c]), qf[c], acc, 0, 0, 0);
+                f32x4_t q = acc * a.inv_scale;
+                if (!a.scale_pow2) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float refined = __builtin_fmaf(__builtin_fmaf(-q[j], a.scale, acc[j]), a.inv_scale, q[j]);
+                        q[j] = __builtin_fabsf(q[j]) < inf ? refined : q[j];
+                    }
+                }
+                s[half] = q;
+            }
+        };
+        // V of group g, lane = feature: the raw bits of the 32 tokens
+        struct VGroup { uint32_t w[32][DL]; };
+        auto load_v = [&](uint32_t g, VGroup& vg) {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                uint32_t token = 32 * g + i;
+                if (token >= vis_max) token = vis_max - 1;            // its probability is +0 and it is masked below
+                const uint8_t* vrow = vb + (uint64_t)(token >> 4) * a.d_tiles * kTileBytes + (token & 15u) * kRowBytes;
+#pragma unroll
+                for (int c = 0; c < DL; ++c) {
+                    const uint32_t d = lane + 64 * c;
+                    vg.w[i][c] = d < a.D ? (uint32_t)*reinterpret_cast<const uint16_t*>(
+                                                   vrow + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2)
+                                         : 0u;
+                }
+            }
+        };
+        // pass 1: the rows' statistics over this wave's groups, then over the waves
+        RowStats st = {-inf, 0.0f, 0u, false, false};
+        KGroup kcur, knxt;
+        if (wave < groups) load_k(wave, kcur);
+#pragma unroll 1
+        for (uint32_t g = wave; g < groups; g += NW) {
+            if (g + NW < groups) load_k(g + NW, knxt);
+            f32x4_t s[2];
+            scores(kcur, s);
+            kcur = knxt;
+            float local = -inf;
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const bool seen = 32 * g + 16 * half + 4 * kg + j < vis;
+                    const float v = s[half][j];
+                    st.nan = st.nan | (seen & (v != v));
+                    st.pinf += (seen & (v == inf)) ? 1u : 0u;
+                    s[half][j] = (seen & (__builtin_fabsf(v) < inf)) ? v : -inf;
+                    local = __builtin_fmaxf(local, s[half][j]);
+                }
+            const float newm = __builtin_fmaxf(st.m, local);
+            st.sum = newm == st.m ? st.sum : st.sum * __expf(st.m - newm);
+            st.m = newm;
+            st.finite = st.finite | (local > -inf);
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) st.sum += s[half][j] == -inf ? 0.0f : __expf(s[half][j] - newm);
+        }
+#pragma unroll
+        for (int off = 16; off <= 32; off *= 2) {
+            const float m2 = __shfl_xor(st.m, off), s2 = __shfl_xor(st.sum, off);
+            const uint32_t p2 = __shfl_xor(st.pinf, off);
+            const int n2 = __shfl_xor((int)st.nan, off), f2 = __shfl_xor((int)st.finite, off);
+            st.merge(m2, s2, p2, n2 != 0, f2 != 0);
+        }
+        __syncthreads();                           // the previous plane's readers are done
+        if (kg == 0) {
+            wave_stats[wave][l16][0] = st.m;
+            wave_stats[wave][l16][1] = st.sum;
+            wave_stats[wave][l16][2] = as_f32(st.pinf);
+            wave_stats[wave][l16][3] = st.nan ? 1.0f : 0.0f;
+            wave_stats[wave][l16][4] = st.finite ? 1.0f : 0.0f;
+        }
+        __syncthreads();
+        st = RowStats{-inf, 0.0f, 0u, false, false};
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+            st.merge(wave_stats[w][l16][0], wave_stats[w][l16][1], as_u32(wave_stats[w][l16][2]),
+                     wave_stats[w][l16][3] != 0.0f, wave_stats[w][l16][4] != 0.0f);
+        const bool nan_row = st.nan || (st.pinf == 0 && !st.finite);
+        const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
+        const float inv_sum = 1.0f / st.sum;
+        // pass 2: probabilities of a group into LDS, then lane = feature
+        float o[16][DL];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+#pragma unroll
+            for (int c = 0; c < DL; ++c) o[r][c] = 0.0f;
+        constexpr bool VAHEAD = DL == 1;                   // wider heads have no registers for two V groups
+        VGroup vcur, vnxt;
+        if (wave < groups) { load_k(wave, kcur); if (VAHEAD) load_v(wave, vcur); }
+#pragma unroll 1
+        for (uint32_t g = wave; g < groups; g += NW) {
+            // the next group's K and V are requested before this group's arithmetic
+            if (!VAHEAD) load_v(g, vcur);
+            if (g + NW < groups) { load_k(g + NW, knxt); if (VAHEAD) load_v(g + NW, vnxt); }
+            f32x4_t s[2];
+            scores(kcur, s);
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                f32x4_t pr;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float v = s[half][j];
+                    const bool seen = (32 * g + 16 * half + 4 * kg + j < vis) & !nan_row;
+                    const float regular = v == -inf ? 0.0f : __expf(v - st.m) * inv_sum;
+                    const float special = v == inf ? pinf_p : 0.0f;
+                    const float e = seen ? (st.pinf ? special : regular) : 0.0f;
+                    // one rounding to BF16, flushed like every operand of the product (p >= 0)
+                    pr[j] = daz_bf16(bf16_rne_sw(as_u32(e)));
+                }
+                *reinterpret_cast<f32x4_t*>(&p_tile[wave][l16][16 * half + 4 * kg]) = pr;
+            }
+            // the wave reads only what it wrote itself: LDS operations of a wave complete in order
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            // every tile row in use takes its probabilities (16-byte broadcasts) and adds.  Where
+            // every row in use sees all eight tokens of a chunk no select is needed.
+            const uint32_t vis_min = a.a + 1 < a.L ? a.a + 1 : a.L;          // what row 0 sees: the least
+#pragma unroll
+            for (int t0 = 0; t0 < 32; t0 += 8) {
+                float value[8][DL];
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+#pragma unroll
+                    for (int c = 0; c < DL; ++c) value[i][c] = daz_bf16(vcur.w[t0 + i][c]);
+                const bool all_seen = 32 * g + t0 + 8 <= vis_min;             // uniform
+#pragma unroll
+                for (int r4 = 0; r4 < 16; r4 += 4) {
+                    if ((uint32_t)r4 >= nrows) break;                         // uniform; rows past nrows hold +0
+                    // four rows at a time: their eight broadcasts are requested together
+                    f32x4_t pa[4], pb[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        pa[q] = *reinterpret_cast<const f32x4_t*>(&p_tile[wave][r4 + q][t0]);
+                        pb[q] = *reinterpret_cast<const f32x4_t*>(&p_tile[wave][r4 + q][t0 + 4]);
+                    }
+                    if (all_seen) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+#pragma unroll
+                            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                                for (int c = 0; c < DL; ++c)
+                                    o[r4 + q][c] = __builtin_fmaf(i < 4 ? pa[q][i & 3] : pb[q][i & 3], value[i][c], o[r4 + q][c]);
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const uint32_t rr = (uint32_t)(r4 + q) / a.grouping;
+                            const uint32_t reach_r = a.a + rr + 1;
+                            const uint32_t vis_r = reach_r < a.L ? reach_r : a.L; // uniform: what this row may see
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) {
+                                const bool seen = 32 * g + t0 + i < vis_r;
+#pragma unroll
+                                for (int c = 0; c < DL; ++c)
+                                    o[r4 + q][c] = seen ? __builtin_fmaf(i < 4 ? pa[q][i & 3] : pb[q][i & 3], value[i][c], o[r4 + q][c])
+                                                        : o[r4 + q][c];
+                            }
+                        }
+                    }
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // p_tile is rewritten by the next group
+            kcur = knxt;
+            if (VAHEAD) vcur = vnxt;
+        }
+        // the waves' partial outputs meet in LDS
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+#pragma unroll
+            for (int c = 0; c < DL; ++c) o_part[wave][r][lane + 64 * c] = o[r][c];
+        __syncthreads();
+        // thread = (tile row, feature): 16 x D outputs over 512 threads
+        for (uint32_t idx = threadIdx.x; idx < 16 * DL * 64; idx += 512) {
+            const uint32_t r = idx / (DL * 64), d = idx - r * (DL * 64);
+            if (r >= nrows || d >= a.D) continue;
+            float sum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += o_part[w][r][d];
+            if (sum == 0.0f) sum = 0.0f;                                   // -0 is stored as +0
+            const uint32_t rr = r / a.grouping, hh = hkv * a.grouping + (r - rr * a.grouping);
+            const float* ws = &wave_stats[0][r][0];
+            // the row's class again, from the merged per-wave statistics
+            bool nan = false, finite = false;
+            uint32_t pinf = 0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                nan = nan || ws[w * 16 * 5 + 3] != 0.0f;
+                finite = finite || ws[w * 16 * 5 + 4] != 0.0f;
+                pinf += as_u32(ws[w * 16 * 5 + 2]);
+            }
+            const bool nan_out = nan || (pinf == 0 && !finite);
+            const uint32_t col = hh * a.D + d;
+            uint8_t* ob = a.out + plane[3] * a.out_plane_bytes
+                    + (uint64_t)(rr >> 4) * a.out_tile_cols * kTileBytes + (rr & 15u) * kRowBytes;
+            *reinterpret_cast<uint16_t*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) =
+                    (uint16_t)(nan_out ? 0x7FC0u : bf16_rne_sw(as_u32(sum)));
+        }
+    }
+}
+
 // One wave per (row, head, plane), the arithmetic and the order of
 // src/cpu/sdpa.cpp:186-336: every score a sequential sum over the features, the sum
 // of exponentials sequential over the tokens, every output a sequential sum over
@@ -564,6 +836,9 @@ int sdpa_shape(const iomx_view* q, const iomx_view* k, const iomx_view* v, const
 
 constexpr uint64_t kMaxMfmaHeadDim = 128;
 
+// all rows of the query heads of one KV head fit one 16-row tile: the decode kernel
+bool sdpa_few_rows(const SdpaShape& s) { return (s.Hq / s.Hkv) * s.R <= kTile && s.D <= kMaxMfmaHeadDim; }
+
 // Workgroups that share the packing of one KV head: enough of them to occupy the
 // chip when planes * Hkv alone would not.
 uint32_t sdpa_pack_splits(const SdpaShape& s, uint64_t L) {
@@ -607,7 +882,7 @@ extern "C" int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_vie
     IOMX_TRY(sdpa_shape(q, k, v, out, a, L, &s));
     if (dtype != IOMX_DT_BF16) return IOMX_ERR_UNSUPPORTED;
     *alignment = 256;
-    if (s.D > kMaxMfmaHeadDim) { *bytes = 0; *alignment = 1; return IOMX_OK; }
+    if (s.D > kMaxMfmaHeadDim || sdpa_few_rows(s)) { *bytes = 0; *alignment = 1; return IOMX_OK; }
     uint64_t header, region;
     return sdpa_layout(s, L, &header, &region, bytes);
 }
@@ -663,6 +938,19 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
     const hipStream_t st = native(stream);
     const uint32_t gz = g.planes < 65535u ? g.planes : 65535u;
 
+    if (path == 0 && sdpa_few_rows(s) && s.Hkv <= 0x7FFFFFFFull) {
+        const dim3 grid(g.Hkv, gz);
+#define IOMX_SDPA_DECODE(N) case N: hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N>), grid, dim3(512), 0, st, g); break;
+        switch (g.d_tiles) {
+            IOMX_SDPA_DECODE(1) IOMX_SDPA_DECODE(2) IOMX_SDPA_DECODE(3) IOMX_SDPA_DECODE(4)
+            IOMX_SDPA_DECODE(5) IOMX_SDPA_DECODE(6) IOMX_SDPA_DECODE(7)
+            default: IOMX_SDPA_DECODE(8)
+        }
+#undef IOMX_SDPA_DECODE
+        record_launch("sdpa_decode", grid.x * grid.y, 512, (uint64_t)g.planes * g.Hq * g.R);
+        IOMX_HIP(hipGetLastError());
+        return IOMX_OK;
+    }
     bool matrix_cores = path == 0 && s.D <= kMaxMfmaHeadDim;
     uint64_t header = 0, region = 0;
     if (matrix_cores) {
@@ -677,8 +965,7 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         // and when all rows of a KV head's query heads fit one tile they share it
         const uint32_t row_tiles = (g.R + kTile - 1) / kTile;
         int mode = 0;
-        if ((uint64_t)g.grouping * g.R <= kTile && g.grouping > 1) mode = 2;
-        else if ((uint64_t)row_tiles * g.Hq * g.planes < 4096 && g.groups >= 8) mode = 1;
+        if ((uint64_t)row_tiles * g.Hq * g.planes < 4096 && g.groups >= 8) mode = 1;
         g.flags = static_cast<uint32_t*>(workspace);
         g.packed_v = static_cast<uint8_t*>(workspace) + header;
         g.packed_k = mode == 2 ? nullptr : g.packed_v + region;
@@ -691,8 +978,7 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
     else hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, M, false>), grid, dim3(sdpa_waves(N, M) * 64), 0, st, g)
 #define IOMX_SDPA(N) \
     case N: \
-        if (mode == 2) { IOMX_SDPA_MODE(N, 2); } \
-        else if (mode == 1) { IOMX_SDPA_MODE(N, 1); } \
+        if (mode == 1) { IOMX_SDPA_MODE(N, 1); } \
         else { IOMX_SDPA_MODE(N, 0); } \
         break;
         switch (g.d_tiles) {
