@@ -289,12 +289,15 @@ int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const 
  *
  * iomx_sdpa_workspace is the pure requirement query (sdpa_workspace_requirements):
  * the bytes and alignment of caller workspace iomx_launch_sdpa needs for these
- * operands (the packed V fragments and flushed K tiles of the visible prefix and one
- * flag word per plane, KV head and pack share; 0 when D exceeds what the matrix-core
- * kernel covers).  The workspace needs no initialisation and must be 256-byte aligned.  path 0 runs the matrix-core kernel
- * (D <= 128) followed by the reference-order kernel, which returns at once unless V
- * holds an infinity or NaN; path 1 runs the reference-order kernel alone (D <= 256,
- * no workspace).
+ * operands.  Requests whose rows fit one 16-row tile per KV head ((Hq/Hkv)*R <= 16, a
+ * decode step) and heads wider than 128 need none (0 bytes, alignment 1); every other
+ * request needs the packed V fragments and flushed K tiles of the visible prefix and
+ * one flag word per plane, KV head and pack share (256-byte aligned, no
+ * initialisation).  path 0: the decode kernel (one launch: scores on the matrix cores,
+ * P*V on the vector units straight from the cache) for the few-row requests, else the
+ * pack kernel, the matrix-core kernel (D <= 128) and the reference-order kernel, which
+ * returns at once unless V holds an infinity or NaN; path 1 runs the reference-order
+ * kernel alone (D <= 256, no workspace).
  */
 int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
                         const iomx_view* out, uint64_t a, uint64_t L, uint64_t* bytes,
