@@ -699,12 +699,10 @@ private:
                                   const iomx_view k = snapshot_view(captured.k);
                                   const iomx_view v = snapshot_view(captured.v);
                                   const iomx_view out = snapshot_view(captured.out);
-                                  // no workspace was asked for: the head is wider than the
-                                  // matrix-core fragments cover, the reference-order kernel runs
+                                  // the library picks the kernel from the shapes, as its
+                                  // workspace query did (a decode step and wide heads use none)
                                   return iomx_launch_sdpa(IOMX_DT_BF16, &q, &k, &v, &out, captured.a,
-                                                          captured.L, scratch, scratch_bytes,
-                                                          captured.workspace_requirements.bytes ? 0 : 1,
-                                                          stream);
+                                                          captured.L, scratch, scratch_bytes, 0, stream);
                               },
                               [&state, entries, lease](bool failed) {
                                   (void)detail::release_or_invalidate_sdpa_entries(
