@@ -141,14 +141,19 @@ struct RowStats {
 // rows against a long prefix would otherwise be one wave's chain of dependent
 // loads).  MODE 2: the same split, and the 16 rows of the tile are the rows of all
 // query heads that share one KV head (grouping * R <= 16: a decode step reads K and
-// V once per KV head instead of once per query head).  In every mode the K
-// fragments of the next group are requested before the current group is multiplied.
+// V once per KV head instead of once per query head; superseded by sdpa_decode and not
+// launched).
 // FULLD: D is a multiple of 32, no operand load needs a guard against the columns past D.
 // waves of a workgroup: four heads, or as many token shares as LDS holds partial outputs for
 constexpr int sdpa_waves(int dt16, int mode) { return mode == 0 ? 4 : dt16 <= 4 ? 8 : 4; }
 
 template <int DT16, int MODE, bool FULLD>
-__global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
+__global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) __attribute__((amdgpu_waves_per_eu(MODE == 0 ? 3 : 2)))
+void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
+    // MODE 0 hides the K latency with three waves per SIMD (a second set of K registers for a
+    // group ahead would cost the third wave); the token-sharing mode has few waves and
+    // requests the next group ahead instead
+    constexpr bool AHEAD = MODE != 0;
     constexpr bool SPLIT = MODE != 0;
     constexpr int NW = sdpa_waves(DT16, MODE);
     constexpr int D32 = (DT16 + 1) / 2;
@@ -262,10 +267,11 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
         RowStats st = {-inf, 0.0f, 0u, false, false};
         {
             KGroup cur, nxt;
-            if (g_first < groups) load_k(g_first, cur);
+            if (AHEAD && g_first < groups) load_k(g_first, cur);
 #pragma unroll 1
             for (uint32_t g = g_first; g < groups; g += g_step) {
-                if (g + g_step < groups) load_k(g + g_step, nxt);     // the next group is in flight meanwhile
+                if (!AHEAD) load_k(g, cur);
+                else if (g + g_step < groups) load_k(g + g_step, nxt);     // the next group is in flight meanwhile
                 f32x4_t s[2];
                 scores(cur, s);
                 // the finite maximum of the lane's eight scores first, then one rescale; written
@@ -292,7 +298,7 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
                         st.sum += s[half][j] == -inf ? 0.0f : __expf(s[half][j] - newm);
-                cur = nxt;
+                if (AHEAD) cur = nxt;
             }
         }
 #pragma unroll
@@ -327,10 +333,11 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
         for (int dt = 0; dt < DT16; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
         {
             KGroup cur, nxt;
-            if (g_first < groups) load_k(g_first, cur);
+            if (AHEAD && g_first < groups) load_k(g_first, cur);
 #pragma unroll 1
             for (uint32_t g = g_first; g < groups; g += g_step) {
-                if (g + g_step < groups) load_k(g + g_step, nxt);
+                if (!AHEAD) load_k(g, cur);
+                else if (g + g_step < groups) load_k(g + g_step, nxt);
                 u32x4 vfr[DT16];
 #pragma unroll
                 for (int dt = 0; dt < DT16; ++dt)
@@ -355,7 +362,7 @@ __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) void sdpa_mfma_bf16_ke
 #pragma unroll
                 for (int dt = 0; dt < DT16; ++dt)
                     o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vfr[dt]), pf, o[dt], 0, 0, 0);
-                cur = nxt;
+                if (AHEAD) cur = nxt;
             }
         }
         if (SPLIT) {
