@@ -458,13 +458,13 @@ __global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const Line
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-template <int WM, int WVM, int WVN>
+template <int WM, int WVM, int WVN, int DEPTH>
 __global__ __launch_bounds__(WVM * WVN * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     constexpr int WN = 4;                                   // wave tile WM x WN, in 16x16 tiles
     constexpr int NW = WVM * WVN;                           // waves, WVM along the rows
     constexpr uint32_t BM = WM * WVM, BN = WN * WVN;        // workgroup tile, in 16x16 tiles
-    constexpr int KS = 1, DEPTH = 4, HALF = WM / 2;
+    constexpr int KS = 1, HALF = WM / 2;                    // DEPTH stage buffers of 32 inner elements
     constexpr int LPS = (BM + BN) / NW;                     // direct loads per wave and stage
     static_assert(LPS == 4 && BM == 2 * NW && BN == 2 * NW, "two row and two output fragments per wave");
     static_assert(WM >= 4 && WM % 2 == 0 && LPS % HALF == 0, "loads spread over the second half of a stage");
@@ -527,10 +527,11 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     // reader role: position of the lane's eight inner elements inside a fragment
     const uint32_t rd_off = (kg >> 1) * kTileBytes + l16 * kRowBytes + (kg & 1u) * 16;
     const uint32_t stages = a.I / 32;
-    // A ring of four stage buffers (one stage = 32 inner elements).  In the middle of
+    // A ring of DEPTH stage buffers (one stage = 32 inner elements; four for the large
+    // tile, five for the small one whose stages are half as long).  In the middle of
     // stage st every wave waits for its own loads of stage st+1 and meets the others
     // at the barrier: from there on stage st+1 is complete in LDS and nobody reads
-    // stage st-1 any more, so the second half of the stage (a) requests stage st+3
+    // stage st-1 any more, so the second half of the stage (a) requests stage st+DEPTH-1
     // into the buffer of st-1, direct loads between the groups of four MFMAs -- a direct load
     // holds its wave at issue until the memory pipeline takes it, and the matrix
     // instructions issued before it keep the matrix core busy meanwhile -- and (b)
@@ -538,8 +539,8 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     // drain at the stage boundary.
     const uint32_t last = stages - 1;
 #pragma unroll
-    for (uint32_t d = 0; d < 3; ++d) issue(d < stages ? d : last, d);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LPS) : "memory");
+    for (uint32_t d = 0; d < DEPTH - 1; ++d) issue(d < stages ? d : last, d);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * LPS) : "memory");
     __builtin_amdgcn_s_barrier();
     bf16x8_t wf[2][WN], xf[4];
     auto rd = [&](uint32_t ring, uint32_t frag) {
@@ -554,8 +555,10 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     // P = parity of the stage (which half of wf holds its output fragments)
     auto stage = [&](auto parity, uint32_t st) {
         constexpr int P = decltype(parity)::value;
-        const uint32_t ring = st & 3u, ring1 = (st + 1) & 3u, ring3 = (st + 3) & 3u;
-        const uint64_t gnext = (uint64_t)(st + 3 < stages ? st + 3 : last) * kFrag;
+        // ring positions of this stage, of the next one and of the one requested now (which
+        // takes the buffer of the stage before this one)
+        const uint32_t ring = st % DEPTH, ring1 = (st + 1) % DEPTH, ring3 = (st + DEPTH - 1) % DEPTH;
+        const uint64_t gnext = (uint64_t)(st + DEPTH - 1 < stages ? st + DEPTH - 1 : last) * kFrag;
 #pragma unroll
         for (int step = 0; step < HALF; ++step) {
             xf[(step + 2) & 3] = rd(ring, wm * WM + step + 2);          // step + 2 < WM in this half
@@ -568,7 +571,7 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, WN, 0);
         }
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPS) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 3) * LPS) : "memory");
         __builtin_amdgcn_s_barrier();
 #pragma unroll
         for (int step = HALF; step < WM; ++step) {
@@ -738,8 +741,8 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                 const uint64_t wgs = (uint64_t)((a.row_blocks + 63) / 64) * a.super_y * 256;
                 if (wgs > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
                 const dim3 grid((uint32_t)wgs);
-                if (bt == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4>), grid, dim3(512), 0, st, a);
-                else hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2>), grid, dim3(256), 0, st, a);
+                if (bt == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4, 4>), grid, dim3(512), 0, st, a);
+                else hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 5>), grid, dim3(256), 0, st, a);
                 record_launch("linear_mfma_lds", grid.x, bt == 16 ? 512 : 256, (uint64_t)row_tiles * o_tiles);
             } else if (path == 0 && row_tiles < 16 && o_tiles <= 0x7FFFFFFFu) {
                 // few rows (decode, last-row logits): one output tile per workgroup, the
