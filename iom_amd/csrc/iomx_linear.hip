@@ -724,17 +724,17 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
     const hipStream_t st = native(stream);
     const uint32_t gy = a.planes < 65535u ? a.planes : 65535u;
 
-    if (dtype == DT_BF16 && (path == 0 || path == 2)) {
+    if (dtype == DT_BF16 && (path == 0 || path == 2 || path == 3)) {
         const uint64_t total_rows = (uint64_t)a.planes * a.R;
         const uint32_t o_tiles = (a.O + kTile - 1) / kTile;
         if (total_rows <= 0x7FFFFFFFull && o_tiles <= 65535u * 8u) {
             const uint32_t row_tiles = (uint32_t)((total_rows + kTile - 1) / kTile);
-            if (path == 0 && row_tiles >= 8 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
+            if ((path == 0 || path == 3) && row_tiles >= 8 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
                 // enough rows for workgroup tiles: operands staged through LDS.  256 x 256
                 // outputs per workgroup when that still gives every CU two workgroups,
                 // 128 x 128 otherwise
                 const uint64_t big = (uint64_t)((row_tiles + 15) / 16) * ((o_tiles + 15) / 16);
-                const uint32_t bt = big >= 512 ? 16 : 8;
+                const uint32_t bt = (big >= 512 || (path == 3 && row_tiles >= 16)) ? 16 : 8;
                 a.row_blocks = (row_tiles + bt - 1) / bt;
                 a.out_blocks = (o_tiles + bt - 1) / bt;
                 a.super_y = (a.out_blocks + 3) / 4;
@@ -744,7 +744,7 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                 if (bt == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4, 4>), grid, dim3(512), 0, st, a);
                 else hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 5>), grid, dim3(256), 0, st, a);
                 record_launch("linear_mfma_lds", grid.x, bt == 16 ? 512 : 256, (uint64_t)row_tiles * o_tiles);
-            } else if (path == 0 && row_tiles < 16 && o_tiles <= 0x7FFFFFFFu) {
+            } else if (path != 2 && row_tiles < 16 && o_tiles <= 0x7FFFFFFFu) {
                 // few rows (decode, last-row logits): one output tile per workgroup, the
                 // inner axis split over its waves
                 // rows that are alone in their plane (R == 1 of many planes) make x the

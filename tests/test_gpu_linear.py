@@ -239,3 +239,29 @@ def test_bf16_matrix_cores_staged_through_lds(hp, window):
     assert np.array_equal(d2.raw(), do.raw())
     for t in (dx, dw, do, d2):
         t.free()
+
+
+@pytest.mark.parametrize("path", [0, 3], ids=["tile128", "tile256"])
+@pytest.mark.parametrize("inner", [32, 64, 96, 160, 288])
+def test_bf16_workgroup_tiled_kernels_on_short_and_odd_inner_extents(inner, path):
+    """One to nine 32-element stages (fewer than the ring holds, odd counts), both workgroup
+    tile sizes; 300 rows over 2 planes with a window, 80 outputs in 5 heads."""
+    xd, wd, s, R, H, D = (2, 160, inner), (80, inner), 7, 150, 5, 16
+    xv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(xd)), 0, 1, 51 + inner)).reshape(xd)
+    wv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(wd)), 0, 0.2, 52 + inner)).reshape(wd)
+    dx, _ = pair(DT_BF16, xd, values=xv)
+    dw, _ = pair(DT_BF16, wd, values=wv)
+    od = (2, H, R, D)
+    do, ho = pair(DT_BF16, od, salt=53)
+    assert iomx.linear(dx.view(), dw.view(), do.view(), s, R, True, H, D, path=path) == 0
+    assert iomx.last_launch().kernel.decode() == "linear_mfma_lds"
+    got = do.view().to_host().transpose(0, 2, 1, 3).reshape(2, R, H * D)
+    for b in range(2):
+        assert bf16_bound(got[b], xv[b, s:s + R], wv).all()
+    mask = iomo.tile_plane(np.ones(od, np.uint16)) == 0
+    assert np.array_equal(do.raw()[mask], ho.storage[mask])
+    d2, _ = pair(DT_BF16, od, salt=53)
+    assert iomx.linear(dx.view(), dw.view(), d2.view(), s, R, True, H, D, path=2) == 0
+    assert np.array_equal(d2.raw(), do.raw())          # same products in the same order
+    for t in (dx, dw, do, d2):
+        t.free()
