@@ -475,10 +475,11 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     const uint32_t total_rows = a.planes * a.R;
     // blockIdx.x -> (row block, output block): XCD = id % 8, 32 consecutive slots of an
-    // XCD = 8 x 4 blocks, eight XCDs stacked along the rows, super-blocks output-major
+    // XCD = one super-block of 8 x 4 blocks; the super-blocks are dealt to the XCDs in
+    // turn, output-major, so every XCD has work whatever the shape of the block grid
     const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-    const uint32_t sb = slot >> 5, jx = slot & 7u, jy = (slot >> 3) & 3u;
-    const uint32_t bx = (sb / a.super_y) * 64 + xcd * 8 + jx, by = (sb % a.super_y) * 4 + jy;
+    const uint32_t sb = (slot >> 5) * 8 + xcd, jx = slot & 7u, jy = (slot >> 3) & 3u;
+    const uint32_t bx = (sb / a.super_y) * 8 + jx, by = (sb % a.super_y) * 4 + jy;
     if (bx >= a.row_blocks || by >= a.out_blocks) return;
     const uint32_t bm0 = bx * BM, bn0 = by * BN;   // first row tile / output tile
     const uint32_t wm = wave % WVM, wn = wave / WVM;
@@ -731,14 +732,17 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
             const uint32_t row_tiles = (uint32_t)((total_rows + kTile - 1) / kTile);
             if ((path == 0 || path == 3) && row_tiles >= 8 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
                 // enough rows for workgroup tiles: operands staged through LDS.  256 x 256
-                // outputs per workgroup when that still gives every CU two workgroups,
-                // 128 x 128 otherwise
+                // outputs per workgroup (one workgroup per CU) when those fill at least
+                // 65 % of the CU slots of the rounds they take, 128 x 128 (two per CU)
+                // otherwise
                 const uint64_t big = (uint64_t)((row_tiles + 15) / 16) * ((o_tiles + 15) / 16);
-                const uint32_t bt = (big >= 512 || (path == 3 && row_tiles >= 16)) ? 16 : 8;
+                const uint64_t rounds = (big + 255) / 256;
+                const uint32_t bt = (big * 100 >= rounds * 256 * 65 || (path == 3 && row_tiles >= 16)) ? 16 : 8;
                 a.row_blocks = (row_tiles + bt - 1) / bt;
                 a.out_blocks = (o_tiles + bt - 1) / bt;
                 a.super_y = (a.out_blocks + 3) / 4;
-                const uint64_t wgs = (uint64_t)((a.row_blocks + 63) / 64) * a.super_y * 256;
+                const uint64_t supers = (uint64_t)((a.row_blocks + 7) / 8) * a.super_y;
+                const uint64_t wgs = (supers + 7) / 8 * 256;
                 if (wgs > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
                 const dim3 grid((uint32_t)wgs);
                 if (bt == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4, 4>), grid, dim3(512), 0, st, a);
