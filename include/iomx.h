@@ -269,8 +269,9 @@ int iomx_launch_rope(int dtype, const iomx_view* x, const iomx_view* out, uint64
  * waves of a workgroup; path 1 forces the scalar recurrence for every leaf; path 2
  * forces the BF16 matrix-core kernel that loads operands straight from global
  * memory (any shape; the fallback of path 0 and the cross-check of the other two);
- * path 3 is path 0 with the 256 x 256 workgroup tile wherever there are 256 rows
- * (path 0 would pick the 128 x 128 tile for small problems): for tests.
+ * paths 3, 4 and 5 are path 0 with the workgroup tile forced to 256 x 256 (wherever
+ * there are 256 rows), 128 x 128 and 64 x 64 (path 0 picks by how many CUs the
+ * problem fills): for tests.
  */
 int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const iomx_view* out,
                        uint64_t s, uint64_t R, int head_planar, uint64_t H, uint64_t D, int path,

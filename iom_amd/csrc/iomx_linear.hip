@@ -641,6 +641,107 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     }
 }
 
+// 64 rows x 64 outputs per workgroup of four waves (a wave: 2 x 2 MFMA tiles): for
+// problems whose larger tiles would leave CUs idle.  A stage of 32 inner elements is
+// 8 KiB; with a ring of DEPTH stages four or five workgroups share a CU, and their
+// waves cover each other's waits, so a stage is simply: wait for the own loads of the
+// stage, barrier (the stage is complete and nobody reads the one before it any more),
+// request the stage DEPTH-1 ahead into the freed buffer, read four fragments, four MFMAs.
+// The fragments of a wave are 4 KiB per 4 MFMAs: the LDS ports, not the matrix cores,
+// bound this kernel (at about half the matrix rate).
+template <int DEPTH>
+__global__ __launch_bounds__(256)
+void linear_mfma_lds64_bf16_kernel(const LinearArgs a) {
+    constexpr uint32_t BM = 4, BN = 4, NW = 4, LPS = 2;
+    constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
+    constexpr uint32_t kStageBytes = (BM + BN) * kFrag;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[DEPTH * kStageBytes];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t l16 = lane & 15u, kg = lane >> 4;
+    const uint32_t total_rows = a.planes * a.R;
+    const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
+    const uint32_t sb = (slot >> 5) * 8 + xcd, jx = slot & 7u, jy = (slot >> 3) & 3u;
+    const uint32_t bx = (sb / a.super_y) * 8 + jx, by = (sb % a.super_y) * 4 + jy;
+    if (bx >= a.row_blocks || by >= a.out_blocks) return;
+    const uint32_t bm0 = bx * BM, bn0 = by * BN;
+    const uint32_t wm = wave & 1u, wn = wave >> 1;
+
+    // loader role: row fragment `wave` and output fragment `wave` of every stage
+    const uint32_t ld_tile = lane >> 5, ld_row = (lane & 31u) >> 1;
+    const uint32_t ld_off = ld_tile * kTileBytes + (lane & 1u) * 16;
+    const uint8_t* src_x;
+    const uint8_t* src_w;
+    {
+        uint32_t idx = (bm0 + wave) * kTile + ld_row;
+        if (idx >= total_rows) idx = 0;            // valid memory; its results are not stored
+        const uint32_t p = idx / a.R, r = idx - p * a.R;
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        const uint32_t srow = a.s + r;
+        src_x = a.x + plane[0] * a.x_plane_bytes + (uint64_t)(srow >> 4) * a.x_tile_cols * kTileBytes
+                + (srow & 15u) * kRowBytes + ld_off;
+        uint32_t o = (bn0 + wave) * kTile + ld_row;
+        if (o >= a.O) o = 0;
+        src_w = a.w + (uint64_t)(o >> 4) * a.w_tile_cols * kTileBytes + (o & 15u) * kRowBytes + ld_off;
+    }
+    const uint32_t stages = a.I / 32, last = stages - 1;
+    auto issue = [&](uint32_t stage, uint32_t buf) {
+        const uint64_t goff = (uint64_t)(stage < stages ? stage : last) * kFrag;
+        uint8_t* base = lds + buf * kStageBytes;
+        __builtin_amdgcn_global_load_lds((gptr_t)(src_x + goff), (lptr_t)(base + wave * kFrag), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(src_w + goff), (lptr_t)(base + (BM + wave) * kFrag), 16, 0, 0);
+    };
+    f32x4_t acc[2][2];
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int n = 0; n < 2; ++n) acc[m][n] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t rd_off = (kg >> 1) * kTileBytes + l16 * kRowBytes + (kg & 1u) * 16;
+    auto rd = [&](uint32_t ring, uint32_t frag) {
+        return __builtin_bit_cast(bf16x8_t,
+                *reinterpret_cast<const u32x4*>(lds + ring * kStageBytes + rd_off + frag * kFrag));
+    };
+#pragma unroll
+    for (uint32_t d = 0; d < DEPTH - 1; ++d) issue(d, d);
+    uint32_t ring = 0, free_ring = DEPTH - 1;
+    for (uint32_t st = 0; st < stages; ++st) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * LPS) : "memory");
+        __builtin_amdgcn_s_barrier();
+        issue(st + DEPTH - 1, free_ring);
+        const bf16x8_t x0 = rd(ring, wm * 2), x1 = rd(ring, wm * 2 + 1);
+        const bf16x8_t w0 = rd(ring, BM + wn * 2), w1 = rd(ring, BM + wn * 2 + 1);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0, acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x0, acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x1, acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1, acc[1][1], 0, 0, 0);
+        free_ring = ring;
+        ring = ring + 1 == DEPTH ? 0 : ring + 1;
+    }
+    // nothing may still be landing in LDS when the workgroup gives it back
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    const uint32_t d_tiles = a.D >> 4;
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+        const uint32_t idx = (bm0 + wm * 2 + m) * kTile + l16;
+        if (idx >= total_rows) continue;
+        const uint32_t p = idx / a.R, r = idx - p * a.R;
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        uint8_t* orow = a.out + plane[1] * a.out_plane_bytes
+                + (uint64_t)(r >> 4) * a.out_tile_cols * kTileBytes + (r & 15u) * kRowBytes;
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            const uint32_t ot = bn0 + wn * 2 + n;
+            if (ot * kTile >= a.O) continue;
+            const uint32_t h = ot / d_tiles, dt = ot - h * d_tiles;
+            *reinterpret_cast<u32x2*>(orow + (uint64_t)h * a.head_stride * a.out_plane_bytes
+                                      + (uint64_t)dt * kTileBytes + kg * 8) =
+                    u32x2{pack_bf16(acc[m][n][0], acc[m][n][1]), pack_bf16(acc[m][n][2], acc[m][n][3])};
+        }
+    }
+}
+
 namespace {
 
 int kernel_leaf(int dtype) {
@@ -725,19 +826,24 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
     const hipStream_t st = native(stream);
     const uint32_t gy = a.planes < 65535u ? a.planes : 65535u;
 
-    if (dtype == DT_BF16 && (path == 0 || path == 2 || path == 3)) {
+    if (dtype == DT_BF16 && path != 1) {
         const uint64_t total_rows = (uint64_t)a.planes * a.R;
         const uint32_t o_tiles = (a.O + kTile - 1) / kTile;
         if (total_rows <= 0x7FFFFFFFull && o_tiles <= 65535u * 8u) {
             const uint32_t row_tiles = (uint32_t)((total_rows + kTile - 1) / kTile);
-            if ((path == 0 || path == 3) && row_tiles >= 8 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
+            if (path != 2 && row_tiles >= 8 && (a.I % 32) == 0 && (a.D & 15u) == 0) {
                 // enough rows for workgroup tiles: operands staged through LDS.  256 x 256
                 // outputs per workgroup (one workgroup per CU) when those fill at least
                 // 65 % of the CU slots of the rounds they take, 128 x 128 (two per CU)
-                // otherwise
+                // otherwise; 64 x 64 (four or five per CU) when there is not even one
+                // 128 x 128 block per CU
                 const uint64_t big = (uint64_t)((row_tiles + 15) / 16) * ((o_tiles + 15) / 16);
+                const uint64_t mid = (uint64_t)((row_tiles + 7) / 8) * ((o_tiles + 7) / 8);
                 const uint64_t rounds = (big + 255) / 256;
-                const uint32_t bt = (big * 100 >= rounds * 256 * 65 || (path == 3 && row_tiles >= 16)) ? 16 : 8;
+                uint32_t bt = big * 100 >= rounds * 256 * 65 ? 16 : mid >= 256 ? 8 : 4;
+                if (path == 3 && row_tiles >= 16) bt = 16;
+                if (path == 4) bt = 8;
+                if (path == 5) bt = 4;
                 a.row_blocks = (row_tiles + bt - 1) / bt;
                 a.out_blocks = (o_tiles + bt - 1) / bt;
                 a.super_y = (a.out_blocks + 3) / 4;
@@ -746,7 +852,8 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                 if (wgs > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
                 const dim3 grid((uint32_t)wgs);
                 if (bt == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4, 4>), grid, dim3(512), 0, st, a);
-                else hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 5>), grid, dim3(256), 0, st, a);
+                else if (bt == 8) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 5>), grid, dim3(256), 0, st, a);
+                else hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4>), grid, dim3(256), 0, st, a);
                 record_launch("linear_mfma_lds", grid.x, bt == 16 ? 512 : 256, (uint64_t)row_tiles * o_tiles);
             } else if (path != 2 && row_tiles < 16 && o_tiles <= 0x7FFFFFFFu) {
                 // few rows (decode, last-row logits): one output tile per workgroup, the

@@ -241,7 +241,7 @@ def test_bf16_matrix_cores_staged_through_lds(hp, window):
         t.free()
 
 
-@pytest.mark.parametrize("path", [0, 3], ids=["tile128", "tile256"])
+@pytest.mark.parametrize("path", [5, 4, 3], ids=["tile64", "tile128", "tile256"])
 @pytest.mark.parametrize("inner", [32, 64, 96, 160, 288])
 def test_bf16_workgroup_tiled_kernels_on_short_and_odd_inner_extents(inner, path):
     """One to nine 32-element stages (fewer than the ring holds, odd counts), both workgroup
