@@ -132,19 +132,22 @@ __device__ __forceinline__ uint64_t rope_encode(T v) {
     else return encode_from<DT, T>(v);
 }
 
-__device__ __forceinline__ void rope_angle(uint32_t column, uint32_t width, uint32_t position,
-                                           float theta, float* sine, float* cosine) {
-    const float exponent = (float)((-2.0 * (double)column) / (double)width);
-    const float frequency = powf(theta, exponent);
-    const float angle = (float)position * frequency;
-    sincosf(angle, sine, cosine);
+__device__ __forceinline__ float rope_frequency(uint32_t column, uint32_t width, float theta) {
+    return powf(theta, (float)((-2.0 * (double)column) / (double)width));
 }
+__device__ __forceinline__ double rope_frequency(uint32_t column, uint32_t width, double theta) {
+    return pow(theta, (-2.0 * (double)column) / (double)width);
+}
+__device__ __forceinline__ void rope_sincos(uint32_t position, float frequency, float* sine, float* cosine) {
+    sincosf((float)position * frequency, sine, cosine);
+}
+__device__ __forceinline__ void rope_sincos(uint32_t position, double frequency, double* sine, double* cosine) {
+    sincos((double)position * frequency, sine, cosine);
+}
+template <typename T>
 __device__ __forceinline__ void rope_angle(uint32_t column, uint32_t width, uint32_t position,
-                                           double theta, double* sine, double* cosine) {
-    const double exponent = (-2.0 * (double)column) / (double)width;
-    const double frequency = pow(theta, exponent);
-    const double angle = (double)position * frequency;
-    sincos(angle, sine, cosine);
+                                           T theta, T* sine, T* cosine) {
+    rope_sincos(position, rope_frequency(column, width, theta), sine, cosine);
 }
 
 // D/2 a multiple of 16: a lane owns tile rows tc and tc + D/32 of one row.
@@ -154,18 +157,22 @@ __global__ __launch_bounds__(256) void rope_pairs_kernel(const RopeArgs a) {
     constexpr int K = BITS / 2;
     constexpr uint32_t kRowBytes = 2 * BITS, kTileBytes = 32 * BITS;
     const uint32_t g = blockIdx.x * 256u + threadIdx.x;
-    if (g >= a.lanes_per_plane) return;
     const uint32_t r = g & 15u, q = g >> 4;
     const uint32_t tr = a.col_tiles > 1 ? fast_div(q, a.div_col_tiles) : q;
     const uint32_t ptc = q - tr * a.col_tiles;
     const uint32_t row = tr * kTile + r;
-    if (row >= a.rows) return;
+    // the 16 lanes of a pair tile need the same 16 frequencies: one power each, exchanged
+    // (every lane of the wave takes part, also those without a row)
+    const T own_frequency = rope_frequency(ptc * kTile + r, a.width, (T)a.theta);
+    T frequency[kTile];
+#pragma unroll
+    for (int i = 0; i < (int)kTile; ++i) frequency[i] = __shfl(own_frequency, i, 16);
+    if (g >= a.lanes_per_plane || row >= a.rows) return;
     const uint32_t position = a.a + row;
     T sine[kTile], cosine[kTile];
     if (position != 0) {
 #pragma unroll
-        for (int i = 0; i < (int)kTile; ++i)
-            rope_angle(ptc * kTile + i, a.width, position, (T)a.theta, &sine[i], &cosine[i]);
+        for (int i = 0; i < (int)kTile; ++i) rope_sincos(position, frequency[i], &sine[i], &cosine[i]);
     }
     const uint64_t off0 = ((uint64_t)tr * a.tile_cols + ptc) * kTileBytes + r * kRowBytes;
     const uint64_t off1 = off0 + (uint64_t)(a.half >> 4) * kTileBytes;

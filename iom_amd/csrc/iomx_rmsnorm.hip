@@ -378,7 +378,8 @@ int launch(const RmsArgs& a, bool band_ok, hipStream_t s) {
     else if (n <= 2048) launch_band<DT, 2, 1024>(a, s);
     else if (n <= 4096) launch_band<DT, 4, 1024>(a, s);
     else if (n <= 8192) launch_band<DT, 8, 1024>(a, s);
-    else launch_band<DT, 16, 1024>(a, s);  // F32 only: BF16 bands this wide are split above
+    else if constexpr (RLeaf<DT>::kBytes != 2) launch_band<DT, 16, 1024>(a, s);
+    else return IOMX_ERR_INVALID;          // unreachable: BF16 bands this wide are split above
     return IOMX_OK;
 }
 

@@ -17,6 +17,8 @@
 //                   masked probability is +0, and +0 times an infinite V of a token
 //                   the row must not see would poison the row on the matrix cores.
 //                   It is also the path for head sizes the fragments do not cover.
+#include <type_traits>
+
 #include "iomx_mfma.hpp"
 
 namespace iomx {
@@ -32,6 +34,7 @@ struct SdpaArgs {
     uint32_t Hq, Hkv, grouping, R, C, D, a, L;
     uint32_t d_tiles, out_tile_cols, kv_tile_rows;
     uint32_t planes, groups;    // leading planes; 32-token groups of the prefix
+    uint32_t plane0;            // sdpa_mfma: first plane of this launch
     uint8_t* packed_v;          // [plane][kv head][group][d tile] fragments of 1 KiB
     uint8_t* packed_k;          // [plane][kv head][token tile][d tile] flushed tiles (null: not packed)
     uint32_t* flags;            // [plane][kv head][pack split]: nonzero = that part of the V prefix
@@ -138,14 +141,24 @@ struct RowStats {
 // MODE 0: a workgroup of four waves = four heads of one row tile, each wave walks
 // all visible tokens (prefill: many row tiles, K and V shared through the caches).
 // MODE 1: one head, the 4 or 8 waves share out the 32-token groups and meet in LDS (few
-// rows against a long prefix would otherwise be one wave's chain of dependent
-// loads).  MODE 2: the same split, and the 16 rows of the tile are the rows of all
-// query heads that share one KV head (grouping * R <= 16: a decode step reads K and
-// V once per KV head instead of once per query head; superseded by sdpa_decode and not
-// launched).
+// rows against a long prefix would otherwise be one wave's chain of dependent loads).
 // FULLD: D is a multiple of 32, no operand load needs a guard against the columns past D.
+//
+// Both passes exist twice.  The plain one assumes what almost every row satisfies -- no
+// NaN and no +infinity among its visible scores and at least one finite score -- and
+// spends two or three vector instructions per score; its sum of exponentials turns NaN
+// or its maximum infinite exactly when the assumption fails, and then the whole tile
+// repeats both passes with the bookkeeping of the special rows
+// (docs/BACKEND_CONTRACT/scaled-dot-product-attention.md: "Formed-score special values").
 // waves of a workgroup: four heads, or as many token shares as LDS holds partial outputs for
 constexpr int sdpa_waves(int dt16, int mode) { return mode == 0 ? 4 : dt16 <= 4 ? 8 : 4; }
+
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+// two finite floats to two BF16, round to nearest even (the conversion instruction of gfx950)
+__device__ __forceinline__ uint32_t cvt_bf16x2(float lo, float hi) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
 
 template <int DT16, int MODE, bool FULLD>
 __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) __attribute__((amdgpu_waves_per_eu(MODE == 0 ? 3 : 2)))
@@ -157,39 +170,41 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     constexpr bool SPLIT = MODE != 0;
     constexpr int NW = sdpa_waves(DT16, MODE);
     constexpr int D32 = (DT16 + 1) / 2;
+    constexpr float kLog2e = 1.44269504088896340736f;
+    // stands in for a maximum of -infinity (nothing seen yet) in exponent arguments
+    constexpr float kFloor = -1.0e30f;
     __shared__ float wave_stats[NW][16][5];
     __shared__ f32x4_t wave_out[SPLIT ? NW - 1 : 1][SPLIT ? DT16 : 1][64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     // which (head, row) the lane's tile row is
-    uint32_t hkv, head, row, last_row;
-    if (MODE == 2) {
-        hkv = blockIdx.y;
-        row = l16 / a.grouping;
-        head = hkv * a.grouping + (l16 - row * a.grouping);
-        last_row = a.R - 1;
-    } else {
-        head = MODE == 1 ? blockIdx.y : blockIdx.y * 4 + wave;
-        if (MODE == 0 && head >= a.Hq) return;          // no barrier on this path
-        hkv = head / a.grouping;
-        row = blockIdx.x * kTile + l16;
-        last_row = blockIdx.x * kTile + 15 < a.R ? blockIdx.x * kTile + 15 : a.R - 1;
-    }
+    const uint32_t head = MODE == 1 ? blockIdx.y : blockIdx.y * 4 + wave;
+    if (MODE == 0 && head >= a.Hq) return;          // no barrier on this path
+    const uint32_t hkv = head / a.grouping;
+    // the row tiles with the longest prefixes are dispatched first
+    const uint32_t first_row = (gridDim.x - 1 - blockIdx.x) * kTile, row = first_row + l16;
+    const uint32_t last_row = first_row + 15 < a.R ? first_row + 15 : a.R - 1;
     const bool row_ok = row < a.R;
     const uint32_t qrow = row_ok ? row : a.R - 1;
-    const uint32_t reach = a.a + row + 1, reach_max = a.a + last_row + 1;
+    const uint32_t reach = a.a + row + 1, reach_min = a.a + first_row + 1, reach_max = a.a + last_row + 1;
     const uint32_t vis = row_ok ? (reach < a.L ? reach : a.L) : 0;     // tokens this lane's row sees
     const uint32_t vis_max = reach_max < a.L ? reach_max : a.L;        // ... and the tile's last row
     const uint32_t groups = (vis_max + 31) / 32;
+    // groups that every row of the tile sees whole need no mask
+    const uint32_t full_groups = (reach_min < a.L ? reach_min : a.L) / 32;
+    // the plain passes let the rows past R mirror the last row (their results are dropped)
+    const uint32_t vis_plain = row_ok ? vis : vis_max;
     const uint32_t g_first = SPLIT ? wave : 0, g_step = SPLIT ? NW : 1;
     const uint32_t c0 = (kg & 1u) * 8u;
     const float inf = __builtin_inff();
-    for (uint32_t p = blockIdx.z; p < a.planes; p += gridDim.z) {
+    // one plane per grid layer (a loop over planes here would make the compiler keep every
+    // lane offset of the body alive across it, far beyond the register file)
+    {
+        const uint32_t p = a.plane0 + blockIdx.z;
         uint64_t plane[4];
         walk_planes(a.walk, p, plane);
         const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
-        const uint8_t* kb = a.k + (plane[1] + (uint64_t)hkv * a.k_head_stride) * a.kv_plane_bytes;
         // wave-uniform bases and 32-bit lane offsets: the packed region of one KV head is far
         // below 4 GiB, and 64-bit addresses per load would cost the registers of a whole wave slot
         const uint8_t* vf = a.packed_v + (((uint64_t)p * a.Hkv + hkv) * a.groups) * a.d_tiles * kFrag;
@@ -204,42 +219,22 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 qf[c] = daz8(load_k8_bits(qb + ((uint64_t)(qrow >> 4) * a.d_tiles + tile) * kTileBytes
                                                   + (qrow & 15u) * kRowBytes, c0, i0, a.D));
         }
-        // K of the 32 tokens of group g: two 16-token tiles, lane (token l16, features
-        // 8*kg..).  Tokens past the prefix read its last token instead (the cache tail
-        // is never touched); their scores are dropped.
+        // K of the 32 tokens of group g, from the flushed copy: two 16-token tiles, lane
+        // (token l16, features 8*kg..); tokens past the prefix and columns past D are zeros there
         struct KGroup { u32x4 w[2][D32]; };
-        constexpr bool KPACK = MODE != 2;      // the flushed copy pays when many waves meet each tile
-        const uint8_t* kp = KPACK ? a.packed_k + (((uint64_t)p * a.Hkv + hkv) * a.groups * 2) * a.d_tiles * kTileBytes
-                                  : nullptr;
+        const uint8_t* kp = a.packed_k + (((uint64_t)p * a.Hkv + hkv) * a.groups * 2) * a.d_tiles * kTileBytes;
         const uint32_t kp_lane = l16 * kRowBytes + c0 * 2;
         auto load_k = [&](uint32_t g, KGroup& kgp) {
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                if (KPACK) {
-#pragma unroll
-                    for (int c = 0; c < D32; ++c) {
-                        const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
-                        kgp.w[half][c] = u32x4{0, 0, 0, 0};
-                        if (FULLD || i0 < a.D)
-                            kgp.w[half][c] = *reinterpret_cast<const u32x4*>(
-                                    kp + (((2 * g + half) * a.d_tiles + tile) * kTileBytes + kp_lane));
-                    }
-                    continue;
-                }
-                uint32_t token = 32 * g + 16 * half + l16;
-                if (token >= a.L) token = a.L - 1;
-                const uint8_t* krow = kb + (uint64_t)(token >> 4) * a.d_tiles * kTileBytes + (token & 15u) * kRowBytes;
+            for (int half = 0; half < 2; ++half)
 #pragma unroll
                 for (int c = 0; c < D32; ++c) {
                     const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
                     kgp.w[half][c] = u32x4{0, 0, 0, 0};
-                    if (FULLD || i0 < a.D) {
-                        const u32x4 w = FULLD ? *reinterpret_cast<const u32x4*>(krow + (uint64_t)tile * kTileBytes + c0 * 2)
-                                              : load_k8_bits(krow + (uint64_t)tile * kTileBytes, c0, i0, a.D);
-                        kgp.w[half][c] = u32x4{daz2(w[0]), daz2(w[1]), daz2(w[2]), daz2(w[3])};
-                    }
+                    if (FULLD || i0 < a.D)
+                        kgp.w[half][c] = *reinterpret_cast<const u32x4*>(
+                                kp + (((2 * g + half) * a.d_tiles + tile) * kTileBytes + kp_lane));
                 }
-            }
         };
         // scores: lane gets tokens 32g + 16*half + 4*kg + j (j < 4) of row l16
         auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2]) {
@@ -263,17 +258,111 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 s[half] = q;
             }
         };
-        // pass 1: the row's statistics
-        RowStats st = {-inf, 0.0f, 0u, false, false};
-        {
+        // the visible groups of this wave, K one group ahead where the mode says so; WITH_V: the
+        // V fragments of the group are requested before its scores are formed
+        auto walk_groups = [&](auto with_v, auto&& body) {
+            constexpr bool WITH_V = decltype(with_v)::value;
             KGroup cur, nxt;
             if (AHEAD && g_first < groups) load_k(g_first, cur);
 #pragma unroll 1
             for (uint32_t g = g_first; g < groups; g += g_step) {
                 if (!AHEAD) load_k(g, cur);
                 else if (g + g_step < groups) load_k(g + g_step, nxt);     // the next group is in flight meanwhile
+                u32x4 vfr[WITH_V ? DT16 : 1];
+                if constexpr (WITH_V) {
+#pragma unroll
+                    for (int dt = 0; dt < DT16; ++dt)
+                        vfr[dt] = *reinterpret_cast<const u32x4*>(vf + ((g * a.d_tiles + dt) * kFrag + vf_lane));
+                }
                 f32x4_t s[2];
                 scores(cur, s);
+                body(g, s, vfr);
+                if (AHEAD) cur = nxt;
+            }
+        };
+        // scores of tokens the lane's row must not see become -infinity (plain passes)
+        auto mask_group = [&](uint32_t g, f32x4_t (&s)[2]) {
+            const int rem = (int)vis_plain - (int)(32 * g + 4 * kg);
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) s[half][j] = 16 * half + j < rem ? s[half][j] : -inf;
+        };
+        // (maximum, sum) of one part of a row joined with another part's
+        auto join = [&](float& m, float& sum, float m2, float sum2) {
+            const float mm = __builtin_fmaxf(m, m2), base = __builtin_fmaxf(mm, kFloor);
+            sum = sum * __builtin_amdgcn_exp2f((__builtin_fmaxf(m, kFloor) - base) * kLog2e)
+                + sum2 * __builtin_amdgcn_exp2f((__builtin_fmaxf(m2, kFloor) - base) * kLog2e);
+            m = mm;
+        };
+        auto mma_v = [&](f32x4_t (&o)[DT16], const u32x4 (&vfr)[DT16], const u32x4& pw) {
+            const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, pw);
+#pragma unroll
+            for (int dt = 0; dt < DT16; ++dt)
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vfr[dt]), pf, o[dt], 0, 0, 0);
+        };
+
+        // ---- plain pass 1: running maximum and sum of exp(score - maximum)
+        float pm = -inf, psum = 0.0f;
+        walk_groups(std::false_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+            if (g >= full_groups) mask_group(g, s);
+            const float local = __builtin_fmaxf(
+                    __builtin_fmaxf(__builtin_fmaxf(s[0][0], s[0][1]), __builtin_fmaxf(s[0][2], s[0][3])),
+                    __builtin_fmaxf(__builtin_fmaxf(s[1][0], s[1][1]), __builtin_fmaxf(s[1][2], s[1][3])));
+            const float newm = __builtin_fmaxf(pm, local);
+            const float base = __builtin_fmaxf(newm, kFloor);
+            psum *= __builtin_amdgcn_exp2f((__builtin_fmaxf(pm, kFloor) - base) * kLog2e);
+            const float nb = -base * kLog2e;
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) psum += __builtin_amdgcn_exp2f(__builtin_fmaf(s[half][j], kLog2e, nb));
+            pm = newm;
+        });
+#pragma unroll
+        for (int off = 16; off <= 32; off *= 2) {
+            const float m2 = __shfl_xor(pm, off), s2 = __shfl_xor(psum, off);
+            join(pm, psum, m2, s2);
+        }
+        if (SPLIT) {
+            if (kg == 0) {
+                wave_stats[wave][l16][0] = pm;
+                wave_stats[wave][l16][1] = psum;
+            }
+            __syncthreads();
+            pm = wave_stats[0][l16][0];
+            psum = wave_stats[0][l16][1];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) join(pm, psum, wave_stats[w][l16][0], wave_stats[w][l16][1]);
+        }
+        // a NaN or +infinity score, or no finite score at all, shows here; every wave of the
+        // workgroup holds the same joined values and decides alike
+        const bool plain = !__any(!(psum > 0.0f && psum < inf && pm < inf));
+
+        f32x4_t o[DT16];
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        bool nan_row = false;
+        if (plain) {
+            // ---- plain pass 2: probabilities, rounded once to BF16 and flushed, times V
+            const float inv_sum = 1.0f / psum, nb = -pm * kLog2e;
+            walk_groups(std::true_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+                if (g >= full_groups) mask_group(g, s);
+                float pr[8];
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[half][j], kLog2e, nb)) * inv_sum;
+                        pr[half * 4 + j] = pv < 1.17549435e-38f ? 0.0f : pv;      // below the BF16 normals
+                    }
+                mma_v(o, vfr, u32x4{cvt_bf16x2(pr[0], pr[1]), cvt_bf16x2(pr[2], pr[3]),
+                                    cvt_bf16x2(pr[4], pr[5]), cvt_bf16x2(pr[6], pr[7])});
+            });
+        } else {
+            // ---- pass 1 with the bookkeeping of the special rows
+            RowStats st = {-inf, 0.0f, 0u, false, false};
+            walk_groups(std::false_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
                 // the finite maximum of the lane's eight scores first, then one rescale; written
                 // with selects only (a branch per element would cost more than the arithmetic)
                 float local = -inf;
@@ -298,52 +387,35 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
                         st.sum += s[half][j] == -inf ? 0.0f : __expf(s[half][j] - newm);
-                if (AHEAD) cur = nxt;
+            });
+#pragma unroll
+            for (int off = 16; off <= 32; off *= 2) {
+                const float m2 = __shfl_xor(st.m, off), s2 = __shfl_xor(st.sum, off);
+                const uint32_t p2 = __shfl_xor(st.pinf, off);
+                const int n2 = __shfl_xor((int)st.nan, off), f2 = __shfl_xor((int)st.finite, off);
+                st.merge(m2, s2, p2, n2 != 0, f2 != 0);
             }
-        }
+            if (SPLIT) {
+                __syncthreads();                       // the readers of the plain statistics are done
+                if (kg == 0) {
+                    wave_stats[wave][l16][0] = st.m;
+                    wave_stats[wave][l16][1] = st.sum;
+                    wave_stats[wave][l16][2] = as_f32(st.pinf);
+                    wave_stats[wave][l16][3] = st.nan ? 1.0f : 0.0f;
+                    wave_stats[wave][l16][4] = st.finite ? 1.0f : 0.0f;
+                }
+                __syncthreads();
+                st = RowStats{-inf, 0.0f, 0u, false, false};
 #pragma unroll
-        for (int off = 16; off <= 32; off *= 2) {
-            const float m2 = __shfl_xor(st.m, off), s2 = __shfl_xor(st.sum, off);
-            const uint32_t p2 = __shfl_xor(st.pinf, off);
-            const int n2 = __shfl_xor((int)st.nan, off), f2 = __shfl_xor((int)st.finite, off);
-            st.merge(m2, s2, p2, n2 != 0, f2 != 0);
-        }
-        if (SPLIT) {
-            __syncthreads();                       // the previous plane's readers are done
-            if (kg == 0) {
-                wave_stats[wave][l16][0] = st.m;
-                wave_stats[wave][l16][1] = st.sum;
-                wave_stats[wave][l16][2] = as_f32(st.pinf);
-                wave_stats[wave][l16][3] = st.nan ? 1.0f : 0.0f;
-                wave_stats[wave][l16][4] = st.finite ? 1.0f : 0.0f;
+                for (int w = 0; w < NW; ++w)
+                    st.merge(wave_stats[w][l16][0], wave_stats[w][l16][1], as_u32(wave_stats[w][l16][2]),
+                             wave_stats[w][l16][3] != 0.0f, wave_stats[w][l16][4] != 0.0f);
             }
-            __syncthreads();
-            st = RowStats{-inf, 0.0f, 0u, false, false};
-#pragma unroll
-            for (int w = 0; w < NW; ++w)
-                st.merge(wave_stats[w][l16][0], wave_stats[w][l16][1], as_u32(wave_stats[w][l16][2]),
-                         wave_stats[w][l16][3] != 0.0f, wave_stats[w][l16][4] != 0.0f);
-        }
-        const bool nan_row = st.nan || (st.pinf == 0 && !st.finite);      // NaN score or all -inf
-        const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
-        const float inv_sum = 1.0f / st.sum;
-        // pass 2: probabilities, rounded once to BF16, times V
-        f32x4_t o[DT16];
-#pragma unroll
-        for (int dt = 0; dt < DT16; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        {
-            KGroup cur, nxt;
-            if (AHEAD && g_first < groups) load_k(g_first, cur);
-#pragma unroll 1
-            for (uint32_t g = g_first; g < groups; g += g_step) {
-                if (!AHEAD) load_k(g, cur);
-                else if (g + g_step < groups) load_k(g + g_step, nxt);
-                u32x4 vfr[DT16];
-#pragma unroll
-                for (int dt = 0; dt < DT16; ++dt)
-                    vfr[dt] = *reinterpret_cast<const u32x4*>(vf + ((g * a.d_tiles + dt) * kFrag + vf_lane));
-                f32x4_t s[2];
-                scores(cur, s);
+            nan_row = st.nan || (st.pinf == 0 && !st.finite);      // NaN score or all -inf
+            const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
+            const float inv_sum = 1.0f / st.sum;
+            // ---- pass 2 of the special rows
+            walk_groups(std::true_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
                 float pr[8];
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
@@ -356,14 +428,9 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                         pr[half * 4 + j] = seen ? (st.pinf ? special : regular) : 0.0f;
                     }
                 // one rounding to BF16, then flushed like every matrix operand (p >= 0)
-                const bf16x8_t pf = __builtin_bit_cast(bf16x8_t,
-                        u32x4{daz2(pack_bf16(pr[0], pr[1])), daz2(pack_bf16(pr[2], pr[3])),
-                              daz2(pack_bf16(pr[4], pr[5])), daz2(pack_bf16(pr[6], pr[7]))});
-#pragma unroll
-                for (int dt = 0; dt < DT16; ++dt)
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vfr[dt]), pf, o[dt], 0, 0, 0);
-                if (AHEAD) cur = nxt;
-            }
+                mma_v(o, vfr, u32x4{daz2(pack_bf16(pr[0], pr[1])), daz2(pack_bf16(pr[2], pr[3])),
+                                    daz2(pack_bf16(pr[4], pr[5])), daz2(pack_bf16(pr[6], pr[7]))});
+            });
         }
         if (SPLIT) {
             if (wave != 0) {
@@ -371,7 +438,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 for (int dt = 0; dt < DT16; ++dt) wave_out[wave - 1][dt][lane] = o[dt];
             }
             __syncthreads();
-            if (wave != 0) continue;
+            if (wave != 0) return;
             // one wave's partial at a time (unrolled, the loads of all of them would be
             // hoisted and would not fit the register file)
 #pragma unroll 1
@@ -380,7 +447,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 for (int dt = 0; dt < DT16; ++dt) o[dt] += wave_out[w][dt][lane];
         }
         // lane holds out[row][head*D + 16*dt + 4*kg + j]
-        if (!row_ok) continue;
+        if (!row_ok) return;
         uint8_t* ob = a.out + plane[3] * a.out_plane_bytes
                 + (uint64_t)(row >> 4) * a.out_tile_cols * kTileBytes + (row & 15u) * kRowBytes;
 #pragma unroll
@@ -442,7 +509,9 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
     const uint32_t groups = (vis_max + 31) / 32;
     const uint32_t c0 = (kg & 1u) * 8u;
     const float inf = __builtin_inff();
-    for (uint32_t p = blockIdx.y; p < a.planes; p += gridDim.y) {
+    // one plane per grid row, as in sdpa_mfma
+    {
+        const uint32_t p = a.plane0 + blockIdx.y;
         uint64_t plane[4];
         walk_planes(a.walk, p, plane);
         const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
@@ -547,7 +616,6 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             const int n2 = __shfl_xor((int)st.nan, off), f2 = __shfl_xor((int)st.finite, off);
             st.merge(m2, s2, p2, n2 != 0, f2 != 0);
         }
-        __syncthreads();                           // the previous plane's readers are done
         if (kg == 0) {
             wave_stats[wave][l16][0] = st.m;
             wave_stats[wave][l16][1] = st.sum;
@@ -946,15 +1014,17 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
     const uint32_t gz = g.planes < 65535u ? g.planes : 65535u;
 
     if (path == 0 && sdpa_few_rows(s) && s.Hkv <= 0x7FFFFFFFull) {
-        const dim3 grid(g.Hkv, gz);
+        for (g.plane0 = 0; g.plane0 < g.planes; g.plane0 += 65535u) {
+            const dim3 grid(g.Hkv, g.planes - g.plane0 < 65535u ? g.planes - g.plane0 : 65535u);
 #define IOMX_SDPA_DECODE(N) case N: hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N>), grid, dim3(512), 0, st, g); break;
-        switch (g.d_tiles) {
-            IOMX_SDPA_DECODE(1) IOMX_SDPA_DECODE(2) IOMX_SDPA_DECODE(3) IOMX_SDPA_DECODE(4)
-            IOMX_SDPA_DECODE(5) IOMX_SDPA_DECODE(6) IOMX_SDPA_DECODE(7)
-            default: IOMX_SDPA_DECODE(8)
-        }
+            switch (g.d_tiles) {
+                IOMX_SDPA_DECODE(1) IOMX_SDPA_DECODE(2) IOMX_SDPA_DECODE(3) IOMX_SDPA_DECODE(4)
+                IOMX_SDPA_DECODE(5) IOMX_SDPA_DECODE(6) IOMX_SDPA_DECODE(7)
+                default: IOMX_SDPA_DECODE(8)
+            }
 #undef IOMX_SDPA_DECODE
-        record_launch("sdpa_decode", grid.x * grid.y, 512, (uint64_t)g.planes * g.Hq * g.R);
+        }
+        record_launch("sdpa_decode", g.Hkv * gz, 512, (uint64_t)g.planes * g.Hq * g.R);
         IOMX_HIP(hipGetLastError());
         return IOMX_OK;
     }
@@ -975,11 +1045,13 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         if ((uint64_t)row_tiles * g.Hq * g.planes < 4096 && g.groups >= 8) mode = 1;
         g.flags = static_cast<uint32_t*>(workspace);
         g.packed_v = static_cast<uint8_t*>(workspace) + header;
-        g.packed_k = mode == 2 ? nullptr : g.packed_v + region;
+        g.packed_k = g.packed_v + region;
         g.pack_splits = sdpa_pack_splits(s, L);
         hipLaunchKernelGGL(sdpa_pack_kernel, dim3(g.Hkv * g.pack_splits, gz), dim3(256), 0, st, g);
-        const dim3 grid(mode == 2 ? 1 : row_tiles, mode == 2 ? g.Hkv : mode == 1 ? g.Hq : (g.Hq + 3) / 4, gz);
         const bool full_d = (g.D & 31u) == 0;
+        for (g.plane0 = 0; g.plane0 < g.planes; g.plane0 += 65535u) {
+        const uint32_t layers = g.planes - g.plane0 < 65535u ? g.planes - g.plane0 : 65535u;
+        const dim3 grid(row_tiles, mode == 1 ? g.Hq : (g.Hq + 3) / 4, layers);
 #define IOMX_SDPA_MODE(N, M) \
     if (full_d) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, M, true>), grid, dim3(sdpa_waves(N, M) * 64), 0, st, g); \
     else hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, M, false>), grid, dim3(sdpa_waves(N, M) * 64), 0, st, g)
@@ -995,7 +1067,9 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         }
 #undef IOMX_SDPA_MODE
 #undef IOMX_SDPA
-        record_launch("sdpa_mfma", grid.x * grid.y * grid.z, 256, (uint64_t)g.planes * g.Hq * g.R);
+        }
+        record_launch("sdpa_mfma", row_tiles * (mode == 1 ? g.Hq : (g.Hq + 3) / 4) * gz, 256,
+                      (uint64_t)g.planes * g.Hq * g.R);
         g.guarded = 1;
     }
     // one grid row per (plane, KV head) pair: when it only has to look at the flags it is

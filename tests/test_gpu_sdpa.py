@@ -169,6 +169,21 @@ def test_tail_future_tokens_and_special_v(R):
     assert np.array_equal(g[1], base.reshape(2, R, 4, 16)[1])
 
 
+@pytest.mark.parametrize("R,kernel", [(1, "sdpa_decode"), (17, "sdpa_mfma")], ids=["decode_kernel", "tiled_kernel_and_guard"])
+def test_more_planes_than_one_grid_holds(R, kernel):
+    """65540 planes (a grid axis holds 65535): seven different planes repeated; every plane's
+    result is the bits of the same plane in a seven-plane call."""
+    n, few = 65540, 7
+    small = random_case(77, (few,), 2, 1, R, 16, 20, 3, 3 + R)
+    want = run(small, 0, expect_kernel=kernel)
+    pick = np.arange(n) % few
+    big = dict(small, leading=[n])
+    for name, shape in (("q", (few, 2, R, 16)), ("k", (few, 1, 20, 16)), ("v", (few, 1, 20, 16))):
+        big[name] = np.array(small[name], np.uint16).reshape(shape)[pick].reshape(-1)
+    got = run(big, 0, expect_kernel=kernel)
+    assert np.array_equal(got, want[pick])
+
+
 def test_incremental_rows_equal_the_prefill():
     case = random_case(9, (), 4, 2, 7, 8, 7, 0, 7)
     full = run(case, 0)
