@@ -455,8 +455,6 @@ __global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const Line
 // modulo 8) cover 8 row blocks x 4 output blocks: the XCD's L2 then serves every
 // operand slice to 4 or 8 workgroups for one fetch from HBM.
 
-typedef __attribute__((address_space(1))) const void* gptr_t;
-typedef __attribute__((address_space(3))) void* lptr_t;
 
 template <int WM, int WVM, int WVN, int DEPTH>
 __global__ __launch_bounds__(WVM * WVN * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))

@@ -8,6 +8,10 @@ namespace iomx {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
+// operands of the direct global -> LDS loader (global_load_lds: 16 bytes a lane, lane i's
+// piece lands at the LDS address + 16*i)
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
 
 // Eight consecutive BF16 of one tile row starting at column c0 (0 or 8), inner
 // indices i0..i0+7, zero where the inner index is past I (tile padding is never

@@ -142,6 +142,10 @@ struct RowStats {
 // all visible tokens (prefill: many row tiles, K and V shared through the caches).
 // MODE 1: one head, the 4 or 8 waves share out the 32-token groups and meet in LDS (few
 // rows against a long prefix would otherwise be one wave's chain of dependent loads).
+// MODE 2: MODE 0 for four heads that share one KV head (grouping a multiple of 4) and D = 64
+// or 128: the workgroup brings every K and V group into LDS once, with the direct loader,
+// three groups deep, and its four waves read their operands from there -- the vector
+// memory pipeline of the CU, which bounds MODE 0, carries a quarter of the bytes.
 // FULLD: D is a multiple of 32, no operand load needs a guard against the columns past D.
 //
 // Both passes exist twice.  The plain one assumes what almost every row satisfies -- no
@@ -151,7 +155,7 @@ struct RowStats {
 // repeats both passes with the bookkeeping of the special rows
 // (docs/BACKEND_CONTRACT/scaled-dot-product-attention.md: "Formed-score special values").
 // waves of a workgroup: four heads, or as many token shares as LDS holds partial outputs for
-constexpr int sdpa_waves(int dt16, int mode) { return mode == 0 ? 4 : dt16 <= 4 ? 8 : 4; }
+constexpr int sdpa_waves(int dt16, int mode) { return mode != 1 ? 4 : dt16 <= 4 ? 8 : 4; }
 
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -161,13 +165,16 @@ __device__ __forceinline__ uint32_t cvt_bf16x2(float lo, float hi) {
 }
 
 template <int DT16, int MODE, bool FULLD>
-__global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) __attribute__((amdgpu_waves_per_eu(MODE == 0 ? 3 : 2)))
+__global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) __attribute__((amdgpu_waves_per_eu(MODE != 1 ? 3 : 2)))
 void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
-    // MODE 0 hides the K latency with three waves per SIMD (a second set of K registers for a
-    // group ahead would cost the third wave); the token-sharing mode has few waves and
-    // requests the next group ahead instead
-    constexpr bool AHEAD = MODE != 0;
-    constexpr bool SPLIT = MODE != 0;
+    // MODE 0 hides the K latency with many waves per SIMD; the token-sharing mode has few
+    // waves and requests the next group ahead instead
+    constexpr bool AHEAD = MODE == 1;
+    constexpr bool SPLIT = MODE == 1;
+    constexpr bool SHARE = MODE == 2;
+    static_assert(!SHARE || (DT16 % 4 == 0 && FULLD), "shared groups: whole KiB chunks per wave");
+    constexpr uint32_t kStage = 2 * DT16 * 1024;           // K group + V group
+    __shared__ __attribute__((aligned(16))) uint8_t kv_ring[SHARE ? 3 * kStage : 16];
     constexpr int NW = sdpa_waves(DT16, MODE);
     constexpr int D32 = (DT16 + 1) / 2;
     constexpr float kLog2e = 1.44269504088896340736f;
@@ -179,11 +186,12 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     // which (head, row) the lane's tile row is
-    const uint32_t head = MODE == 1 ? blockIdx.y : blockIdx.y * 4 + wave;
-    if (MODE == 0 && head >= a.Hq) return;          // no barrier on this path
+    const uint32_t head = MODE == 1 ? blockIdx.x : blockIdx.x * 4 + wave;
+    if (MODE == 0 && head >= a.Hq) return;          // no barrier on this path (MODE 2: Hq is a multiple of 4)
     const uint32_t hkv = head / a.grouping;
-    // the row tiles with the longest prefixes are dispatched first
-    const uint32_t first_row = (gridDim.x - 1 - blockIdx.x) * kTile, row = first_row + l16;
+    // grid = (heads, planes, row tiles): the row tiles with the longest prefixes are dispatched
+    // first, for every head and plane, and the short ones fill the end of the launch
+    const uint32_t first_row = (gridDim.z - 1 - blockIdx.z) * kTile, row = first_row + l16;
     const uint32_t last_row = first_row + 15 < a.R ? first_row + 15 : a.R - 1;
     const bool row_ok = row < a.R;
     const uint32_t qrow = row_ok ? row : a.R - 1;
@@ -201,7 +209,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     // one plane per grid layer (a loop over planes here would make the compiler keep every
     // lane offset of the body alive across it, far beyond the register file)
     {
-        const uint32_t p = a.plane0 + blockIdx.z;
+        const uint32_t p = a.plane0 + blockIdx.y;
         uint64_t plane[4];
         walk_planes(a.walk, p, plane);
         const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
@@ -262,6 +270,59 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         // V fragments of the group are requested before its scores are formed
         auto walk_groups = [&](auto with_v, auto&& body) {
             constexpr bool WITH_V = decltype(with_v)::value;
+            if constexpr (SHARE) {
+                // wave w brings in KiB chunks w, w+4, .. of the K group (and of the V group) of
+                // every stage; lane i fetches 16-byte piece i of a chunk, and the loader puts it at
+                // chunk + 16*i, so a group lies in LDS as it lies in the packed regions
+                constexpr int LPS = (WITH_V ? 2 : 1) * (DT16 / 4);        // direct loads per wave and stage
+                auto issue = [&](uint32_t g, uint32_t buf) {
+                    const uint32_t gg = g < groups ? g : groups - 1;      // past the end: a valid group again, unused
+                    uint8_t* stage = kv_ring + buf * kStage;
+#pragma unroll
+                    for (int j = 0; j < DT16 / 4; ++j) {
+                        const uint32_t chunk = wave + 4 * j;
+                        __builtin_amdgcn_global_load_lds((gptr_t)(kp + ((gg * DT16 + chunk) * kFrag + vf_lane)),
+                                                         (lptr_t)(stage + chunk * kFrag), 16, 0, 0);
+                        if constexpr (WITH_V)
+                            __builtin_amdgcn_global_load_lds((gptr_t)(vf + ((gg * DT16 + chunk) * kFrag + vf_lane)),
+                                                             (lptr_t)(stage + (DT16 + chunk) * kFrag), 16, 0, 0);
+                    }
+                };
+                issue(0, 0);
+                issue(1, 1);
+                uint32_t buf = 0;
+#pragma unroll 1
+                for (uint32_t g = 0; g < groups; ++g) {
+                    // the own loads of group g have landed; past the barrier everybody's have, and
+                    // nobody reads the buffer of group g-1 any more: it takes group g+2
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPS) : "memory");
+                    __builtin_amdgcn_s_barrier();
+                    issue(g + 2, buf == 0 ? 2 : buf - 1);
+                    const uint8_t* stage = kv_ring + buf * kStage;
+                    KGroup cur;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half)
+#pragma unroll
+                        for (int c = 0; c < D32; ++c)
+                            cur.w[half][c] = *reinterpret_cast<const u32x4*>(
+                                    stage + ((half * DT16 + 2 * c + (kg >> 1)) * kTileBytes + kp_lane));
+                    u32x4 vfr[WITH_V ? DT16 : 1];
+                    if constexpr (WITH_V) {
+#pragma unroll
+                        for (int dt = 0; dt < DT16; ++dt)
+                            vfr[dt] = *reinterpret_cast<const u32x4*>(stage + ((DT16 + dt) * kFrag + vf_lane));
+                    }
+                    f32x4_t s[2];
+                    scores(cur, s);
+                    body(g, s, vfr);
+                    buf = buf == 2 ? 0 : buf + 1;
+                }
+                // nothing in flight and nobody reading when the next pass (or the next workgroup)
+                // takes the ring
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                return;
+            }
             KGroup cur, nxt;
             if (AHEAD && g_first < groups) load_k(g_first, cur);
 #pragma unroll 1
@@ -337,7 +398,9 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         }
         // a NaN or +infinity score, or no finite score at all, shows here; every wave of the
         // workgroup holds the same joined values and decides alike
-        const bool plain = !__any(!(psum > 0.0f && psum < inf && pm < inf));
+        const bool odd = !(psum > 0.0f && psum < inf && pm < inf);
+        // (sharing the groups, the four waves also share the decision: they meet at barriers)
+        const bool plain = SHARE ? !__syncthreads_or(odd ? 1 : 0) : !__any(odd);
 
         f32x4_t o[DT16];
 #pragma unroll
@@ -1035,7 +1098,7 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         IOMX_TRY(sdpa_layout(s, L, &header, &region, &need));
         if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
             return IOMX_ERR_INVALID;
-        if (s.Hkv > 65535u) matrix_cores = false;
+        if (s.Hkv > 65535u || (s.R + kTile - 1) / kTile > 65535u) matrix_cores = false;
     }
     if (matrix_cores) {
         // few row tiles against a long prefix: the waves of a workgroup split the tokens,
@@ -1043,6 +1106,7 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         const uint32_t row_tiles = (g.R + kTile - 1) / kTile;
         int mode = 0;
         if ((uint64_t)row_tiles * g.Hq * g.planes < 4096 && g.groups >= 8) mode = 1;
+        else if ((g.D == 64 || g.D == 128) && g.grouping % 4 == 0) mode = 2;
         g.flags = static_cast<uint32_t*>(workspace);
         g.packed_v = static_cast<uint8_t*>(workspace) + header;
         g.packed_k = g.packed_v + region;
@@ -1051,7 +1115,7 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         const bool full_d = (g.D & 31u) == 0;
         for (g.plane0 = 0; g.plane0 < g.planes; g.plane0 += 65535u) {
         const uint32_t layers = g.planes - g.plane0 < 65535u ? g.planes - g.plane0 : 65535u;
-        const dim3 grid(row_tiles, mode == 1 ? g.Hq : (g.Hq + 3) / 4, layers);
+        const dim3 grid(mode == 1 ? g.Hq : (g.Hq + 3) / 4, layers, row_tiles);
 #define IOMX_SDPA_MODE(N, M) \
     if (full_d) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, M, true>), grid, dim3(sdpa_waves(N, M) * 64), 0, st, g); \
     else hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, M, false>), grid, dim3(sdpa_waves(N, M) * 64), 0, st, g)
@@ -1060,7 +1124,11 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         if (mode == 1) { IOMX_SDPA_MODE(N, 1); } \
         else { IOMX_SDPA_MODE(N, 0); } \
         break;
-        switch (g.d_tiles) {
+        if (mode == 2 && g.d_tiles == 4)
+            hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<4, 2, true>), grid, dim3(256), 0, st, g);
+        else if (mode == 2)
+            hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<8, 2, true>), grid, dim3(256), 0, st, g);
+        else switch (g.d_tiles) {
             IOMX_SDPA(1) IOMX_SDPA(2) IOMX_SDPA(3) IOMX_SDPA(4)
             IOMX_SDPA(5) IOMX_SDPA(6) IOMX_SDPA(7)
             default: IOMX_SDPA(8)
