@@ -39,7 +39,8 @@ struct LinearArgs {
     uint32_t row_tiles;       // ceil(R / 16)
     uint32_t lanes_per_plane; // row_tiles * 16 * H * out_tile_cols
     uint32_t planes;
-    uint32_t row_blocks, out_blocks, super_y;   // workgroup-tiled kernel: 256-row / 256-output blocks
+    uint32_t row_blocks, out_blocks, blocks_per_xcd;   // workgroup-tiled kernels: blocks of rows / of outputs
+    uint32_t out_tile0;                         // ... and the first output tile of this launch
 };
 
 // ---------------------------------------------------------------------------
@@ -450,11 +451,24 @@ __global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const Line
 // {4-7, 8-11, 16-19, 28-31} (and the same +32) together; with lane l reading row l%16,
 // inner elements 8*(l/16).., of the plain tiled fragment each such group touches 16
 // different 16-byte bank groups, so the operand reads are conflict-free as stored.
-//
-// Workgroups are numbered so that the 32 that run together on one XCD (ids equal
-// modulo 8) cover 8 row blocks x 4 output blocks: the XCD's L2 then serves every
-// operand slice to 4 or 8 workgroups for one fetch from HBM.
 
+
+// blockIdx.x -> (row block, output block).  The blocks are put in one sequence: panels of
+// eight row blocks, inside a panel output block by output block; XCD id % 8 takes the id/8-th
+// block of its eighth of the sequence.  So every XCD gets the same number of blocks (give or
+// take one), and the 32 or 64 workgroups that run together on it cover about 8 row blocks x
+// 4 or 8 output blocks: its L2 serves every operand slice to several workgroups for one fetch.
+__device__ __forceinline__ bool block_of_workgroup(const LinearArgs& a, uint32_t* bx, uint32_t* by) {
+    const uint32_t xcd = blockIdx.x & 7u, idx = blockIdx.x >> 3;
+    const uint32_t at = xcd * a.blocks_per_xcd + idx;
+    if (at >= a.row_blocks * a.out_blocks) return false;
+    const uint32_t panel_blocks = 8 * a.out_blocks;
+    const uint32_t panel = at / panel_blocks, rem = at - panel * panel_blocks;
+    const uint32_t left = a.row_blocks - panel * 8, height = left < 8 ? left : 8;
+    *by = rem / height;
+    *bx = panel * 8 + (rem - *by * height);
+    return true;
+}
 
 template <int WM, int WVM, int WVN, int DEPTH>
 __global__ __launch_bounds__(WVM * WVN * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -472,14 +486,9 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     const uint32_t total_rows = a.planes * a.R;
-    // blockIdx.x -> (row block, output block): XCD = id % 8, 32 consecutive slots of an
-    // XCD = one super-block of 8 x 4 blocks; the super-blocks are dealt to the XCDs in
-    // turn, output-major, so every XCD has work whatever the shape of the block grid
-    const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-    const uint32_t sb = (slot >> 5) * 8 + xcd, jx = slot & 7u, jy = (slot >> 3) & 3u;
-    const uint32_t bx = (sb / a.super_y) * 8 + jx, by = (sb % a.super_y) * 4 + jy;
-    if (bx >= a.row_blocks || by >= a.out_blocks) return;
-    const uint32_t bm0 = bx * BM, bn0 = by * BN;   // first row tile / output tile
+    uint32_t bx, by;
+    if (!block_of_workgroup(a, &bx, &by)) return;
+    const uint32_t bm0 = bx * BM, bn0 = a.out_tile0 + by * BN;   // first row tile / output tile
     const uint32_t wm = wave % WVM, wn = wave / WVM;
 
     // loader role: this wave brings in row fragments wave, wave+NW and output fragments
@@ -657,11 +666,9 @@ void linear_mfma_lds64_bf16_kernel(const LinearArgs a) {
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     const uint32_t total_rows = a.planes * a.R;
-    const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3;
-    const uint32_t sb = (slot >> 5) * 8 + xcd, jx = slot & 7u, jy = (slot >> 3) & 3u;
-    const uint32_t bx = (sb / a.super_y) * 8 + jx, by = (sb % a.super_y) * 4 + jy;
-    if (bx >= a.row_blocks || by >= a.out_blocks) return;
-    const uint32_t bm0 = bx * BM, bn0 = by * BN;
+    uint32_t bx, by;
+    if (!block_of_workgroup(a, &bx, &by)) return;
+    const uint32_t bm0 = bx * BM, bn0 = a.out_tile0 + by * BN;
     const uint32_t wm = wave & 1u, wn = wave >> 1;
 
     // loader role: row fragment `wave` and output fragment `wave` of every stage
@@ -842,17 +849,38 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                 if (path == 3 && row_tiles >= 16) bt = 16;
                 if (path == 4) bt = 8;
                 if (path == 5) bt = 4;
-                a.row_blocks = (row_tiles + bt - 1) / bt;
-                a.out_blocks = (o_tiles + bt - 1) / bt;
-                a.super_y = (a.out_blocks + 3) / 4;
-                const uint64_t supers = (uint64_t)((a.row_blocks + 7) / 8) * a.super_y;
-                const uint64_t wgs = (supers + 7) / 8 * 256;
-                if (wgs > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
-                const dim3 grid((uint32_t)wgs);
-                if (bt == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4, 4>), grid, dim3(512), 0, st, a);
-                else if (bt == 8) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 5>), grid, dim3(256), 0, st, a);
-                else hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4>), grid, dim3(256), 0, st, a);
-                record_launch("linear_mfma_lds", grid.x, bt == 16 ? 512 : 256, (uint64_t)row_tiles * o_tiles);
+                // output tiles [first, first + count) with workgroup tiles of bt x bt 16x16 tiles
+                auto launch_part = [&](uint32_t first, uint32_t count, uint32_t tile) -> int {
+                    LinearArgs b = a;
+                    b.out_tile0 = first;
+                    b.row_blocks = (row_tiles + tile - 1) / tile;
+                    b.out_blocks = (count + tile - 1) / tile;
+                    const uint64_t blocks = (uint64_t)b.row_blocks * b.out_blocks;
+                    if (blocks > 0x7FFFFFF0ull) return IOMX_ERR_OVERFLOW;
+                    b.blocks_per_xcd = (uint32_t)((blocks + 7) / 8);
+                    const uint64_t wgs = (uint64_t)b.blocks_per_xcd * 8;
+                    const dim3 grid((uint32_t)wgs);
+                    if (tile == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4, 4>), grid, dim3(512), 0, st, b);
+                    else if (tile == 8) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 5>), grid, dim3(256), 0, st, b);
+                    else hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4>), grid, dim3(256), 0, st, b);
+                    record_launch("linear_mfma_lds", grid.x, tile == 16 ? 512 : 256, (uint64_t)row_tiles * count);
+                    return IOMX_OK;
+                };
+                // 256 x 256 blocks that fill whole rounds of the 256 CUs, and the rest of the
+                // output range with smaller tiles in a second launch, when the last round of the
+                // large tiles would run on few CUs (say 352 blocks: 256 + 96 -> 256 large blocks,
+                // then 384 blocks of 128 x 128 at half the duration)
+                const uint32_t rb16 = (row_tiles + 15) / 16, ob16 = (o_tiles + 15) / 16;
+                const uint32_t ob_whole = (uint32_t)((big / 256) * 256 / rb16);
+                if (path == 0 && bt == 16 && big > 256 && big * 100 < rounds * 256 * 85
+                    && ob_whole >= 1 && ob_whole < ob16 && (uint64_t)ob_whole * rb16 * 100 >= (big / 256) * 256 * 90) {
+                    const uint32_t rest = o_tiles - ob_whole * 16;
+                    const uint64_t rest_mid = (uint64_t)((row_tiles + 7) / 8) * ((rest + 7) / 8);
+                    IOMX_TRY(launch_part(0, ob_whole * 16, 16));
+                    IOMX_TRY(launch_part(ob_whole * 16, rest, rest_mid >= 256 ? 8 : 4));
+                } else {
+                    IOMX_TRY(launch_part(0, o_tiles, bt));
+                }
             } else if (path != 2 && row_tiles < 16 && o_tiles <= 0x7FFFFFFFu) {
                 // few rows (decode, last-row logits): one output tile per workgroup, the
                 // inner axis split over its waves
