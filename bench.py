@@ -652,9 +652,9 @@ def main():
         "softmax_causal": lambda: wl_softmax(timer, max(K // 20, 3), 2, 32, 32, 2048, 2048, True),
         "chain": lambda: wl_chain(timer, max(K // 10, 5), max(W // 10, 2)),
         "layer_ops": lambda: wl_layer_ops(timer, max(K // 4, 5), max(W // 4, 2)),
-        "linear": lambda: wl_linear(timer, max(K // 20, 5), 2),
-        "sdpa": lambda: wl_sdpa(timer, max(K // 20, 5), 2),
-        "decoder_layer": lambda: wl_decoder_layer(timer, max(K // 20, 5), 2),
+        "linear": lambda: wl_linear(timer, max(K // 5, 10), max(W // 2, 5)),
+        "sdpa": lambda: wl_sdpa(timer, max(K // 5, 10), max(W // 2, 5)),
+        "decoder_layer": lambda: wl_decoder_layer(timer, max(K // 5, 10), max(W // 2, 5)),
         "other_leaves": lambda: wl_other_leaves(timer, max(K // 10, 5), max(W // 10, 2)),
     }
 

@@ -1,16 +1,18 @@
 // Causal grouped-query attention, BF16: q [B..,Hq,R,D], k and v [B..,Hkv,C,D],
 // out [B..,R,Hq*D]; row r sees tokens t < min(L, a+r+1).
 //
-//   sdpa_pack_v     V of the visible prefix, transposed into matrix-core operand
+//   sdpa_pack       V of the visible prefix, transposed into matrix-core operand
 //                   fragments in the caller's workspace (subnormals flushed to signed
-//                   zero, zeros past L and past D), and a flag raised when a V value
-//                   of the prefix is infinite or NaN.
+//                   zero, zeros past L and past D), K copied tile for tile with the
+//                   same flush, and a flag raised when a V value of the prefix is
+//                   infinite or NaN.
 //   sdpa_mfma       one wave = one head x 16 rows.  Pass 1 forms the scores
 //                   (K tile x Q tile on the matrix cores, binary32) and the row's
 //                   maximum and sum of exponentials; pass 2 forms them again, turns
 //                   them into the normalised probability rounded once to BF16, and
 //                   multiplies by the packed V fragments (binary32 accumulation),
 //                   one BF16 rounding at the store.  Scores never leave registers.
+//   sdpa_decode     few rows per KV head (a decode step): one launch, no workspace.
 //   sdpa_rows       the scalar recurrence in the reference's order (one wave per
 //                   row: sequential sums over features and over tokens).  It runs
 //                   after sdpa_mfma and returns at once unless the flag is up: a
