@@ -161,6 +161,7 @@ constexpr int sdpa_waves(int dt16, int mode) { return mode != 1 ? 4 : dt16 <= 4 
 
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
 // two finite floats to two BF16, round to nearest even (the conversion instruction of gfx950)
 __device__ __forceinline__ uint32_t cvt_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
@@ -556,6 +557,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
     constexpr int D32 = (DT16 + 1) / 2;
     constexpr int NW = 8;
     constexpr int DL = (DT16 + 3) / 4;                 // features per lane (lane, lane + 64)
+    constexpr int PD = DT16 > 6 ? 1 : 2;               // groups in flight per wave (registers allow one at D > 96)
     __shared__ float wave_stats[NW][16][5];
     __shared__ __attribute__((aligned(16))) float p_tile[NW][16][32];
     __shared__ float o_part[NW][16][DL * 64];
@@ -627,32 +629,40 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             }
         };
         // V of group g, lane = feature: the raw bits of the 32 tokens
-        struct VGroup { uint32_t w[32][DL]; };
-        auto load_v = [&](uint32_t g, VGroup& vg) {
+        // V of eight tokens from token t0 of group g on, lane = feature: flushed values
+        auto load_v8 = [&](uint32_t g, uint32_t t0, float (&value)[8][DL]) {
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                uint32_t token = 32 * g + i;
+            for (int i = 0; i < 8; ++i) {
+                uint32_t token = 32 * g + t0 + i;
                 if (token >= vis_max) token = vis_max - 1;            // its probability is +0 and it is masked below
                 const uint8_t* vrow = vb + (uint64_t)(token >> 4) * a.d_tiles * kTileBytes + (token & 15u) * kRowBytes;
 #pragma unroll
                 for (int c = 0; c < DL; ++c) {
                     const uint32_t d = lane + 64 * c;
-                    vg.w[i][c] = d < a.D ? (uint32_t)*reinterpret_cast<const uint16_t*>(
-                                                   vrow + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2)
-                                         : 0u;
+                    value[i][c] = d < a.D ? daz_bf16(*reinterpret_cast<const uint16_t*>(
+                                                    vrow + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2))
+                                          : 0.0f;
                 }
             }
         };
         // pass 1: the rows' statistics over this wave's groups, then over the waves
         RowStats st = {-inf, 0.0f, 0u, false, false};
-        KGroup kcur, knxt;
-        if (wave < groups) load_k(wave, kcur);
+        // a ring of PD groups of K (and of V in pass 2): group g + PD*NW is requested as soon as
+        // group g has been multiplied, so PD groups per wave are in flight -- one wave's chain of
+        // dependent loads is what a long prefix costs here
+        KGroup kr[PD];
+#pragma unroll
+        for (int slot = 0; slot < PD; ++slot)
+            if (wave + slot * NW < groups) load_k(wave + slot * NW, kr[slot]);
 #pragma unroll 1
-        for (uint32_t g = wave; g < groups; g += NW) {
-            if (g + NW < groups) load_k(g + NW, knxt);
+        for (uint32_t g0 = wave; g0 < groups; g0 += PD * NW) {
+#pragma unroll
+          for (int slot = 0; slot < PD; ++slot) {
+            const uint32_t g = g0 + slot * NW;
+            if (g >= groups) break;                                   // uniform
             f32x4_t s[2];
-            scores(kcur, s);
-            kcur = knxt;
+            scores(kr[slot], s);
+            if (g + PD * NW < groups) load_k(g + PD * NW, kr[slot]);
             float local = -inf;
 #pragma unroll
             for (int half = 0; half < 2; ++half)
@@ -672,7 +682,8 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
 #pragma unroll
             for (int half = 0; half < 2; ++half)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) st.sum += s[half][j] == -inf ? 0.0f : __expf(s[half][j] - newm);
+                for (int e = 0; e < 4; ++e) st.sum += s[half][e] == -inf ? 0.0f : __expf(s[half][e] - newm);
+          }
         }
 #pragma unroll
         for (int off = 16; off <= 32; off *= 2) {
@@ -697,50 +708,108 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         const bool nan_row = st.nan || (st.pinf == 0 && !st.finite);
         const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
         const float inv_sum = 1.0f / st.sum;
-        // pass 2: probabilities of a group into LDS, then lane = feature
-        float o[16][DL];
+        // pass 2.  A group that every row in use sees whole goes through the matrix cores: the
+        // probabilities stay in the lanes that formed the scores, V is loaded straight from the
+        // cache in the operand order (lane (feature l16, kg): tokens 32g + 4kg + j and
+        // 32g + 16 + 4kg + j), flushed in registers.  The group on the diagonal and the ragged last
+        // group take the vector units: probabilities to LDS, lane = feature, and a token a row
+        // must not see is left out of that row's sum by a select.
+        const uint32_t vis_min = a.a + 1 < a.L ? a.a + 1 : a.L;          // what row 0 sees: the least
+        const uint32_t full_groups = vis_min / 32;
+        struct VFrag { u32x4 w[DT16]; };
+        auto load_vf = [&](uint32_t g, VFrag& vf) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
+            for (int dt = 0; dt < DT16; ++dt) {
+                // pairs of 16-bit loads into the halves of one register
+                u16x2_t h[4];
 #pragma unroll
-            for (int c = 0; c < DL; ++c) o[r][c] = 0.0f;
-        constexpr bool VAHEAD = DL == 1;                   // wider heads have no registers for two V groups
-        VGroup vcur, vnxt;
-        if (wave < groups) { load_k(wave, kcur); if (VAHEAD) load_v(wave, vcur); }
-#pragma unroll 1
-        for (uint32_t g = wave; g < groups; g += NW) {
-            // the next group's K and V are requested before this group's arithmetic
-            if (!VAHEAD) load_v(g, vcur);
-            if (g + NW < groups) { load_k(g + NW, knxt); if (VAHEAD) load_v(g + NW, vnxt); }
-            f32x4_t s[2];
-            scores(kcur, s);
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t token = 32 * g + (j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4));   // < vis_min <= L
+                    uint16_t bits = 0;
+                    if (dt * kTile + l16 < a.D)
+                        bits = *reinterpret_cast<const uint16_t*>(
+                                vb + ((token >> 4) * a.d_tiles + dt) * kTileBytes + (token & 15u) * kRowBytes + l16 * 2);
+                    h[j >> 1][j & 1] = bits;
+                }
+                vf.w[dt] = u32x4{daz2(__builtin_bit_cast(uint32_t, h[0])), daz2(__builtin_bit_cast(uint32_t, h[1])),
+                                 daz2(__builtin_bit_cast(uint32_t, h[2])), daz2(__builtin_bit_cast(uint32_t, h[3]))};
+            }
+        };
+        f32x4_t om[DT16];                                   // matrix-core part: out[row l16][16 dt + 4 kg + j]
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                f32x4_t pr;
+        for (int dt = 0; dt < DT16; ++dt) om[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        // the probabilities of a group, rounded once to BF16 and flushed like every operand of the
+        // product (p >= 0), two to a word
+        auto probabilities = [&](uint32_t g, const f32x4_t (&s)[2]) -> u32x4 {
+            float pr[8];
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const float v = s[half][j];
                     const bool seen = (32 * g + 16 * half + 4 * kg + j < vis) & !nan_row;
                     const float regular = v == -inf ? 0.0f : __expf(v - st.m) * inv_sum;
                     const float special = v == inf ? pinf_p : 0.0f;
-                    const float e = seen ? (st.pinf ? special : regular) : 0.0f;
-                    // one rounding to BF16, flushed like every operand of the product (p >= 0)
-                    pr[j] = daz_bf16(bf16_rne_sw(as_u32(e)));
+                    pr[half * 4 + j] = seen ? (st.pinf ? special : regular) : 0.0f;
                 }
-                *reinterpret_cast<f32x4_t*>(&p_tile[wave][l16][16 * half + 4 * kg]) = pr;
+            return u32x4{daz2(pack_bf16(pr[0], pr[1])), daz2(pack_bf16(pr[2], pr[3])),
+                         daz2(pack_bf16(pr[4], pr[5])), daz2(pack_bf16(pr[6], pr[7]))};
+        };
+        {
+            VFrag vr[PD];
+#pragma unroll
+            for (int slot = 0; slot < PD; ++slot)
+                if (wave + slot * NW < full_groups) {
+                    load_k(wave + slot * NW, kr[slot]);
+                    load_vf(wave + slot * NW, vr[slot]);
+                }
+#pragma unroll 1
+            for (uint32_t g0 = wave; g0 < full_groups; g0 += PD * NW) {
+#pragma unroll
+                for (int slot = 0; slot < PD; ++slot) {
+                    const uint32_t g = g0 + slot * NW;
+                    if (g >= full_groups) break;                              // uniform
+                    f32x4_t s[2];
+                    scores(kr[slot], s);
+                    if (g + PD * NW < full_groups) load_k(g + PD * NW, kr[slot]);
+                    const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, probabilities(g, s));
+#pragma unroll
+                    for (int dt = 0; dt < DT16; ++dt)
+                        om[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vr[slot].w[dt]), pf, om[dt], 0, 0, 0);
+                    if (g + PD * NW < full_groups) load_vf(g + PD * NW, vr[slot]);
+                }
+            }
+        }
+        float o[16][DL];                                    // vector part: out[row r][lane + 64 c]
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+#pragma unroll
+            for (int c = 0; c < DL; ++c) o[r][c] = 0.0f;
+        // the one or two groups past the fully visible ones, each with the wave whose turn it is
+#pragma unroll 1
+        for (uint32_t g = full_groups + (wave + NW - full_groups % NW) % NW; g < groups; g += NW) {
+            KGroup kt;
+            load_k(g, kt);
+            f32x4_t s[2];
+            scores(kt, s);
+            const u32x4 pw = probabilities(g, s);
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                f32x4_t pe;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t pair = pw[half * 2 + (j >> 1)];
+                    pe[j] = as_f32((j & 1) ? (pair & 0xFFFF0000u) : (pair << 16));
+                }
+                *reinterpret_cast<f32x4_t*>(&p_tile[wave][l16][16 * half + 4 * kg]) = pe;
             }
             // the wave reads only what it wrote itself: LDS operations of a wave complete in order
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            // every tile row in use takes its probabilities (16-byte broadcasts) and adds.  Where
-            // every row in use sees all eight tokens of a chunk no select is needed.
-            const uint32_t vis_min = a.a + 1 < a.L ? a.a + 1 : a.L;          // what row 0 sees: the least
+            // every tile row in use takes its probabilities (16-byte broadcasts) and adds
 #pragma unroll
             for (int t0 = 0; t0 < 32; t0 += 8) {
                 float value[8][DL];
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-#pragma unroll
-                    for (int c = 0; c < DL; ++c) value[i][c] = daz_bf16(vcur.w[t0 + i][c]);
-                const bool all_seen = 32 * g + t0 + 8 <= vis_min;             // uniform
+                load_v8(g, t0, value);
 #pragma unroll
                 for (int r4 = 0; r4 < 16; r4 += 4) {
                     if ((uint32_t)r4 >= nrows) break;                         // uniform; rows past nrows hold +0
@@ -751,41 +820,34 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                         pa[q] = *reinterpret_cast<const f32x4_t*>(&p_tile[wave][r4 + q][t0]);
                         pb[q] = *reinterpret_cast<const f32x4_t*>(&p_tile[wave][r4 + q][t0 + 4]);
                     }
-                    if (all_seen) {
 #pragma unroll
-                        for (int q = 0; q < 4; ++q)
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t rr = (uint32_t)(r4 + q) / a.grouping;
+                        const uint32_t reach_r = a.a + rr + 1;
+                        const uint32_t vis_r = reach_r < a.L ? reach_r : a.L; // uniform: what this row may see
 #pragma unroll
-                            for (int i = 0; i < 8; ++i)
+                        for (int i = 0; i < 8; ++i) {
+                            const bool seen = 32 * g + t0 + i < vis_r;
 #pragma unroll
-                                for (int c = 0; c < DL; ++c)
-                                    o[r4 + q][c] = __builtin_fmaf(i < 4 ? pa[q][i & 3] : pb[q][i & 3], value[i][c], o[r4 + q][c]);
-                    } else {
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) {
-                            const uint32_t rr = (uint32_t)(r4 + q) / a.grouping;
-                            const uint32_t reach_r = a.a + rr + 1;
-                            const uint32_t vis_r = reach_r < a.L ? reach_r : a.L; // uniform: what this row may see
-#pragma unroll
-                            for (int i = 0; i < 8; ++i) {
-                                const bool seen = 32 * g + t0 + i < vis_r;
-#pragma unroll
-                                for (int c = 0; c < DL; ++c)
-                                    o[r4 + q][c] = seen ? __builtin_fmaf(i < 4 ? pa[q][i & 3] : pb[q][i & 3], value[i][c], o[r4 + q][c])
-                                                        : o[r4 + q][c];
-                            }
+                            for (int c = 0; c < DL; ++c)
+                                o[r4 + q][c] = seen ? __builtin_fmaf(i < 4 ? pa[q][i & 3] : pb[q][i & 3], value[i][c], o[r4 + q][c])
+                                                    : o[r4 + q][c];
                         }
                     }
                 }
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // p_tile is rewritten by the next group
-            kcur = knxt;
-            if (VAHEAD) vcur = vnxt;
         }
-        // the waves' partial outputs meet in LDS
+        // the waves' partial outputs meet in LDS: the vector part, then the matrix-core part on
+        // top of it (LDS operations of a wave complete in order)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
 #pragma unroll
             for (int c = 0; c < DL; ++c) o_part[wave][r][lane + 64 * c] = o[r][c];
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o_part[wave][l16][dt * 16 + 4 * kg + j] += om[dt][j];
         __syncthreads();
         // thread = (tile row, feature): 16 x D outputs over 512 threads
         for (uint32_t idx = threadIdx.x; idx < 16 * DL * 64; idx += 512) {
