@@ -352,6 +352,32 @@ def test_linear_full_size_by_linearity_and_sampled_rows():
         t.free()
 
 
+@pytest.mark.parametrize("rows,outs,planar", [(4096, 5632, False), (6144, 5632, False), (4100, 5600, True), (1000, 2096, False)],
+                         ids=["352_blocks", "528_blocks", "ragged_head_planar", "ragged_small"])
+def test_linear_tile_mix_equals_the_direct_kernel(rows, outs, planar):
+    """Shapes whose 256 x 256 blocks do not fill whole rounds of the CUs run as two launches
+    with different tiles (or with the smaller tiles alone); ragged row and output counts leave
+    partial blocks at both edges.  All workgroup-tiled kernels add the same products in the
+    same order as the direct kernel: the outputs are the same bits, the padding is untouched."""
+    I, D = 64, 16 if planar else outs
+    H = outs // D
+    x = datagen.bf16_rne(datagen.normal_f32(rows * I, 0, 1, 301)).reshape(1, rows, I)
+    w = datagen.bf16_rne(datagen.normal_f32(outs * I, 0, 0.1, 302)).reshape(outs, I)
+    dx = iomx.DeviceTensor(DT_BF16, (1, rows, I)); dx.view().from_host(x)
+    dw = iomx.DeviceTensor(DT_BF16, (outs, I)); dw.view().from_host(w)
+    od = (1, H, rows, D) if planar else (1, rows, outs)
+    outs_ = []
+    for path in (0, 2):
+        do = iomx.DeviceTensor(DT_BF16, od, fill=0x5A)
+        assert iomx.linear(dx.view(), dw.view(), do.view(), 0, rows, planar, H, D, path=path) == 0
+        assert iomx.last_launch().kernel.decode() == ("linear_mfma_lds" if path == 0 else "linear_mfma")
+        outs_.append(do.raw().copy())
+        do.free()
+    assert np.array_equal(outs_[0], outs_[1])
+    for t in (dx, dw):
+        t.free()
+
+
 def test_attention_full_size_by_uniform_scores_and_sampled_rows():
     """Prefill of the benchmark shape (8 sequences, 32 query / 4 KV heads, R = L = 512,
     D = 64).  Heads whose queries are zero give every visible token the same probability:
