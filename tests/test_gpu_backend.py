@@ -315,3 +315,39 @@ def test_bad_factory_configuration_is_rejected_before_any_native_effect():
     assert b"invalid_argument" in l.iomc_last_error()
     assert not l.iomc_mi355x_device_create(0, 1000, 16)           # not a multiple of 32
     assert not l.iomc_mi355x_device_create(99, 1 << 20, 16)       # no such ordinal
+
+
+def test_submit_and_wait_cost_through_device_ops(devices, capsys):
+    """What a caller pays on top of the kernel: one add submitted and waited for through
+    DeviceOps (validation, snapshots, registry entries, admission, launch, event, completion
+    thread), and a burst of 64 submissions with one wait.  Printed for the record; the bounds
+    only catch a queue that has started to serialise on something slow."""
+    import time
+    del devices                      # (the shared fixture keeps four operations in flight; the default is 16)
+    gpu = iomo.mi355x_backend(arena_bytes=1 << 29, max_in_flight=16)
+    small = (1, 16, 2048)
+    big = (16, 512, 2048)
+    for dims, label in ((small, "64 KiB"), (big, "32 MiB")):
+        a, b, o = (gpu.tensor(DT_BF16, dims) for _ in range(3))
+        av, bv, ov = a.view(), b.view(), o.view()
+        for _ in range(20):
+            assert gpu.wait(gpu.l.iomc_binary(gpu.queue, OP_ADD, av.h, bv.h, ov.h)) == 0
+        single = []
+        for _ in range(200):
+            t0 = time.perf_counter()
+            tok = gpu.l.iomc_binary(gpu.queue, OP_ADD, av.h, bv.h, ov.h)
+            assert gpu.wait(tok) == 0
+            single.append(time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        for _ in range(64):
+            tok = gpu.l.iomc_binary(gpu.queue, OP_ADD, av.h, bv.h, ov.h)
+            assert tok > 0
+        assert gpu.wait(tok) == 0
+        burst = (time.perf_counter() - t0) / 64
+        single.sort()
+        with capsys.disabled():
+            print("\n  DeviceOps add BF16 %s: submit+wait median %.1f us (p90 %.1f), burst of 64 %.1f us per op"
+                  % (label, single[100] * 1e6, single[180] * 1e6, burst * 1e6), flush=True)
+        assert single[100] < 2e-3 and burst < 1e-3
+        close(a, b, o)
+    gpu.close()
