@@ -148,6 +148,8 @@ struct RowStats {
 // or 128: the workgroup brings every K and V group into LDS once, with the direct loader,
 // three groups deep, and its four waves read their operands from there -- the vector
 // memory pipeline of the CU, which bounds MODE 0, carries a quarter of the bytes.
+// MODE 3: the same ring for any grouping: the four waves are four consecutive row tiles of one
+// head (the workgroup walks the groups of its last tile; a wave sits out the groups past its own).
 // FULLD: D is a multiple of 32, no operand load needs a guard against the columns past D.
 //
 // Both passes exist twice.  The plain one assumes what almost every row satisfies -- no
@@ -174,7 +176,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     // waves and requests the next group ahead instead
     constexpr bool AHEAD = MODE == 1;
     constexpr bool SPLIT = MODE == 1;
-    constexpr bool SHARE = MODE == 2;
+    constexpr bool SHARE = MODE == 2 || MODE == 3;
     static_assert(!SHARE || (DT16 % 4 == 0 && FULLD), "shared groups: whole KiB chunks per wave");
     constexpr uint32_t kStage = 2 * DT16 * 1024;           // K group + V group
     __shared__ __attribute__((aligned(16))) uint8_t kv_ring[SHARE ? 3 * kStage : 16];
@@ -189,19 +191,25 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     // which (head, row) the lane's tile row is
-    const uint32_t head = MODE == 1 ? blockIdx.x : blockIdx.x * 4 + wave;
+    const uint32_t head = (MODE == 1 || MODE == 3) ? blockIdx.x : blockIdx.x * 4 + wave;
     if (MODE == 0 && head >= a.Hq) return;          // no barrier on this path (MODE 2: Hq is a multiple of 4)
     const uint32_t hkv = head / a.grouping;
     // grid = (heads, planes, row tiles): the row tiles with the longest prefixes are dispatched
     // first, for every head and plane, and the short ones fill the end of the launch
-    const uint32_t first_row = (gridDim.z - 1 - blockIdx.z) * kTile, row = first_row + l16;
+    const uint32_t slab = gridDim.z - 1 - blockIdx.z;
+    const uint32_t first_row = (MODE == 3 ? slab * 4 + wave : slab) * kTile, row = first_row + l16;
+    const bool ghost = MODE == 3 && first_row >= a.R;       // a wave past the last row tile: barriers only
     const uint32_t last_row = first_row + 15 < a.R ? first_row + 15 : a.R - 1;
     const bool row_ok = row < a.R;
     const uint32_t qrow = row_ok ? row : a.R - 1;
     const uint32_t reach = a.a + row + 1, reach_min = a.a + first_row + 1, reach_max = a.a + last_row + 1;
     const uint32_t vis = row_ok ? (reach < a.L ? reach : a.L) : 0;     // tokens this lane's row sees
     const uint32_t vis_max = reach_max < a.L ? reach_max : a.L;        // ... and the tile's last row
-    const uint32_t groups = (vis_max + 31) / 32;
+    const uint32_t groups = ghost ? 0 : (vis_max + 31) / 32;
+    // the groups the workgroup brings in: those of its last row tile (MODE 3), else the wave's own
+    const uint32_t slab_last = slab * 64 + 63 < a.R ? slab * 64 + 63 : a.R - 1;
+    const uint32_t slab_reach = a.a + slab_last + 1;
+    const uint32_t ring_groups = MODE == 3 ? ((slab_reach < a.L ? slab_reach : a.L) + 31) / 32 : groups;
     // groups that every row of the tile sees whole need no mask
     const uint32_t full_groups = (reach_min < a.L ? reach_min : a.L) / 32;
     // the plain passes let the rows past R mirror the last row (their results are dropped)
@@ -279,7 +287,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 // chunk + 16*i, so a group lies in LDS as it lies in the packed regions
                 constexpr int LPS = (WITH_V ? 2 : 1) * (DT16 / 4);        // direct loads per wave and stage
                 auto issue = [&](uint32_t g, uint32_t buf) {
-                    const uint32_t gg = g < groups ? g : groups - 1;      // past the end: a valid group again, unused
+                    const uint32_t gg = g < ring_groups ? g : ring_groups - 1;   // past the end: a valid group again, unused
                     uint8_t* stage = kv_ring + buf * kStage;
 #pragma unroll
                     for (int j = 0; j < DT16 / 4; ++j) {
@@ -295,13 +303,15 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 issue(1, 1);
                 uint32_t buf = 0;
 #pragma unroll 1
-                for (uint32_t g = 0; g < groups; ++g) {
+                for (uint32_t g = 0; g < ring_groups; ++g) {
                     // the own loads of group g have landed; past the barrier everybody's have, and
                     // nobody reads the buffer of group g-1 any more: it takes group g+2
                     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPS) : "memory");
                     __builtin_amdgcn_s_barrier();
                     issue(g + 2, buf == 0 ? 2 : buf - 1);
                     const uint8_t* stage = kv_ring + buf * kStage;
+                    buf = buf == 2 ? 0 : buf + 1;
+                    if (MODE == 3 && g >= groups) continue;               // uniform: past this wave's own tile
                     KGroup cur;
 #pragma unroll
                     for (int half = 0; half < 2; ++half)
@@ -318,7 +328,6 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                     f32x4_t s[2];
                     scores(cur, s);
                     body(g, s, vfr);
-                    buf = buf == 2 ? 0 : buf + 1;
                 }
                 // nothing in flight and nobody reading when the next pass (or the next workgroup)
                 // takes the ring
@@ -401,7 +410,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         }
         // a NaN or +infinity score, or no finite score at all, shows here; every wave of the
         // workgroup holds the same joined values and decides alike
-        const bool odd = !(psum > 0.0f && psum < inf && pm < inf);
+        const bool odd = !ghost && !(psum > 0.0f && psum < inf && pm < inf);
         // (sharing the groups, the four waves also share the decision: they meet at barriers)
         const bool plain = SHARE ? !__syncthreads_or(odd ? 1 : 0) : !__any(odd);
 
@@ -1171,6 +1180,7 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         int mode = 0;
         if ((uint64_t)row_tiles * g.Hq * g.planes < 4096 && g.groups >= 8) mode = 1;
         else if ((g.D == 64 || g.D == 128) && g.grouping % 4 == 0) mode = 2;
+        else if ((g.D == 64 || g.D == 128) && row_tiles >= 4) mode = 3;
         g.flags = static_cast<uint32_t*>(workspace);
         g.packed_v = static_cast<uint8_t*>(workspace) + header;
         g.packed_k = g.packed_v + region;
@@ -1179,7 +1189,7 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         const bool full_d = (g.D & 31u) == 0;
         for (g.plane0 = 0; g.plane0 < g.planes; g.plane0 += 65535u) {
         const uint32_t layers = g.planes - g.plane0 < 65535u ? g.planes - g.plane0 : 65535u;
-        const dim3 grid(mode == 1 ? g.Hq : (g.Hq + 3) / 4, layers, row_tiles);
+        const dim3 grid(mode == 1 || mode == 3 ? g.Hq : (g.Hq + 3) / 4, layers, mode == 3 ? (row_tiles + 3) / 4 : row_tiles);
 #define IOMX_SDPA_MODE(N, M) \
     if (full_d) hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, M, true>), grid, dim3(sdpa_waves(N, M) * 64), 0, st, g); \
     else hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<N, M, false>), grid, dim3(sdpa_waves(N, M) * 64), 0, st, g)
@@ -1192,6 +1202,10 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
             hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<4, 2, true>), grid, dim3(256), 0, st, g);
         else if (mode == 2)
             hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<8, 2, true>), grid, dim3(256), 0, st, g);
+        else if (mode == 3 && g.d_tiles == 4)
+            hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<4, 3, true>), grid, dim3(256), 0, st, g);
+        else if (mode == 3)
+            hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<8, 3, true>), grid, dim3(256), 0, st, g);
         else switch (g.d_tiles) {
             IOMX_SDPA(1) IOMX_SDPA(2) IOMX_SDPA(3) IOMX_SDPA(4)
             IOMX_SDPA(5) IOMX_SDPA(6) IOMX_SDPA(7)
@@ -1200,7 +1214,7 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
 #undef IOMX_SDPA_MODE
 #undef IOMX_SDPA
         }
-        record_launch("sdpa_mfma", row_tiles * (mode == 1 ? g.Hq : (g.Hq + 3) / 4) * gz, 256,
+        record_launch("sdpa_mfma", (mode == 3 ? (row_tiles + 3) / 4 : row_tiles) * (mode == 1 || mode == 3 ? g.Hq : (g.Hq + 3) / 4) * gz, 256,
                       (uint64_t)g.planes * g.Hq * g.R);
         g.guarded = 1;
     }

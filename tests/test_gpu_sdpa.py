@@ -86,7 +86,8 @@ def test_reference_fixtures(index, path, kernel):
 
 SEEDED = [((), 2, 1, 5, 8, 12, 3, 9), ((2,), 4, 2, 17, 16, 40, 20, 37), ((2, 2), 4, 1, 3, 33, 20, 0, 2),
           ((), 8, 2, 1, 64, 70, 69, 70), ((3,), 2, 2, 16, 5, 16, 0, 16), ((2,), 8, 2, 40, 64, 100, 50, 90),
-          ((), 4, 4, 33, 128, 64, 10, 43), ((), 2, 1, 70, 48, 200, 100, 170), ((), 8, 2, 33, 128, 64, 10, 43)]
+          ((), 4, 4, 33, 128, 64, 10, 43), ((), 2, 1, 70, 48, 200, 100, 170), ((), 8, 2, 33, 128, 64, 10, 43),
+          ((2,), 4, 4, 70, 64, 100, 20, 90), ((), 6, 3, 100, 128, 120, 10, 110)]
 
 
 def float64_attention(case):
@@ -169,14 +170,17 @@ def test_tail_future_tokens_and_special_v(R):
     assert np.array_equal(g[1], base.reshape(2, R, 4, 16)[1])
 
 
+@pytest.mark.parametrize("Hkv", [2, 8], ids=["four_heads_share", "four_row_tiles_share"])
 @pytest.mark.parametrize("D", [64, 128])
-def test_special_scores_where_four_heads_share_the_groups(D):
-    """Eight query heads on two KV heads (the tiled kernel's four waves read K and V from one
-    LDS ring and fall back to the special-row passes together): K rows that make scores of
-    +infinity and -infinity, a NaN in one Q row, a row of zero scores."""
-    case = random_case(61, (2,), 8, 2, 40, D, 70, 20, 60)
-    q = np.array(case["q"], np.uint16).reshape(2, 8, 40, D).copy()
-    k = np.array(case["k"], np.uint16).reshape(2, 2, 70, D).copy()
+def test_special_scores_where_four_waves_share_the_groups(D, Hkv):
+    """Eight query heads on two KV heads (the tiled kernel's four waves = four heads read K and
+    V from one LDS ring and fall back to the special-row passes together) or on eight (four
+    waves = four row tiles of one head, the last workgroup with waves past the last tile): K
+    rows that make scores of +infinity and -infinity, a NaN in one Q row, a row of zero scores."""
+    R = 40 if Hkv == 2 else 72
+    case = random_case(61, (2,), 8, Hkv, R, D, 100, 20, 20 + R)
+    q = np.array(case["q"], np.uint16).reshape(2, 8, R, D).copy()
+    k = np.array(case["k"], np.uint16).reshape(2, Hkv, 100, D).copy()
     k[0, 0, 5, 3] = 0x7F80            # +inf in one feature: the score is +inf or -inf by the sign of q
     k[1, 1, 9, 2] = 0xFF80
     q[0, 6, 3, 7] = 0x7FC0            # NaN row (plane 0, head 6, row 3)
@@ -185,13 +189,15 @@ def test_special_scores_where_four_heads_share_the_groups(D):
     got = run(special, 0, expect_kernel="sdpa_mfma")
     want = oracle(special)
     assert close_to_oracle(got, want) == []
-    g = got.reshape(2, 40, 8, D)
+    g = got.reshape(2, R, 8, D)
     assert np.all((g[0, 3, 6] & 0x7FFF) > 0x7F80)                    # the NaN row is NaN
-    # plane 1, KV head 0 (heads 0..3) has nothing special: bits equal those of the plain case
-    plain = run(case, 0).reshape(2, 40, 8, D)
-    keep = np.ones((40, 4), bool)
-    keep[30, 1] = False
-    assert np.array_equal(g[1][:, :4][keep], plain[1][:, :4][keep])
+    # plane 1, KV head 0 (its query heads) has nothing special: bits equal those of the plain case
+    plain = run(case, 0).reshape(2, R, 8, D)
+    heads = 8 // Hkv
+    keep = np.ones((R, heads), bool)
+    if heads > 1:
+        keep[30, 1] = False
+    assert np.array_equal(g[1][:, :heads][keep], plain[1][:, :heads][keep])
 
 
 @pytest.mark.parametrize("R,kernel", [(1, "sdpa_decode"), (17, "sdpa_mfma")], ids=["decode_kernel", "tiled_kernel_and_guard"])
