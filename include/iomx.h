@@ -298,9 +298,9 @@ int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const 
  * one flag word per plane, KV head and pack share (256-byte aligned, no
  * initialisation).  path 0: the decode kernel (one launch: scores on the matrix cores,
  * P*V on the vector units straight from the cache) for the few-row requests, else the
- * pack kernel, the matrix-core kernel (D <= 128) and the reference-order kernel, which
- * returns at once unless V holds an infinity or NaN; path 1 runs the reference-order
- * kernel alone (D <= 256, no workspace).
+ * pack kernel and the matrix-core kernel (D <= 128), which forms the rows of a KV head
+ * whose V holds an infinity or NaN in the reference's order instead; path 1 runs the
+ * reference-order kernel alone (D <= 256, no workspace).
  */
 int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
                         const iomx_view* out, uint64_t a, uint64_t L, uint64_t* bytes,

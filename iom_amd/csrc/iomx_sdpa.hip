@@ -14,11 +14,11 @@
 //                   one BF16 rounding at the store.  Scores never leave registers.
 //   sdpa_decode     few rows per KV head (a decode step): one launch, no workspace.
 //   sdpa_rows       the scalar recurrence in the reference's order (one wave per
-//                   row: sequential sums over features and over tokens).  It runs
-//                   after sdpa_mfma and returns at once unless the flag is up: a
+//                   row: sequential sums over features and over tokens): the path
+//                   for head sizes the fragments do not cover.  sdpa_mfma forms its
+//                   rows the same way where the flag of their KV head is up: a
 //                   masked probability is +0, and +0 times an infinite V of a token
 //                   the row must not see would poison the row on the matrix cores.
-//                   It is also the path for head sizes the fragments do not cover.
 #include <type_traits>
 
 #include "iomx_mfma.hpp"
@@ -42,7 +42,6 @@ struct SdpaArgs {
     uint32_t* flags;            // [plane][kv head][pack split]: nonzero = that part of the V prefix
                                 // holds an infinity or NaN
     uint32_t pack_splits;       // workgroups sharing the fragments of one KV head
-    uint32_t guarded;           // sdpa_rows: skip the rows whose KV head has no flag up
     float scale;                // sqrtf(D)
     float inv_scale;            // 1 / scale, rounded
     uint32_t scale_pow2;        // scale is a power of two: the product with inv_scale is the quotient
@@ -140,6 +139,124 @@ struct RowStats {
     }
 };
 
+// Orders the LDS traffic of one wave: its lanes run in lockstep and its LDS operations
+// complete in order.
+__device__ __forceinline__ void wave_sync() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// One row of one head in the reference's own order of operations (src/cpu/sdpa.cpp:132-336):
+// sequential sums over features and over tokens, by one wave; pbuf = 64 floats of LDS of this wave.
+__device__ __forceinline__ void sdpa_reference_row(const SdpaArgs& a, uint32_t p, uint32_t hkv, uint32_t head,
+                                                uint32_t row, uint32_t lane, float* pbuf) {
+    const float inf = __builtin_inff();
+    const uint32_t reach = a.a + row + 1;
+    const uint32_t vis = reach < a.L ? reach : a.L;
+    uint64_t plane[4];
+    walk_planes(a.walk, p, plane);
+    const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes
+            + (uint64_t)(row >> 4) * a.d_tiles * kTileBytes + (row & 15u) * kRowBytes;
+    const uint8_t* kb = a.k + (plane[1] + (uint64_t)hkv * a.k_head_stride) * a.kv_plane_bytes;
+    const uint8_t* vb = a.v + (plane[2] + (uint64_t)hkv * a.v_head_stride) * a.kv_plane_bytes;
+    auto element = [&](const uint8_t* row_base, uint32_t d) {
+        return daz_bf16(*reinterpret_cast<const uint16_t*>(row_base + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2));
+    };
+    auto score = [&](uint32_t t) {
+        const uint8_t* kr = kb + (uint64_t)(t >> 4) * a.d_tiles * kTileBytes + (t & 15u) * kRowBytes;
+        float dot = 0.0f;
+        for (uint32_t d = 0; d < a.D; ++d) dot = dot + element(qb, d) * element(kr, d);   // products are exact
+        return dot / a.scale;
+    };
+    // classes and maximum
+    float m = -inf;
+    uint32_t pinf = 0;
+    bool nan = false, not_ninf = false;
+    for (uint32_t t = lane; t < vis; t += 64) {
+        const float s = score(t);
+        nan = nan || s != s;
+        pinf += s == inf ? 1u : 0u;
+        not_ninf = not_ninf || s != -inf;
+        if (s > m) m = s;
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off *= 2) {
+        // every lane takes part in every exchange (no short-circuit around a shuffle)
+        const float m2 = __shfl_xor(m, off);
+        const uint32_t p2 = __shfl_xor(pinf, off);
+        const int n2 = __shfl_xor((int)nan, off), f2 = __shfl_xor((int)not_ninf, off);
+        m = m2 > m ? m2 : m;
+        pinf += p2;
+        nan = nan || n2 != 0;
+        not_ninf = not_ninf || f2 != 0;
+    }
+    uint8_t* ob = a.out + plane[3] * a.out_plane_bytes
+            + (uint64_t)(row >> 4) * a.out_tile_cols * kTileBytes + (row & 15u) * kRowBytes;
+    auto store = [&](uint32_t d, uint32_t bits) {
+        const uint32_t col = head * a.D + d;
+        *reinterpret_cast<uint16_t*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) = (uint16_t)bits;
+    };
+    if (nan || !not_ninf) {
+        for (uint32_t d = lane; d < a.D; d += 64) store(d, 0x7FC0u);
+        return;
+    }
+    // sum of exponentials in token order
+    float sum = 0.0f;
+    if (pinf == 0) {
+        for (uint32_t t0 = 0; t0 < vis; t0 += 64) {
+            const uint32_t t = t0 + lane;
+            float e = 0.0f;
+            if (t < vis) {
+                const float s = score(t);
+                if (s != -inf) e = expf(s - m);
+            }
+            for (int i = 0; i < 64; ++i) sum = sum + __shfl(e, i);     // adding +0 changes nothing
+        }
+    }
+    const float pinf_p = pinf ? 1.0f / (float)pinf : 0.0f;
+    // out = sum over tokens of P * V, features over lanes (up to 256)
+    float result[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t t0 = 0; t0 < vis; t0 += 64) {
+        const uint32_t t = t0 + lane;
+        float pr = 0.0f;
+        if (t < vis) {
+            const float s = score(t);
+            if (pinf) pr = s == inf ? pinf_p : 0.0f;
+            else if (s != -inf) pr = expf(s - m) / sum;
+        }
+        wave_sync();                                   // the previous chunk's readers are done
+        pbuf[lane] = daz_bf16(bf16_rne_sw(as_u32(pr)));
+        wave_sync();
+        const uint32_t n = vis - t0 < 64 ? vis - t0 : 64;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t d = lane + 64 * c;
+            if (d >= a.D) continue;
+            for (uint32_t i = 0; i < n; ++i) {
+                const uint32_t tt = t0 + i;
+                const uint8_t* vr = vb + (uint64_t)(tt >> 4) * a.d_tiles * kTileBytes + (tt & 15u) * kRowBytes;
+                result[c] = result[c] + pbuf[i] * element(vr, d);             // products are exact
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t d = lane + 64 * c;
+        if (d >= a.D) continue;
+        float val = result[c];
+        if (val == 0.0f) val = 0.0f;
+        store(d, bf16_rne_sw(as_u32(val)));
+    }
+}
+
+// KV heads of plane p whose V prefix holds an infinity or NaN (any share's flag up)
+__device__ __forceinline__ bool sdpa_flag_up(const SdpaArgs& a, uint32_t p, uint32_t hkv) {
+    uint32_t up = 0;
+    const uint64_t pair = (uint64_t)p * a.Hkv + hkv;
+    for (uint32_t i = 0; i < a.pack_splits; ++i) up |= a.flags[pair * a.pack_splits + i];
+    return up != 0;                       // uniform: every lane reads the same words
+}
+
 // MODE 0: a workgroup of four waves = four heads of one row tile, each wave walks
 // all visible tokens (prefill: many row tiles, K and V shared through the caches).
 // MODE 1: one head, the 4 or 8 waves share out the 32-token groups and meet in LDS (few
@@ -221,6 +338,16 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     // lane offset of the body alive across it, far beyond the register file)
     {
         const uint32_t p = a.plane0 + blockIdx.y;
+        if (sdpa_flag_up(a, p, hkv)) {
+            // V of this KV head holds an infinity or NaN.  A masked probability is +0, and on the
+            // matrix cores +0 times an infinite V of a token the row must not see would poison
+            // the row: these rows are formed in the reference's order instead.  (All waves of a
+            // workgroup that meets at barriers share the KV head and leave together.)
+            float* pbuf = &wave_stats[wave][0][0];
+            for (uint32_t r = SPLIT ? wave : 0; r < kTile; r += SPLIT ? NW : 1)
+                if (first_row + r < a.R) sdpa_reference_row(a, p, hkv, head, first_row + r, lane, pbuf);
+            return;
+        }
         uint64_t plane[4];
         walk_planes(a.walk, p, plane);
         const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
@@ -894,117 +1021,14 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
 __global__ __launch_bounds__(64) void sdpa_rows_kernel(const SdpaArgs a) {
     __shared__ float pbuf[64];
     const uint32_t lane = threadIdx.x;
-    const float inf = __builtin_inff();
-    // blockIdx.y walks the (plane, KV head) pairs, blockIdx.x the rows of the pair's
-    // query heads; a guarded launch leaves a pair whose flags are all down at once
+    // blockIdx.y walks the (plane, KV head) pairs, blockIdx.x the rows of the pair's query heads
     const uint32_t pairs = a.planes * a.Hkv, per_pair = a.grouping * a.R;
     for (uint32_t pair = blockIdx.y; pair < pairs; pair += gridDim.y) {
-      const uint32_t p = pair / a.Hkv, hkv = pair - p * a.Hkv;
-      if (a.guarded) {
-          uint32_t up = 0;
-          for (uint32_t i = 0; i < a.pack_splits; ++i) up |= a.flags[(uint64_t)pair * a.pack_splits + i];
-          if (up == 0) continue;            // uniform: every lane reads the same words
-      }
-      for (uint32_t it = blockIdx.x; it < per_pair; it += gridDim.x) {
-        const uint32_t hg = it / a.R, row = it - hg * a.R;
-        const uint32_t head = hkv * a.grouping + hg;
-        const uint32_t reach = a.a + row + 1;
-        const uint32_t vis = reach < a.L ? reach : a.L;
-        uint64_t plane[4];
-        walk_planes(a.walk, p, plane);
-        const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes
-                + (uint64_t)(row >> 4) * a.d_tiles * kTileBytes + (row & 15u) * kRowBytes;
-        const uint8_t* kb = a.k + (plane[1] + (uint64_t)hkv * a.k_head_stride) * a.kv_plane_bytes;
-        const uint8_t* vb = a.v + (plane[2] + (uint64_t)hkv * a.v_head_stride) * a.kv_plane_bytes;
-        auto element = [&](const uint8_t* row_base, uint32_t d) {
-            return daz_bf16(*reinterpret_cast<const uint16_t*>(row_base + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2));
-        };
-        auto score = [&](uint32_t t) {
-            const uint8_t* kr = kb + (uint64_t)(t >> 4) * a.d_tiles * kTileBytes + (t & 15u) * kRowBytes;
-            float dot = 0.0f;
-            for (uint32_t d = 0; d < a.D; ++d) dot = dot + element(qb, d) * element(kr, d);   // products are exact
-            return dot / a.scale;
-        };
-        // classes and maximum
-        float m = -inf;
-        uint32_t pinf = 0;
-        bool nan = false, not_ninf = false;
-        for (uint32_t t = lane; t < vis; t += 64) {
-            const float s = score(t);
-            nan = nan || s != s;
-            pinf += s == inf ? 1u : 0u;
-            not_ninf = not_ninf || s != -inf;
-            if (s > m) m = s;
+        const uint32_t p = pair / a.Hkv, hkv = pair - p * a.Hkv;
+        for (uint32_t it = blockIdx.x; it < per_pair; it += gridDim.x) {
+            const uint32_t hg = it / a.R, row = it - hg * a.R;
+            sdpa_reference_row(a, p, hkv, hkv * a.grouping + hg, row, lane, pbuf);
         }
-#pragma unroll
-        for (int off = 1; off < 64; off *= 2) {
-            // every lane takes part in every exchange (no short-circuit around a shuffle)
-            const float m2 = __shfl_xor(m, off);
-            const uint32_t p2 = __shfl_xor(pinf, off);
-            const int n2 = __shfl_xor((int)nan, off), f2 = __shfl_xor((int)not_ninf, off);
-            m = m2 > m ? m2 : m;
-            pinf += p2;
-            nan = nan || n2 != 0;
-            not_ninf = not_ninf || f2 != 0;
-        }
-        uint8_t* ob = a.out + plane[3] * a.out_plane_bytes
-                + (uint64_t)(row >> 4) * a.out_tile_cols * kTileBytes + (row & 15u) * kRowBytes;
-        auto store = [&](uint32_t d, uint32_t bits) {
-            const uint32_t col = head * a.D + d;
-            *reinterpret_cast<uint16_t*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) = (uint16_t)bits;
-        };
-        if (nan || !not_ninf) {
-            for (uint32_t d = lane; d < a.D; d += 64) store(d, 0x7FC0u);
-            continue;
-        }
-        // sum of exponentials in token order
-        float sum = 0.0f;
-        if (pinf == 0) {
-            for (uint32_t t0 = 0; t0 < vis; t0 += 64) {
-                const uint32_t t = t0 + lane;
-                float e = 0.0f;
-                if (t < vis) {
-                    const float s = score(t);
-                    if (s != -inf) e = expf(s - m);
-                }
-                for (int i = 0; i < 64; ++i) sum = sum + __shfl(e, i);     // adding +0 changes nothing
-            }
-        }
-        const float pinf_p = pinf ? 1.0f / (float)pinf : 0.0f;
-        // out = sum over tokens of P * V, features over lanes (up to 256)
-        float result[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (uint32_t t0 = 0; t0 < vis; t0 += 64) {
-            const uint32_t t = t0 + lane;
-            float pr = 0.0f;
-            if (t < vis) {
-                const float s = score(t);
-                if (pinf) pr = s == inf ? pinf_p : 0.0f;
-                else if (s != -inf) pr = expf(s - m) / sum;
-            }
-            __syncthreads();
-            pbuf[lane] = daz_bf16(bf16_rne_sw(as_u32(pr)));
-            __syncthreads();
-            const uint32_t n = vis - t0 < 64 ? vis - t0 : 64;
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const uint32_t d = lane + 64 * c;
-                if (d >= a.D) continue;
-                for (uint32_t i = 0; i < n; ++i) {
-                    const uint32_t tt = t0 + i;
-                    const uint8_t* vr = vb + (uint64_t)(tt >> 4) * a.d_tiles * kTileBytes + (tt & 15u) * kRowBytes;
-                    result[c] = result[c] + pbuf[i] * element(vr, d);             // products are exact
-                }
-            }
-        }
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint32_t d = lane + 64 * c;
-            if (d >= a.D) continue;
-            float val = result[c];
-            if (val == 0.0f) val = 0.0f;
-            store(d, bf16_rne_sw(as_u32(val)));
-        }
-      }
     }
 }
 
@@ -1216,19 +1240,16 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
         }
         record_launch("sdpa_mfma", (mode == 3 ? (row_tiles + 3) / 4 : row_tiles) * (mode == 1 || mode == 3 ? g.Hq : (g.Hq + 3) / 4) * gz, 256,
                       (uint64_t)g.planes * g.Hq * g.R);
-        g.guarded = 1;
+        IOMX_HIP(hipGetLastError());
+        return IOMX_OK;
     }
-    // one grid row per (plane, KV head) pair: when it only has to look at the flags it is
-    // gone in a few microseconds
+    // the reference-order kernel: one grid row per (plane, KV head) pair
     const uint64_t pairs = (uint64_t)g.planes * g.Hkv, per_pair = (uint64_t)g.grouping * g.R;
     if (pairs > 0x7FFFFFFFull || per_pair > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
     const uint32_t gy = (uint32_t)(pairs < 65535 ? pairs : 65535);
-    uint64_t gx = matrix_cores ? (8192 + gy - 1) / gy : per_pair;     // guarded: a modest grid
-    if (gx > per_pair) gx = per_pair;
-    if (gx > 65535) gx = 65535;
-    const dim3 rows_grid((uint32_t)gx, gy);
+    const dim3 rows_grid((uint32_t)(per_pair < 65535 ? per_pair : 65535), gy);
     hipLaunchKernelGGL(sdpa_rows_kernel, rows_grid, dim3(64), 0, st, g);
-    if (!matrix_cores) record_launch("sdpa_rows", rows_grid.x * rows_grid.y, 64, pairs * per_pair);
+    record_launch("sdpa_rows", rows_grid.x * rows_grid.y, 64, pairs * per_pair);
     IOMX_HIP(hipGetLastError());
     return IOMX_OK;
 }
