@@ -442,16 +442,15 @@ __global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const Line
 // 16x16 tiles (1 KiB, contiguous in memory) that feeds one MFMA operand; a stage
 // holds 16 row-tile and 16 output-tile fragments per 32 inner elements.  Fragments
 // go from global memory to LDS with the direct loader (global_load_lds, 16 bytes a
-// lane, no registers) into the other half of a double buffer while the matrix
-// cores work on this half, so every operand crosses L2->CU once per workgroup
-// instead of once per wave.
+// lane, no registers) into a ring of stage buffers, several stages ahead of the
+// matrix cores, so every operand crosses L2->CU once per workgroup instead of once
+// per wave.
 //
 // The direct loader puts lane i's 16 bytes at fragment + 16*i, so a fragment lies in
 // LDS as it lies in memory.  ds_read_b128 serves the lanes {0-3, 12-15, 20-23, 24-27},
 // {4-7, 8-11, 16-19, 28-31} (and the same +32) together; with lane l reading row l%16,
 // inner elements 8*(l/16).., of the plain tiled fragment each such group touches 16
 // different 16-byte bank groups, so the operand reads are conflict-free as stored.
-
 
 // blockIdx.x -> (row block, output block).  The blocks are put in one sequence: panels of
 // eight row blocks, inside a panel output block by output block; XCD id % 8 takes the id/8-th
@@ -535,77 +534,55 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     // reader role: position of the lane's eight inner elements inside a fragment
     const uint32_t rd_off = (kg >> 1) * kTileBytes + l16 * kRowBytes + (kg & 1u) * 16;
     const uint32_t stages = a.I / 32;
-    // A ring of DEPTH stage buffers (one stage = 32 inner elements; four for the large
-    // tile, five for the small one whose stages are half as long).  In the middle of
-    // stage st every wave waits for its own loads of stage st+1 and meets the others
-    // at the barrier: from there on stage st+1 is complete in LDS and nobody reads
-    // stage st-1 any more, so the second half of the stage (a) requests stage st+DEPTH-1
-    // into the buffer of st-1, direct loads between the groups of four MFMAs -- a direct load
-    // holds its wave at issue until the memory pipeline takes it, and the matrix
-    // instructions issued before it keep the matrix core busy meanwhile -- and (b)
-    // already reads the first operands of stage st+1, so the matrix core does not
-    // drain at the stage boundary.
+    // A ring of DEPTH stage buffers (one stage = 32 inner elements; four for the large tile,
+    // five for the small one whose stages are half as long) and two register sets of operand
+    // fragments.  At the top of stage st every wave waits for its own loads of stage st+1 and
+    // meets the others at the barrier: from there on stage st+1 is complete in LDS.  During the
+    // stage the MFMAs run on the register set of stage st while the other set is read from the
+    // buffer of stage st+1, one row fragment per step -- the matrix core never waits for LDS at a
+    // stage boundary -- and the second half of the steps requests stage st+DEPTH-1 with direct
+    // loads between the MFMA groups (a direct load holds its wave at issue until the memory
+    // pipeline takes it; the MFMAs issued before it keep the matrix core busy meanwhile) into a
+    // buffer whose stage everyone has long read into registers.
     const uint32_t last = stages - 1;
 #pragma unroll
     for (uint32_t d = 0; d < DEPTH - 1; ++d) issue(d < stages ? d : last, d);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * LPS) : "memory");
     __builtin_amdgcn_s_barrier();
-    bf16x8_t wf[2][WN], xf[4];
+    static_assert(WN <= WM, "one output fragment read per step");
+    bf16x8_t wf[2][WN], xf[2][WM];
     auto rd = [&](uint32_t ring, uint32_t frag) {
         return __builtin_bit_cast(bf16x8_t,
                 *reinterpret_cast<const u32x4*>(lds + ring * kStageBytes + rd_off + frag * kFrag));
     };
 #pragma unroll
     for (int n = 0; n < WN; ++n) wf[0][n] = rd(0, BM + wn * WN + n);
-    xf[0] = rd(0, wm * WM);
-    xf[1] = rd(0, wm * WM + 1);
-    // one stage = WM steps (one row fragment against the WN output fragments);
-    // P = parity of the stage (which half of wf holds its output fragments)
+#pragma unroll
+    for (int m = 0; m < WM; ++m) xf[0][m] = rd(0, wm * WM + m);
+    // P = parity of the stage (which register set holds its fragments)
     auto stage = [&](auto parity, uint32_t st) {
         constexpr int P = decltype(parity)::value;
-        // ring positions of this stage, of the next one and of the one requested now (which
-        // takes the buffer of the stage before this one)
-        const uint32_t ring = st % DEPTH, ring1 = (st + 1) % DEPTH, ring3 = (st + DEPTH - 1) % DEPTH;
+        // ring positions of the next stage and of the one requested now
+        const uint32_t ring1 = (st + 1) % DEPTH, ring3 = (st + DEPTH - 1) % DEPTH;
         const uint64_t gnext = (uint64_t)(st + DEPTH - 1 < stages ? st + DEPTH - 1 : last) * kFrag;
-#pragma unroll
-        for (int step = 0; step < HALF; ++step) {
-            xf[(step + 2) & 3] = rd(ring, wm * WM + step + 2);          // step + 2 < WM in this half
-#pragma unroll
-            for (int n = 0; n < WN; ++n)
-                acc[step][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[P][n], xf[step & 3], acc[step][n], 0, 0, 0);
-        }
-#pragma unroll
-        for (int step = 0; step < HALF; ++step) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, WN, 0);
-        }
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 3) * LPS) : "memory");
         __builtin_amdgcn_s_barrier();
 #pragma unroll
-        for (int step = HALF; step < WM; ++step) {
-            if (step + 2 < WM) xf[(step + 2) & 3] = rd(ring, wm * WM + step + 2);
-            else xf[(step + 2) & 3] = rd(ring1, wm * WM + step + 2 - WM);
-            if (step == HALF + 1) {
-#pragma unroll
-                for (int n = 0; n < WN; ++n) wf[P ^ 1][n] = rd(ring1, BM + wn * WN + n);
-            }
+        for (int step = 0; step < WM; ++step) {
+            if (step < WN) wf[P ^ 1][step] = rd(ring1, BM + wn * WN + step);
+            xf[P ^ 1][step] = rd(ring1, wm * WM + step);
 #pragma unroll
             for (int n = 0; n < WN; ++n)
-                acc[step][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[P][n], xf[step & 3], acc[step][n], 0, 0, 0);
+                acc[step][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[P][n], xf[P][step], acc[step][n], 0, 0, 0);
+            if (step >= HALF) {
 #pragma unroll
-            for (int i = 0; i < LPS / HALF; ++i) {
-                const int j = (step - HALF) * (LPS / HALF) + i;
-                const uint32_t frag = j < 2 ? wave + NW * j : BM + wave + NW * (j - 2);
-                __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + gnext),
-                                                 (lptr_t)(lds + ring3 * kStageBytes + frag * kFrag), 16, 0, 0);
+                for (int i = 0; i < LPS / HALF; ++i) {
+                    const int j = (step - HALF) * (LPS / HALF) + i;
+                    const uint32_t frag = j < 2 ? wave + NW * j : BM + wave + NW * (j - 2);
+                    __builtin_amdgcn_global_load_lds((gptr_t)(src[j] + gnext),
+                                                     (lptr_t)(lds + ring3 * kStageBytes + frag * kFrag), 16, 0, 0);
+                }
             }
-        }
-#pragma unroll
-        for (int step = HALF; step < WM; ++step) {
-            if (step == HALF + 1) __builtin_amdgcn_sched_group_barrier(0x100, WN + 1, 0);
-            else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, WN, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, LPS / HALF, 0);
         }
     };
     uint32_t st = 0;
