@@ -293,7 +293,11 @@ int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const 
  * iomx_sdpa_workspace is the pure requirement query (sdpa_workspace_requirements):
  * the bytes and alignment of caller workspace iomx_launch_sdpa needs for these
  * operands.  Requests whose rows fit one 16-row tile per KV head ((Hq/Hkv)*R <= 16, a
- * decode step) and heads wider than 128 need none (0 bytes, alignment 1); every other
+ * decode step) and heads wider than 128 need none (0 bytes, alignment 1) -- except a
+ * decode step of few sequences against a long prefix (2048 tokens or more, fewer than
+ * 128 planes x KV heads), whose token groups are shared out over several workgroups per
+ * KV head: that one needs 32 + 4*D bytes per plane, KV head, share and tile row for the
+ * shares' statistics and partial sums (256-byte aligned, no initialisation); every other
  * request needs the packed V fragments and flushed K tiles of the visible prefix and
  * one flag word per plane, KV head and pack share (256-byte aligned, no
  * initialisation).  path 0: the decode kernel (one launch: scores on the matrix cores,

@@ -36,7 +36,9 @@ struct SdpaArgs {
     uint32_t Hq, Hkv, grouping, R, C, D, a, L;
     uint32_t d_tiles, out_tile_cols, kv_tile_rows;
     uint32_t planes, groups;    // leading planes; 32-token groups of the prefix
-    uint32_t plane0;            // sdpa_mfma: first plane of this launch
+    uint32_t plane0;            // first plane of this launch
+    float* decode_stats;        // sdpa_decode in shares: [pair][share][row][8] statistics
+    float* decode_sums;         // ... and [pair][share][row][D] partial output sums
     uint8_t* packed_v;          // [plane][kv head][group][d tile] fragments of 1 KiB
     uint8_t* packed_k;          // [plane][kv head][token tile][d tile] flushed tiles (null: not packed)
     uint32_t* flags;            // [plane][kv head][pack split]: nonzero = that part of the V prefix
@@ -688,7 +690,14 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 // the probabilities of a group broadcast from LDS -- so nothing is packed or
 // transposed, no workspace is used, and a token a row must not see is left out of that
 // row's sum by a select (an infinite V there cannot reach it).
-template <int DT16>
+// PHASE 0: the whole step in one launch.  A long prefix of few sequences leaves most CUs idle
+// that way, so the token groups can also be shared out over several workgroups per KV head
+// (grid z), in two launches that keep the arithmetic of the one: PHASE 1 forms the statistics of
+// a share of the groups and leaves them in the workspace; PHASE 2 joins the statistics of all
+// shares (every workgroup in the same order, so all hold the same values), forms the
+// probabilities of its share and leaves its partial output sums; sdpa_decode_join_kernel adds the
+// partial sums in share order and stores the rows.
+template <int DT16, int PHASE>
 __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a) {
     constexpr int D32 = (DT16 + 1) / 2;
     constexpr int NW = 8;
@@ -710,6 +719,11 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
     const uint32_t vis = row_ok ? (reach < a.L ? reach : a.L) : 0;
     const uint32_t vis_max = reach_max < a.L ? reach_max : a.L;
     const uint32_t groups = (vis_max + 31) / 32;
+    // this workgroup's share of the groups: [g_lo, g_hi)
+    const uint32_t shares = PHASE == 0 ? 1 : gridDim.z, share = PHASE == 0 ? 0 : blockIdx.z;
+    const uint32_t per_share = (groups + shares - 1) / shares;
+    const uint32_t g_lo = share * per_share < groups ? share * per_share : groups;
+    const uint32_t g_hi = g_lo + per_share < groups ? g_lo + per_share : groups;
     const uint32_t c0 = (kg & 1u) * 8u;
     const float inf = __builtin_inff();
     // one plane per grid row, as in sdpa_mfma
@@ -787,18 +801,19 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         // group g has been multiplied, so PD groups per wave are in flight -- one wave's chain of
         // dependent loads is what a long prefix costs here
         KGroup kr[PD];
+        if (PHASE != 2) {
 #pragma unroll
         for (int slot = 0; slot < PD; ++slot)
-            if (wave + slot * NW < groups) load_k(wave + slot * NW, kr[slot]);
+            if (g_lo + wave + slot * NW < g_hi) load_k(g_lo + wave + slot * NW, kr[slot]);
 #pragma unroll 1
-        for (uint32_t g0 = wave; g0 < groups; g0 += PD * NW) {
+        for (uint32_t g0 = g_lo + wave; g0 < g_hi; g0 += PD * NW) {
 #pragma unroll
           for (int slot = 0; slot < PD; ++slot) {
             const uint32_t g = g0 + slot * NW;
-            if (g >= groups) break;                                   // uniform
+            if (g >= g_hi) break;                                     // uniform
             f32x4_t s[2];
             scores(kr[slot], s);
-            if (g + PD * NW < groups) load_k(g + PD * NW, kr[slot]);
+            if (g + PD * NW < g_hi) load_k(g + PD * NW, kr[slot]);
             float local = -inf;
 #pragma unroll
             for (int half = 0; half < 2; ++half)
@@ -841,6 +856,27 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         for (int w = 0; w < NW; ++w)
             st.merge(wave_stats[w][l16][0], wave_stats[w][l16][1], as_u32(wave_stats[w][l16][2]),
                      wave_stats[w][l16][3] != 0.0f, wave_stats[w][l16][4] != 0.0f);
+        }
+        // the statistics of a share: [pair][share][row][8] floats of the workspace
+        float* share_stats = a.decode_stats + (((uint64_t)p * a.Hkv + hkv) * shares) * 16 * 8;
+        if (PHASE == 1) {
+            if (threadIdx.x < 16) {
+                float* dst = share_stats + ((uint64_t)share * 16 + l16) * 8;
+                dst[0] = st.m;
+                dst[1] = st.sum;
+                dst[2] = as_f32(st.pinf);
+                dst[3] = st.nan ? 1.0f : 0.0f;
+                dst[4] = st.finite ? 1.0f : 0.0f;
+            }
+            return;
+        }
+        if (PHASE == 2) {
+            st = RowStats{-inf, 0.0f, 0u, false, false};
+            for (uint32_t sh = 0; sh < shares; ++sh) {
+                const float* src = share_stats + ((uint64_t)sh * 16 + l16) * 8;
+                st.merge(src[0], src[1], as_u32(src[2]), src[3] != 0.0f, src[4] != 0.0f);
+            }
+        }
         const bool nan_row = st.nan || (st.pinf == 0 && !st.finite);
         const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
         const float inv_sum = 1.0f / st.sum;
@@ -852,6 +888,9 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         // must not see is left out of that row's sum by a select.
         const uint32_t vis_min = a.a + 1 < a.L ? a.a + 1 : a.L;          // what row 0 sees: the least
         const uint32_t full_groups = vis_min / 32;
+        // of this share: the fully visible groups end at full_hi, the others start at tail_lo
+        const uint32_t full_hi = full_groups < g_hi ? full_groups : g_hi;
+        const uint32_t tail_lo = full_groups > g_lo ? full_groups : g_lo;
         struct VFrag { u32x4 w[DT16]; };
         auto load_vf = [&](uint32_t g, VFrag& vf) {
 #pragma unroll
@@ -895,24 +934,24 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             VFrag vr[PD];
 #pragma unroll
             for (int slot = 0; slot < PD; ++slot)
-                if (wave + slot * NW < full_groups) {
-                    load_k(wave + slot * NW, kr[slot]);
-                    load_vf(wave + slot * NW, vr[slot]);
+                if (g_lo + wave + slot * NW < full_hi) {
+                    load_k(g_lo + wave + slot * NW, kr[slot]);
+                    load_vf(g_lo + wave + slot * NW, vr[slot]);
                 }
 #pragma unroll 1
-            for (uint32_t g0 = wave; g0 < full_groups; g0 += PD * NW) {
+            for (uint32_t g0 = g_lo + wave; g0 < full_hi; g0 += PD * NW) {
 #pragma unroll
                 for (int slot = 0; slot < PD; ++slot) {
                     const uint32_t g = g0 + slot * NW;
-                    if (g >= full_groups) break;                              // uniform
+                    if (g >= full_hi) break;                                  // uniform
                     f32x4_t s[2];
                     scores(kr[slot], s);
-                    if (g + PD * NW < full_groups) load_k(g + PD * NW, kr[slot]);
+                    if (g + PD * NW < full_hi) load_k(g + PD * NW, kr[slot]);
                     const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, probabilities(g, s));
 #pragma unroll
                     for (int dt = 0; dt < DT16; ++dt)
                         om[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vr[slot].w[dt]), pf, om[dt], 0, 0, 0);
-                    if (g + PD * NW < full_groups) load_vf(g + PD * NW, vr[slot]);
+                    if (g + PD * NW < full_hi) load_vf(g + PD * NW, vr[slot]);
                 }
             }
         }
@@ -921,9 +960,9 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         for (int r = 0; r < 16; ++r)
 #pragma unroll
             for (int c = 0; c < DL; ++c) o[r][c] = 0.0f;
-        // the one or two groups past the fully visible ones, each with the wave whose turn it is
+        // the one or two groups past the fully visible ones, one per wave
 #pragma unroll 1
-        for (uint32_t g = full_groups + (wave + NW - full_groups % NW) % NW; g < groups; g += NW) {
+        for (uint32_t g = tail_lo + wave; g < g_hi; g += NW) {
             KGroup kt;
             load_k(g, kt);
             f32x4_t s[2];
@@ -992,6 +1031,11 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             float sum = 0.0f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) sum += o_part[w][r][d];
+            if (PHASE == 2) {
+                // [pair][share][row][D] partial sums of the workspace
+                a.decode_sums[((((uint64_t)p * a.Hkv + hkv) * shares + share) * 16 + r) * a.D + d] = sum;
+                continue;
+            }
             if (sum == 0.0f) sum = 0.0f;                                   // -0 is stored as +0
             const uint32_t rr = r / a.grouping, hh = hkv * a.grouping + (r - rr * a.grouping);
             const float* ws = &wave_stats[0][r][0];
@@ -1011,6 +1055,37 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             *reinterpret_cast<uint16_t*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) =
                     (uint16_t)(nan_out ? 0x7FC0u : bf16_rne_sw(as_u32(sum)));
         }
+    }
+}
+
+// The partial sums of the shares of one KV head, added in share order, and the rows' classes
+// from the joined statistics: the rows of sdpa_decode in two launches.
+__global__ __launch_bounds__(512) void sdpa_decode_join_kernel(const SdpaArgs a, uint32_t shares) {
+    const uint32_t hkv = blockIdx.x, p = a.plane0 + blockIdx.y;
+    const uint32_t nrows = a.grouping * a.R;
+    const uint64_t pair = (uint64_t)p * a.Hkv + hkv;
+    uint64_t plane[4];
+    walk_planes(a.walk, p, plane);
+    for (uint32_t idx = threadIdx.x; idx < nrows * a.D; idx += 512) {
+        const uint32_t r = idx / a.D, d = idx - r * a.D;
+        float sum = 0.0f;
+        bool nan = false, finite = false;
+        uint32_t pinf = 0;
+        for (uint32_t sh = 0; sh < shares; ++sh) {
+            sum += a.decode_sums[((pair * shares + sh) * 16 + r) * a.D + d];
+            const float* st = a.decode_stats + ((pair * shares + sh) * 16 + r) * 8;
+            nan = nan || st[3] != 0.0f;
+            finite = finite || st[4] != 0.0f;
+            pinf += as_u32(st[2]);
+        }
+        if (sum == 0.0f) sum = 0.0f;                                       // -0 is stored as +0
+        const bool nan_out = nan || (pinf == 0 && !finite);
+        const uint32_t rr = r / a.grouping, hh = hkv * a.grouping + (r - rr * a.grouping);
+        const uint32_t col = hh * a.D + d;
+        uint8_t* ob = a.out + plane[3] * a.out_plane_bytes
+                + (uint64_t)(rr >> 4) * a.out_tile_cols * kTileBytes + (rr & 15u) * kRowBytes;
+        *reinterpret_cast<uint16_t*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) =
+                (uint16_t)(nan_out ? 0x7FC0u : bf16_rne_sw(as_u32(sum)));
     }
 }
 
@@ -1074,6 +1149,26 @@ constexpr uint64_t kMaxMfmaHeadDim = 128;
 // all rows of the query heads of one KV head fit one 16-row tile: the decode kernel
 bool sdpa_few_rows(const SdpaShape& s) { return (s.Hq / s.Hkv) * s.R <= kTile && s.D <= kMaxMfmaHeadDim; }
 
+// Workgroups that share the token groups of one KV head in a decode step (sdpa_decode): one,
+// unless the prefix is long and planes * Hkv workgroups would leave most CUs idle; then enough
+// for about one workgroup per CU, each with at least 16 groups (two per wave).
+uint32_t sdpa_decode_shares(const SdpaShape& s, uint64_t a, uint64_t L) {
+    const uint64_t reach = a + s.R, vis = reach < L ? reach : L;
+    const uint64_t groups = (vis + 31) / 32, heads = s.planes * s.Hkv;
+    if (groups < 64 || heads >= 128) return 1;
+    uint64_t shares = 256 / heads;
+    if (shares > groups / 16) shares = groups / 16;
+    if (shares > 64) shares = 64;
+    return (uint32_t)(shares > 1 ? shares : 1);
+}
+
+// Workspace of a decode step in shares: [pair][share][16 rows][8] statistics, then
+// [pair][share][16 rows][D] partial sums, binary32.
+uint64_t sdpa_decode_stats_floats(const SdpaShape& s, uint32_t shares) { return s.planes * s.Hkv * shares * 16 * 8; }
+uint64_t sdpa_decode_workspace(const SdpaShape& s, uint32_t shares) {
+    return (sdpa_decode_stats_floats(s, shares) + s.planes * s.Hkv * shares * 16 * s.D) * 4;
+}
+
 // Workgroups that share the packing of one KV head: enough of them to occupy the
 // chip when planes * Hkv alone would not.
 uint32_t sdpa_pack_splits(const SdpaShape& s, uint64_t L) {
@@ -1117,6 +1212,10 @@ extern "C" int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_vie
     IOMX_TRY(sdpa_shape(q, k, v, out, a, L, &s));
     if (dtype != IOMX_DT_BF16) return IOMX_ERR_UNSUPPORTED;
     *alignment = 256;
+    if (s.D <= kMaxMfmaHeadDim && sdpa_few_rows(s)) {
+        const uint32_t shares = sdpa_decode_shares(s, a, L);
+        if (shares > 1) { *bytes = sdpa_decode_workspace(s, shares); return IOMX_OK; }
+    }
     if (s.D > kMaxMfmaHeadDim || sdpa_few_rows(s)) { *bytes = 0; *alignment = 1; return IOMX_OK; }
     uint64_t header, region;
     return sdpa_layout(s, L, &header, &region, bytes);
@@ -1174,9 +1273,27 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
     const uint32_t gz = g.planes < 65535u ? g.planes : 65535u;
 
     if (path == 0 && sdpa_few_rows(s) && s.Hkv <= 0x7FFFFFFFull) {
+        const uint32_t shares = sdpa_decode_shares(s, a, L);
+        if (shares > 1) {
+            // (shares > 1 implies fewer than 128 planes: one launch of each phase)
+            if (!workspace || workspace_bytes < sdpa_decode_workspace(s, shares)
+                || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+                return IOMX_ERR_INVALID;
+            g.decode_stats = static_cast<float*>(workspace);
+            g.decode_sums = g.decode_stats + sdpa_decode_stats_floats(s, shares);
+        }
         for (g.plane0 = 0; g.plane0 < g.planes; g.plane0 += 65535u) {
-            const dim3 grid(g.Hkv, g.planes - g.plane0 < 65535u ? g.planes - g.plane0 : 65535u);
-#define IOMX_SDPA_DECODE(N) case N: hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N>), grid, dim3(512), 0, st, g); break;
+            const dim3 grid(g.Hkv, g.planes - g.plane0 < 65535u ? g.planes - g.plane0 : 65535u, shares);
+#define IOMX_SDPA_DECODE(N) \
+    case N: \
+        if (shares == 1) { \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0>), grid, dim3(512), 0, st, g); \
+        } else { \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 1>), grid, dim3(512), 0, st, g); \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 2>), grid, dim3(512), 0, st, g); \
+            hipLaunchKernelGGL(sdpa_decode_join_kernel, dim3(grid.x, grid.y), dim3(512), 0, st, g, shares); \
+        } \
+        break;
             switch (g.d_tiles) {
                 IOMX_SDPA_DECODE(1) IOMX_SDPA_DECODE(2) IOMX_SDPA_DECODE(3) IOMX_SDPA_DECODE(4)
                 IOMX_SDPA_DECODE(5) IOMX_SDPA_DECODE(6) IOMX_SDPA_DECODE(7)
@@ -1184,7 +1301,7 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
             }
 #undef IOMX_SDPA_DECODE
         }
-        record_launch("sdpa_decode", g.Hkv * gz, 512, (uint64_t)g.planes * g.Hq * g.R);
+        record_launch("sdpa_decode", g.Hkv * gz * shares, 512, (uint64_t)g.planes * g.Hq * g.R);
         IOMX_HIP(hipGetLastError());
         return IOMX_OK;
     }

@@ -215,6 +215,57 @@ def test_more_planes_than_one_grid_holds(R, kernel):
     assert np.array_equal(got, want[pick])
 
 
+LONG_DECODE = [((), 8, 2, 1, 64, 2200, 2199, 2200), ((3,), 16, 2, 2, 128, 2100, 2050, 2052),
+               ((), 4, 4, 3, 32, 2500, 2400, 2403), ((2,), 8, 1, 1, 64, 4100, 4095, 4096)]
+
+
+@pytest.mark.parametrize("spec", LONG_DECODE, ids=[str(i) for i in range(len(LONG_DECODE))])
+def test_decode_step_against_a_long_prefix_in_shares(spec):
+    """Few sequences against a prefix of 64 or more token groups: several workgroups per KV head
+    share the groups (statistics, then partial sums, then the join).  Against the oracle with the
+    fixture rule and the float64 budget; one case per edge: two rows per head on the diagonal,
+    three leading planes, one KV head, a prefix that is a multiple of the share size."""
+    lead, Hq, Hkv, R, D, C, a, L = spec
+    case = random_case(81 + R, lead, Hq, Hkv, R, D, C, a, L)
+    q, k, v, o = device_operands(case)
+    rc, nbytes, align = iomx.sdpa_workspace(q.view(), k.view(), v.view(), o.view(), a, L)
+    assert rc == 0 and nbytes > 0 and align == 256
+    for t in (q, k, v, o):
+        t.free()
+    got = run(case, 0, fill=0xFF, expect_kernel="sdpa_decode")
+    want = oracle(case)
+    assert len(close_to_oracle(got, want)) <= 0.001 * got.size
+    ref64, budget = float64_attention(case)
+    g = datagen.bf16_to_f32(got.reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    assert np.all(np.abs(g - ref64) <= budget)
+
+
+def test_decode_in_shares_with_special_scores_and_values():
+    """Special scores that fall into different shares (a +infinity score in the first and the last
+    share, a NaN query row, a row of -infinity scores), an infinite V at a token only the second
+    row of each head may see, and NaN / infinity in the cache tail."""
+    Hq, Hkv, R, D, C, a, L = 8, 2, 2, 64, 2300, 2200, 2202
+    case = random_case(91, (2,), Hq, Hkv, R, D, C, a, L)
+    q = np.array(case["q"], np.uint16).reshape(2, Hq, R, D).copy()
+    k = np.array(case["k"], np.uint16).reshape(2, Hkv, C, D).copy()
+    v = np.array(case["v"], np.uint16).reshape(2, Hkv, C, D).copy()
+    k[0, 0, 3, 5] = 0x7F80            # +inf or -inf scores by the sign of q, first share
+    k[0, 0, 2190, 5] = 0x7F80         # ... and last share
+    q[1, 2, 1, 9] = 0x7FC0            # a NaN row
+    k[1, 1, :, :] = 0x0000
+    k[1, 1, :L, 0] = 0xFF80           # every visible score of KV head 1 of plane 1 is -inf or +inf or NaN
+    v[0, 1, 2201, 7] = 0x7F80         # visible to row 1 (a + 1 + 1 = 2202 tokens) but not to row 0
+    k[:, :, L:, :] = 0x7FC0
+    v[:, :, L:, :] = 0xFF80
+    special = dict(case, q=q.reshape(-1).tolist(), k=k.reshape(-1).tolist(), v=v.reshape(-1).tolist())
+    got = run(special, 0, expect_kernel="sdpa_decode")
+    want = oracle(special)
+    assert close_to_oracle(got, want) == []
+    g = got.reshape(2, R, Hq, D)
+    assert np.all(g[0, 1, 4:, 7] == 0x7F80) and np.all((g[0, 0, 4:, :] & 0x7F80) != 0x7F80)
+    assert np.all((g[1, 1, 2] & 0x7FFF) > 0x7F80)
+
+
 def test_incremental_rows_equal_the_prefill():
     case = random_case(9, (), 4, 2, 7, 8, 7, 0, 7)
     full = run(case, 0)
@@ -313,6 +364,11 @@ def test_backend_prefill_then_decode_and_rejections(devices):
                 q=np.array(case["q"], np.uint16).reshape(2, 8, 24, 64)[:, :, :1].reshape(-1).tolist())
     outs = [backend_run(dev, step) for dev in (cpu, gpu)]
     assert close_to_oracle(outs[1][1], outs[0][1]) == []
+    # a decode step against a long prefix: the backend asks for and passes the workspace of the shares
+    far = random_case(93, (), 8, 2, 1, 64, 2200, 2199, 2200)
+    outs = [backend_run(dev, far) for dev in (cpu, gpu)]
+    assert outs[0][0] > 0 and outs[1][0] > 0
+    assert len(close_to_oracle(outs[1][1], outs[0][1])) <= 0.001 * outs[0][1].size
     # admission and capability answers are the reference's own
     for bad in (dict(case, L=0), dict(case, L=49), dict(case, a=48), dict(case, a=30)):
         assert backend_run(cpu, bad)[0] == backend_run(gpu, bad)[0] < 0
