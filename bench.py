@@ -406,12 +406,12 @@ def wl_decoder_layer(timer, steps, warmup):
     projections (head planar), rope on q and k, cache append of k and v, attention, output
     projection, residual add, rmsnorm, gate / up projections, silu * up, down projection,
     residual add.  Prefill: 8 sequences, and one sequence, of 512 tokens into an empty
-    512-token cache; decode: one token for 64 sequences at position 511.  Each operation is
-    also timed alone."""
+    512-token cache; decode: one token for 64 sequences, and for one sequence, at position 511.
+    Each operation is also timed alone."""
     out = []
     H, Hq, Hkv, D, FF, C = 2048, 32, 4, 64, 5632, 512
     st = timer.stream
-    for name, B, S, a in (("prefill", 8, 512, 0), ("prefill", 1, 512, 0), ("decode", 64, 1, 511)):
+    for name, B, S, a in (("prefill", 8, 512, 0), ("prefill", 1, 512, 0), ("decode", 64, 1, 511), ("decode", 1, 1, 511)):
         L = a + S
         x = device_tensor(BF16, (B, S, H), "normal", 121)
         w_n1, w_n2 = (device_tensor(BF16, (1, H), "uniform_half_3half", s) for s in (122, 123))

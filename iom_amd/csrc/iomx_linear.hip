@@ -873,7 +873,7 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                     while (nt > 1 && (uint64_t)((o_tiles + nt - 1) / nt) * row_tiles < 256) nt /= 2;
                 } else {
                     mt = row_tiles == 1 ? 1 : row_tiles == 2 ? 2 : 4;
-                    nt = mt == 1 ? 2 : 1;
+                    nt = mt == 1 && (o_tiles + 1) / 2 >= 256 ? 2 : 1;      // a workgroup for every CU first
                 }
                 const dim3 grid((o_tiles + nt - 1) / nt, (row_tiles + mt - 1) / mt);
 #define IOMX_SPLITK(M, N) \
