@@ -633,14 +633,20 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
 // request the stage DEPTH-1 ahead into the freed buffer, read four fragments, four MFMAs.
 // The fragments of a wave are 4 KiB per 4 MFMAs: the LDS ports, not the matrix cores,
 // bound this kernel (at about half the matrix rate).
-template <int DEPTH>
-__global__ __launch_bounds__(256)
+//
+// KS > 1: when even these blocks are fewer than the CUs, KS groups of four waves each walk a
+// KS-th of the inner axis with a ring of their own, and the partial sums meet in LDS at the end
+// (in group order; the sum is then not the single sequence of the other kernels).
+template <int DEPTH, int KS>
+__global__ __launch_bounds__(256 * KS)
 void linear_mfma_lds64_bf16_kernel(const LinearArgs a) {
     constexpr uint32_t BM = 4, BN = 4, NW = 4, LPS = 2;
     constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
     constexpr uint32_t kStageBytes = (BM + BN) * kFrag;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[DEPTH * kStageBytes];
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    __shared__ __attribute__((aligned(16))) uint8_t all_rings[KS * DEPTH * kStageBytes];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t slice = (threadIdx.x >> 6) / NW, wave = (threadIdx.x >> 6) % NW;   // group and role in it
+    uint8_t* lds = all_rings + slice * DEPTH * kStageBytes;
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     const uint32_t total_rows = a.planes * a.R;
     uint32_t bx, by;
@@ -666,9 +672,13 @@ void linear_mfma_lds64_bf16_kernel(const LinearArgs a) {
         if (o >= a.O) o = 0;
         src_w = a.w + (uint64_t)(o >> 4) * a.w_tile_cols * kTileBytes + (o & 15u) * kRowBytes + ld_off;
     }
-    const uint32_t stages = a.I / 32, last = stages - 1;
+    // this group's stages: [s_lo, s_hi) of the I / 32; every group runs `per` iterations
+    const uint32_t stages = a.I / 32, per = (stages + KS - 1) / KS;
+    const uint32_t s_lo = slice * per < stages ? slice * per : stages;
+    const uint32_t s_hi = s_lo + per < stages ? s_lo + per : stages;
+    const uint32_t last = s_hi > s_lo ? s_hi - 1 : 0;
     auto issue = [&](uint32_t stage, uint32_t buf) {
-        const uint64_t goff = (uint64_t)(stage < stages ? stage : last) * kFrag;
+        const uint64_t goff = (uint64_t)(stage < s_hi ? stage : last) * kFrag;
         uint8_t* base = lds + buf * kStageBytes;
         __builtin_amdgcn_global_load_lds((gptr_t)(src_x + goff), (lptr_t)(base + wave * kFrag), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((gptr_t)(src_w + goff), (lptr_t)(base + (BM + wave) * kFrag), 16, 0, 0);
@@ -684,23 +694,40 @@ void linear_mfma_lds64_bf16_kernel(const LinearArgs a) {
                 *reinterpret_cast<const u32x4*>(lds + ring * kStageBytes + rd_off + frag * kFrag));
     };
 #pragma unroll
-    for (uint32_t d = 0; d < DEPTH - 1; ++d) issue(d, d);
+    for (uint32_t d = 0; d < DEPTH - 1; ++d) issue(s_lo + d, d);
     uint32_t ring = 0, free_ring = DEPTH - 1;
-    for (uint32_t st = 0; st < stages; ++st) {
+    for (uint32_t st = s_lo; st < s_lo + per; ++st) {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * LPS) : "memory");
         __builtin_amdgcn_s_barrier();
         issue(st + DEPTH - 1, free_ring);
-        const bf16x8_t x0 = rd(ring, wm * 2), x1 = rd(ring, wm * 2 + 1);
-        const bf16x8_t w0 = rd(ring, BM + wn * 2), w1 = rd(ring, BM + wn * 2 + 1);
-        acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0, acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x0, acc[0][1], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x1, acc[1][0], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1, acc[1][1], 0, 0, 0);
+        if (KS == 1 || st < s_hi) {                        // (the last group may have fewer stages)
+            const bf16x8_t x0 = rd(ring, wm * 2), x1 = rd(ring, wm * 2 + 1);
+            const bf16x8_t w0 = rd(ring, BM + wn * 2), w1 = rd(ring, BM + wn * 2 + 1);
+            acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x0, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x1, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1, acc[1][1], 0, 0, 0);
+        }
         free_ring = ring;
         ring = ring + 1 == DEPTH ? 0 : ring + 1;
     }
     // nothing may still be landing in LDS when the workgroup gives it back
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (KS > 1) {
+        // the groups' partial sums through the (now idle) rings: [group - 1][wave][tile][lane]
+        __syncthreads();
+        f32x4_t* part = reinterpret_cast<f32x4_t*>(all_rings);
+        if (slice > 0) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) part[(((slice - 1) * NW + wave) * 4 + t) * 64 + lane] = acc[t >> 1][t & 1];
+        }
+        __syncthreads();
+        if (slice > 0) return;
+#pragma unroll 1
+        for (uint32_t g = 0; g + 1 < KS; ++g)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[t >> 1][t & 1] += part[((g * NW + wave) * 4 + t) * 64 + lane];
+    }
 
     const uint32_t d_tiles = a.D >> 4;
 #pragma unroll
@@ -839,7 +866,14 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                     const dim3 grid((uint32_t)wgs);
                     if (tile == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4, 4>), grid, dim3(512), 0, st, b);
                     else if (tile == 8) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 5>), grid, dim3(256), 0, st, b);
-                    else hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4>), grid, dim3(256), 0, st, b);
+                    else {
+                        // fewer blocks than CUs: two or four groups of waves share the inner axis
+                        const uint32_t stages = a.I / 32;
+                        const uint32_t ks = path == 5 ? 1 : blocks <= 128 && stages >= 32 ? 4 : blocks <= 256 && stages >= 16 ? 2 : 1;
+                        if (ks == 4) hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4, 4>), grid, dim3(1024), 0, st, b);
+                        else if (ks == 2) hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4, 2>), grid, dim3(512), 0, st, b);
+                        else hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4, 1>), grid, dim3(256), 0, st, b);
+                    }
                     record_launch("linear_mfma_lds", grid.x, tile == 16 ? 512 : 256, (uint64_t)row_tiles * count);
                     return IOMX_OK;
                 };
