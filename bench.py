@@ -93,10 +93,17 @@ class Timer:
         self.stream = stream
         self.start, self.stop = iomx.Event(True), iomx.Event(True)
 
-    def run(self, launch, steps: int, warmup: int):
+    def run(self, launch, steps: int, warmup: int, warm_ms: float = 0.0):
+        """warm_ms: keep launching warm-up steps until that much wall time has passed (the
+        matrix-core kernels take some 20 ms of load to reach their steady clocks)."""
+        t_warm = time.perf_counter()
         for i in range(warmup):
             launch(i)
         self.stream.synchronize()
+        while (time.perf_counter() - t_warm) * 1e3 < warm_ms:
+            for i in range(max(warmup, 1)):
+                launch(i)
+            self.stream.synchronize()
         iomx.synchronize()
         t0 = time.perf_counter()
         self.start.record(self.stream)
@@ -340,7 +347,7 @@ def wl_linear(timer, steps, warmup):
         def launch(i):
             check(iomx.linear(x.view(), w.view(), o.view(), 0, S, False, 1, O, 0, timer.stream), "linear")
 
-        wall, ev = timer.run(launch, steps, warmup)
+        wall, ev = timer.run(launch, steps, warmup, warm_ms=30.0)
         flops = 2.0 * B * S * I * O
         r = report("linear_bf16_%s_[64,512,2048]x[%d,2048]" % (name, O), 2 * (B * S * I + O * I + B * S * O),
                    B * S * O, wall, ev, iomx.last_launch().kernel.decode())
@@ -386,7 +393,7 @@ def wl_sdpa(timer, steps, warmup):
         def launch(i):
             check(iomx.sdpa(qv, k.view(), v.view(), ov, a, L, ws, 0, timer.stream), "sdpa")
 
-        wall, ev = timer.run(launch, steps, warmup)
+        wall, ev = timer.run(launch, steps, warmup, warm_ms=30.0)
         visible = sum(min(L, a + r + 1) for r in range(R))
         flops = 4.0 * B * Hq * D * visible
         r = report("sdpa_bf16_%s_B%d_Hq32_Hkv4_R%d_L%d_D64" % (name, B, R, L),
@@ -451,7 +458,7 @@ def wl_decoder_layer(timer, steps, warmup):
             for label, op in ops:
                 check(op(), label)
 
-        wall, ev = timer.run(layer, steps, warmup)
+        wall, ev = timer.run(layer, steps, warmup, warm_ms=30.0)
         each = {}
         for label, op in ops:
             _, e = timer.run(lambda i: check(op(), label), steps, 1)
