@@ -93,9 +93,10 @@ class Timer:
         self.stream = stream
         self.start, self.stop = iomx.Event(True), iomx.Event(True)
 
-    def run(self, launch, steps: int, warmup: int, warm_ms: float = 0.0):
-        """warm_ms: keep launching warm-up steps until that much wall time has passed (the
-        matrix-core kernels take some 20 ms of load to reach their steady clocks)."""
+    def run(self, launch, steps: int, warmup: int, warm_ms: float = 20.0):
+        """After the `warmup` steps, warm-up steps go on until warm_ms of wall time have passed:
+        the clocks take some 20 ms of load to settle (2 % on the streaming kernels, 15-20 % on
+        the matrix-core ones, which ask for 30 ms)."""
         t_warm = time.perf_counter()
         for i in range(warmup):
             launch(i)
