@@ -86,6 +86,13 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
         float x[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) x[j] = as_f32(kNegInf);
+        if (k * 256u >= visible) {
+            // the whole 256-column chunk is past the visible limit (the same for every lane):
+            // nothing to load, to compare or, below, to exponentiate
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s[k][j] = x[j];
+            continue;
+        }
         if (col + 4 <= visible) {
             const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(srow + col));
             x[0] = as_f32(v.x) * a.scale; x[1] = as_f32(v.y) * a.scale;
@@ -125,20 +132,24 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
     } else {
         float part = 0.0f;
 #pragma unroll
-        for (int k = 0; k < K; ++k)
+        for (int k = 0; k < K; ++k) {
+            if (k * 256u >= visible) continue;            // uniform; stored as +0 below
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const float e = exp_nonpos(s[k][j] - m);  // 0 for masked and -inf scores
                 s[k][j] = e;
                 part = part + e;
             }
+        }
         // e * (1/sum) instead of e / sum: at most one binary32 unit apart, which a
         // BF16 result shows only at a rounding boundary
         const float inv_sum = 1.0f / wave_sum(part);
 #pragma unroll
-        for (int k = 0; k < K; ++k)
+        for (int k = 0; k < K; ++k) {
+            if (k * 256u >= visible) continue;
 #pragma unroll
             for (int j = 0; j < 4; ++j) s[k][j] = s[k][j] * inv_sum;
+        }
     }
 #pragma unroll
     for (int k = 0; k < K; ++k) {
@@ -146,11 +157,14 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
         if (col >= a.pcols32) continue;
         // elements at or beyond the visible limit are +0
         const uint32_t nvis = visible > col ? visible - col : 0u;
-        float pr[4];
+        uint32_t lo = 0, hi = 0;
+        if (k * 256u < visible) {                          // uniform
+            float pr[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) pr[j] = ((uint32_t)j < nvis) ? s[k][j] : 0.0f;
-        const uint32_t lo = pack_bf16(pr[0], pr[1]);
-        const uint32_t hi = pack_bf16(pr[2], pr[3]);
+            for (int j = 0; j < 4; ++j) pr[j] = ((uint32_t)j < nvis) ? s[k][j] : 0.0f;
+            lo = pack_bf16(pr[0], pr[1]);
+            hi = pack_bf16(pr[2], pr[3]);
+        }
         if (col + 4 <= a.pcols32) {
             __builtin_nontemporal_store(u32x2{lo, hi}, reinterpret_cast<u32x2*>(prow + col));
         } else {
