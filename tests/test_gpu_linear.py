@@ -265,3 +265,33 @@ def test_bf16_workgroup_tiled_kernels_on_short_and_odd_inner_extents(inner, path
     assert np.array_equal(d2.raw(), do.raw())          # same products in the same order
     for t in (dx, dw, do, d2):
         t.free()
+
+
+@pytest.mark.parametrize("inner", [544, 1056, 2048, 4128])
+def test_bf16_small_tiles_with_the_inner_axis_shared_by_groups_of_waves(inner):
+    """Few 64 x 64 blocks and a long inner axis: two or four groups of waves each take a part
+    of the stages (17, 33, 64 or 129 of them: parts of unequal length, a last part that is
+    shorter) and their partial sums meet in LDS.  300 rows over 2 planes with a window, 80
+    outputs in 5 heads; the contract's BF16 bound against float64, one-hot rows exactly, and
+    untouched padding."""
+    xd, wd, s, R, H, D = (2, 160, inner), (80, inner), 7, 150, 5, 16
+    xv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(xd)), 0, 1, 61 + inner)).reshape(xd)
+    wv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(wd)), 0, 0.2, 62 + inner)).reshape(wd)
+    xv[1, s + 3, :] = 0
+    xv[1, s + 3, inner - 1] = 0x3F80              # a one-hot row in the last stage of the last group
+    xv[0, s + 149, :] = 0
+    xv[0, s + 149, 0] = 0x3F80                    # ... and in the first stage of the first
+    dx, _ = pair(DT_BF16, xd, values=xv)
+    dw, _ = pair(DT_BF16, wd, values=wv)
+    od = (2, H, R, D)
+    do, ho = pair(DT_BF16, od, salt=63)
+    assert iomx.linear(dx.view(), dw.view(), do.view(), s, R, True, H, D, path=0) == 0
+    assert iomx.last_launch().kernel.decode() == "linear_mfma_lds"
+    got = do.view().to_host().transpose(0, 2, 1, 3).reshape(2, R, H * D)
+    for b in range(2):
+        assert bf16_bound(got[b], xv[b, s:s + R], wv).all()
+    assert np.array_equal(got[1, 3], wv[:, inner - 1]) and np.array_equal(got[0, 149], wv[:, 0])
+    mask = iomo.tile_plane(np.ones(od, np.uint16)) == 0
+    assert np.array_equal(do.raw()[mask], ho.storage[mask])
+    for t in (dx, dw, do):
+        t.free()
