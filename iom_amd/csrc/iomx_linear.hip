@@ -290,8 +290,10 @@ __global__ __launch_bounds__(256) void linear_mfma_bf16_kernel(const LinearArgs 
 // stream, and their partial sums meet in LDS (added in wave order, so the result
 // does not depend on timing).  When each row is the only row of its plane (one
 // token per sequence) a 128-byte line of x holds 32 useful bytes, so x costs MT x
-// 4 bytes of line traffic per weight byte-row it meets: the launch picks MT = 1 and
-// lets NT output tiles share each x fragment.
+// 4 bytes of line traffic per weight byte-row it meets: with one or two row tiles
+// the launch picks MT = 1 and lets NT output tiles share each x fragment; with more
+// row tiles and many output tiles, 2 x 2, 2 x 4 or 4 x 4 tiles per workgroup read
+// both operands less often from L2, which is what bounds those launches.
 template <int MT, int NT>
 __global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const LinearArgs a) {
     constexpr uint32_t kTileBytes = 512, kRowBytes = 32;
@@ -299,7 +301,12 @@ __global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const Line
     const uint32_t lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     const uint32_t total_rows = a.planes * a.R;
-    const uint32_t ot0 = blockIdx.x * NT, rt0 = blockIdx.y * MT;
+    // workgroup id % 8 is the XCD: the row blocks of one output block run next to each
+    // other on one XCD, so the weight rows they share come from that XCD's L2
+    const uint32_t in_xcd = blockIdx.x >> 3;
+    const uint32_t out_block = (in_xcd / a.row_blocks) * 8 + (blockIdx.x & 7u);
+    if (out_block >= a.out_blocks) return;
+    const uint32_t ot0 = out_block * NT, rt0 = (in_xcd % a.row_blocks) * MT;
     const uint8_t* xrow[MT];
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
@@ -892,7 +899,7 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                 } else {
                     IOMX_TRY(launch_part(0, o_tiles, bt));
                 }
-            } else if (path != 2 && row_tiles < 16 && o_tiles <= 0x7FFFFFFFu) {
+            } else if (path != 2 && row_tiles < 16 && o_tiles <= 0x3FFFFFu) {
                 // few rows (decode, last-row logits): one output tile per workgroup, the
                 // inner axis split over its waves
                 // rows that are alone in their plane (R == 1 of many planes) make x the
@@ -909,12 +916,27 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                     mt = row_tiles == 1 ? 1 : row_tiles == 2 ? 2 : 4;
                     nt = mt == 1 && (o_tiles + 1) / 2 >= 256 ? 2 : 1;      // a workgroup for every CU first
                 }
-                const dim3 grid((o_tiles + nt - 1) / nt, (row_tiles + mt - 1) / mt);
+                // two to four row tiles (a decode step of 17-64 sequences) against many
+                // outputs: larger workgroup tiles, where enough of them remain for the CUs
+                // (measured: 64 rows x [5632,2048] 18 -> 15 us, x [4096,4096] 30 -> 22 us,
+                // x [32000,2048] 97 -> 43 us)
+                if (row_tiles >= 3 && row_tiles <= 4) {
+                    if (o_tiles >= 640 && (uint64_t)o_tiles * a.I >= 2500000u) { mt = 4; nt = 4; }
+                    else if (o_tiles >= 352) { mt = 2; nt = 4; }
+                    else if (o_tiles >= 256) { mt = 2; nt = 2; }
+                } else if (row_tiles == 2 && o_tiles >= 1024) {
+                    mt = 2; nt = 4;
+                }
+                LinearArgs b = a;
+                b.row_blocks = (row_tiles + mt - 1) / mt;
+                b.out_blocks = (uint32_t)((o_tiles + nt - 1) / nt);
+                const dim3 grid((b.out_blocks + 7) / 8 * 8 * b.row_blocks);
 #define IOMX_SPLITK(M, N) \
-    if (mt == M && nt == N) hipLaunchKernelGGL((linear_mfma_splitk_bf16_kernel<M, N>), grid, dim3(256), 0, st, a)
+    if (mt == M && nt == N) hipLaunchKernelGGL((linear_mfma_splitk_bf16_kernel<M, N>), grid, dim3(256), 0, st, b)
                 IOMX_SPLITK(1, 1); IOMX_SPLITK(1, 2); IOMX_SPLITK(1, 4); IOMX_SPLITK(2, 1); IOMX_SPLITK(4, 1);
+                IOMX_SPLITK(2, 2); IOMX_SPLITK(2, 4); IOMX_SPLITK(4, 4);
 #undef IOMX_SPLITK
-                record_launch("linear_mfma_splitk", grid.x * grid.y, 256, (uint64_t)row_tiles * o_tiles);
+                record_launch("linear_mfma_splitk", grid.x, 256, (uint64_t)row_tiles * o_tiles);
             } else if (row_tiles <= 4) {
                 const dim3 grid((row_tiles + 1) / 2, (o_tiles + 15) / 16);
                 hipLaunchKernelGGL((linear_mfma_bf16_kernel<1, 8>), grid, dim3(256), 0, st, a);

@@ -295,3 +295,39 @@ def test_bf16_small_tiles_with_the_inner_axis_shared_by_groups_of_waves(inner):
     assert np.array_equal(do.raw()[mask], ho.storage[mask])
     for t in (dx, dw, do):
         t.free()
+
+
+# (x dims, s, R, head planar, H, D, inner, workgroups expected): decode steps of 17-64
+# sequences, where one workgroup takes two or four row tiles against two or four output
+# tiles; ragged last row tile, ragged last output tile, ragged inner axis, rows of one plane
+DECODE_TILES = [
+    ((64, 1), 0, 1, False, 1, 4096, 200, 2 * 128),              # 2 x 2
+    ((50, 1), 0, 1, False, 1, 5640, 96, 2 * 96),                # 2 x 4: 353 output tiles -> 89 blocks, padded to 96
+    ((33, 1), 0, 1, True, 88, 64, 160, 2 * 88),                 # 2 x 4: three row tiles, head planar
+    ((1, 70), 5, 60, False, 1, 5632, 72, 2 * 88),               # 2 x 4: rows of one plane
+    ((20, 1), 0, 1, False, 1, 16384, 64, 256),                  # 2 x 4: two row tiles
+    ((64, 1), 0, 1, False, 1, 10248, 3912, 168),                # 4 x 4: 641 output tiles -> 161 blocks, padded to 168
+]
+
+
+@pytest.mark.parametrize("case", range(len(DECODE_TILES)))
+def test_bf16_decode_steps_with_larger_workgroup_tiles(case):
+    lead, s, R, hp, H, D, inner, workgroups = DECODE_TILES[case]
+    xd, wd = lead + (inner,), (H * D, inner)
+    xv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(xd)), 0, 1, 61 + case)).reshape(xd)
+    wv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(wd)), 0, 0.05, 71 + case)).reshape(wd)
+    dx, _ = pair(DT_BF16, xd, values=xv)
+    dw, _ = pair(DT_BF16, wd, values=wv)
+    od = xd[:-2] + ((H, R, D) if hp else (R, H * D))
+    do, ho = pair(DT_BF16, od, salt=81 + case)
+    assert iomx.linear(dx.view(), dw.view(), do.view(), s, R, hp, H, D) == 0
+    ll = iomx.last_launch()
+    assert ll.kernel.decode() == "linear_mfma_splitk" and ll.grid == workgroups
+    got = do.view().to_host()
+    g3 = got.reshape(xd[0], H, R, D).transpose(0, 2, 1, 3).reshape(xd[0], R, H * D) if hp else got
+    for b in range(xd[0]):
+        assert bf16_bound(g3[b], xv[b, s:s + R], wv).all(), b
+    mask = iomo.tile_plane(np.ones(od, np.uint16)) == 0
+    assert np.array_equal(do.raw()[mask], ho.storage[mask])     # padding untouched
+    for t in (dx, dw, do):
+        t.free()
