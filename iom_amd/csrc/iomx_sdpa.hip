@@ -734,14 +734,17 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
         const uint8_t* kb = a.k + (plane[1] + (uint64_t)hkv * a.k_head_stride) * a.kv_plane_bytes;
         const uint8_t* vb = a.v + (plane[2] + (uint64_t)hkv * a.v_head_stride) * a.kv_plane_bytes;
+        // the raw bits of q: flushed after K and V have been requested, so that nothing waits
+        // for q alone
+        u32x4 q_bits[D32];
         bf16x8_t qf[D32];
 #pragma unroll
         for (int c = 0; c < D32; ++c) {
             const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
-            qf[c] = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
+            q_bits[c] = u32x4{0, 0, 0, 0};
             if (i0 < a.D)
-                qf[c] = daz8(load_k8_bits(qb + ((uint64_t)(qrow >> 4) * a.d_tiles + tile) * kTileBytes
-                                                  + (qrow & 15u) * kRowBytes, c0, i0, a.D));
+                q_bits[c] = load_k8_bits(qb + ((uint64_t)(qrow >> 4) * a.d_tiles + tile) * kTileBytes
+                                            + (qrow & 15u) * kRowBytes, c0, i0, a.D);
         }
         // K of group g (two 16-token tiles), requested one group ahead of its use
         struct KGroup { u32x4 w[2][D32]; };
@@ -795,16 +798,57 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                 }
             }
         };
+        // pass 2 sends a group that every row in use sees whole through the matrix cores with V
+        // loaded straight from the cache in the operand order (lane (feature l16, kg): tokens
+        // 32g + 4kg + j and 32g + 16 + 4kg + j), flushed in registers
+        const uint32_t vis_min = a.a + 1 < a.L ? a.a + 1 : a.L;          // what row 0 sees: the least
+        const uint32_t full_groups = vis_min / 32;
+        // of this share: the fully visible groups end at full_hi, the others start at tail_lo
+        const uint32_t full_hi = full_groups < g_hi ? full_groups : g_hi;
+        const uint32_t tail_lo = full_groups > g_lo ? full_groups : g_lo;
+        struct VFrag { u32x4 w[DT16]; };
+        auto load_vf = [&](uint32_t g, VFrag& vf) {
+#pragma unroll
+            for (int dt = 0; dt < DT16; ++dt) {
+                // pairs of 16-bit loads into the halves of one register
+                u16x2_t h[4];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t token = 32 * g + (j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4));   // < vis_min <= L
+                    uint16_t bits = 0;
+                    if (dt * kTile + l16 < a.D)
+                        bits = *reinterpret_cast<const uint16_t*>(
+                                vb + ((token >> 4) * a.d_tiles + dt) * kTileBytes + (token & 15u) * kRowBytes + l16 * 2);
+                    h[j >> 1][j & 1] = bits;
+                }
+                // raw bits: they are flushed where they are used, so a request does not wait here
+                vf.w[dt] = u32x4{__builtin_bit_cast(uint32_t, h[0]), __builtin_bit_cast(uint32_t, h[1]),
+                                 __builtin_bit_cast(uint32_t, h[2]), __builtin_bit_cast(uint32_t, h[3])};
+            }
+        };
         // pass 1: the rows' statistics over this wave's groups, then over the waves
         RowStats st = {-inf, 0.0f, 0u, false, false};
         // a ring of PD groups of K (and of V in pass 2): group g + PD*NW is requested as soon as
         // group g has been multiplied, so PD groups per wave are in flight -- one wave's chain of
         // dependent loads is what a long prefix costs here
         KGroup kr[PD];
+        VFrag vr[PD];
+        // a wave whose groups all fit the ring still holds their K after pass 1; V of the first
+        // groups of pass 2 is requested here, together with K, so the step waits for memory once
+        const bool ring_kept = PHASE == 0 && g_lo + wave + PD * NW >= g_hi;
         if (PHASE != 2) {
 #pragma unroll
         for (int slot = 0; slot < PD; ++slot)
             if (g_lo + wave + slot * NW < g_hi) load_k(g_lo + wave + slot * NW, kr[slot]);
+        if (PHASE == 0) {
+#pragma unroll
+            for (int slot = 0; slot < PD; ++slot)
+                if (g_lo + wave + slot * NW < full_hi) load_vf(g_lo + wave + slot * NW, vr[slot]);
+        }
+        }
+#pragma unroll
+        for (int c = 0; c < D32; ++c) qf[c] = daz8(q_bits[c]);
+        if (PHASE != 2) {
 #pragma unroll 1
         for (uint32_t g0 = g_lo + wave; g0 < g_hi; g0 += PD * NW) {
 #pragma unroll
@@ -886,30 +930,6 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         // 32g + 16 + 4kg + j), flushed in registers.  The group on the diagonal and the ragged last
         // group take the vector units: probabilities to LDS, lane = feature, and a token a row
         // must not see is left out of that row's sum by a select.
-        const uint32_t vis_min = a.a + 1 < a.L ? a.a + 1 : a.L;          // what row 0 sees: the least
-        const uint32_t full_groups = vis_min / 32;
-        // of this share: the fully visible groups end at full_hi, the others start at tail_lo
-        const uint32_t full_hi = full_groups < g_hi ? full_groups : g_hi;
-        const uint32_t tail_lo = full_groups > g_lo ? full_groups : g_lo;
-        struct VFrag { u32x4 w[DT16]; };
-        auto load_vf = [&](uint32_t g, VFrag& vf) {
-#pragma unroll
-            for (int dt = 0; dt < DT16; ++dt) {
-                // pairs of 16-bit loads into the halves of one register
-                u16x2_t h[4];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const uint32_t token = 32 * g + (j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4));   // < vis_min <= L
-                    uint16_t bits = 0;
-                    if (dt * kTile + l16 < a.D)
-                        bits = *reinterpret_cast<const uint16_t*>(
-                                vb + ((token >> 4) * a.d_tiles + dt) * kTileBytes + (token & 15u) * kRowBytes + l16 * 2);
-                    h[j >> 1][j & 1] = bits;
-                }
-                vf.w[dt] = u32x4{daz2(__builtin_bit_cast(uint32_t, h[0])), daz2(__builtin_bit_cast(uint32_t, h[1])),
-                                 daz2(__builtin_bit_cast(uint32_t, h[2])), daz2(__builtin_bit_cast(uint32_t, h[3]))};
-            }
-        };
         f32x4_t om[DT16];                                   // matrix-core part: out[row l16][16 dt + 4 kg + j]
 #pragma unroll
         for (int dt = 0; dt < DT16; ++dt) om[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
@@ -931,12 +951,11 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                          daz2(pack_bf16(pr[4], pr[5])), daz2(pack_bf16(pr[6], pr[7]))};
         };
         {
-            VFrag vr[PD];
 #pragma unroll
             for (int slot = 0; slot < PD; ++slot)
                 if (g_lo + wave + slot * NW < full_hi) {
-                    load_k(g_lo + wave + slot * NW, kr[slot]);
-                    load_vf(g_lo + wave + slot * NW, vr[slot]);
+                    if (!ring_kept) load_k(g_lo + wave + slot * NW, kr[slot]);
+                    if (PHASE != 0) load_vf(g_lo + wave + slot * NW, vr[slot]);
                 }
 #pragma unroll 1
             for (uint32_t g0 = g_lo + wave; g0 < full_hi; g0 += PD * NW) {
@@ -950,7 +969,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                     const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, probabilities(g, s));
 #pragma unroll
                     for (int dt = 0; dt < DT16; ++dt)
-                        om[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vr[slot].w[dt]), pf, om[dt], 0, 0, 0);
+                        om[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(daz8(vr[slot].w[dt]), pf, om[dt], 0, 0, 0);
                     if (g + PD * NW < full_hi) load_vf(g + PD * NW, vr[slot]);
                 }
             }
