@@ -294,7 +294,7 @@ __global__ __launch_bounds__(256) void linear_mfma_bf16_kernel(const LinearArgs 
 // the launch picks MT = 1 and lets NT output tiles share each x fragment; with more
 // row tiles and many output tiles, 2 x 2, 2 x 4 or 4 x 4 tiles per workgroup read
 // both operands less often from L2, which is what bounds those launches.
-template <int MT, int NT>
+template <int MT, int NT, int SETS>
 __global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const LinearArgs a) {
     constexpr uint32_t kTileBytes = 512, kRowBytes = 32;
     __shared__ f32x4_t partial[3][MT][NT][64];
@@ -334,29 +334,79 @@ __global__ __launch_bounds__(256) void linear_mfma_splitk_bf16_kernel(const Line
     const uint32_t tile_off = (kg >> 1) * kTileBytes, c0 = (kg & 1u) * 8u;
     const uint32_t lane_off = tile_off + c0 * 2;
     const uint32_t full_steps = a.I >> 5;
-    // kBatch slices a wave are requested before the first is multiplied: a wave has
-    // only a few slices, and what it waits for is memory latency
-    constexpr uint32_t kBatch = (MT + NT) <= 5 ? 8 : 4;
-    uint32_t step = wave;
-    for (; step + 4 * (kBatch - 1) < full_steps; step += 4 * kBatch) {
-        bf16x8_t wf[kBatch][NT], xf[kBatch][MT];
+    // SETS == 2 where a launch has at most one workgroup per CU (nothing else covers a wave's
+    // waits there); with more workgroups than that the single set, which leaves registers for
+    // a second workgroup per CU, was faster (64 rows x [32000,2048]: 43 against 48-50 us)
+    uint32_t step;
+    if constexpr (SETS == 2) {
+        // Two register sets of kBatch slices each: while one set is multiplied the other is on
+        // its way, so a wave always has kBatch to 2 x kBatch slices in flight -- what a wave waits
+        // for is memory latency, and with one set it waited once per set.  The slices are still
+        // multiplied in increasing order.
+        constexpr uint32_t kBatch = (MT + NT) <= 3 ? 8 : 4;
+        bf16x8_t wf0[kBatch][NT], xf0[kBatch][MT], wf1[kBatch][NT], xf1[kBatch][MT];
+        auto request = [&](uint32_t at, bf16x8_t (&wf)[kBatch][NT], bf16x8_t (&xf)[kBatch][MT]) {
 #pragma unroll
-        for (uint32_t u = 0; u < kBatch; ++u) {
-            const uint64_t off = (uint64_t)(step + 4 * u) * (2 * kTileBytes) + lane_off;
-#pragma unroll
-            for (int n = 0; n < NT; ++n)
-                wf[u][n] = __builtin_bit_cast(bf16x8_t, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[n] + off)));
-#pragma unroll
-            for (int m = 0; m < MT; ++m)
-                xf[u][m] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(xrow[m] + off));
-        }
-#pragma unroll
-        for (uint32_t u = 0; u < kBatch; ++u)
-#pragma unroll
-            for (int m = 0; m < MT; ++m)
+            for (uint32_t u = 0; u < kBatch; ++u) {
+                const uint64_t off = (uint64_t)(at + 4 * u) * (2 * kTileBytes) + lane_off;
 #pragma unroll
                 for (int n = 0; n < NT; ++n)
-                    acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][n], xf[u][m], acc[m][n], 0, 0, 0);
+                    wf[u][n] = __builtin_bit_cast(bf16x8_t, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[n] + off)));
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    xf[u][m] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(xrow[m] + off));
+            }
+        };
+        auto multiply = [&](const bf16x8_t (&wf)[kBatch][NT], const bf16x8_t (&xf)[kBatch][MT]) {
+#pragma unroll
+            for (uint32_t u = 0; u < kBatch; ++u)
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+#pragma unroll
+                    for (int n = 0; n < NT; ++n)
+                        acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][n], xf[u][m], acc[m][n], 0, 0, 0);
+        };
+        constexpr uint32_t kSpan = 4 * kBatch;                 // inner steps between the sets of one wave
+        step = wave;
+        bool whole = step + 4 * (kBatch - 1) < full_steps;     // a whole set starts at step
+        if (whole) request(step, wf0, xf0);
+        while (whole) {
+            bool next = step + kSpan + 4 * (kBatch - 1) < full_steps;
+            if (next) request(step + kSpan, wf1, xf1);
+            multiply(wf0, xf0);
+            step += kSpan;
+            if (!next) break;
+            next = step + kSpan + 4 * (kBatch - 1) < full_steps;
+            if (next) request(step + kSpan, wf0, xf0);
+            multiply(wf1, xf1);
+            step += kSpan;
+            whole = next;
+        }
+    } else {
+        // kBatch slices a wave are requested before the first is multiplied: a wave has
+        // only a few slices, and what it waits for is memory latency
+        constexpr uint32_t kBatch = (MT + NT) <= 5 ? 8 : 4;
+        step = wave;
+        for (; step + 4 * (kBatch - 1) < full_steps; step += 4 * kBatch) {
+            bf16x8_t wf[kBatch][NT], xf[kBatch][MT];
+#pragma unroll
+            for (uint32_t u = 0; u < kBatch; ++u) {
+                const uint64_t off = (uint64_t)(step + 4 * u) * (2 * kTileBytes) + lane_off;
+#pragma unroll
+                for (int n = 0; n < NT; ++n)
+                    wf[u][n] = __builtin_bit_cast(bf16x8_t, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow[n] + off)));
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    xf[u][m] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4*>(xrow[m] + off));
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < kBatch; ++u)
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+#pragma unroll
+                    for (int n = 0; n < NT; ++n)
+                        acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][n], xf[u][m], acc[m][n], 0, 0, 0);
+        }
     }
     for (; step < full_steps; step += 4) {
         const uint64_t off = (uint64_t)step * (2 * kTileBytes) + lane_off;
@@ -931,8 +981,12 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                 b.row_blocks = (row_tiles + mt - 1) / mt;
                 b.out_blocks = (uint32_t)((o_tiles + nt - 1) / nt);
                 const dim3 grid((b.out_blocks + 7) / 8 * 8 * b.row_blocks);
+                const bool two_sets = grid.x <= 256 && !(mt == 4 && nt == 4);
 #define IOMX_SPLITK(M, N) \
-    if (mt == M && nt == N) hipLaunchKernelGGL((linear_mfma_splitk_bf16_kernel<M, N>), grid, dim3(256), 0, st, b)
+    if (mt == M && nt == N) { \
+        if (two_sets) hipLaunchKernelGGL((linear_mfma_splitk_bf16_kernel<M, N, 2>), grid, dim3(256), 0, st, b); \
+        else hipLaunchKernelGGL((linear_mfma_splitk_bf16_kernel<M, N, 1>), grid, dim3(256), 0, st, b); \
+    }
                 IOMX_SPLITK(1, 1); IOMX_SPLITK(1, 2); IOMX_SPLITK(1, 4); IOMX_SPLITK(2, 1); IOMX_SPLITK(4, 1);
                 IOMX_SPLITK(2, 2); IOMX_SPLITK(2, 4); IOMX_SPLITK(4, 4);
 #undef IOMX_SPLITK

@@ -307,6 +307,12 @@ DECODE_TILES = [
     ((1, 70), 5, 60, False, 1, 5632, 72, 2 * 88),               # 2 x 4: rows of one plane
     ((20, 1), 0, 1, False, 1, 16384, 64, 256),                  # 2 x 4: two row tiles
     ((64, 1), 0, 1, False, 1, 10248, 3912, 168),                # 4 x 4: 641 output tiles -> 161 blocks, padded to 168
+    # long inner axes: at most 256 workgroups walk it with two register sets of slices in
+    # turn (several whole sets, then single slices, then the ragged end), more with one set
+    ((64, 1), 0, 1, False, 1, 4096, 2080, 256),                 # 2 x 2, two sets of 4 slices
+    ((64, 1), 0, 1, False, 1, 2048, 5648, 256),                 # 1 x 2, two sets of 8 slices, ragged end
+    ((3, 1), 0, 1, False, 1, 2048, 1504, 128),                  # 1 x 1, two sets: an odd number of whole sets
+    ((1, 1), 0, 1, False, 1, 5632, 2048, 352),                  # 1 x 1, one set of 8 slices
 ]
 
 
