@@ -313,6 +313,9 @@ DECODE_TILES = [
     ((64, 1), 0, 1, False, 1, 2048, 5648, 256),                 # 1 x 2, two sets of 8 slices, ragged end
     ((3, 1), 0, 1, False, 1, 2048, 1504, 128),                  # 1 x 1, two sets: an odd number of whole sets
     ((1, 1), 0, 1, False, 1, 5632, 2048, 352),                  # 1 x 1, one set of 8 slices
+    # many row blocks of one row tile each next to one another in the workgroup sequence
+    ((100, 1), 0, 1, False, 1, 2048, 96, 7 * 64),               # 1 x 2, seven row blocks
+    ((130, 1), 0, 1, False, 1, 272, 40, 9 * 24),                # 1 x 1, nine row blocks, 17 output blocks padded to 24
 ]
 
 
