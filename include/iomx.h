@@ -32,7 +32,8 @@ typedef enum iomx_status {
     IOMX_OK = 0,
     IOMX_ERR_INVALID = -1,     /* malformed request (std::invalid_argument)   */
     IOMX_ERR_UNSUPPORTED = -2, /* leaf or shape outside this library's scope  */
-    IOMX_ERR_OVERFLOW = -3     /* address arithmetic would overflow           */
+    IOMX_ERR_OVERFLOW = -3,    /* address arithmetic would overflow           */
+    IOMX_ERR_EXHAUSTED = -4    /* needs more scratch than a fixed array holds */
 } iomx_status;
 
 const char* iomx_error_string(int status);
@@ -312,6 +313,25 @@ int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_view* k, const
 int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
                      const iomx_view* out, uint64_t a, uint64_t L, void* workspace,
                      uint64_t workspace_bytes, int path, iomx_stream_t stream);
+
+/*
+ * iomx_launch_sdpa for callers that cannot allocate or bring a workspace (code under
+ * HIP graph capture, serving loops and harnesses in which hipMalloc is forbidden).  It
+ * has no counterpart in the reference, where the caller always leases the workspace
+ * from the device arena.  Same operands, same kernels, same bits as iomx_launch_sdpa;
+ * what that entry point keeps in the caller's workspace goes into a fixed array of
+ * IOMX_SDPA_STATIC_BYTES that the library's code object carries once per GPU until the
+ * process ends.  No hipMalloc, hipFree or allocating call is made.  A request whose
+ * iomx_sdpa_workspace figure exceeds IOMX_SDPA_STATIC_BYTES returns IOMX_ERR_EXHAUSTED
+ * before any launch.  The address of the array on the current device is looked up on
+ * the first call made on that device (not under capture; later calls may be captured).
+ * All calls on one GPU share the one array: calls that overlap in time on the same GPU,
+ * from several streams or threads, race; calls in one stream's order do not.
+ */
+#define IOMX_SDPA_STATIC_BYTES (16u << 20)
+int iomx_launch_sdpa_static(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
+                            const iomx_view* out, uint64_t a, uint64_t L, int path,
+                            iomx_stream_t stream);
 
 /* Element strides of one softmax-stage buffer (src/rocm/sdpa_softmax.hpp:14-22). */
 typedef struct iomx_stage_layout {

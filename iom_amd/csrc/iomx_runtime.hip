@@ -42,6 +42,7 @@ const char* iomx_error_string(int status) {
         case IOMX_ERR_INVALID: return "iomx: invalid request";
         case IOMX_ERR_UNSUPPORTED: return "iomx: unsupported leaf or shape";
         case IOMX_ERR_OVERFLOW: return "iomx: address arithmetic overflows";
+        case IOMX_ERR_EXHAUSTED: return "iomx: request exceeds the fixed scratch array";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));

@@ -19,6 +19,7 @@
 //                   rows the same way where the flag of their KV head is up: a
 //                   masked probability is +0, and +0 times an infinite V of a token
 //                   the row must not see would poison the row on the matrix cores.
+#include <atomic>
 #include <type_traits>
 
 #include "iomx_mfma.hpp"
@@ -1240,9 +1241,11 @@ extern "C" int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_vie
     return sdpa_layout(s, L, &header, &region, bytes);
 }
 
-extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
-                                const iomx_view* out, uint64_t a, uint64_t L, void* workspace,
-                                uint64_t workspace_bytes, int path, iomx_stream_t stream) {
+// The launches of one attention request; `workspace` is the caller's buffer
+// (iomx_launch_sdpa) or this device's copy of the fixed array (iomx_launch_sdpa_static).
+static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
+                       const iomx_view* out, uint64_t a, uint64_t L, void* workspace,
+                       uint64_t workspace_bytes, int path, iomx_stream_t stream) {
     SdpaShape s;
     IOMX_TRY(sdpa_shape(q, k, v, out, a, L, &s));
     if (dtype != IOMX_DT_BF16) return IOMX_ERR_UNSUPPORTED;
@@ -1388,4 +1391,54 @@ extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* 
     record_launch("sdpa_rows", rows_grid.x * rows_grid.y, 64, pairs * per_pair);
     IOMX_HIP(hipGetLastError());
     return IOMX_OK;
+}
+
+extern "C" int iomx_launch_sdpa(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
+                                const iomx_view* out, uint64_t a, uint64_t L, void* workspace,
+                                uint64_t workspace_bytes, int path, iomx_stream_t stream) {
+    return sdpa_launch(dtype, q, k, v, out, a, L, workspace, workspace_bytes, path, stream);
+}
+
+// ---- attention without a caller workspace and without any allocation ----------
+//
+// The packed V fragments / flushed K tiles of a prefill (or the shares' statistics
+// and partial sums of a long-prefix decode step) go into a fixed array that the code
+// object itself carries, one copy per GPU.  In host code the array's name is only a
+// handle for hipGetSymbolAddress: the address a kernel may use is looked up once per
+// device, with that device current, and kept.
+
+static __device__ __align__(256) unsigned char scratch[IOMX_SDPA_STATIC_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_address[kMaxDevices];
+
+int scratch_of_current_device(void** address) {
+    int device = -1;
+    IOMX_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return IOMX_ERR_UNSUPPORTED;
+    void* known = g_scratch_address[device].load(std::memory_order_acquire);
+    if (known == nullptr) {
+        IOMX_HIP(hipGetSymbolAddress(&known, HIP_SYMBOL(scratch)));
+        if (known == nullptr || (reinterpret_cast<uintptr_t>(known) & 255u) != 0) return IOMX_ERR_INVALID;
+        g_scratch_address[device].store(known, std::memory_order_release);
+    }
+    *address = known;
+    return IOMX_OK;
+}
+}  // namespace
+
+extern "C" int iomx_launch_sdpa_static(int dtype, const iomx_view* q, const iomx_view* k,
+                                       const iomx_view* v, const iomx_view* out, uint64_t a,
+                                       uint64_t L, int path, iomx_stream_t stream) {
+    uint64_t need = 0, alignment = 1;
+    IOMX_TRY(iomx_sdpa_workspace(dtype, q, k, v, out, a, L, &need, &alignment));
+    if (path != 0) need = 0;  // the reference-order kernel keeps nothing outside its operands
+    if (need > IOMX_SDPA_STATIC_BYTES) return IOMX_ERR_EXHAUSTED;
+    void* address = nullptr;
+    IOMX_TRY(scratch_of_current_device(&address));
+    // Every word of the part in use is written by the pack kernel (or by the first two
+    // decode phases) before it is read in the same call, so what an earlier call left
+    // in the array needs no clearing.
+    return sdpa_launch(dtype, q, k, v, out, a, L, address, IOMX_SDPA_STATIC_BYTES, path, stream);
 }

@@ -58,7 +58,8 @@ SYMBOLS = [
     "iomx_stream_synchronize", "iomx_event_create", "iomx_event_destroy", "iomx_event_record",
     "iomx_event_synchronize", "iomx_event_query", "iomx_event_elapsed_ms",
     "iomx_stream_begin_capture", "iomx_stream_end_capture", "iomx_graph_launch", "iomx_graph_destroy",
-    "iomx_launch_linear", "iomx_sdpa_workspace", "iomx_launch_sdpa", "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
+    "iomx_launch_linear", "iomx_sdpa_workspace", "iomx_launch_sdpa", "iomx_launch_sdpa_static",
+    "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
     "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul",
     "iomx_launch_copy", "iomx_launch_scatter", "iomx_launch_gather", "iomx_launch_softmax",
     "iomx_last_launch", "iomx_selftest_bf16_convert", "iomx_selftest_f16_binary",
@@ -157,6 +158,8 @@ def lib() -> C.CDLL:
                                           C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
         l.iomx_launch_sdpa.argtypes = [C.c_int, VP, VP, VP, VP, C.c_uint64, C.c_uint64, C.c_void_p,
                                        C.c_uint64, C.c_int, C.c_void_p]
+        l.iomx_launch_sdpa_static.argtypes = [C.c_int, VP, VP, VP, VP, C.c_uint64, C.c_uint64,
+                                              C.c_int, C.c_void_p]
         l.iomx_launch_embedding.argtypes = [C.c_int, C.c_int, VP, VP, VP, P, P]
         l.iomx_launch_rope.argtypes = [C.c_int, VP, VP, C.c_uint64, C.c_double, P]
         l.iomx_launch_scatter.argtypes = [C.c_int, VP, P, P]
@@ -483,6 +486,17 @@ def sdpa(q: DeviceView, k: DeviceView, v: DeviceView, out: DeviceView, a: int, L
     return lib().iomx_launch_sdpa(out.dtype, C.byref(cq), C.byref(ck), C.byref(cv), C.byref(co), a, L,
                                   workspace.ptr if workspace is not None else None,
                                   workspace.nbytes if workspace is not None else 0, path, _h(stream))
+
+
+SDPA_STATIC_BYTES = 16 << 20
+
+
+def sdpa_static(q: DeviceView, k: DeviceView, v: DeviceView, out: DeviceView, a: int, L: int,
+                path: int = 0, stream: Optional[Stream] = None) -> int:
+    """sdpa() with the workspace in the library's fixed per-GPU array: no allocation."""
+    cq, ck, cv, co = q.cview(), k.cview(), v.cview(), out.cview()
+    return lib().iomx_launch_sdpa_static(out.dtype, C.byref(cq), C.byref(ck), C.byref(cv),
+                                         C.byref(co), a, L, path, _h(stream))
 
 
 def cache_append(src: DeviceView, dst: DeviceView, a: int, stream: Optional[Stream] = None) -> int:
