@@ -8,8 +8,8 @@
 // inside the wave and the waves through LDS, then scales the registers and
 // stores: HBM sees x once and out once.
 //
-//   rmsnorm_band     F a multiple of 16 and a band that fits the register
-//                    budget (at most 16 chunks per lane of a 1024-lane workgroup).
+//   rmsnorm_band     F a multiple of 16: a band, or one of 2..8 row groups of it,
+//                    resident in the registers of one workgroup.
 //   rmsnorm_generic  any F and any band size: two passes over the band, the
 //                    second served by L2, with per-element column masks.
 #include "iomx_leaves.hpp"
@@ -102,104 +102,45 @@ __device__ __forceinline__ float inverse_rms(float sum, uint32_t feats, float ep
     return 1.0f / root;
 }
 
-// The band kernel: one band per workgroup, K 128-bit chunks per lane held in
-// registers between the two passes.  Whole-band loads and stores stream past
-// the caches; the scale row stays cached.  Keeping the register count low keeps
-// two 1024-lane workgroups resident per compute unit, so one band's loads
-// overlap the other's arithmetic and stores.  (Variants measured and dropped on
-// MI355X, [32768,2048]: a persistent workgroup that prefetches its next band
-// into a second register set, the scale row decoded once into registers, sixteen
-// lanes finishing the row totals for everyone, and a barrier-free kernel with
-// four rows per wave, and two passes with the second read served by the caches:
-// all slower, by 3-20 %.)
+// The resident kernel.  A band is cut into S parts of 16/S rows (S = 1: the whole
+// band); one workgroup of THREADS lanes owns one part and holds its K 128-bit chunks per
+// lane in registers between the two passes, so HBM sees x once and out once.  Inside a
+// tile the rows of a part are one contiguous run of kChunksPerTile/S chunks; a lane's
+// chunk index within its part maps to (tile, chunk in the run), the same lane always
+// sees the same row, and the lanes of a wave that share a row differ in the position
+// inside the row piece (low lane bits) and in the tile (bits above the run).
 //
-// The sum of squares uses a fused multiply-add per element (one rounding instead
-// of the reference's two): the total differs from the sequential reference
-// recurrence by a few units in the last place either way, far inside the bar.
-template <int DT, int K, int THREADS>
+// What the order of the code is for (each point measured on MI355X at [32768,2048]):
+//  * x and the scale row are requested together, before anything waits: a scale chunk
+//    fetched after the barrier sits in the path between the last load and the first
+//    store of a workgroup, and the compiler otherwise waits for each store's
+//    acknowledgement before it fetches the next scale chunk (stores and loads share
+//    one counter);
+//  * the values unpacked for the sum of squares are not kept: the raw chunks are made
+//    opaque after pass 1, so a lane holds 2*K*4 raw registers instead of K*8 decoded
+//    ones plus the scale, and two 1024-lane workgroups stay resident per compute unit
+//    (at most 64 registers) with K = 4;
+//  * all results are formed first and stored back to back.
+// FULL says that K*THREADS chunks cover a part exactly, which removes every bounds test.
+// PRE is the early scale request: a lane has room for it with up to four chunks of a
+// 2-byte leaf or eight of a 4-byte leaf (128 registers at most for 1024 lanes); without it
+// the scale chunk is fetched where it is used.
+//
+// The sum of squares uses a fused multiply-add per element (one rounding instead of the
+// reference's two): the total differs from the sequential reference recurrence by a few
+// units in the last place either way, far inside the bar.
+template <int DT, int K, int S, int THREADS, bool FULL, bool PRE>
 __global__ __launch_bounds__(THREADS) void rmsnorm_band_kernel(const RmsArgs a) {
     using L = RLeaf<DT>;
-    constexpr int kWaves = THREADS / 64;
-    __shared__ __attribute__((aligned(16))) float partial[kTile][kWaves];
-    const uint32_t tid = threadIdx.x;
-    const uint32_t row = lane_row<DT>(tid);
-    const uint32_t band = blockIdx.x;
-    uint32_t p = 0, tr = band;
-    if (a.walk.nlead != 0) {
-        p = band / a.tile_rows;
-        tr = band - p * a.tile_rows;
-    }
-    uint64_t plane[2];
-    walk_planes(a.walk, p, plane);
-    const uint8_t* xb = a.x + plane[0] * a.plane_bytes + (uint64_t)tr * a.band_bytes;
-    uint8_t* ob = a.out + plane[1] * a.plane_bytes + (uint64_t)tr * a.band_bytes;
-    u32x4 cur[K];
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const uint32_t c = tid + k * THREADS;
-        cur[k] = u32x4{0, 0, 0, 0};
-        if (c < a.band_chunks)
-            cur[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xb + (uint64_t)c * 16));
-    }
-    float acc = 0.0f;
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-        float f[L::kPerChunk];
-        unpack<DT>(cur[k], f);
-#pragma unroll
-        for (uint32_t e = 0; e < L::kPerChunk; ++e) acc = __builtin_fmaf(f[e], f[e], acc);
-    }
-    acc = row_sum_in_wave<DT>(acc);
-    float inverse;
-    if constexpr (kWaves > 1) {
-        if (row_leader<DT>(tid)) partial[row][tid / 64] = acc;
-        __syncthreads();
-        float total = 0.0f;
-#pragma unroll
-        for (int wv = 0; wv < kWaves; ++wv) total = total + partial[row][wv];
-        inverse = inverse_rms(total, a.feats, a.eps);
-    } else {
-        inverse = inverse_rms(acc, a.feats, a.eps);
-    }
-    if (tr * kTile + row >= a.rows) return;
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const uint32_t c = tid + k * THREADS;
-        if (c < a.band_chunks) {
-            const uint32_t soff = ((c / L::kChunksPerTile) * L::kChunksPerTile
-                                   + (c % L::kChunksPerRow)) * 16;
-            float f[L::kPerChunk], sc[L::kPerChunk];
-            unpack<DT>(cur[k], f);
-            unpack<DT>(*reinterpret_cast<const u32x4*>(a.scale + soff), sc);
-#pragma unroll
-            for (uint32_t e = 0; e < L::kPerChunk; ++e) {
-                const float normalized = f[e] * inverse;
-                f[e] = normalized * sc[e];
-            }
-            u32x4* dst = reinterpret_cast<u32x4*>(ob + (uint64_t)c * 16);
-            __builtin_nontemporal_store(pack<DT>(f), dst);
-        }
-    }
-}
-
-// Wide rows: the band is cut into S parts of 16/S rows each, one workgroup per
-// part, so that a workgroup still holds only K chunks per lane (two workgroups
-// stay resident per compute unit) however large F is.  Inside a tile the rows
-// of one part are one contiguous run of kChunksPerTile/S chunks; a lane's chunk
-// index within its part maps to (tile, chunk in the run), and the lanes of a
-// wave that share a row differ in the position inside the row piece (low bits)
-// and in the tile (bits above the run).
-template <int DT, int K, int S>
-__global__ __launch_bounds__(1024) void rmsnorm_split_kernel(const RmsArgs a) {
-    using L = RLeaf<DT>;
-    constexpr int THREADS = 1024;
     constexpr int kWaves = THREADS / 64;
     constexpr uint32_t SUB = L::kChunksPerTile / S;   // chunks of one part in one tile
     constexpr uint32_t RP = kTile / S;                // rows of one part
     static_assert(SUB >= L::kChunksPerRow, "a part holds whole row pieces");
+    static_assert(THREADS % 64 == 0 && (SUB >= 64 ? SUB % 64 == 0 : 64 % SUB == 0), "lane keeps its row");
     __shared__ __attribute__((aligned(16))) float partial[RP][kWaves];
     const uint32_t tid = threadIdx.x;
-    const uint32_t band = blockIdx.x / S, part = blockIdx.x % S;
+    const uint32_t band = S == 1 ? blockIdx.x : blockIdx.x / S;
+    const uint32_t part = S == 1 ? 0u : blockIdx.x % S;
     const uint32_t w = tid % SUB;
     const uint32_t row = w / L::kChunksPerRow;        // within the part
     uint32_t p = 0, tr = band;
@@ -213,14 +154,24 @@ __global__ __launch_bounds__(1024) void rmsnorm_split_kernel(const RmsArgs a) {
     uint8_t* ob = a.out + plane[1] * a.plane_bytes + (uint64_t)tr * a.band_bytes;
     const uint32_t part_chunks = a.band_chunks / S;
     uint32_t chunk[K];
-    u32x4 cur[K];
+    u32x4 cur[K], scl[PRE ? K : 1];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const uint32_t c = tid + k * THREADS;
-        chunk[k] = (c / SUB) * L::kChunksPerTile + part * SUB + w;
+        chunk[k] = S == 1 ? c : (c / SUB) * L::kChunksPerTile + part * SUB + w;
         cur[k] = u32x4{0, 0, 0, 0};
-        if (c < part_chunks)
+        if (FULL || c < part_chunks)
             cur[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xb + (uint64_t)chunk[k] * 16));
+    }
+    if constexpr (PRE) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const uint32_t soff = ((chunk[k] / L::kChunksPerTile) * L::kChunksPerTile
+                                   + (chunk[k] % L::kChunksPerRow)) * 16;
+            scl[k] = u32x4{0, 0, 0, 0};
+            if (FULL || tid + k * THREADS < part_chunks)
+                scl[k] = *reinterpret_cast<const u32x4*>(a.scale + soff);
+        }
     }
     float acc = 0.0f;
 #pragma unroll
@@ -229,6 +180,10 @@ __global__ __launch_bounds__(1024) void rmsnorm_split_kernel(const RmsArgs a) {
         unpack<DT>(cur[k], f);
 #pragma unroll
         for (uint32_t e = 0; e < L::kPerChunk; ++e) acc = __builtin_fmaf(f[e], f[e], acc);
+    }
+    if constexpr (L::kBytes == 2) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) asm volatile("" : "+v"(cur[k]));
     }
     // lanes of the wave that hold the same row: every lane bit that is not a row bit
     uint32_t shared_bits = 0;
@@ -239,28 +194,51 @@ __global__ __launch_bounds__(1024) void rmsnorm_split_kernel(const RmsArgs a) {
             shared_bits |= bit;
         }
     }
-    if ((tid & shared_bits) == 0) partial[row][tid / 64] = acc;
-    __syncthreads();
-    float total = 0.0f;
+    float total = acc;
+    if constexpr (kWaves > 1) {
+        if ((tid & shared_bits) == 0) partial[row][tid / 64] = acc;
+        __syncthreads();
+        total = 0.0f;
 #pragma unroll
-    for (int wv = 0; wv < kWaves; ++wv) total = total + partial[row][wv];
+        for (int wv = 0; wv < kWaves; ++wv) total = total + partial[row][wv];
+    }
     const float inverse = inverse_rms(total, a.feats, a.eps);
     if (tr * kTile + part * RP + row >= a.rows) return;
+    if constexpr (PRE) {
+        u32x4 res[K];
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        if (tid + k * THREADS < part_chunks) {
-            const uint32_t c = chunk[k];
-            const uint32_t soff = ((c / L::kChunksPerTile) * L::kChunksPerTile
-                                   + (c % L::kChunksPerRow)) * 16;
+        for (int k = 0; k < K; ++k) {
             float f[L::kPerChunk], sc[L::kPerChunk];
             unpack<DT>(cur[k], f);
-            unpack<DT>(*reinterpret_cast<const u32x4*>(a.scale + soff), sc);
+            unpack<DT>(scl[k], sc);
 #pragma unroll
             for (uint32_t e = 0; e < L::kPerChunk; ++e) {
                 const float normalized = f[e] * inverse;
                 f[e] = normalized * sc[e];
             }
-            __builtin_nontemporal_store(pack<DT>(f), reinterpret_cast<u32x4*>(ob + (uint64_t)c * 16));
+            res[k] = pack<DT>(f);
+        }
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if (FULL || tid + k * THREADS < part_chunks)
+                __builtin_nontemporal_store(res[k], reinterpret_cast<u32x4*>(ob + (uint64_t)chunk[k] * 16));
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if (FULL || tid + k * THREADS < part_chunks) {
+                const uint32_t soff = ((chunk[k] / L::kChunksPerTile) * L::kChunksPerTile
+                                       + (chunk[k] % L::kChunksPerRow)) * 16;
+                float f[L::kPerChunk], sc[L::kPerChunk];
+                unpack<DT>(cur[k], f);
+                unpack<DT>(*reinterpret_cast<const u32x4*>(a.scale + soff), sc);
+#pragma unroll
+                for (uint32_t e = 0; e < L::kPerChunk; ++e) {
+                    const float normalized = f[e] * inverse;
+                    f[e] = normalized * sc[e];
+                }
+                __builtin_nontemporal_store(pack<DT>(f), reinterpret_cast<u32x4*>(ob + (uint64_t)chunk[k] * 16));
+            }
         }
     }
 }
@@ -334,52 +312,57 @@ __global__ __launch_bounds__(256) void rmsnorm_generic_kernel(const RmsArgs a) {
 
 namespace {
 
-template <int DT, int K, int THREADS>
+template <int DT, int K, int S, int THREADS, bool PRE = (K * (int)RLeaf<DT>::kPerChunk <= 32)>
 void launch_band(const RmsArgs& a, hipStream_t s) {
-    hipLaunchKernelGGL((rmsnorm_band_kernel<DT, K, THREADS>), dim3(a.total_bands), dim3(THREADS), 0,
-                       s, a);
-    record_launch("rmsnorm_band", a.total_bands, THREADS, a.total_bands);
+    const uint32_t grid = a.total_bands * S;
+    if ((uint32_t)(K * THREADS * S) == a.band_chunks)
+        hipLaunchKernelGGL((rmsnorm_band_kernel<DT, K, S, THREADS, true, PRE>), dim3(grid), dim3(THREADS), 0, s, a);
+    else
+        hipLaunchKernelGGL((rmsnorm_band_kernel<DT, K, S, THREADS, false, PRE>), dim3(grid), dim3(THREADS), 0, s, a);
+    record_launch(S == 1 ? "rmsnorm_band" : "rmsnorm_split", grid, THREADS, grid);
 }
 
-template <int DT, int K, int S>
-void launch_split(const RmsArgs& a, hipStream_t s) {
-    hipLaunchKernelGGL((rmsnorm_split_kernel<DT, K, S>), dim3(a.total_bands * S), dim3(1024), 0, s, a);
-    record_launch("rmsnorm_split", a.total_bands * S, 1024, (uint64_t)a.total_bands * S);
-}
-
-// Chunks one 1024-lane workgroup can hold in registers without spilling: K = 8 per
-// lane for BF16 (whose unpacked chunk is eight floats), 16 for F32.  Measured on
-// MI355X with rows of 4096..16384 features: the fewest, largest parts win (runs of
-// 256 bytes or more per tile), and sixteen parts (32-byte runs) lose even to the
-// two-pass kernel, so the split stops at eight.
-template <int DT>
-constexpr uint32_t kResidentChunks = (RLeaf<DT>::kBytes == 2 ? 8u : 16u) * 1024u;
-
+// Which shape of the resident kernel: n = 128-bit chunks of one band (2F for the 2-byte
+// leaves, 4F for F32).  Measured on MI355X over 128 MiB of rows of 512..16384 features
+// (GB/s of x + out, average of three runs of 40 launches):
+//   * four chunks per lane is the sweet spot; at equal bytes per workgroup 512 lanes do as
+//     well as 1024 (BF16 n = 2048: K4 T512 5890, K2 T1024 5440; F32 n = 4096: K4 S2 T512
+//     5930, K4 S1 T1024 5780), more chunks per lane cost 5-10 % (F32 n = 8192: K4 S2 5950,
+//     K8 S1 5420), except for very wide F32 rows, where sixteen chunks on two parts beat
+//     eight on four (n = 32768: 5890 against 5220);
+//   * a part's runs should stay at 256 bytes or more per tile: 128-byte runs cost 5-20 %
+//     and 32-byte runs (sixteen parts) lose even to the two-pass kernel;
+//   * a shape whose K * THREADS * S chunks exceed n idles lanes in proportion, so the
+//     four-part shapes are kept for the widths they fit exactly.
 template <int DT>
 int launch(const RmsArgs& a, bool band_ok, hipStream_t s) {
     const uint32_t n = a.band_chunks;
-    constexpr int KS = RLeaf<DT>::kBytes == 2 ? 8 : 16;
-    if (band_ok && n > kResidentChunks<DT> && n <= 8 * kResidentChunks<DT>
-        && (uint64_t)a.total_bands * 8 <= 0x7FFFFFFFull) {
-        if (n <= 2 * kResidentChunks<DT>) launch_split<DT, KS, 2>(a, s);
-        else if (n <= 4 * kResidentChunks<DT>) launch_split<DT, KS, 4>(a, s);
-        else launch_split<DT, KS, 8>(a, s);
-        return IOMX_OK;
-    }
-    if (!band_ok || n > kResidentChunks<DT> || a.total_bands > 0x7FFFFFFFu) {
+    constexpr bool wide = RLeaf<DT>::kBytes != 2;      // 64 chunks per tile instead of 32
+    if (!band_ok || a.total_bands > 0x7FFFFFFFu / 8 || n > (wide ? 131072u : 65536u)) {
         const uint32_t cap = 1u << 20;
         const uint32_t grid = a.total_bands < cap ? a.total_bands : cap;
         hipLaunchKernelGGL((rmsnorm_generic_kernel<DT>), dim3(grid), dim3(256), 0, s, a);
         record_launch("rmsnorm_generic", grid, 256, a.total_bands);
-    } else if (n <= 64) launch_band<DT, 1, 64>(a, s);
-    else if (n <= 256) launch_band<DT, 1, 256>(a, s);
-    else if (n <= 512) launch_band<DT, 1, 512>(a, s);
-    else if (n <= 1024) launch_band<DT, 1, 1024>(a, s);
-    else if (n <= 2048) launch_band<DT, 2, 1024>(a, s);
-    else if (n <= 4096) launch_band<DT, 4, 1024>(a, s);
-    else if (n <= 8192) launch_band<DT, 8, 1024>(a, s);
-    else if constexpr (RLeaf<DT>::kBytes != 2) launch_band<DT, 16, 1024>(a, s);
-    else return IOMX_ERR_INVALID;          // unreachable: BF16 bands this wide are split above
+        return IOMX_OK;
+    }
+    if (n <= 64) launch_band<DT, 1, 1, 64>(a, s);
+    else if (n <= 256) launch_band<DT, 1, 1, 256>(a, s);
+    else if (n <= 512) launch_band<DT, 2, 1, 256>(a, s);
+    else if (n <= 1024) launch_band<DT, 2, 1, 512>(a, s);
+    else if (n <= 2048) launch_band<DT, 4, 1, 512>(a, s);
+    else if (n <= 4096) launch_band<DT, 4, 2, 512>(a, s);
+    else if (n <= 8192) launch_band<DT, 4, 2, 1024>(a, s);
+    else if (n == 16384) launch_band<DT, 4, 4, 1024>(a, s);
+    else if (n <= 16384) launch_band<DT, 8, 2, 1024>(a, s);
+    else if (n <= 32768) {
+        if constexpr (wide) launch_band<DT, 16, 2, 1024>(a, s);
+        else launch_band<DT, 8, 4, 1024, true>(a, s);
+    } else if (n <= 65536) {
+        if constexpr (wide) launch_band<DT, 8, 8, 1024>(a, s);
+        else launch_band<DT, 8, 8, 1024>(a, s);
+    } else {
+        if constexpr (wide) launch_band<DT, 16, 8, 1024>(a, s);
+    }
     return IOMX_OK;
 }
 

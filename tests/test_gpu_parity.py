@@ -314,8 +314,8 @@ RMS_CASES = [
     ((16, 31), [], "rmsnorm_generic"), ((3, 5, 130), [], "rmsnorm_generic"),
     ((2, 3, 17, 64), [("permute", ([1, 0],))], "rmsnorm_band"),
     ((6, 16, 48), [("slice", (0, 0, 3, 2))], "rmsnorm_band"),
-    ((40, 2048), [], "rmsnorm_band"), ((33, 256), [], "rmsnorm_band"), ((16, 512), [], "rmsnorm_band"),
-    ((2, 20, 1024), [], "rmsnorm_band"), ((48, 4096), [], "rmsnorm_band"), ((20, 5632), [], None),
+    ((40, 2048), [], "rmsnorm_split"), ((33, 256), [], "rmsnorm_band"), ((16, 512), [], "rmsnorm_band"),
+    ((2, 20, 1024), [], None), ((48, 4096), [], "rmsnorm_split"), ((20, 5632), [], None),
     ((16, 8192), [], None), ((16, 16384), [], "rmsnorm_split"), ((4, 40000), [], None),
     # wide rows cut into 2..8 parts per band, with tail rows and strided planes
     ((35, 32768), [], "rmsnorm_split"), ((3, 19, 16384), [("slice", (0, 0, 2, 2))], "rmsnorm_split"),
