@@ -555,6 +555,38 @@ def wl_chain(timer, steps, warmup):
                   "6 launches")
 
 
+def wl_hbm_ceiling(timer, steps, warmup, sizes_mib=(64, 128, 256), modes=None):
+    """What this GPU gives a bare stream in the launch shape of the elementwise kernels
+    (iomx_probe_stream): read-only, write-only, copy and two-read-one-write, per operand size.
+    Not an operation of the hot path: the practical ceiling the operations are compared with."""
+    table = ((iomx.PROBE_READ, "read", 1), (iomx.PROBE_WRITE, "write", 1),
+             (iomx.PROBE_COPY, "copy", 2), (iomx.PROBE_ADD, "add_2r1w", 3))
+    rows = []
+    for mib in sizes_mib:
+        nb = mib << 20
+        sets = [tuple(iomx.Buffer(nb) for _ in range(3)) for _ in range(ROT)]
+        for a, b, o in sets:
+            a.fill(0x3C, timer.stream)
+            b.fill(0x01, timer.stream)
+            o.fill(0x00, timer.stream)
+        timer.stream.synchronize()
+        for mode, name, mult in table:
+            if modes is not None and name not in modes:
+                continue
+
+            def launch(i):
+                a, b, o = sets[i % ROT]
+                check(iomx.probe_stream(mode, a, b, o, nb, timer.stream), "probe")
+
+            wall, ev = timer.run(launch, steps, warmup)
+            rows.append(report(f"hbm_probe_{name}_{mib}MiB_per_operand", mult * nb, nb // 4, wall, ev,
+                               iomx.last_launch().kernel.decode()))
+        for bufs in sets:
+            for t in bufs:
+                t.free()
+    return rows
+
+
 # ------------------------------------------------------------------ CPU baseline
 
 def cpu_baseline():
@@ -665,6 +697,7 @@ def main():
         "sdpa": lambda: wl_sdpa(timer, max(K // 5, 10), max(W // 2, 5)),
         "decoder_layer": lambda: wl_decoder_layer(timer, max(K // 5, 10), max(W // 2, 5)),
         "other_leaves": lambda: wl_other_leaves(timer, max(K // 10, 5), max(W // 10, 2)),
+        "hbm_ceiling": lambda: wl_hbm_ceiling(timer, K, W),
     }
 
     if args.only:
@@ -675,11 +708,14 @@ def main():
         return
 
     head = table["bcast_add_bf16"]()
+    # the bare copy of the headline's size, in the same run: what a stream of 128 MiB in and
+    # 128 MiB out reaches on this box with nothing else in the kernel
+    ceiling = wl_hbm_ceiling(timer, K, W, sizes_mib=(128,), modes=("copy",))[0]
     detail = []
     if not args.no_detail:
         for key in ("bcast_mul_bf16", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "copy_bf16", "add_f32",
                     "add_i32", "rmsnorm_bf16", "rmsnorm_f32", "silu_mul", "softmax", "softmax_causal",
-                    "chain", "layer_ops", "linear", "sdpa", "decoder_layer"):
+                    "chain", "layer_ops", "linear", "sdpa", "decoder_layer", "hbm_ceiling"):
             r = table[key]()
             detail.extend(r if isinstance(r, list) else [r])
     cpu = None if args.no_cpu else cpu_baseline()
@@ -699,6 +735,13 @@ def main():
                    "device": props.name.decode(), "compute_units": props.compute_units},
         "roofline": {"bound": "hbm", "achieved": head["GB_per_s"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": head["hbm_frac"], "traffic": traffic_of("bcast_add_bf16"),
+                     "traffic_source": "not measured in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
+                                       "this workload, scaled by the copy kernel, as committed in "
+                                       "profiles/hbm_traffic.json",
+                     "practical_peak": ceiling["GB_per_s"],
+                     "practical_peak_what": "bare copy probe (iomx_probe_stream), 128 MiB in + 128 MiB "
+                                            "out, measured in this run",
+                     "frac_of_practical_peak": round(head["GB_per_s"] / ceiling["GB_per_s"], 4),
                      "kernel": "elementwise_stream_kernel<BF16,ADD,FULL,ROWVEC,BANDS>",
                      "ms_per_launch": head["ms_per_launch"]},
         "cpu_baseline": cpu,

@@ -372,6 +372,20 @@ typedef struct iomx_launch_info {
 } iomx_launch_info;
 int iomx_last_launch(iomx_launch_info* info);
 
+/*
+ * Bandwidth probes (no counterpart in the reference): one launch of a bare stream over
+ * `bytes` bytes per operand (a multiple of 4096, operands 16-byte aligned), in the launch
+ * shape of the elementwise kernels -- one 128-bit chunk per lane, one-shot grid,
+ * nontemporal access -- and with nothing else in the kernel.  They measure what this GPU
+ * gives a read-only stream (a), a write-only stream (out), a copy (a -> out) and a
+ * two-read-one-write stream (a + b -> out, 32-bit integer adds), which is the practical
+ * ceiling the operation kernels are compared with.  READ needs `out` only as a pointer to
+ * 4 KiB of writable memory that it never writes.
+ */
+enum { IOMX_PROBE_READ = 0, IOMX_PROBE_WRITE = 1, IOMX_PROBE_COPY = 2, IOMX_PROBE_ADD = 3 };
+int iomx_probe_stream(int mode, const void* a, const void* b, void* out, uint64_t bytes,
+                      iomx_stream_t stream);
+
 /* Compares the hardware BF16 conversion with the software round-to-nearest-
  * even rule over all 2^32 binary32 encodings; *mismatches receives the count. */
 int iomx_selftest_bf16_convert(uint64_t* mismatches, iomx_stream_t stream);

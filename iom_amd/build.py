@@ -28,6 +28,7 @@ SOURCES = [
     "iomx_layer.hip",
     "iomx_linear.hip",
     "iomx_sdpa.hip",
+    "iomx_probe.hip",
 ]
 
 # -ffp-contract=off: no fused multiply-add may replace the reference's two

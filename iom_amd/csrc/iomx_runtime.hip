@@ -17,6 +17,19 @@ void record_launch(const char* kernel, uint32_t grid, uint32_t block, uint64_t w
     g_last_launch.work_items = work;
 }
 
+// IOMX_OK when [ptr, ptr + bytes) lies inside one device allocation.
+int device_range(const void* ptr, size_t bytes) {
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, const_cast<void*>(ptr)) != hipSuccess) {
+        (void)hipGetLastError();
+        return IOMX_ERR_INVALID;
+    }
+    const uintptr_t b = reinterpret_cast<uintptr_t>(base), p = reinterpret_cast<uintptr_t>(ptr);
+    if (p < b || bytes > size || p - b > size - bytes) return IOMX_ERR_INVALID;
+    return IOMX_OK;
+}
+
 __global__ void fill_kernel(u32x4* __restrict__ dst, uint64_t chunks, uint32_t word) {
     const u32x4 v = {word, word, word, word};
     for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < chunks;
@@ -142,12 +155,21 @@ int iomx_fill_async(void* ptr, uint8_t value, size_t bytes, iomx_stream_t stream
     return IOMX_OK;
 }
 
+// The blocking copies check the device side of the request against the allocation it
+// points into before the runtime sees it: a range that runs past its allocation comes back
+// as IOMX_ERR_INVALID instead of as a fault inside a staging copy.
 int iomx_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    if (bytes == 0) return IOMX_OK;
+    if (!dst || !src) return IOMX_ERR_INVALID;
+    IOMX_TRY(device_range(dst, bytes));
     IOMX_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
     return IOMX_OK;
 }
 
 int iomx_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    if (bytes == 0) return IOMX_OK;
+    if (!dst || !src) return IOMX_ERR_INVALID;
+    IOMX_TRY(device_range(src, bytes));
     IOMX_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
     return IOMX_OK;
 }

@@ -62,7 +62,7 @@ SYMBOLS = [
     "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
     "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul",
     "iomx_launch_copy", "iomx_launch_scatter", "iomx_launch_gather", "iomx_launch_softmax",
-    "iomx_last_launch", "iomx_selftest_bf16_convert", "iomx_selftest_f16_binary",
+    "iomx_last_launch", "iomx_selftest_bf16_convert", "iomx_selftest_f16_binary", "iomx_probe_stream",
 ]
 
 
@@ -168,6 +168,7 @@ def lib() -> C.CDLL:
         l.iomx_last_launch.argtypes = [C.POINTER(LaunchInfo)]
         l.iomx_selftest_bf16_convert.argtypes = [C.POINTER(C.c_uint64), P]
         l.iomx_selftest_f16_binary.argtypes = [C.POINTER(C.c_uint64), P]
+        l.iomx_probe_stream.argtypes = [C.c_int, P, P, P, C.c_uint64, P]
         _lib = l
     return _lib
 
@@ -258,6 +259,25 @@ class Event:
             self.h = C.c_void_p()
 
 
+_STAGE_BYTES = 32 << 20
+_stage = None
+
+
+def _staging():
+    """(address, numpy window) of one page-locked host buffer, allocated on first use and kept
+    for the life of the process.  Every transfer of this module goes host array -> this buffer
+    (a numpy copy) -> device by an asynchronous copy that is waited for, and back the same way:
+    the runtime then always moves page-locked memory by DMA and never has to choose, per call
+    and per size, between pinning the caller's pages, its own staging copies and direct host
+    access to device memory."""
+    global _stage
+    if _stage is None:
+        p = C.c_void_p()
+        check(lib().iomx_host_alloc(C.byref(p), _STAGE_BYTES), "host_alloc")
+        _stage = (p.value, np.ctypeslib.as_array((C.c_uint8 * _STAGE_BYTES).from_address(p.value)))
+    return _stage
+
+
 class Buffer:
     """One device allocation."""
 
@@ -267,16 +287,32 @@ class Buffer:
         check(lib().iomx_malloc(C.byref(self.ptr), max(self.nbytes, 16)), "malloc")
 
     def upload(self, arr: np.ndarray, offset: int = 0):
+        """Host array -> device, through the page-locked staging buffer (see _staging)."""
         arr = np.ascontiguousarray(arr)
-        assert offset + arr.nbytes <= self.nbytes
-        check(lib().iomx_memcpy_h2d(self.ptr.value + offset, arr.ctypes.data, arr.nbytes), "h2d")
+        if not self.ptr or offset < 0 or offset + arr.nbytes > self.nbytes:
+            raise ValueError(f"upload of {arr.nbytes} bytes at {offset} into a buffer of {self.nbytes}")
+        src = arr.reshape(-1).view(np.uint8)
+        address, window = _staging()
+        for at in range(0, src.size, _STAGE_BYTES):
+            m = min(_STAGE_BYTES, src.size - at)
+            window[:m] = src[at:at + m]
+            check(lib().iomx_memcpy_h2d_async(self.ptr.value + offset + at, address, m, None), "h2d")
+            check(lib().iomx_stream_synchronize(None), "h2d sync")
 
     def download(self, dtype, count: Optional[int] = None, offset: int = 0) -> np.ndarray:
         itemsize = np.dtype(dtype).itemsize
         if count is None:
             count = (self.nbytes - offset) // itemsize
+        if not self.ptr or offset < 0 or count < 0 or offset + count * itemsize > self.nbytes:
+            raise ValueError(f"download of {count} x {itemsize} bytes at {offset} from a buffer of {self.nbytes}")
         out = np.empty(count, dtype=dtype)
-        check(lib().iomx_memcpy_d2h(out.ctypes.data, self.ptr.value + offset, out.nbytes), "d2h")
+        dst = out.view(np.uint8)
+        address, window = _staging()
+        for at in range(0, dst.size, _STAGE_BYTES):
+            m = min(_STAGE_BYTES, dst.size - at)
+            check(lib().iomx_memcpy_d2h_async(address, self.ptr.value + offset + at, m, None), "d2h")
+            check(lib().iomx_stream_synchronize(None), "d2h sync")
+            dst[at:at + m] = window[:m]
         return out
 
     def fill(self, byte: int, stream: Optional[Stream] = None):
@@ -486,6 +522,16 @@ def sdpa(q: DeviceView, k: DeviceView, v: DeviceView, out: DeviceView, a: int, L
     return lib().iomx_launch_sdpa(out.dtype, C.byref(cq), C.byref(ck), C.byref(cv), C.byref(co), a, L,
                                   workspace.ptr if workspace is not None else None,
                                   workspace.nbytes if workspace is not None else 0, path, _h(stream))
+
+
+PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_ADD = range(4)
+
+
+def probe_stream(mode: int, a: Optional["Buffer"], b: Optional["Buffer"], out: "Buffer", nbytes: int,
+                 stream: Optional[Stream] = None) -> int:
+    """One launch of a bare bandwidth probe over `nbytes` bytes per operand."""
+    return lib().iomx_probe_stream(mode, a.ptr if a is not None else None,
+                                   b.ptr if b is not None else None, out.ptr, nbytes, _h(stream))
 
 
 SDPA_STATIC_BYTES = 16 << 20
