@@ -560,7 +560,8 @@ def wl_hbm_ceiling(timer, steps, warmup, sizes_mib=(64, 128, 256), modes=None):
     (iomx_probe_stream): read-only, write-only, copy and two-read-one-write, per operand size.
     Not an operation of the hot path: the practical ceiling the operations are compared with."""
     table = ((iomx.PROBE_READ, "read", 1), (iomx.PROBE_WRITE, "write", 1),
-             (iomx.PROBE_COPY, "copy", 2), (iomx.PROBE_ADD, "add_2r1w", 3))
+             (iomx.PROBE_COPY, "copy", 2), (iomx.PROBE_ADD, "add_2r1w", 3),
+             (iomx.PROBE_HELD_COPY, "held_copy_4x1024_barrier", 2))
     rows = []
     for mib in sizes_mib:
         nb = mib << 20

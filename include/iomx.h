@@ -380,9 +380,12 @@ int iomx_last_launch(iomx_launch_info* info);
  * gives a read-only stream (a), a write-only stream (out), a copy (a -> out) and a
  * two-read-one-write stream (a + b -> out, 32-bit integer adds), which is the practical
  * ceiling the operation kernels are compared with.  READ needs `out` only as a pointer to
- * 4 KiB of writable memory that it never writes.
+ * 4 KiB of writable memory that it never writes.  HELD_COPY is the memory side of the
+ * resident RMSNorm kernel alone (a -> out; bytes a multiple of 64 KiB): 1024-lane workgroups
+ * that load four chunks per lane, meet at a barrier and store.
  */
-enum { IOMX_PROBE_READ = 0, IOMX_PROBE_WRITE = 1, IOMX_PROBE_COPY = 2, IOMX_PROBE_ADD = 3 };
+enum { IOMX_PROBE_READ = 0, IOMX_PROBE_WRITE = 1, IOMX_PROBE_COPY = 2, IOMX_PROBE_ADD = 3,
+       IOMX_PROBE_HELD_COPY = 4 };
 int iomx_probe_stream(int mode, const void* a, const void* b, void* out, uint64_t bytes,
                       iomx_stream_t stream);
 

@@ -33,6 +33,18 @@ __global__ __launch_bounds__(64) void probe_add_kernel(const u32x4* __restrict__
     __builtin_nontemporal_store(v, out + c);
 }
 
+// The memory side of the resident RMSNorm kernel and nothing else: a 1024-lane workgroup loads
+// four chunks per lane (64 KiB, one BF16 band of 2048 features), meets at a barrier and stores.
+__global__ __launch_bounds__(1024) void probe_held_copy_kernel(const u32x4* __restrict__ a, u32x4* __restrict__ out) {
+    const size_t base = (size_t)blockIdx.x * 4096 + threadIdx.x;
+    u32x4 held[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) held[k] = __builtin_nontemporal_load(a + base + k * 1024);
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 4; ++k) __builtin_nontemporal_store(held[k], out + base + k * 1024);
+}
+
 }  // namespace iomx
 
 using namespace iomx;
@@ -67,6 +79,11 @@ extern "C" int iomx_probe_stream(int mode, const void* a, const void* b, void* o
             if (!a || !b) return IOMX_ERR_INVALID;
             hipLaunchKernelGGL(probe_add_kernel, dim3((uint32_t)(chunks / 64)), dim3(64), 0, s, pa, pb, po);
             record_launch("probe_add", (uint32_t)(chunks / 64), 64, chunks);
+            break;
+        case IOMX_PROBE_HELD_COPY:
+            if (!a || bytes % 65536 != 0) return IOMX_ERR_INVALID;
+            hipLaunchKernelGGL(probe_held_copy_kernel, dim3((uint32_t)(chunks / 4096)), dim3(1024), 0, s, pa, po);
+            record_launch("probe_held_copy", (uint32_t)(chunks / 4096), 1024, chunks);
             break;
         default:
             return IOMX_ERR_INVALID;

@@ -524,7 +524,7 @@ def sdpa(q: DeviceView, k: DeviceView, v: DeviceView, out: DeviceView, a: int, L
                                   workspace.nbytes if workspace is not None else 0, path, _h(stream))
 
 
-PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_ADD = range(4)
+PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_ADD, PROBE_HELD_COPY = range(5)
 
 
 def probe_stream(mode: int, a: Optional["Buffer"], b: Optional["Buffer"], out: "Buffer", nbytes: int,
