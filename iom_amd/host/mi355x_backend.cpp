@@ -24,6 +24,8 @@
 //     the caller's raw workspace: host -> workspace, then the scatter kernel (or
 //     the gather kernel, then workspace -> host).
 #include <array>
+#include <atomic>
+#include <chrono>
 #include <condition_variable>
 #include <cstddef>
 #include <cstdint>
@@ -51,11 +53,90 @@
 #include "src/iom_internal.hpp"  // iom::detail::UnsupportedOperation, leaf_bits
 
 #include "iomx.h"
+#include "mi355x_testing.hpp"
 
 namespace iom {
+
+namespace rocm_detail {
+namespace {
+std::atomic<SubmissionFault> g_armed_fault{SubmissionFault::none};
+}
+void inject_submission_fault_for_testing(SubmissionFault fault) noexcept {
+    g_armed_fault.store(fault, std::memory_order_release);
+}
+bool consume_submission_fault(SubmissionFault fault) noexcept {
+    if (g_armed_fault.load(std::memory_order_relaxed) != fault) return false;
+    SubmissionFault expected = fault;
+    return g_armed_fault.compare_exchange_strong(expected, SubmissionFault::none,
+                                                 std::memory_order_acq_rel);
+}
+std::atomic<std::size_t> event_create_count_for_testing{0};
+std::atomic<std::size_t> event_destroy_count_for_testing{0};
+std::atomic<std::size_t> stream_create_count_for_testing{0};
+std::atomic<std::size_t> stream_destroy_count_for_testing{0};
+std::atomic<std::size_t> device_allocation_count_for_testing{0};
+std::atomic<std::size_t> device_free_count_for_testing{0};
+std::atomic<std::size_t> linear_native_bf16_launch_count_for_testing{0};
+std::atomic<std::size_t> linear_scalar_launch_count_for_testing{0};
+std::atomic<std::size_t> silu_launch_count_for_testing{0};
+}  // namespace rocm_detail
+
 namespace {
 
+using rocm_detail::SubmissionFault;
+using rocm_detail::consume_submission_fault;
+
 constexpr std::size_t kArenaAlignment = 256;
+// What an injected native failure reports: hipErrorLaunchFailure's code, never raised by a kernel here.
+constexpr int kInjectedDeviceError = 719;
+
+// Counted wrappers of the native resource calls (the counters are the test seams' evidence
+// that a rejected queue creates nothing and that a retained lease destroys nothing).
+int counted_event_create(iomx_event_t* event) {
+    if (consume_submission_fault(SubmissionFault::queue_event_create)) return kInjectedDeviceError;
+    const int status = iomx_event_create(event, 0);
+    if (status == IOMX_OK) rocm_detail::event_create_count_for_testing.fetch_add(1);
+    return status;
+}
+void counted_event_destroy(iomx_event_t event) noexcept {
+    (void)iomx_event_destroy(event);
+    rocm_detail::event_destroy_count_for_testing.fetch_add(1);
+}
+int counted_stream_create(iomx_stream_t* stream) {
+    if (consume_submission_fault(SubmissionFault::queue_stream_create)) return kInjectedDeviceError;
+    const int status = iomx_stream_create(stream);
+    if (status == IOMX_OK) rocm_detail::stream_create_count_for_testing.fetch_add(1);
+    return status;
+}
+void counted_stream_destroy(iomx_stream_t stream) noexcept {
+    if (stream == nullptr) return;
+    (void)iomx_stream_destroy(stream);
+    rocm_detail::stream_destroy_count_for_testing.fetch_add(1);
+}
+
+// A callable with in-place storage: the per-operation completion actions capture a few
+// registry ids and references, and a std::function would put them on the heap once per
+// operation.  Captures must be trivially copyable, so a move is a byte copy.
+template <typename Signature, std::size_t Bytes>
+class InlineFunction;
+template <typename R, typename... A, std::size_t Bytes>
+class InlineFunction<R(A...), Bytes> {
+public:
+    InlineFunction() = default;
+    template <typename F, typename = std::enable_if_t<!std::is_same_v<std::decay_t<F>, InlineFunction>>>
+    InlineFunction(F f) {  // NOLINT: implicit on purpose, like std::function
+        static_assert(sizeof(F) <= Bytes, "capture does not fit the in-place storage");
+        static_assert(std::is_trivially_copyable_v<F> && std::is_trivially_destructible_v<F>,
+                      "captures must be plain data");
+        new (storage_) F(f);
+        invoke_ = [](void* self, A... args) -> R { return (*static_cast<F*>(self))(args...); };
+    }
+    explicit operator bool() const noexcept { return invoke_ != nullptr; }
+    R operator()(A... args) { return invoke_(storage_, args...); }
+private:
+    alignas(std::max_align_t) unsigned char storage_[Bytes] = {};
+    R (*invoke_)(void*, A...) = nullptr;
+};
 
 [[noreturn]] void throw_status(int status, const char* what) {
     std::string message(what);
@@ -139,11 +220,13 @@ public:
         check(iomx_set_device(static_cast<int>(ordinal_)), "set device");
         if (iomx_malloc(&arena_, arena_bytes_) != IOMX_OK || arena_ == nullptr)
             throw std::bad_alloc();
+        rocm_detail::device_allocation_count_for_testing.fetch_add(1);
         try {
             allocator_ = std::make_unique<ListAllocator>(arena_, arena_bytes_, kArenaAlignment);
             check(iomx_stream_create(&transfer_stream_), "transfer stream");
         } catch (...) {
             (void)iomx_free(arena_);
+            rocm_detail::device_free_count_for_testing.fetch_add(1);
             throw;
         }
     }
@@ -154,11 +237,15 @@ public:
             (void)iomx_stream_synchronize(transfer_stream_);
             (void)iomx_stream_destroy(transfer_stream_);
         }
+        // Leases that a failed final synchronisation left here: the device-wide
+        // synchronisation below is their covering proof; either way they end with the device.
+        (void)iomx_device_synchronize();
+        discard_retained_leases();
         // Quarantined storage is returned to the allocator's host-side books when
         // the registry state is destroyed (after this body); the device range
         // itself can go now.
-        (void)iomx_device_synchronize();
         (void)iomx_free(arena_);
+        rocm_detail::device_free_count_for_testing.fetch_add(1);
     }
 
     [[nodiscard]] BackendKind backend_kind() const noexcept override { return BackendKind::ROCM; }
@@ -187,6 +274,99 @@ public:
         try { allocator_->free(address); } catch (...) {}
     }
     [[nodiscard]] Allocator& data_allocator() noexcept { return *guarded_allocator_; }
+
+    // A workspace owner goes away (src/rocm/device.cpp:243-264).  A range that an accepted
+    // operation still leases -- the caller dropped the workspace before it waited -- must not
+    // return to the allocator while the kernel may use it: it is parked in the quarantine,
+    // which gives it back at the device's end.
+    void release_workspace(const RawWorkspace* owner, void* address, std::size_t bytes) noexcept {
+        if (address == nullptr) return;
+        bool retained = false;
+        {
+            std::lock_guard<std::mutex> lock(registry_state_.allocation_mutex);
+            retained = detail::workspace_range_retained(registry_state_.workspace_leases, owner,
+                                                        address, bytes);
+        }
+        if (retained) {
+            try {
+                registry_state_.quarantine.emplace<detail::AllocatorCleanupAction>(
+                        *guarded_allocator_, address, bytes);
+            } catch (...) {
+                // the range simply stays unavailable
+            }
+            return;
+        }
+        release(address);
+    }
+
+    // src/rocm/device_tensor.cpp:22-41: storage handed to a tensor is device memory of this
+    // ordinal inside this device's arena.
+    void validate_storage(void* address) const {
+        int owner = -1;
+        const int status = iomx_pointer_device(address, &owner);
+        const std::uintptr_t raw = reinterpret_cast<std::uintptr_t>(address);
+        const std::uintptr_t base = reinterpret_cast<std::uintptr_t>(arena_);
+        if (status != IOMX_OK || owner != ordinal() || raw < base || raw - base >= arena_bytes_)
+            throw std::runtime_error("MI355X tensor storage is incompatible with the owning device");
+    }
+
+    // ---- queue leases whose completion could not be proved ---------------------------
+    // (src/shared/gpu_queue_lifecycle.inl:94-180)  A queue whose final stream synchronisation
+    // fails leaves its stream, completion events, status cells and its place among the four
+    // queues here.  Nothing of it is destroyed or reused until a later synchronisation of that
+    // same stream succeeds (reclaim) or the device ends.
+    struct QueueLease {
+        iomx_stream_t stream = nullptr;
+        std::vector<iomx_event_t> events;
+        std::uint32_t* status_cells = nullptr;
+    };
+    static void destroy_lease(QueueLease& lease) noexcept {
+        for (iomx_event_t event : lease.events) counted_event_destroy(event);
+        lease.events.clear();
+        counted_stream_destroy(lease.stream);
+        lease.stream = nullptr;
+        if (lease.status_cells != nullptr) (void)iomx_host_free(lease.status_cells);
+        lease.status_cells = nullptr;
+    }
+    void retain_unknown_lease(QueueLease lease) noexcept {
+        std::lock_guard<std::mutex> lock(retained_mutex_);
+        try {
+            retained_leases_.push_back(std::move(lease));
+        } catch (...) {
+            // no room to remember it: the native objects stay alive, unreferenced
+        }
+    }
+    void reclaim_retained_leases() noexcept {
+        std::lock_guard<std::mutex> lock(retained_mutex_);
+        (void)iomx_set_device(ordinal());
+        for (std::size_t i = 0; i < retained_leases_.size();) {
+            const bool proved = !consume_submission_fault(SubmissionFault::stream_synchronize)
+                    && iomx_stream_synchronize(retained_leases_[i].stream) == IOMX_OK;
+            if (!proved) { ++i; continue; }
+            destroy_lease(retained_leases_[i]);
+            retained_leases_.erase(retained_leases_.begin() + static_cast<std::ptrdiff_t>(i));
+        }
+    }
+    void discard_retained_leases() noexcept {
+        std::lock_guard<std::mutex> lock(retained_mutex_);
+        for (QueueLease& lease : retained_leases_) destroy_lease(lease);
+        retained_leases_.clear();
+    }
+    [[nodiscard]] std::size_t retained_lease_count() noexcept {
+        std::lock_guard<std::mutex> lock(retained_mutex_);
+        return retained_leases_.size();
+    }
+    // A retained lease keeps its place among the device's four queues: together with the
+    // live queues (counted by the common layer) it may not exceed four.
+    void admit_queue() {
+        std::lock_guard<std::mutex> lock(retained_mutex_);
+        if (live_queues_ + retained_leases_.size() >= 4) throw std::bad_alloc();
+        ++live_queues_;
+    }
+    void retire_queue() noexcept {
+        std::lock_guard<std::mutex> lock(retained_mutex_);
+        if (live_queues_ != 0) --live_queues_;
+    }
 
     // Host transfers: one at a time per device, never waiting on any queue.
     void transfer(const TensorView& view, RawWorkspaceView workspace,
@@ -249,6 +429,9 @@ private:
     iomx_stream_t transfer_stream_ = nullptr;
     std::mutex transfer_mutex_;
     bool transfer_poisoned_ = false;
+    std::mutex retained_mutex_;
+    std::vector<QueueLease> retained_leases_;
+    std::size_t live_queues_ = 0;
     // Destroyed first (declared last): draining its quarantine uses the allocator.
     detail::RegistryState registry_state_;
 };
@@ -265,6 +448,7 @@ public:
         bytes_ = view().spec().tiled_storage_nbytes();
         address_ = device_.allocate(bytes_);
         try {
+            device_.validate_storage(address_);
             device_.zero_fill(address_, bytes_);
         } catch (...) {
             device_.release(address_);
@@ -321,7 +505,7 @@ public:
             : RawWorkspace(device, bytes), device_(device) {
         if (bytes != 0) address_ = device_.allocate(bytes);
     }
-    ~Mi355xWorkspace() noexcept override { device_.release(address_); }
+    ~Mi355xWorkspace() noexcept override { device_.release_workspace(this, address_, byte_size()); }
 
 private:
     [[nodiscard]] void* workspace_address() const noexcept override { return address_; }
@@ -339,12 +523,15 @@ public:
             : DeviceOps(device), device_(device),
               registry_queue_id_(detail::allocate_queue_id(device.registry_state())) {
         const std::size_t capacity = device.queue_config().max_in_flight_per_queue;
+        // a lease retained by an earlier queue keeps its place: refused before any native resource
+        device_.admit_queue();
         try {
             check(iomx_set_device(device_.ordinal()), "set device");
             events_.reserve(capacity);
+            free_events_.reserve(capacity);
             for (std::size_t i = 0; i < capacity; ++i) {
                 iomx_event_t event = nullptr;
-                check(iomx_event_create(&event, 0), "completion event");
+                check(counted_event_create(&event), "completion event");
                 events_.push_back(event);
                 free_events_.push_back(event);
             }
@@ -354,10 +541,11 @@ public:
             void* cells = nullptr;
             check(iomx_host_alloc(&cells, capacity * sizeof(std::uint32_t)), "status cells");
             status_cells_ = static_cast<std::uint32_t*>(cells);
-            check(iomx_stream_create(&stream_), "queue stream");
+            check(counted_stream_create(&stream_), "queue stream");
             completer_ = std::thread([this] { run_completer(); });
         } catch (...) {
             destroy_native();
+            device_.retire_queue();
             throw;
         }
     }
@@ -374,19 +562,45 @@ public:
         if (completer_.joinable()) completer_.join();
         close_and_drain();
         (void)iomx_set_device(device_.ordinal());
-        if (stream_ != nullptr) (void)iomx_stream_synchronize(stream_);
-        destroy_native();
+        // The final proof that nothing of this queue still runs.  Without it nothing native is
+        // destroyed or reused: the whole lease moves to the device, keeps its place among the
+        // four queues, and ends at a later proof on the same stream or with the device.
+        const bool proved = stream_ == nullptr
+                || (!consume_submission_fault(SubmissionFault::stream_synchronize)
+                    && iomx_stream_synchronize(stream_) == IOMX_OK);
+        if (proved) {
+            destroy_native();
+        } else {
+            Mi355xDevice::QueueLease lease;
+            lease.stream = stream_;
+            lease.events = std::move(events_);
+            lease.status_cells = status_cells_;
+            stream_ = nullptr;
+            events_.clear();
+            free_events_.clear();
+            status_cells_ = nullptr;
+            device_.retain_unknown_lease(std::move(lease));
+        }
+        device_.retire_queue();
         device_.registry_state().registry.invalidate_entries_for_queue(registry_queue_id_);
+    }
+
+    void snapshot(rocm_detail::QueueResourceSnapshot& out) {
+        std::lock_guard<std::mutex> lock(mutex_);
+        out.events_total = events_.size();
+        out.events_in_use = events_.size() - free_events_.size();
+        out.operations_in_flight = in_flight_.size() + (completing_ ? 1 : 0);
     }
 
     [[nodiscard]] std::string_view backend_label() const noexcept override { return "MI355X"; }
 
 private:
-    using Finish = std::function<void(bool failed)>;
+    // What completion does with the operation's registry entries and workspace lease.
+    using Finish = InlineFunction<void(bool failed), 160>;
 
     // After native completion: turns a data error the kernel reported into the
     // operation's retained failure (null = none).
-    using Verify = std::function<std::exception_ptr(const std::uint32_t& status)>;
+    using Verify = std::exception_ptr (*)(std::uint32_t status);
 
     struct InFlight {
         std::uint64_t sequence = 0;
@@ -394,7 +608,7 @@ private:
         std::uint32_t* status = nullptr;
         std::exception_ptr failure;
         Finish finish;
-        Verify verify;
+        Verify verify = nullptr;
     };
 
     static detail::FenceResult fence_pending(const detail::Fence&) noexcept {
@@ -407,10 +621,10 @@ private:
     }
 
     void destroy_native() noexcept {
-        for (iomx_event_t event : events_) (void)iomx_event_destroy(event);
+        for (iomx_event_t event : events_) counted_event_destroy(event);
         events_.clear();
         free_events_.clear();
-        if (stream_ != nullptr) (void)iomx_stream_destroy(stream_);
+        counted_stream_destroy(stream_);
         stream_ = nullptr;
         if (status_cells_ != nullptr) (void)iomx_host_free(status_cells_);
         status_cells_ = nullptr;
@@ -426,7 +640,11 @@ private:
     // record the completion event, hand the rest to the completion thread.
     // Throws only before anything was launched.
     template <typename Launch>
-    void start(std::uint64_t sequence, Launch&& launch, Finish finish, Verify verify = {}) {
+    void start(std::uint64_t sequence, Launch&& launch, Finish finish, Verify verify = nullptr) {
+        // a completion resource that cannot be had is a failure before acceptance: the common
+        // layer rolls the request back and reports a device error (OID -5)
+        if (consume_submission_fault(SubmissionFault::event_create))
+            throw std::runtime_error("MI355X completion resource is unavailable (injected)");
         iomx_event_t event = nullptr;
         {
             std::lock_guard<std::mutex> lock(mutex_);
@@ -438,45 +656,98 @@ private:
         InFlight item;
         item.sequence = sequence;
         item.event = event;
-        item.finish = std::move(finish);
-        item.verify = std::move(verify);
+        item.finish = finish;
+        item.verify = verify;
         item.status = status_cell(event);
         int status = iomx_set_device(device_.ordinal());
         if (status == IOMX_OK) {
-            if constexpr (std::is_invocable_v<Launch&, iomx_stream_t, std::uint32_t*>)
+            if (consume_submission_fault(SubmissionFault::kernel_launch))
+                status = kInjectedDeviceError;      // the launch is not made
+            else if constexpr (std::is_invocable_v<Launch&, iomx_stream_t, std::uint32_t*>)
                 status = launch(stream_, item.status);
             else
                 status = launch(stream_);
         }
-        if (status == IOMX_OK) status = iomx_event_record(event, stream_);
+        if (status == IOMX_OK) {
+            status = consume_submission_fault(SubmissionFault::event_record)
+                    ? kInjectedDeviceError : iomx_event_record(event, stream_);
+        }
         if (status != IOMX_OK) {
             try { throw_status(status, "MI355X kernel submission"); }
             catch (...) { item.failure = std::current_exception(); }
         }
+        bool wake = false;
         {
             std::lock_guard<std::mutex> lock(mutex_);
             in_flight_.push_back(std::move(item));
+            pending_.store(in_flight_.size(), std::memory_order_release);
+            wake = completer_sleeping_;
         }
-        cv_.notify_all();
+        if (wake) cv_.notify_one();
+    }
+
+    static void relax() noexcept {
+#if defined(__x86_64__) || defined(__i386__)
+        __builtin_ia32_pause();
+#endif
+    }
+
+    // The next launched operation, in submission order.  The completion thread polls for a
+    // short while before it sleeps: a session that submits one operation, waits and submits the
+    // next (src/session.cpp:2000-2045) then never pays a thread wake-up per operation.
+    bool next_in_flight(InFlight& item) {
+        const auto give_up = std::chrono::steady_clock::now() + std::chrono::microseconds(150);
+        for (unsigned spins = 0;; ++spins) {
+            if (pending_.load(std::memory_order_acquire) != 0) {
+                std::lock_guard<std::mutex> lock(mutex_);
+                if (!in_flight_.empty()) {
+                    item = std::move(in_flight_.front());
+                    in_flight_.pop_front();
+                    pending_.store(in_flight_.size(), std::memory_order_release);
+                    completing_ = true;
+                    return true;
+                }
+            }
+            if ((spins & 63u) == 63u && std::chrono::steady_clock::now() > give_up) break;
+            relax();
+        }
+        std::unique_lock<std::mutex> lock(mutex_);
+        completer_sleeping_ = true;
+        cv_.wait(lock, [this] { return shutdown_ || !in_flight_.empty(); });
+        completer_sleeping_ = false;
+        if (in_flight_.empty()) return false;
+        item = std::move(in_flight_.front());
+        in_flight_.pop_front();
+        pending_.store(in_flight_.size(), std::memory_order_release);
+        completing_ = true;
+        return true;
+    }
+
+    // Completion of one event: polled while the kernel is short, then a blocking wait.
+    [[nodiscard]] static int await_event(iomx_event_t event) noexcept {
+        const auto give_up = std::chrono::steady_clock::now() + std::chrono::microseconds(300);
+        for (unsigned spins = 0;; ++spins) {
+            int done = 0;
+            const int status = iomx_event_query(event, &done);
+            if (status != IOMX_OK) return status;
+            if (done) return IOMX_OK;
+            if ((spins & 15u) == 15u && std::chrono::steady_clock::now() > give_up) break;
+            relax();
+        }
+        return iomx_event_synchronize(event);
     }
 
     void run_completer() noexcept {
         (void)iomx_set_device(device_.ordinal());
         for (;;) {
             InFlight item;
-            {
-                std::unique_lock<std::mutex> lock(mutex_);
-                cv_.wait(lock, [this] { return shutdown_ || !in_flight_.empty(); });
-                if (in_flight_.empty()) return;
-                item = std::move(in_flight_.front());
-                in_flight_.pop_front();
-            }
+            if (!next_in_flight(item)) return;
             if (!item.failure) {
-                const int status = iomx_event_synchronize(item.event);
+                const int status = await_event(item.event);
                 if (status != IOMX_OK) {
                     try { throw_status(status, "MI355X kernel completion"); }
                     catch (...) { item.failure = std::current_exception(); }
-                } else if (item.verify) {
+                } else if (item.verify != nullptr) {
                     // a native failure takes precedence over the status word
                     item.failure = item.verify(*item.status);
                 }
@@ -487,6 +758,7 @@ private:
             {
                 std::lock_guard<std::mutex> lock(mutex_);
                 free_events_.push_back(item.event);
+                completing_ = false;
             }
             try { if (item.finish) item.finish(static_cast<bool>(item.failure)); } catch (...) {}
             try { complete(item.sequence, std::move(item.failure)); } catch (...) {}
@@ -645,9 +917,18 @@ private:
                                   const iomx_view w = view_of(captured.w);
                                   const iomx_view out = view_of(captured.out);
                                   const bool planar = captured.layout == LinearOutputLayout::head_planar;
-                                  return iomx_launch_linear(code, &x, &w, &out, captured.start_row,
-                                                            captured.rows, planar ? 1 : 0, captured.heads,
-                                                            captured.head_dim, 0, stream);
+                                  const int status = iomx_launch_linear(
+                                          code, &x, &w, &out, captured.start_row, captured.rows,
+                                          planar ? 1 : 0, captured.heads, captured.head_dim, 0, stream);
+                                  iomx_launch_info info{};
+                                  if (status == IOMX_OK && iomx_last_launch(&info) == IOMX_OK) {
+                                      const std::string_view kernel(info.kernel);
+                                      if (kernel.rfind("linear_mfma", 0) == 0)
+                                          rocm_detail::linear_native_bf16_launch_count_for_testing.fetch_add(1);
+                                      else
+                                          rocm_detail::linear_scalar_launch_count_for_testing.fetch_add(1);
+                                  }
+                                  return status;
                               },
                               [&state, entries, lease](bool failed) {
                                   (void)detail::release_or_invalidate_binary_entries(
@@ -699,6 +980,8 @@ private:
                                   const iomx_view k = snapshot_view(captured.k);
                                   const iomx_view v = snapshot_view(captured.v);
                                   const iomx_view out = snapshot_view(captured.out);
+                                  if (consume_submission_fault(SubmissionFault::sdpa_launch))
+                                      return kInjectedDeviceError;
                                   // the library picks the kernel from the shapes, as its
                                   // workspace query did (a decode step and wide heads use none)
                                   return iomx_launch_sdpa(IOMX_DT_BF16, &q, &k, &v, &out, captured.a,
@@ -836,7 +1119,9 @@ private:
                                   int status = iomx_launch_embedding(code, index_code, &table, &indices,
                                                                      &out, control, stream);
                                   if (status == IOMX_OK)
-                                      status = iomx_memcpy_d2h_async(cell, control, sizeof(*cell), stream);
+                                      status = consume_submission_fault(SubmissionFault::embedding_status_copy)
+                                              ? kInjectedDeviceError
+                                              : iomx_memcpy_d2h_async(cell, control, sizeof(*cell), stream);
                                   return status;
                               },
                               [&state, entries, lease](bool failed) {
@@ -844,7 +1129,7 @@ private:
                                           state.registry, entries, failed, true);
                                   detail::complete_workspace_lease(state, lease, true);
                               },
-                              [](const std::uint32_t& status) -> std::exception_ptr {
+                              [](std::uint32_t status) -> std::exception_ptr {
                                   if (status == 0) return nullptr;
                                   return std::make_exception_ptr(std::invalid_argument(
                                           "MI355X embedding index is negative or out of range"));
@@ -882,6 +1167,9 @@ private:
                                   };
                                   const iomx_view x = view_of(captured.x);
                                   const iomx_view y = view_of(captured.y);
+                                  if (consume_submission_fault(SubmissionFault::silu_launch))
+                                      return kInjectedDeviceError;     // never reaches the kernel
+                                  rocm_detail::silu_launch_count_for_testing.fetch_add(1);
                                   return iomx_launch_silu(code, &x, &y, stream);
                               },
                               [&registry, entries](bool failed) {
@@ -906,6 +1194,9 @@ private:
     std::condition_variable cv_;
     std::vector<iomx_event_t> free_events_;
     std::deque<InFlight> in_flight_;
+    std::atomic<std::size_t> pending_{0};   // in_flight_.size(), readable without the lock
+    bool completer_sleeping_ = false;
+    bool completing_ = false;
     bool shutdown_ = false;
     std::thread completer_;
 };
@@ -923,6 +1214,24 @@ std::unique_ptr<DeviceOps> Mi355xDevice::create_ops() {
 }
 
 }  // namespace
+
+namespace rocm_detail {
+void queue_resource_snapshot_for_testing(DeviceOps& queue, QueueResourceSnapshot& snapshot) {
+    auto* mine = dynamic_cast<Mi355xQueue*>(&queue);
+    if (mine == nullptr) throw std::invalid_argument("not an MI355X queue");
+    mine->snapshot(snapshot);
+}
+std::size_t retained_queue_lease_count_for_testing(Device& device) {
+    auto* mine = dynamic_cast<Mi355xDevice*>(&device);
+    if (mine == nullptr) throw std::invalid_argument("not an MI355X device");
+    return mine->retained_lease_count();
+}
+void reclaim_retained_queue_leases_for_testing(Device& device) {
+    auto* mine = dynamic_cast<Mi355xDevice*>(&device);
+    if (mine == nullptr) throw std::invalid_argument("not an MI355X device");
+    mine->reclaim_retained_leases();
+}
+}  // namespace rocm_detail
 
 // include/iom/rocm/device.hpp:22-24.  Configuration errors are reported before
 // any native effect (include/iom/detail/gpu_arena_config.hpp:18-53).

@@ -36,6 +36,7 @@
 #endif
 #ifdef IOMC_WITH_MI355X
 #include "iom/rocm/device.hpp"
+#include "../iom_amd/host/mi355x_testing.hpp"  // fault injection and resource counters
 #endif
 
 namespace {
@@ -95,6 +96,9 @@ struct iomc_view {
 };
 struct iomc_queue {
     std::unique_ptr<iom::DeviceOps> ops;
+};
+struct iomc_workspace {
+    std::unique_ptr<iom::RawWorkspace> workspace;
 };
 
 namespace {
@@ -472,5 +476,105 @@ int iomc_sdpa_matches(std::uint16_t actual, std::uint16_t expected_bits, std::ui
 int iomc_wait(iomc_queue* queue, std::int64_t token) {
     return guarded_status([&] { queue->ops->wait(token); });
 }
+
+// ---- submissions that do not wait, with the workspace owned by the caller ---------------
+// (what the conformance drivers do when they test lifetimes: drop an owner while its
+// operation is still in flight, test/rocm/test_rocm_conformance.cpp)
+
+iomc_workspace* iomc_workspace_create(iomc_device* device, std::size_t bytes) {
+    return guarded([&]() -> iomc_workspace* {
+        auto holder = std::make_unique<iomc_workspace>();
+        holder->workspace = device->device->create_workspace(bytes);
+        return holder.release();
+    }, nullptr);
+}
+
+void iomc_workspace_destroy(iomc_workspace* workspace) { delete workspace; }
+
+std::int64_t iomc_sdpa_workspace_bytes(
+        iomc_queue* queue, const iomc_view* q, const iomc_view* k, const iomc_view* v,
+        const iomc_view* out, std::size_t a, std::size_t L) {
+    try {
+        return static_cast<std::int64_t>(queue->ops->sdpa_workspace_requirements(
+                q->view, k->view, v->view, out->view, a, L).bytes);
+    } catch (...) {
+        return classify(std::current_exception());
+    }
+}
+
+std::int64_t iomc_sdpa_submit(
+        iomc_queue* queue, const iomc_view* q, const iomc_view* k, const iomc_view* v,
+        iomc_view* out, std::size_t a, std::size_t L, iomc_workspace* workspace) {
+    if (workspace == nullptr) return queue->ops->sdpa(q->view, k->view, v->view, out->view, a, L);
+    return queue->ops->sdpa(q->view, k->view, v->view, out->view, a, L, workspace->workspace->view());
+}
+
+std::int64_t iomc_embedding_submit(
+        iomc_queue* queue, const iomc_view* table, const iomc_view* indices, iomc_view* out,
+        iomc_workspace* workspace) {
+    if (workspace == nullptr) return queue->ops->embedding(table->view, indices->view, out->view);
+    return queue->ops->embedding(table->view, indices->view, out->view, workspace->workspace->view());
+}
+
+std::int64_t iomc_embedding_workspace_bytes(
+        iomc_queue* queue, const iomc_view* table, const iomc_view* indices, const iomc_view* out) {
+    try {
+        return static_cast<std::int64_t>(queue->ops->embedding_workspace_requirements(
+                table->view, indices->view, out->view).bytes);
+    } catch (...) {
+        return classify(std::current_exception());
+    }
+}
+
+#ifdef IOMC_WITH_MI355X
+// ---- the MI355X backend's test seams (iom_amd/host/mi355x_testing.hpp) -------------------
+
+// fault: numeric value of iom::rocm_detail::SubmissionFault
+void iomc_inject_fault(int fault) {
+    iom::rocm_detail::inject_submission_fault_for_testing(
+            static_cast<iom::rocm_detail::SubmissionFault>(fault));
+}
+
+// which: 0 event create, 1 event destroy, 2 stream create, 3 stream destroy, 4 device
+// allocations, 5 device frees, 6 native BF16 linear launches, 7 scalar linear launches, 8 SiLU launches
+std::uint64_t iomc_test_counter(int which) {
+    using namespace iom::rocm_detail;
+    switch (which) {
+        case 0: return event_create_count_for_testing.load();
+        case 1: return event_destroy_count_for_testing.load();
+        case 2: return stream_create_count_for_testing.load();
+        case 3: return stream_destroy_count_for_testing.load();
+        case 4: return device_allocation_count_for_testing.load();
+        case 5: return device_free_count_for_testing.load();
+        case 6: return linear_native_bf16_launch_count_for_testing.load();
+        case 7: return linear_scalar_launch_count_for_testing.load();
+        case 8: return silu_launch_count_for_testing.load();
+        default: return ~std::uint64_t{0};
+    }
+}
+
+int iomc_queue_snapshot(iomc_queue* queue, std::uint64_t* out3) {
+    return guarded_status([&] {
+        iom::rocm_detail::QueueResourceSnapshot snapshot;
+        iom::rocm_detail::queue_resource_snapshot_for_testing(*queue->ops, snapshot);
+        out3[0] = snapshot.events_total;
+        out3[1] = snapshot.events_in_use;
+        out3[2] = snapshot.operations_in_flight;
+    });
+}
+
+std::int64_t iomc_retained_leases(iomc_device* device) {
+    return guarded([&]() -> std::int64_t {
+        return static_cast<std::int64_t>(
+                iom::rocm_detail::retained_queue_lease_count_for_testing(*device->device));
+    }, std::int64_t{-1});
+}
+
+void iomc_reclaim_leases(iomc_device* device) {
+    (void)guarded_status([&] {
+        iom::rocm_detail::reclaim_retained_queue_leases_for_testing(*device->device);
+    });
+}
+#endif  // IOMC_WITH_MI355X
 
 }  // extern "C"

@@ -472,7 +472,36 @@ def bind_iomc(l: C.CDLL) -> C.CDLL:
     l.iomc_rope.argtypes = [P, P, P, C.c_size_t, C.c_double]
     l.iomc_embedding.restype = C.c_int64
     l.iomc_embedding.argtypes = [P, P, P, P, P, C.POINTER(C.c_int)]
+    l.iomc_workspace_create.restype = P
+    l.iomc_workspace_create.argtypes = [P, C.c_size_t]
+    l.iomc_workspace_destroy.argtypes = [P]
+    l.iomc_sdpa_workspace_bytes.restype = C.c_int64
+    l.iomc_sdpa_workspace_bytes.argtypes = [P, P, P, P, P, C.c_size_t, C.c_size_t]
+    l.iomc_sdpa_submit.restype = C.c_int64
+    l.iomc_sdpa_submit.argtypes = [P, P, P, P, P, C.c_size_t, C.c_size_t, P]
+    l.iomc_embedding_submit.restype = C.c_int64
+    l.iomc_embedding_submit.argtypes = [P, P, P, P, P]
+    l.iomc_embedding_workspace_bytes.restype = C.c_int64
+    l.iomc_embedding_workspace_bytes.argtypes = [P, P, P, P]
+    if hasattr(l, "iomc_inject_fault"):
+        l.iomc_inject_fault.argtypes = [C.c_int]
+        l.iomc_inject_fault.restype = None
+        l.iomc_test_counter.restype = C.c_uint64
+        l.iomc_test_counter.argtypes = [C.c_int]
+        l.iomc_queue_snapshot.argtypes = [P, U64P]
+        l.iomc_retained_leases.restype = C.c_int64
+        l.iomc_retained_leases.argtypes = [P]
+        l.iomc_reclaim_leases.argtypes = [P]
+        l.iomc_reclaim_leases.restype = None
     return l
+
+
+# numeric values of iom::rocm_detail::SubmissionFault (iom_amd/host/mi355x_testing.hpp)
+(FAULT_NONE, FAULT_EVENT_CREATE, FAULT_QUEUE_EVENT_CREATE, FAULT_QUEUE_STREAM_CREATE,
+ FAULT_KERNEL_LAUNCH, FAULT_EMBEDDING_STATUS_COPY, FAULT_EVENT_RECORD, FAULT_STREAM_SYNCHRONIZE,
+ FAULT_SILU_LAUNCH, FAULT_SDPA_LAUNCH) = range(10)
+(COUNT_EVENT_CREATE, COUNT_EVENT_DESTROY, COUNT_STREAM_CREATE, COUNT_STREAM_DESTROY,
+ COUNT_DEVICE_ALLOC, COUNT_DEVICE_FREE, COUNT_LINEAR_NATIVE, COUNT_LINEAR_SCALAR, COUNT_SILU) = range(9)
 
 
 class IomTensor:
@@ -633,6 +662,60 @@ class IomBackend:
 
     def sdpa(self, q, k, v, out, a, L) -> int:
         return self.run(self.l.iomc_sdpa(self.dev, self.queue, q.h, k.h, v.h, out.h, a, L))
+
+    # ---- submissions that do not wait (the caller waits, and owns any workspace) --------
+
+    def submit(self, name: str, *args) -> int:
+        """The oid of iomc_<name>(queue, ...) without waiting for it."""
+        return getattr(self.l, "iomc_" + name)(self.queue, *[getattr(a, "h", a) for a in args])
+
+    def workspace(self, nbytes: int):
+        h = self.l.iomc_workspace_create(self.dev, nbytes)
+        if not h:
+            raise RuntimeError(self.error())
+        return h
+
+    def drop_workspace(self, handle):
+        self.l.iomc_workspace_destroy(handle)
+
+    def sdpa_workspace_bytes(self, q, k, v, out, a, L) -> int:
+        return self.l.iomc_sdpa_workspace_bytes(self.queue, q.h, k.h, v.h, out.h, a, L)
+
+    def sdpa_submit(self, q, k, v, out, a, L, workspace=None) -> int:
+        return self.l.iomc_sdpa_submit(self.queue, q.h, k.h, v.h, out.h, a, L, workspace)
+
+    def embedding_workspace_bytes(self, table, indices, out) -> int:
+        return self.l.iomc_embedding_workspace_bytes(self.queue, table.h, indices.h, out.h)
+
+    def embedding_submit(self, table, indices, out, workspace=None) -> int:
+        return self.l.iomc_embedding_submit(self.queue, table.h, indices.h, out.h, workspace)
+
+    # ---- the MI355X backend's test seams ------------------------------------------------
+
+    def inject(self, fault: int):
+        self.l.iomc_inject_fault(fault)
+
+    def counter(self, which: int) -> int:
+        return int(self.l.iomc_test_counter(which))
+
+    def snapshot(self):
+        """(events_total, events_in_use, operations_in_flight) of this queue."""
+        out = (C.c_uint64 * 3)()
+        rc = self.l.iomc_queue_snapshot(self.queue, out)
+        if rc != 0:
+            raise RuntimeError(self.error())
+        return tuple(int(v) for v in out)
+
+    def retained_leases(self) -> int:
+        return int(self.l.iomc_retained_leases(self.dev))
+
+    def reclaim_leases(self):
+        self.l.iomc_reclaim_leases(self.dev)
+
+    def close_queue(self):
+        if self.queue:
+            self.l.iomc_queue_destroy(self.queue)
+            self.queue = None
 
     def close(self):
         if self.queue:

@@ -38,3 +38,38 @@ def test_cxx_backend_exports_the_factory():
     undefined = subprocess.check_output(["nm", "-D", "--undefined-only", path]).decode()
     assert "iomx_launch_binary" in undefined
     assert not re.search(r"\bhip[A-Z]", undefined)
+
+
+def test_cxx_backend_links_nothing_of_the_checkers_or_of_the_cpu_backend():
+    """The product library needs IOM's backend-independent layer (libiom.so, built beside it)
+    and the kernel library, found next to itself; nothing under oracle/, and no symbol of the
+    reference CPU backend."""
+    path = os.path.join(ROOT, "iom_amd", "lib", "libiom_mi355x.so")
+    if not os.path.exists(path):
+        pytest.skip("C++ backend not built (needs the reference headers)")
+    dynamic = subprocess.check_output(["readelf", "-d", path]).decode()
+    needed = re.findall(r"\(NEEDED\)\s+Shared library: \[([^\]]+)\]", dynamic)
+    assert "libiomx.so" in needed and "libiom.so" in needed
+    assert not [n for n in needed if "oracle" in n or "core" in n or "cpu" in n or "ref" in n], needed
+    runpath = re.findall(r"\((?:RUNPATH|RPATH)\)\s+Library (?:runpath|rpath): \[([^\]]*)\]", dynamic)
+    assert runpath == ["$ORIGIN"], runpath
+    undefined = subprocess.check_output(["nm", "-D", "--undefined-only", "-C", path]).decode()
+    assert "iom::cpu" not in undefined and "make_cpu_device" not in undefined
+    # the same holds for the layer it links: IOM's facade, without any backend
+    facade = os.path.join(ROOT, "iom_amd", "lib", "libiom.so")
+    defined = subprocess.check_output(["nm", "-D", "--defined-only", "-C", facade]).decode()
+    assert "iom::DeviceOps::wait" in defined
+    assert "make_cpu_device" not in defined and "iom::cpu" not in defined
+    assert "oracle" not in subprocess.check_output(["readelf", "-d", facade]).decode()
+
+
+def test_cxx_backend_exports_its_test_seams():
+    path = os.path.join(ROOT, "iom_amd", "lib", "libiom_mi355x.so")
+    if not os.path.exists(path):
+        pytest.skip("C++ backend not built (needs the reference headers)")
+    out = subprocess.check_output(["nm", "-D", "--defined-only", "-C", path]).decode()
+    for name in ("iom::rocm_detail::inject_submission_fault_for_testing",
+                 "iom::rocm_detail::queue_resource_snapshot_for_testing",
+                 "iom::rocm_detail::reclaim_retained_queue_leases_for_testing",
+                 "iom::rocm_detail::event_create_count_for_testing"):
+        assert name in out, name
