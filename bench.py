@@ -627,13 +627,119 @@ def cpu_baseline():
     once()
     samples = sorted(once() for _ in range(13))
     med = samples[6]
-    return {
+    result = {
         "value": round(alg / med / 1e9, 5), "unit": "GB/s", "cores": 1, "kind": kind,
         "sample": "broadcast ADD BF16 [8,512,2048]+[1,2048] (1/8 of the GPU workload), "
                   "submit to wait, median of 13 after 1 warm-up",
         "Melem_per_s": round(n / med / 1e6, 3), "seconds_per_run": round(med, 4),
         "host_cpus": os.cpu_count(),
     }
+    if iomo.ref512_available():
+        # the same sample on the reference's opt-in AVX-512 BF16 build (this CPU has the ISA)
+        fast = iomo.ref_backend_avx512()
+        fx, fb, fo = fast.tensor(BF16, dims), fast.tensor(BF16, vdims), fast.tensor(BF16, dims)
+        fx.view().from_host(x)
+        fb.view().from_host(b)
+
+        def once_fast():
+            t0 = time.perf_counter()
+            assert fast.binary(iomo.OP_ADD, fx.view(), fb.view(), fo.view()) > 0
+            return time.perf_counter() - t0
+        once_fast()
+        fmed = sorted(once_fast() for _ in range(13))[6]
+        result["avx512_bf16_build"] = {"value": round(alg / fmed / 1e9, 5), "unit": "GB/s", "cores": 1,
+                                       "kind": "reference, AVX_512_BF16_ENABLED build",
+                                       "Melem_per_s": round(n / fmed / 1e6, 3),
+                                       "seconds_per_run": round(fmed, 5)}
+        fast.close()
+    return result
+
+
+def cpu_baseline_per_config():
+    """The reference CPU backend (one worker thread per queue = 1 core) on a bounded sample of
+    every other configuration: median of 5 after 1 warm-up (test/cpu/test_cpu_bench.cpp:45-83),
+    about a second per row.  Where the reference's AVX-512 BF16 build exists and this CPU has
+    the ISA, the same samples are timed on it and labelled separately.  The softmax stage has no
+    entry of its own in the CPU backend: its row times the CPU restatement (kind "port")."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import iomo
+    if not iomo.ref_available():
+        return []
+    rows = []
+
+    def timed(once):
+        once()
+        samples = sorted(once() for _ in range(5))
+        return samples[2]
+
+    def sample_set(ref, kind):
+        def tensor(dtype, dims, what, salt):
+            t = ref.tensor(dtype, dims)
+            if what is not None:
+                t.view().from_host(synth(dtype, int(np.prod(dims)), what, salt).reshape(dims))
+            return t
+
+        def row(name, sample, alg_bytes, elements, submit):
+            def once():
+                t0 = time.perf_counter()
+                token = submit()
+                assert token > 0, ref.error()
+                return time.perf_counter() - t0
+            med = timed(once)
+            rows.append({"workload": name, "sample": sample, "kind": kind, "cores": 1,
+                         "GB_per_s": round(alg_bytes / med / 1e9, 5),
+                         "Melem_per_s": round(elements / med / 1e6, 3), "seconds_per_run": round(med, 4)})
+
+        for dtype, label, what in ((F32, "add_f32", "uniform_pm1"), (I32, "add_i32", "uniform_i20")):
+            dims = (1024, 1024)
+            a, b, o = tensor(dtype, dims, what, 1), tensor(dtype, dims, what, 2), tensor(dtype, dims, None, 0)
+            n = 1 << 20
+            row(label, "[1024,1024] (1/16 of [4096,4096])", 12 * n, n,
+                lambda: ref.binary(iomo.OP_ADD, a.view(), b.view(), o.view()))
+            for t in (a, b, o):
+                t.close()
+        dims, n = (2, 512, 2048), 2 * 512 * 2048
+        x, v, o = tensor(BF16, dims, "normal", 11), tensor(BF16, (1, 2048), "normal_0p02", 23), tensor(BF16, dims, None, 0)
+        row("bcast_mul_bf16", "[2,512,2048]*[1,2048] (1/32)", 4 * n + 4096, n,
+            lambda: ref.binary(iomo.OP_MUL, x.view(), v.view(), o.view()))
+        for t in (x, v, o):
+            t.close()
+        for dtype, label in ((BF16, "rmsnorm_bf16"), (F32, "rmsnorm_f32")):
+            dims, n, es = (1024, 2048), 1024 * 2048, iomx.leaf_bytes(dtype)
+            x, w, o = tensor(dtype, dims, "normal", 31), tensor(dtype, (1, 2048), "uniform_half_3half", 5), tensor(dtype, dims, None, 0)
+            row(label, "[1024,2048] (1/32 of [32768,2048])", (2 * n + 2048) * es, n,
+                lambda: ref.rmsnorm(x.view(), w.view(), o.view(), 1e-5))
+            for t in (x, w, o):
+                t.close()
+        dims, n = (512, 5632), 512 * 5632
+        g, u, act, prod = (tensor(BF16, dims, "normal", 41), tensor(BF16, dims, "normal", 42),
+                           tensor(BF16, dims, None, 0), tensor(BF16, dims, None, 0))
+        row("silu_bf16", "[512,5632] (1/64 of [32768,5632])", 4 * n, n, lambda: ref.silu(g.view(), act.view()))
+        row("mul_bf16", "[512,5632] (1/64)", 6 * n, n, lambda: ref.binary(iomo.OP_MUL, act.view(), u.view(), prod.view()))
+        for t in (g, u, act, prod):
+            t.close()
+
+    ref = iomo.ref_backend()
+    sample_set(ref, "reference")
+    ref.close()
+    if iomo.ref512_available():
+        ref = iomo.ref_backend_avx512()
+        sample_set(ref, "reference, AVX_512_BF16_ENABLED build")
+        ref.close()
+    # softmax stage: the CPU restatement of src/cpu/sdpa.cpp:214-309 on 512 causal rows of 2048 scores
+    R, Cc = 512, 2048
+    one = datagen.normal_f32(R * Cc, 0.0, 3.0, 61).reshape(1, 1, R, Cc)
+    one[0, 0][np.triu_indices(R, 1, Cc)] = -np.inf
+
+    def once():
+        t0 = time.perf_counter()
+        iomo.softmax(one, Cc - 1, Cc)
+        return time.perf_counter() - t0
+    med = timed(once)
+    rows.append({"workload": "softmax_f32_to_bf16_mask_as_data", "sample": "[1,1,512,2048] (1/8192)",
+                 "kind": "port", "cores": 1, "GB_per_s": round(6 * R * Cc / med / 1e9, 5),
+                 "Melem_per_s": round(R * Cc / med / 1e6, 3), "seconds_per_run": round(med, 4)})
+    return rows
 
 
 def traffic_of(key):
@@ -699,6 +805,7 @@ def main():
         "decoder_layer": lambda: wl_decoder_layer(timer, max(K // 5, 10), max(W // 2, 5)),
         "other_leaves": lambda: wl_other_leaves(timer, max(K // 10, 5), max(W // 10, 2)),
         "hbm_ceiling": lambda: wl_hbm_ceiling(timer, K, W),
+        "cpu_per_config": cpu_baseline_per_config,
     }
 
     if args.only:
@@ -720,6 +827,8 @@ def main():
             r = table[key]()
             detail.extend(r if isinstance(r, list) else [r])
     cpu = None if args.no_cpu else cpu_baseline()
+    if cpu is not None and not args.no_detail:
+        cpu["per_config"] = cpu_baseline_per_config()
 
     line = {
         "metric": "achieved HBM GB/s (% of MI355X peak) for ADD, broadcast ADD, RMSNorm",

@@ -739,6 +739,29 @@ def ref_backend(max_in_flight: int = 16) -> IomBackend:
     return IomBackend(_ref_lib, _ref_lib.iomc_cpu_device_create(max_in_flight))
 
 
+REF512_PATH = os.path.join(HERE, "_ref", "libiom_ref_avx512.so")
+_ref512_lib: Optional[C.CDLL] = None
+
+
+def ref512_available() -> bool:
+    """The reference's opt-in AVX-512 BF16 CPU build (make ref512) and a CPU that has the ISA."""
+    if not os.path.exists(REF512_PATH):
+        return False
+    try:
+        with open("/proc/cpuinfo") as f:
+            return "avx512_bf16" in f.read()
+    except OSError:
+        return False
+
+
+def ref_backend_avx512(max_in_flight: int = 16) -> IomBackend:
+    """The reference CPU backend built with AVX_512_BF16_ENABLED (a timing baseline only)."""
+    global _ref512_lib
+    if _ref512_lib is None:
+        _ref512_lib = bind_iomc(_load(REF512_PATH))
+    return IomBackend(_ref512_lib, _ref512_lib.iomc_cpu_device_create(max_in_flight))
+
+
 MI355X_SHIM_PATH = os.path.join(HERE, "_ref", "libiom_mi355x_shim.so")
 _mi355x_lib: Optional[C.CDLL] = None
 

@@ -215,6 +215,54 @@ def test_config4_softmax_rows_of_2048():
     pb.free()
 
 
+def test_config4_softmax_at_the_full_2_to_the_32_elements():
+    """[32,32,2048,2048]: 2^32 scores (16 GiB), 8 GiB of probabilities, 2,097,152 rows -- the launch
+    the benchmark times.  Every (plane, head) holds the same matrix, so every output matrix must be
+    the first one; the matrices on both sides of the 2^31- and 2^32-element and -byte offsets are
+    downloaded and compared whole, and the oracle checks sampled rows of the LAST matrix, where a
+    32-bit slip in the row or offset arithmetic would show."""
+    planes, heads, R, Cc = 32, 32, 2048, 2048
+    mats = planes * heads
+    one = datagen.normal_f32(R * Cc, 0, 3, 61).reshape(R, Cc)
+    one[np.triu_indices(R, 1, Cc)] = -np.inf
+    n = mats * R * Cc
+    assert n == 1 << 32
+    sb, pb = iomx.Buffer(n * 4), iomx.Buffer(n * 2)
+    sb.upload(one)
+    copied = 1
+    while copied < mats:                                  # doubling device-to-device copies
+        m = min(copied, mats - copied)
+        iomx.check(iomx.lib().iomx_memcpy_d2d_async(sb.ptr.value + copied * one.nbytes, sb.ptr.value,
+                                                   m * one.nbytes, None), "d2d")
+        iomx.synchronize()
+        copied += m
+    assert np.array_equal(sb.download(np.float32, R * Cc, (mats - 1) * one.nbytes).view(np.uint32),
+                          one.reshape(-1).view(np.uint32))
+    upper = np.triu_indices(R, 1, Cc)
+    rows = [0, 1, 15, 16, 17, 255, 1023, 1024, 2046, 2047] + list(range(500, 522))
+    # matrices next to the offsets 2^32 bytes of P (512), 2^32 bytes / 2^30 elements of scores (256),
+    # 2^31 elements (512), and the two ends
+    sampled = [0, 255, 256, 511, 512, 767, 1022, 1023]
+    for a_pos, name in ((Cc - 1, "mask as data"), (0, "positional")):
+        pb.fill(0xAA)
+        d = iomx.softmax_desc(sb.ptr.value, pb.ptr.value, planes, heads, R, Cc, a_pos, Cc)
+        assert iomx.softmax(d) == 0
+        assert iomx.last_launch().kernel.decode() == "softmax_rows"
+        iomx.synchronize()
+        first = pb.download(np.uint16, R * Cc, 0).reshape(R, Cc)
+        assert np.all(first[upper] == 0), name                                  # masked entries are +0
+        p = datagen.bf16_to_f32(first.reshape(-1)).reshape(R, Cc).astype(np.float64)
+        assert np.abs(p.sum(axis=1) - 1.0).max() < 2.0 ** -6                    # rows sum to one
+        for m in sampled[1:]:
+            got = pb.download(np.uint16, R * Cc, m * R * Cc * 2).reshape(R, Cc)
+            assert np.array_equal(got, first), (name, m)
+        last = pb.download(np.uint16, R * Cc, (mats - 1) * R * Cc * 2).reshape(R, Cc)
+        want = iomo.softmax(one[rows].reshape(1, 1, len(rows), Cc), a=Cc - 1, L=Cc)[0, 0]
+        assert np.abs(last[rows].astype(np.int64) - want.astype(np.int64)).max() <= 1, name
+    sb.free()
+    pb.free()
+
+
 def silu64(x):
     with np.errstate(all="ignore"):
         return x / (1.0 + np.exp(-x))
@@ -409,7 +457,11 @@ def test_attention_full_size_by_uniform_scores_and_sampled_rows():
         budget = 2.0 ** -8 * (np.cumsum(np.abs(vv), axis=0) * p[:, None]) + 2.0 ** -8 * np.abs(want) + 2.0 ** -20
         g = datagen.bf16_to_f32(got[b, :, h * D:(h + 1) * D].reshape(-1)).astype(np.float64).reshape(R, D)
         assert (np.abs(g - want) <= budget).all()
-    # sampled rows against the oracle: a one-row attention at position r over r+1 tokens
+    # sampled rows against the oracle (a one-row attention at position r over r+1 tokens): both
+    # sit inside the float64 budget of the BF16 probability on EVERY element, hence within twice
+    # that budget of each other; how many pairs also miss the reference's fixture rule (2 BF16
+    # steps or 2^-10, which is not a bound under cancellation) is printed, not asserted
+    from test_gpu_sdpa import float64_attention
     from test_oracle_sdpa import bf16_class, matches
     for b, r in ((0, 0), (2, 17), (5, 255), (7, 511)):
         hq = iomo.HostTensor(DT_BF16, (Hq, 1, D)); hq.view().from_logical(q[b, :, r:r + 1])
@@ -418,7 +470,13 @@ def test_attention_full_size_by_uniform_scores_and_sampled_rows():
         ho = iomo.HostTensor(DT_BF16, (1, Hq * D))
         assert iomo.sdpa(hq.view(), hk.view(), hv.view(), ho.view(), r, r + 1) == 0
         want = ho.view().to_logical().reshape(-1)
-        bad = [i for i, (g, w) in enumerate(zip(got[b, r], want)) if not matches(int(g), int(w), bf16_class(int(w)))]
-        assert len(bad) <= 2, (b, r, bad[:5])          # the fixture rule is not a cancellation bound
-    for t in (dq, dk, dv, do, ws):
-        t.free()
+        case = {"leading": [], "Hq": Hq, "Hkv": Hkv, "R": 1, "D": D, "C": R, "a": r, "L": r + 1,
+                "q": q[b, :, r:r + 1].reshape(-1), "k": k[b].reshape(-1), "v": v[b].reshape(-1)}
+        ref64, budget = float64_attention(case)
+        g = datagen.bf16_to_f32(got[b, r]).astype(np.float64).reshape(ref64.shape)
+        w = datagen.bf16_to_f32(want).astype(np.float64).reshape(ref64.shape)
+        assert np.all(np.abs(g - ref64) <= budget), (b, r)
+        assert np.all(np.abs(w - ref64) <= budget), (b, r)
+        assert np.all(np.abs(g - w) <= 2 * budget), (b, r)
+        outside = [i for i, (x, y) in enumerate(zip(got[b, r], want)) if not matches(int(x), int(y), bf16_class(int(y)))]
+        print(f"  attention row (b={b}, r={r}): {len(outside)} of {want.size} outside the fixture rule", flush=True)
