@@ -33,7 +33,7 @@ from iom_amd import iomx  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 BF16, F32, I32 = iomx.DT_BF16, iomx.DT_F32, iomx.DT_I32
-ADD, MUL = iomx.OP_ADD, iomx.OP_MUL
+ADD, MUL, DIV = iomx.OP_ADD, iomx.OP_MUL, iomx.OP_DIV
 BASE = 1 << 22  # elements of the seeded base pattern that is repeated over big tensors
 
 
@@ -791,6 +791,10 @@ def main():
                                             hd, (1, 2048), ("normal", "normal_0p02")),
         "bcast_mul_bf16": lambda: wl_binary(timer, K, W, "bcast_mul_bf16_[64,512,2048]*[1,2048]", BF16, MUL,
                                             hd, (1, 2048), ("normal", "normal_0p02")),
+        "bcast_div_bf16": lambda: wl_binary(timer, K, W, "bcast_div_bf16_[64,512,2048]/[1,2048]", BF16, DIV,
+                                            hd, (1, 2048), ("normal", "normal_0p02")),
+        "div_f32": lambda: wl_binary(timer, K, W, "div_f32_[4096,4096]", F32, DIV, (4096, 4096),
+                                     (4096, 4096), ("uniform_pm1", "uniform_pm1")),
         "bcast_add_bf16_sliced": lambda: wl_binary(
             timer, K, W, "bcast_add_bf16_lhs=slice(0,0,64,2)of[128,512,2048]", BF16, ADD, hd, (1, 2048),
             ("normal", "normal_0p02"), lhs_view=((128, 512, 2048), lambda v: v.slice(0, 0, 64, 2))),
@@ -835,7 +839,7 @@ def main():
     ceiling = wl_hbm_ceiling(timer, K, W, sizes_mib=(128,), modes=("copy",))[0]
     detail = []
     if not args.no_detail:
-        for key in ("bcast_mul_bf16", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "copy_bf16", "add_f32",
+        for key in ("bcast_mul_bf16", "bcast_div_bf16", "div_f32", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "copy_bf16", "add_f32",
                     "add_i32", "rmsnorm_bf16", "rmsnorm_f32", "silu_mul", "softmax", "softmax_causal",
                     "chain", "layer_ops", "linear", "sdpa", "decoder_layer", "hbm_ceiling"):
             r = table[key]()

@@ -58,7 +58,7 @@ enum {
 };
 
 /* Order of BinaryOp in src/shared/scalar_binary_codec.hpp:9. */
-enum { IOMX_OP_ADD = 0, IOMX_OP_MUL = 1, IOMX_OP_SUB = 2 };
+enum { IOMX_OP_ADD = 0, IOMX_OP_MUL = 1, IOMX_OP_SUB = 2, IOMX_OP_DIV = 3 };
 
 /*
  * One operand: what DeviceOps::BinaryViewSnapshot / CopyViewSnapshot carry
@@ -148,6 +148,9 @@ int iomx_graph_destroy(iomx_graph_t graph);
  * DeviceOps::binary_impl (include/iom/iom.hpp:846-956); element rule of
  * src/shared/scalar_binary_codec.hpp:120-178 over the 21 numeric leaves
  * (src/device_ops_binary.cpp:26-46; BOOL and F8_E8M0 are IOMX_ERR_UNSUPPORTED).
+ * IOMX_OP_DIV takes the nine floating leaves only (src/device_ops_binary.cpp:174-175):
+ * a zero or an infinity divided by its like is NaN, any other division by zero is
+ * the signed overflow value of the leaf.
  * Integers wrap modulo 2^width.  Floating leaves are one IEEE operation with
  * one round-to-nearest-even encode and gradual underflow; overflow gives
  * infinity where the leaf has one and the largest finite magnitude otherwise
@@ -395,7 +398,7 @@ int iomx_selftest_bf16_convert(uint64_t* mismatches, iomx_stream_t stream);
 
 /* Compares the packed F16 arithmetic of the streaming kernels (hardware F16 <->
  * binary32 conversions around one binary32 operation) with the integer-rounded
- * binary64 rule for all 2^32 operand pairs and ADD, MUL, SUB; *mismatches receives
+ * binary64 rule for all 2^32 operand pairs and ADD, MUL, SUB, DIV; *mismatches receives
  * the count. */
 int iomx_selftest_f16_binary(uint64_t* mismatches, iomx_stream_t stream);
 

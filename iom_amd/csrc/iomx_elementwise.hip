@@ -24,9 +24,22 @@ namespace iomx {
 // a [.,R,1] column vector, a [.,1,1] scalar (the last two on the padded kernel only).
 enum { MODE_FULL = 0, MODE_ROWVEC = 1, MODE_COLVEC = 2, MODE_SCALAR = 3 };
 
-// Internal operation codes: the three public binary operations keep their ABI
+// Internal operation codes: the four public binary operations keep their ABI
 // values; the rest are private to this file.
-enum { OP_SILU_MUL = 3, OP_SILU = 4, OP_COPY = 5 };
+enum { OP_SILU = 4, OP_COPY = 5, OP_SILU_MUL = 6 };
+
+// The binary operations that broadcast (everything else takes whole planes only).
+constexpr bool is_arithmetic(int op) { return op >= IOMX_OP_ADD && op <= IOMX_OP_DIV; }
+
+// One IEEE operation in the carrier T.  Division needs no special cases beside
+// IEEE's own: 0/0 and inf/inf are NaN, x/0 is a signed infinity, x/inf a signed zero.
+template <int OP, typename T>
+__device__ __forceinline__ T arith(T x, T y) {
+    if constexpr (OP == IOMX_OP_ADD) return x + y;
+    else if constexpr (OP == IOMX_OP_MUL) return x * y;
+    else if constexpr (OP == IOMX_OP_SUB) return x - y;
+    else return x / y;
+}
 
 template <int OP>
 struct Arity { static constexpr int kInputs = (OP == OP_SILU || OP == OP_COPY) ? 1 : 2; };
@@ -140,30 +153,20 @@ __device__ __forceinline__ uint32_t op_word(uint32_t a, uint32_t b) {
             return r;
         }
     } else if constexpr (DT == IOMX_DT_F32) {
-        const float x = as_f32(a), y = as_f32(b);
-        float r;
-        if constexpr (OP == IOMX_OP_ADD) r = x + y;
-        else if constexpr (OP == IOMX_OP_MUL) r = x * y;
-        else r = x - y;
-        return as_u32(canonical(r));
+        return as_u32(canonical(arith<OP>(as_f32(a), as_f32(b))));
     } else if constexpr (DT == IOMX_DT_F16) {
+        // a binary32 quotient of two F16 values narrows with one rounding as well:
+        // 24 significand bits are the 2*11 + 2 that make the second rounding harmless
         const f32x2 x = f16_pair(a), y = f16_pair(b);
-        f32x2 r;
-        if constexpr (OP == IOMX_OP_ADD) r = x + y;
-        else if constexpr (OP == IOMX_OP_MUL) r = x * y;
-        else r = x - y;
-        return pack_f16(r.x, r.y);
+        return pack_f16(arith<OP>(x.x, y.x), arith<OP>(x.y, y.y));
     } else {
         // BF16 pair.  The binary32 result of one operation on two BF16 values
         // is exact or correctly rounded with enough guard bits that the single
         // narrowing below is the only rounding that matters; binary32
-        // subnormals are kept, so tiny products round once as well.
-        const float xl = bf16_lo(a), yl = bf16_lo(b), xh = bf16_hi(a), yh = bf16_hi(b);
-        float rl, rh;
-        if constexpr (OP == IOMX_OP_ADD) { rl = xl + yl; rh = xh + yh; }
-        else if constexpr (OP == IOMX_OP_MUL) { rl = xl * yl; rh = xh * yh; }
-        else { rl = xl - yl; rh = xh - yh; }
-        return pack_bf16(rl, rh);
+        // subnormals are kept, so tiny products and quotients round once as well
+        // (a quotient is correctly rounded to 24 >= 2*8 + 2 bits; in the binary32
+        // subnormal range the BF16 grid is coarser by the same 16 bits).
+        return pack_bf16(arith<OP>(bf16_lo(a), bf16_lo(b)), arith<OP>(bf16_hi(a), bf16_hi(b)));
     }
 }
 
@@ -183,9 +186,7 @@ __device__ __forceinline__ uint64_t op_wide(uint64_t a, uint64_t b) {
         else if constexpr (OP == OP_SILU_MUL) {
             const double act = silu_carrier(x);
             r = ((act != act) ? as_f64(kQuietNanF64) : act) * y;
-        } else if constexpr (OP == IOMX_OP_ADD) r = x + y;
-        else if constexpr (OP == IOMX_OP_MUL) r = x * y;
-        else r = x - y;
+        } else r = arith<OP>(x, y);
         return (r != r) ? kQuietNanF64 : as_u64(r);
     }
 }
@@ -478,7 +479,7 @@ __global__ __launch_bounds__(kBlock) void elementwise_general_kernel(const Gener
 
 // Self test: the packed F16 arithmetic of the streaming kernels (hardware
 // conversions around one binary32 operation) against the integer-rounded binary64
-// rule of the tile-row kernels, for every pair of binary16 encodings and the three
+// rule of the tile-row kernels, for every pair of binary16 encodings and the four
 // operations.
 __global__ __launch_bounds__(256) void f16_binary_selftest_kernel(unsigned long long* mismatches) {
     unsigned long long bad = 0;
@@ -490,12 +491,15 @@ __global__ __launch_bounds__(256) void f16_binary_selftest_kernel(unsigned long 
         const uint32_t add = op_word<IOMX_DT_F16, IOMX_OP_ADD>(wa, wb);
         const uint32_t mul = op_word<IOMX_DT_F16, IOMX_OP_MUL>(wa, wb);
         const uint32_t sub = op_word<IOMX_DT_F16, IOMX_OP_SUB>(wa, wb);
+        const uint32_t div = op_word<IOMX_DT_F16, IOMX_OP_DIV>(wa, wb);
         bad += (add & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_ADD>(a0, b0);
         bad += (add >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_ADD>(a1, b1);
         bad += (mul & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_MUL>(a0, b0);
         bad += (mul >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_MUL>(a1, b1);
         bad += (sub & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_SUB>(a0, b0);
         bad += (sub >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_SUB>(a1, b1);
+        bad += (div & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_DIV>(a0, b0);
+        bad += (div >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_DIV>(a1, b1);
     }
     if (bad) atomicAdd(mismatches, bad);
 }
@@ -609,7 +613,7 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
                                dim3(kPlanesBlock), 0, s, pa);                                   \
     } while (0)
         if (lm == MODE_FULL && rm == MODE_FULL) IOMX_PLANES(MODE_FULL, MODE_FULL);
-        else if constexpr (OP <= IOMX_OP_SUB) {
+        else if constexpr (is_arithmetic(OP)) {
             if (lm == MODE_FULL) IOMX_PLANES(MODE_FULL, MODE_ROWVEC);
             else IOMX_PLANES(MODE_ROWVEC, MODE_FULL);
         } else {
@@ -639,6 +643,7 @@ int dispatch(int op, bool planes, int lm, int rm, const BinaryArgs& pa, const Ge
         default: break;
     }
     if constexpr (is_float_class(DT)) {
+        if (op == IOMX_OP_DIV) return launch<DT, IOMX_OP_DIV>(planes, lm, rm, pa, ga, s);
         if (op == OP_SILU) return launch<DT, OP_SILU>(planes, lm, rm, pa, ga, s);
         if (op == OP_SILU_MUL) return launch<DT, OP_SILU_MUL>(planes, lm, rm, pa, ga, s);
     }
@@ -654,7 +659,7 @@ int launch_padded(int lm, int rm, const PaddedArgs& pa, hipStream_t s) {
 #define IOMX_PADDED(LMV, RMV)                                                                  \
     hipLaunchKernelGGL((elementwise_padded_kernel<DT, OP, LMV, RMV>), grid, dim3(kPlanesBlock), 0, s, pa)
     if (lm == MODE_FULL && rm == MODE_FULL) IOMX_PADDED(MODE_FULL, MODE_FULL);
-    else if constexpr (OP <= IOMX_OP_SUB) {
+    else if constexpr (is_arithmetic(OP)) {
         if (lm == MODE_FULL && rm == MODE_ROWVEC) IOMX_PADDED(MODE_FULL, MODE_ROWVEC);
         else if (lm == MODE_FULL && rm == MODE_COLVEC) IOMX_PADDED(MODE_FULL, MODE_COLVEC);
         else if (lm == MODE_FULL && rm == MODE_SCALAR) IOMX_PADDED(MODE_FULL, MODE_SCALAR);
@@ -682,6 +687,7 @@ int dispatch_padded(int op, int lm, int rm, const PaddedArgs& pa, hipStream_t s)
         default: break;
     }
     if constexpr (is_float_class(DT)) {
+        if (op == IOMX_OP_DIV) return launch_padded<DT, IOMX_OP_DIV>(lm, rm, pa, s);
         if (op == OP_SILU) return launch_padded<DT, OP_SILU>(lm, rm, pa, s);
         if (op == OP_SILU_MUL) return launch_padded<DT, OP_SILU_MUL>(lm, rm, pa, s);
     }
@@ -723,6 +729,10 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
         if (alias == ALIAS_NONE || snap[k].broadcasts || !same_window(*v[k], *out))
             return IOMX_ERR_INVALID;
     }
+    // division is defined on the floating leaves only, refused after the shape and alias
+    // checks (src/device_ops_binary.cpp:170-176)
+    if (op == IOMX_OP_DIV && (dtype < IOMX_DT_F4_E2M1 || dtype == IOMX_DT_F8_E8M0))
+        return IOMX_ERR_UNSUPPORTED;
 
     Matrix m[3];
     for (int k = 0; k < 3; ++k) m[k] = matrix_of(*v[k]);
@@ -746,7 +756,7 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
     }
     // the chunk-mapped kernels take at most one operand that is not whole planes
     bool modes_ok = mode[0] == MODE_FULL || mode[1] == MODE_FULL;
-    if (op > IOMX_OP_SUB && (mode[0] != MODE_FULL || mode[1] != MODE_FULL)) modes_ok = false;
+    if (!is_arithmetic(op) && (mode[0] != MODE_FULL || mode[1] != MODE_FULL)) modes_ok = false;
     const bool lean_modes = mode[0] <= MODE_ROWVEC && mode[1] <= MODE_ROWVEC;
     bool planes_ok = modes_ok && lean_modes && no_pad;
 
@@ -943,7 +953,7 @@ int iomx_selftest_f16_binary(uint64_t* mismatches, iomx_stream_t stream) {
 
 int iomx_launch_binary(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs,
                        const iomx_view* out, iomx_stream_t stream) {
-    if (op < IOMX_OP_ADD || op > IOMX_OP_SUB) return IOMX_ERR_INVALID;
+    if (!is_arithmetic(op)) return IOMX_ERR_INVALID;
     if (!rhs) return IOMX_ERR_INVALID;
     return run(op, dtype, lhs, rhs, out, ALIAS_EXACT, stream);
 }

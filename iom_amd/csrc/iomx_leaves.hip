@@ -293,6 +293,7 @@ int dispatch_rows(int op, const RowsArgs& a, dim3 grid, hipStream_t s) {
         default: break;
     }
     if constexpr (is_float_leaf(DT)) {
+        if (op == IOMX_OP_DIV) { launch_rows_kernel<DT, IOMX_OP_DIV>(a, grid, s); return IOMX_OK; }
         if (op == ROWS_OP_SILU) { launch_rows_kernel<DT, ROWS_OP_SILU>(a, grid, s); return IOMX_OK; }
     }
     return IOMX_ERR_UNSUPPORTED;

@@ -19,7 +19,7 @@ struct RowsRequest {
     bool brow[2], bcol[2];
 };
 
-// op: IOMX_OP_ADD / MUL / SUB, ROWS_OP_SILU (one input), ROWS_OP_COPY (one input).
+// op: IOMX_OP_ADD / MUL / SUB / DIV (DIV on floating leaves), ROWS_OP_SILU (one input), ROWS_OP_COPY (one input).
 int launch_rows(int op, int dtype, const RowsRequest& r, hipStream_t stream);
 
 struct RowsRmsnormRequest {

@@ -292,6 +292,14 @@ IOMX_HD uint32_t encode_f32(float r) {
     return sign | field;
 }
 
+template <int OP, typename T>
+IOMX_HD T leaf_arith(T x, T y) {
+    if constexpr (OP == IOMX_OP_ADD) return x + y;
+    else if constexpr (OP == IOMX_OP_MUL) return x * y;
+    else if constexpr (OP == IOMX_OP_SUB) return x - y;
+    else return x / y;
+}
+
 template <int DT, int OP>
 IOMX_HD uint64_t leaf_binary(uint64_t a, uint64_t b) {
     constexpr int BITS = bits_of(DT);
@@ -305,16 +313,17 @@ IOMX_HD uint64_t leaf_binary(uint64_t a, uint64_t b) {
         }
     } else {
         // IEEE arithmetic supplies the special cases of the reference rule: opposite
-        // infinities and infinity times zero give NaN, an exact zero sum is +0 unless
-        // both operands are -0, NaN operands give NaN.
+        // infinities, infinity times zero, 0/0 and inf/inf give NaN, an exact zero sum
+        // is +0 unless both operands are -0, NaN operands give NaN.  A quotient is not
+        // exact in the carrier, but it is correctly rounded to at least 2p + 2 bits for
+        // a leaf of p significand bits (24 for p <= 11, 53 for F32), so the encode's
+        // rounding still equals one rounding of the exact quotient.
         if constexpr (BITS <= 8) {
             const float x = decode_f32<DT>((uint32_t)a), y = decode_f32<DT>((uint32_t)b);
-            const float r = OP == IOMX_OP_ADD ? x + y : (OP == IOMX_OP_MUL ? x * y : x - y);
-            return encode_f32<DT>(r);
+            return encode_f32<DT>(leaf_arith<OP>(x, y));
         }
         const double x = decode<DT>(a), y = decode<DT>(b);
-        const double r = OP == IOMX_OP_ADD ? x + y : (OP == IOMX_OP_MUL ? x * y : x - y);
-        return encode<DT>(r);
+        return encode<DT>(leaf_arith<OP>(x, y));
     }
 }
 

@@ -809,11 +809,11 @@ private:
 
     oid binary_impl(const BinaryRequest& request) override {
         const int code = binary_code(request.out.spec.data_type);
-        if (code < 0 || request.operation == BinaryOperation::Div)
-            throw detail::UnsupportedOperation();
+        if (code < 0) throw detail::UnsupportedOperation();
         int op = IOMX_OP_ADD;
         if (request.operation == BinaryOperation::Mul) op = IOMX_OP_MUL;
         if (request.operation == BinaryOperation::Sub) op = IOMX_OP_SUB;
+        if (request.operation == BinaryOperation::Div) op = IOMX_OP_DIV;
         std::lock_guard<std::mutex> order(submission_mutex_);
         return submit_binary(
                 request, device_.registry_state(), registry_queue_id_, pending_fence(),

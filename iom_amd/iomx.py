@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libiomx.so")
  DT_U64, DT_F4_E2M1, DT_F6_E2M3, DT_F6_E3M2, DT_F8_E4M3FN, DT_F8_E5M2, DT_F8_E8M0, DT_F16,
  DT_BF16, DT_F32, DT_F64) = range(23)
 LEAF_BITS = (8, 2, 2, 4, 4, 8, 8, 16, 16, 32, 32, 64, 64, 4, 6, 6, 8, 8, 8, 16, 16, 32, 64)
-OP_ADD, OP_MUL, OP_SUB = 0, 1, 2
+OP_ADD, OP_MUL, OP_SUB, OP_DIV = 0, 1, 2, 3
 TILE = 16
 
 

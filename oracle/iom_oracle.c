@@ -208,8 +208,12 @@ static long double codec_arith(int op, long double x, long double y) {
         if ((isinf(x) && y == 0) || (isinf(y) && x == 0)) return (long double)NAN;
         return x * y;
     }
-    if (isinf(x) && isinf(y) && signbit(x) == signbit(y)) return (long double)NAN;
-    return x - y;
+    if (op == IOMO_OP_SUB) {
+        if (isinf(x) && isinf(y) && signbit(x) == signbit(y)) return (long double)NAN;
+        return x - y;
+    }
+    if ((x == 0 && y == 0) || (isinf(x) && isinf(y))) return (long double)NAN;
+    return x / y;
 }
 
 static long double positive_nan(void) { return fabsl((long double)NAN); }
@@ -220,6 +224,7 @@ uint64_t iomo_scalar_binary(int op, int dtype, uint64_t a, uint64_t b) {
     const unsigned width = integer_width(dtype);
     if (width) {
         const uint64_t mask = width == 64 ? ~0ull : (1ull << width) - 1;
+        if (op == IOMO_OP_DIV) return 0;   /* :166; refused before it is reached */
         if (op == IOMO_OP_ADD) return (a + b) & mask;
         if (op == IOMO_OP_MUL) return (a * b) & mask;
         return (a - b) & mask;
@@ -310,8 +315,28 @@ static uint64_t narrow_nan(fmt_t f) {
     return (emask << f.fbits) | (f.finite_only ? fmask : 1ull << (f.fbits - 1));
 }
 
+/* Quotient of two finite non-zero values of a format of at most 16 bits, rounded once:
+ * the operands are integers times powers of two (at most 11 significand bits), so the
+ * quotient's leading 40-odd bits come from one integer division, and the remainder
+ * becomes a sticky bit below them.  That integer, scaled, is an exact binary64 number
+ * which lies strictly between the same pair of neighbours of the narrow grid, and on
+ * the same side of their midpoint, as the true quotient; narrow_round does the rest. */
+static uint64_t narrow_quotient(uint64_t a, uint64_t b, fmt_t f) {
+    const uint64_t emask = (1ull << f.ebits) - 1, fmask = (1ull << f.fbits) - 1;
+    const uint64_t ea = (a >> f.fbits) & emask, eb = (b >> f.fbits) & emask;
+    const uint64_t ma = ea ? (1ull << f.fbits) + (a & fmask) : (a & fmask);
+    const uint64_t mb = eb ? (1ull << f.fbits) + (b & fmask) : (b & fmask);
+    const int sa = (int)(ea ? ea : 1), sb = (int)(eb ? eb : 1);   /* the bias and fbits cancel */
+    const int negative = (int)(((a ^ b) >> (f.ebits + f.fbits)) & 1);
+    const uint64_t n = ma << 40;
+    const uint64_t q = ((n / mb) << 1) | (n % mb != 0);
+    const double v = ldexp((double)q, sa - sb - 41);             /* q < 2^53: exact */
+    return narrow_round(negative ? -v : v, f);
+}
+
 uint64_t iomo_scalar_binary_ieee(int op, int dtype, uint64_t a, uint64_t b) {
     const unsigned width = integer_width(dtype);
+    if (width && op == IOMO_OP_DIV) return 0;
     if (width == 64) {
         if (op == IOMO_OP_ADD) return a + b;
         if (op == IOMO_OP_MUL) return a * b;
@@ -331,7 +356,8 @@ uint64_t iomo_scalar_binary_ieee(int op, int dtype, uint64_t a, uint64_t b) {
         volatile float r;
         if (op == IOMO_OP_ADD) r = x + y;
         else if (op == IOMO_OP_MUL) r = x * y;
-        else r = x - y;
+        else if (op == IOMO_OP_SUB) r = x - y;
+        else r = x / y;
         if (r != r) return 0x7FC00000u;
         return f32_bits(r);
     }
@@ -343,11 +369,12 @@ uint64_t iomo_scalar_binary_ieee(int op, int dtype, uint64_t a, uint64_t b) {
         volatile double r;
         if (op == IOMO_OP_ADD) r = x + y;
         else if (op == IOMO_OP_MUL) r = x * y;
-        else r = x - y;
+        else if (op == IOMO_OP_SUB) r = x - y;
+        else r = x / y;
         if (r != r) return 0x7FF8000000000000ull;
         return f64_bits(r);
     }
-    if (dtype == IOMO_DT_BF16) {
+    if (dtype == IOMO_DT_BF16 && op != IOMO_OP_DIV) {
         const float x = f32_from_bits((uint32_t)a << 16);
         const float y = f32_from_bits((uint32_t)b << 16);
         if (op == IOMO_OP_MUL) {
@@ -385,6 +412,16 @@ uint64_t iomo_scalar_binary_ieee(int op, int dtype, uint64_t a, uint64_t b) {
     int sx, sy;
     const double x = narrow_value(a, f, &sx), y = narrow_value(b, f, &sy);
     if (sx == 2 || sy == 2) return narrow_nan(f);
+    if (op == IOMO_OP_DIV) {
+        const uint64_t emask = (1ull << f.ebits) - 1, fmask = (1ull << f.fbits) - 1;
+        const uint64_t finite_emax = top_exponent_is_special(f) ? emask - 1 : emask;
+        const uint64_t sign = ((a ^ b) >> (f.ebits + f.fbits) & 1) << (f.ebits + f.fbits);
+        if ((sx == 1 && sy == 1) || (x == 0 && y == 0)) return narrow_nan(f);
+        if (sx == 1 || y == 0)   /* infinite quotient: infinity, or the largest finite value */
+            return sign | (f.infs ? emask << f.fbits : (finite_emax << f.fbits) | fmask);
+        if (sy == 1 || x == 0) return sign;
+        return narrow_quotient(a, b, f);
+    }
     if (op == IOMO_OP_MUL) {
         if ((sx == 1 && y == 0) || (sy == 1 && x == 0)) return narrow_nan(f);
     } else if (sx == 1 && sy == 1) {
@@ -510,7 +547,7 @@ int iomo_binary(int op, int dtype, const iomo_view* lhs, const iomo_view* rhs,
     fmt_t numeric;
     if (!bits || (!integer_width(dtype) && !float_format(dtype, &numeric)))
         return IOMO_ERR_UNSUPPORTED;   /* BOOL and F8_E8M0 (src/device_ops_binary.cpp:26-46) */
-    if (op < IOMO_OP_ADD || op > IOMO_OP_SUB) return IOMO_ERR_INVALID;
+    if (op < IOMO_OP_ADD || op > IOMO_OP_DIV) return IOMO_ERR_INVALID;
     if (!view_ok(lhs) || !view_ok(rhs) || !view_ok(out)) return IOMO_ERR_INVALID;
     /* src/device_ops_binary.cpp:121-143: right-aligned broadcast */
     const uint32_t rank = lhs->rank > rhs->rank ? lhs->rank : rhs->rank;
@@ -524,6 +561,9 @@ int iomo_binary(int op, int dtype, const iomo_view* lhs, const iomo_view* rhs,
     if (out->rank != rank) return IOMO_ERR_INVALID;
     for (uint32_t i = 0; i < rank; ++i)
         if (out->dims[i] != rdims[i]) return IOMO_ERR_INVALID;
+    /* src/device_ops_binary.cpp:174-175: division on the floating leaves only, refused
+     * after the shape checks */
+    if (op == IOMO_OP_DIV && integer_width(dtype)) return IOMO_ERR_UNSUPPORTED;
 
     bsnap_t ls, rs, os;
     snapshot(lhs, rdims, rank, &ls);

@@ -1,6 +1,6 @@
 /*
  * iom_oracle.h — CPU restatement of IOM's reference CPU backend for the
- * memory-bound tensor ops (binary ADD/SUB/MUL, RMSNorm, SiLU, the softmax
+ * memory-bound tensor ops (binary ADD/SUB/MUL/DIV, RMSNorm, SiLU, the softmax
  * stage of SDPA, tiled copy, host transfer scatter/gather).
  *
  * THIS IS TEST INFRASTRUCTURE.  It is the checker the GPU path is compared
@@ -13,7 +13,10 @@
  * Pinning status (what fixes each function's results, beyond this file):
  *   iomo_scalar_binary   reference KATs test/backend/test_scalar_add.cpp:42-132,
  *                        closed form (IEEE-754 single rounding, two's-complement
- *                        wrap), and the compiled reference CPU backend.
+ *                        wrap), and the compiled reference CPU backend.  DIV:
+ *                        the KATs of :50-53,94,101, an integer quotient with a
+ *                        sticky bit, numpy's binary16/binary32 division, and the
+ *                        compiled reference over every pair of the narrow leaves.
  *   iomo_binary          broadcast fixtures of backend_conformance_add_gpu.hpp:242-394,
  *                        brute-force index invariant, compiled reference.
  *   iomo_rmsnorm         closed form for all-ones rows
@@ -54,7 +57,7 @@ enum {
 };
 
 /* Binary operations in the order of scalar_binary_codec.hpp:9. */
-enum { IOMO_OP_ADD = 0, IOMO_OP_MUL = 1, IOMO_OP_SUB = 2 };
+enum { IOMO_OP_ADD = 0, IOMO_OP_MUL = 1, IOMO_OP_SUB = 2, IOMO_OP_DIV = 3 };
 
 enum {
     IOMO_OK = 0,

@@ -31,7 +31,7 @@ INTEGER_LEAVES = tuple(range(DT_I2, DT_U64 + 1))
 FLOAT_LEAVES = (DT_F4_E2M1, DT_F6_E2M3, DT_F6_E3M2, DT_F8_E4M3FN, DT_F8_E5M2, DT_F16, DT_BF16,
                 DT_F32, DT_F64)
 NUMERIC_LEAVES = INTEGER_LEAVES + FLOAT_LEAVES     # BOOL and F8_E8M0 carry no arithmetic
-OP_ADD, OP_MUL, OP_SUB = 0, 1, 2
+OP_ADD, OP_MUL, OP_SUB, OP_DIV = 0, 1, 2, 3
 TILE = 16
 
 

@@ -16,7 +16,7 @@ import datagen
 import iomo
 from iom_amd import iomx
 from iomo import (ALL_LEAVES, DT_BOOL, DT_F16, DT_F64, DT_F8_E8M0, DT_I16, DT_I64, DT_U16, DT_U4,
-                  DT_U64, FLOAT_LEAVES, LEAF_BITS, LEAF_NAME, NUMERIC_LEAVES, OP_ADD, OP_MUL, OP_SUB)
+                  DT_U64, FLOAT_LEAVES, LEAF_BITS, LEAF_NAME, NUMERIC_LEAVES, OP_ADD, OP_DIV, OP_MUL, OP_SUB)
 
 pytestmark = pytest.mark.gpu
 
@@ -113,8 +113,10 @@ def test_copy_between_views(dtype, dims, family):
 # -- binary ---------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", NARROW, ids=names(NARROW))
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 def test_binary_every_pair_of_a_narrow_leaf(dtype, op):
+    if op == OP_DIV and dtype not in FLOAT_LEAVES:
+        pytest.skip("division is defined on the floating leaves only")
     n = 1 << LEAF_BITS[dtype]
     every = np.arange(n).astype(np.uint8)
     dl, hl = pair(dtype, (n, 1), values=every.reshape(n, 1))
@@ -148,8 +150,10 @@ def test_binary_every_8bit_pair_on_whole_planes(dtype, op):
 
 
 @pytest.mark.parametrize("dtype", [DT_I16, DT_U16, DT_F16], ids=["I16", "U16", "F16"])
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 def test_binary_16bit_pairs_on_whole_planes(dtype, op):
+    if op == OP_DIV and dtype != DT_F16:
+        pytest.skip("division is defined on the floating leaves only")
     """4 million operand pairs (specials against everything) as whole planes: the packed
     two-lane integer arithmetic and the hardware F16 conversions, against the codec."""
     n = 2048
@@ -210,13 +214,31 @@ def test_binary_views_and_broadcasts(dtype, case):
         t.free()
 
 
+@pytest.mark.parametrize("dtype", [d for d in ROWS_NUMERIC if d in FLOAT_LEAVES],
+                         ids=names([d for d in ROWS_NUMERIC if d in FLOAT_LEAVES]))
+@pytest.mark.parametrize("case", range(len(ROWS_CASES)))
+def test_division_views_and_broadcasts(dtype, case):
+    ld, ls, rd, rs, od, os_ = ROWS_CASES[case]
+    dl, hl = pair(dtype, ld, salt=0x400 + case)
+    dr, hr = pair(dtype, rd, salt=0x500 + case)
+    do, ho = pair(dtype, od, salt=0x600 + case)
+    rc = iomx.binary(OP_DIV, apply(dl.view(), ls), apply(dr.view(), rs), apply(do.view(), os_))
+    assert rc == 0, iomx.lib().iomx_error_string(rc)
+    assert kernel_name().startswith("rows_") == on_rows(dtype)
+    assert iomo.binary(OP_DIV, apply(hl.view(), ls), apply(hr.view(), rs), apply(ho.view(), os_),
+                       ieee=True) == 0
+    assert same_storage(do, ho)
+    for t in (dl, dr, do):
+        t.free()
+
+
 def half_specials():
     return np.array([0x0000, 0x8000, 0x0001, 0x8001, 0x03FF, 0x0400, 0x83FF, 0x8400, 0x3C00, 0xBC00,
                      0x3C01, 0x3BFF, 0x7BFF, 0xFBFF, 0x7C00, 0xFC00, 0x7C01, 0x7E00, 0xFE00, 0xFFFF,
                      0x0002, 0x1400, 0x13FF, 0x6800, 0x7800, 0x3555, 0x4248], np.uint16)
 
 
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 def test_binary_f16_four_million_pairs_against_the_codec(op):
     n = 2048
     vals = np.concatenate([half_specials(), datagen.pattern_bits(16, n - half_specials().size, 41)])
@@ -245,7 +267,7 @@ def double_specials():
                      0x4340000000000000, 0x3FD5555555555555], np.uint64)
 
 
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 def test_binary_f64_specials_and_random_pairs(op):
     n = 1024
     k = n - double_specials().size

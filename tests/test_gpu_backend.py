@@ -12,7 +12,7 @@ import pytest
 import datagen
 import iomo
 from iomo import (ALL_LEAVES, DT_BF16, DT_BOOL, DT_F32, DT_F64, DT_I32, FLOAT_LEAVES, LEAF_BITS,
-                  LEAF_NAME, NUMERIC_LEAVES, OP_ADD, OP_MUL, OP_SUB)
+                  LEAF_NAME, NUMERIC_LEAVES, OP_ADD, OP_DIV, OP_MUL, OP_SUB)
 
 pytestmark = pytest.mark.gpu
 
@@ -74,10 +74,12 @@ CASES = [
 
 
 @pytest.mark.parametrize("dtype", [DT_I32, DT_F32, DT_BF16])
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 @pytest.mark.parametrize("case", range(len(CASES)))
 def test_binary_matches_reference_cpu_backend_bit_for_bit(devices, dtype, op, case):
     cpu, gpu = devices
+    if op == OP_DIV and dtype == DT_I32:
+        pytest.skip("refused by both backends: test_integer_division_is_refused_like_the_reference")
     ld, ls, rd, rs, od, os_ = CASES[case]
     cl, gl = both(devices, dtype, ld, salt=0x100 + case)
     cr, gr = both(devices, dtype, rd, salt=0x200 + case)
@@ -172,6 +174,45 @@ def test_binary_every_other_numeric_leaf(devices, dtype, case):
 
 
 OTHER_FLOAT = [d for d in FLOAT_LEAVES if d not in (DT_F32, DT_BF16)]
+
+
+@pytest.mark.parametrize("dtype", OTHER_FLOAT, ids=[LEAF_NAME[d] for d in OTHER_FLOAT])
+@pytest.mark.parametrize("case", [0, 1, 2, 3])
+def test_division_every_other_float_leaf(devices, dtype, case):
+    """Bit for bit against the reference CPU backend (F64 divides whole numbers by powers of
+    two, which neither carrier rounds)."""
+    cpu, gpu = devices
+    ld, ls, rd, rs, od, os_ = CASES[case]
+    if dtype == DT_F64:
+        num = lambda dims, salt: (datagen.uniform_i32(int(np.prod(dims)), -1000, 1000, salt)
+                                  .view(np.int32).astype(np.float64).view(np.uint64).reshape(dims))
+        den = lambda dims, salt: np.ldexp(
+            1.0, datagen.uniform_i32(int(np.prod(dims)), -8, 8, salt).view(np.int32)
+        ).view(np.uint64).reshape(dims)
+        cl, gl = both(devices, dtype, ld, values=num(ld, 1 + case))
+        cr, gr = both(devices, dtype, rd, values=den(rd, 2 + case))
+    else:
+        cl, gl = both(devices, dtype, ld, salt=0x400 + case)
+        cr, gr = both(devices, dtype, rd, salt=0x500 + case)
+    co, go = both(devices, dtype, od, salt=0x600 + case)
+    tc = cpu.binary(OP_DIV, apply(cl.view(), ls), apply(cr.view(), rs), apply(co.view(), os_))
+    tg = gpu.binary(OP_DIV, apply(gl.view(), ls), apply(gr.view(), rs), apply(go.view(), os_))
+    assert tc > 0 and tg > 0, (tc, tg, gpu.error())
+    assert np.array_equal(co.view().to_host(), go.view().to_host())
+    close(cl, gl, cr, gr, co, go)
+
+
+def test_integer_division_is_refused_like_the_reference(devices):
+    cpu, gpu = devices
+    for dtype in (DT_I32, iomo.DT_U8, iomo.DT_I4, iomo.DT_U64):
+        ca, ga = both(devices, dtype, (2, 16, 16), salt=1)
+        co, go = both(devices, dtype, (2, 16, 16), salt=2)
+        before = go.view().to_host().copy()
+        tc = cpu.binary(OP_DIV, ca.view(), ca.view(), co.view())
+        tg = gpu.binary(OP_DIV, ga.view(), ga.view(), go.view())
+        assert tc < 0 and tg == tc, (tc, tg)
+        assert np.array_equal(go.view().to_host(), before)
+        close(ca, ga, co, go)
 
 
 @pytest.mark.parametrize("dtype", OTHER_FLOAT, ids=[LEAF_NAME[d] for d in OTHER_FLOAT])

@@ -24,7 +24,7 @@ import datagen
 import golden_cases as gc
 import iomo
 from iom_amd import iomx
-from iomo import DT_BF16, DT_F32, DT_I32, DT_U32, OP_ADD, OP_MUL, OP_SUB
+from iomo import DT_BF16, DT_F32, DT_I32, DT_U32, OP_ADD, OP_DIV, OP_MUL, OP_SUB
 
 pytestmark = pytest.mark.gpu
 
@@ -133,9 +133,11 @@ BINARY_CASES = [
 
 
 @pytest.mark.parametrize("dtype", [DT_I32, DT_F32, DT_BF16])
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 @pytest.mark.parametrize("case", range(len(BINARY_CASES)))
 def test_binary_bit_exact_against_oracle(dtype, op, case):
+    if op == OP_DIV and dtype == DT_I32:
+        pytest.skip("division is defined on the floating leaves only")
     ld, ls, rd, rs, od, os_, family = BINARY_CASES[case]
     dl, hl = pair(dtype, ld, salt=0x100 + case)
     dr, hr = pair(dtype, rd, salt=0x200 + case)
@@ -181,6 +183,14 @@ def test_binary_rejections_match_the_reference_rules():
     assert iomx.binary(OP_ADD, a.view(), b.view(), o.view()) == -1          # not broadcastable
     assert iomx.binary(OP_ADD, a.view(), a.view(), b.view()) == -1          # wrong output shape
     assert iomx.binary(7, a.view(), a.view(), o.view()) == -1               # unknown operation
+    # integer division is refused, but only after the shape checks (device_ops_binary.cpp:121-176)
+    for dtype in (DT_I32, DT_U32, 1, 5, 12):
+        i = iomx.DeviceTensor(dtype, (2, 16, 16))
+        j = iomx.DeviceTensor(dtype, (3, 16, 16))
+        assert iomx.binary(OP_DIV, i.view(), i.view(), i.view()) == -2
+        assert iomx.binary(OP_DIV, i.view(), j.view(), i.view()) == -1
+        i.free()
+        j.free()
     for code in (0, 18, 23, -1):         # BOOL, F8_E8M0: no arithmetic; unknown leaf codes
         assert iomx.lib().iomx_launch_binary(OP_ADD, code, C.byref(a.view().cview()),
                                              C.byref(a.view().cview()), C.byref(o.view().cview()),
@@ -193,7 +203,8 @@ def test_binary_rejections_match_the_reference_rules():
 
 @pytest.mark.parametrize("dtype,op", [(DT_F32, OP_ADD), (DT_I32, OP_ADD), (DT_BF16, OP_ADD),
                                       (DT_BF16, OP_MUL), (DT_F32, OP_MUL), (DT_I32, OP_MUL),
-                                      (DT_F32, OP_SUB), (DT_BF16, OP_SUB)])
+                                      (DT_F32, OP_SUB), (DT_BF16, OP_SUB),
+                                      (DT_F32, OP_DIV), (DT_BF16, OP_DIV)])
 def test_binary_directed_encodings_cross_product(dtype, op):
     """Every special encoding against every other, F32/BF16 through the codec oracle."""
     if dtype == DT_I32:
@@ -223,7 +234,7 @@ def test_binary_directed_encodings_cross_product(dtype, op):
 
 def test_bf16_every_encoding_against_a_spread_of_partners():
     """All 65536 BF16 values as lhs, against 48 partners chosen across the exponent
-    range (includes the subnormal-product band for MUL), bit-exact for all three ops."""
+    range (includes the subnormal product and quotient bands), bit-exact for all four ops."""
     partners = np.array([0x0000, 0x8000, 0x0001, 0x807F, 0x0080, 0x00FF, 0x0100, 0x1F80, 0x2000,
                          0x2041, 0x3000, 0x3F80, 0xBF80, 0x3F81, 0x3FFF, 0x4000, 0x4049, 0x5F00,
                          0x7F00, 0x7F7F, 0xFF7F, 0x7F80, 0xFF80, 0x7FC0, 0x1001, 0x9001, 0x0800,
@@ -236,7 +247,7 @@ def test_bf16_every_encoding_against_a_spread_of_partners():
     da, ha = pair(DT_BF16, A.shape, values=A)
     db, hb = pair(DT_BF16, B.shape, values=B)
     do, ho = pair(DT_BF16, A.shape)
-    for op in (OP_ADD, OP_MUL, OP_SUB):
+    for op in (OP_ADD, OP_MUL, OP_SUB, OP_DIV):
         assert iomx.binary(op, da.view(), db.view(), do.view()) == 0
         assert iomo.binary(op, ha.view(), hb.view(), ho.view(), ieee=True) == 0
         got = do.raw()
@@ -246,8 +257,9 @@ def test_bf16_every_encoding_against_a_spread_of_partners():
     Lr = iomo.lib()
     a_flat, b_flat = A.reshape(-1), B.reshape(-1)
     for i in idx[:3000]:
-        assert Lr.iomo_scalar_binary(OP_MUL, DT_BF16, int(a_flat[i]), int(b_flat[i])) == \
-            Lr.iomo_scalar_binary_ieee(OP_MUL, DT_BF16, int(a_flat[i]), int(b_flat[i]))
+        for op in (OP_MUL, OP_DIV):
+            assert Lr.iomo_scalar_binary(op, DT_BF16, int(a_flat[i]), int(b_flat[i])) == \
+                Lr.iomo_scalar_binary_ieee(op, DT_BF16, int(a_flat[i]), int(b_flat[i]))
     for t in (da, db, do):
         t.free()
 

@@ -10,7 +10,7 @@ import pytest
 import datagen
 import iomo
 from iomo import (ALL_LEAVES, DT_F16, DT_F64, DT_I16, DT_I64, DT_U16, DT_U64, FLOAT_LEAVES,
-                  LEAF_BITS, LEAF_NAME, NUMERIC_LEAVES, OP_ADD, OP_MUL, OP_SUB)
+                  LEAF_BITS, LEAF_NAME, NUMERIC_LEAVES, OP_ADD, OP_DIV, OP_MUL, OP_SUB)
 
 NARROW = [d for d in NUMERIC_LEAVES if LEAF_BITS[d] <= 8]
 names = lambda ds: [LEAF_NAME[d] for d in ds]
@@ -92,9 +92,11 @@ def test_copy_between_views(ref, dtype):
 # -- binary operations -----------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", NARROW, ids=names(NARROW))
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 def test_binary_every_pair_of_a_narrow_leaf(ref, dtype, op):
     """[n,1] x [1,n] -> [n,n] holds every operand pair of the leaf."""
+    if op == OP_DIV and dtype not in iomo.FLOAT_LEAVES:
+        pytest.skip("division is defined on the floating leaves only")
     n = 1 << LEAF_BITS[dtype]
     every = np.arange(n, dtype=np.uint8 if n <= 256 else np.uint16)
     rl, hl = both(ref, dtype, (n, 1), values=every.reshape(n, 1))
@@ -114,7 +116,7 @@ def half_specials():
                      0x0002, 0x1400, 0x13FF, 0x6800, 0x7800, 0x3555, 0x4248], np.uint16)
 
 
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 def test_binary_f16_specials_and_random_pairs(ref, op):
     n = 1200
     vals = np.concatenate([half_specials(), datagen.pattern_bits(16, n - half_specials().size, 41)])
@@ -136,7 +138,8 @@ def test_f16_closed_form_against_numpy_half():
     a = np.concatenate([half_specials(), datagen.pattern_bits(16, 4000, 51)])
     b = np.concatenate([half_specials()[::-1], datagen.pattern_bits(16, 4000, 52)])
     with np.errstate(all="ignore"):
-        for op, fn in ((OP_ADD, np.add), (OP_MUL, np.multiply), (OP_SUB, np.subtract)):
+        for op, fn in ((OP_ADD, np.add), (OP_MUL, np.multiply), (OP_SUB, np.subtract),
+                       (OP_DIV, np.divide)):
             r = fn(a.view(np.float16), b.view(np.float16)).view(np.uint16)
             for x, y, z in zip(a.tolist(), b.tolist(), r.tolist()):
                 got = L.iomo_scalar_binary_ieee(op, DT_F16, x, y)
@@ -184,7 +187,7 @@ def finite_doubles(n, salt):
     return (sign << np.uint64(63)) | (exp << np.uint64(52)) | frac
 
 
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 def test_binary_f64_codec_and_binary64_carrier(ref, op):
     n = 600
     vals = np.concatenate([double_specials(), finite_doubles(n - double_specials().size, 71)])
@@ -206,7 +209,7 @@ def test_binary_f64_codec_and_binary64_carrier(ref, op):
     # and binary64 itself, stated with numpy
     with np.errstate(all="ignore"):
         a, b = vals.view(np.float64).reshape(n, 1), other.view(np.float64).reshape(1, n)
-        closed = {OP_ADD: a + b, OP_MUL: a * b, OP_SUB: a - b}[op]
+        closed = {OP_ADD: a + b, OP_MUL: a * b, OP_SUB: a - b, OP_DIV: a / b}[op]
     bits = closed.view(np.uint64).copy()
     bits[np.isnan(closed)] = 0x7FF8000000000000
     if op == OP_ADD:     # exact-zero sums are +0 unless both operands are -0

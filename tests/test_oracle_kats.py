@@ -16,7 +16,7 @@ import pytest
 
 import datagen
 import iomo
-from iomo import DT_BF16, DT_F32, DT_I32, DT_U32, OP_ADD, OP_MUL, OP_SUB
+from iomo import DT_BF16, DT_F32, DT_I32, DT_U32, OP_ADD, OP_DIV, OP_MUL, OP_SUB
 
 L = iomo.lib()
 
@@ -91,6 +91,18 @@ KATS = [
     (OP_ADD, DT_F32, 0xFF7FFFFF, 0xFF7FFFFF, 0xFF800000),
     (OP_MUL, DT_F32, 0xFF7FFFFF, 0x40000000, 0xFF800000),
     (OP_SUB, DT_F32, 0xFF7FFFFF, 0x7F7FFFFF, 0xFF800000),
+    # division: test_scalar_add.cpp:50-53 and the overflow cases of :94,:101
+    (OP_DIV, DT_F32, 0, 0, 0x7FC00000), (OP_DIV, DT_F32, 0x80000000, 1, 0x80000000),
+    (OP_DIV, DT_F32, 0x80000000, 0x80000000, 0x7FC00000),
+    (OP_DIV, DT_F32, 0x3F800000, 0x7F800000, 0),
+    (OP_DIV, DT_BF16, 0x7F7F, 0x3F00, 0x7F80), (OP_DIV, DT_BF16, 0xFF7F, 0x3F00, 0xFF80),
+    (OP_DIV, DT_F32, 0x7F7FFFFF, 0x3F000000, 0x7F800000),
+    (OP_DIV, DT_F32, 0xFF7FFFFF, 0x3F000000, 0xFF800000),
+    # what IEEE 754 fixes: x/0 is a signed infinity, inf/inf is NaN, 1/3 rounds to nearest
+    (OP_DIV, DT_F32, 0x3F800000, 0x80000000, 0xFF800000),
+    (OP_DIV, DT_F32, 0x7F800000, 0xFF800000, 0x7FC00000),
+    (OP_DIV, DT_F32, 0x3F800000, 0x40400000, 0x3EAAAAAB),
+    (OP_DIV, DT_BF16, 0x3F80, 0x4040, 0x3EAB), (OP_DIV, DT_BF16, 0x4000, 0x4040, 0x3F2B),
     # NaN payloads and signs collapse to the positive canonical quiet NaN
     (OP_ADD, DT_F32, 0xFFC12345, 0x3F800000, 0x7FC00000),
     (OP_MUL, DT_BF16, 0xFFFF, 0x3F80, 0x7FC0),
@@ -132,9 +144,11 @@ def _check_codec_equals_closed_form(op, dtype, a, b):
             L.iomo_scalar_binary_ieee(op, dtype, x, y), (op, dtype, hex(x), hex(y))
 
 
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 @pytest.mark.parametrize("dtype", [DT_I32, DT_F32, DT_BF16])
 def test_codec_equals_ieee_closed_form_on_hash_patterns(op, dtype):
+    if op == OP_DIV and dtype == DT_I32:
+        pytest.skip("division is defined on the floating leaves only")
     bits = 16 if dtype == DT_BF16 else 32
     n = 20000
     a = datagen.pattern_bits(bits, n, 0x1234 + op)
@@ -162,12 +176,53 @@ def test_bf16_mul_closed_form_over_the_subnormal_product_band():
     _check_codec_equals_closed_form(OP_MUL, DT_BF16, a, b ^ 0x8000)
 
 
+def test_bf16_quotient_is_rounded_once_over_the_subnormal_band():
+    """Quotients that land in [2^-140, 2^-120): below 2^-126 the BF16 grid is fixed at 2^-133
+    and a binary32 quotient is already rounded to the 2^-149 grid.  Three statements of the
+    rule must agree there: the codec (64-bit carrier), the integer quotient with a sticky bit,
+    and binary32 division followed by round-to-nearest-even narrowing (what a device computes)."""
+    sigs = [0, 1, 2, 3, 0x2A, 0x3F, 0x40, 0x41, 0x55, 0x7E, 0x7F]
+    a, b = [], []
+    for ea in range(1, 120, 3):
+        for eb in range(100, 255):
+            if -142 <= ea - eb <= -118:
+                for sa in sigs:
+                    for sb in sigs:
+                        a.append((ea << 7) | sa)
+                        b.append((eb << 7) | sb)
+    a = np.array(a, np.uint16)
+    b = np.array(b, np.uint16) ^ 0x8000
+    _check_codec_equals_closed_form(OP_DIV, DT_BF16, a[::3], b[::3])
+    with np.errstate(all="ignore"):
+        via_f32 = datagen.bf16_rne(datagen.bf16_to_f32(a) / datagen.bf16_to_f32(b))
+    idx = np.arange(0, a.size, 7)
+    want = np.array([L.iomo_scalar_binary(OP_DIV, DT_BF16, int(a[i]), int(b[i])) for i in idx],
+                    np.uint16)
+    assert np.array_equal(via_f32[idx], want)
+    assert (want & 0x7FFF).min() == 0 and ((want & 0x7FFF) > 0).any()
+
+
+def test_bf16_quotient_through_binary32_equals_the_codec_on_hash_patterns():
+    n = 60000
+    a = datagen.pattern_bits(16, n, 0x51)
+    b = datagen.pattern_bits(16, n, 0x52)
+    b[::5] = a[::5] ^ (datagen.pattern_bits(16, n, 0x53)[::5] & 0x7)   # quotients next to one
+    with np.errstate(all="ignore"):
+        q = datagen.bf16_to_f32(a) / datagen.bf16_to_f32(b)
+    got = datagen.bf16_rne(q)
+    got[np.isnan(q)] = 0x7FC0
+    want = np.array([L.iomo_scalar_binary(OP_DIV, DT_BF16, int(x), int(y))
+                     for x, y in zip(a.tolist(), b.tolist())], np.uint16)
+    assert np.array_equal(got, want)
+
+
 def test_f32_closed_form_equals_numpy_ieee():
     n = 200000
     a = datagen.pattern_bits(32, n, 5)
     b = datagen.pattern_bits(32, n, 6)
     with np.errstate(all="ignore"):
-        for op, fn in ((OP_ADD, np.add), (OP_SUB, np.subtract), (OP_MUL, np.multiply)):
+        for op, fn in ((OP_ADD, np.add), (OP_SUB, np.subtract), (OP_MUL, np.multiply),
+                       (OP_DIV, np.divide)):
             r = fn(a.view(np.float32), b.view(np.float32)).view(np.uint32).copy()
             r[np.isnan(r.view(np.float32))] = 0x7FC00000
             idx = np.arange(0, n, 97)

@@ -8,7 +8,7 @@ import pytest
 
 import datagen
 import iomo
-from iomo import DT_BF16, DT_F32, DT_I32, OP_ADD, OP_MUL, OP_SUB
+from iomo import DT_BF16, DT_F32, DT_I32, OP_ADD, OP_DIV, OP_MUL, OP_SUB
 
 BITS = {DT_BF16: 16, DT_F32: 32, DT_I32: 32}
 
@@ -48,9 +48,11 @@ BINARY_CASES = [
 
 
 @pytest.mark.parametrize("dtype", [DT_I32, DT_F32, DT_BF16])
-@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
 @pytest.mark.parametrize("case", range(len(BINARY_CASES)))
 def test_binary_bit_exact(ref, dtype, op, case):
+    if op == OP_DIV and dtype == DT_I32:
+        pytest.skip("integer division is refused; see test_division_of_integer_leaves_is_refused")
     ld, ls, rd, rs, od, os_ = BINARY_CASES[case]
     rl, hl = both(ref, dtype, ld, salt=0x100 + case)
     rr, hr = both(ref, dtype, rd, salt=0x200 + case)
@@ -82,6 +84,15 @@ def test_binary_exact_alias(ref, dtype, which):
         rc = iomo.binary(OP_MUL, ha.view(), ha.view(), ha.view())
     assert tok > 0 and rc == 0
     assert np.array_equal(ra.view().to_host(), ha.view().to_logical())
+
+
+def test_division_of_integer_leaves_is_refused(ref):
+    a, ha = both(ref, DT_I32, (2, 16, 16), salt=1)
+    b, hb = both(ref, DT_I32, (2, 16, 16), salt=2)
+    o, ho = both(ref, DT_I32, (2, 16, 16), salt=3)
+    assert ref.binary(OP_DIV, a.view(), b.view(), o.view()) < 0
+    assert iomo.binary(OP_DIV, ha.view(), hb.view(), ho.view()) == -2
+    assert np.array_equal(o.view().to_host(), ho.view().to_logical())      # untouched
 
 
 def test_reference_rejects_what_the_oracle_rejects(ref):
