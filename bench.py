@@ -374,6 +374,54 @@ def wl_linear(timer, steps, warmup):
     return out
 
 
+_VENDOR_GEMM = r"""
+import json, sys, time, torch
+steps = int(sys.argv[1])
+M, K = 64 * 512, 2048
+x = torch.randn(M, K, device="cuda", dtype=torch.bfloat16)
+for N, name in ((2048, "o_proj"), (5632, "gate_proj")):
+    w = torch.randn(N, K, device="cuda", dtype=torch.bfloat16) * 0.02
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.03:
+        for _ in range(5):
+            torch.nn.functional.linear(x, w)
+        torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        torch.nn.functional.linear(x, w)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    tf = 2.0 * M * K * N / (ms * 1e-3) / 1e12
+    print(json.dumps({"workload": "vendor_gemm_bf16_%s_[32768,2048]x[%d,2048]" % (name, N),
+                      "kernel": "torch.nn.functional.linear (hipBLASLt / rocBLAS)",
+                      "ms_per_launch": round(ms, 5), "TFLOP_per_s": round(tf, 1),
+                      "mfma_frac_of_2500": round(tf / 2500.0, 4)}), flush=True)
+"""
+
+
+def wl_vendor_gemm(timer, steps, warmup):
+    """The vendor's GEMM library (torch.nn.functional.linear, BF16, row-major operands) on the two
+    prefill shapes of wl_linear, on this box while this process idles: what a tuned library
+    reaches here, beside the 2500 TFLOP/s of the data sheet.  A yardstick only -- nothing of the
+    product calls it.  It runs in a child process (torch carries a HIP runtime of its own, which
+    finds no device in a process where the system's runtime already holds it) and is left out
+    under the profiler."""
+    import subprocess
+    if under_profiler():
+        return [{"workload": "vendor_gemm", "skipped": "not run under the profiler"}]
+    try:
+        p = subprocess.run([sys.executable, "-c", _VENDOR_GEMM, str(steps)], capture_output=True,
+                           text=True, timeout=300)
+    except Exception as exc:   # pragma: no cover
+        return [{"workload": "vendor_gemm", "skipped": "child failed: %s" % exc}]
+    rows = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")]
+    if p.returncode != 0 or not rows:
+        return [{"workload": "vendor_gemm", "skipped": "child exit %d: %s" % (p.returncode, p.stderr[-200:])}]
+    return rows
+
+
 def wl_sdpa(timer, steps, warmup):
     """BF16 causal grouped-query attention at TinyLlama's head shape (32 query heads, 4 KV
     heads, D = 64): a 512-token prefill of 8 sequences and a decode step of 64 sequences
@@ -815,6 +863,7 @@ def main():
         "chain": lambda: wl_chain(timer, max(K // 10, 5), max(W // 10, 2)),
         "layer_ops": lambda: wl_layer_ops(timer, max(K // 4, 5), max(W // 4, 2)),
         "linear": lambda: wl_linear(timer, max(K // 5, 10), max(W // 2, 5)),
+        "vendor_gemm": lambda: wl_vendor_gemm(timer, max(K // 5, 10), max(W // 2, 5)),
         "sdpa": lambda: wl_sdpa(timer, max(K // 5, 10), max(W // 2, 5)),
         "decoder_layer": lambda: wl_decoder_layer(timer, max(K // 5, 10), max(W // 2, 5)),
         "other_leaves": lambda: wl_other_leaves(timer, max(K // 10, 5), max(W // 10, 2)),
@@ -841,7 +890,7 @@ def main():
     if not args.no_detail:
         for key in ("bcast_mul_bf16", "bcast_div_bf16", "div_f32", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "copy_bf16", "add_f32",
                     "add_i32", "rmsnorm_bf16", "rmsnorm_f32", "silu_mul", "softmax", "softmax_causal",
-                    "chain", "layer_ops", "linear", "sdpa", "decoder_layer", "hbm_ceiling"):
+                    "chain", "layer_ops", "linear", "vendor_gemm", "sdpa", "decoder_layer", "hbm_ceiling"):
             r = table[key]()
             detail.extend(r if isinstance(r, list) else [r])
     cpu = None if args.no_cpu else cpu_baseline()

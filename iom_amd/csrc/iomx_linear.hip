@@ -606,7 +606,7 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     for (uint32_t d = 0; d < DEPTH - 1; ++d) issue(d < stages ? d : last, d);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * LPS) : "memory");
     __builtin_amdgcn_s_barrier();
-    static_assert(WN <= WM, "one output fragment read per step");
+    static_assert(WN <= WM, "WM + WN fragment reads fit two a step");
     bf16x8_t wf[2][WN], xf[2][WM];
     auto rd = [&](uint32_t ring, uint32_t frag) {
         return __builtin_bit_cast(bf16x8_t,
@@ -626,11 +626,24 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
         __builtin_amdgcn_s_barrier();
 #pragma unroll
         for (int step = 0; step < WM; ++step) {
-            if (step < WN) wf[P ^ 1][step] = rd(ring1, BM + wn * WN + step);
-            xf[P ^ 1][step] = rd(ring1, wm * WM + step);
 #pragma unroll
             for (int n = 0; n < WN; ++n)
                 acc[step][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[P][n], xf[P][step], acc[step][n], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            // the WM + WN fragments of the next stage, two a step behind the step's MFMAs, the
+            // last ones two steps before the stage ends: the wait for them at the top of the
+            // next stage finds them landed
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                constexpr int kReads = WM + WN;
+                const int f = 2 * step + i;
+                if (f < 2 * WN) {
+                    if (f & 1) wf[P ^ 1][f >> 1] = rd(ring1, BM + wn * WN + (f >> 1));
+                    else xf[P ^ 1][f >> 1] = rd(ring1, wm * WM + (f >> 1));
+                } else if (f < kReads) {
+                    xf[P ^ 1][f - WN] = rd(ring1, wm * WM + (f - WN));
+                }
+            }
             if (step >= HALF) {
 #pragma unroll
                 for (int i = 0; i < LPS / HALF; ++i) {
@@ -640,6 +653,9 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
                                                      (lptr_t)(lds + ring3 * kStageBytes + frag * kFrag), 16, 0, 0);
                 }
             }
+            // the step stays as written: left to itself the scheduler sinks the LDS reads of the
+            // next stage to just before their use, and the matrix core waits for LDS there
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
     uint32_t st = 0;
