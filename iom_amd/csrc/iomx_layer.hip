@@ -206,6 +206,74 @@ __global__ __launch_bounds__(256) void rope_pairs_kernel(const RopeArgs a) {
     }
 }
 
+// BF16, D/2 a multiple of 16: a lane owns one 16-byte chunk (eight columns of one row) of pair
+// tile tc and the matching chunk of tile tc + D/32, so a wave's request is 1 KiB of consecutive
+// memory.  A word holds columns 2j and 2j + 1, and the hardware conversion packs two results
+// with the rounding of the software encode (nearest even, gradual underflow; NaN made
+// canonical first).  The planes a lane walks are independent of each other, so the next
+// plane's chunks are requested before the present ones are rotated and stored.
+__global__ __launch_bounds__(256) void rope_pairs_bf16_kernel(const RopeArgs a) {
+    constexpr uint32_t kRowBytes = 32, kTileBytes = 512;
+    const uint32_t g = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t h = g & 1u, r = (g >> 1) & 15u, q = g >> 5;
+    const uint32_t tr = a.col_tiles > 1 ? fast_div(q, a.div_col_tiles) : q;
+    const uint32_t ptc = q - tr * a.col_tiles;
+    const uint32_t row = tr * kTile + r;
+    // the 32 lanes of a pair tile need its 16 frequencies: one power each, exchanged
+    const float own_frequency = rope_frequency(ptc * kTile + (g & 15u), a.width, (float)a.theta);
+    float frequency[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) frequency[i] = __shfl(own_frequency, (int)(8u * h) + i, 32);
+    if (g >= 2u * a.lanes_per_plane || row >= a.rows) return;
+    const uint32_t position = a.a + row;
+    float sine[8], cosine[8];
+    if (position != 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) rope_sincos(position, frequency[i], &sine[i], &cosine[i]);
+    }
+    const uint64_t off0 = ((uint64_t)tr * a.tile_cols + ptc) * kTileBytes + r * kRowBytes + h * 16u;
+    const uint64_t off1 = off0 + (uint64_t)(a.half >> 4) * kTileBytes;
+    uint32_t p = blockIdx.y;
+    if (p >= a.planes) return;
+    auto request = [&](uint32_t which, u32x4* first, u32x4* second) {
+        uint64_t pl[2];
+        walk_planes(a.walk, which, pl);
+        const uint8_t* xb = a.x + pl[0] * a.plane_bytes;
+        *first = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xb + off0));
+        *second = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xb + off1));
+    };
+    u32x4 f, s2, nf = {}, ns = {};
+    request(p, &f, &s2);
+    for (;;) {
+        const uint32_t following = p + gridDim.y;
+        const bool more = following < a.planes;
+        if (more) request(following, &nf, &ns);
+        uint64_t plane[2];
+        walk_planes(a.walk, p, plane);
+        uint8_t* ob = a.out + plane[1] * a.plane_bytes;
+        if (position != 0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = 2 * j;
+                const float fa = bf16_lo(f[j]), fb = bf16_hi(f[j]);
+                const float sa = bf16_lo(s2[j]), sb = bf16_hi(s2[j]);
+                const float fca = fa * cosine[i], ssa = sa * sine[i];
+                const float sca = sa * cosine[i], fsa = fa * sine[i];
+                const float fcb = fb * cosine[i + 1], ssb = sb * sine[i + 1];
+                const float scb = sb * cosine[i + 1], fsb = fb * sine[i + 1];
+                f[j] = pack_bf16(fca - ssa, fcb - ssb);
+                s2[j] = pack_bf16(sca + fsa, scb + fsb);
+            }
+        }
+        __builtin_nontemporal_store(f, reinterpret_cast<u32x4*>(ob + off0));
+        __builtin_nontemporal_store(s2, reinterpret_cast<u32x4*>(ob + off1));
+        if (!more) break;
+        f = nf;
+        s2 = ns;
+        p = following;
+    }
+}
+
 // One row per plane (a decode step): every plane has the same position, so the 16
 // lanes of a group evaluate one angle each, exchange them, and then rotate the row
 // of 16 different planes: no lane repeats the powf / sincos work of another.
@@ -358,7 +426,10 @@ uint32_t planes_in_grid(uint64_t lanes_per_plane, uint64_t planes) {
 template <int DT, typename T>
 void launch_rope(const RopeArgs& a, bool aligned, dim3 grid, hipStream_t s) {
     if (aligned && a.rows == 1) hipLaunchKernelGGL((rope_row_kernel<DT, T>), grid, dim3(256), 0, s, a);
-    else if (aligned) hipLaunchKernelGGL((rope_pairs_kernel<DT, T>), grid, dim3(256), 0, s, a);
+    else if (aligned && DT == DT_BF16 && a.lanes_per_plane <= 0x7FFFFF00u) {
+        const dim3 chunks((uint32_t)((2ull * a.lanes_per_plane + 255) / 256), grid.y, 1);
+        hipLaunchKernelGGL(rope_pairs_bf16_kernel, chunks, dim3(256), 0, s, a);
+    } else if (aligned) hipLaunchKernelGGL((rope_pairs_kernel<DT, T>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((rope_general_kernel<DT, T>), grid, dim3(256), 0, s, a);
 }
 
