@@ -122,6 +122,20 @@ int iomx_event_synchronize(iomx_event_t event);
 /* *done = 1 when the event has completed, 0 while it is pending. */
 int iomx_event_query(iomx_event_t event, int* done);
 int iomx_event_elapsed_ms(iomx_event_t start, iomx_event_t stop, float* ms);
+/*
+ * Completion word: after everything submitted to the stream before this call has
+ * finished, the device stores `value` to a 32-bit word in memory of iomx_host_alloc,
+ * which the host may poll directly.  `device_word` is the word's address as the device
+ * sees it, from iomx_host_device_address (asked once: the lookup costs more than the
+ * store).  No counterpart in the reference, whose queue learns of completion from an
+ * event (src/shared/gpu_queue_operations.inl:717-818); a host that waits for one short
+ * operation at a time sees the word about 2 us earlier than the event.  The store is a
+ * one-lane kernel (hipStreamWriteValue32 reaches the host as early, but on this runtime
+ * every launch that follows one takes 10 us longer); the call costs a launch, more than
+ * iomx_event_record.
+ */
+int iomx_host_device_address(void* host, void** device);
+int iomx_stream_write_word(iomx_stream_t stream, void* device_word, uint32_t value);
 
 /*
  * Recording and replay of a fixed sequence of launches (HIP graph).  No counterpart in

@@ -37,6 +37,12 @@ __global__ void fill_kernel(u32x4* __restrict__ dst, uint64_t chunks, uint32_t w
         dst[i] = v;
 }
 
+// One lane stores a word for the host to see: stream order puts it behind everything
+// submitted before, the system-scope release behind their writes.
+__global__ void write_word_kernel(uint32_t* word, uint32_t value) {
+    __hip_atomic_store(word, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 __global__ void fill_bytes_kernel(uint8_t* __restrict__ dst, uint64_t bytes, uint8_t value) {
     for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < bytes;
          i += (uint64_t)gridDim.x * blockDim.x)
@@ -265,6 +271,21 @@ int iomx_event_query(iomx_event_t event, int* done) {
     if (e == hipSuccess) { *done = 1; return IOMX_OK; }
     if (e == hipErrorNotReady) { (void)hipGetLastError(); *done = 0; return IOMX_OK; }
     return (int)e;
+}
+
+int iomx_host_device_address(void* host, void** device) {
+    if (!host || !device) return IOMX_ERR_INVALID;
+    *device = nullptr;
+    IOMX_HIP(hipHostGetDevicePointer(device, host, 0));
+    return IOMX_OK;
+}
+
+int iomx_stream_write_word(iomx_stream_t stream, void* device_word, uint32_t value) {
+    if (!device_word || (reinterpret_cast<uintptr_t>(device_word) & 3u)) return IOMX_ERR_INVALID;
+    hipLaunchKernelGGL(write_word_kernel, dim3(1), dim3(1), 0, native(stream),
+                       static_cast<uint32_t*>(device_word), value);
+    IOMX_HIP(hipGetLastError());
+    return IOMX_OK;
 }
 
 int iomx_event_elapsed_ms(iomx_event_t start, iomx_event_t stop, float* ms) {

@@ -26,12 +26,14 @@
 #include <array>
 #include <atomic>
 #include <chrono>
+#include <cstring>
 #include <condition_variable>
 #include <cstddef>
 #include <cstdint>
 #include <deque>
 #include <exception>
 #include <functional>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <new>
@@ -538,9 +540,16 @@ public:
             // one page-locked status word per completion event (the embedding lookup
             // reports an invalid id through it,
             // docs/BACKEND_CONTRACT/embedding-lookup.md:178-203)
+            // and one completion word per event behind them: an operation submitted to an idle
+            // queue signals through its word, which the completion thread sees earlier than
+            // the event (see start())
             void* cells = nullptr;
-            check(iomx_host_alloc(&cells, capacity * sizeof(std::uint32_t)), "status cells");
+            check(iomx_host_alloc(&cells, 2 * capacity * sizeof(std::uint32_t)), "status cells");
             status_cells_ = static_cast<std::uint32_t*>(cells);
+            std::memset(status_cells_, 0, 2 * capacity * sizeof(std::uint32_t));
+            void* device_side = nullptr;
+            check(iomx_host_device_address(status_cells_, &device_side), "status cells");
+            cells_on_device_ = static_cast<std::uint32_t*>(device_side);
             check(counted_stream_create(&stream_), "queue stream");
             completer_ = std::thread([this] { run_completer(); });
         } catch (...) {
@@ -568,6 +577,7 @@ public:
         const bool proved = stream_ == nullptr
                 || (!consume_submission_fault(SubmissionFault::stream_synchronize)
                     && iomx_stream_synchronize(stream_) == IOMX_OK);
+        release_unobserved_leases(proved);
         if (proved) {
             destroy_native();
         } else {
@@ -606,6 +616,8 @@ private:
         std::uint64_t sequence = 0;
         iomx_event_t event = nullptr;
         std::uint32_t* status = nullptr;
+        std::uint32_t* word = nullptr;      // completion word, or null: completion by the event
+        std::uint32_t ticket = 0;
         std::exception_ptr failure;
         Finish finish;
         Verify verify = nullptr;
@@ -635,6 +647,10 @@ private:
             if (events_[i] == event) return status_cells_ + i;
         return nullptr;
     }
+    [[nodiscard]] std::uint32_t* completion_word(iomx_event_t event) noexcept {
+        std::uint32_t* cell = status_cell(event);
+        return cell == nullptr ? nullptr : cell + events_.size();
+    }
 
     // Runs inside the common admission dispatch: launch on the queue stream,
     // record the completion event, hand the rest to the completion thread.
@@ -646,16 +662,30 @@ private:
         if (consume_submission_fault(SubmissionFault::event_create))
             throw std::runtime_error("MI355X completion resource is unavailable (injected)");
         iomx_event_t event = nullptr;
+        // An operation that finds the queue idle is most likely one its caller is about to wait
+        // for (the session submits, waits, submits: src/session.cpp:2000-2045): it signals through
+        // a completion word, which costs the submitting thread 1.7 us more than recording the
+        // event and reaches the completion thread 4 us earlier.  Behind other operations the
+        // event is recorded: there the submitting thread is the one that must not be held up.
+        bool idle = false;
+        std::uint32_t ticket = 0;
         {
             std::lock_guard<std::mutex> lock(mutex_);
             if (shutdown_) throw std::logic_error("MI355X queue is shut down");
             if (free_events_.empty()) throw detail::AdmissionResourceUnavailable();
             event = free_events_.back();
             free_events_.pop_back();
+            idle = in_flight_.empty() && !completing_;
+            if (idle && ++ticket_ == 0) ++ticket_;
+            ticket = ticket_;
         }
         InFlight item;
         item.sequence = sequence;
         item.event = event;
+        if (idle) {
+            item.word = completion_word(event);
+            item.ticket = ticket;
+        }
         item.finish = finish;
         item.verify = verify;
         item.status = status_cell(event);
@@ -669,8 +699,10 @@ private:
                 status = launch(stream_);
         }
         if (status == IOMX_OK) {
-            status = consume_submission_fault(SubmissionFault::event_record)
-                    ? kInjectedDeviceError : iomx_event_record(event, stream_);
+            if (consume_submission_fault(SubmissionFault::event_record)) status = kInjectedDeviceError;
+            else if (item.word != nullptr)
+                status = iomx_stream_write_word(stream_, cells_on_device_ + (item.word - status_cells_), item.ticket);
+            else status = iomx_event_record(event, stream_);
         }
         if (status != IOMX_OK) {
             try { throw_status(status, "MI355X kernel submission"); }
@@ -737,13 +769,26 @@ private:
         return iomx_event_synchronize(event);
     }
 
+    // Completion through the word: polled like the event; a word that has not arrived within
+    // the polling time is waited for on the stream, which also reports what went wrong.
+    [[nodiscard]] int await_word(const std::uint32_t* word, std::uint32_t ticket) noexcept {
+        const auto give_up = std::chrono::steady_clock::now() + std::chrono::microseconds(300);
+        for (unsigned spins = 0;; ++spins) {
+            if (__atomic_load_n(word, __ATOMIC_ACQUIRE) == ticket) return IOMX_OK;
+            if ((spins & 63u) == 63u && std::chrono::steady_clock::now() > give_up) break;
+            relax();
+        }
+        return iomx_stream_synchronize(stream_);
+    }
+
     void run_completer() noexcept {
         (void)iomx_set_device(device_.ordinal());
         for (;;) {
             InFlight item;
             if (!next_in_flight(item)) return;
             if (!item.failure) {
-                const int status = await_event(item.event);
+                const int status = item.word != nullptr ? await_word(item.word, item.ticket)
+                                                        : await_event(item.event);
                 if (status != IOMX_OK) {
                     try { throw_status(status, "MI355X kernel completion"); }
                     catch (...) { item.failure = std::current_exception(); }
@@ -763,6 +808,43 @@ private:
             try { if (item.finish) item.finish(static_cast<bool>(item.failure)); } catch (...) {}
             try { complete(item.sequence, std::move(item.failure)); } catch (...) {}
         }
+    }
+
+    // Workspace leases of finished attention requests that no caller has observed yet.
+    [[nodiscard]] bool keep_until_observed(std::uint64_t sequence, const detail::WorkspaceLease& lease) noexcept {
+        try {
+            std::lock_guard<std::mutex> lock(observed_mutex_);
+            return unobserved_leases_.emplace(sequence, lease).second;
+        } catch (...) {
+            return false;
+        }
+    }
+
+    // wait() has seen the token's terminal state: its workspace range may be leased again
+    // (src/shared/gpu_queue_operations.inl:1188-1205).  Repeated waits find nothing.
+    void fence_through_sequence(std::uint64_t sequence) noexcept override {
+        detail::WorkspaceLease lease{};
+        {
+            std::lock_guard<std::mutex> lock(observed_mutex_);
+            const auto found = unobserved_leases_.find(sequence);
+            if (found == unobserved_leases_.end()) return;
+            lease = found->second;
+            unobserved_leases_.erase(found);
+        }
+        detail::complete_workspace_lease(device_.registry_state(), lease, true);
+    }
+
+    // Queue teardown: whatever no caller observed (src/shared/gpu_queue_operations.inl:1207-1226).
+    void release_unobserved_leases(bool covering_proof) noexcept {
+        std::map<std::uint64_t, detail::WorkspaceLease> leases;
+        try {
+            std::lock_guard<std::mutex> lock(observed_mutex_);
+            leases.swap(unobserved_leases_);
+        } catch (...) {
+            return;   // the ranges stay reserved, never reused unsafely
+        }
+        for (const auto& entry : leases)
+            detail::complete_workspace_lease(device_.registry_state(), entry.second, covering_proof);
     }
 
     // ---- hooks ----------------------------------------------------------------
@@ -987,10 +1069,17 @@ private:
                                   return iomx_launch_sdpa(IOMX_DT_BF16, &q, &k, &v, &out, captured.a,
                                                           captured.L, scratch, scratch_bytes, 0, stream);
                               },
-                              [&state, entries, lease](bool failed) {
+                              [this, &state, entries, lease, sequence](bool failed) {
                                   (void)detail::release_or_invalidate_sdpa_entries(
                                           state.registry, entries, failed, true);
-                                  detail::complete_workspace_lease(state, lease, true);
+                                  // Successful attention keeps its workspace range leased until
+                                  // the caller observes the token (wait -> fence_through_sequence):
+                                  // a second submission on the same range is then refused as
+                                  // exhaustion whether or not the first has already finished
+                                  // (src/shared/gpu_queue_operations.inl:1113-1147).  A failed
+                                  // one, or one that leased nothing, releases at once.
+                                  if (failed || lease.entry_id == 0 || !keep_until_observed(sequence, lease))
+                                      detail::complete_workspace_lease(state, lease, true);
                               });
                     } catch (...) {
                         state.registry.remove_entries(std::span<const detail::EntryId>(
@@ -1190,6 +1279,7 @@ private:
     iomx_stream_t stream_ = nullptr;
     std::vector<iomx_event_t> events_;
     std::uint32_t* status_cells_ = nullptr;
+    std::uint32_t* cells_on_device_ = nullptr;   // the same cells at the address the device uses
     std::mutex mutex_;
     std::condition_variable cv_;
     std::vector<iomx_event_t> free_events_;
@@ -1197,6 +1287,9 @@ private:
     std::atomic<std::size_t> pending_{0};   // in_flight_.size(), readable without the lock
     bool completer_sleeping_ = false;
     bool completing_ = false;
+    std::uint32_t ticket_ = 0;          // last value handed to a completion word; never 0
+    std::mutex observed_mutex_;
+    std::map<std::uint64_t, detail::WorkspaceLease> unobserved_leases_;
     bool shutdown_ = false;
     std::thread completer_;
 };

@@ -56,7 +56,7 @@ SYMBOLS = [
     "iomx_memcpy_h2d", "iomx_memcpy_d2h", "iomx_memcpy_h2d_async", "iomx_memcpy_d2h_async",
     "iomx_memcpy_d2d_async", "iomx_stream_create", "iomx_stream_destroy",
     "iomx_stream_synchronize", "iomx_event_create", "iomx_event_destroy", "iomx_event_record",
-    "iomx_event_synchronize", "iomx_event_query", "iomx_event_elapsed_ms",
+    "iomx_event_synchronize", "iomx_event_query", "iomx_event_elapsed_ms", "iomx_host_device_address", "iomx_stream_write_word",
     "iomx_stream_begin_capture", "iomx_stream_end_capture", "iomx_graph_launch", "iomx_graph_destroy",
     "iomx_launch_linear", "iomx_sdpa_workspace", "iomx_launch_sdpa", "iomx_launch_sdpa_static",
     "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
@@ -141,6 +141,8 @@ def lib() -> C.CDLL:
         l.iomx_event_record.argtypes = [P, P]
         l.iomx_event_synchronize.argtypes = [P]
         l.iomx_event_query.argtypes = [P, C.POINTER(C.c_int)]
+        l.iomx_host_device_address.argtypes = [P, C.POINTER(P)]
+        l.iomx_stream_write_word.argtypes = [P, P, C.c_uint32]
         l.iomx_event_elapsed_ms.argtypes = [P, P, C.POINTER(C.c_float)]
         l.iomx_launch_binary.argtypes = [C.c_int, C.c_int, VP, VP, VP, P]
         l.iomx_launch_rmsnorm.argtypes = [C.c_int, VP, VP, VP, C.c_float, P]

@@ -190,6 +190,45 @@ def test_one_device_allocation_and_eager_queue_resources(gpu):
         t.close()
 
 
+def test_attention_keeps_its_workspace_leased_until_the_token_is_observed(gpu):
+    """test/backend/backend_conformance_sdpa.hpp:562-626: a second accepted use of the same live
+    range is exhaustion (-4) until the caller has waited for the first -- also when the first has
+    long finished on the device -- and a queue that goes away releases what nobody observed."""
+    import time
+    case = random_case(23, (), 4, 2, 40, 32, 48, 3, 43)
+    qd, kd, od = shapes(case)
+    t = [gpu.tensor(DT_BF16, d) for d in (qd, kd, kd, od)]
+    for tensor, name, d in zip(t, "qkv", (qd, kd, kd)):
+        tensor.view().from_host(np.array(case[name], np.uint16).reshape(d))
+    views = [x.view() for x in t]
+    need = gpu.sdpa_workspace_bytes(*views, 3, 43)
+    assert need > 0
+    ws = gpu.workspace(need)
+    first = gpu.sdpa_submit(*views, 3, 43, ws)
+    assert first > 0
+    assert gpu.sdpa_submit(*views, 3, 43, ws) == -4            # while it may still run
+    time.sleep(0.05)                                            # finished by now, not yet observed
+    assert gpu.snapshot() == (C_IN_FLIGHT, 0, 0)
+    assert gpu.sdpa_submit(*views, 3, 43, ws) == -4
+    assert gpu.wait(first) == 0 and gpu.wait(first) == 0
+    want = t[3].view().to_host()
+    again = gpu.sdpa_submit(*views, 3, 43, ws)                  # observed: the range is free again
+    assert again > 0 and gpu.wait(again) == 0, gpu.error()
+    assert np.array_equal(t[3].view().to_host(), want)
+    # never observed: the queue's end releases it
+    other = gpu.second_queue()
+    unseen = other.sdpa_submit(*views, 3, 43, ws)
+    assert unseen > 0
+    time.sleep(0.05)
+    assert gpu.sdpa_submit(*views, 3, 43, ws) == -4
+    other.close()
+    last = gpu.sdpa_submit(*views, 3, 43, ws)
+    assert last > 0 and gpu.wait(last) == 0, gpu.error()
+    gpu.drop_workspace(ws)
+    for x in t:
+        x.close()
+
+
 def test_a_failed_final_synchronisation_retains_the_whole_queue_lease(gpu):
     a, b = gpu.tensor(DT_F32, (32, 32)), gpu.tensor(DT_F32, (32, 32))
     doomed = gpu.second_queue()

@@ -69,3 +69,47 @@ def test_recorded_decode_step_replays_to_the_eager_result():
     for t in (x, wn, wq, wk, kc, vc, n1, q, qr, k, kr, attn, out, ws):
         t.free()
     st.close()
+
+
+def test_completion_word_arrives_after_the_work_before_it():
+    """iomx_stream_write_word: the host polls a page-locked word; once it holds the value,
+    everything submitted to the stream before it has finished and its results are visible."""
+    import ctypes as C
+    import time
+    L = iomx.lib()
+    iomx.check(L.iomx_set_device(0))
+    st = iomx.Stream()
+    cells = C.c_void_p()
+    iomx.check(L.iomx_host_alloc(C.byref(cells), 64))
+    word = C.cast(cells, C.POINTER(C.c_uint32))
+    word[0] = 0
+    on_device = C.c_void_p()
+    iomx.check(L.iomx_host_device_address(cells, C.byref(on_device)))
+    dims = (32, 512, 2048)                                  # 64 MiB per operand: tens of microseconds
+    n = int(np.prod(dims))
+    a, b, o = (iomx.DeviceTensor(DT_BF16, dims) for _ in range(3))
+    va = datagen.bf16_rne(datagen.normal_f32(n, 0, 1, 7)).reshape(dims)
+    vb = datagen.bf16_rne(datagen.normal_f32(n, 0, 1, 8)).reshape(dims)
+    a.view().from_host(va)
+    b.view().from_host(vb)
+    for ticket in (1, 2, 0xFFFFFFFF):
+        o.view().from_host(np.zeros(dims, np.uint16))
+        assert iomx.binary(ADD, a.view(), b.view(), o.view(), st) == 0
+        iomx.check(L.iomx_stream_write_word(st.h, on_device, ticket))
+        deadline = time.monotonic() + 10.0
+        while word[0] != ticket:
+            assert time.monotonic() < deadline, "the completion word never arrived"
+        got = o.buf.download(np.uint16)                     # no wait for the stream in between
+        want = iomx.DeviceTensor(DT_BF16, dims)
+        assert iomx.binary(ADD, a.view(), b.view(), want.view()) == 0
+        assert np.array_equal(got, want.raw())
+        want.free()
+    # a misaligned or null word is refused before anything is submitted
+    assert L.iomx_stream_write_word(st.h, None, 1) == -1
+    assert L.iomx_stream_write_word(st.h, C.c_void_p(on_device.value + 2), 1) == -1
+    assert L.iomx_host_device_address(None, C.byref(on_device)) == -1
+    st.synchronize()
+    for t in (a, b, o):
+        t.free()
+    iomx.check(L.iomx_host_free(cells))
+    st.close()
