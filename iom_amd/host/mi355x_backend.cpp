@@ -26,10 +26,10 @@
 #include <array>
 #include <atomic>
 #include <chrono>
-#include <cstring>
 #include <condition_variable>
 #include <cstddef>
 #include <cstdint>
+#include <cstring>
 #include <deque>
 #include <exception>
 #include <functional>
