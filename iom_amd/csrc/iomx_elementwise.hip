@@ -313,8 +313,11 @@ template <int DT, int OP, int LM, int RM, int SHAPE>
 __global__ __launch_bounds__(kPlanesBlock) void elementwise_stream_kernel(const FlatArgs a) {
     const uint64_t cb = (uint64_t)blockIdx.x * kPlanesBlock + threadIdx.x;
     if (cb >= a.seg_chunks) return;
+    // with a row-vector operand and a single segment (a plane of one band) FLAT and AXIS2 still
+    // need the lane's chunk of the vector
+    constexpr bool kVector = LM == MODE_ROWVEC || RM == MODE_ROWVEC;
     if constexpr (SHAPE == SHAPE_FLAT) {
-        stream_chunk<DT, OP, LM, RM>(a.src[0], a.src[1], a.out, cb * 16, 0);
+        stream_chunk<DT, OP, LM, RM>(a.src[0], a.src[1], a.out, cb * 16, kVector ? rowvec_offset<DT>(cb) : 0);
     } else if constexpr (SHAPE == SHAPE_BANDS) {
         const uint64_t voff = rowvec_offset<DT>(cb);
         for (uint32_t y = blockIdx.y; y < a.segments; y += gridDim.y)
@@ -343,7 +346,8 @@ __global__ __launch_bounds__(kPlanesBlock) void elementwise_stream_kernel(const 
             for (uint32_t y = blockIdx.y; y < a.n1; y += gridDim.y)
                 stream_chunk<DT, OP, LM, RM>(a.src[0] + z * a.step0[0] + y * a.step1[0],
                                              a.src[1] + z * a.step0[1] + y * a.step1[1],
-                                             a.out + z * a.step0[2] + y * a.step1[2], cb * 16, 0);
+                                             a.out + z * a.step0[2] + y * a.step1[2], cb * 16,
+                                             kVector ? rowvec_offset<DT>(cb) : 0);
     }
 }
 

@@ -193,6 +193,8 @@ ROWS_CASES = [
     ((2, 1, 16, 16), [], (1, 5, 16, 16), [], (2, 5, 16, 16), []),
     ((5, 64, 272), [], (5, 64, 272), [], (5, 64, 272), []),
     ((3, 40, 4112), [], (1, 4112), [], (3, 40, 4112), []),
+    ((16, 64), [], (1, 64), [], (16, 64), []),
+    ((4, 6, 16, 32), [("slice", (0, 0, 2, 2)), ("slice", (1, 1, 2, 2))], (2, 2, 1, 32), [], (2, 2, 16, 32), []),
 ]
 
 

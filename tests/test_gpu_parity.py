@@ -129,6 +129,14 @@ BINARY_CASES = [
     ((7, 3, 48, 80), [], (3, 1, 80), [], (7, 3, 48, 80), [], "binary_rowvec"),
     ((4, 160, 4112), [], (1, 4112), [], (4, 160, 4112), [], "binary_rowvec"),
     ((2, 16, 16), [], (1, 16), [], (2, 16, 16), [], "binary_rowvec"),
+    # a row vector against planes of a single band: the lane's chunk of the vector must still be
+    # found where the launch has no band axis (one plane; two strided leading axes)
+    ((16, 64), [], (1, 64), [], (16, 64), [], "binary_rowvec"),
+    ((1, 64), [], (16, 64), [], (16, 64), [], "binary_rowvec"),
+    ((4, 6, 16, 32), [("slice", (0, 0, 2, 2)), ("slice", (1, 1, 2, 2))], (2, 2, 1, 32), [],
+     (2, 2, 16, 32), [], "binary_rowvec"),
+    ((1, 3, 16, 48), [("slice", (1, 0, 2, 2))], (5, 2, 1, 48), [("slice", (0, 2, 2, 1))],
+     (4, 3, 16, 48), [("slice", (0, 0, 2, 2)), ("slice", (1, 0, 2, 2))], "binary_rowvec"),
 ]
 
 
