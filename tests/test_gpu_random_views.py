@@ -158,3 +158,353 @@ def test_rmsnorm_on_random_views(case):
     assert np.array_equal(got[~touched], want[~touched])
     for t in (dx, dw, do):
         t.free()
+
+
+# Row widths on both sides of every switch of the RMSNorm launch rule (chunks of one band:
+# 64, 256, ... 131072; a BF16 tile column is 32 chunks of a band, an F32 one 64), whole tiles
+# and ragged widths, with a partial last band and two planes.
+BOUNDARY_TILE_COLUMNS = sorted({t + d for t in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096)
+                                for d in (-1, 0, 1) if t + d >= 1})
+
+
+@pytest.mark.parametrize("dtype", [DT_BF16, DT_F32], ids=["BF16", "F32"])
+@pytest.mark.parametrize("tile_columns", BOUNDARY_TILE_COLUMNS)
+def test_rmsnorm_on_both_sides_of_every_launch_boundary(dtype, tile_columns):
+    for feats in (tile_columns * 16, tile_columns * 16 - 5):
+        dims = (2, 19, feats)
+        n = int(np.prod(dims))
+        x32 = datagen.normal_f32(n, 0, 1, 0x1100 + tile_columns)
+        w32 = datagen.uniform_f32(feats, 0.5, 1.5, 0x1200 + tile_columns)
+        enc = datagen.bf16_rne if dtype == DT_BF16 else (lambda v: v.view(np.uint32))
+        dx = iomx.DeviceTensor(dtype, dims, fill=0x5A)
+        hx = iomo.HostTensor(dtype, dims, fill=0x5A)
+        dx.view().from_host(enc(x32).reshape(dims))
+        hx.view().from_logical(enc(x32).reshape(dims))
+        dw = iomx.DeviceTensor(dtype, (1, feats), fill=0x5A)
+        hw = iomo.HostTensor(dtype, (1, feats), fill=0x5A)
+        dw.view().from_host(enc(w32).reshape(1, feats))
+        hw.view().from_logical(enc(w32).reshape(1, feats))
+        do, ho = pair(dtype, dims, 0x1300 + tile_columns)
+        assert iomx.rmsnorm(dx.view(), dw.view(), do.view(), 1e-5) == 0
+        assert iomo.rmsnorm(hx.view(), hw.view(), ho.view(), 1e-5) == 0
+        got, want = do.view().to_host(), ho.view().to_logical()
+        if dtype == DT_F32:
+            g, w = got.view(np.float32), want.view(np.float32)
+            assert np.all(np.abs(g - w) <= 1e-5 * np.abs(w) + 1e-30), (feats, iomx.last_launch().kernel)
+        else:
+            assert np.abs(got.astype(np.int64) - want.astype(np.int64)).max() <= 1, (feats, iomx.last_launch().kernel)
+        pad = iomo.tile_plane(np.ones(dims, ho.storage.dtype)) == 0
+        assert np.array_equal(do.raw()[pad], ho.storage[pad])
+        for t in (dx, dw, do):
+            t.free()
+
+
+def gpu_softmax(scores, a, L, scale, pcols):
+    scores = np.ascontiguousarray(scores, np.float32)
+    planes, heads, prow, scol = scores.shape
+    sb = iomx.Buffer(scores.nbytes)
+    pb = iomx.Buffer(planes * heads * prow * pcols * 2)
+    sb.upload(scores)
+    pb.fill(0xAA)
+    d = iomx.softmax_desc(sb.ptr.value, pb.ptr.value, planes, heads, prow, scol, a, L, scale, None)
+    d.probability_layout = iomx.dense_layout(heads, prow, pcols)
+    rc = iomx.softmax(d)
+    assert rc == 0, iomx.lib().iomx_error_string(rc)
+    iomx.synchronize()
+    out = pb.download(np.uint16).reshape(planes, heads, prow, pcols)
+    sb.free()
+    pb.free()
+    return out
+
+
+SOFTMAX_COLUMNS = sorted({c + d for c in (8, 256, 512, 1024, 2048, 4096) for d in (-4, -1, 0, 1, 4)} | {4, 5, 5000})
+
+
+@pytest.mark.parametrize("cols", SOFTMAX_COLUMNS)
+def test_softmax_on_both_sides_of_every_launch_boundary(cols):
+    """Row lengths around every switch of the softmax launch rule (chunks of 256 columns per
+    lane group: 256 ... 4096, then the generic kernel), lengths that are no multiple of four,
+    the causal limit inside the first chunk, inside a middle chunk and at the row's end, and a
+    probability row wider than the score row."""
+    planes, heads, rows = 2, 2, 9
+    shape = (planes, heads, rows, cols)
+    s = datagen.normal_f32(int(np.prod(shape)), 0, 3, 0x1400 + cols).reshape(shape)
+    r = np.arange(rows)[:, None]
+    t = np.arange(cols)[None, :]
+    for L, a in ((cols, cols - rows if cols > rows else 0), (max(cols - 3, 1), 0), (cols, max(cols // 2 - 4, 0))):
+        for pcols in (cols, cols + 4):
+            got = gpu_softmax(s, a, L, 0.125, pcols)
+            want = iomo.softmax(s, a=a, L=L, scale=0.125)
+            masked = np.broadcast_to((t > a + r) | (t >= L), shape)
+            view = got[..., :cols]
+            assert np.all(view[masked] == 0), (cols, L, a, pcols, iomx.last_launch().kernel)
+            assert np.all(got[..., cols:] == 0)
+            step = np.abs(view[~masked].astype(np.int64) - want[~masked].astype(np.int64))
+            assert step.max() <= 1, (cols, L, a, pcols, iomx.last_launch().kernel)
+
+
+def bf16_values(count, salt):
+    """BF16 encodings with exponents within 2^-3 .. 2^1: sums of a few hundred products stay far
+    from overflow and from total cancellation."""
+    v = datagen.pattern_bits(16, count, salt).astype(np.uint64)
+    exp = (v >> np.uint64(7)) & np.uint64(0xFF)
+    exp = exp % np.uint64(5) + np.uint64(124)
+    return ((v & np.uint64(0x807F)) | (exp << np.uint64(7))).astype(np.uint16)
+
+
+@pytest.mark.parametrize("case", range(160))
+def test_linear_bf16_on_random_shapes_and_views(case):
+    """Rows, inner extent, heads and head size drawn at random, so the choice among the scalar,
+    direct, split-inner and workgroup-tiled kernels and every ragged edge of their tiles is
+    exercised; x is reached through strided leading axes, the output is ordinary or head-planar
+    and pre-filled.  Bar: |actual - q| <= max(ulp(q), 2^-7, 2^-6 |q|) against float64 rounded once
+    (docs/BACKEND_CONTRACT/linear-projections.md:334-341); nothing outside the window changes."""
+    rng = view_cases.Stream(case, 505)
+    nlead = rng.below(3)
+    lead = tuple(1 + rng.below(3) for _ in range(nlead))
+    big = rng.chance(1, 4)
+    R = (1, 1, 3, 16, 17, 40, 130, 300)[rng.below(8 if big else 6)]
+    s = rng.below(20)
+    x_rows = s + R + rng.below(5)
+    inner = (16, 32, 40, 64, 96, 200, 256, 512, 1000)[rng.below(9 if big else 7)]
+    D = (16, 32, 48, 64, 80, 128)[rng.below(6)]
+    H = 1 + rng.below(8 if big else 4)
+    head_planar = rng.chance(1, 2)
+    x_owner, x_steps = view_cases.viewed_operand(rng, lead, x_rows, inner)
+    xv = bf16_values(int(np.prod(x_owner)), 0x1500 + case).reshape(x_owner)
+    wv = bf16_values(H * D * inner, 0x1600 + case).reshape(H * D, inner)
+    dx = iomx.DeviceTensor(DT_BF16, x_owner, fill=0x5A)
+    hx = iomo.HostTensor(DT_BF16, x_owner, fill=0x5A)
+    dx.view().from_host(xv)
+    hx.view().from_logical(xv)
+    dw = iomx.DeviceTensor(DT_BF16, (H * D, inner), fill=0x5A)
+    dw.view().from_host(wv)
+    out_dims = lead + ((H, R, D) if head_planar else (R, H * D))
+    do, ho = pair(DT_BF16, out_dims, 0x1700 + case)
+    dxv = view_cases.apply(dx.view(), x_steps)
+    # the ordinary layout is one head as wide as the weight (src/device_ops_neural.cpp)
+    rc = iomx.linear(dxv, dw.view(), do.view(), s, R, head_planar, H if head_planar else 1,
+                     D if head_planar else H * D)
+    assert rc == 0, (iomx.lib().iomx_error_string(rc), x_owner, x_steps, s, R, H, D, head_planar)
+    kernel = iomx.last_launch().kernel.decode()
+    got = do.view().to_host()
+    x_logical = view_cases.apply(hx.view(), x_steps).to_logical()
+    planes = int(np.prod(lead)) if lead else 1
+    x3 = x_logical.reshape(planes, x_rows, inner)[:, s:s + R, :]
+    g3 = (got.reshape(planes, H, R, D).transpose(0, 2, 1, 3).reshape(planes, R, H * D) if head_planar
+          else got.reshape(planes, R, H * D))
+    x64 = datagen.bf16_to_f32(x3.reshape(-1)).astype(np.float64).reshape(x3.shape)
+    w64 = datagen.bf16_to_f32(wv.reshape(-1)).astype(np.float64).reshape(wv.shape)
+    ref = x64 @ w64.T
+    q = datagen.bf16_to_f32(datagen.bf16_rne(ref.astype(np.float32).reshape(-1))).astype(np.float64).reshape(ref.shape)
+    g = datagen.bf16_to_f32(g3.reshape(-1)).astype(np.float64).reshape(ref.shape)
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(q), 1e-30))) - 7)
+    ok = np.abs(g - q) <= np.maximum(np.maximum(ulp, 2.0 ** -7), 2.0 ** -6 * np.abs(q))
+    assert ok.all(), (kernel, x_owner, x_steps, s, R, inner, H, D, head_planar, int((~ok).sum()))
+    pad = iomo.tile_plane(np.ones(out_dims, np.uint16)) == 0
+    assert np.array_equal(do.raw()[pad], ho.storage[pad]), kernel
+    for t in (dx, dw, do):
+        t.free()
+
+
+@pytest.mark.parametrize("case", range(120))
+def test_rope_on_random_views(case):
+    """Head sizes on both kernels' sides (D/2 a multiple of 16 or not), one row or many, any
+    start position, x and out reached through different strided views.  Bar: one leaf spacing
+    plus 2^-9 of the pair's norm against float64 (the CPU arithmetic differs from the device's
+    in the last place of sine and cosine); at most twice that from the oracle; the rest of the
+    output owner is what it was."""
+    rng = view_cases.Stream(case, 606)
+    dtype = DT_BF16 if case % 4 else DT_F32
+    nlead = 1 + rng.below(3)                         # rope needs rank >= 3
+    lead = tuple(1 + rng.below(4) for _ in range(nlead))
+    rows = (1, 1, 5, 16, 17, 33, 40)[rng.below(7)]
+    D = (2, 10, 32, 40, 64, 64, 96, 128, 160)[rng.below(9)]
+    a = (0, 0, 1, 7, 500, 4000)[rng.below(6)]
+    theta = (10000.0, 500000.0)[rng.below(2)]
+    xo, xs = view_cases.viewed_operand(rng, lead, rows, D)
+    oo, os_ = view_cases.viewed_operand(rng, lead, rows, D)
+    x32 = datagen.normal_f32(int(np.prod(xo)), 0, 1, 0x1800 + case)
+    enc = datagen.bf16_rne if dtype == DT_BF16 else (lambda v: v.view(np.uint32))
+    dx = iomx.DeviceTensor(dtype, xo, fill=0x5A)
+    hx = iomo.HostTensor(dtype, xo, fill=0x5A)
+    dx.view().from_host(enc(x32).reshape(xo))
+    hx.view().from_logical(enc(x32).reshape(xo))
+    do, ho = pair(dtype, oo, 0x1900 + case)
+    dxv, hxv = view_cases.apply(dx.view(), xs), view_cases.apply(hx.view(), xs)
+    dov, hov = view_cases.apply(do.view(), os_), view_cases.apply(ho.view(), os_)
+    rc = iomx.rope(dxv, dov, a, theta)
+    assert rc == 0, (iomx.lib().iomx_error_string(rc), xo, xs, oo, os_, a)
+    kernel = iomx.last_launch().kernel.decode()
+    assert iomo.rope(hxv, hov, a, theta) == 0
+    to64 = (lambda raw: datagen.bf16_to_f32(raw.reshape(-1)).astype(np.float64).reshape(raw.shape)) \
+        if dtype == DT_BF16 else (lambda raw: raw.view(np.float32).astype(np.float64))
+    x = to64(hxv.to_logical())
+    got, want = to64(dov.to_host()), to64(hov.to_logical())
+    half = D // 2
+    c = np.arange(half)
+    ang = (a + np.arange(rows))[:, None] * theta ** (-2.0 * c / D)[None, :]
+    x1, x2 = x[..., :half], x[..., half:]
+    ref = np.concatenate([x1 * np.cos(ang) - x2 * np.sin(ang), x2 * np.cos(ang) + x1 * np.sin(ang)], -1)
+    norm = np.sqrt(x1 * x1 + x2 * x2)
+    norm = np.concatenate([norm, norm], -1)
+    fbits = 7 if dtype == DT_BF16 else 23
+    spacing = np.ldexp(1.0, (np.floor(np.log2(np.maximum(np.abs(ref), 2.0 ** -126))) - fbits).astype(np.int64))
+    # positions in the thousands lose bits of the angle in binary32: 2^-9 of the norm covers it
+    bound = spacing + np.ldexp(norm, -9)
+    assert (np.abs(got - ref) <= bound).all(), (kernel, xo, xs, oo, os_, a, D)
+    assert (np.abs(got - want) <= 2 * bound).all(), (kernel, xo, xs, oo, os_, a, D)
+    marker = iomo.HostTensor(dtype, oo, fill=0)
+    mv = view_cases.apply(marker.view(), os_)
+    mv.from_logical(np.full(mv.dims, 1, iomo.NP_OF[dtype]))
+    untouched = marker.storage == 0
+    assert np.array_equal(do.raw()[untouched], ho.storage[untouched]), kernel
+    for t in (dx, do):
+        t.free()
+
+
+@pytest.mark.parametrize("case", range(120))
+def test_attention_on_random_shapes(case):
+    """Grouping, head size, new rows, prefix and cache capacity drawn at random: the decode
+    kernel and its shares, the four work mappings of the tiled kernel and the row kernel
+    (D > 128) each get ragged tiles, partial groups and rows that see one token or all.  Bar on
+    every element: the float64 evaluation within the BF16-probability budget
+    (test_gpu_sdpa.float64_attention); nothing outside the logical output is written."""
+    import test_gpu_sdpa as ts
+    rng = view_cases.Stream(case, 707)
+    lead = ((), (2,), (1, 3), (3,))[rng.below(4)]
+    grouping = (1, 2, 4, 8)[rng.below(4)]
+    Hkv = 1 + rng.below(4 if grouping < 8 else 2)
+    R = (1, 1, 2, 5, 16, 17, 33, 64, 70, 130)[rng.below(10)]
+    D = (16, 32, 48, 64, 64, 80, 96, 128, 128, 160)[rng.below(10)]
+    a = (0, 0, 3, 31, 32, 100, 500, 2100)[rng.below(8 if R <= 2 else 7)]
+    L = a + R - (rng.below(R) if rng.chance(1, 4) else 0)          # some rows see a truncated prefix
+    C = a + R + rng.below(40)                                       # the new rows fit the cache
+    spec = ts.random_case(0x2000 + case, lead, Hkv * grouping, Hkv, R, D, C, a, L)
+    got = ts.run(spec, 0, fill=0xFF)
+    ref64, budget = ts.float64_attention(spec)
+    g = datagen.bf16_to_f32(got.reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    worst = np.abs(g - ref64) - budget
+    assert np.all(worst <= 0), (iomx.last_launch().kernel, lead, Hkv, grouping, R, D, C, a, L, float(worst.max()))
+
+
+@pytest.mark.parametrize("case", range(100))
+def test_cache_append_on_random_views(case):
+    """R new rows written at position a of a cache of capacity C, any leaf, source and cache
+    reached through different strided views: the whole cache owner equals the oracle's bit for
+    bit (the rows before a, after a + R, the tile padding and the planes outside the view keep
+    their pre-filled bits)."""
+    rng = view_cases.Stream(case, 808)
+    dtype = (DT_BF16, DT_F32, DT_I8, DT_U4, DT_F16, DT_F6_E2M3, DT_I64, iomo.DT_BOOL)[case % 8]
+    nlead = 1 + rng.below(3)
+    lead = tuple(1 + rng.below(4) for _ in range(nlead))
+    R = (1, 1, 3, 16, 17, 40)[rng.below(6)]
+    D = (2, 16, 24, 64, 128)[rng.below(5)]
+    a = (0, 1, 15, 16, 37)[rng.below(5)]
+    capacity = a + R + rng.below(20)
+    so, ss = view_cases.viewed_operand(rng, lead, R, D)
+    co, cs = view_cases.viewed_operand(rng, lead, capacity, D)
+    ds, hs = pair(dtype, so, 0x2100 + case)
+    dc, hc = pair(dtype, co, 0x2200 + case)
+    rc = iomx.cache_append(view_cases.apply(ds.view(), ss), view_cases.apply(dc.view(), cs), a)
+    assert rc == 0, (iomx.lib().iomx_error_string(rc), so, ss, co, cs, a)
+    assert iomo.cache_append(view_cases.apply(hs.view(), ss), view_cases.apply(hc.view(), cs), a) == 0
+    assert same_storage(dc, hc), (LEAF_NAME[dtype], so, ss, co, cs, a, R, D)
+    assert same_storage(ds, hs)
+    ds.free()
+    dc.free()
+
+
+@pytest.mark.parametrize("case", range(100))
+def test_embedding_on_random_views(case):
+    """Rows of a [V,F] table gathered by ids of any integer leaf into [..., R, F]: ids and output
+    reached through strided views, table possibly one plane of a larger owner; payloads of any
+    leaf.  The whole output owner equals the oracle's and the status word stays clear."""
+    rng = view_cases.Stream(case, 909)
+    dtype = (DT_BF16, DT_F32, DT_I8, DT_U4, DT_F16, DT_F6_E2M3, DT_I64, iomo.DT_F8_E8M0)[case % 8]
+    index_dtype = (DT_I32, iomo.DT_U8, iomo.DT_I16, iomo.DT_U64, iomo.DT_U32, iomo.DT_I64)[rng.below(6)]
+    nlead = rng.below(3)
+    lead = tuple(1 + rng.below(4) for _ in range(nlead))
+    R = (1, 2, 9, 16, 21)[rng.below(5)]
+    F = (1, 16, 33, 40, 128, 300)[rng.below(6)]
+    V = (1, 7, 37, 100)[rng.below(4)]
+    io, isteps = view_cases.viewed_operand(rng, lead, 1, R)
+    oo, osteps = view_cases.viewed_operand(rng, lead, R, F)
+    to, tsteps = view_cases.viewed_operand(rng, (), V, F)
+    if rng.chance(1, 2):                              # the table as one plane of a rank-3 owner
+        planes = 2 + rng.below(2)
+        to, tsteps = (planes,) + to, [("select", (0, rng.below(planes)))] + tsteps
+    dt, ht = pair(dtype, to, 0x2300 + case)
+    ids = (datagen.pattern_bits(32, int(np.prod(io)), 0x2400 + case) % V).astype(iomo.NP_OF[index_dtype]).reshape(io)
+    di = iomx.DeviceTensor(index_dtype, io, fill=0x5A)
+    hi = iomo.HostTensor(index_dtype, io, fill=0x5A)
+    di.view().from_host(ids)
+    hi.view().from_logical(ids)
+    do, ho = pair(dtype, oo, 0x2500 + case)
+    status = iomx.Buffer(32)
+    status.fill(0xFF)
+    iomx.synchronize()
+    rc = iomx.embedding(view_cases.apply(dt.view(), tsteps), view_cases.apply(di.view(), isteps),
+                        view_cases.apply(do.view(), osteps), status)
+    assert rc == 0, (iomx.lib().iomx_error_string(rc), to, tsteps, io, isteps, oo, osteps)
+    iomx.synchronize()
+    assert int(status.download(np.uint32)[0]) == 0
+    assert iomo.embedding(view_cases.apply(ht.view(), tsteps), view_cases.apply(hi.view(), isteps),
+                          view_cases.apply(ho.view(), osteps)) == 0
+    assert same_storage(do, ho), (LEAF_NAME[dtype], LEAF_NAME[index_dtype], to, tsteps, io, isteps, oo, osteps)
+    status.free()
+    for t in (dt, di, do):
+        t.free()
+
+
+@pytest.fixture(scope="module")
+def devices():
+    if not iomo.mi355x_available():
+        pytest.skip("oracle/_ref/libiom_mi355x_shim.so not built (needs the reference headers)")
+    gpu = iomo.mi355x_backend(arena_bytes=1 << 28, max_in_flight=4)
+    cpu = iomo.cpu_backend_beside_mi355x()
+    yield cpu, gpu
+    gpu.close()
+    cpu.close()
+
+
+@pytest.mark.parametrize("case", range(200))
+def test_backend_binary_and_copy_on_random_views(devices, case):
+    """The same random views through `DeviceOps` on make_rocm_device and on the reference CPU
+    backend in one process: what the backend makes of a TensorView's snapshot (plane offset,
+    physical and result-aligned strides, broadcast flags) must lead to the bits the reference
+    computes.  Binary operations over every numeric leaf except F64 (whose CPU carrier rounds
+    twice) and, every fourth case, a copy."""
+    cpu, gpu = devices
+    leaves = [d for d in iomo.NUMERIC_LEAVES if d != DT_F64]
+    dtype = leaves[case % len(leaves)]
+    op = (OP_ADD, OP_MUL, OP_SUB, OP_DIV)[(case // len(leaves)) % 4]
+    if op == OP_DIV and dtype not in FLOAT_LEAVES:
+        op = OP_MUL
+    if case % 4 == 3:
+        lead, rows, cols, operands = view_cases.unary_case(case)
+    else:
+        lead, rows, cols, operands = view_cases.binary_case(case)
+    tensors = []
+    for i, (dims, _) in enumerate(operands):
+        values = datagen.pattern_bits(LEAF_BITS[dtype], int(np.prod(dims)), 0x2600 + 3 * case + i).reshape(dims)
+        pairs = []
+        for dev in (cpu, gpu):
+            t = dev.tensor(dtype, dims)
+            t.view().from_host(values)
+            pairs.append(t)
+        tensors.append(pairs)
+    cv = [view_cases.apply(t[0].view(), steps) for t, (_, steps) in zip(tensors, operands)]
+    gv = [view_cases.apply(t[1].view(), steps) for t, (_, steps) in zip(tensors, operands)]
+    if case % 4 == 3:
+        tc, tg = cpu.copy(cv[0], cv[1]), gpu.copy(gv[0], gv[1])
+    else:
+        tc, tg = cpu.binary(op, cv[0], cv[1], cv[2]), gpu.binary(op, gv[0], gv[1], gv[2])
+    assert tc > 0 and tg > 0, (tc, tg, gpu.error(), LEAF_NAME[dtype], operands)
+    out = tensors[-1]
+    # the whole output owner, read back through each backend's own host transfer
+    assert np.array_equal(out[0].view().to_host(), out[1].view().to_host()), \
+        (LEAF_NAME[dtype], op, lead, rows, cols, operands)
+    for pairs in tensors:
+        for t in pairs:
+            t.close()
