@@ -508,3 +508,72 @@ def test_backend_binary_and_copy_on_random_views(devices, case):
     for pairs in tensors:
         for t in pairs:
             t.close()
+
+
+GRID_LIMIT_CASES = [
+    # (leaf, lhs owner, lhs steps, rhs owner, rhs steps, out owner, out steps): each has more planes,
+    # bands or (plane, band) pairs than the 65535 a grid axis holds, so the kernels' own loops run
+    ("BANDS", DT_BF16, (16 * 70000, 16), [], (1, 16), [], (16 * 70000, 16), []),
+    ("AXIS1", DT_BF16, (140000, 16, 16), [("slice", (0, 1, 70000, 2))], (70000, 16, 16), [], (70000, 16, 16), []),
+    ("AXIS2B", DT_BF16, (2, 1400, 1600, 16), [("slice", (1, 0, 700, 2))], (1, 16), [], (2, 700, 1600, 16), []),
+    ("PLANES", DT_F32, (50, 80, 42, 16, 16), [("slice", (1, 0, 40, 2)), ("slice", (2, 1, 40, 1))], (40, 1, 16, 16), [],
+     (50, 40, 40, 16, 16), []),
+    ("padded", DT_I32, (70000, 17, 16), [], (17, 1), [], (70000, 17, 16), []),
+    ("rows", DT_U4, (70000, 16, 16), [], (1, 16), [], (70000, 16, 16), []),
+    ("general", DT_F16, (1, 16), [], (70000, 16, 1), [], (70000, 16, 16), []),
+]
+
+
+@pytest.mark.parametrize("case", range(len(GRID_LIMIT_CASES)), ids=[c[0] for c in GRID_LIMIT_CASES])
+def test_more_planes_or_bands_than_a_grid_axis_holds(case):
+    _, dtype, ld, ls, rd, rs, od, os_ = GRID_LIMIT_CASES[case]
+    dl, hl = pair(dtype, ld, 0x2700 + case)
+    dr, hr = pair(dtype, rd, 0x2800 + case)
+    do, ho = pair(dtype, od, 0x2900 + case)
+    rc = iomx.binary(OP_ADD, view_cases.apply(dl.view(), ls), view_cases.apply(dr.view(), rs),
+                     view_cases.apply(do.view(), os_))
+    assert rc == 0, iomx.lib().iomx_error_string(rc)
+    kernel = iomx.last_launch().kernel.decode()
+    assert iomo.binary(OP_ADD, view_cases.apply(hl.view(), ls), view_cases.apply(hr.view(), rs),
+                       view_cases.apply(ho.view(), os_), ieee=True) == 0
+    assert same_storage(do, ho), kernel
+    # and a copy of the same output window back over the left operand's window where shapes agree
+    if tuple(view_cases.apply(hl.view(), ls).dims) == tuple(view_cases.apply(ho.view(), os_).dims):
+        assert iomx.copy(view_cases.apply(do.view(), os_), view_cases.apply(dl.view(), ls)) == 0
+        assert iomo.copy(view_cases.apply(ho.view(), os_), view_cases.apply(hl.view(), ls)) == 0
+        assert same_storage(dl, hl), iomx.last_launch().kernel.decode()
+    for t in (dl, dr, do):
+        t.free()
+
+
+def test_row_kernels_with_more_bands_or_planes_than_a_grid_axis_holds():
+    """RMSNorm and SiLU over 70000 bands of one plane and over 70000 planes of one band, RoPE
+    over 70000 planes: every grid these launches use has an axis that stops at 65535."""
+    for dims in ((16 * 70000, 32), (70000, 16, 32)):
+        n = int(np.prod(dims))
+        x = datagen.bf16_rne(datagen.normal_f32(n, 0, 1, 0x2A00)).reshape(dims)
+        w = datagen.bf16_rne(datagen.uniform_f32(32, 0.5, 1.5, 0x2A01)).reshape(1, 32)
+        dx = iomx.DeviceTensor(DT_BF16, dims)
+        hx = iomo.HostTensor(DT_BF16, dims)
+        dx.view().from_host(x)
+        hx.view().from_logical(x)
+        dw = iomx.DeviceTensor(DT_BF16, (1, 32))
+        hw = iomo.HostTensor(DT_BF16, (1, 32))
+        dw.view().from_host(w)
+        hw.view().from_logical(w)
+        do, ho = pair(DT_BF16, dims, 0x2A02)
+        assert iomx.rmsnorm(dx.view(), dw.view(), do.view(), 1e-5) == 0
+        assert iomo.rmsnorm(hx.view(), hw.view(), ho.view(), 1e-5) == 0
+        assert np.abs(do.raw().astype(np.int64) - ho.storage.astype(np.int64)).max() <= 1
+        assert iomx.silu(dx.view(), do.view()) == 0
+        assert iomo.silu(hx.view(), ho.view()) == 0
+        assert np.abs(do.raw().astype(np.int64) - ho.storage.astype(np.int64)).max() <= 1
+        if len(dims) == 3:
+            assert iomx.rope(dx.view(), do.view(), 3, 10000.0) == 0
+            assert iomo.rope(hx.view(), ho.view(), 3, 10000.0) == 0
+            got = datagen.bf16_to_f32(do.raw()).astype(np.float64)
+            want = datagen.bf16_to_f32(ho.storage).astype(np.float64)
+            assert np.all(np.abs(got - want) <= 2.0 ** -6 * np.maximum(np.abs(want), 1.0))
+            assert float((do.raw() == ho.storage).mean()) > 0.9
+        for t in (dx, dw, do):
+            t.free()
