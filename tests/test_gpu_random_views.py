@@ -577,3 +577,23 @@ def test_row_kernels_with_more_bands_or_planes_than_a_grid_axis_holds():
             assert float((do.raw() == ho.storage).mean()) > 0.9
         for t in (dx, dw, do):
             t.free()
+
+
+@pytest.mark.parametrize("case", range(120))
+def test_host_transfer_on_random_views(case):
+    """Logical row-major bytes written through a strided view land in the slots the oracle's
+    layout rule names and nowhere else (every leaf, ragged tiles), and read back unchanged."""
+    dtype = iomo.ALL_LEAVES[case % len(iomo.ALL_LEAVES)]
+    lead, rows, cols, operands = view_cases.unary_case(case, salt=1010)
+    dims, steps = operands[0]
+    dt, ht = pair(dtype, dims, 0x2B00 + case)
+    dv, hv = view_cases.apply(dt.view(), steps), view_cases.apply(ht.view(), steps)
+    values = datagen.pattern_bits(LEAF_BITS[dtype], int(np.prod(hv.dims)), 0x2C00 + case).reshape(hv.dims)
+    if dtype == iomo.DT_BOOL:
+        values = values & 1
+    dv.from_host(values)
+    hv.from_logical(values)
+    assert same_storage(dt, ht), (LEAF_NAME[dtype], dims, steps)
+    assert np.array_equal(dv.to_host(), values)
+    assert np.array_equal(dt.view().to_host(), ht.view().to_logical())
+    dt.free()
