@@ -597,3 +597,57 @@ def test_host_transfer_on_random_views(case):
     assert np.array_equal(dv.to_host(), values)
     assert np.array_equal(dt.view().to_host(), ht.view().to_logical())
     dt.free()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_backend_random_operation_sequences_keep_queue_order(devices, seed):
+    """150 dependent operations on a pool of eight owners, submitted without waiting (four
+    credits, so most are parked and started from the completion thread), every result feeding
+    later ones through views: at the end all owners equal what the reference CPU backend holds
+    after the same sequence.  Only bit-exact operations (ADD / MUL / SUB / DIV with exact-alias
+    in-place forms, copy between disjoint windows)."""
+    cpu, gpu = devices
+    rng = view_cases.Stream(seed, 1111)
+    dtype = (DT_F32, DT_BF16, DT_I32)[seed % 3]
+    dims = (4, 17, 33)
+    pool = []
+    for i in range(8):
+        values = datagen.pattern_bits(LEAF_BITS[dtype], int(np.prod(dims)), 0x2D00 + 8 * seed + i).reshape(dims)
+        if dtype != DT_I32:
+            # moderate magnitudes: long products stay finite for a while, then saturate alike
+            enc = datagen.bf16_rne if dtype == DT_BF16 else (lambda v: v.view(np.uint32))
+            values = enc(datagen.normal_f32(int(np.prod(dims)), 0, 1, 0x2E00 + 8 * seed + i)).reshape(dims)
+        pair_ = []
+        for dev in (cpu, gpu):
+            t = dev.tensor(dtype, dims)
+            t.view().from_host(values)
+            pair_.append(t)
+        pool.append(pair_)
+    windows = [lambda v: v, lambda v: v.slice(0, 0, 2, 2), lambda v: v.slice(0, 1, 2, 2), lambda v: v.slice(0, 2, 2, 1)]
+    tokens = []
+    for step in range(150):
+        kind = rng.below(5)
+        out, a, b = rng.below(8), rng.below(8), rng.below(8)
+        w = windows[rng.below(4)] if kind != 4 else windows[1 + rng.below(3)]
+        for which, dev in enumerate((cpu, gpu)):
+            ov = w(pool[out][which].view())
+            if kind == 4:                                  # copy from another owner's window
+                src = a if a != out else (out + 1) % 8
+                tok = dev.l.iomc_copy(dev.queue, w(pool[src][which].view()).h, ov.h)
+            else:
+                op = (OP_ADD, OP_MUL, OP_SUB, OP_DIV if dtype != DT_I32 else OP_ADD)[kind]
+                # an input that is the output owner must be the identical window (exact alias)
+                tok = dev.l.iomc_binary(dev.queue, op, w(pool[a][which].view()).h, w(pool[b][which].view()).h, ov.h)
+            assert tok > 0, (step, kind, tok, dev.error())
+            if which == 1:
+                tokens.append(tok)
+            else:
+                assert cpu.wait(tok) == 0
+    for tok in tokens:
+        assert gpu.wait(tok) == 0, gpu.error()
+    assert gpu.snapshot()[1:] == (0, 0)
+    for i, (c, g) in enumerate(pool):
+        assert np.array_equal(c.view().to_host(), g.view().to_host()), (seed, i)
+    for c, g in pool:
+        c.close()
+        g.close()
