@@ -102,8 +102,11 @@ def test_silu_on_random_views(case):
     assert iomo.silu(hxv, hov) == 0
     got, want = dov.to_host(), hov.to_logical()
     if dtype == DT_F32:
-        g, w = got.view(np.float32), want.view(np.float32)
-        assert np.all(np.abs(g - w) <= 4e-7 * np.abs(w) + 1e-37), (lead, rows, cols, operands)
+        # each side is within 4 binary32 units of the exact value (test_scalar_silu.cpp:163-167)
+        def ordered(bits):
+            b = bits.astype(np.int64)
+            return np.where(b & 0x80000000, 0x80000000 - b, b)
+        assert np.abs(ordered(got) - ordered(want)).max() <= 8, (lead, rows, cols, operands)
     elif dtype == DT_F64:
         g, w = got.view(np.float64), want.view(np.float64)
         assert np.all(np.abs(g - w) <= 1e-6 * np.abs(w) + 1e-300), (lead, rows, cols, operands)

@@ -68,8 +68,8 @@ def binary_case(case: int):
     rng = Stream(case, 101)
     nlead = rng.below(4)
     lead = tuple(1 + rng.below(4) for _ in range(nlead))
-    rows = (1, 5, 15, 16, 17, 33)[rng.below(6)]
-    cols = (1, 7, 16, 17, 31, 48)[rng.below(6)]
+    rows = (1, 5, 15, 16, 17, 33, 32, 48)[rng.below(8)]
+    cols = (1, 7, 16, 17, 31, 48, 256, 1040)[rng.below(8)]
     # every axis of the result is held in full by at least one input (the output shape is
     # exactly the broadcast of the two); the other input may have extent 1 there
     shape = lead + (rows, cols)
@@ -97,8 +97,8 @@ def unary_case(case: int, salt: int = 202):
     rng = Stream(case, salt)
     nlead = rng.below(4)
     lead = tuple(1 + rng.below(4) for _ in range(nlead))
-    rows = (1, 5, 15, 16, 17, 33)[rng.below(6)]
-    cols = (2, 8, 16, 18, 32, 48)[rng.below(6)]
+    rows = (1, 5, 15, 16, 17, 33, 32, 48)[rng.below(8)]
+    cols = (2, 8, 16, 18, 32, 48, 256, 1040)[rng.below(8)]
     return lead, rows, cols, [viewed_operand(rng, lead, rows, cols), viewed_operand(rng, lead, rows, cols)]
 
 
