@@ -8,6 +8,8 @@ bit-exact (F64 against the binary64-carrier rule); RMSNorm is within one encodin
 leaf / 1e-5 relative.  The same cases run between the oracle and the compiled reference in
 test_oracle_random_views.py.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -654,3 +656,68 @@ def test_backend_random_operation_sequences_keep_queue_order(devices, seed):
     for c, g in pool:
         c.close()
         g.close()
+
+
+@pytest.mark.parametrize("case", range(100))
+def test_softmax_stage_on_random_layouts(case):
+    """The stage's two layouts drawn at random: row, head and plane strides with gaps, a plane
+    offset, a column stride of 1 or 2, a probability region with more physical rows and columns
+    than the logical extent, alignments that allow the row kernel or force the generic one.
+    Both buffers are flat and pre-filled; the oracle runs on the same layouts, so the whole
+    probability buffer is compared: written entries within one BF16 step (masked ones exactly
+    +0), every other element untouched."""
+    rng = view_cases.Stream(case, 1212)
+    planes, heads = 1 + rng.below(3), 1 + rng.below(3)
+    rows = (1, 4, 9, 17)[rng.below(4)]
+    cols = (4, 5, 64, 250, 256, 300, 1024, 1100)[rng.below(8)]
+    a = (0, 0, 3, 40)[rng.below(4)]
+    L = min(cols, a + rows) if rng.chance(1, 2) else cols
+    L = max(L, 1)
+
+    def layout(phys_rows, phys_cols):
+        l = iomx.StageLayout()
+        l.column_stride = 2 if rng.chance(1, 6) else 1
+        quantum = 4 if rng.chance(2, 3) else 1                       # multiples of 4 keep the row kernel
+        l.row_stride = phys_cols * l.column_stride + quantum * rng.below(4)
+        l.head_stride = phys_rows * l.row_stride + quantum * rng.below(5)
+        l.plane_stride = heads * l.head_stride + quantum * rng.below(5)
+        l.plane_offset = quantum * rng.below(6)
+        l.rows, l.columns = phys_rows, phys_cols
+        size = l.plane_offset + planes * l.plane_stride + 8
+        return l, int(size)
+    sl, s_size = layout(rows, cols)
+    pl, p_size = layout(rows + rng.below(3), cols + (0, 0, 4, 7)[rng.below(4)])
+    logical = datagen.normal_f32(planes * heads * rows * cols, 0, 3, 0x2F00 + case).reshape(planes, heads, rows, cols)
+    flat = np.full(s_size, np.nan, np.float32)
+    idx = (sl.plane_offset + np.arange(planes)[:, None, None, None] * sl.plane_stride
+           + np.arange(heads)[None, :, None, None] * sl.head_stride
+           + np.arange(rows)[None, None, :, None] * sl.row_stride
+           + np.arange(cols)[None, None, None, :] * sl.column_stride)
+    flat[idx] = logical
+    want = np.full(p_size, 0xAAAA, np.uint16)
+    d = iomo.SoftmaxDesc()
+    d.planes, d.heads, d.rows, d.a, d.L, d.scale = planes, heads, rows, a, L, 0.125
+    d.scores, d.p_bf16 = flat.ctypes.data, want.ctypes.data
+    for name in ("plane_offset", "plane_stride", "head_stride", "row_stride", "column_stride", "rows", "columns"):
+        setattr(d.scores_layout, name, getattr(sl, name))
+        setattr(d.probability_layout, name, getattr(pl, name))
+    assert iomo.lib().iomo_softmax(ctypes.byref(d)) == 0
+    sb, pb = iomx.Buffer(flat.nbytes), iomx.Buffer(want.nbytes)
+    sb.upload(flat)
+    pb.upload(np.full(p_size, 0xAAAA, np.uint16))
+    g = iomx.SoftmaxDesc()
+    g.planes, g.heads, g.rows, g.a, g.L, g.scale = planes, heads, rows, a, L, 0.125
+    g.scores, g.p_bf16 = sb.ptr.value, pb.ptr.value
+    g.scores_layout, g.probability_layout = sl, pl
+    rc = iomx.softmax(g)
+    assert rc == 0, iomx.lib().iomx_error_string(rc)
+    iomx.synchronize()
+    kernel = iomx.last_launch().kernel.decode()
+    got = pb.download(np.uint16)
+    untouched = want == 0xAAAA
+    assert np.array_equal(got[untouched], want[untouched]), (kernel, planes, heads, rows, cols, a, L)
+    assert np.array_equal(got == 0, want == 0), kernel
+    step = np.abs(got[~untouched].astype(np.int64) - want[~untouched].astype(np.int64))
+    assert step.max() <= 1, (kernel, planes, heads, rows, cols, a, L, int(step.max()))
+    sb.free()
+    pb.free()
