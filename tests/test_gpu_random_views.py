@@ -721,3 +721,54 @@ def test_softmax_stage_on_random_layouts(case):
     assert step.max() <= 1, (kernel, planes, heads, rows, cols, a, L, int(step.max()))
     sb.free()
     pb.free()
+
+
+@pytest.mark.parametrize("case", range(80))
+def test_attention_through_random_views(case):
+    """q, k, v and out each reached through their own select / strided slice / permute of the
+    leading axes (the head axis included), pre-filled owners: the float64 budget on every
+    element, and nothing of the output owner outside the window changes."""
+    import test_gpu_sdpa as ts
+    rng = view_cases.Stream(case, 1313)
+    lead = ((), (2,), (2, 2), (3,))[rng.below(4)]
+    grouping = (1, 2, 4)[rng.below(3)]
+    Hkv = 1 + rng.below(3)
+    Hq = Hkv * grouping
+    R = (1, 3, 16, 20, 40)[rng.below(5)]
+    D = (16, 32, 64, 128)[rng.below(4)]
+    a = (0, 2, 31, 100)[rng.below(4)]
+    L = a + R
+    cap = L + rng.below(20)
+    spec = ts.random_case(0x3000 + case, lead, Hq, Hkv, R, D, cap, a, L)
+    qd, kd, od = ts.shapes(spec)
+    owners, views = [], []
+    for name, dims in (("q", qd), ("k", kd), ("v", kd), (None, od)):
+        owner_dims, steps = view_cases.viewed_operand(rng, dims[:-2], dims[-2], dims[-1])
+        t = iomx.DeviceTensor(DT_BF16, owner_dims, fill=0xFF)
+        view = view_cases.apply(t.view(), steps)
+        if name:
+            view.from_host(np.array(spec[name], np.uint16).reshape(dims))
+        owners.append((t, owner_dims, steps))
+        views.append(view)
+    out_owner, out_dims, out_steps = owners[3]
+    before = out_owner.raw().copy()
+    rc, nbytes, _ = iomx.sdpa_workspace(views[0], views[1], views[2], views[3], a, L)
+    assert rc == 0
+    ws = iomx.Buffer(nbytes) if nbytes else None
+    rc = iomx.sdpa(views[0], views[1], views[2], views[3], a, L, ws)
+    assert rc == 0, (iomx.lib().iomx_error_string(rc), [o[1:] for o in owners])
+    iomx.synchronize()
+    kernel = iomx.last_launch().kernel.decode()
+    got = views[3].to_host()
+    ref64, budget = ts.float64_attention(spec)
+    g = datagen.bf16_to_f32(got.reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    assert np.all(np.abs(g - ref64) <= budget), (kernel, [o[1:] for o in owners])
+    marker = iomo.HostTensor(DT_BF16, out_dims, fill=0)
+    mv = view_cases.apply(marker.view(), out_steps)
+    mv.from_logical(np.full(mv.dims, 1, np.uint16))
+    untouched = marker.storage == 0
+    assert np.array_equal(out_owner.raw()[untouched], before[untouched]), kernel
+    for t, _, _ in owners:
+        t.free()
+    if ws:
+        ws.free()
