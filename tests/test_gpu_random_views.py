@@ -772,3 +772,45 @@ def test_attention_through_random_views(case):
         t.free()
     if ws:
         ws.free()
+
+
+@pytest.mark.parametrize("case", range(105))
+def test_linear_scalar_recurrence_on_random_shapes_and_views(case):
+    """The contract's scalar recurrence (every numeric leaf; the path of everything that is not
+    BF16) on random shapes, row windows and strided x and out views: bit for bit against the
+    oracle over the whole output owner."""
+    import test_gpu_linear as tl
+    rng = view_cases.Stream(case, 1414)
+    dtype = iomo.NUMERIC_LEAVES[case % len(iomo.NUMERIC_LEAVES)]
+    nlead = rng.below(3)
+    lead = tuple(1 + rng.below(3) for _ in range(nlead))
+    R = (1, 3, 16, 17, 33)[rng.below(5)]
+    s = rng.below(6)
+    x_rows = s + R + rng.below(4)
+    inner = (1, 3, 16, 40, 65)[rng.below(5)]
+    D = (1, 5, 16, 17, 33)[rng.below(5)]
+    H = 1 + rng.below(3)
+    head_planar = rng.chance(1, 2)
+    xo, xs = view_cases.viewed_operand(rng, lead, x_rows, inner)
+    out_lead = lead + ((H,) if head_planar else ())
+    oo, os_ = view_cases.viewed_operand(rng, out_lead, R, D if head_planar else H * D)
+    dx, hx = tl.pair(dtype, xo, values=tl.small_values(dtype, int(np.prod(xo)), 0x3100 + case).reshape(xo))
+    dw, hw = tl.pair(dtype, (H * D, inner), values=tl.small_values(dtype, H * D * inner, 0x3200 + case).reshape(H * D, inner))
+    do, ho = tl.pair(dtype, oo, salt=0x3300 + case)
+    args = (s, R, head_planar, H if head_planar else 1, D if head_planar else H * D)
+    rc = iomx.linear(view_cases.apply(dx.view(), xs), dw.view(), view_cases.apply(do.view(), os_), *args,
+                     path=0 if dtype == DT_BF16 and case % 2 else 1)
+    assert rc == 0, (iomx.lib().iomx_error_string(rc), LEAF_NAME[dtype], xo, xs, oo, os_, args)
+    kernel = iomx.last_launch().kernel.decode()
+    assert iomo.linear(view_cases.apply(hx.view(), xs), hw.view(), view_cases.apply(ho.view(), os_), *args) == 0
+    if kernel == "linear_rows":
+        assert same_storage(do, ho), (LEAF_NAME[dtype], xo, xs, oo, os_, args)
+    else:                                             # BF16 on the matrix cores: the owner outside the window
+        marker = iomo.HostTensor(dtype, oo, fill=0)
+        mv = view_cases.apply(marker.view(), os_)
+        mv.from_logical(np.full(mv.dims, 1, np.uint16))
+        untouched = marker.storage == 0
+        assert np.array_equal(do.raw()[untouched], ho.storage[untouched]), kernel
+        # (values on this path: test_linear_bf16_on_random_shapes_and_views, against float64)
+    for t in (dx, dw, do):
+        t.free()
