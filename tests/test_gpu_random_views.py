@@ -814,3 +814,69 @@ def test_linear_scalar_recurrence_on_random_shapes_and_views(case):
         # (values on this path: test_linear_bf16_on_random_shapes_and_views, against float64)
     for t in (dx, dw, do):
         t.free()
+
+
+@pytest.mark.parametrize("case", range(150))
+def test_rejections_on_random_views(case):
+    """A valid random binary request, then one thing wrong with it: the library refuses it with
+    the class the reference's validation order gives (src/device_ops_binary.cpp:102-181: shape
+    and broadcast and alias errors are invalid_argument = -1 and come before the leaf's
+    Unsupported = -2), launches nothing and leaves every owner as it was."""
+    rng = view_cases.Stream(case, 1717)
+    dtype = (DT_F32, DT_BF16, DT_I32, DT_U4, DT_F16)[case % 5]
+    lead, rows, cols, operands = view_cases.binary_case(case)
+    owners = [pair(dtype, dims, 0x3400 + 3 * case + i) for i, (dims, _) in enumerate(operands)]
+    dv = [view_cases.apply(d.view(), steps) for (d, _), (_, steps) in zip(owners, operands)]
+    hv = [view_cases.apply(h.view(), steps) for (_, h), (_, steps) in zip(owners, operands)]
+    kind = case % 6
+    op, code, expect = OP_ADD, dtype, -1
+    extra = []
+    if kind == 0:                                     # output one row short or one plane long
+        bad = list(operands[2][0])
+        bad[-2 if rng.chance(1, 2) or len(bad) == 2 else 0] += 1
+        t = pair(dtype, tuple(bad), 0x3500 + case)
+        extra.append(t)
+        dv[2], hv[2] = t[0].view(), t[1].view()
+    elif kind == 1:                                   # an input that cannot broadcast
+        bad = list(dv[0].dims)
+        bad[-1] = cols + 2
+        t = pair(dtype, tuple(bad), 0x3600 + case)
+        extra.append(t)
+        dv[0], hv[0] = t[0].view(), t[1].view()
+    elif kind == 2:                                   # an input inside the output's owner, other window
+        dims = (2,) + tuple(dv[2].dims)
+        t = pair(dtype, dims, 0x3700 + case)
+        extra.append(t)
+        dv[2], hv[2] = t[0].view().select(0, 0), t[1].view().select(0, 0)
+        if tuple(dv[0].dims) == tuple(dv[2].dims):
+            dv[0], hv[0] = t[0].view().select(0, 1), t[1].view().select(0, 1)
+        else:
+            dv[1], hv[1] = dv[2], hv[2]               # a broadcasting input may not alias at all
+            if tuple(dv[1].dims) == tuple(dv[2].dims) and tuple(dv[0].dims) == tuple(dv[2].dims):
+                expect = 0
+    elif kind == 3:                                   # a leaf without arithmetic
+        code, expect = (iomo.DT_BOOL, iomo.DT_F8_E8M0)[rng.below(2)], -2
+    elif kind == 4:                                   # integer division: refused after the shape checks
+        op = OP_DIV
+        expect = -2 if dtype in (DT_I32, DT_U4) else 0
+    else:                                             # unknown operation
+        op = 4 + rng.below(100)
+    before = [d.raw().copy() for d, _ in owners + extra]
+    if kind == 3:
+        a, b, o = (v.cview() for v in dv)
+        rc = iomx.lib().iomx_launch_binary(op, code, ctypes.byref(a), ctypes.byref(b), ctypes.byref(o), None)
+    else:
+        rc = iomx.binary(op, dv[0], dv[1], dv[2])
+    if kind == 2 and expect == -1:
+        # whether the request is an exact alias (allowed) depends on the drawn shapes: decide by rule
+        same = [tuple(v.dims) == tuple(dv[2].dims) and v.owner is dv[2].owner and v.plane_offset == dv[2].plane_offset
+                and tuple(v.plane_strides) == tuple(dv[2].plane_strides) for v in dv[:2]]
+        shares = [v.owner is dv[2].owner for v in dv[:2]]
+        expect = -1 if any(s and not e for s, e in zip(shares, same)) else 0
+    assert rc == expect, (kind, rc, expect, LEAF_NAME[dtype], operands)
+    if expect != 0:
+        iomx.synchronize()
+        for (d, _), image in zip(owners + extra, before):
+            assert np.array_equal(d.raw(), image)
+    for d, _ in owners + extra:
+        d.free()
