@@ -880,3 +880,120 @@ def test_rejections_on_random_views(case):
             assert np.array_equal(d.raw(), image)
     for d, _ in owners + extra:
         d.free()
+
+
+def on_both(devices, dtype, dims, values):
+    out = []
+    for dev in devices:
+        t = dev.tensor(dtype, dims)
+        t.view().from_host(values)
+        out.append(t)
+    return out
+
+
+def prefilled(devices, dtype, dims, salt):
+    values = datagen.pattern_bits(LEAF_BITS[dtype], int(np.prod(dims)), salt).reshape(dims)
+    if dtype == iomo.DT_BOOL:
+        values = values & 1
+    return on_both(devices, dtype, dims, values)
+
+
+def bf16_steps(a, b):
+    return np.abs(a.astype(np.int64) - b.astype(np.int64))
+
+
+@pytest.mark.parametrize("case", range(120))
+def test_backend_layer_operations_on_random_views(devices, case):
+    """RMSNorm, SiLU, RoPE, cache append, embedding and the linear projection through `DeviceOps`
+    on make_rocm_device and on the reference CPU backend, operands reached through random views:
+    every hook turns its own kind of request snapshot into kernel arguments, and each must lead
+    to what the reference computes (data movement bit for bit; RMSNorm and SiLU within one BF16
+    step; RoPE within two; linear within the contract's bound of either result)."""
+    cpu, gpu = devices
+    rng = view_cases.Stream(case, 1818)
+    kind = case % 6
+    nlead = 1 + rng.below(2)
+    lead = tuple(1 + rng.below(3) for _ in range(nlead))
+    R = (1, 3, 16, 17, 33)[rng.below(5)]
+    D = (16, 32, 64, 128)[rng.below(4)]
+    dt = DT_BF16
+    x32 = lambda n, s: datagen.bf16_rne(datagen.normal_f32(n, 0, 1, s))
+    closing = []
+
+    def make(dims, values=None, salt=None):
+        pair_ = on_both(devices, dt, dims, values) if values is not None else prefilled(devices, dt, dims, salt)
+        closing.extend(pair_)
+        return pair_
+    if kind in (0, 1, 2):                                   # rmsnorm / silu / rope: x -> out, same shape
+        xo, xs = view_cases.viewed_operand(rng, lead, R, D)
+        oo, os_ = view_cases.viewed_operand(rng, lead, R, D)
+        x = make(xo, x32(int(np.prod(xo)), 0x3800 + case).reshape(xo))
+        o = make(oo, salt=0x3900 + case)
+        xv = [view_cases.apply(t.view(), xs) for t in x]
+        ov = [view_cases.apply(t.view(), os_) for t in o]
+        if kind == 0:
+            w = make((1, D), x32(D, 0x3A00 + case).reshape(1, D))
+            tokens = [dev.rmsnorm(xv[i], w[i].view(), ov[i], 1e-5) for i, dev in enumerate(devices)]
+            bar = 1
+        elif kind == 1:
+            tokens = [dev.silu(xv[i], ov[i]) for i, dev in enumerate(devices)]
+            bar = 1
+        else:
+            a = (0, 5, 300)[rng.below(3)]
+            tokens = [dev.rope(xv[i], ov[i], a, 10000.0) for i, dev in enumerate(devices)]
+            bar = 2
+        assert all(t > 0 for t in tokens), (tokens, gpu.error())
+        c, g = o[0].view().to_host(), o[1].view().to_host()
+        assert bf16_steps(c, g).max() <= bar, (kind, xo, xs, oo, os_)
+    elif kind == 3:                                         # cache append
+        a = (0, 1, 16, 37)[rng.below(4)]
+        cap = a + R + rng.below(10)
+        so, ss = view_cases.viewed_operand(rng, lead, R, D)
+        co, cs = view_cases.viewed_operand(rng, lead, cap, D)
+        s_, c_ = make(so, salt=0x3B00 + case), make(co, salt=0x3C00 + case)
+        tokens = [dev.cache_append(view_cases.apply(s_[i].view(), ss), view_cases.apply(c_[i].view(), cs), a)
+                  for i, dev in enumerate(devices)]
+        assert all(t > 0 for t in tokens), (tokens, gpu.error())
+        assert np.array_equal(c_[0].view().to_host(), c_[1].view().to_host()), (so, ss, co, cs, a)
+    elif kind == 4:                                         # embedding
+        V, F = (7, 37, 100)[rng.below(3)], (16, 33, 128)[rng.below(3)]
+        io, isteps = view_cases.viewed_operand(rng, lead, 1, R)
+        oo, os_ = view_cases.viewed_operand(rng, lead, R, F)
+        table = make((V, F), salt=0x3D00 + case)
+        ids = (datagen.pattern_bits(32, int(np.prod(io)), 0x3E00 + case) % V).astype(np.uint32).reshape(io)
+        idx = on_both(devices, iomo.DT_U32, io, ids)
+        closing.extend(idx)
+        o = make(oo, salt=0x3F00 + case)
+        for i, dev in enumerate(devices):
+            token, status = dev.embedding(table[i].view(), view_cases.apply(idx[i].view(), isteps),
+                                          view_cases.apply(o[i].view(), os_))
+            assert token > 0 and status == 0, (token, status, dev.error())
+        assert np.array_equal(o[0].view().to_host(), o[1].view().to_host()), (io, isteps, oo, os_)
+    else:                                                   # linear, ordinary or head-planar
+        s = rng.below(5)
+        x_rows = s + R + rng.below(3)
+        inner = (32, 64, 96)[rng.below(3)]
+        H = 1 + rng.below(3)
+        hp = rng.chance(1, 2)
+        xo, xs = view_cases.viewed_operand(rng, lead, x_rows, inner)
+        oo, os_ = view_cases.viewed_operand(rng, lead + ((H,) if hp else ()), R, D if hp else H * D)
+        x = make(xo, bf16_values(int(np.prod(xo)), 0x4000 + case).reshape(xo))
+        w = make((H * D, inner), bf16_values(H * D * inner, 0x4100 + case).reshape(H * D, inner))
+        o = make(oo, salt=0x4200 + case)
+        args = (s, R, hp, H if hp else 1, D if hp else H * D)
+        tokens = [dev.linear(view_cases.apply(x[i].view(), xs), w[i].view(), view_cases.apply(o[i].view(), os_), *args)
+                  for i, dev in enumerate(devices)]
+        assert all(t > 0 for t in tokens), (tokens, gpu.error())
+        cv, gv = (view_cases.apply(o[i].view(), os_).to_host() for i in range(2))
+        c64 = datagen.bf16_to_f32(cv.reshape(-1)).astype(np.float64)
+        g64 = datagen.bf16_to_f32(gv.reshape(-1)).astype(np.float64)
+        ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(c64), 1e-30))) - 7)
+        assert np.all(np.abs(g64 - c64) <= 2 * np.maximum(np.maximum(ulp, 2.0 ** -7), 2.0 ** -6 * np.abs(c64)))
+        # outside the window both owners still hold the pre-filled pattern
+        marker = iomo.HostTensor(dt, oo, fill=0)
+        mv = view_cases.apply(marker.view(), os_)
+        mv.from_logical(np.full(mv.dims, 1, np.uint16))
+        outside = iomo.untile_plane(marker.storage, oo) == 0
+        assert np.array_equal(o[0].view().to_host()[outside], o[1].view().to_host()[outside])
+    for t in closing:
+        t.close()
