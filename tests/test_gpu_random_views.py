@@ -997,3 +997,47 @@ def test_backend_layer_operations_on_random_views(devices, case):
         assert np.array_equal(o[0].view().to_host()[outside], o[1].view().to_host()[outside])
     for t in closing:
         t.close()
+
+
+@pytest.mark.parametrize("case", range(48))
+def test_backend_attention_on_random_views(devices, case):
+    """Attention through `DeviceOps` on both backends with q, k, v and out behind random views:
+    both results inside the float64 budget of the BF16 probability, hence within twice the
+    budget of each other (the reference's own fixture rule is no bound under cancellation)."""
+    import test_gpu_sdpa as ts
+    cpu, gpu = devices
+    rng = view_cases.Stream(case, 1919)
+    lead = ((), (2,), (2, 2))[rng.below(3)]
+    grouping = (1, 2, 4)[rng.below(3)]
+    Hkv = 1 + rng.below(2)
+    Hq = Hkv * grouping
+    R = (1, 3, 17, 40)[rng.below(4)]
+    D = (16, 64, 128)[rng.below(3)]
+    a = (0, 2, 31, 90)[rng.below(4)]
+    L = a + R
+    cap = L + rng.below(12)
+    spec = ts.random_case(0x4300 + case, lead, Hq, Hkv, R, D, cap, a, L)
+    qd, kd, od = ts.shapes(spec)
+    tensors, views = [], []
+    for name, dims in (("q", qd), ("k", kd), ("v", kd), (None, od)):
+        owner_dims, steps = view_cases.viewed_operand(rng, dims[:-2], dims[-2], dims[-1])
+        pair_ = prefilled(devices, DT_BF16, owner_dims, 0x4400 + 4 * case + len(tensors))
+        vs = [view_cases.apply(t.view(), steps) for t in pair_]
+        if name:
+            for v in vs:
+                v.from_host(np.array(spec[name], np.uint16).reshape(dims))
+        tensors.append(pair_)
+        views.append(vs)
+    for i, dev in enumerate(devices):
+        tok = dev.sdpa(views[0][i], views[1][i], views[2][i], views[3][i], a, L)
+        assert tok > 0, (tok, dev.error())
+    ref64, budget = ts.float64_attention(spec)
+    results = []
+    for i in range(2):
+        got = views[3][i].to_host()
+        results.append(datagen.bf16_to_f32(got.reshape(-1)).astype(np.float64).reshape(ref64.shape))
+        assert np.all(np.abs(results[i] - ref64) <= budget), ("cpu", "gpu")[i]
+    assert np.all(np.abs(results[0] - results[1]) <= 2 * budget)
+    for pair_ in tensors:
+        for t in pair_:
+            t.close()
