@@ -1041,3 +1041,61 @@ def test_backend_attention_on_random_views(devices, case):
     for pair_ in tensors:
         for t in pair_:
             t.close()
+
+
+def test_four_queues_driven_from_four_threads(devices):
+    """Four host threads, each with a queue of its own on the one device, run 120 dependent
+    operations on their own owners while creating and closing scratch tensors and reading results
+    back (arena, registry and transfer path are shared by all of them).  Every thread's owners
+    end up as the reference CPU backend leaves them after the same sequence."""
+    import threading
+    cpu, gpu = devices
+    dims = (3, 17, 33)
+    count = int(np.prod(dims))
+    plans, pools, queues, errors = [], [], [], []
+    for th in range(4):
+        rng = view_cases.Stream(th, 2020)
+        plans.append([(rng.below(4), rng.below(4), rng.below(4), rng.below(3), rng.below(7)) for _ in range(120)])
+        values = [datagen.normal_f32(count, 0, 1, 0x4500 + 4 * th + i).view(np.uint32).reshape(dims) for i in range(4)]
+        pools.append(([on_both((cpu,), DT_F32, dims, v)[0] for v in values],
+                      [on_both((gpu,), DT_F32, dims, v)[0] for v in values]))
+        queues.append(gpu if th == 0 else gpu.second_queue())
+
+    def drive(th):
+        try:
+            q = queues[th]
+            pool = pools[th][1]
+            tokens = []
+            for out, a, b, op, extra in plans[th]:
+                tok = q.l.iomc_binary(q.queue, (OP_ADD, OP_MUL, OP_SUB)[op], pool[a].view().h, pool[b].view().h,
+                                      pool[out].view().h)
+                assert tok > 0, (th, tok, q.error())
+                tokens.append(tok)
+                if extra == 0:                          # a scratch owner comes and goes
+                    t = gpu.tensor(DT_F32, (2, 16, 16))
+                    t.view().from_host(np.zeros((2, 16, 16), np.uint32))
+                    t.close()
+                elif extra == 1:                        # observe an earlier result mid-stream
+                    assert q.wait(tokens[len(tokens) // 2]) == 0
+                    pool[a].view().to_host()
+            for tok in tokens:
+                assert q.wait(tok) == 0, q.error()
+        except BaseException as exc:                    # reported by the main thread
+            errors.append((th, repr(exc)))
+    threads = [threading.Thread(target=drive, args=(th,)) for th in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert errors == []
+    for th in range(4):
+        pool = pools[th][0]
+        for out, a, b, op, _ in plans[th]:
+            assert cpu.binary((OP_ADD, OP_MUL, OP_SUB)[op], pool[a].view(), pool[b].view(), pool[out].view()) > 0
+        for c, g in zip(*pools[th]):
+            assert np.array_equal(c.view().to_host(), g.view().to_host()), th
+    for th in range(1, 4):
+        queues[th].close()
+    for th in range(4):
+        for t in pools[th][0] + pools[th][1]:
+            t.close()
