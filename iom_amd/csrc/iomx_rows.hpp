@@ -250,15 +250,15 @@ IOMX_HD float decode_f32(uint32_t raw) {
     constexpr Fmt f = fmt_of(DT);
     constexpr uint32_t emask = (1u << f.ebits) - 1u, fmask = (1u << f.fbits) - 1u;
     const uint32_t frac = raw & fmask, exp = (raw >> f.fbits) & emask;
-    float v;
-    if (top_special(f) && exp == emask) {
-        v = (f.infs && frac == 0) ? __builtin_inff() : __builtin_nanf("");
-    } else {
-        const int m = exp ? (int)((1u << f.fbits) + frac) : (int)frac;
-        const int scale = (int)(exp ? exp : 1u) - f.bias - f.fbits;
-        v = ldexpf((float)m, scale);
-    }
-    return ((raw >> (f.ebits + f.fbits)) & 1u) ? -v : v;
+    const uint32_t sign = ((raw >> (f.ebits + f.fbits)) & 1u) << 31;
+    if (top_special(f) && exp == emask)
+        return as_f32_hd(sign | ((f.infs && frac == 0) ? 0x7F800000u : 0x7FC00000u));
+    // a normal value re-biased into binary32 (every leaf exponent is inside its range), a
+    // subnormal one as its integer fraction times the leaf's smallest step: both exact
+    constexpr float kStep = 1.0f / (float)(1u << (f.bias - 1 + f.fbits));       // 2^(1 - bias - fbits)
+    const uint32_t normal = ((exp + 127u - (uint32_t)f.bias) << 23) | (frac << (23 - f.fbits));
+    const float magnitude = exp ? as_f32_hd(normal) : (float)frac * kStep;
+    return as_f32_hd(as_u32_hd(magnitude) | sign);
 }
 
 template <int DT>
