@@ -310,7 +310,8 @@ def wl_other_leaves(timer, steps, warmup):
     dims, F = (64, 512, 2048), 2048
     n = int(np.prod(dims))
     for name, dtype in (("f16", iomx.DT_F16), ("u8", iomx.DT_U8), ("f8_e4m3fn", iomx.DT_F8_E4M3FN),
-                        ("u4", iomx.DT_U4), ("f64", iomx.DT_F64)):
+                        ("u4", iomx.DT_U4), ("f6_e3m2", iomx.DT_F6_E3M2), ("f4_e2m1", iomx.DT_F4_E2M1),
+                        ("f64", iomx.DT_F64)):
         bits = iomx.LEAF_BITS[dtype]
         def owner(d, salt):
             t = iomx.DeviceTensor(dtype, d, fill=None)
@@ -320,6 +321,8 @@ def wl_other_leaves(timer, steps, warmup):
                 raw[1::2] = (raw[1::2] & 0x800FFFFF) | 0x3FE00000
             elif dtype == iomx.DT_F16:
                 raw = (raw & 0xBBFFBBFF)
+            elif dtype == iomx.DT_F8_E4M3FN:   # magnitudes below 2: no NaN encodings, no overflow
+                raw = (raw & 0xBFBFBFBF)
             t.upload_raw(raw)
             return t
         lhs, rhs, o = owner(dims, 1), owner((1, F), 2), iomx.DeviceTensor(dtype, dims, fill=None)

@@ -42,6 +42,41 @@ struct RowsArgs {
     uint32_t brow[2], bcol[2];
 };
 
+// A tile row of an 8-bit floating leaf through the conversion instructions: taken
+// when no input lies in the all-NaN top exponent of F8_E4M3FN and every result is a
+// number no larger than the largest finite value (false for a NaN result); the caller
+// computes any other row element by element on the raw bits.
+template <int DT, int OP, int N>
+__device__ __forceinline__ bool hw_f8_row(const uint32_t (&in)[N][4], const uint32_t (&bcol)[2],
+                                          uint32_t (&res)[4]) {
+    bool plain = true;
+    if constexpr (DT == DT_F8_E4M3FN) {
+#pragma unroll
+        for (int k = 0; k < N; ++k)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) plain &= !e4m3_top_exponent(in[k][j]);
+    }
+    float r[kTile];
+#pragma unroll
+    for (int i = 0; i < (int)kTile; ++i) {
+        const float x = bcol[0] ? hw_f8_value<DT>(in[0][0], 0) : hw_f8_value<DT>(in[0][i >> 2], i & 3);
+        if constexpr (N == 2) {
+            const float y = bcol[1] ? hw_f8_value<DT>(in[1][0], 0) : hw_f8_value<DT>(in[1][i >> 2], i & 3);
+            r[i] = leaf_arith<OP>(x, y);
+        } else {
+            r[i] = silu_carrier(x);
+        }
+        plain &= __builtin_fabsf(r[i]) <= hw_f8_limit<DT>();
+    }
+    if (!plain) return false;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t w = hw_f8_pack<DT>(r[4 * j], r[4 * j + 1], 0u, false);
+        res[j] = hw_f8_pack<DT>(r[4 * j + 2], r[4 * j + 3], w, true);
+    }
+    return true;
+}
+
 template <int DT, int OP>
 __global__ __launch_bounds__(256) void rows_kernel(const RowsArgs a) {
     constexpr int BITS = bits_of(DT);
@@ -61,13 +96,22 @@ __global__ __launch_bounds__(256) void rows_kernel(const RowsArgs a) {
             const uint32_t tck = a.bcol[k] ? 0u : t.tc;
             const uint8_t* src = a.src[k] + plane[k] * a.plane_bytes[k]
                     + ((uint64_t)(rk >> 4) * a.tile_cols[k] + tck) * kTileBytes + (rk & 15u) * kRowBytes;
-            load_row<BITS>(src, in[k]);
+            // an operand that broadcasts is read again by other lanes and stays cached
+            if (a.brow[k] | a.bcol[k]) load_row<BITS>(src, in[k]);
+            else load_row<BITS, true>(src, in[k]);
         }
         uint32_t res[K];
+        bool converted = false;
+        if constexpr (has_hw_f8(DT) && OP != ROWS_OP_COPY) converted = hw_f8_row<DT, OP>(in, a.bcol, res);
         if constexpr (OP == ROWS_OP_COPY) {
 #pragma unroll
             for (int j = 0; j < K; ++j) res[j] = in[0][j];
-        } else {
+        } else if constexpr (!is_float_leaf(DT) && BITS <= 4) {
+#pragma unroll
+            for (int j = 0; j < K; ++j)
+                res[j] = swar_word<BITS, OP>(a.bcol[0] ? splat_lane<BITS>(in[0][0]) : in[0][j],
+                                             a.bcol[1] ? splat_lane<BITS>(in[1][0]) : in[1][j]);
+        } else if (!converted) {
 #pragma unroll
             for (int j = 0; j < K; ++j) res[j] = 0;
 #pragma unroll
@@ -85,7 +129,7 @@ __global__ __launch_bounds__(256) void rows_kernel(const RowsArgs a) {
         }
         uint8_t* dst = a.out + plane[2] * a.plane_bytes[2]
                 + ((uint64_t)(t.row >> 4) * a.tile_cols[2] + t.tc) * kTileBytes + (t.row & 15u) * kRowBytes;
-        store_row<BITS>(dst, res, t.ncols);
+        store_row<BITS, true>(dst, res, t.ncols);
     }
 }
 

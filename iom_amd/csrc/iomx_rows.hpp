@@ -61,22 +61,28 @@ constexpr bool top_special(Fmt f) { return !f.finite_only || f.ebits >= 4; }
 // Tile rows as word arrays
 // ---------------------------------------------------------------------------
 
-template <int BITS>
+// STREAM: read past the caches (an operand that no other lane reads again).
+template <int BITS, bool STREAM = false>
 IOMX_HD void load_row(const uint8_t* p, uint32_t (&w)[BITS / 2]) {
     constexpr int K = BITS / 2;
     if constexpr (K == 1) {
-        w[0] = *reinterpret_cast<const uint32_t*>(p);
+        w[0] = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p))
+                      : *reinterpret_cast<const uint32_t*>(p);
     } else if constexpr (K == 2) {
-        const u32x2 v = *reinterpret_cast<const u32x2*>(p);
+        const u32x2 v = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p))
+                               : *reinterpret_cast<const u32x2*>(p);
         w[0] = v.x;
         w[1] = v.y;
     } else if constexpr (K == 3) {
 #pragma unroll
-        for (int j = 0; j < 3; ++j) w[j] = reinterpret_cast<const uint32_t*>(p)[j];
+        for (int j = 0; j < 3; ++j)
+            w[j] = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p) + j)
+                          : reinterpret_cast<const uint32_t*>(p)[j];
     } else {
 #pragma unroll
         for (int j = 0; j < K / 4; ++j) {
-            const u32x4 v = reinterpret_cast<const u32x4*>(p)[j];
+            const u32x4 v = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p) + j)
+                                   : reinterpret_cast<const u32x4*>(p)[j];
             w[4 * j] = v.x;
             w[4 * j + 1] = v.y;
             w[4 * j + 2] = v.z;
@@ -120,21 +126,29 @@ IOMX_HD void put(uint32_t (&w)[BITS / 2], int i, uint64_t v) {
 
 // Stores the first ncols elements of a tile row and nothing else: whole words
 // where they are covered, a read-modify-write of the one partly covered word.
-template <int BITS>
+template <int BITS, bool STREAM = false>
 IOMX_HD void store_row(uint8_t* p, const uint32_t (&w)[BITS / 2], uint32_t ncols) {
     constexpr int K = BITS / 2;
     if (ncols == kTile) {
         if constexpr (K == 1) {
-            *reinterpret_cast<uint32_t*>(p) = w[0];
+            if constexpr (STREAM) __builtin_nontemporal_store(w[0], reinterpret_cast<uint32_t*>(p));
+            else *reinterpret_cast<uint32_t*>(p) = w[0];
         } else if constexpr (K == 2) {
-            *reinterpret_cast<u32x2*>(p) = u32x2{w[0], w[1]};
+            if constexpr (STREAM) __builtin_nontemporal_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(p));
+            else *reinterpret_cast<u32x2*>(p) = u32x2{w[0], w[1]};
         } else if constexpr (K == 3) {
 #pragma unroll
-            for (int j = 0; j < 3; ++j) reinterpret_cast<uint32_t*>(p)[j] = w[j];
+            for (int j = 0; j < 3; ++j) {
+                if constexpr (STREAM) __builtin_nontemporal_store(w[j], reinterpret_cast<uint32_t*>(p) + j);
+                else reinterpret_cast<uint32_t*>(p)[j] = w[j];
+            }
         } else {
 #pragma unroll
-            for (int j = 0; j < K / 4; ++j)
-                reinterpret_cast<u32x4*>(p)[j] = u32x4{w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]};
+            for (int j = 0; j < K / 4; ++j) {
+                const u32x4 v = u32x4{w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]};
+                if constexpr (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p) + j);
+                else reinterpret_cast<u32x4*>(p)[j] = v;
+            }
         }
         return;
     }
@@ -327,6 +341,41 @@ IOMX_HD uint64_t leaf_binary(uint64_t a, uint64_t b) {
     }
 }
 
+// A whole word of 2- or 4-bit integers at once (sixteen or eight lanes; the wrap of
+// two's complement does not see the sign).  Sum and difference keep carries and
+// borrows inside a lane by handling each lane's top bit apart; the 2-bit product is
+// two bits of boolean algebra; the 4-bit products are formed two at a time, on nibbles
+// j and j + 4 moved to the bottom of the two 16-bit halves of a word.
+template <int BITS>
+IOMX_HD uint32_t splat_lane(uint32_t w) {
+    return BITS == 2 ? (w & 3u) * 0x55555555u : (w & 15u) * 0x11111111u;
+}
+
+template <int BITS, int OP>
+IOMX_HD uint32_t swar_word(uint32_t a, uint32_t b) {
+    static_assert(BITS == 2 || BITS == 4, "sub-byte integer lanes");
+    constexpr uint32_t H = BITS == 2 ? 0xAAAAAAAAu : 0x88888888u, L = ~H;
+    if constexpr (OP == IOMX_OP_ADD) {
+        return ((a & L) + (b & L)) ^ ((a ^ b) & H);
+    } else if constexpr (OP == IOMX_OP_SUB) {
+        return ((a | H) - (b & L)) ^ ((a ^ ~b) & H);
+    } else if constexpr (BITS == 2) {
+        // (2*a1 + a0)(2*b1 + b0) mod 4 = 2*(a1 b0 xor a0 b1) + a0 b0
+        const uint32_t low = a & b & 0x55555555u;
+        const uint32_t high = (((a >> 1) & b) ^ (a & (b >> 1))) & 0x55555555u;
+        return low | (high << 1);
+    } else {
+        uint32_t r = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t x = (a >> (4 * j)) & 0x000F000Fu, y = (b >> (4 * j)) & 0x000F000Fu;
+            const uint32_t p = ((x & 0xFFFFu) * (y & 0xFFFFu)) | (((x >> 16) * (y >> 16)) << 16);
+            r |= (p & 0x000F000Fu) << (4 * j);
+        }
+        return r;
+    }
+}
+
 // x * sigmoid(x), two-branch form of src/shared/scalar_silu.hpp:69-97; one
 // exponential of a non-positive argument serves both branches.
 IOMX_HD float silu_carrier(float x) {
@@ -369,6 +418,55 @@ IOMX_HD uint64_t encode_from(T v) {
 }
 
 #if defined(__HIPCC__)
+
+// The conversion instructions of the two 8-bit floating leaves.  They agree with the
+// leaf's own rule on every value up to the largest finite one (the same grid, the same
+// round-to-nearest-even, subnormals included).  Outside that they do not: the top
+// exponent of F8_E4M3FN holds values up to 448 for the hardware and is all NaN for the
+// leaf (src/shared/scalar_binary_codec.hpp:51,73), and what an overflow or a NaN
+// becomes is the leaf's choice.  So a caller converts by hardware only what
+// hw_f8_limit bounds and sends every other element through decode_f32 / encode_f32.
+constexpr bool has_hw_f8(int dt) { return dt == DT_F8_E4M3FN || dt == DT_F8_E5M2; }
+
+template <int DT>
+constexpr float hw_f8_limit() { return DT == DT_F8_E4M3FN ? 240.0f : 57344.0f; }
+
+// Element `byte` (a constant after unrolling) of a word of four.
+template <int DT>
+__device__ __forceinline__ float hw_f8_value(uint32_t word, int byte) {
+    if constexpr (DT == DT_F8_E4M3FN) {
+        switch (byte) {
+            case 0: return __builtin_amdgcn_cvt_f32_fp8(word, 0);
+            case 1: return __builtin_amdgcn_cvt_f32_fp8(word, 1);
+            case 2: return __builtin_amdgcn_cvt_f32_fp8(word, 2);
+            default: return __builtin_amdgcn_cvt_f32_fp8(word, 3);
+        }
+    } else {
+        switch (byte) {
+            case 0: return __builtin_amdgcn_cvt_f32_bf8(word, 0);
+            case 1: return __builtin_amdgcn_cvt_f32_bf8(word, 1);
+            case 2: return __builtin_amdgcn_cvt_f32_bf8(word, 2);
+            default: return __builtin_amdgcn_cvt_f32_bf8(word, 3);
+        }
+    }
+}
+
+// Two rounded values into the lower or upper half of a word, the other half kept.
+template <int DT>
+__device__ __forceinline__ uint32_t hw_f8_pack(float first, float second, uint32_t word, bool upper) {
+    if constexpr (DT == DT_F8_E4M3FN) {
+        return upper ? __builtin_amdgcn_cvt_pk_fp8_f32(first, second, word, true)
+                     : __builtin_amdgcn_cvt_pk_fp8_f32(first, second, word, false);
+    } else {
+        return upper ? __builtin_amdgcn_cvt_pk_bf8_f32(first, second, word, true)
+                     : __builtin_amdgcn_cvt_pk_bf8_f32(first, second, word, false);
+    }
+}
+
+// True if one of the four bytes has all four exponent bits of F8_E4M3FN set.
+__device__ __forceinline__ bool e4m3_top_exponent(uint32_t word) {
+    return (((word & 0x78787878u) + 0x08080808u) & 0x80808080u) != 0;
+}
 
 struct TileRow {
     uint32_t row, tc, ncols;

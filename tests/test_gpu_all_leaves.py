@@ -130,6 +130,76 @@ def test_binary_every_pair_of_a_narrow_leaf(dtype, op):
         t.free()
 
 
+F8_CONVERTED = [iomo.DT_F8_E4M3FN, iomo.DT_F8_E5M2]
+
+
+def f8_table(dtype):
+    """Value of each of the 256 encodings (src/shared/scalar_binary_codec.hpp:45-66): the top
+    exponent of F8_E4M3FN is NaN throughout, that of F8_E5M2 holds the infinities and NaN."""
+    ebits, fbits, bias = {iomo.DT_F8_E4M3FN: (4, 3, 7), iomo.DT_F8_E5M2: (5, 2, 15)}[dtype]
+    raw = np.arange(256)
+    frac, exp = raw & ((1 << fbits) - 1), (raw >> fbits) & ((1 << ebits) - 1)
+    value = np.where(exp == 0, frac * 2.0 ** (1 - bias - fbits), (1 + frac / (1 << fbits)) * 2.0 ** (exp - bias))
+    top = exp == (1 << ebits) - 1
+    special = np.where((frac == 0) & (dtype == iomo.DT_F8_E5M2), np.inf, np.nan)
+    return np.where(raw >> 7, -1.0, 1.0) * np.where(top, special, value)
+
+
+def regrouped(in_range):
+    """Indices of a row of 288: those in range first, padded to whole tile rows, then the others."""
+    good, bad = np.flatnonzero(in_range), np.flatnonzero(~in_range)
+    if good.size:
+        good = np.concatenate([good, np.full(-good.size % 16, good[0])])
+    row = np.concatenate([good, bad]).astype(np.int64)
+    return np.concatenate([row, np.full(288 - row.size, row[-1])])
+
+
+@pytest.mark.parametrize("dtype", F8_CONVERTED, ids=names(F8_CONVERTED))
+@pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB, OP_DIV])
+def test_f8_pairs_regrouped_by_the_range_of_their_result(dtype, op):
+    """The tile-row kernel rounds a tile row with the conversion instructions when all sixteen
+    results are numbers within the leaf's finite range, and element by element otherwise; in the
+    all-pairs table above a pair in range often shares its tile row with one that is not.  Here a
+    row holds one left operand against all 256 right operands regrouped, those with a result in
+    range first and padded to whole tile rows, so every such pair goes through the instructions."""
+    table = f8_table(dtype)
+    limit = {iomo.DT_F8_E4M3FN: 240.0, iomo.DT_F8_E5M2: 57344.0}[dtype]
+    rhs = np.zeros((256, 288), np.uint8)
+    with np.errstate(all="ignore"):
+        for x in range(256):
+            r = {OP_ADD: table[x] + table, OP_SUB: table[x] - table, OP_MUL: table[x] * table,
+                 OP_DIV: table[x] / table}[op]
+            rhs[x] = regrouped(np.abs(r) <= limit)
+    lhs = np.repeat(np.arange(256, dtype=np.uint8).reshape(256, 1), 288, axis=1)
+    dl, hl = pair(dtype, (256, 288), values=lhs)
+    dr, hr = pair(dtype, (256, 288), values=rhs)
+    do, ho = pair(dtype, (256, 288))
+    assert iomx.binary(op, dl.view(), dr.view(), do.view()) == 0
+    assert kernel_name() == "rows_binary"
+    assert iomo.binary(op, hl.view(), hr.view(), ho.view()) == 0
+    assert same_storage(do, ho)
+    for t in (dl, dr, do):
+        t.free()
+
+
+@pytest.mark.parametrize("dtype", F8_CONVERTED, ids=names(F8_CONVERTED))
+def test_f8_silu_regrouped_by_the_range_of_its_result(dtype):
+    """Every finite encoding in tile rows of finite encodings only (see the test above)."""
+    table = f8_table(dtype)
+    vals = regrouped(np.isfinite(table)).astype(np.uint8).reshape(1, 288)
+    dx, hx = pair(dtype, (1, 288), values=vals)
+    do, ho = pair(dtype, (1, 288))
+    assert iomx.silu(dx.view(), do.view()) == 0
+    assert kernel_name() == "rows_silu"
+    assert iomo.silu(hx.view(), ho.view()) == 0
+    got, want = do.view().to_host().reshape(-1), ho.view().to_logical().reshape(-1)
+    nan = is_nan(want, dtype)
+    assert np.array_equal(got[nan], want[nan])
+    assert steps_apart(got[~nan], want[~nan], dtype).max() <= 1
+    dx.free()
+    do.free()
+
+
 @pytest.mark.parametrize("dtype", [iomo.DT_I8, iomo.DT_U8], ids=["I8", "U8"])
 @pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
 def test_binary_every_8bit_pair_on_whole_planes(dtype, op):
