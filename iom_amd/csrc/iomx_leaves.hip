@@ -77,6 +77,28 @@ __device__ __forceinline__ bool hw_f8_row(const uint32_t (&in)[N][4], const uint
     return true;
 }
 
+// A tile row of a 4- or 6-bit floating leaf through the scaled conversions.  Operands
+// are finite, so only a quotient can be a NaN (0/0).
+template <int DT, int OP, int N>
+__device__ __forceinline__ void hw_f46_row(const uint32_t (&in)[N][bits_of(DT) / 2], const uint32_t (&bcol)[2],
+                                           uint32_t (&res)[bits_of(DT) / 2]) {
+    float v[N][kTile], r[kTile];
+#pragma unroll
+    for (int k = 0; k < N; ++k) hw_f46_decode<DT>(in[k], v[k]);
+#pragma unroll
+    for (int i = 0; i < (int)kTile; ++i) {
+        const float x = bcol[0] ? v[0][0] : v[0][i];
+        if constexpr (N == 2) {
+            const float y = bcol[1] ? v[1][0] : v[1][i];
+            r[i] = leaf_arith<OP>(x, y);
+            if constexpr (OP == IOMX_OP_DIV) r[i] = (r[i] != r[i]) ? hw_f46_largest<DT>() : r[i];
+        } else {
+            r[i] = silu_carrier(x);
+        }
+    }
+    hw_f46_encode<DT>(r, res);
+}
+
 template <int DT, int OP>
 __global__ __launch_bounds__(256) void rows_kernel(const RowsArgs a) {
     constexpr int BITS = bits_of(DT);
@@ -103,6 +125,10 @@ __global__ __launch_bounds__(256) void rows_kernel(const RowsArgs a) {
         uint32_t res[K];
         bool converted = false;
         if constexpr (has_hw_f8(DT) && OP != ROWS_OP_COPY) converted = hw_f8_row<DT, OP>(in, a.bcol, res);
+        if constexpr (has_hw_f46(DT) && OP != ROWS_OP_COPY) {
+            hw_f46_row<DT, OP>(in, a.bcol, res);
+            converted = true;
+        }
         if constexpr (OP == ROWS_OP_COPY) {
 #pragma unroll
             for (int j = 0; j < K; ++j) res[j] = in[0][j];

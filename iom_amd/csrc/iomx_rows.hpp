@@ -468,6 +468,71 @@ __device__ __forceinline__ bool e4m3_top_exponent(uint32_t word) {
     return (((word & 0x78787878u) + 0x08080808u) & 0x80808080u) != 0;
 }
 
+// The scaled conversions of the 4- and 6-bit floating leaves, at scale 1: their decode
+// is exact, and their encode is the leaf's own rule for every binary32 input (the same
+// round-to-nearest-even, subnormals included, saturation at the largest finite magnitude,
+// infinities too) except that a NaN keeps its sign where the leaf stores the positive
+// largest magnitude (src/shared/scalar_binary_codec.hpp:80) - the caller replaces a NaN
+// by that value first.  Checked against decode_f32 / encode_f32 on the device for all
+// encodings and a dense sweep of binary32 values.
+constexpr bool has_hw_f46(int dt) { return dt == DT_F4_E2M1 || dt == DT_F6_E2M3 || dt == DT_F6_E3M2; }
+
+template <int DT>
+constexpr float hw_f46_largest() { return DT == DT_F4_E2M1 ? 6.0f : DT == DT_F6_E2M3 ? 7.5f : 28.0f; }
+
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x32_t __attribute__((ext_vector_type(32)));
+typedef uint32_t u32x6_t __attribute__((ext_vector_type(6)));
+
+// Sixteen values of one tile row (two words of F4, three of F6).
+template <int DT>
+__device__ __forceinline__ void hw_f46_decode(const uint32_t (&w)[bits_of(DT) / 2], float (&v)[kTile]) {
+    if constexpr (DT == DT_F4_E2M1) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const f32x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 0);
+            const f32x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 1);
+            const f32x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 2);
+            const f32x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[j], 1.0f, 3);
+            v[8 * j] = p0.x; v[8 * j + 1] = p0.y; v[8 * j + 2] = p1.x; v[8 * j + 3] = p1.y;
+            v[8 * j + 4] = p2.x; v[8 * j + 5] = p2.y; v[8 * j + 6] = p3.x; v[8 * j + 7] = p3.y;
+        }
+    } else {
+        // the instruction converts thirty-two: the upper sixteen are zeros here
+        const u32x6_t s = {w[0], w[1], w[2], 0u, 0u, 0u};
+        f32x32_t d;
+        if constexpr (DT == DT_F6_E2M3) d = __builtin_amdgcn_cvt_scalef32_pk32_f32_fp6(s, 1.0f);
+        else d = __builtin_amdgcn_cvt_scalef32_pk32_f32_bf6(s, 1.0f);
+#pragma unroll
+        for (int i = 0; i < (int)kTile; ++i) v[i] = d[i];
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ void hw_f46_encode(const float (&r)[kTile], uint32_t (&w)[bits_of(DT) / 2]) {
+    if constexpr (DT == DT_F4_E2M1) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            uint32_t x = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, r[8 * j], r[8 * j + 1], 1.0f, 0);
+            x = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(x, r[8 * j + 2], r[8 * j + 3], 1.0f, 1);
+            x = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(x, r[8 * j + 4], r[8 * j + 5], 1.0f, 2);
+            w[j] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(x, r[8 * j + 6], r[8 * j + 7], 1.0f, 3);
+        }
+    } else {
+        // result 2i comes from the first operand's element i, result 2i + 1 from the second's
+        f32x16_t even, odd;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            even[i] = i < 8 ? r[2 * i] : 0.0f;
+            odd[i] = i < 8 ? r[2 * i + 1] : 0.0f;
+        }
+        u32x6_t e;
+        if constexpr (DT == DT_F6_E2M3) e = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(even, odd, 1.0f);
+        else e = __builtin_amdgcn_cvt_scalef32_2xpk16_bf6_f32(even, odd, 1.0f);
+        w[0] = e[0]; w[1] = e[1]; w[2] = e[2];
+    }
+}
+
 struct TileRow {
     uint32_t row, tc, ncols;
     bool live;
