@@ -304,8 +304,8 @@ def wl_layer_ops(timer, steps, warmup):
 
 
 def wl_other_leaves(timer, steps, warmup):
-    """The tile-row kernels that serve every leaf outside I32/U32/F32/BF16, on the headline
-    shape: correctness-first paths, measured so that their cost is known."""
+    """The leaves outside I32/U32/F32/BF16 on the headline shape: F16, U8 and F64 on the
+    chunk-mapped kernels, F8, F6, F4 and U4 on the tile-row kernel."""
     out = []
     dims, F = (64, 512, 2048), 2048
     n = int(np.prod(dims))

@@ -33,12 +33,14 @@ def _device():
     yield
 
 
-def pair(dtype, dims, salt):
+def pair(dtype, dims, salt, small=False):
     dt = iomx.DeviceTensor(dtype, dims, fill=0x5A)
     ht = iomo.HostTensor(dtype, dims, fill=0x5A)
     values = datagen.pattern_bits(LEAF_BITS[dtype], int(np.prod(dims)), salt).reshape(dims)
     if dtype == iomo.DT_BOOL:
         values = values & 1                              # BOOL host bytes are zero or one
+    if small and dtype in (iomo.DT_F8_E4M3FN, iomo.DT_F8_E5M2):
+        values = values & 0xBF                           # magnitudes below 2: no NaN, no overflow
     dt.view().from_host(values)
     ht.view().from_logical(values)
     return dt, ht
@@ -55,7 +57,10 @@ def test_binary_on_random_views(case):
     if op == OP_DIV and dtype not in FLOAT_LEAVES:
         op = OP_SUB
     lead, rows, cols, operands = view_cases.binary_case(case)
-    owners = [pair(dtype, dims, 0x900 + 3 * case + i) for i, (dims, _) in enumerate(operands)]
+    # every other round of four operations draws small magnitudes for the 8-bit floating leaves:
+    # tile rows that the kernel rounds with the conversion instructions, not element by element
+    small = (case // (4 * len(LEAVES))) % 2 == 1
+    owners = [pair(dtype, dims, 0x900 + 3 * case + i, small) for i, (dims, _) in enumerate(operands)]
     dv = [view_cases.apply(d.view(), steps) for (d, _), (_, steps) in zip(owners, operands)]
     hv = [view_cases.apply(h.view(), steps) for (_, h), (_, steps) in zip(owners, operands)]
     rc = iomx.binary(op, dv[0], dv[1], dv[2])
