@@ -13,6 +13,9 @@ oracle on sampled planes / rows, and through size-independent properties.
                                                             sampled rows within the native bound
   attention 8 x 32/4 heads, R = L = 512, D = 64 BF16        uniform-score closed form, sampled
                                                             rows against the oracle
+  beyond 4 GiB: ADD / MUL on [40,64,2^20] BF16 through each elementwise kernel family against the
+            closed form; RMSNorm, linear, RoPE, SiLU and copy on [40,32768,2048] BF16 against the
+            same operation on one plane                     bit-exact, every element
 """
 import numpy as np
 import pytest
@@ -134,6 +137,99 @@ def test_config2_broadcast_bf16(op, layout):
     want = bf16_op(src, vec[column_of_storage((512, F))][np.arange(src.size) % plane], op)
     assert np.array_equal(got, want)
     for t in (x, v, o):
+        t.free()
+
+
+def test_elementwise_on_tensors_beyond_4_gib():
+    """[40,64,2^20] BF16: 128 MiB per plane, 5 GiB per tensor, 2.7 * 10^9 elements - byte offsets and
+    element counts that do not fit 32 bits, through each kernel family of the elementwise path:
+    the padded-band kernel (a scalar per plane), the dense streaming shape, the tile-row bands of a
+    row-vector operand (32 MiB per band) and the strided plane walk (every other plane, the operands
+    of the upper half beyond the 4 GiB mark).  Every plane of a result has the same closed form,
+    checked in full."""
+    planes, rows, cols = 40, 64, 1 << 20
+    plane = rows * cols
+    a, a_raw = upload(DT_BF16, (1, rows, cols), "normal", 71)
+    zero = iomx.DeviceTensor(DT_BF16, (planes, 1, 1), fill=0)
+    vec = datagen.bf16_rne(datagen.uniform_f32(cols, 0.5, 1.5, 72))
+    r = iomx.DeviceTensor(DT_BF16, (1, cols))
+    r.upload_raw(vector_storage(vec))
+    t = iomx.DeviceTensor(DT_BF16, (planes, rows, cols), fill=0x5A)
+    u = iomx.DeviceTensor(DT_BF16, (planes, rows, cols), fill=0x5A)
+
+    def every_plane(tensor, want, which=range(planes)):
+        got = tensor.raw().reshape(planes, plane)
+        for p in which:
+            assert np.array_equal(got[p], want), p
+
+    assert iomx.binary(OP_ADD, a.view(), zero.view(), t.view()) == 0            # t = a + 0
+    assert iomx.last_launch().kernel.decode() == "binary_padded"
+    e1 = bf16_op(a_raw, np.zeros_like(a_raw), OP_ADD)
+    every_plane(t, e1)
+
+    assert iomx.binary(OP_ADD, t.view(), t.view(), u.view()) == 0               # u = t + t
+    assert iomx.last_launch().kernel.decode() == "binary_planes"
+    e2 = bf16_op(e1, e1, OP_ADD)
+    every_plane(u, e2)
+
+    assert iomx.binary(OP_MUL, u.view(), r.view(), t.view()) == 0               # t = u * r
+    assert iomx.last_launch().kernel.decode() == "binary_rowvec"
+    e3 = bf16_op(e2, vec[column_of_storage((rows, cols))], OP_MUL)
+    every_plane(t, e3)
+
+    # even planes of t plus odd planes of u into the odd planes of w; its even planes stay as filled
+    w = iomx.DeviceTensor(DT_BF16, (planes, rows, cols), fill=0x5A)
+    half = planes // 2
+    assert iomx.binary(OP_ADD, t.view().slice(0, 0, half, 2), u.view().slice(0, 1, half, 2),
+                       w.view().slice(0, 1, half, 2)) == 0
+    assert iomx.last_launch().kernel.decode() == "binary_planes"
+    every_plane(w, bf16_op(e3, e2, OP_ADD), range(1, planes, 2))
+    every_plane(w, np.full(plane, 0x5A5A, np.uint16), range(0, planes, 2))
+    w.free()
+    for x in (a, zero, r, t, u):
+        x.free()
+
+
+def test_rmsnorm_linear_rope_silu_and_copy_beyond_4_gib():
+    """[40,32768,2048] BF16 (5 GiB, 1,310,720 rows): forty copies of one plane.  Each operation on the
+    whole tensor must give, in every plane, the bits that the same operation gives on that one plane
+    alone (the [32768,2048] launch that the closed forms above check)."""
+    planes, rows, cols = 40, 32768, 2048
+    plane = rows * cols
+    one, _ = upload(DT_BF16, (1, rows, cols), "normal", 73)
+    zero = iomx.DeviceTensor(DT_BF16, (planes, 1, 1), fill=0)
+    scale = iomx.DeviceTensor(DT_BF16, (1, cols))
+    scale.upload_raw(vector_storage(datagen.bf16_rne(datagen.uniform_f32(cols, 0.5, 1.5, 74))))
+    x = iomx.DeviceTensor(DT_BF16, (planes, rows, cols), fill=None)
+    y = iomx.DeviceTensor(DT_BF16, (planes, rows, cols), fill=0x5A)
+    x1 = iomx.DeviceTensor(DT_BF16, (1, rows, cols), fill=None)
+    y1 = iomx.DeviceTensor(DT_BF16, (1, rows, cols), fill=0x5A)
+    assert iomx.binary(OP_ADD, one.view(), zero.view(), x.view()) == 0           # forty copies of one + 0
+    assert iomx.binary(OP_ADD, one.view(), zero.view().slice(0, 0, 1), x1.view()) == 0
+
+    def same_in_every_plane(big, small):
+        got, want = big.raw().reshape(planes, plane), small.raw()
+        for p in range(planes):
+            assert np.array_equal(got[p], want), p
+
+    same_in_every_plane(x, x1)
+    assert iomx.rmsnorm(x.view(), scale.view(), y.view(), 1e-5) == 0
+    assert iomx.rmsnorm(x1.view(), scale.view(), y1.view(), 1e-5) == 0
+    same_in_every_plane(y, y1)
+    weight, _ = upload(DT_BF16, (cols, cols), "normal_small", 75)
+    assert iomx.linear(x.view(), weight.view(), y.view(), 0, rows, False, 1, cols) == 0
+    assert iomx.last_launch().kernel.decode() == "linear_mfma_lds"
+    assert iomx.linear(x1.view(), weight.view(), y1.view(), 0, rows, False, 1, cols) == 0
+    same_in_every_plane(y, y1)
+    assert iomx.rope(x.view(), y.view(), 3, 10000.0) == 0
+    assert iomx.rope(x1.view(), y1.view(), 3, 10000.0) == 0
+    same_in_every_plane(y, y1)
+    assert iomx.silu(x.view(), y.view()) == 0
+    assert iomx.silu(x1.view(), y1.view()) == 0
+    same_in_every_plane(y, y1)
+    assert iomx.copy(y.view(), x.view()) == 0
+    same_in_every_plane(x, y1)
+    for t in (one, zero, scale, weight, x, y, x1, y1):
         t.free()
 
 
