@@ -233,6 +233,91 @@ def test_rmsnorm_linear_rope_silu_and_copy_beyond_4_gib():
         t.free()
 
 
+def test_attention_cache_append_and_embedding_beyond_4_gib():
+    """K and V caches [40,8,65536,128] BF16 (5 GiB each, forty copies of one sequence): a decode
+    step over the whole prefix gives every sequence the same bits (and those of a call on one
+    sequence alone within the reference's acceptance rule, since that call may share out the
+    tokens differently); an append of sixteen rows and an embedding lookup into a 5 GiB result
+    give, for every sequence, the bits of the same call on one sequence alone."""
+    B, Hq, Hkv, C, D = 40, 32, 8, 65536, 128
+    zero = iomx.DeviceTensor(DT_BF16, (B, 1, 1, 1), fill=0)
+
+    def copies(dims, kind, salt):
+        """(forty copies, the one) of a pattern plane, as value + 0."""
+        src, _ = upload(DT_BF16, (1,) + dims, kind, salt)
+        big = iomx.DeviceTensor(DT_BF16, (B,) + dims, fill=None)
+        one = iomx.DeviceTensor(DT_BF16, (1,) + dims, fill=None)
+        assert iomx.binary(OP_ADD, src.view(), zero.view(), big.view()) == 0
+        assert iomx.binary(OP_ADD, src.view(), zero.view().slice(0, 0, 1), one.view()) == 0
+        src.free()
+        return big, one
+
+    def same_for_every_sequence(big, small):
+        got, want = big.raw().reshape(B, -1), small.raw().reshape(-1)
+        for b in range(B):
+            differ = np.flatnonzero(got[b] != want)
+            assert differ.size == 0, (b, differ.size, differ[:4], got[b][differ[:4]], want[differ[:4]],
+                                      iomx.last_launch().kernel.decode())
+
+    k, k1 = copies((Hkv, C, D), "normal", 81)
+    v, v1 = copies((Hkv, C, D), "normal", 82)
+    same_for_every_sequence(k, k1)
+
+    # sixteen new rows at positions 65000..65015 of every head
+    new, new1 = copies((Hkv, 16, D), "normal", 84)
+    assert iomx.cache_append(new.view(), k.view(), 65000) == 0
+    assert iomx.cache_append(new1.view(), k1.view(), 65000) == 0
+    same_for_every_sequence(k, k1)
+
+    # a decode step (one query row) and a sixteen-row step over the whole prefix
+    for R in (1, 16):
+        o = iomx.DeviceTensor(DT_BF16, (B, R, Hq * D), fill=0x5A)
+        o1 = iomx.DeviceTensor(DT_BF16, (1, R, Hq * D), fill=0x5A)
+        rows = datagen.bf16_rne(datagen.normal_f32(Hq * R * D, 0, 1, 85 + R)).reshape(1, Hq, R, D)
+        qq = iomx.DeviceTensor(DT_BF16, (B, Hq, R, D)); qq.view().from_host(np.repeat(rows, B, axis=0))
+        qq1 = iomx.DeviceTensor(DT_BF16, (1, Hq, R, D)); qq1.view().from_host(rows)
+        for dq, do, dk, dv in ((qq, o, k, v), (qq1, o1, k1, v1)):
+            rc, nbytes, _ = iomx.sdpa_workspace(dq.view(), dk.view(), dv.view(), do.view(), C - R, C)
+            assert rc == 0
+            ws = iomx.Buffer(max(nbytes, 256))
+            assert iomx.sdpa(dq.view(), dk.view(), dv.view(), do.view(), C - R, C, ws) == 0
+            iomx.synchronize()
+            ws.free()
+        # within the launch every sequence must have the same bits; the launch on one sequence may
+        # share out the tokens differently (other partial sums), so it is held to the reference's
+        # acceptance rule for attention instead
+        whole = o.view().to_host()
+        for b in range(1, B):
+            assert np.array_equal(whole[b], whole[0]), b
+        alone = o1.view().to_host().reshape(-1)
+        from test_oracle_sdpa import bf16_class, matches
+        outside = [i for i, (x, y) in enumerate(zip(whole[0].reshape(-1), alone))
+                   if not matches(int(x), int(y), bf16_class(int(y)))]
+        assert not outside, (R, len(outside))
+        for t in (o, o1, qq, qq1):
+            t.free()
+
+    # embedding: [40,1,32768] ids into [40,32768,2048]
+    V, F, R = 32000, 2048, 32768
+    table, _ = upload(DT_BF16, (V, F), "normal", 90)
+    ids_one = (datagen.pattern_bits(32, R, 91) % V).astype(np.int32).reshape(1, 1, R)
+    ids = iomx.DeviceTensor(DT_I32, (B, 1, R)); ids.view().from_host(np.repeat(ids_one, B, axis=0))
+    ids1 = iomx.DeviceTensor(DT_I32, (1, 1, R)); ids1.view().from_host(ids_one)
+    out = iomx.DeviceTensor(DT_BF16, (B, R, F), fill=0x5A)
+    out1 = iomx.DeviceTensor(DT_BF16, (1, R, F), fill=0x5A)
+    status = iomx.Buffer(32)
+    for t, i, o in ((table, ids, out), (table, ids1, out1)):
+        status.fill(0xFF)
+        iomx.synchronize()
+        assert iomx.embedding(t.view(), i.view(), o.view(), status) == 0
+        iomx.synchronize()
+        assert int(status.download(np.uint32)[0]) == 0
+    same_for_every_sequence(out, out1)
+    for t in (zero, k, k1, v, v1, new, new1, table, ids, ids1, out, out1):
+        t.free()
+    status.free()
+
+
 @pytest.mark.parametrize("dtype", [DT_BF16, DT_F32])
 def test_config3_rmsnorm_32768x2048(dtype):
     R, F = 32768, 2048
