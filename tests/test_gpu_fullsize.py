@@ -167,6 +167,15 @@ def test_elementwise_on_tensors_beyond_4_gib():
     e1 = bf16_op(a_raw, np.zeros_like(a_raw), OP_ADD)
     every_plane(t, e1)
 
+    # the host transfers of the same 5 GiB: tiled -> logical rows, and back into the other tensor
+    logical = t.view().to_host()
+    rows_of_e1 = e1.reshape(rows // 16, cols // 16, 16, 16).transpose(0, 2, 1, 3).reshape(rows, cols)
+    for p in range(planes):
+        assert np.array_equal(logical[p], rows_of_e1), p
+    u.view().from_host(logical)
+    del logical
+    every_plane(u, e1)
+
     assert iomx.binary(OP_ADD, t.view(), t.view(), u.view()) == 0               # u = t + t
     assert iomx.last_launch().kernel.decode() == "binary_planes"
     e2 = bf16_op(e1, e1, OP_ADD)
