@@ -14,8 +14,11 @@ oracle on sampled planes / rows, and through size-independent properties.
   attention 8 x 32/4 heads, R = L = 512, D = 64 BF16        uniform-score closed form, sampled
                                                             rows against the oracle
   beyond 4 GiB: ADD / MUL on [40,64,2^20] BF16 through each elementwise kernel family against the
-            closed form; RMSNorm, linear, RoPE, SiLU and copy on [40,32768,2048] BF16 against the
-            same operation on one plane                     bit-exact, every element
+            closed form, and its host transfers; one [65536,65536] plane (2^32 elements);
+            RMSNorm, linear, RoPE, SiLU and copy on [40,32768,2048] BF16, cache append and
+            embedding at 5 GiB against the same operation on one plane
+                                                            bit-exact, every element
+            a decode step over 5 GiB K and V caches         identical for every sequence
 """
 import numpy as np
 import pytest
@@ -197,6 +200,50 @@ def test_elementwise_on_tensors_beyond_4_gib():
     w.free()
     for x in (a, zero, r, t, u):
         x.free()
+
+
+def test_elementwise_on_one_plane_of_8_gib():
+    """One [65536,65536] BF16 matrix: 2^32 elements, 8 GiB, offsets inside a single plane beyond
+    32 bits.  A row vector plus a column of zeros (two broadcast operands: the per-piece general
+    kernel) gives 4096 identical bands; then the dense shape and the tile-row bands on them, and
+    RMSNorm (65536 features a row) and SiLU against the same launch on one band."""
+    n = 65536
+    vec = datagen.bf16_rne(datagen.uniform_f32(n, 0.5, 1.5, 76))
+    r = iomx.DeviceTensor(DT_BF16, (1, n))
+    r.upload_raw(vector_storage(vec))
+    c = iomx.DeviceTensor(DT_BF16, (n, 1), fill=0)
+    x = iomx.DeviceTensor(DT_BF16, (n, n), fill=0x5A)
+    y = iomx.DeviceTensor(DT_BF16, (n, n), fill=0x5A)
+    col = column_of_storage((16, n))
+
+    def every_band(tensor, want):
+        got = tensor.raw().reshape(n // 16, 16 * n)
+        for band in range(n // 16):
+            assert np.array_equal(got[band], want), band
+
+    assert iomx.binary(OP_ADD, r.view(), c.view(), x.view()) == 0                # x[i][j] = r[j] + 0
+    assert iomx.last_launch().kernel.decode() == "binary_general"
+    e1 = bf16_op(vec[col], np.zeros(col.size, np.uint16), OP_ADD)
+    every_band(x, e1)
+    assert iomx.binary(OP_ADD, x.view(), x.view(), y.view()) == 0                # y = x + x
+    assert iomx.last_launch().kernel.decode() == "binary_planes"
+    e2 = bf16_op(e1, e1, OP_ADD)
+    every_band(y, e2)
+    assert iomx.binary(OP_MUL, r.view(), y.view(), x.view()) == 0                # x = r * y
+    assert iomx.last_launch().kernel.decode() == "binary_rowvec"
+    every_band(x, bf16_op(vec[col], e2, OP_MUL))
+    # RMSNorm and SiLU of the 65536 identical rows against the same launch on one band of them
+    xs = iomx.DeviceTensor(DT_BF16, (16, n), fill=None)
+    ys = iomx.DeviceTensor(DT_BF16, (16, n), fill=0x5A)
+    xs.upload_raw(x.raw()[:16 * n])
+    assert iomx.rmsnorm(x.view(), r.view(), y.view(), 1e-5) == 0
+    assert iomx.rmsnorm(xs.view(), r.view(), ys.view(), 1e-5) == 0
+    every_band(y, ys.raw())
+    assert iomx.silu(x.view(), y.view()) == 0
+    assert iomx.silu(xs.view(), ys.view()) == 0
+    every_band(y, ys.raw())
+    for t in (r, c, x, y, xs, ys):
+        t.free()
 
 
 def test_rmsnorm_linear_rope_silu_and_copy_beyond_4_gib():
