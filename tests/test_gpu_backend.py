@@ -392,3 +392,35 @@ def test_submit_and_wait_cost_through_device_ops(devices, capsys):
         assert single[100] < 2e-3 and burst < 1e-3
         close(a, b, o)
     gpu.close()
+
+
+def test_tensors_beyond_4_gib_in_a_large_arena():
+    """An 18 GiB arena with two [40,64,2^20] BF16 tensors (5 GiB each) and room for the 5 GiB
+    staging range of a whole-tensor transfer: arena offsets, window byte counts and the host
+    transfers of the backend beyond 32 bits.  t = a + 0 over forty planes
+    (a scalar per plane), u = t * r with a row vector; every plane against the closed form."""
+    if not iomo.mi355x_available():
+        pytest.skip("oracle/_ref/libiom_mi355x_shim.so not built (needs the reference headers)")
+    gpu = iomo.mi355x_backend(arena_bytes=18 << 30, max_in_flight=4)
+    planes, rows, cols = 40, 64, 1 << 20
+    a_values = datagen.bf16_rne(datagen.normal_f32(rows * cols, 0, 1, 301)).reshape(1, rows, cols)
+    r_values = datagen.bf16_rne(datagen.uniform_f32(cols, 0.5, 1.5, 302)).reshape(1, cols)
+    a = gpu.tensor(DT_BF16, (1, rows, cols)); a.view().from_host(a_values)
+    r = gpu.tensor(DT_BF16, (1, cols)); r.view().from_host(r_values)
+    zero = gpu.tensor(DT_BF16, (planes, 1, 1)); zero.view().from_host(np.zeros((planes, 1, 1), np.uint16))
+    t = gpu.tensor(DT_BF16, (planes, rows, cols))
+    u = gpu.tensor(DT_BF16, (planes, rows, cols))
+    assert gpu.binary(OP_ADD, a.view(), zero.view(), t.view()) > 0, gpu.error()
+    assert gpu.binary(OP_MUL, t.view(), r.view(), u.view()) > 0, gpu.error()
+    fa = datagen.bf16_to_f32(a_values.reshape(-1))
+    e1 = datagen.bf16_rne(fa + np.float32(0)).reshape(rows, cols)
+    e2 = datagen.bf16_rne(datagen.bf16_to_f32(e1.reshape(-1)).reshape(rows, cols)
+                          * datagen.bf16_to_f32(r_values.reshape(-1))[None, :]).reshape(rows, cols)
+    got = t.view().to_host()
+    for p in range(planes):
+        assert np.array_equal(got[p], e1), p
+    got = u.view().to_host()
+    for p in range(planes):
+        assert np.array_equal(got[p], e2), p
+    close(a, r, zero, t, u)
+    gpu.close()
