@@ -289,7 +289,8 @@ int iomx_launch_rope(int dtype, const iomx_view* x, const iomx_view* out, uint64
  * memory (any shape; the fallback of path 0 and the cross-check of the other two);
  * paths 3, 4 and 5 are path 0 with the workgroup tile forced to 256 x 256 (wherever
  * there are 256 rows), 128 x 128 and 64 x 64 (path 0 picks by how many CUs the
- * problem fills): for tests.
+ * problem fills), path 6 forces 128 x 128 with two groups of waves that each take
+ * half of the inner axis (I % 64 == 0, else as path 0): for tests.
  */
 int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const iomx_view* out,
                        uint64_t s, uint64_t R, int head_planar, uint64_t H, uint64_t D, int path,

@@ -526,11 +526,15 @@ __device__ __forceinline__ bool block_of_workgroup(const LinearArgs& a, uint32_t
     return true;
 }
 
-template <int WM, int WVM, int WVN, int DEPTH>
-__global__ __launch_bounds__(WVM * WVN * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// GROUPS > 1: that many sets of WVM x WVN waves in one workgroup, each with a ring of its own
+// over a GROUPS-th of the inner axis (I / 32 divisible by GROUPS); the partial sums meet in LDS
+// at the end, in group order.  For launches with fewer blocks than CUs, whose duration is the
+// time one workgroup needs for its chain of stages.
+template <int WM, int WVM, int WVN, int DEPTH, int GROUPS = 1>
+__global__ __launch_bounds__(WVM * WVN * 64 * GROUPS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     constexpr int WN = 4;                                   // wave tile WM x WN, in 16x16 tiles
-    constexpr int NW = WVM * WVN;                           // waves, WVM along the rows
+    constexpr int NW = WVM * WVN;                           // waves of a group, WVM along the rows
     constexpr uint32_t BM = WM * WVM, BN = WN * WVN;        // workgroup tile, in 16x16 tiles
     constexpr int KS = 1, HALF = WM / 2;                    // DEPTH stage buffers of 32 inner elements
     constexpr int LPS = (BM + BN) / NW;                     // direct loads per wave and stage
@@ -538,14 +542,19 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     static_assert(WM >= 4 && WM % 2 == 0 && LPS % HALF == 0, "loads spread over the second half of a stage");
     constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
     constexpr uint32_t kStageFrags = (BM + BN) * KS, kStageBytes = kStageFrags * kFrag;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[DEPTH * kStageBytes];
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    __shared__ __attribute__((aligned(16))) uint8_t all_rings[GROUPS * DEPTH * kStageBytes];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t group = GROUPS > 1 ? (threadIdx.x >> 6) / NW : 0, wave = (threadIdx.x >> 6) % NW;
+    uint8_t* lds = all_rings + group * (DEPTH * kStageBytes);
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     const uint32_t total_rows = a.planes * a.R;
     uint32_t bx, by;
     if (!block_of_workgroup(a, &bx, &by)) return;
     const uint32_t bm0 = bx * BM, bn0 = a.out_tile0 + by * BN;   // first row tile / output tile
     const uint32_t wm = wave % WVM, wn = wave / WVM;
+    // this group's part of the inner axis: stages [group * stages, (group + 1) * stages)
+    const uint32_t stages = a.I / 32 / GROUPS;
+    const uint64_t group_off = (uint64_t)group * stages * kFrag;
 
     // loader role: this wave brings in row fragments wave, wave+NW and output fragments
     // wave, wave+NW of every 32-element slice; lane i fetches 16-byte chunk i
@@ -561,13 +570,14 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
         walk_planes(a.walk, p, plane);
         const uint32_t srow = a.s + r;
         src[j] = a.x + plane[0] * a.x_plane_bytes + (uint64_t)(srow >> 4) * a.x_tile_cols * kTileBytes
-                + (srow & 15u) * kRowBytes + ld_off;
+                + (srow & 15u) * kRowBytes + ld_off + group_off;
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         uint32_t o = (bn0 + wave + NW * j) * kTile + ld_row;
         if (o >= a.O) o = 0;
-        src[2 + j] = a.w + (uint64_t)(o >> 4) * a.w_tile_cols * kTileBytes + (o & 15u) * kRowBytes + ld_off;
+        src[2 + j] = a.w + (uint64_t)(o >> 4) * a.w_tile_cols * kTileBytes + (o & 15u) * kRowBytes + ld_off
+                + group_off;
     }
     auto issue = [&](uint32_t stage, uint32_t buf) {
 #pragma unroll
@@ -590,7 +600,6 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
 
     // reader role: position of the lane's eight inner elements inside a fragment
     const uint32_t rd_off = (kg >> 1) * kTileBytes + l16 * kRowBytes + (kg & 1u) * 16;
-    const uint32_t stages = a.I / 32;
     // A ring of DEPTH stage buffers (one stage = 32 inner elements; four for the large tile,
     // five for the small one whose stages are half as long) and two register sets of operand
     // fragments.  At the top of stage st every wave waits for its own loads of stage st+1 and
@@ -666,6 +675,28 @@ void linear_mfma_lds_bf16_kernel(const LinearArgs a) {
     if (st < stages) stage(std::integral_constant<int, 0>{}, st);
     // nothing may still be landing in LDS when the workgroup gives it back
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (GROUPS > 1) {
+        // the other groups' partial sums through the (now idle) rings: [group - 1][wave][tile][lane]
+        __syncthreads();
+        f32x4_t* part = reinterpret_cast<f32x4_t*>(all_rings);
+        static_assert((GROUPS - 1) * NW * WM * WN * 1024 <= GROUPS * DEPTH * kStageBytes, "partial sums fit the rings");
+        if (group > 0) {
+#pragma unroll
+            for (int m = 0; m < WM; ++m)
+#pragma unroll
+                for (int n = 0; n < WN; ++n)
+                    part[((((group - 1) * NW + wave) * WM + m) * WN + n) * 64 + lane] = acc[m][n];
+        }
+        __syncthreads();
+        if (group > 0) return;
+#pragma unroll 1
+        for (uint32_t g = 0; g + 1 < GROUPS; ++g)
+#pragma unroll
+            for (int m = 0; m < WM; ++m)
+#pragma unroll
+                for (int n = 0; n < WN; ++n)
+                    acc[m][n] += part[(((g * NW + wave) * WM + m) * WN + n) * 64 + lane];
+    }
 
     // lane holds outputs o = tile*16 + 4*(lane/16) + j (j < 4) of row l16 of its row tiles.
     // Heads are whole tiles wide here, so head and tile of an output tile are the same
@@ -927,6 +958,18 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                 if (path == 4) bt = 8;
                 if (path == 5) bt = 4;
                 // output tiles [first, first + count) with workgroup tiles of bt x bt 16x16 tiles
+                // 130 to 256 blocks of 128 x 128 are one round in which each CU has a single workgroup
+                // and the launch lasts as long as that workgroup's chain of stages: two groups of
+                // waves then each take half of the inner axis (measured at 384-640 rows x
+                // [4096..8192, 2048 or 4096]: 12-38 % faster than the 64 x 64 blocks, e.g. 512 rows x
+                // [5632,2048] 21.4 -> 17.5 us, 640 rows x [5632,4096] 50.7 -> 31.8 us; with 128
+                // blocks or fewer the 64 x 64 blocks with their own groups stay ahead)
+                uint32_t groups = 1;
+                const bool halves = (a.I / 32) % 2 == 0 && a.I >= 128;
+                if (halves && (path == 6 || (path == 0 && bt != 16 && mid >= 130 && mid <= 256 && a.I >= 1024))) {
+                    bt = 8;
+                    groups = 2;
+                }
                 auto launch_part = [&](uint32_t first, uint32_t count, uint32_t tile) -> int {
                     LinearArgs b = a;
                     b.out_tile0 = first;
@@ -937,17 +980,29 @@ extern "C" int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view
                     b.blocks_per_xcd = (uint32_t)((blocks + 7) / 8);
                     const uint64_t wgs = (uint64_t)b.blocks_per_xcd * 8;
                     const dim3 grid((uint32_t)wgs);
-                    if (tile == 16) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4, 4>), grid, dim3(512), 0, st, b);
-                    else if (tile == 8) hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 5>), grid, dim3(256), 0, st, b);
-                    else {
+                    uint32_t threads = 256;
+                    if (tile == 16) {
+                        threads = 512;
+                        hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<8, 2, 4, 4>), grid, dim3(512), 0, st, b);
+                    } else if (tile == 8 && groups == 2) {
+                        threads = 512;
+                        hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 4, 2>), grid, dim3(512), 0, st, b);
+                    } else if (tile == 8) {
+                        hipLaunchKernelGGL((linear_mfma_lds_bf16_kernel<4, 2, 2, 5>), grid, dim3(256), 0, st, b);
+                    } else {
                         // fewer blocks than CUs: two or four groups of waves share the inner axis
                         const uint32_t stages = a.I / 32;
-                        const uint32_t ks = path == 5 ? 1 : blocks <= 128 && stages >= 32 ? 4 : blocks <= 256 && stages >= 16 ? 2 : 1;
+                        // (measured at 512 rows: [2048,5632] 26 -> 20 us and [2048,2048] 12 -> 10 us with
+                        // four groups instead of two; 256 rows x [5632,2048], 352 blocks, 14 -> 13 us with two)
+                        const uint32_t ks = path == 5 ? 1
+                                : (blocks <= 128 && stages >= 32) || (blocks <= 256 && stages >= 64) ? 4
+                                : (blocks <= 256 && stages >= 16) || (blocks <= 384 && stages >= 32) ? 2 : 1;
+                        threads = 256 * ks;
                         if (ks == 4) hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4, 4>), grid, dim3(1024), 0, st, b);
                         else if (ks == 2) hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4, 2>), grid, dim3(512), 0, st, b);
                         else hipLaunchKernelGGL((linear_mfma_lds64_bf16_kernel<4, 1>), grid, dim3(256), 0, st, b);
                     }
-                    record_launch("linear_mfma_lds", grid.x, tile == 16 ? 512 : 256, (uint64_t)row_tiles * count);
+                    record_launch("linear_mfma_lds", grid.x, threads, (uint64_t)row_tiles * count);
                     return IOMX_OK;
                 };
                 // 256 x 256 blocks that fill whole rounds of the 256 CUs, and the rest of the

@@ -297,6 +297,60 @@ def test_bf16_small_tiles_with_the_inner_axis_shared_by_groups_of_waves(inner):
         t.free()
 
 
+@pytest.mark.parametrize("inner", [128, 192, 448, 2048])
+def test_bf16_tiles_of_128_with_the_inner_axis_in_two_halves(inner):
+    """128 x 128 blocks whose two groups of waves each take half of the stages (2, 3, 7 and 32
+    stages a group: fewer than the ring holds, odd counts) and add their partial sums in LDS.
+    300 rows over 2 planes with a window, 80 outputs in 5 heads; the contract's BF16 bound
+    against float64, one-hot rows at both ends of both halves exactly, untouched padding."""
+    xd, wd, s, R, H, D = (2, 160, inner), (80, inner), 7, 150, 5, 16
+    xv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(xd)), 0, 1, 71 + inner)).reshape(xd)
+    wv = datagen.bf16_rne(datagen.normal_f32(int(np.prod(wd)), 0, 0.2, 72 + inner)).reshape(wd)
+    hot = {(1, 3): inner - 1, (0, 149): 0, (1, 77): inner // 2, (0, 20): inner // 2 - 1}
+    for (b, r), i in hot.items():
+        xv[b, s + r, :] = 0
+        xv[b, s + r, i] = 0x3F80
+    dx, _ = pair(DT_BF16, xd, values=xv)
+    dw, _ = pair(DT_BF16, wd, values=wv)
+    od = (2, H, R, D)
+    do, ho = pair(DT_BF16, od, salt=73)
+    assert iomx.linear(dx.view(), dw.view(), do.view(), s, R, True, H, D, path=6) == 0
+    assert iomx.last_launch().kernel.decode() == "linear_mfma_lds"
+    assert iomx.last_launch().block == 512
+    got = do.view().to_host().transpose(0, 2, 1, 3).reshape(2, R, H * D)
+    for b in range(2):
+        assert bf16_bound(got[b], xv[b, s:s + R], wv).all()
+    for (b, r), i in hot.items():
+        assert np.array_equal(got[b, r], wv[:, i]), (b, r, i)
+    mask = iomo.tile_plane(np.ones(od, np.uint16)) == 0
+    assert np.array_equal(do.raw()[mask], ho.storage[mask])
+    for t in (dx, dw, do):
+        t.free()
+
+
+def test_bf16_one_round_of_128_blocks_takes_the_two_halves():
+    """512 rows x [5632,2048] is 176 blocks of 128 x 128: one workgroup on each of 176 CUs, so the
+    launch picks the two-group form; sampled rows against float64, and the rows of a second
+    plane with the same values give the same bits."""
+    S, I, O = 512, 2048, 5632
+    xv = datagen.bf16_rne(datagen.normal_f32(S * I, 0, 1, 81)).reshape(1, S, I)
+    wv = datagen.bf16_rne(datagen.normal_f32(O * I, 0, 0.02, 82)).reshape(O, I)
+    dx, _ = pair(DT_BF16, (1, S, I), values=xv)
+    dw, _ = pair(DT_BF16, (O, I), values=wv)
+    do, _ = pair(DT_BF16, (1, S, O), salt=83)
+    assert iomx.linear(dx.view(), dw.view(), do.view(), 0, S, False, 1, O) == 0
+    launch = iomx.last_launch()
+    assert launch.kernel.decode() == "linear_mfma_lds" and launch.block == 512 and launch.grid == 176
+    got = do.view().to_host()
+    for r in (0, 17, 255, 256, 511):
+        assert bf16_bound(got[0, r:r + 1], xv[0, r:r + 1], wv).all()
+    d2, _ = pair(DT_BF16, (1, S, O), salt=84)
+    assert iomx.linear(dx.view(), dw.view(), d2.view(), 0, S, False, 1, O, path=6) == 0
+    assert np.array_equal(d2.raw(), do.raw())
+    for t in (dx, dw, do, d2):
+        t.free()
+
+
 # (x dims, s, R, head planar, H, D, inner, workgroups expected): decode steps of 17-64
 # sequences, where one workgroup takes two or four row tiles against two or four output
 # tiles; ragged last row tile, ragged last output tile, ragged inner axis, rows of one plane
