@@ -57,7 +57,7 @@ def test_binary_on_random_views(case):
     if op == OP_DIV and dtype not in FLOAT_LEAVES:
         op = OP_SUB
     lead, rows, cols, operands = view_cases.binary_case(case)
-    # every other round of four operations draws small magnitudes for the 8-bit floating leaves:
+    # every other block of four operations draws small magnitudes for the 8-bit floating leaves:
     # tile rows that the kernel rounds with the conversion instructions, not element by element
     small = (case // (4 * len(LEAVES))) % 2 == 1
     owners = [pair(dtype, dims, 0x900 + 3 * case + i, small) for i, (dims, _) in enumerate(operands)]
