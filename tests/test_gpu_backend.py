@@ -424,3 +424,37 @@ def test_tensors_beyond_4_gib_in_a_large_arena():
         assert np.array_equal(got[p], e2), p
     close(a, r, zero, t, u)
     gpu.close()
+
+
+def test_rank_eight_operands_like_the_reference_conformance_cases(devices):
+    """test/backend/backend_conformance_common.hpp:581-690: a rank-eight owner against a rank-two
+    operand, and the rank-eight broadcast add (a row vector per plane against one column vector)
+    with its closed form; both against the reference CPU backend as well."""
+    cpu, gpu = devices
+    DT_U8 = iomo.DT_U8
+    # rank eight + rank two
+    dims8 = (1, 1, 1, 1, 1, 1, 17, 33)
+    a_vals = datagen.pattern_bits(8, 17 * 33, 0x8A).reshape(dims8)
+    b_vals = datagen.pattern_bits(8, 17 * 33, 0x8B).reshape(17, 33)
+    results = []
+    for dev in (cpu, gpu):
+        l = dev.tensor(DT_U8, dims8); l.view().from_host(a_vals)
+        r = dev.tensor(DT_U8, (17, 33)); r.view().from_host(b_vals)
+        o = dev.tensor(DT_U8, dims8); o.view().from_host(np.zeros(dims8, np.uint8))
+        assert dev.binary(OP_ADD, l.view(), r.view(), o.view()) > 0, dev.error()
+        results.append(o.view().to_host())
+        close(l, r, o)
+    assert np.array_equal(results[0], results[1])
+    assert np.array_equal(results[1].reshape(17, 33), (a_vals.reshape(17, 33) + b_vals).astype(np.uint8))
+    # the rank-eight broadcast: lhs [.., 17, 1] carries one plane, rhs [.., 2, 1, 33] a row per plane
+    lhs_dims, rhs_dims, out_dims = (1, 1, 1, 1, 1, 1, 17, 1), (1, 1, 1, 1, 1, 2, 1, 33), (1, 1, 1, 1, 1, 2, 17, 33)
+    lhs_vals = datagen.pattern_bits(8, 17, 0x8C).reshape(lhs_dims)
+    rhs_vals = datagen.pattern_bits(8, 66, 0x8D).reshape(rhs_dims)
+    want = (lhs_vals.reshape(1, 17, 1).astype(np.uint32) + rhs_vals.reshape(2, 1, 33)).astype(np.uint8)
+    for dev in (cpu, gpu):
+        l = dev.tensor(DT_U8, lhs_dims); l.view().from_host(lhs_vals)
+        r = dev.tensor(DT_U8, rhs_dims); r.view().from_host(rhs_vals)
+        o = dev.tensor(DT_U8, out_dims); o.view().from_host(np.full(out_dims, 0xAA, np.uint8))
+        assert dev.binary(OP_ADD, l.view(), r.view(), o.view()) > 0, dev.error()
+        assert np.array_equal(o.view().to_host().reshape(2, 17, 33), want)
+        close(l, r, o)

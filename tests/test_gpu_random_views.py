@@ -73,6 +73,28 @@ def test_binary_on_random_views(case):
         d.free()
 
 
+@pytest.mark.parametrize("case", range(120))
+def test_binary_on_random_views_of_rank_up_to_eight(case):
+    """Five or six leading axes of extent 1-2 (rank seven or eight, the largest a shape can have:
+    include/iom/tensor.hpp:83-85), sliced, permuted and broadcast like the cases above."""
+    dtype = (iomo.DT_BF16, iomo.DT_I32, iomo.DT_U8, iomo.DT_F32, iomo.DT_U4, iomo.DT_F8_E5M2)[case % 6]
+    op = (OP_ADD, OP_MUL, OP_SUB)[(case // 6) % 3]
+    draw = case
+    lead, rows, cols, operands = view_cases.binary_case(draw, max_lead=6, max_extent=2, salt=0x808)
+    while len(lead) < 5:
+        draw += 1000
+        lead, rows, cols, operands = view_cases.binary_case(draw, max_lead=6, max_extent=2, salt=0x808)
+    owners = [pair(dtype, dims, 0x3F00 + 3 * case + i, True) for i, (dims, _) in enumerate(operands)]
+    dv = [view_cases.apply(d.view(), steps) for (d, _), (_, steps) in zip(owners, operands)]
+    hv = [view_cases.apply(h.view(), steps) for (_, h), (_, steps) in zip(owners, operands)]
+    rc = iomx.binary(op, dv[0], dv[1], dv[2])
+    assert rc == 0, (iomx.lib().iomx_error_string(rc), LEAF_NAME[dtype], operands)
+    assert iomo.binary(op, hv[0], hv[1], hv[2], ieee=True) == 0
+    assert same_storage(*owners[2]), (LEAF_NAME[dtype], op, lead, rows, cols, operands)
+    for d, _ in owners:
+        d.free()
+
+
 @pytest.mark.parametrize("case", range(CASES // 2))
 def test_copy_on_random_views(case):
     dtype = (LEAVES + (iomo.DT_BOOL, iomo.DT_F8_E8M0, iomo.DT_U2))[case % (len(LEAVES) + 3)]

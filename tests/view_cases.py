@@ -63,11 +63,11 @@ def viewed_operand(rng: Stream, lead: tuple, rows: int, cols: int):
     return tuple(owner) + (rows, cols), steps
 
 
-def binary_case(case: int):
+def binary_case(case: int, max_lead: int = 3, max_extent: int = 4, salt: int = 101):
     """(result lead, rows, cols, [lhs, rhs, out]) with lhs/rhs/out = (owner dims, steps)."""
-    rng = Stream(case, 101)
-    nlead = rng.below(4)
-    lead = tuple(1 + rng.below(4) for _ in range(nlead))
+    rng = Stream(case, salt)
+    nlead = rng.below(max_lead + 1)
+    lead = tuple(1 + rng.below(max_extent) for _ in range(nlead))
     rows = (1, 5, 15, 16, 17, 33, 32, 48)[rng.below(8)]
     cols = (1, 7, 16, 17, 31, 48, 256, 1040)[rng.below(8)]
     # every axis of the result is held in full by at least one input (the output shape is
