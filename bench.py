@@ -335,6 +335,22 @@ def wl_other_leaves(timer, steps, warmup):
                           iomx.last_launch().kernel.decode()))
         for t in (lhs, rhs, o):
             t.free()
+    # RMSNorm of a narrow leaf on the tile-row kernel (one workgroup per row)
+    rows, F = 32768, 2048
+    x = iomx.DeviceTensor(iomx.DT_F8_E4M3FN, (rows, F), fill=None)
+    x.upload_raw(datagen.pattern_bits(32, x.nbytes // 4, 5) & 0xBFBFBFBF)
+    w = iomx.DeviceTensor(iomx.DT_F8_E4M3FN, (1, F), fill=None)
+    w.upload_raw((datagen.pattern_bits(32, w.nbytes // 4, 6) & 0x07070707) | 0x38383838)   # 1.0 .. 1.875
+    y = iomx.DeviceTensor(iomx.DT_F8_E4M3FN, (rows, F), fill=None)
+
+    def norm(i):
+        check(iomx.rmsnorm(x.view(), w.view(), y.view(), 1e-5, timer.stream), "rmsnorm f8")
+
+    wall, ev = timer.run(norm, steps, warmup)
+    out.append(report("rmsnorm_f8_e4m3fn_[32768,2048]", 2 * rows * F + F, rows * F, wall, ev,
+                      iomx.last_launch().kernel.decode()))
+    for t in (x, w, y):
+        t.free()
     return out
 
 

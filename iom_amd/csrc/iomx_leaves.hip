@@ -42,63 +42,6 @@ struct RowsArgs {
     uint32_t brow[2], bcol[2];
 };
 
-// A tile row of an 8-bit floating leaf through the conversion instructions: taken
-// when no input lies in the all-NaN top exponent of F8_E4M3FN and every result is a
-// number no larger than the largest finite value (false for a NaN result); the caller
-// computes any other row element by element on the raw bits.
-template <int DT, int OP, int N>
-__device__ __forceinline__ bool hw_f8_row(const uint32_t (&in)[N][4], const uint32_t (&bcol)[2],
-                                          uint32_t (&res)[4]) {
-    bool plain = true;
-    if constexpr (DT == DT_F8_E4M3FN) {
-#pragma unroll
-        for (int k = 0; k < N; ++k)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) plain &= !e4m3_top_exponent(in[k][j]);
-    }
-    float r[kTile];
-#pragma unroll
-    for (int i = 0; i < (int)kTile; ++i) {
-        const float x = bcol[0] ? hw_f8_value<DT>(in[0][0], 0) : hw_f8_value<DT>(in[0][i >> 2], i & 3);
-        if constexpr (N == 2) {
-            const float y = bcol[1] ? hw_f8_value<DT>(in[1][0], 0) : hw_f8_value<DT>(in[1][i >> 2], i & 3);
-            r[i] = leaf_arith<OP>(x, y);
-        } else {
-            r[i] = silu_carrier(x);
-        }
-        plain &= __builtin_fabsf(r[i]) <= hw_f8_limit<DT>();
-    }
-    if (!plain) return false;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        uint32_t w = hw_f8_pack<DT>(r[4 * j], r[4 * j + 1], 0u, false);
-        res[j] = hw_f8_pack<DT>(r[4 * j + 2], r[4 * j + 3], w, true);
-    }
-    return true;
-}
-
-// A tile row of a 4- or 6-bit floating leaf through the scaled conversions.  Operands
-// are finite, so only a quotient can be a NaN (0/0).
-template <int DT, int OP, int N>
-__device__ __forceinline__ void hw_f46_row(const uint32_t (&in)[N][bits_of(DT) / 2], const uint32_t (&bcol)[2],
-                                           uint32_t (&res)[bits_of(DT) / 2]) {
-    float v[N][kTile], r[kTile];
-#pragma unroll
-    for (int k = 0; k < N; ++k) hw_f46_decode<DT>(in[k], v[k]);
-#pragma unroll
-    for (int i = 0; i < (int)kTile; ++i) {
-        const float x = bcol[0] ? v[0][0] : v[0][i];
-        if constexpr (N == 2) {
-            const float y = bcol[1] ? v[1][0] : v[1][i];
-            r[i] = leaf_arith<OP>(x, y);
-            if constexpr (OP == IOMX_OP_DIV) r[i] = (r[i] != r[i]) ? hw_f46_largest<DT>() : r[i];
-        } else {
-            r[i] = silu_carrier(x);
-        }
-    }
-    hw_f46_encode<DT>(r, res);
-}
-
 template <int DT, int OP>
 __global__ __launch_bounds__(256) void rows_kernel(const RowsArgs a) {
     constexpr int BITS = bits_of(DT);
@@ -123,21 +66,29 @@ __global__ __launch_bounds__(256) void rows_kernel(const RowsArgs a) {
             else load_row<BITS, true>(src, in[k]);
         }
         uint32_t res[K];
-        bool converted = false;
-        if constexpr (has_hw_f8(DT) && OP != ROWS_OP_COPY) converted = hw_f8_row<DT, OP>(in, a.bcol, res);
-        if constexpr (has_hw_f46(DT) && OP != ROWS_OP_COPY) {
-            hw_f46_row<DT, OP>(in, a.bcol, res);
-            converted = true;
-        }
         if constexpr (OP == ROWS_OP_COPY) {
 #pragma unroll
             for (int j = 0; j < K; ++j) res[j] = in[0][j];
+        } else if constexpr (has_hw_convert(DT)) {
+            // the 4-, 6- and 8-bit floating leaves: one binary32 operation between the conversions.
+            // Their operands are finite or (F8) decode to the infinity or NaN they stand for.
+            float v[kInputs][kTile], r[kTile];
+#pragma unroll
+            for (int k = 0; k < kInputs; ++k) hw_decode_row<DT>(in[k], v[k]);
+#pragma unroll
+            for (int i = 0; i < (int)kTile; ++i) {
+                const float x = a.bcol[0] ? v[0][0] : v[0][i];
+                if constexpr (kInputs == 2) r[i] = leaf_arith<OP>(x, a.bcol[1] ? v[1][0] : v[1][i]);
+                else r[i] = silu_carrier(x);
+            }
+            // finite operands: only a quotient (0/0) can be a NaN
+            hw_encode_row<DT, OP == IOMX_OP_DIV || has_hw_f8(DT)>(r, res);
         } else if constexpr (!is_float_leaf(DT) && BITS <= 4) {
 #pragma unroll
             for (int j = 0; j < K; ++j)
                 res[j] = swar_word<BITS, OP>(a.bcol[0] ? splat_lane<BITS>(in[0][0]) : in[0][j],
                                              a.bcol[1] ? splat_lane<BITS>(in[1][0]) : in[1][j]);
-        } else if (!converted) {
+        } else {
 #pragma unroll
             for (int j = 0; j < K; ++j) res[j] = 0;
 #pragma unroll
@@ -185,17 +136,46 @@ __device__ __forceinline__ T wave_sum(T v) {
     return v;
 }
 
+// Sixteen elements of a tile row in the carrier T and back: by the conversion instructions
+// for the narrow floating leaves, element by element otherwise.
+template <int DT, typename T>
+__device__ __forceinline__ void decode_row(const uint32_t (&w)[bits_of(DT) / 2], T (&v)[kTile]) {
+    if constexpr (has_hw_convert(DT)) {
+        hw_decode_row<DT>(w, v);
+    } else {
+#pragma unroll
+        for (int i = 0; i < (int)kTile; ++i) v[i] = decode_as<DT, T>(get<bits_of(DT)>(w, i));
+    }
+}
+template <int DT, typename T>
+__device__ __forceinline__ void encode_row(const T (&y)[kTile], uint32_t (&w)[bits_of(DT) / 2]) {
+    if constexpr (has_hw_convert(DT)) {
+        hw_encode_row<DT>(y, w);
+    } else {
+#pragma unroll
+        for (int j = 0; j < bits_of(DT) / 2; ++j) w[j] = 0;
+#pragma unroll
+        for (int i = 0; i < (int)kTile; ++i) put<bits_of(DT)>(w, i, encode_from<DT, T>(y[i]));
+    }
+}
+
 // Order of src/cpu/queue.cpp:1187-1234 in the carrier T: mean = sum / F,
 // shifted = mean + eps, root = sqrt, inverse = 1 / root, y = (x*inverse)*scale;
 // a NaN result is stored in its positive form (:1124-1134).
-template <int DT, typename T>
+// PER_WAVE: a wave per row, four rows per workgroup, no LDS and no barrier - for rows of at most
+// 8192 features, where a workgroup per row would leave most lanes idle (2048 features are 128 tile
+// rows: two a lane).  Otherwise a workgroup per row.
+template <int DT, typename T, bool PER_WAVE>
 __global__ __launch_bounds__(256) void rows_rmsnorm_kernel(const RowsRmsArgs a) {
     constexpr int BITS = bits_of(DT);
     constexpr int K = BITS / 2;
     constexpr uint32_t kRowBytes = 2 * BITS, kTileBytes = 32 * BITS;
+    constexpr uint32_t kLanes = PER_WAVE ? 64 : 256, kRowsPerGroup = PER_WAVE ? 4 : 1;
     __shared__ T part[4];
-    const uint32_t tid = threadIdx.x;
-    for (uint32_t lin = blockIdx.x; lin < a.total_rows; lin += gridDim.x) {
+    const uint32_t tid = PER_WAVE ? (threadIdx.x & 63u) : threadIdx.x;
+    const uint32_t first = PER_WAVE ? blockIdx.x * 4u + (threadIdx.x >> 6) : blockIdx.x;
+    for (uint64_t lin64 = first; lin64 < a.total_rows; lin64 += (uint64_t)gridDim.x * kRowsPerGroup) {
+        const uint32_t lin = (uint32_t)lin64;
         const uint32_t p = a.rows > 1 ? fast_div(lin, a.div_rows) : lin;
         const uint32_t row = lin - p * a.rows;
         uint64_t plane[2];
@@ -204,44 +184,44 @@ __global__ __launch_bounds__(256) void rows_rmsnorm_kernel(const RowsRmsArgs a) 
         const uint8_t* xrow = a.x + plane[0] * a.plane_bytes + inplane;
         uint8_t* orow = a.out + plane[1] * a.plane_bytes + inplane;
         T acc = 0;
-        for (uint32_t tc = tid; tc < a.tile_cols; tc += 256) {
+        for (uint32_t tc = tid; tc < a.tile_cols; tc += kLanes) {
             uint32_t w[K];
             load_row<BITS>(xrow + (uint64_t)tc * kTileBytes, w);
             const uint32_t left = a.feats - tc * kTile;
+            T v[kTile];
+            decode_row<DT, T>(w, v);
 #pragma unroll
-            for (int i = 0; i < (int)kTile; ++i) {
-                if ((uint32_t)i < left) {
-                    const T v = decode_as<DT, T>(get<BITS>(w, i));
-                    acc = acc + v * v;
-                }
-            }
+            for (int i = 0; i < (int)kTile; ++i)
+                if ((uint32_t)i < left) acc = acc + v[i] * v[i];
         }
         acc = wave_sum(acc);
-        if ((tid & 63u) == 0) part[tid >> 6] = acc;
-        __syncthreads();
-        const T total = ((part[0] + part[1]) + part[2]) + part[3];
+        T total = acc;
+        if constexpr (!PER_WAVE) {
+            if ((tid & 63u) == 0) part[tid >> 6] = acc;
+            __syncthreads();
+            total = ((part[0] + part[1]) + part[2]) + part[3];
+        }
         const T mean = total / (T)a.feats;
         const T shifted = mean + (T)a.eps;
         const T root = carrier_sqrt(shifted);
         const T inverse = (T)1 / root;
-        for (uint32_t tc = tid; tc < a.tile_cols; tc += 256) {
+        for (uint32_t tc = tid; tc < a.tile_cols; tc += kLanes) {
             uint32_t w[K], s[K], res[K];
             load_row<BITS>(xrow + (uint64_t)tc * kTileBytes, w);
             load_row<BITS>(a.scale + (uint64_t)tc * kTileBytes, s);
-#pragma unroll
-            for (int j = 0; j < K; ++j) res[j] = 0;
+            T v[kTile], g[kTile], y[kTile];
+            decode_row<DT, T>(w, v);
+            decode_row<DT, T>(s, g);
 #pragma unroll
             for (int i = 0; i < (int)kTile; ++i) {
-                const T v = decode_as<DT, T>(get<BITS>(w, i));
-                const T g = decode_as<DT, T>(get<BITS>(s, i));
-                const T normalized = v * inverse;
-                const T y = normalized * g;
-                put<BITS>(res, i, encode_from<DT, T>(y));
+                const T normalized = v[i] * inverse;
+                y[i] = normalized * g[i];
             }
+            encode_row<DT, T>(y, res);
             const uint32_t left = a.feats - tc * kTile;
             store_row<BITS>(orow + (uint64_t)tc * kTileBytes, res, left < kTile ? left : kTile);
         }
-        __syncthreads();
+        if constexpr (!PER_WAVE) __syncthreads();
     }
 }
 
@@ -453,9 +433,14 @@ int launch_rows_rmsnorm(int dtype, const RowsRmsnormRequest& r, hipStream_t stre
     a.total_rows = (uint32_t)total;
     a.div_rows = make_fast_div(a.rows);
     a.eps = r.eps;
-    const uint32_t grid = a.total_rows < (1u << 20) ? a.total_rows : (1u << 20);
-#define IOMX_RMS(DTV, T) \
-    hipLaunchKernelGGL((rows_rmsnorm_kernel<DTV, T>), dim3(grid), dim3(256), 0, stream, a)
+    const bool per_wave = a.tile_cols <= 512;
+    const uint32_t groups = per_wave ? (a.total_rows + 3) / 4 : a.total_rows;
+    const uint32_t grid = groups < (1u << 20) ? groups : (1u << 20);
+#define IOMX_RMS(DTV, T)                                                                                       \
+    do {                                                                                                       \
+        if (per_wave) hipLaunchKernelGGL((rows_rmsnorm_kernel<DTV, T, true>), dim3(grid), dim3(256), 0, stream, a); \
+        else hipLaunchKernelGGL((rows_rmsnorm_kernel<DTV, T, false>), dim3(grid), dim3(256), 0, stream, a);     \
+    } while (0)
     switch (dtype) {
         case DT_F4_E2M1: IOMX_RMS(DT_F4_E2M1, float); break;
         case DT_F6_E2M3: IOMX_RMS(DT_F6_E2M3, float); break;

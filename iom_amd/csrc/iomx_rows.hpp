@@ -533,6 +533,61 @@ __device__ __forceinline__ void hw_f46_encode(const float (&r)[kTile], uint32_t 
     }
 }
 
+// A tile row of one of the five leaves above, decoded and rounded by the conversion
+// instructions wherever they agree with the leaf's rule, by decode_f32 / encode_f32
+// elsewhere: exact for every encoding, the leaf's rounding for every binary32 value.
+constexpr bool has_hw_convert(int dt) { return has_hw_f8(dt) || has_hw_f46(dt); }
+
+template <int DT>
+__device__ __forceinline__ void hw_decode_row(const uint32_t (&w)[bits_of(DT) / 2], float (&v)[kTile]) {
+    if constexpr (has_hw_f46(DT)) {
+        hw_f46_decode<DT>(w, v);
+    } else {
+        // a row with the all-NaN top exponent of F8_E4M3FN in it goes element by element
+        bool special = false;
+        if constexpr (DT == DT_F8_E4M3FN)
+            special = e4m3_top_exponent(w[0]) | e4m3_top_exponent(w[1]) | e4m3_top_exponent(w[2]) | e4m3_top_exponent(w[3]);
+        if (special) {
+#pragma unroll
+            for (int i = 0; i < (int)kTile; ++i) v[i] = decode_f32<DT>((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+        } else {
+#pragma unroll
+            for (int i = 0; i < (int)kTile; ++i) v[i] = hw_f8_value<DT>(w[i >> 2], i & 3);
+        }
+    }
+}
+
+// NANS = false: the caller knows that no value is a NaN (sums, differences and products of the
+// finite 4- and 6-bit values), which spares those leaves the replacement of a NaN.
+template <int DT, bool NANS = true>
+__device__ __forceinline__ void hw_encode_row(const float (&r)[kTile], uint32_t (&w)[bits_of(DT) / 2]) {
+    if constexpr (has_hw_f46(DT)) {
+        if constexpr (NANS) {
+            float s[kTile];
+#pragma unroll
+            for (int i = 0; i < (int)kTile; ++i) s[i] = (r[i] != r[i]) ? hw_f46_largest<DT>() : r[i];
+            hw_f46_encode<DT>(s, w);
+        } else {
+            hw_f46_encode<DT>(r, w);
+        }
+    } else {
+        // the instructions when all sixteen are numbers within the finite range (false for a NaN)
+        bool plain = true;
+#pragma unroll
+        for (int i = 0; i < (int)kTile; ++i) plain &= __builtin_fabsf(r[i]) <= hw_f8_limit<DT>();
+        if (plain) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                w[j] = hw_f8_pack<DT>(r[4 * j + 2], r[4 * j + 3], hw_f8_pack<DT>(r[4 * j], r[4 * j + 1], 0u, false), true);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[j] = 0;
+#pragma unroll
+            for (int i = 0; i < (int)kTile; ++i) w[i >> 2] |= encode_f32<DT>(r[i]) << (8 * (i & 3));
+        }
+    }
+}
+
 struct TileRow {
     uint32_t row, tc, ncols;
     bool live;
