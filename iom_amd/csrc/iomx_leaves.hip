@@ -377,6 +377,15 @@ int launch_rows(int op, int dtype, const RowsRequest& r, hipStream_t stream) {
     for (int k = 0; k < 2; ++k) { a.brow[k] = r.brow[k]; a.bcol[k] = r.bcol[k]; }
     dim3 grid;
     IOMX_TRY(plane_grid(r.m[2].tile_rows, r.m[2].tile_cols, r.walk.planes, &a.rows_per_plane, &grid));
+    // A lane's tile row is 4 to 16 bytes for the leaves of at most 8 bits: where the launch has
+    // workgroups to spare a lane walks four planes (two for the 8-bit leaves) with the one
+    // decomposition of its index (measured on [64,512,2048]: F6 21.8 -> 17.5 us, F4 16.9 -> 14.1,
+    // U4 14.2 -> 12.0, F8 24.4 -> 22.5; eight planes a lane were slower again)
+    if (bits <= 8) {
+        uint32_t per = bits == 8 ? 2 : 4;
+        while (per > 1 && (uint64_t)grid.x * ((grid.y + per - 1) / per) < 4096) per /= 2;
+        grid.y = (grid.y + per - 1) / per;
+    }
     const char* name = "rows_binary";
     if (op == ROWS_OP_COPY) {
         switch (bits) {
