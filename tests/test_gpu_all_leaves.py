@@ -200,6 +200,33 @@ def test_f8_silu_regrouped_by_the_range_of_its_result(dtype):
     do.free()
 
 
+@pytest.mark.parametrize("dtype", [iomo.DT_U2, iomo.DT_I4, iomo.DT_F4_E2M1, iomo.DT_F6_E2M3, iomo.DT_F8_E5M2],
+                         ids=["U2", "I4", "F4_E2M1", "F6_E2M3", "F8_E5M2"])
+def test_row_kernel_with_several_planes_per_lane(dtype):
+    """A launch large enough that a lane of the tile-row kernel walks two or more planes (the grid
+    covers fewer planes than the view has): seven planes, every other one of a larger owner, so the
+    last lane group has a plane less; a row vector on the right.  Against the oracle, padding and
+    skipped planes untouched."""
+    dims, owner = (7, 1024, 4096), (14, 1024, 4096)
+    dl, hl = pair(dtype, owner, salt=0x771)
+    dr, hr = pair(dtype, (1, 4096), salt=0x772)
+    do, ho = pair(dtype, owner, salt=0x773)
+    if dtype == iomo.DT_F8_E5M2:                      # finite magnitudes below 2: the converted route
+        for t, h, d in ((dl, hl, owner), (dr, hr, (1, 4096))):
+            v = (pattern(dtype, int(np.prod(d)), 0x774 + len(d)) & 0xBF).reshape(d)
+            t.view().from_host(v)
+            h.view().from_logical(v)
+    sl = lambda t: t.view().slice(0, 1, 7, 2)
+    assert iomx.binary(OP_MUL, sl(dl), dr.view(), sl(do)) == 0
+    assert kernel_name() == "rows_binary"
+    launch = iomx.last_launch()
+    assert launch.work_items == 7 * 1024 * 256                  # every tile row of every plane ...
+    assert iomo.binary(OP_MUL, sl(hl), hr.view(), sl(ho), ieee=True) == 0
+    assert same_storage(do, ho)
+    for t in (dl, dr, do):
+        t.free()
+
+
 @pytest.mark.parametrize("dtype", [iomo.DT_I8, iomo.DT_U8], ids=["I8", "U8"])
 @pytest.mark.parametrize("op", [OP_ADD, OP_MUL, OP_SUB])
 def test_binary_every_8bit_pair_on_whole_planes(dtype, op):
