@@ -441,6 +441,90 @@ def wl_vendor_gemm(timer, steps, warmup):
     return rows
 
 
+_VENDOR_STREAM = r"""
+import json, sys, time, torch
+steps = int(sys.argv[1])
+ROT = 6
+def timed(name, kernel, alg_bytes, launch):
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.03:
+        for i in range(ROT):
+            launch(i)
+        torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        launch(i)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    gbs = alg_bytes / (ms * 1e-3) / 1e9
+    print(json.dumps({"workload": name, "kernel": kernel, "algorithmic_bytes": alg_bytes,
+                      "ms_per_launch": round(ms, 5), "GB_per_s": round(gbs, 1),
+                      "hbm_frac": round(gbs / 8000.0, 4)}), flush=True)
+
+# broadcast ADD BF16 [64*512, 2048] + [2048], row-major, out-of-place into preallocated outputs
+M, F = 64 * 512, 2048
+xs = [torch.randn(M, F, device="cuda", dtype=torch.bfloat16) for _ in range(ROT)]
+os_ = [torch.empty(M, F, device="cuda", dtype=torch.bfloat16) for _ in range(ROT)]
+b = torch.randn(F, device="cuda", dtype=torch.bfloat16) * 0.02
+timed("vendor_stream_torch_add_bf16_[32768,2048]+[2048]", "torch.add(out=) elementwise kernel",
+      (2 * M * F + F) * 2, lambda i: torch.add(xs[i % ROT], b, out=os_[i % ROT]))
+# copy of 128 MiB through the same tensors
+timed("vendor_stream_torch_copy_128MiB", "Tensor.copy_ (same dtype, contiguous)",
+      2 * M * F * 2, lambda i: os_[i % ROT].copy_(xs[i % ROT]))
+del xs, os_
+# ADD F32 [4096,4096]
+N = 4096
+a = [torch.rand(N, N, device="cuda") * 2 - 1 for _ in range(ROT)]
+c = [torch.rand(N, N, device="cuda") * 2 - 1 for _ in range(ROT)]
+o = [torch.empty(N, N, device="cuda") for _ in range(ROT)]
+timed("vendor_stream_torch_add_f32_[4096,4096]", "torch.add(out=) elementwise kernel",
+      3 * N * N * 4, lambda i: torch.add(a[i % ROT], c[i % ROT], out=o[i % ROT]))
+"""
+
+
+def wl_vendor_stream(timer, steps, warmup):
+    """Streams this repository did not write, on the same box and sizes as the headline workloads:
+    the elementwise kernels of the importable torch (broadcast ADD BF16 [32768,2048]+[2048],
+    ADD F32 [4096,4096], a 128 MiB Tensor.copy_; row-major tensors, six rotating sets = 1.5-2.3 GiB)
+    in a child process, and the HIP runtime's own device-to-device copy of 128 MiB through
+    iomx_memcpy_d2d_async in this one.  Yardsticks only -- nothing of the product calls them."""
+    import subprocess
+    rows = []
+    nb = 128 << 20
+    sets = [(iomx.Buffer(nb), iomx.Buffer(nb)) for _ in range(ROT)]
+    for a, o in sets:
+        a.fill(0x3C, timer.stream)
+        o.fill(0x00, timer.stream)
+    timer.stream.synchronize()
+
+    def d2d(i):
+        a, o = sets[i % ROT]
+        check(iomx.lib().iomx_memcpy_d2d_async(o.ptr, a.ptr, nb, timer.stream.h), "d2d")
+
+    wall, ev = timer.run(d2d, steps, warmup)
+    rows.append(report("vendor_stream_runtime_d2d_copy_128MiB", 2 * nb, nb // 4, wall, ev,
+                       "hipMemcpyAsync device-to-device (runtime's own copy)"))
+    for a, o in sets:
+        a.free()
+        o.free()
+    if under_profiler():
+        rows.append({"workload": "vendor_stream_torch", "skipped": "child not run under the profiler"})
+        return rows
+    try:
+        p = subprocess.run([sys.executable, "-c", _VENDOR_STREAM, str(steps)], capture_output=True,
+                           text=True, timeout=300)
+    except Exception as exc:   # pragma: no cover
+        rows.append({"workload": "vendor_stream_torch", "skipped": "child failed: %s" % exc})
+        return rows
+    child = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")]
+    if p.returncode != 0 or not child:
+        rows.append({"workload": "vendor_stream_torch",
+                     "skipped": "child exit %d: %s" % (p.returncode, p.stderr[-200:])})
+    return rows + child
+
+
 def wl_sdpa(timer, steps, warmup):
     """BF16 causal grouped-query attention at TinyLlama's head shape (32 query heads, 4 KV
     heads, D = 64): a 512-token prefill of 8 sequences and a decode step of 64 sequences
@@ -626,10 +710,37 @@ def wl_chain(timer, steps, warmup):
     wall, ev = timer.run(launch, steps, warmup)
     nh, nf = B * S * H, B * S * FF
     alg = 2 * (4 * nh + 2 * H) + 2 * (6 * nh) + 4 * nf + 6 * nf
+    public = report("tinyllama_layer_non_gemm_chain_bf16_[64,512]", alg, 4 * nh + 2 * nf, wall, ev,
+                    "6 launches: the public operations")
+
+    # The same chain as BASELINE words it (RMSNorm -> residual ADD -> RMSNorm -> SiLU*up -> residual
+    # ADD) with what may be fused privately fused: add + rmsnorm in one launch (x2 stored once and
+    # normalised from the registers that hold it) and SiLU*up in one launch.  Same bits in n1, x2,
+    # n2, prod and next; act is never stored.  Fewer bytes have to cross HBM, so this row's
+    # algorithmic bytes are its own: 4nh + 8nh + 6nf + 6nh (+ the two weight rows).
+    def launch_private(i):
+        check(iomx.rmsnorm(x.view(), w1.view(), n1.view(), 1e-5, st), "rmsnorm1")
+        check(iomx.add_rmsnorm(x.view(), attn.view(), x2.view(), w2.view(), n2.view(), 1e-5, st), "add_rmsnorm")
+        check(iomx.silu_mul(gate.view(), up.view(), prod.view(), st), "silu_mul")
+        check(iomx.binary(ADD, x2.view(), down.view(), nxt.view(), st), "add2")
+
+    wall, ev = timer.run(launch_private, steps, warmup)
+    alg_private = (4 * nh + 2 * H) + (8 * nh + 2 * H) + 6 * nf + 6 * nh
+    private = report("tinyllama_layer_non_gemm_chain_private_fusions_bf16_[64,512]", alg_private,
+                     4 * nh + 2 * nf, wall, ev,
+                     "4 launches: rmsnorm, add_rmsnorm, silu_mul, add",
+                     {"same_results_as": "the 6-launch public chain (x2, n2, prod, next bit-identical)",
+                      "speedup_over_public_chain": round(public["ms_per_launch"] / (ev if ev else 1), 3)})
+
+    def one(i):
+        check(iomx.add_rmsnorm(x.view(), attn.view(), x2.view(), w2.view(), n2.view(), 1e-5, st), "add_rmsnorm")
+
+    wall, ev = timer.run(one, steps * 4, warmup * 4)
+    fused = report("add_rmsnorm_bf16_[64,512,2048]_private", 8 * nh + 2 * H, nh, wall, ev,
+                   iomx.last_launch().kernel.decode())
     for t in (x, attn, down, gate, up, w1, w2, n1, x2, n2, nxt, act, prod):
         t.free()
-    return report("tinyllama_layer_non_gemm_chain_bf16_[64,512]", alg, 4 * nh + 2 * nf, wall, ev,
-                  "6 launches")
+    return [public, private, fused]
 
 
 def wl_hbm_ceiling(timer, steps, warmup, sizes_mib=(64, 128, 256), modes=None):
@@ -658,7 +769,7 @@ def wl_hbm_ceiling(timer, steps, warmup, sizes_mib=(64, 128, 256), modes=None):
 
             wall, ev = timer.run(launch, steps, warmup)
             rows.append(report(f"hbm_probe_{name}_{mib}MiB_per_operand", mult * nb, nb // 4, wall, ev,
-                               iomx.last_launch().kernel.decode()))
+                               iomx.PROBE_KERNEL[mode]))
         for bufs in sets:
             for t in bufs:
                 t.free()
@@ -883,6 +994,7 @@ def main():
         "layer_ops": lambda: wl_layer_ops(timer, max(K // 4, 5), max(W // 4, 2)),
         "linear": lambda: wl_linear(timer, max(K // 5, 10), max(W // 2, 5)),
         "vendor_gemm": lambda: wl_vendor_gemm(timer, max(K // 5, 10), max(W // 2, 5)),
+        "vendor_stream": lambda: wl_vendor_stream(timer, K, W),
         "sdpa": lambda: wl_sdpa(timer, max(K // 5, 10), max(W // 2, 5)),
         "decoder_layer": lambda: wl_decoder_layer(timer, max(K // 5, 10), max(W // 2, 5)),
         "other_leaves": lambda: wl_other_leaves(timer, max(K // 10, 5), max(W // 10, 2)),
@@ -905,7 +1017,12 @@ def main():
     # the bare copy of the headline's size, in the same run: what a stream of 128 MiB in and
     # 128 MiB out reaches on this box with nothing else in the kernel
     ceiling = wl_hbm_ceiling(timer, K, W, sizes_mib=(128,), modes=("copy",))[0]
-    detail = []
+    # streams this repository did not write, same box, same sizes: the runtime's device-to-device
+    # copy and the elementwise kernels of the importable torch
+    vendor = wl_vendor_stream(timer, K, W)
+    vendor_rates = [r["GB_per_s"] for r in vendor if "GB_per_s" in r]
+    vendor_best = max(vendor, key=lambda r: r.get("GB_per_s", 0.0)) if vendor_rates else None
+    detail = list(vendor)
     if not args.no_detail:
         for key in ("bcast_mul_bf16", "bcast_div_bf16", "div_f32", "bcast_add_bf16_sliced", "bcast_add_bf16_permuted", "copy_bf16", "add_f32",
                     "add_i32", "rmsnorm_bf16", "rmsnorm_f32", "silu_mul", "softmax", "softmax_causal",
@@ -938,6 +1055,13 @@ def main():
                      "practical_peak_what": "bare copy probe (iomx_probe_stream), 128 MiB in + 128 MiB "
                                             "out, measured in this run",
                      "frac_of_practical_peak": round(head["GB_per_s"] / ceiling["GB_per_s"], 4),
+                     "vendor_peak": vendor_best["GB_per_s"] if vendor_best else None,
+                     "vendor_peak_what": ("best of the vendor streams timed in this run (runtime "
+                                          "device-to-device copy of 128 MiB; torch.add BF16 "
+                                          "[32768,2048]+[2048]; torch.add F32 [4096,4096]; "
+                                          "Tensor.copy_ of 128 MiB): " + vendor_best["workload"])
+                     if vendor_best else "vendor streams not measured",
+                     "frac_of_best_peak": round(head["GB_per_s"] / max([ceiling["GB_per_s"]] + vendor_rates), 4),
                      "kernel": "elementwise_stream_kernel<BF16,ADD,FULL,ROWVEC,BANDS>",
                      "ms_per_launch": head["ms_per_launch"]},
         "cpu_baseline": cpu,

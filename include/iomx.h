@@ -209,6 +209,20 @@ int iomx_launch_silu_mul(int dtype, const iomx_view* gate, const iomx_view* up,
                          const iomx_view* y, iomx_stream_t stream);
 
 /*
+ * sum = x + y and out = rmsnorm(sum, scale, eps) in one launch: the residual add and
+ * the norm that follows it in a decoder layer (src/session.cpp:2500 then :1996).  A
+ * private fast path with no counterpart operation in the reference: both outputs equal,
+ * bit for bit, iomx_launch_binary(ADD) followed by iomx_launch_rmsnorm on its result,
+ * while the sum crosses HBM once instead of three times.  BF16, F16 and F32; all four
+ * tensors of one shape whose two matrix extents are multiples of 16; `sum` may be the
+ * identical window of x or y, `out` shares storage with none of the others.  Any other
+ * request is IOMX_ERR_UNSUPPORTED (make the two launches) or IOMX_ERR_INVALID.
+ */
+int iomx_launch_add_rmsnorm(int dtype, const iomx_view* x, const iomx_view* y,
+                            const iomx_view* sum, const iomx_view* scale,
+                            const iomx_view* out, float eps, iomx_stream_t stream);
+
+/*
  * Same-spec copy of the selected planes' logical elements, any leaf.  Replaces
  * grid_stride_copy_kernel (src/shared/standard_tiled_copy_metadata.inl:241-282)
  * behind DeviceOps::copy_impl (src/device_ops_copy.cpp:9-52).
@@ -389,33 +403,6 @@ typedef struct iomx_launch_info {
     uint64_t work_items;
 } iomx_launch_info;
 int iomx_last_launch(iomx_launch_info* info);
-
-/*
- * Bandwidth probes (no counterpart in the reference): one launch of a bare stream over
- * `bytes` bytes per operand (a multiple of 4096, operands 16-byte aligned), in the launch
- * shape of the elementwise kernels -- one 128-bit chunk per lane, one-shot grid,
- * nontemporal access -- and with nothing else in the kernel.  They measure what this GPU
- * gives a read-only stream (a), a write-only stream (out), a copy (a -> out) and a
- * two-read-one-write stream (a + b -> out, 32-bit integer adds), which is the practical
- * ceiling the operation kernels are compared with.  READ needs `out` only as a pointer to
- * 4 KiB of writable memory that it never writes.  HELD_COPY is the memory side of the
- * resident RMSNorm kernel alone (a -> out; bytes a multiple of 64 KiB): 1024-lane workgroups
- * that load four chunks per lane, meet at a barrier and store.
- */
-enum { IOMX_PROBE_READ = 0, IOMX_PROBE_WRITE = 1, IOMX_PROBE_COPY = 2, IOMX_PROBE_ADD = 3,
-       IOMX_PROBE_HELD_COPY = 4 };
-int iomx_probe_stream(int mode, const void* a, const void* b, void* out, uint64_t bytes,
-                      iomx_stream_t stream);
-
-/* Compares the hardware BF16 conversion with the software round-to-nearest-
- * even rule over all 2^32 binary32 encodings; *mismatches receives the count. */
-int iomx_selftest_bf16_convert(uint64_t* mismatches, iomx_stream_t stream);
-
-/* Compares the packed F16 arithmetic of the streaming kernels (hardware F16 <->
- * binary32 conversions around one binary32 operation) with the integer-rounded
- * binary64 rule for all 2^32 operand pairs and ADD, MUL, SUB, DIV; *mismatches receives
- * the count. */
-int iomx_selftest_f16_binary(uint64_t* mismatches, iomx_stream_t stream);
 
 #ifdef __cplusplus
 }

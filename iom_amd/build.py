@@ -1,4 +1,5 @@
-"""Compiles libiomx.so (HIP kernels + C ABI) for gfx950, in-tree.
+"""Compiles libiomx.so (HIP kernels + C ABI) and libiomx_probe.so (bandwidth probes and device
+self-tests for the benchmark and the tests) for gfx950, in-tree.
 
     python -m iom_amd.build
 
@@ -17,6 +18,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libiomx.so")
+PROBE_LIB = os.path.join(LIBDIR, "libiomx_probe.so")
 
 SOURCES = [
     "iomx_runtime.hip",
@@ -28,8 +30,10 @@ SOURCES = [
     "iomx_layer.hip",
     "iomx_linear.hip",
     "iomx_sdpa.hip",
-    "iomx_probe.hip",
 ]
+# measurement and self-tests: a library of its own, so that libiomx.so exports operations and
+# runtime only
+PROBE_SOURCES = ["iomx_probe.hip"]
 
 # -ffp-contract=off: no fused multiply-add may replace the reference's two
 # roundings.  Packed FP32 instructions are disabled for the device pass.
@@ -51,7 +55,7 @@ def build_iomx(verbose: bool = True) -> str:
     os.makedirs(LIBDIR, exist_ok=True)
     objs = []
     procs = []
-    for src in SOURCES:
+    for src in SOURCES + PROBE_SOURCES:
         obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
         cmd = [hipcc(), *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
                "-c", os.path.join(CSRC, src), "-o", obj]
@@ -65,7 +69,12 @@ def build_iomx(verbose: bool = True) -> str:
             raise RuntimeError(f"hipcc failed on {src}:\n{text}")
         if verbose and text:
             print(text)
+    probe_objs = objs[len(SOURCES):]
+    objs = objs[:len(SOURCES)]
     subprocess.check_call([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
+    subprocess.check_call([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB,
+                           *probe_objs])
+    objs += probe_objs
     for obj in objs:
         os.remove(obj)
     if verbose:

@@ -1,7 +1,15 @@
+// Measurement and self-test code, built into a library of its own (libiomx_probe.so) that only
+// the benchmark and the tests load: nothing here is an operation or part of the runtime.
+//
 // Bandwidth probes: the bare streams that the operation kernels are judged against.
 // One 128-bit chunk per lane, one-shot grid, nontemporal access -- the launch shape of
 // elementwise_stream_kernel without any of its address arithmetic or operations.
-#include "iomx_common.hpp"
+//
+// Device self-tests: the hardware conversions and the packed arithmetic of the streaming kernels
+// (iomx_common.hpp, iomx_arith.hpp -- the very inline functions the kernels use) against the
+// software rules, over every encoding.
+#include "iomx_arith.hpp"
+#include "iomx_probe.h"
 
 namespace iomx {
 
@@ -45,9 +53,84 @@ __global__ __launch_bounds__(1024) void probe_held_copy_kernel(const u32x4* __re
     for (int k = 0; k < 4; ++k) __builtin_nontemporal_store(held[k], out + base + k * 1024);
 }
 
+// Self test: the packed F16 arithmetic of the streaming kernels (hardware
+// conversions around one binary32 operation) against the integer-rounded binary64
+// rule of the tile-row kernels, for every pair of binary16 encodings and the four
+// operations.
+__global__ __launch_bounds__(256) void f16_binary_selftest_kernel(unsigned long long* mismatches) {
+    unsigned long long bad = 0;
+    for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < (1ull << 31); i += (uint64_t)gridDim.x * 256) {
+        const uint64_t p0 = 2 * i, p1 = 2 * i + 1;   // pair index = a * 65536 + b
+        const uint32_t a0 = (uint32_t)(p0 >> 16), b0 = (uint32_t)(p0 & 0xFFFFu);
+        const uint32_t a1 = (uint32_t)(p1 >> 16), b1 = (uint32_t)(p1 & 0xFFFFu);
+        const uint32_t wa = a0 | (a1 << 16), wb = b0 | (b1 << 16);
+        const uint32_t add = op_word<IOMX_DT_F16, IOMX_OP_ADD>(wa, wb);
+        const uint32_t mul = op_word<IOMX_DT_F16, IOMX_OP_MUL>(wa, wb);
+        const uint32_t sub = op_word<IOMX_DT_F16, IOMX_OP_SUB>(wa, wb);
+        const uint32_t div = op_word<IOMX_DT_F16, IOMX_OP_DIV>(wa, wb);
+        bad += (add & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_ADD>(a0, b0);
+        bad += (add >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_ADD>(a1, b1);
+        bad += (mul & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_MUL>(a0, b0);
+        bad += (mul >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_MUL>(a1, b1);
+        bad += (sub & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_SUB>(a0, b0);
+        bad += (sub >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_SUB>(a1, b1);
+        bad += (div & 0xFFFFu) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_DIV>(a0, b0);
+        bad += (div >> 16) != (uint32_t)leaf_binary<DT_F16, IOMX_OP_DIV>(a1, b1);
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
+// All 2^32 binary32 encodings through the hardware BF16 conversion against the software
+// round-to-nearest-even rule.
+__global__ __launch_bounds__(256) void bf16_convert_selftest_kernel(unsigned long long* mismatches) {
+    unsigned long long bad = 0;
+    // 2^32 encodings, two per step so the packed conversion sees both halves
+    for (uint64_t i = (blockIdx.x * 256ull + threadIdx.x) * 2; i < (1ull << 32);
+         i += (uint64_t)gridDim.x * 256 * 2) {
+        const uint32_t b0 = (uint32_t)i, b1 = (uint32_t)i + 1u;
+        const uint32_t packed = pack_bf16(as_f32(b0), as_f32(b1));
+        bad += (packed & 0xFFFFu) != bf16_rne_sw(b0);
+        bad += (packed >> 16) != bf16_rne_sw(b1);
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
+namespace {
+
+int count_mismatches(void (*kernel)(unsigned long long*), uint32_t grid, uint64_t* mismatches,
+                     iomx_stream_t stream) {
+    if (!mismatches) return IOMX_ERR_INVALID;
+    unsigned long long* counter = nullptr;
+    IOMX_HIP(hipMalloc(reinterpret_cast<void**>(&counter), sizeof(*counter)));
+    const hipStream_t s = native(stream);
+    int rc = IOMX_OK;
+    hipError_t e = hipMemsetAsync(counter, 0, sizeof(*counter), s);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), 0, s, counter);
+        e = hipGetLastError();
+    }
+    unsigned long long host = 0;
+    if (e == hipSuccess) e = hipMemcpyAsync(&host, counter, sizeof(host), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) rc = (int)e;
+    (void)hipFree(counter);
+    *mismatches = host;
+    return rc;
+}
+
+}  // namespace
+
 }  // namespace iomx
 
 using namespace iomx;
+
+extern "C" int iomx_selftest_f16_binary(uint64_t* mismatches, iomx_stream_t stream) {
+    return count_mismatches(f16_binary_selftest_kernel, 8192, mismatches, stream);
+}
+
+extern "C" int iomx_selftest_bf16_convert(uint64_t* mismatches, iomx_stream_t stream) {
+    return count_mismatches(bf16_convert_selftest_kernel, 4096, mismatches, stream);
+}
 
 extern "C" int iomx_probe_stream(int mode, const void* a, const void* b, void* out, uint64_t bytes,
                                  iomx_stream_t stream) {
@@ -64,26 +147,21 @@ extern "C" int iomx_probe_stream(int mode, const void* a, const void* b, void* o
         case IOMX_PROBE_READ:
             if (!a) return IOMX_ERR_INVALID;
             hipLaunchKernelGGL(probe_read_kernel, dim3((uint32_t)(chunks / 256)), dim3(256), 0, s, pa, po);
-            record_launch("probe_read", (uint32_t)(chunks / 256), 256, chunks);
             break;
         case IOMX_PROBE_WRITE:
             hipLaunchKernelGGL(probe_write_kernel, dim3((uint32_t)(chunks / 256)), dim3(256), 0, s, po);
-            record_launch("probe_write", (uint32_t)(chunks / 256), 256, chunks);
             break;
         case IOMX_PROBE_COPY:
             if (!a) return IOMX_ERR_INVALID;
             hipLaunchKernelGGL(probe_copy_kernel, dim3((uint32_t)(chunks / 64)), dim3(64), 0, s, pa, po);
-            record_launch("probe_copy", (uint32_t)(chunks / 64), 64, chunks);
             break;
         case IOMX_PROBE_ADD:
             if (!a || !b) return IOMX_ERR_INVALID;
             hipLaunchKernelGGL(probe_add_kernel, dim3((uint32_t)(chunks / 64)), dim3(64), 0, s, pa, pb, po);
-            record_launch("probe_add", (uint32_t)(chunks / 64), 64, chunks);
             break;
         case IOMX_PROBE_HELD_COPY:
             if (!a || bytes % 65536 != 0) return IOMX_ERR_INVALID;
             hipLaunchKernelGGL(probe_held_copy_kernel, dim3((uint32_t)(chunks / 4096)), dim3(1024), 0, s, pa, po);
-            record_launch("probe_held_copy", (uint32_t)(chunks / 4096), 1024, chunks);
             break;
         default:
             return IOMX_ERR_INVALID;

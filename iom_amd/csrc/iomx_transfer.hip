@@ -54,19 +54,6 @@ __global__ __launch_bounds__(256) void transfer_kernel(const TransferArgs a) {
     }
 }
 
-__global__ __launch_bounds__(256) void bf16_convert_selftest_kernel(unsigned long long* mismatches) {
-    unsigned long long bad = 0;
-    // 2^32 encodings, two per step so the packed conversion sees both halves
-    for (uint64_t i = (blockIdx.x * 256ull + threadIdx.x) * 2; i < (1ull << 32);
-         i += (uint64_t)gridDim.x * 256 * 2) {
-        const uint32_t b0 = (uint32_t)i, b1 = (uint32_t)i + 1u;
-        const uint32_t packed = pack_bf16(as_f32(b0), as_f32(b1));
-        bad += (packed & 0xFFFFu) != bf16_rne_sw(b0);
-        bad += (packed >> 16) != bf16_rne_sw(b1);
-    }
-    if (bad) atomicAdd(mismatches, bad);
-}
-
 namespace {
 
 int run_transfer(int dtype, const iomx_view* view, const void* logical, bool scatter,
@@ -128,26 +115,6 @@ int iomx_launch_scatter(int dtype, const iomx_view* dst, const void* logical, io
 
 int iomx_launch_gather(int dtype, const iomx_view* src, void* logical, iomx_stream_t stream) {
     return run_transfer(dtype, src, logical, false, stream);
-}
-
-int iomx_selftest_bf16_convert(uint64_t* mismatches, iomx_stream_t stream) {
-    if (!mismatches) return IOMX_ERR_INVALID;
-    unsigned long long* counter = nullptr;
-    IOMX_HIP(hipMalloc(reinterpret_cast<void**>(&counter), sizeof(*counter)));
-    const hipStream_t s = native(stream);
-    int rc = IOMX_OK;
-    hipError_t e = hipMemsetAsync(counter, 0, sizeof(*counter), s);
-    if (e == hipSuccess) {
-        hipLaunchKernelGGL(bf16_convert_selftest_kernel, dim3(4096), dim3(256), 0, s, counter);
-        e = hipGetLastError();
-    }
-    unsigned long long host = 0;
-    if (e == hipSuccess) e = hipMemcpyAsync(&host, counter, sizeof(host), hipMemcpyDeviceToHost, s);
-    if (e == hipSuccess) e = hipStreamSynchronize(s);
-    if (e != hipSuccess) rc = (int)e;
-    (void)hipFree(counter);
-    *mismatches = host;
-    return rc;
 }
 
 }  // extern "C"

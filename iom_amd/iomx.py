@@ -11,6 +11,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libiomx.so")
+PROBE_LIB_PATH = os.path.join(HERE, "lib", "libiomx_probe.so")
 
 # numeric values of iom::DataType (include/iom/tensor.hpp:10-33)
 (DT_BOOL, DT_I2, DT_U2, DT_I4, DT_U4, DT_I8, DT_U8, DT_I16, DT_U16, DT_I32, DT_U32, DT_I64,
@@ -18,6 +19,8 @@ LIB_PATH = os.path.join(HERE, "lib", "libiomx.so")
  DT_BF16, DT_F32, DT_F64) = range(23)
 LEAF_BITS = (8, 2, 2, 4, 4, 8, 8, 16, 16, 32, 32, 64, 64, 4, 6, 6, 8, 8, 8, 16, 16, 32, 64)
 OP_ADD, OP_MUL, OP_SUB, OP_DIV = 0, 1, 2, 3
+# status codes of include/iomx.h (positive values are HIP error codes)
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_OVERFLOW, ERR_EXHAUSTED = 0, -1, -2, -3, -4
 TILE = 16
 
 
@@ -60,10 +63,14 @@ SYMBOLS = [
     "iomx_stream_begin_capture", "iomx_stream_end_capture", "iomx_graph_launch", "iomx_graph_destroy",
     "iomx_launch_linear", "iomx_sdpa_workspace", "iomx_launch_sdpa", "iomx_launch_sdpa_static",
     "iomx_launch_cache_append", "iomx_launch_embedding", "iomx_launch_rope",
-    "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul",
+    "iomx_launch_binary", "iomx_launch_rmsnorm", "iomx_launch_silu", "iomx_launch_silu_mul", "iomx_launch_add_rmsnorm",
     "iomx_launch_copy", "iomx_launch_scatter", "iomx_launch_gather", "iomx_launch_softmax",
-    "iomx_last_launch", "iomx_selftest_bf16_convert", "iomx_selftest_f16_binary", "iomx_probe_stream",
+    "iomx_last_launch",
 ]
+
+# every symbol include/iomx_probe.h declares (libiomx_probe.so: measurement and self-tests,
+# loaded by the benchmark and the tests only)
+PROBE_SYMBOLS = ["iomx_probe_stream", "iomx_selftest_bf16_convert", "iomx_selftest_f16_binary"]
 
 
 class View(C.Structure):
@@ -152,6 +159,7 @@ def lib() -> C.CDLL:
         l.iomx_graph_destroy.argtypes = [P]
         l.iomx_launch_silu.argtypes = [C.c_int, VP, VP, P]
         l.iomx_launch_silu_mul.argtypes = [C.c_int, VP, VP, VP, P]
+        l.iomx_launch_add_rmsnorm.argtypes = [C.c_int, VP, VP, VP, VP, VP, C.c_float, P]
         l.iomx_launch_copy.argtypes = [C.c_int, VP, VP, P]
         l.iomx_launch_cache_append.argtypes = [C.c_int, VP, VP, C.c_uint64, P]
         l.iomx_launch_linear.argtypes = [C.c_int, VP, VP, VP, C.c_uint64, C.c_uint64, C.c_int, C.c_uint64,
@@ -168,9 +176,6 @@ def lib() -> C.CDLL:
         l.iomx_launch_gather.argtypes = [C.c_int, VP, P, P]
         l.iomx_launch_softmax.argtypes = [C.POINTER(SoftmaxDesc), P]
         l.iomx_last_launch.argtypes = [C.POINTER(LaunchInfo)]
-        l.iomx_selftest_bf16_convert.argtypes = [C.POINTER(C.c_uint64), P]
-        l.iomx_selftest_f16_binary.argtypes = [C.POINTER(C.c_uint64), P]
-        l.iomx_probe_stream.argtypes = [C.c_int, P, P, P, C.c_uint64, P]
         _lib = l
     return _lib
 
@@ -487,6 +492,14 @@ def rmsnorm(x: DeviceView, scale: DeviceView, out: DeviceView, eps: float, strea
     return lib().iomx_launch_rmsnorm(out.dtype, C.byref(a), C.byref(b), C.byref(o), eps, _h(stream))
 
 
+def add_rmsnorm(x: DeviceView, y: DeviceView, total: DeviceView, scale: DeviceView, out: DeviceView,
+                eps: float, stream=None) -> int:
+    """total = x + y, out = rmsnorm(total, scale): the private fusion of ADD and RMSNorm."""
+    a, b, t, w, o = x.cview(), y.cview(), total.cview(), scale.cview(), out.cview()
+    return lib().iomx_launch_add_rmsnorm(out.dtype, C.byref(a), C.byref(b), C.byref(t), C.byref(w), C.byref(o),
+                                         eps, _h(stream))
+
+
 def silu(x: DeviceView, y: DeviceView, stream=None) -> int:
     a, o = x.cview(), y.cview()
     return lib().iomx_launch_silu(y.dtype, C.byref(a), C.byref(o), _h(stream))
@@ -527,13 +540,32 @@ def sdpa(q: DeviceView, k: DeviceView, v: DeviceView, out: DeviceView, a: int, L
 
 
 PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_ADD, PROBE_HELD_COPY = range(5)
+PROBE_KERNEL = ("probe_read", "probe_write", "probe_copy", "probe_add", "probe_held_copy")
+
+_probe_lib: Optional[C.CDLL] = None
+
+
+def probe_lib() -> C.CDLL:
+    """The measurement and self-test library (include/iomx_probe.h).  Raises when not built."""
+    global _probe_lib
+    if _probe_lib is None:
+        lib()   # the backend library first: both must see one HIP runtime state
+        if not os.path.exists(PROBE_LIB_PATH):
+            raise ImportError(f"{PROBE_LIB_PATH} is missing: build it with `python -m iom_amd.build`")
+        l = C.CDLL(PROBE_LIB_PATH)
+        P = C.c_void_p
+        l.iomx_selftest_bf16_convert.argtypes = [C.POINTER(C.c_uint64), P]
+        l.iomx_selftest_f16_binary.argtypes = [C.POINTER(C.c_uint64), P]
+        l.iomx_probe_stream.argtypes = [C.c_int, P, P, P, C.c_uint64, P]
+        _probe_lib = l
+    return _probe_lib
 
 
 def probe_stream(mode: int, a: Optional["Buffer"], b: Optional["Buffer"], out: "Buffer", nbytes: int,
                  stream: Optional[Stream] = None) -> int:
     """One launch of a bare bandwidth probe over `nbytes` bytes per operand."""
-    return lib().iomx_probe_stream(mode, a.ptr if a is not None else None,
-                                   b.ptr if b is not None else None, out.ptr, nbytes, _h(stream))
+    return probe_lib().iomx_probe_stream(mode, a.ptr if a is not None else None,
+                                         b.ptr if b is not None else None, out.ptr, nbytes, _h(stream))
 
 
 SDPA_STATIC_BYTES = 16 << 20

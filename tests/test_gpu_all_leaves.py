@@ -273,7 +273,7 @@ def test_binary_16bit_pairs_on_whole_planes(dtype, op):
 def test_f16_streaming_arithmetic_equals_the_codec_rule_for_every_pair():
     import ctypes as C
     bad = C.c_uint64(123)
-    iomx.check(iomx.lib().iomx_selftest_f16_binary(C.byref(bad), None))
+    iomx.check(iomx.probe_lib().iomx_selftest_f16_binary(C.byref(bad), None))
     assert bad.value == 0
 
 

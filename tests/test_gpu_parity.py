@@ -77,7 +77,7 @@ def kernel_name():
 
 def test_hardware_bf16_conversion_is_rne_for_every_binary32_encoding():
     bad = C.c_uint64(123)
-    iomx.check(iomx.lib().iomx_selftest_bf16_convert(C.byref(bad), None))
+    iomx.check(iomx.probe_lib().iomx_selftest_bf16_convert(C.byref(bad), None))
     assert bad.value == 0
 
 

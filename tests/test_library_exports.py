@@ -21,6 +21,20 @@ def test_libiomx_exports_every_symbol_of_the_header():
     assert lib.iomx_error_string(-1).decode().startswith("iomx")
 
 
+def test_probe_library_exports_every_symbol_of_its_header_and_the_backend_none_of_them():
+    """Measurement and self-test code lives in libiomx_probe.so; libiomx.so holds operations and
+    runtime only."""
+    from iom_amd import iomx
+    header = open(os.path.join(ROOT, "include", "iomx_probe.h")).read()
+    declared = set(re.findall(r"\b(iomx_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(iomx.PROBE_SYMBOLS), declared ^ set(iomx.PROBE_SYMBOLS)
+    probe = iomx.probe_lib()
+    for name in sorted(declared):
+        assert hasattr(probe, name), name
+    exported = subprocess.check_output(["nm", "-D", "--defined-only", iomx.LIB_PATH]).decode()
+    assert "probe" not in exported and "selftest" not in exported
+
+
 def test_status_queries_do_not_need_a_gpu():
     from iom_amd import iomx
     assert iomx.device_count() >= 0
