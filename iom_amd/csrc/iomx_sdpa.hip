@@ -1413,12 +1413,20 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::atomic<void*> g_scratch_address[kMaxDevices];
 
-int scratch_of_current_device(void** address) {
+// The first call on a device looks the address up, and a symbol lookup is not a call to make
+// under stream capture: there the request is refused (make one eager call first, or any call on
+// another stream), so that a captured call is launches only.
+int scratch_of_current_device(hipStream_t stream, void** address) {
     int device = -1;
     IOMX_HIP(hipGetDevice(&device));
     if (device < 0 || device >= kMaxDevices) return IOMX_ERR_UNSUPPORTED;
     void* known = g_scratch_address[device].load(std::memory_order_acquire);
     if (known == nullptr) {
+        if (stream != nullptr) {
+            hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+            IOMX_HIP(hipStreamIsCapturing(stream, &capture));
+            if (capture != hipStreamCaptureStatusNone) return IOMX_ERR_INVALID;
+        }
         IOMX_HIP(hipGetSymbolAddress(&known, HIP_SYMBOL(scratch)));
         if (known == nullptr || (reinterpret_cast<uintptr_t>(known) & 255u) != 0) return IOMX_ERR_INVALID;
         g_scratch_address[device].store(known, std::memory_order_release);
@@ -1436,7 +1444,7 @@ extern "C" int iomx_launch_sdpa_static(int dtype, const iomx_view* q, const iomx
     if (path != 0) need = 0;  // the reference-order kernel keeps nothing outside its operands
     if (need > IOMX_SDPA_STATIC_BYTES) return IOMX_ERR_EXHAUSTED;
     void* address = nullptr;
-    IOMX_TRY(scratch_of_current_device(&address));
+    IOMX_TRY(scratch_of_current_device(native(stream), &address));
     // Every word of the part in use is written by the pack kernel (or by the first two
     // decode phases) before it is read in the same call, so what an earlier call left
     // in the array needs no clearing.

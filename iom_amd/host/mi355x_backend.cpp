@@ -606,7 +606,11 @@ public:
 
 private:
     // What completion does with the operation's registry entries and workspace lease.
-    using Finish = InlineFunction<void(bool failed), 160>;
+    // failed: the operation's terminal state is a failure.  proved: the device has provably
+    // finished with the operands (the completion event or word was seen, or the stream was
+    // synchronised after a failed submission); without proof owners and workspace ranges are
+    // quarantined instead of released (src/shared/gpu_queue_operations.inl:1031-1046).
+    using Finish = InlineFunction<void(bool failed, bool proved), 160>;
 
     // After native completion: turns a data error the kernel reported into the
     // operation's retained failure (null = none).
@@ -621,6 +625,7 @@ private:
         std::exception_ptr failure;
         Finish finish;
         Verify verify = nullptr;
+        bool deny_proof = false;            // test seam: the proving synchronisation fails too
     };
 
     static detail::FenceResult fence_pending(const detail::Fence&) noexcept {
@@ -700,7 +705,10 @@ private:
         }
         if (status == IOMX_OK) {
             if (consume_submission_fault(SubmissionFault::event_record)) status = kInjectedDeviceError;
-            else if (item.word != nullptr)
+            else if (consume_submission_fault(SubmissionFault::event_record_unproved)) {
+                status = kInjectedDeviceError;
+                item.deny_proof = true;
+            } else if (item.word != nullptr)
                 status = iomx_stream_write_word(stream_, cells_on_device_ + (item.word - status_cells_), item.ticket);
             else status = iomx_event_record(event, stream_);
         }
@@ -786,26 +794,33 @@ private:
         for (;;) {
             InFlight item;
             if (!next_in_flight(item)) return;
+            bool proved = true;
             if (!item.failure) {
                 const int status = item.word != nullptr ? await_word(item.word, item.ticket)
                                                         : await_event(item.event);
                 if (status != IOMX_OK) {
                     try { throw_status(status, "MI355X kernel completion"); }
                     catch (...) { item.failure = std::current_exception(); }
+                    // the wait itself failed: only a synchronisation of the stream can still
+                    // show that the kernel is done with its operands
+                    proved = iomx_stream_synchronize(stream_) == IOMX_OK;
                 } else if (item.verify != nullptr) {
                     // a native failure takes precedence over the status word
                     item.failure = item.verify(*item.status);
                 }
             } else {
-                // the stream may still hold earlier work: keep completion in order
-                (void)iomx_stream_synchronize(stream_);
+                // The submission failed after its launch (or with earlier work still on the
+                // stream): nothing signals its end, so the stream is synchronised -- which also
+                // keeps completion in order -- and only a successful synchronisation proves that
+                // the operands are free.
+                proved = !item.deny_proof && iomx_stream_synchronize(stream_) == IOMX_OK;
             }
             {
                 std::lock_guard<std::mutex> lock(mutex_);
                 free_events_.push_back(item.event);
                 completing_ = false;
             }
-            try { if (item.finish) item.finish(static_cast<bool>(item.failure)); } catch (...) {}
+            try { if (item.finish) item.finish(static_cast<bool>(item.failure), proved); } catch (...) {}
             try { complete(item.sequence, std::move(item.failure)); } catch (...) {}
         }
     }
@@ -873,11 +888,11 @@ private:
                                           captured.destination.plane_strides);
                                   return iomx_launch_copy(code, &src, &dst, stream);
                               },
-                              [&registry, entries](bool failed) {
+                              [&registry, entries](bool failed, bool proved) {
                                   const detail::SequenceOutcome outcome{
                                           entries.source, entries.destination, nullptr, true};
                                   (void)detail::release_or_invalidate_entries(
-                                          registry, outcome, failed, true);
+                                          registry, outcome, failed, proved);
                               });
                     } catch (...) {
                         registry.remove_entry_if_present(
@@ -915,10 +930,10 @@ private:
                                   const iomx_view out = view_of(captured.out);
                                   return iomx_launch_binary(op, code, &lhs, &rhs, &out, stream);
                               },
-                              [&state, entries, lease](bool failed) {
+                              [&state, entries, lease](bool failed, bool proved) {
                                   (void)detail::release_or_invalidate_binary_entries(
-                                          state.registry, entries, failed, true);
-                                  detail::complete_workspace_lease(state, lease, true);
+                                          state.registry, entries, failed, proved);
+                                  detail::complete_workspace_lease(state, lease, proved);
                               });
                     } catch (...) {
                         state.registry.remove_entries(std::span<const detail::EntryId>(
@@ -955,9 +970,9 @@ private:
                                   return iomx_launch_rmsnorm(code, &x, &scale, &out,
                                                              captured.epsilon, stream);
                               },
-                              [&registry, entries](bool failed) {
+                              [&registry, entries](bool failed, bool proved) {
                                   (void)detail::release_or_invalidate_binary_entries(
-                                          registry, entries, failed, true);
+                                          registry, entries, failed, proved);
                               });
                     } catch (...) {
                         registry.remove_entries(std::span<const detail::EntryId>(
@@ -1012,10 +1027,10 @@ private:
                                   }
                                   return status;
                               },
-                              [&state, entries, lease](bool failed) {
+                              [&state, entries, lease](bool failed, bool proved) {
                                   (void)detail::release_or_invalidate_binary_entries(
-                                          state.registry, entries, failed, true);
-                                  detail::complete_workspace_lease(state, lease, true);
+                                          state.registry, entries, failed, proved);
+                                  detail::complete_workspace_lease(state, lease, proved);
                               });
                     } catch (...) {
                         state.registry.remove_entries(std::span<const detail::EntryId>(
@@ -1069,9 +1084,9 @@ private:
                                   return iomx_launch_sdpa(IOMX_DT_BF16, &q, &k, &v, &out, captured.a,
                                                           captured.L, scratch, scratch_bytes, 0, stream);
                               },
-                              [this, &state, entries, lease, sequence](bool failed) {
+                              [this, &state, entries, lease, sequence](bool failed, bool proved) {
                                   (void)detail::release_or_invalidate_sdpa_entries(
-                                          state.registry, entries, failed, true);
+                                          state.registry, entries, failed, proved);
                                   // Successful attention keeps its workspace range leased until
                                   // the caller observes the token (wait -> fence_through_sequence):
                                   // a second submission on the same range is then refused as
@@ -1079,7 +1094,7 @@ private:
                                   // (src/shared/gpu_queue_operations.inl:1113-1147).  A failed
                                   // one, or one that leased nothing, releases at once.
                                   if (failed || lease.entry_id == 0 || !keep_until_observed(sequence, lease))
-                                      detail::complete_workspace_lease(state, lease, true);
+                                      detail::complete_workspace_lease(state, lease, proved);
                               });
                     } catch (...) {
                         state.registry.remove_entries(std::span<const detail::EntryId>(
@@ -1121,10 +1136,10 @@ private:
                                   return iomx_launch_cache_append(code, &source, &destination,
                                                                   captured.a, stream);
                               },
-                              [&state, entries, lease](bool failed) {
+                              [&state, entries, lease](bool failed, bool proved) {
                                   (void)detail::release_or_invalidate_binary_entries(
-                                          state.registry, entries, failed, true);
-                                  detail::complete_workspace_lease(state, lease, true);
+                                          state.registry, entries, failed, proved);
+                                  detail::complete_workspace_lease(state, lease, proved);
                               });
                     } catch (...) {
                         state.registry.remove_entries(std::span<const detail::EntryId>(
@@ -1157,9 +1172,9 @@ private:
                                   return iomx_launch_rope(code, &x, &out, captured.a, captured.theta,
                                                           stream);
                               },
-                              [&registry, entries](bool failed) {
+                              [&registry, entries](bool failed, bool proved) {
                                   (void)detail::release_or_invalidate_binary_entries(
-                                          registry, entries, failed, true);
+                                          registry, entries, failed, proved);
                               });
                     } catch (...) {
                         registry.remove_entries(std::span<const detail::EntryId>(
@@ -1213,10 +1228,10 @@ private:
                                               : iomx_memcpy_d2h_async(cell, control, sizeof(*cell), stream);
                                   return status;
                               },
-                              [&state, entries, lease](bool failed) {
+                              [&state, entries, lease](bool failed, bool proved) {
                                   (void)detail::release_or_invalidate_binary_entries(
-                                          state.registry, entries, failed, true);
-                                  detail::complete_workspace_lease(state, lease, true);
+                                          state.registry, entries, failed, proved);
+                                  detail::complete_workspace_lease(state, lease, proved);
                               },
                               [](std::uint32_t status) -> std::exception_ptr {
                                   if (status == 0) return nullptr;
@@ -1261,9 +1276,9 @@ private:
                                   rocm_detail::silu_launch_count_for_testing.fetch_add(1);
                                   return iomx_launch_silu(code, &x, &y, stream);
                               },
-                              [&registry, entries](bool failed) {
+                              [&registry, entries](bool failed, bool proved) {
                                   (void)detail::release_or_invalidate_binary_entries(
-                                          registry, entries, failed, true);
+                                          registry, entries, failed, proved);
                               });
                     } catch (...) {
                         registry.remove_entries(std::span<const detail::EntryId>(

@@ -27,6 +27,8 @@ enum class SubmissionFault {
     stream_synchronize,     // queue destruction: the final proof of completion fails
     silu_launch,            // after acceptance, before the native SiLU launch
     sdpa_launch,            // after acceptance of an attention request
+    event_record_unproved,  // as event_record, and the stream synchronisation that would prove the
+                            // failed submission's work finished fails as well
 };
 
 void inject_submission_fault_for_testing(SubmissionFault fault) noexcept;

@@ -499,7 +499,7 @@ def bind_iomc(l: C.CDLL) -> C.CDLL:
 # numeric values of iom::rocm_detail::SubmissionFault (iom_amd/host/mi355x_testing.hpp)
 (FAULT_NONE, FAULT_EVENT_CREATE, FAULT_QUEUE_EVENT_CREATE, FAULT_QUEUE_STREAM_CREATE,
  FAULT_KERNEL_LAUNCH, FAULT_EMBEDDING_STATUS_COPY, FAULT_EVENT_RECORD, FAULT_STREAM_SYNCHRONIZE,
- FAULT_SILU_LAUNCH, FAULT_SDPA_LAUNCH) = range(10)
+ FAULT_SILU_LAUNCH, FAULT_SDPA_LAUNCH, FAULT_EVENT_RECORD_UNPROVED) = range(11)
 (COUNT_EVENT_CREATE, COUNT_EVENT_DESTROY, COUNT_STREAM_CREATE, COUNT_STREAM_DESTROY,
  COUNT_DEVICE_ALLOC, COUNT_DEVICE_FREE, COUNT_LINEAR_NATIVE, COUNT_LINEAR_SCALAR, COUNT_SILU) = range(9)
 

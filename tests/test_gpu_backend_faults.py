@@ -17,7 +17,7 @@ import iomo
 from iomo import (COUNT_DEVICE_ALLOC, COUNT_DEVICE_FREE, COUNT_EVENT_CREATE, COUNT_EVENT_DESTROY,
                   COUNT_LINEAR_NATIVE, COUNT_LINEAR_SCALAR, COUNT_SILU, COUNT_STREAM_CREATE,
                   COUNT_STREAM_DESTROY, DT_BF16, DT_F32, DT_U8, DT_U16, FAULT_EMBEDDING_STATUS_COPY,
-                  FAULT_EVENT_CREATE, FAULT_EVENT_RECORD, FAULT_KERNEL_LAUNCH, FAULT_NONE,
+                  FAULT_EVENT_CREATE, FAULT_EVENT_RECORD, FAULT_EVENT_RECORD_UNPROVED, FAULT_KERNEL_LAUNCH, FAULT_NONE,
                   FAULT_QUEUE_EVENT_CREATE, FAULT_QUEUE_STREAM_CREATE, FAULT_SDPA_LAUNCH,
                   FAULT_SILU_LAUNCH, FAULT_STREAM_SYNCHRONIZE, OP_ADD)
 from test_oracle_sdpa import random_case, shapes
@@ -302,5 +302,52 @@ def test_a_workspace_dropped_before_the_wait_stays_out_of_the_allocator(gpu):
     assert np.array_equal(t[3].view().to_host(), want)
     assert not successor.view().to_host().any()
     successor.close()
+    for x in t:
+        x.close()
+
+
+def test_a_failed_submission_without_proof_of_completion_keeps_its_workspace_range(gpu):
+    """The completion event of an accepted attention request cannot be recorded, and the stream
+    synchronisation that would still prove the kernel finished fails as well: the operation
+    retires as failed, and its workspace range -- which the kernel may still be writing for all
+    the host knows -- is never handed out again.  With the proof (the plain event_record fault)
+    the range returns to the allocator."""
+    case = random_case(19, (2,), 8, 2, 300, 64, 320, 10, 310)
+    qd, kd, od = shapes(case)
+    t = [gpu.tensor(DT_BF16, d) for d in (qd, kd, kd, od)]
+    for tensor, name, d in zip(t, "qkv", (qd, kd, kd)):
+        tensor.view().from_host(np.array(case[name], np.uint16).reshape(d))
+    views = [x.view() for x in t]
+    need = gpu.sdpa_workspace_bytes(*views, 10, 310)
+    assert need > 0
+
+    def first_fit():
+        probe = gpu.tensor(DT_U8, (need // 256, 16, 16))
+        address = gpu.l.iomc_view_native_handle(probe.view().h)
+        probe.close()
+        return address
+
+    # proved: the failed operation's range is free again once its owner goes away
+    address = first_fit()
+    ws = gpu.workspace(need)
+    gpu.inject(FAULT_EVENT_RECORD)
+    token = gpu.sdpa_submit(*views, 10, 310, ws)
+    assert token > 0 and gpu.wait(token) == -5
+    gpu.drop_workspace(ws)
+    assert first_fit() == address
+    # unproved: the same range stays out of the allocator
+    ws = gpu.workspace(need)
+    gpu.inject(FAULT_EVENT_RECORD_UNPROVED)
+    token = gpu.sdpa_submit(*views, 10, 310, ws)
+    gpu.inject(FAULT_NONE)
+    assert token > 0 and gpu.wait(token) == -5
+    assert gpu.wait(token) == -5                                          # the failure repeats
+    gpu.drop_workspace(ws)
+    assert first_fit() != address
+    # the queue goes on working, with a workspace elsewhere in the arena
+    ws = gpu.workspace(need)
+    token = gpu.sdpa_submit(*views, 10, 310, ws)
+    assert token > 0 and gpu.wait(token) == 0, gpu.error()
+    gpu.drop_workspace(ws)
     for x in t:
         x.close()

@@ -92,14 +92,23 @@ def test_completion_word_arrives_after_the_work_before_it():
     vb = datagen.bf16_rne(datagen.normal_f32(n, 0, 1, 8)).reshape(dims)
     a.view().from_host(va)
     b.view().from_host(vb)
+    after_add = iomx.Event(timing=False)
     for ticket in (1, 2, 0xFFFFFFFF):
         o.view().from_host(np.zeros(dims, np.uint16))
         assert iomx.binary(ADD, a.view(), b.view(), o.view(), st) == 0
+        after_add.record(st)
         iomx.check(L.iomx_stream_write_word(st.h, on_device, ticket))
         deadline = time.monotonic() + 10.0
         while word[0] != ticket:
             assert time.monotonic() < deadline, "the completion word never arrived"
-        got = o.buf.download(np.uint16)                     # no wait for the stream in between
+        # the moment the word is seen, the work before it must already be complete: an event
+        # recorded between the ADD and the word reports done without anybody waiting for it
+        done = C.c_int(-1)
+        iomx.check(L.iomx_event_query(after_add.h, C.byref(done)))
+        assert done.value == 1, "the word arrived before the work recorded ahead of it"
+        # (the download below runs on the null stream, which does not wait for `st`:
+        # iomx_stream_create makes non-blocking streams)
+        got = o.buf.download(np.uint16)
         want = iomx.DeviceTensor(DT_BF16, dims)
         assert iomx.binary(ADD, a.view(), b.view(), want.view()) == 0
         assert np.array_equal(got, want.raw())

@@ -118,6 +118,10 @@ def float64_attention(case):
     return out, budget + 2.0 ** -8 * np.abs(out) + 2.0 ** -126
 
 
+# seeded shapes whose matrix-core result has outputs outside the fixture rule, and how many
+FIXTURE_RULE_CAP = {((2,), 8, 2, 40, 64, 100, 50, 90): 4}
+
+
 @pytest.mark.parametrize("path", [0, 1], ids=["matrix_cores", "reference_order"])
 @pytest.mark.parametrize("spec", SEEDED, ids=[str(i) for i in range(len(SEEDED))])
 def test_seeded_shapes_against_the_oracle(spec, path):
@@ -141,8 +145,13 @@ def test_seeded_shapes_against_the_oracle(spec, path):
     assert np.all(np.abs(g - w) <= 2 * budget)                 # hence within twice the budget of each other
     if path == 1:
         assert outside == [] and exact >= 0.98 * got.size     # same order of operations; only expf may differ
-    # (on the matrix-core path the count outside the fixture rule is printed above, not asserted: the
-    # rule -- two BF16 steps or 2^-10 -- is not a bound under cancellation; the budget is, on every element)
+    else:
+        # The reference's own acceptance rule for a native kernel -- two BF16 steps or 2^-10
+        # (docs/BACKEND_CONTRACT/scaled-dot-product-attention.md:282-287) -- holds on every element of
+        # every seeded shape but one, where 4 of 40960 outputs that cancel to near zero miss it (the
+        # rule is not a bound under cancellation; the float64 budget above is, on every element).
+        # That count is a cap: a kernel change that worsens it fails here.
+        assert len(outside) <= FIXTURE_RULE_CAP.get(spec, 0), (spec, len(outside))
 
 
 @pytest.mark.parametrize("R", [6, 20], ids=["decode_kernel", "tiled_kernel_and_guard"])
@@ -241,7 +250,7 @@ def test_decode_step_against_a_long_prefix_in_shares(spec):
     assert np.all(np.abs(g - ref64) <= budget)                 # every element inside the float64 budget
     assert np.all(np.abs(w - ref64) <= budget)                 # ... as is the oracle
     assert np.all(np.abs(g - w) <= 2 * budget)
-    print(spec, "outside the fixture rule:", len(close_to_oracle(got, want)), "of", got.size, flush=True)
+    assert close_to_oracle(got, want) == []                    # and the reference's fixture rule holds
 
 
 def test_decode_in_shares_with_special_scores_and_values():

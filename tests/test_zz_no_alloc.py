@@ -126,3 +126,35 @@ def test_a_request_beyond_the_array_is_rejected_before_any_launch():
     assert iomx.sdpa_static(q.view(), k.view(), v.view(), o.view(), 4000, 5000) == -1
     for t in (q, k, v, o):
         t.free()
+
+
+def test_captured_into_a_graph_after_an_eager_call_and_replayed():
+    """One eager call first (it looks the array's address up), then the entry point recorded into a
+    graph on a stream of its own and replayed twice, with eager work on the same array and a
+    synchronisation between the replays: every replay gives the bits of iomx_launch_sdpa."""
+    spec = PREFILL_ROW[2]
+    case = random_case(430, *spec)
+    want, _, _ = with_caller_workspace(case)
+    got, _ = with_static_scratch(case)                       # the eager call
+    assert np.array_equal(got, want)
+    q, k, v, o = operands(case)
+    st = iomx.Stream()
+    st.begin_capture()
+    rc = iomx.sdpa_static(q.view(), k.view(), v.view(), o.view(), case["a"], case["L"], 0, st)
+    graph = st.end_capture()
+    assert rc == 0
+    other = random_case(431, *PREFILL_ROW[1])
+    for replay in range(2):
+        o.buf.fill(0x5A)
+        iomx.synchronize()
+        graph.launch(st)
+        st.synchronize()
+        assert np.array_equal(o.raw(), want), replay
+        # eager work that overwrites the array between the replays
+        got_other, _ = with_static_scratch(other)
+        want_other, _, _ = with_caller_workspace(other)
+        assert np.array_equal(got_other, want_other)
+    graph.close()
+    st.close()
+    for t in (q, k, v, o):
+        t.free()
