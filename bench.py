@@ -528,11 +528,14 @@ def wl_vendor_stream(timer, steps, warmup):
 def wl_sdpa(timer, steps, warmup):
     """BF16 causal grouped-query attention at TinyLlama's head shape (32 query heads, 4 KV
     heads, D = 64): a 512-token prefill of 8 sequences and a decode step of 64 sequences
-    against a 512-token cache.  Algorithmic bytes: q, the visible K and V prefix and out,
+    against a 512-token cache; and a 4096-token prefill of one sequence at D = 64 and at
+    D = 128 with 8 KV heads.  Algorithmic bytes: q, the visible K and V prefix and out,
     once each; flops: 4 * D per (row, visible token, head)."""
     out = []
-    Hq, Hkv, D, C = 32, 4, 64, 512
-    for name, B, R, a, L in (("prefill", 8, 512, 0, 512), ("decode", 64, 1, 511, 512)):
+    for name, B, R, a, L, Hq, Hkv, D in (("prefill", 8, 512, 0, 512, 32, 4, 64), ("decode", 64, 1, 511, 512, 32, 4, 64),
+                                         ("prefill", 1, 4096, 0, 4096, 32, 4, 64),
+                                         ("prefill", 1, 4096, 0, 4096, 32, 8, 128)):
+        C = L
         q = device_tensor(BF16, (B, Hq, R, D), "normal", 111)
         k = device_tensor(BF16, (B, Hkv, C, D), "normal", 112)
         v = device_tensor(BF16, (B, Hkv, C, D), "normal", 113)
@@ -548,7 +551,7 @@ def wl_sdpa(timer, steps, warmup):
         wall, ev = timer.run(launch, steps, warmup, warm_ms=30.0)
         visible = sum(min(L, a + r + 1) for r in range(R))
         flops = 4.0 * B * Hq * D * visible
-        r = report("sdpa_bf16_%s_B%d_Hq32_Hkv4_R%d_L%d_D64" % (name, B, R, L),
+        r = report("sdpa_bf16_%s_B%d_Hq%d_Hkv%d_R%d_L%d_D%d" % (name, B, Hq, Hkv, R, L, D),
                    2 * (B * Hq * R * D * 2 + 2 * B * Hkv * L * D), B * Hq * R * D, wall, ev,
                    iomx.last_launch().kernel.decode())
         r["TFLOP_per_s"] = round(flops / (ev * 1e-3) / 1e12, 2)

@@ -21,6 +21,7 @@
 //                   the row must not see would poison the row on the matrix cores.
 #include <atomic>
 #include <type_traits>
+#include <utility>
 
 #include "iomx_mfma.hpp"
 
@@ -289,6 +290,67 @@ __device__ __forceinline__ uint32_t cvt_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
 
+// LDS reads written out as instructions (see the shared-ring walk of sdpa_mfma): the 32-bit LDS
+// address of a pointer into a __shared__ array, one 128-bit read at a constant offset from it,
+// and the wait that makes every such read issued so far usable.
+__device__ __forceinline__ uint32_t lds_address(const void* shared) {
+    return (uint32_t)(uintptr_t)(lptr_t)shared;
+}
+template <int OFFSET>
+__device__ __forceinline__ u32x4 lds_read_b128(uint32_t address) {
+    static_assert(OFFSET >= 0 && OFFSET < 65536 && OFFSET % 16 == 0, "immediate offset of ds_read_b128");
+    u32x4 value;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(value) : "v"(address), "n"(OFFSET));
+    return value;
+}
+__device__ __forceinline__ void lds_reads_landed() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// max(a, b, c) as the one instruction (the compiler's own maximum first makes every operand a
+// quiet NaN or itself, an instruction apiece; the scores here come out of multiplications and
+// selects and need none of that).
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+__device__ __forceinline__ float max2(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
+// Eight products e[i] * scale, those below the smallest normal number as zeros, rounded to BF16
+// (nearest even) and packed in order.  The multiplications run with the mode register's binary32
+// denormal field on "flush", which makes the zeroing part of the multiplication instead of a
+// compare and a select per product; the field is set back before anything else executes.
+__device__ __forceinline__ u32x4 scaled_flushed_bf16x8(const float (&e)[8], float scale) {
+    float p[8];
+    asm volatile(
+            "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 4, 2), 0\n\t"
+            "v_mul_f32 %0, %8, %16\n\t"
+            "v_mul_f32 %1, %9, %16\n\t"
+            "v_mul_f32 %2, %10, %16\n\t"
+            "v_mul_f32 %3, %11, %16\n\t"
+            "v_mul_f32 %4, %12, %16\n\t"
+            "v_mul_f32 %5, %13, %16\n\t"
+            "v_mul_f32 %6, %14, %16\n\t"
+            "v_mul_f32 %7, %15, %16\n\t"
+            "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 4, 2), 3"
+            : "=&v"(p[0]), "=&v"(p[1]), "=&v"(p[2]), "=&v"(p[3]), "=&v"(p[4]), "=&v"(p[5]), "=&v"(p[6]), "=&v"(p[7])
+            : "v"(e[0]), "v"(e[1]), "v"(e[2]), "v"(e[3]), "v"(e[4]), "v"(e[5]), "v"(e[6]), "v"(e[7]), "v"(scale));
+    return u32x4{cvt_bf16x2(p[0], p[1]), cvt_bf16x2(p[2], p[3]), cvt_bf16x2(p[4], p[5]), cvt_bf16x2(p[6], p[7])};
+}
+
+template <class F, int... I>
+__device__ __forceinline__ void static_for_each(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_each(f, std::make_integer_sequence<int, N>{});
+}
+
 template <int DT16, int MODE, bool FULLD>
 __global__ __launch_bounds__(sdpa_waves(DT16, MODE) * 64) __attribute__((amdgpu_waves_per_eu(MODE != 1 ? 3 : 2)))
 void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
@@ -385,14 +447,21 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                                 kp + (((2 * g + half) * a.d_tiles + tile) * kTileBytes + kp_lane));
                 }
         };
-        // scores: lane gets tokens 32g + 16*half + 4*kg + j (j < 4) of row l16
-        auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2]) {
+        // scores: lane gets tokens 32g + 16*half + 4*kg + j (j < 4) of row l16.  `bare` (plain
+        // passes, sqrt(D) a power of two): the dot products themselves -- the division is exact
+        // there, so the passes fold it into the constant of their exponent argument and get the
+        // same bits with one multiplication less per score.
+        auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2], bool bare) {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int c = 0; c < D32; ++c)
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kgp.w[half][c]), qf[c], acc, 0, 0, 0);
+                if (bare) {
+                    s[half] = acc;
+                    continue;
+                }
                 // dot / sqrt(D): the product with the reciprocal is the quotient when sqrt(D) is
                 // a power of two; otherwise one correction step of the remainder makes it the
                 // correctly rounded quotient in all but halfway cases of the last bit
@@ -409,7 +478,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         };
         // the visible groups of this wave, K one group ahead where the mode says so; WITH_V: the
         // V fragments of the group are requested before its scores are formed
-        auto walk_groups = [&](auto with_v, auto&& body) {
+        auto walk_groups = [&](auto with_v, bool bare, auto&& body) {
             constexpr bool WITH_V = decltype(with_v)::value;
             if constexpr (SHARE) {
                 // wave w brings in KiB chunks w, w+4, .. of the K group (and of the V group) of
@@ -442,21 +511,36 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                     const uint8_t* stage = kv_ring + buf * kStage;
                     buf = buf == 2 ? 0 : buf + 1;
                     if (MODE == 3 && g >= groups) continue;               // uniform: past this wave's own tile
+                    // The operands come out of LDS through ds_read instructions the compiler does
+                    // not see as such.  Left to itself it waits, before every LDS read, for every
+                    // direct load still in flight (it cannot tell the ring's stages apart), which
+                    // is a full trip to the cache per group, every group; the counted wait and the
+                    // barrier above already say exactly what this stage needs.
                     KGroup cur;
+                    const uint32_t k_at = lds_address(stage + ((kg >> 1) * kTileBytes + kp_lane));
+                    static_for<2 * D32>([&](auto index) {
+                        constexpr int half = decltype(index)::value / D32, c = decltype(index)::value % D32;
+                        cur.w[half][c] = lds_read_b128<(half * DT16 + 2 * c) * (int)kTileBytes>(k_at);
+                    });
+                    u32x4 vfr[WITH_V ? DT16 : 1];
+                    if constexpr (WITH_V) {
+                        const uint32_t v_at = lds_address(stage + vf_lane);
+                        static_for<DT16>([&](auto index) {
+                            constexpr int dt = decltype(index)::value;
+                            vfr[dt] = lds_read_b128<(DT16 + dt) * (int)kFrag>(v_at);
+                        });
+                    }
+                    lds_reads_landed();
 #pragma unroll
                     for (int half = 0; half < 2; ++half)
 #pragma unroll
-                        for (int c = 0; c < D32; ++c)
-                            cur.w[half][c] = *reinterpret_cast<const u32x4*>(
-                                    stage + ((half * DT16 + 2 * c + (kg >> 1)) * kTileBytes + kp_lane));
-                    u32x4 vfr[WITH_V ? DT16 : 1];
+                        for (int c = 0; c < D32; ++c) asm volatile("" : "+v"(cur.w[half][c]));
                     if constexpr (WITH_V) {
 #pragma unroll
-                        for (int dt = 0; dt < DT16; ++dt)
-                            vfr[dt] = *reinterpret_cast<const u32x4*>(stage + ((DT16 + dt) * kFrag + vf_lane));
+                        for (int dt = 0; dt < DT16; ++dt) asm volatile("" : "+v"(vfr[dt]));
                     }
                     f32x4_t s[2];
-                    scores(cur, s);
+                    scores(cur, s, bare);
                     body(g, s, vfr);
                 }
                 // nothing in flight and nobody reading when the next pass (or the next workgroup)
@@ -478,7 +562,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                         vfr[dt] = *reinterpret_cast<const u32x4*>(vf + ((g * a.d_tiles + dt) * kFrag + vf_lane));
                 }
                 f32x4_t s[2];
-                scores(cur, s);
+                scores(cur, s, bare);
                 body(g, s, vfr);
                 if (AHEAD) cur = nxt;
             }
@@ -491,11 +575,18 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) s[half][j] = 16 * half + j < rem ? s[half][j] : -inf;
         };
+        // The plain passes work on the dot products themselves where dividing by sqrt(D) is exact
+        // (a power of two): the division moves into the constant of the exponent argument,
+        // 2^(dot * (log2 e / sqrt(D)) - max * (log2 e / sqrt(D))), which is the same binary32 value as
+        // 2^((dot / sqrt(D)) * log2 e - ...) bit for bit, since scaling by a power of two commutes
+        // with rounding.  The running maximum is then a maximum of dot products.
+        const bool bare = a.scale_pow2 != 0;
+        const float kls = bare ? kLog2e * a.inv_scale : kLog2e;
         // (maximum, sum) of one part of a row joined with another part's
         auto join = [&](float& m, float& sum, float m2, float sum2) {
             const float mm = __builtin_fmaxf(m, m2), base = __builtin_fmaxf(mm, kFloor);
-            sum = sum * __builtin_amdgcn_exp2f((__builtin_fmaxf(m, kFloor) - base) * kLog2e)
-                + sum2 * __builtin_amdgcn_exp2f((__builtin_fmaxf(m2, kFloor) - base) * kLog2e);
+            sum = sum * __builtin_amdgcn_exp2f((__builtin_fmaxf(m, kFloor) - base) * kls)
+                + sum2 * __builtin_amdgcn_exp2f((__builtin_fmaxf(m2, kFloor) - base) * kls);
             m = mm;
         };
         auto mma_v = [&](f32x4_t (&o)[DT16], const u32x4 (&vfr)[DT16], const u32x4& pw) {
@@ -507,19 +598,19 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 
         // ---- plain pass 1: running maximum and sum of exp(score - maximum)
         float pm = -inf, psum = 0.0f;
-        walk_groups(std::false_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+        walk_groups(std::false_type{}, bare, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
             if (g >= full_groups) mask_group(g, s);
-            const float local = __builtin_fmaxf(
-                    __builtin_fmaxf(__builtin_fmaxf(s[0][0], s[0][1]), __builtin_fmaxf(s[0][2], s[0][3])),
-                    __builtin_fmaxf(__builtin_fmaxf(s[1][0], s[1][1]), __builtin_fmaxf(s[1][2], s[1][3])));
-            const float newm = __builtin_fmaxf(pm, local);
-            const float base = __builtin_fmaxf(newm, kFloor);
-            psum *= __builtin_amdgcn_exp2f((__builtin_fmaxf(pm, kFloor) - base) * kLog2e);
-            const float nb = -base * kLog2e;
+            // (the maximum instruction itself: a NaN among its operands is passed over, and the
+            // row's sum below turns NaN from that score's exponential all the same)
+            const float newm = max3(max3(s[0][0], s[0][1], s[0][2]), max3(s[0][3], s[1][0], s[1][1]),
+                                    max3(s[1][2], s[1][3], pm));
+            const float base = max2(newm, kFloor);
+            psum *= __builtin_amdgcn_exp2f((max2(pm, kFloor) - base) * kls);
+            const float nb = -base * kls;
 #pragma unroll
             for (int half = 0; half < 2; ++half)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) psum += __builtin_amdgcn_exp2f(__builtin_fmaf(s[half][j], kLog2e, nb));
+                for (int j = 0; j < 4; ++j) psum += __builtin_amdgcn_exp2f(__builtin_fmaf(s[half][j], kls, nb));
             pm = newm;
         });
 #pragma unroll
@@ -550,24 +641,22 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         bool nan_row = false;
         if (plain) {
             // ---- plain pass 2: probabilities, rounded once to BF16 and flushed, times V
-            const float inv_sum = 1.0f / psum, nb = -pm * kLog2e;
-            walk_groups(std::true_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+            const float inv_sum = 1.0f / psum, nb = -pm * kls;
+            walk_groups(std::true_type{}, bare, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
                 if (g >= full_groups) mask_group(g, s);
-                float pr[8];
+                float e[8];
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[half][j], kLog2e, nb)) * inv_sum;
-                        pr[half * 4 + j] = pv < 1.17549435e-38f ? 0.0f : pv;      // below the BF16 normals
-                    }
-                mma_v(o, vfr, u32x4{cvt_bf16x2(pr[0], pr[1]), cvt_bf16x2(pr[2], pr[3]),
-                                    cvt_bf16x2(pr[4], pr[5]), cvt_bf16x2(pr[6], pr[7])});
+                    for (int j = 0; j < 4; ++j)
+                        e[half * 4 + j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[half][j], kls, nb));
+                // probabilities below the BF16 normals are zeros as matrix operands
+                mma_v(o, vfr, scaled_flushed_bf16x8(e, inv_sum));
             });
         } else {
             // ---- pass 1 with the bookkeeping of the special rows
             RowStats st = {-inf, 0.0f, 0u, false, false};
-            walk_groups(std::false_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+            walk_groups(std::false_type{}, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
                 // the finite maximum of the lane's eight scores first, then one rescale; written
                 // with selects only (a branch per element would cost more than the arithmetic)
                 float local = -inf;
@@ -620,7 +709,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
             const float inv_sum = 1.0f / st.sum;
             // ---- pass 2 of the special rows
-            walk_groups(std::true_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+            walk_groups(std::true_type{}, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
                 float pr[8];
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
