@@ -67,6 +67,21 @@ __device__ __forceinline__ float daz_bf16(uint32_t h) {
     return as_f32(((h & 0x7F80u) ? h : (h & 0x8000u)) << 16);
 }
 
+// LDS reads written out as instructions (see the shared-ring walk of sdpa_mfma): the 32-bit LDS
+// address of a pointer into a __shared__ array, one 128-bit read at a constant offset from it,
+// and the wait that makes every such read issued so far usable.
+__device__ __forceinline__ uint32_t lds_address(const void* shared) {
+    return (uint32_t)(uintptr_t)(lptr_t)shared;
+}
+template <int OFFSET>
+__device__ __forceinline__ u32x4 lds_read_b128(uint32_t address) {
+    static_assert(OFFSET >= 0 && OFFSET < 65536 && OFFSET % 16 == 0, "immediate offset of ds_read_b128");
+    u32x4 value;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(value) : "v"(address), "n"(OFFSET));
+    return value;
+}
+__device__ __forceinline__ void lds_reads_landed() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
 // One workgroup packs a share of the fragments of one KV head of one plane and writes
 // that share's flag word (every word is written on every call, so the workspace needs
 // no clearing).
@@ -78,10 +93,18 @@ __device__ __forceinline__ float daz_bf16(uint32_t h) {
 // prefix and columns past D as zeros, so that the many waves that meet a K tile do not
 // each flush it again.
 __global__ __launch_bounds__(256) void sdpa_pack_kernel(const SdpaArgs a) {
+    // a wave's staging area for the transposition: the two 16x16 V tiles of a fragment as they lie
+    __shared__ __attribute__((aligned(16))) uint8_t turn[4][2 * kTileBytes];
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
     const uint32_t hkv = blockIdx.x / a.pack_splits, split = blockIdx.x - hkv * a.pack_splits;
     const uint32_t frags = a.groups * a.d_tiles;
+    // lane = 16-byte chunk of the two tiles of a group: tile lane/32, row (lane%32)/2, half lane%2
+    const uint32_t in_tile = lane >> 5, r = (lane & 31u) >> 1, half = lane & 1u;
+    // the transposing read: the sixteen lanes of quarter kg supply the 8-byte pieces of rows
+    // 4kg .. 4kg+3 (lane 4i + c: row 4kg + i, columns 4c .. 4c+3), and lane (kg, d) receives
+    // column d of those four rows -- tokens 4kg .. 4kg+3 of feature d, the fragment's order
+    const uint32_t turn_at = lds_address(&turn[wave][0]) + (4 * kg + (l16 >> 2)) * kRowBytes + (l16 & 3u) * 8;
     for (uint32_t p = blockIdx.y; p < a.planes; p += gridDim.y) {
         uint64_t plane[4];
         walk_planes(a.walk, p, plane);
@@ -91,33 +114,33 @@ __global__ __launch_bounds__(256) void sdpa_pack_kernel(const SdpaArgs a) {
         bool special = false;
         for (uint32_t frag = split * 4 + wave; frag < frags; frag += 4 * a.pack_splits) {
             const uint32_t g = frag / a.d_tiles, dt = frag - g * a.d_tiles;
-            const uint32_t d = dt * kTile + l16;
-            uint32_t h[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t token = 32 * g + (j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4));
-                uint32_t bits = 0;
-                if (token < a.L && d < a.D) {
-                    bits = *reinterpret_cast<const uint16_t*>(
-                            vb + ((uint64_t)(token >> 4) * a.d_tiles + dt) * kTileBytes + (token & 15u) * kRowBytes + l16 * 2);
-                    special = special || (bits & 0x7F80u) == 0x7F80u;
-                    if ((bits & 0x7F80u) == 0) bits &= 0x8000u;
-                }
-                h[j] = bits;
+            const uint32_t tt = 2 * g + in_tile;
+            const uint64_t tile_row = ((uint64_t)tt * a.d_tiles + dt) * kTileBytes + r * kRowBytes;
+            // both operands are requested before anything is stored (a load is not moved across a
+            // store it cannot be told apart from: that would be two trips to memory in a row);
+            // tokens past the prefix and columns past D are zeros
+            u32x4 vw = {0, 0, 0, 0}, kw = {0, 0, 0, 0};
+            if (tt * kTile + r < a.L) {
+                vw = load_k8_bits(vb + tile_row, half * 8, dt * kTile + half * 8, a.D);
+                if (a.packed_k) kw = load_k8_bits(kb + tile_row, half * 8, dt * kTile + half * 8, a.D);
             }
-            *reinterpret_cast<u32x4*>(a.packed_v + (head_frags + frag) * kFrag + lane * 16) =
-                    u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                special = special || (vw[i] & 0x7F80u) == 0x7F80u || (vw[i] & 0x7F800000u) == 0x7F800000u;
+            vw = u32x4{daz2(vw[0]), daz2(vw[1]), daz2(vw[2]), daz2(vw[3])};
+            *reinterpret_cast<u32x4*>(&turn[wave][lane * 16]) = vw;
+            u32x2 lo, hi;
+            // (the "memory" clobber keeps the store above ahead of the reads; a wave's LDS
+            // instructions execute in order, so the reads see all sixty-four lanes' pieces)
+            asm volatile("ds_read_b64_tr_b16 %0, %2\n\t"
+                         "ds_read_b64_tr_b16 %1, %2 offset:512\n\t"
+                         "s_waitcnt lgkmcnt(0)"
+                         : "=&v"(lo), "=&v"(hi) : "v"(turn_at) : "memory");
+            *reinterpret_cast<u32x4*>(a.packed_v + (head_frags + frag) * kFrag + lane * 16) = u32x4{lo.x, lo.y, hi.x, hi.y};
             if (a.packed_k) {
-                // lane = 16-byte chunk of the two tiles: tile lane/32, row (lane%32)/2, half lane%2
-                const uint32_t tt = 2 * g + (lane >> 5), r = (lane & 31u) >> 1, half = lane & 1u;
-                const uint32_t token = tt * kTile + r;
-                u32x4 w = {0, 0, 0, 0};
-                if (token < a.L)
-                    w = load_k8_bits(kb + ((uint64_t)tt * a.d_tiles + dt) * kTileBytes + r * kRowBytes,
-                                     half * 8, dt * kTile + half * 8, a.D);
-                w = u32x4{daz2(w[0]), daz2(w[1]), daz2(w[2]), daz2(w[3])};
+                kw = u32x4{daz2(kw[0]), daz2(kw[1]), daz2(kw[2]), daz2(kw[3])};
                 *reinterpret_cast<u32x4*>(a.packed_k + ((head_frags * 2 + (uint64_t)tt * a.d_tiles + dt) * kTileBytes)
-                                          + (lane & 31u) * 16) = w;
+                                          + (lane & 31u) * 16) = kw;
             }
         }
         const int any = __syncthreads_or(special ? 1 : 0);
@@ -290,21 +313,6 @@ __device__ __forceinline__ uint32_t cvt_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
 
-// LDS reads written out as instructions (see the shared-ring walk of sdpa_mfma): the 32-bit LDS
-// address of a pointer into a __shared__ array, one 128-bit read at a constant offset from it,
-// and the wait that makes every such read issued so far usable.
-__device__ __forceinline__ uint32_t lds_address(const void* shared) {
-    return (uint32_t)(uintptr_t)(lptr_t)shared;
-}
-template <int OFFSET>
-__device__ __forceinline__ u32x4 lds_read_b128(uint32_t address) {
-    static_assert(OFFSET >= 0 && OFFSET < 65536 && OFFSET % 16 == 0, "immediate offset of ds_read_b128");
-    u32x4 value;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(value) : "v"(address), "n"(OFFSET));
-    return value;
-}
-__device__ __forceinline__ void lds_reads_landed() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-
 // max(a, b, c) as the one instruction (the compiler's own maximum first makes every operand a
 // quiet NaN or itself, an instruction apiece; the scores here come out of multiplications and
 // selects and need none of that).
@@ -420,6 +428,31 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         // below 4 GiB, and 64-bit addresses per load would cost the registers of a whole wave slot
         const uint8_t* vf = a.packed_v + (((uint64_t)p * a.Hkv + hkv) * a.groups) * a.d_tiles * kFrag;
         const uint32_t vf_lane = lane * 16;
+        const uint8_t* kp = a.packed_k + (((uint64_t)p * a.Hkv + hkv) * a.groups * 2) * a.d_tiles * kTileBytes;
+        const uint32_t kp_lane = l16 * kRowBytes + c0 * 2;
+        // One direct load of a wave's share of the K group (and of the V group) g into ring stage buf:
+        // wave w brings in KiB chunks w, w+4, .. ; lane i fetches 16-byte piece i of a chunk, and the
+        // loader puts it at chunk + 16*i, so a group lies in LDS as it lies in the packed regions.
+        auto issue = [&](auto with_v, uint32_t g, uint32_t buf) {
+            if constexpr (SHARE) {
+                const uint32_t gg = g < ring_groups ? g : ring_groups - 1;   // past the end: a valid group again, unused
+                uint8_t* stage = kv_ring + buf * kStage;
+#pragma unroll
+                for (int j = 0; j < DT16 / 4; ++j) {
+                    const uint32_t chunk = wave + 4 * j;
+                    __builtin_amdgcn_global_load_lds((gptr_t)(kp + ((gg * DT16 + chunk) * kFrag + vf_lane)),
+                                                     (lptr_t)(stage + chunk * kFrag), 16, 0, 0);
+                    if constexpr (decltype(with_v)::value)
+                        __builtin_amdgcn_global_load_lds((gptr_t)(vf + ((gg * DT16 + chunk) * kFrag + vf_lane)),
+                                                         (lptr_t)(stage + (DT16 + chunk) * kFrag), 16, 0, 0);
+                }
+            }
+        };
+        // the first two K groups of pass 1 are on their way while Q is fetched and flushed
+        if (SHARE && ring_groups != 0) {
+            issue(std::false_type{}, 0, 0);
+            issue(std::false_type{}, 1, 1);
+        }
         // the row tile of Q, flushed, as the B operand of every score tile
         bf16x8_t qf[D32];
 #pragma unroll
@@ -433,8 +466,6 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         // K of the 32 tokens of group g, from the flushed copy: two 16-token tiles, lane
         // (token l16, features 8*kg..); tokens past the prefix and columns past D are zeros there
         struct KGroup { u32x4 w[2][D32]; };
-        const uint8_t* kp = a.packed_k + (((uint64_t)p * a.Hkv + hkv) * a.groups * 2) * a.d_tiles * kTileBytes;
-        const uint32_t kp_lane = l16 * kRowBytes + c0 * 2;
         auto load_k = [&](uint32_t g, KGroup& kgp) {
 #pragma unroll
             for (int half = 0; half < 2; ++half)
@@ -478,28 +509,15 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         };
         // the visible groups of this wave, K one group ahead where the mode says so; WITH_V: the
         // V fragments of the group are requested before its scores are formed
-        auto walk_groups = [&](auto with_v, bool bare, auto&& body) {
+        // `primed`: the first two stages of the ring have been requested already
+        auto walk_groups = [&](auto with_v, bool bare, bool primed, auto&& body) {
             constexpr bool WITH_V = decltype(with_v)::value;
             if constexpr (SHARE) {
-                // wave w brings in KiB chunks w, w+4, .. of the K group (and of the V group) of
-                // every stage; lane i fetches 16-byte piece i of a chunk, and the loader puts it at
-                // chunk + 16*i, so a group lies in LDS as it lies in the packed regions
                 constexpr int LPS = (WITH_V ? 2 : 1) * (DT16 / 4);        // direct loads per wave and stage
-                auto issue = [&](uint32_t g, uint32_t buf) {
-                    const uint32_t gg = g < ring_groups ? g : ring_groups - 1;   // past the end: a valid group again, unused
-                    uint8_t* stage = kv_ring + buf * kStage;
-#pragma unroll
-                    for (int j = 0; j < DT16 / 4; ++j) {
-                        const uint32_t chunk = wave + 4 * j;
-                        __builtin_amdgcn_global_load_lds((gptr_t)(kp + ((gg * DT16 + chunk) * kFrag + vf_lane)),
-                                                         (lptr_t)(stage + chunk * kFrag), 16, 0, 0);
-                        if constexpr (WITH_V)
-                            __builtin_amdgcn_global_load_lds((gptr_t)(vf + ((gg * DT16 + chunk) * kFrag + vf_lane)),
-                                                             (lptr_t)(stage + (DT16 + chunk) * kFrag), 16, 0, 0);
-                    }
-                };
-                issue(0, 0);
-                issue(1, 1);
+                if (!primed) {
+                    issue(with_v, 0, 0);
+                    issue(with_v, 1, 1);
+                }
                 uint32_t buf = 0;
 #pragma unroll 1
                 for (uint32_t g = 0; g < ring_groups; ++g) {
@@ -507,7 +525,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                     // nobody reads the buffer of group g-1 any more: it takes group g+2
                     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPS) : "memory");
                     __builtin_amdgcn_s_barrier();
-                    issue(g + 2, buf == 0 ? 2 : buf - 1);
+                    issue(with_v, g + 2, buf == 0 ? 2 : buf - 1);
                     const uint8_t* stage = kv_ring + buf * kStage;
                     buf = buf == 2 ? 0 : buf + 1;
                     if (MODE == 3 && g >= groups) continue;               // uniform: past this wave's own tile
@@ -598,7 +616,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 
         // ---- plain pass 1: running maximum and sum of exp(score - maximum)
         float pm = -inf, psum = 0.0f;
-        walk_groups(std::false_type{}, bare, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+        walk_groups(std::false_type{}, bare, true, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
             if (g >= full_groups) mask_group(g, s);
             // (the maximum instruction itself: a NaN among its operands is passed over, and the
             // row's sum below turns NaN from that score's exponential all the same)
@@ -642,7 +660,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         if (plain) {
             // ---- plain pass 2: probabilities, rounded once to BF16 and flushed, times V
             const float inv_sum = 1.0f / psum, nb = -pm * kls;
-            walk_groups(std::true_type{}, bare, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+            walk_groups(std::true_type{}, bare, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
                 if (g >= full_groups) mask_group(g, s);
                 float e[8];
 #pragma unroll
@@ -656,7 +674,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         } else {
             // ---- pass 1 with the bookkeeping of the special rows
             RowStats st = {-inf, 0.0f, 0u, false, false};
-            walk_groups(std::false_type{}, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+            walk_groups(std::false_type{}, false, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
                 // the finite maximum of the lane's eight scores first, then one rescale; written
                 // with selects only (a branch per element would cost more than the arithmetic)
                 float local = -inf;
@@ -709,7 +727,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
             const float inv_sum = 1.0f / st.sum;
             // ---- pass 2 of the special rows
-            walk_groups(std::true_type{}, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+            walk_groups(std::true_type{}, false, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
                 float pr[8];
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
