@@ -543,13 +543,29 @@ __device__ __forceinline__ void hw_decode_row(const uint32_t (&w)[bits_of(DT) / 
     if constexpr (has_hw_f46(DT)) {
         hw_f46_decode<DT>(w, v);
     } else {
-        // a row with the all-NaN top exponent of F8_E4M3FN in it goes element by element
+        // The top exponent of F8_E4M3FN is all NaN for the leaf and holds numbers for the
+        // instruction: in a row that has such a byte every element is still converted by the
+        // instruction, and the bytes in question are replaced by the leaf's NaN (with the
+        // byte's sign, as decode_f32 gives it).
         bool special = false;
         if constexpr (DT == DT_F8_E4M3FN)
             special = e4m3_top_exponent(w[0]) | e4m3_top_exponent(w[1]) | e4m3_top_exponent(w[2]) | e4m3_top_exponent(w[3]);
-        if (special) {
+        // (decided for the wave as a whole: lanes that took different sides would make the wave
+        // walk both, and the replacement below is harmless for a row that needs none)
+        if (__any(special)) {
+            // a byte with the top exponent gets all three fraction bits set, four bytes at a time:
+            // that is the one encoding of the top exponent the instruction reads as NaN as well
+            // (the empty statement keeps this side a branch: folded into selects it would run, and
+            // cost its instructions, in every row)
+            asm volatile("");
+            uint32_t fixed[4];
 #pragma unroll
-            for (int i = 0; i < (int)kTile; ++i) v[i] = decode_f32<DT>((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t top = (((w[j] & 0x78787878u) + 0x08080808u) & 0x80808080u) >> 7;   // 1 per such byte
+                fixed[j] = w[j] | (top * 7u);
+            }
+#pragma unroll
+            for (int i = 0; i < (int)kTile; ++i) v[i] = hw_f8_value<DT>(fixed[i >> 2], i & 3);
         } else {
 #pragma unroll
             for (int i = 0; i < (int)kTile; ++i) v[i] = hw_f8_value<DT>(w[i >> 2], i & 3);
@@ -575,15 +591,60 @@ __device__ __forceinline__ void hw_encode_row(const float (&r)[kTile], uint32_t 
         bool plain = true;
 #pragma unroll
         for (int i = 0; i < (int)kTile; ++i) plain &= __builtin_fabsf(r[i]) <= hw_f8_limit<DT>();
-        if (plain) {
+        if (__all(plain)) {       // for the wave as a whole, as in hw_decode_row
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 w[j] = hw_f8_pack<DT>(r[4 * j + 2], r[4 * j + 3], hw_f8_pack<DT>(r[4 * j], r[4 * j + 1], 0u, false), true);
         } else {
+            // Some element is a NaN, an infinity or beyond the largest finite value.
+            asm volatile("");     // stays a branch, as in hw_decode_row
+            if constexpr (DT == DT_F8_E4M3FN) {
+                // Every number, infinities included, clamped to the largest finite magnitude first
+                // (240: what lies above rounds or saturates there); a NaN stays one.  No number
+                // then lands in the top exponent, so a byte that has it came from a NaN: the
+                // instruction stored 0x7F or 0xFF for it, and the leaf's NaN is 0x7F.
 #pragma unroll
-            for (int j = 0; j < 4; ++j) w[j] = 0;
+                for (int j = 0; j < 4; ++j) {
+                    float t[4];
 #pragma unroll
-            for (int i = 0; i < (int)kTile; ++i) w[i >> 2] |= encode_f32<DT>(r[i]) << (8 * (i & 3));
+                    for (int k = 0; k < 4; ++k) {
+                        const float x = r[4 * j + k];
+                        const float clamped = __builtin_fminf(__builtin_fmaxf(x, -240.0f), 240.0f);
+                        t[k] = (x != x) ? as_f32_hd(0x7FC00000u) : clamped;
+                    }
+                    const uint32_t word = hw_f8_pack<DT>(t[2], t[3], hw_f8_pack<DT>(t[0], t[1], 0u, false), true);
+                    w[j] = word & ~(((word & 0x78787878u) + 0x08080808u) & 0x80808080u);
+                }
+                return;
+            }
+            constexpr Fmt f = fmt_of(DT);
+            constexpr uint32_t emask = (1u << f.ebits) - 1u, fmask = (1u << f.fbits) - 1u;
+            constexpr uint32_t largest = ((emask - 1u) << f.fbits) | fmask;
+            constexpr uint32_t over = f.infs ? (emask << f.fbits) : largest;
+            constexpr uint32_t nan = (emask << f.fbits) | (f.finite_only ? fmask : 1u << (f.fbits - 1));
+            // F8_E5M2: the rest still goes through the instructions (a zero stands in for the odd
+            // ones), and the bytes of the odd ones are what encode_f32 stores for them: the leaf's
+            // NaN, or the signed overflow value -- 57344 below the halfway point to 2^16 and
+            // infinity from there on (the tie goes to the even neighbour, the infinity's place).
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float t[4];
+                uint32_t keep = 0xFFFFFFFFu, put = 0u;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float x = r[4 * j + k];
+                    const bool odd = !(__builtin_fabsf(x) <= hw_f8_limit<DT>());
+                    const uint32_t sign = (as_u32_hd(x) >> 31) << 7;
+                    uint32_t code = sign | over;
+                    if constexpr (DT == DT_F8_E5M2) code = __builtin_fabsf(x) < 61440.0f ? (sign | largest) : code;
+                    code = (x != x) ? nan : code;
+                    t[k] = odd ? 0.0f : x;
+                    keep = odd ? keep & ~(0xFFu << (8 * k)) : keep;
+                    put = odd ? put | (code << (8 * k)) : put;
+                }
+                const uint32_t word = hw_f8_pack<DT>(t[2], t[3], hw_f8_pack<DT>(t[0], t[1], 0u, false), true);
+                w[j] = (word & keep) | put;
+            }
         }
     }
 }
