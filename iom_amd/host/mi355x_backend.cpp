@@ -560,6 +560,11 @@ public:
     }
 
     ~Mi355xQueue() override {
+        // Owner fences of this queue's outstanding work are invalidated before anything drains
+        // (src/shared/gpu_queue_lifecycle.inl:96-101): an operand of accepted work that nobody
+        // waited for, destroyed after its queue, is then quarantined until the device ends
+        // instead of depending on how far the drain below happened to get.
+        device_.registry_state().registry.invalidate_entries_for_queue(registry_queue_id_);
         // Stop accepting, fail what never started, then let the completion thread
         // finish everything that was launched before the native objects go away.
         close_and_drain();

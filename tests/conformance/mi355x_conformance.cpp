@@ -369,6 +369,433 @@ TEST_CASE("MI355X: full shared suite with the RoPE contract") {
     CHECK_FALSE(f.gate.armed());
 }
 
+// ---- what the reference's accelerator driver asserts through backend seams ----------------------
+//
+// test/rocm/test_rocm_conformance.cpp holds, beside the shared runners above, scenarios written
+// against the reference ROCm backend's own fault seams (a failed launch, a failed event record, a
+// failed status copy) and against owner addresses.  The same behaviours, asked of this backend
+// through its own seams (mi355x_testing.hpp: one launch per operation, so the reference's "third
+// plane launch" is `kernel_launch` here), with the reference's shared helpers for data and
+// expected values.
+
+namespace {
+
+using Owner = std::unique_ptr<iom::Tensor>;
+
+// Owners created now must not sit where the given (released) owners sat.
+void expect_not_recycled(iom::Device& device, std::initializer_list<iom::TensorSpec> specs,
+                         std::initializer_list<const void*> retired) {
+    std::vector<Owner> fresh;
+    for (const iom::TensorSpec& spec : specs) {
+        fresh.push_back(device.create_tensor(spec));
+    }
+    for (const Owner& owner : fresh) {
+        for (const void* address : retired) {
+            CHECK_NE(static_cast<const void*>(owner->view().native_handle()), address);
+        }
+    }
+}
+
+// Raw tiled bytes of an owner, through the oracle above.
+std::vector<std::byte> raw_storage(RawStorageOracle& oracle, const iom::TensorSpec& spec, const iom::TensorView& view) {
+    oracle.set_owner_spec(spec);
+    return oracle.observe(view);
+}
+
+}  // namespace
+
+TEST_CASE("MI355X backend: a launch that fails after acceptance repeats its failure and the owners serve the next one") {
+    const auto device = make_candidate();
+    const iom::TensorSpec spec{iom::TensorShape{{2, 16, 16}}, iom::DataType::U8};
+    auto lhs = device->create_tensor(spec);
+    auto out = device->create_tensor(spec);
+    std::vector<std::byte> pattern(spec.logical_nbytes());
+    for (std::size_t i = 0; i < pattern.size(); ++i) {
+        pattern[i] = static_cast<std::byte>((i * 5 + 1) & 0xff);
+    }
+    conf::copy_from_host(lhs->view(), pattern);
+    auto queue = device->create_ops();
+
+    arm(seams::SubmissionFault::kernel_launch);
+    const iom::oid failed = queue->add(lhs->view(), lhs->view(), out->view());
+    disarm();
+    REQUIRE(iom::oid_is_token(failed));
+    conf::expect_repeated_runtime_failure(*queue, failed);
+
+    const iom::oid next = queue->add(lhs->view(), lhs->view(), out->view());
+    REQUIRE(iom::oid_is_token(next));
+    CHECK_EQ(conf::token_sequence(next), conf::token_sequence(failed) + 1);
+    CHECK_NOTHROW(queue->wait(next));
+    const std::vector<std::byte> doubled = conf::read_logical(out->view());
+    for (std::size_t i = 0; i < doubled.size(); ++i) {
+        CHECK_EQ(static_cast<unsigned>(doubled[i]), (static_cast<unsigned>(pattern[i]) * 2u) & 0xffu);
+    }
+}
+
+TEST_CASE("MI355X backend: only accepted submissions take a sequence, and a failed one's operands are not recycled") {
+    const auto device = make_candidate();
+    const iom::TensorSpec spec{iom::TensorShape{{3, 16, 16}}, iom::DataType::U8};
+    const iom::TensorSpec other{iom::TensorShape{{3, 16, 17}}, iom::DataType::U8};
+    auto source = device->create_tensor(spec);
+    auto destination = device->create_tensor(spec);
+    auto misfit = device->create_tensor(other);
+    const std::vector<std::byte> bytes(spec.logical_nbytes(), std::byte{0x3c});
+    conf::copy_from_host(source->view(), bytes);
+    conf::copy_from_host(destination->view(), bytes);
+    auto queue = device->create_ops();
+
+    // rejected by validation, then by a completion resource that cannot be had: no sequence
+    CHECK_EQ(queue->copy(source->view(), misfit->view()), iom::to_oid(iom::OidError::InvalidArgument));
+    const iom::oid first = queue->copy(source->view(), destination->view());
+    CHECK_EQ(conf::token_sequence(first), 1u);
+    CHECK_NOTHROW(queue->wait(first));
+    arm(seams::SubmissionFault::event_create);
+    CHECK_EQ(queue->copy(source->view(), destination->view()), iom::to_oid(iom::OidError::DeviceError));
+    const iom::oid second = queue->copy(source->view(), destination->view());
+    CHECK_EQ(conf::token_sequence(second), 2u);
+    CHECK_NOTHROW(queue->wait(second));
+
+    // accepted, then failed: the launch, and the record of the completion event
+    arm(seams::SubmissionFault::kernel_launch);
+    const iom::oid third = queue->copy(source->view(), destination->view());
+    CHECK_EQ(conf::token_sequence(third), 3u);
+    conf::expect_repeated_runtime_failure(*queue, third);
+    arm(seams::SubmissionFault::event_record);
+    const iom::oid fourth = queue->copy(source->view(), destination->view());
+    CHECK_EQ(conf::token_sequence(fourth), 4u);
+    conf::expect_repeated_runtime_failure(*queue, fourth);
+    disarm();
+
+    // a second device: the owners of a failed copy go away, their ranges do not come back
+    {
+        const auto second_device = make_candidate();
+        auto a = second_device->create_tensor(spec);
+        auto b = second_device->create_tensor(spec);
+        auto doomed = second_device->create_ops();
+        arm(seams::SubmissionFault::kernel_launch);
+        const iom::oid failure = doomed->copy(a->view(), b->view());
+        disarm();
+        CHECK_EQ(conf::token_sequence(failure), 1u);
+        conf::expect_repeated_runtime_failure(*doomed, failure);
+        const void* was_a = a->view().native_handle();
+        const void* was_b = b->view().native_handle();
+        a.reset();
+        b.reset();
+        expect_not_recycled(*second_device, {spec, spec}, {was_a, was_b});
+    }
+}
+
+TEST_CASE("MI355X backend: queue destruction drains pending copies around a failed one") {
+    const auto device = make_candidate();
+    const iom::TensorSpec spec{iom::TensorShape{{3, 16, 16}}, iom::DataType::U8};
+    auto source = device->create_tensor(spec);
+    auto destination = device->create_tensor(spec);
+    const std::vector<std::byte> bytes(spec.logical_nbytes(), std::byte{0x5a});
+    conf::copy_from_host(source->view(), bytes);
+    conf::copy_from_host(destination->view(), bytes);
+    {
+        auto queue = device->create_ops();
+        for (int i = 0; i < 32; ++i) {
+            CHECK(iom::oid_is_token(queue->copy(source->view(), destination->view())));
+        }
+        arm(seams::SubmissionFault::kernel_launch);
+        CHECK(iom::oid_is_token(queue->copy(source->view(), destination->view())));
+        for (int i = 0; i < 32; ++i) {
+            CHECK(iom::oid_is_token(queue->copy(source->view(), destination->view())));
+        }
+    }
+    disarm();
+    conf::require_logical_bytes(destination->view(), bytes, "destination after the drained queue");
+}
+
+TEST_CASE("MI355X backend: a source destroyed before the wait stays intact until both of its copies are done") {
+    const iom::TensorSpec spec{iom::TensorShape{{8192, 4096}}, iom::DataType::F32};       // 128 MiB
+    const std::vector<std::byte> expected = conf::encode_standard_tiled_storage(spec);
+    const std::vector<std::byte> zeros(spec.tiled_storage_nbytes(), std::byte{0});
+    const auto device = make_candidate();
+    RawStorageOracle oracle;
+    auto source = device->create_tensor(spec);
+    auto first_destination = device->create_tensor(spec);
+    auto second_destination = device->create_tensor(spec);
+    oracle.set_owner_spec(spec);
+    oracle.seed(source->view(), expected);
+    oracle.seed(first_destination->view(), zeros);
+    oracle.seed(second_destination->view(), zeros);
+    auto queue = device->create_ops();
+    const iom::oid first = queue->copy(source->view(), first_destination->view());
+    const iom::oid second = queue->copy(source->view(), second_destination->view());
+    source.reset();
+    auto fresh = device->create_tensor(spec);       // zero-filled at creation, wherever it lands
+    CHECK_NOTHROW(queue->wait(first));
+    CHECK_NOTHROW(queue->wait(second));
+    CHECK(raw_storage(oracle, spec, first_destination->view()) == expected);
+    CHECK(raw_storage(oracle, spec, second_destination->view()) == expected);
+}
+
+TEST_CASE("MI355X backend: operands of work nobody waited for are quarantined once their queue is gone") {
+    const iom::TensorSpec spec{iom::TensorShape{{4096, 2048}}, iom::DataType::F32};
+    const auto device = make_candidate();
+    auto source = device->create_tensor(spec);
+    auto destination = device->create_tensor(spec);
+    {
+        auto queue = device->create_ops();
+        CHECK(iom::oid_is_token(queue->copy(source->view(), destination->view())));
+    }
+    const void* was_source = source->view().native_handle();
+    const void* was_destination = destination->view().native_handle();
+    source.reset();
+    destination.reset();
+    expect_not_recycled(*device, {spec, spec}, {was_source, was_destination});
+}
+
+TEST_CASE("MI355X backend: cache append failures retire, a new queue appends correctly, pending operands are quarantined") {
+    const auto device = make_candidate();
+    struct Shape { std::vector<std::size_t> source, destination; std::size_t position; seams::SubmissionFault fault; };
+    const Shape shapes[] = {
+            {{1, 1, 1, 17}, {1, 1, 17, 17}, 1, seams::SubmissionFault::event_record},
+            {{2, 1, 1, 33}, {2, 1, 33, 33}, 15, seams::SubmissionFault::kernel_launch}};
+    std::uint64_t salt = 0x7c0;
+    for (const Shape& shape : shapes) {
+        const iom::TensorSpec source_spec{iom::TensorShape{shape.source}, iom::DataType::F32};
+        const iom::TensorSpec destination_spec{iom::TensorShape{shape.destination}, iom::DataType::F32};
+        auto source = device->create_tensor(source_spec);
+        auto destination = device->create_tensor(destination_spec);
+        const std::vector<std::byte> row = conf::encode_cache_append_logical(source_spec, ++salt);
+        conf::copy_from_host(source->view(), row);
+        conf::copy_from_host(destination->view(), conf::encode_logical(destination_spec, ++salt));
+        auto queue = device->create_ops();
+        arm(shape.fault);
+        const iom::oid failed = queue->cache_append(source->view(), destination->view(), shape.position);
+        disarm();
+        REQUIRE(iom::oid_is_token(failed));
+        conf::expect_repeated_runtime_failure(*queue, failed);
+
+        auto other_destination = device->create_tensor(destination_spec);
+        const std::vector<std::byte> before = conf::encode_logical(destination_spec, ++salt);
+        conf::copy_from_host(other_destination->view(), before);
+        auto other_queue = device->create_ops();
+        const iom::oid appended = other_queue->cache_append(source->view(), other_destination->view(), shape.position);
+        REQUIRE(iom::oid_is_token(appended));
+        CHECK_NOTHROW(other_queue->wait(appended));
+        CHECK_NOTHROW(other_queue->wait(appended));
+        conf::require_logical_bytes(
+                other_destination->view(),
+                conf::cache_append_expected_logical(source_spec, destination_spec, shape.position, row, before),
+                "append on a new queue after a retired failure");
+    }
+    // appends pending (one of them failed) when the queue goes: their operands do not come back
+    {
+        const iom::TensorSpec source_spec{iom::TensorShape{{3, 16, 16}}, iom::DataType::U8};
+        const iom::TensorSpec destination_spec{iom::TensorShape{{3, 64, 16}}, iom::DataType::U8};
+        auto source = device->create_tensor(source_spec);
+        auto destination = device->create_tensor(destination_spec);
+        conf::copy_from_host(source->view(), conf::encode_cache_append_logical(source_spec, ++salt));
+        conf::copy_from_host(destination->view(), conf::encode_logical(destination_spec, ++salt));
+        const void* was_source = source->view().native_handle();
+        const void* was_destination = destination->view().native_handle();
+        {
+            auto queue = device->create_ops();
+            for (int i = 0; i < 4; ++i) {
+                CHECK(iom::oid_is_token(queue->cache_append(source->view(), destination->view(), 1)));
+            }
+            arm(seams::SubmissionFault::kernel_launch);
+            CHECK(iom::oid_is_token(queue->cache_append(source->view(), destination->view(), 1)));
+        }
+        disarm();
+        source.reset();
+        destination.reset();
+        expect_not_recycled(*device, {source_spec, destination_spec}, {was_source, was_destination});
+    }
+    // a large source destroyed right after submission is still what gets appended
+    {
+        const iom::TensorSpec source_spec{iom::TensorShape{{32, 1, 8192, 128}}, iom::DataType::U8};
+        const iom::TensorSpec destination_spec{iom::TensorShape{{32, 1, 16384, 128}}, iom::DataType::U8};
+        auto source = device->create_tensor(source_spec);
+        auto destination = device->create_tensor(destination_spec);
+        const std::vector<std::byte> rows = conf::encode_cache_append_logical(source_spec, ++salt);
+        const std::vector<std::byte> before = conf::encode_logical(destination_spec, ++salt);
+        conf::copy_from_host(source->view(), rows);
+        conf::copy_from_host(destination->view(), before);
+        auto queue = device->create_ops();
+        const iom::oid token = queue->cache_append(source->view(), destination->view(), 17);
+        REQUIRE(iom::oid_is_token(token));
+        source.reset();
+        auto intruder = device->create_tensor(source_spec);
+        conf::copy_from_host(intruder->view(), conf::encode_cache_append_logical(source_spec, ++salt));
+        CHECK_NOTHROW(queue->wait(token));
+        conf::require_logical_bytes(
+                destination->view(),
+                conf::cache_append_expected_logical(source_spec, destination_spec, 17, rows, before),
+                "append whose source owner went away before the wait");
+    }
+}
+
+TEST_CASE("MI355X backend: an embedding whose status word cannot be fetched retires as failed and the queue goes on") {
+    const auto device = make_candidate();
+    const iom::TensorSpec table_spec{iom::TensorShape{{4, 8}}, iom::DataType::U8};
+    const iom::TensorSpec index_spec{iom::TensorShape{{1, 8}}, iom::DataType::U32};
+    const iom::TensorSpec output_spec{iom::TensorShape{{8, 8}}, iom::DataType::U8};
+    auto table = device->create_tensor(table_spec);
+    auto indices = device->create_tensor(index_spec);
+    auto output = device->create_tensor(output_spec);
+    conf::copy_from_host(table->view(), std::vector<std::byte>(table_spec.logical_nbytes()));
+    conf::copy_from_host(indices->view(), std::vector<std::byte>(index_spec.logical_nbytes()));
+    auto workspace = device->create_workspace(32);
+    auto queue = device->create_ops();
+    for (const seams::SubmissionFault fault :
+         {seams::SubmissionFault::embedding_status_copy, seams::SubmissionFault::kernel_launch}) {
+        arm(fault);
+        const iom::oid failed = queue->embedding(table->view(), indices->view(), output->view(), workspace->view());
+        disarm();
+        REQUIRE(iom::oid_is_token(failed));
+        conf::expect_repeated_runtime_failure(*queue, failed);
+        const iom::oid next = queue->embedding(table->view(), indices->view(), output->view(), workspace->view());
+        REQUIRE(iom::oid_is_token(next));
+        CHECK_NOTHROW(queue->wait(next));
+    }
+}
+
+TEST_CASE("MI355X backend: SiLU launch evidence, accepted failure, recovery, and quarantine after an unrecorded completion") {
+    const auto device = make_candidate();
+    {
+        const conf::SiluReferenceCase fixture = conf::silu_make_pattern_case(
+                conf::SiluReferenceCaseKind::ordinary, iom::DataType::F32, {2}, 2, 17, "mi355x-failure/F32");
+        const iom::TensorSpec spec = conf::silu_case_spec(fixture);
+        auto input = device->create_tensor(spec);
+        auto output = device->create_tensor(spec);
+        const std::vector<std::byte> input_bytes = conf::silu_pack_bits(iom::DataType::F32, fixture.input_bits);
+        conf::copy_from_host(input->view(), input_bytes);
+        conf::copy_from_host(output->view(), std::vector<std::byte>(spec.logical_nbytes(), conf::kReadbackSentinel));
+        const std::vector<conf::SiluReferenceValue> expected = conf::silu_evaluate(fixture);
+        auto queue = device->create_ops();
+        const std::size_t launches = seams::silu_launch_count_for_testing.load();
+        const iom::oid healthy = queue->silu(input->view(), output->view());
+        REQUIRE(iom::oid_is_token(healthy));
+        CHECK_NOTHROW(queue->wait(healthy));
+        CHECK_EQ(seams::silu_launch_count_for_testing.load(), launches + 1);
+        // the fault is consumed before the launch: accepted, failed, and no kernel ran
+        arm(seams::SubmissionFault::silu_launch);
+        const iom::oid failed = queue->silu(input->view(), output->view());
+        disarm();
+        REQUIRE(iom::oid_is_token(failed));
+        CHECK_EQ(conf::token_sequence(failed), conf::token_sequence(healthy) + 1);
+        conf::expect_repeated_runtime_failure(*queue, failed);
+        CHECK_EQ(seams::silu_launch_count_for_testing.load(), launches + 1);
+        const iom::oid again = queue->silu(input->view(), output->view());
+        REQUIRE(iom::oid_is_token(again));
+        CHECK_EQ(conf::token_sequence(again), conf::token_sequence(failed) + 1);
+        CHECK_NOTHROW(queue->wait(again));
+        CHECK_NOTHROW(queue->wait(again));
+        CHECK_EQ(seams::silu_launch_count_for_testing.load(), launches + 2);
+        const std::string mismatch = conf::silu_compare(
+                iom::DataType::F32, conf::read_logical(output->view()), expected, "activation after the failure");
+        CHECK_MESSAGE(mismatch.empty(), mismatch);
+        conf::require_logical_bytes(input->view(), input_bytes, "input after the failure");
+    }
+    {
+        // the completion event cannot be recorded: the operands stay out of the arena, and fresh
+        // operands on a fresh queue give the reference activation
+        const conf::SiluReferenceCase fixture = conf::silu_make_pattern_case(
+                conf::SiluReferenceCaseKind::boundary_sizes, iom::DataType::BF16, {2}, 17, 17, "mi355x-unrecorded/BF16");
+        const iom::TensorSpec spec = conf::silu_case_spec(fixture);
+        const std::vector<std::byte> input_bytes = conf::silu_pack_bits(iom::DataType::BF16, fixture.input_bits);
+        const std::vector<conf::SiluReferenceValue> expected = conf::silu_evaluate(fixture);
+        auto input = device->create_tensor(spec);
+        auto output = device->create_tensor(spec);
+        conf::copy_from_host(input->view(), input_bytes);
+        const void* was_input = input->view().native_handle();
+        const void* was_output = output->view().native_handle();
+        {
+            auto queue = device->create_ops();
+            arm(seams::SubmissionFault::event_record);
+            const iom::oid failed = queue->silu(input->view(), output->view());
+            disarm();
+            REQUIRE(iom::oid_is_token(failed));
+            conf::expect_repeated_runtime_failure(*queue, failed);
+        }
+        input.reset();
+        output.reset();
+        auto fresh_input = device->create_tensor(spec);
+        auto fresh_output = device->create_tensor(spec);
+        for (const void* retired : {was_input, was_output}) {
+            CHECK_NE(static_cast<const void*>(fresh_input->view().native_handle()), retired);
+            CHECK_NE(static_cast<const void*>(fresh_output->view().native_handle()), retired);
+        }
+        conf::copy_from_host(fresh_input->view(), input_bytes);
+        conf::copy_from_host(fresh_output->view(),
+                             std::vector<std::byte>(spec.logical_nbytes(), conf::kReadbackSentinel));
+        auto queue = device->create_ops();
+        const iom::oid token = queue->silu(fresh_input->view(), fresh_output->view());
+        REQUIRE(iom::oid_is_token(token));
+        CHECK_NOTHROW(queue->wait(token));
+        const std::string mismatch = conf::silu_compare(
+                iom::DataType::BF16, conf::read_logical(fresh_output->view()), expected, "activation on fresh operands");
+        CHECK_MESSAGE(mismatch.empty(), mismatch);
+    }
+}
+
+TEST_CASE("MI355X backend: TinyLlama-shaped attention, prefill of 17 rows and the decode step that follows it") {
+    Fixture f;
+    RawStorageOracle native_storage;
+    const conf::SdpaConformanceConfig config{
+            f.devices(), conf::kSdpaCurrentSupportedDataTypes, true, &f.gate, &native_storage, {}, {}};
+    const conf::SdpaReferenceCase prefill = conf::sdpa_oracle::make_exact_capacity_case(iom::DataType::BF16);
+    const conf::SdpaReferenceCase decode = conf::sdpa_incremental_slice(prefill, prefill.rows - 1);
+    REQUIRE_EQ(prefill.rows, std::size_t{17});
+    REQUIRE_EQ(decode.rows, std::size_t{1});
+    (void)conf::sdpa_detail::run_reference_case(config, prefill, "prefill of 17 rows");
+    (void)conf::sdpa_detail::run_reference_case(config, decode, "decode step");
+    CHECK_FALSE(f.gate.armed());
+}
+
+TEST_CASE("MI355X backend: workspaces are ranges of the one arena, and requirement queries are pure") {
+    const std::size_t allocations = seams::device_allocation_count_for_testing.load();
+    const auto device = iom::make_rocm_device(0, iom::DeviceMemoryConfig{1u * 1024 * 1024});
+    CHECK_EQ(seams::device_allocation_count_for_testing.load(), allocations + 1);     // the arena itself
+    auto empty = device->create_workspace(0);
+    REQUIRE(empty != nullptr);
+    CHECK(empty->empty());
+    CHECK_EQ(empty->byte_size(), std::size_t{0});
+    CHECK(empty->view().owner_identity() == empty.get());
+    CHECK(&empty->view().device() == device.get());
+    auto workspace = device->create_workspace(4096);
+    REQUIRE(workspace != nullptr);
+    const iom::RawWorkspaceView view = workspace->view();
+    CHECK_EQ(view.byte_size(), std::size_t{4096});
+    CHECK(view.owner_identity() == workspace.get());
+    CHECK_NOTHROW((void)iom::detail::WorkspaceValidation::validated(*device, view, 4096, 32, {}));
+    auto another = device->create_workspace(256);
+    REQUIRE(another != nullptr);
+    CHECK(workspace->view() == view);                                                 // stable
+    CHECK_THROWS_AS((void)device->create_workspace(2u * 1024 * 1024), std::bad_alloc);
+    another.reset();
+    auto reused = device->create_workspace(256);
+    REQUIRE(reused != nullptr);
+    CHECK_EQ(reused->byte_size(), std::size_t{256});
+    CHECK_EQ(seams::device_allocation_count_for_testing.load(), allocations + 1);     // nothing since
+
+    // queries: no workspace for the binary operations, the staged logical bytes for host transfers
+    Fixture f;
+    const iom::TensorSpec spec{iom::TensorShape{{2, 3, 17, 33}}, iom::DataType::F32};
+    auto lhs = f.candidate->create_tensor(spec);
+    auto rhs = f.candidate->create_tensor(spec);
+    auto out = f.candidate->create_tensor(spec);
+    auto queue = f.candidate->create_ops();
+    const iom::WorkspaceRequirements none{0, 1};
+    for (int repeat = 0; repeat < 2; ++repeat) {
+        CHECK(queue->add_workspace_requirements(lhs->view(), rhs->view(), out->view()) == none);
+        CHECK(queue->mul_workspace_requirements(lhs->view(), rhs->view(), out->view()) == none);
+        CHECK(queue->sub_workspace_requirements(lhs->view(), rhs->view(), out->view()) == none);
+        CHECK(queue->div_workspace_requirements(lhs->view(), rhs->view(), out->view()) == none);
+    }
+    const iom::WorkspaceRequirements staged{iom::gpu_algorithm::compute_staging_size(spec.logical_nbytes()), 32};
+    CHECK(lhs->view().copy_from_host_workspace_requirements() == staged);
+    CHECK(lhs->view().copy_to_host_workspace_requirements() == staged);
+    auto foreign_tensor = f.reference->create_tensor(spec);
+    CHECK_THROWS_AS((void)queue->add_workspace_requirements(foreign_tensor->view(), rhs->view(), out->view()),
+                    std::invalid_argument);
+}
+
 int main(int argc, char** argv) {
     int devices = 0;
     if (iomx_device_count(&devices) != IOMX_OK || devices < 1) {

@@ -44,6 +44,33 @@ SCENARIOS = {
     "MI355X: full shared suite with the RoPE contract": "run_backend_conformance",
 }
 
+# behaviours the reference's own accelerator driver asserts through backend seams
+# (test/rocm/test_rocm_conformance.cpp:374-540, 798-838, 1242-1288, 1366-1492, 1906-2221, 2314-2407),
+# asked of this backend through its seams with the reference's shared helpers for data and values
+BACKEND_CASES = {
+    "MI355X backend: a launch that fails after acceptance repeats its failure and the owners serve the next one":
+        "ROCm ADD retained launch failure keeps owners reusable",
+    "MI355X backend: only accepted submissions take a sequence, and a failed one's operands are not recycled":
+        "ROCm submission remains transactional across post-enqueue failures",
+    "MI355X backend: queue destruction drains pending copies around a failed one":
+        "ROCm queue destruction fences pending copies",
+    "MI355X backend: a source destroyed before the wait stays intact until both of its copies are done":
+        "ROCm pre-wait source destruction / shared-operand copies",
+    "MI355X backend: operands of work nobody waited for are quarantined once their queue is gone":
+        "ROCm operands destroyed after queue teardown remain quarantined",
+    "MI355X backend: cache append failures retire, a new queue appends correctly, pending operands are quarantined":
+        "ROCm cache append retained event / launch failure, queue teardown, source retention",
+    "MI355X backend: an embedding whose status word cannot be fetched retires as failed and the queue goes on":
+        "ROCm embedding status transfer failure retires safely",
+    "MI355X backend: SiLU launch evidence, accepted failure, recovery, and quarantine after an unrecorded completion":
+        "ROCm SiLU accepted native failure / failed drain",
+    "MI355X backend: TinyLlama-shaped attention, prefill of 17 rows and the decode step that follows it":
+        "ROCm TinyLlama SDPA native QK/PV decode and prefill",
+    "MI355X backend: workspaces are ranges of the one arena, and requirement queries are pure":
+        "ROCm raw workspace suballocates the arena / workspace requirement queries",
+}
+SCENARIOS.update(BACKEND_CASES)
+
 CASE_LINE = re.compile(r"^\[ (?: ok |FAIL) \] (.*): (\d+) assertions, (\d+) failed$")
 DONE_LINE = re.compile(r"^\[ done \] (\d+) cases, (\d+) failed; (\d+) assertions, (\d+) failed$")
 
