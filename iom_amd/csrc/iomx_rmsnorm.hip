@@ -371,6 +371,10 @@ bool band_kernel_serves(uint32_t n, uint32_t total_bands) {
     return total_bands <= 0x7FFFFFFFu / 8 && n <= (wide ? 131072u : 65536u);
 }
 
+// (The fused add + norm takes the shape the norm alone takes: the order in which a row's squares
+// are summed follows from K, S and the lanes, and the fused result is to be the two launches'
+// result bit for bit.  Two chunks per lane on 1024 lanes would be 2 % faster for the fused kernel
+// at [32768,2048] BF16, 94.2 against 95.8 us.)
 template <int DT, bool ADD>
 void launch_resident(const RmsArgsT<ADD ? 4 : 2>& a, hipStream_t s) {
     const uint32_t n = a.band_chunks;
@@ -380,12 +384,7 @@ void launch_resident(const RmsArgsT<ADD ? 4 : 2>& a, hipStream_t s) {
     else if (n <= 512) launch_band<DT, 2, 1, 256, ADD>(a, s);
     else if (n <= 1024) launch_band<DT, 2, 1, 512, ADD>(a, s);
     else if (n <= 2048) launch_band<DT, 4, 1, 512, ADD>(a, s);
-    else if (n <= 4096) {
-        // with the add in front a lane has two operands in flight per chunk: two chunks per lane
-        // on 1024 lanes then do 2 % better than four on 512 (BF16 [32768,2048]: 94.2 against 95.8 us)
-        if constexpr (ADD) launch_band<DT, 2, 2, 1024, ADD>(a, s);
-        else launch_band<DT, 4, 2, 512, ADD>(a, s);
-    }
+    else if (n <= 4096) launch_band<DT, 4, 2, 512, ADD>(a, s);
     else if (n <= 8192) launch_band<DT, 4, 2, 1024, ADD>(a, s);
     else if (n == 16384) launch_band<DT, 4, 4, 1024, ADD>(a, s);
     else if (n <= 16384) launch_band<DT, 8, 2, 1024, ADD>(a, s);
