@@ -56,9 +56,11 @@ constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
 // Subnormal operands of the matrix stages become zeros of the same sign
 // (src/cpu/sdpa.cpp:57-60), two BF16 per word.
 __device__ __forceinline__ uint32_t daz2(uint32_t w) {
-    const uint32_t lo = (w & 0x00007F80u) ? 0x0000FFFFu : 0x00008000u;
-    const uint32_t hi = (w & 0x7F800000u) ? 0xFFFF0000u : 0x80000000u;
-    return w & (lo | hi);
+    // bit 15 of a half of `normal` is set where that half's exponent field is not zero (the field
+    // sits in bits 7..14, so adding 0x7FFF carries into bit 15 exactly then and never past it)
+    const uint32_t normal = ((w & 0x7F807F80u) + 0x7FFF7FFFu) & 0x80008000u;
+    // 0x7FFF under every such bit, and the sign bits always
+    return w & ((normal - (normal >> 15)) | 0x80008000u);
 }
 __device__ __forceinline__ bf16x8_t daz8(u32x4 v) {
     return __builtin_bit_cast(bf16x8_t, u32x4{daz2(v[0]), daz2(v[1]), daz2(v[2]), daz2(v[3])});
@@ -81,6 +83,12 @@ __device__ __forceinline__ u32x4 lds_read_b128(uint32_t address) {
     return value;
 }
 __device__ __forceinline__ void lds_reads_landed() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// one 32-bit word, waited for
+__device__ __forceinline__ uint32_t lds_read_b32(uint32_t address) {
+    uint32_t value;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(value) : "v"(address) : "memory");
+    return value;
+}
 
 // One workgroup packs a share of the fragments of one KV head of one plane and writes
 // that share's flag word (every word is written on every call, so the workspace needs
@@ -277,11 +285,15 @@ __device__ __forceinline__ void sdpa_reference_row(const SdpaArgs& a, uint32_t p
 }
 
 // KV heads of plane p whose V prefix holds an infinity or NaN (any share's flag up)
-__device__ __forceinline__ bool sdpa_flag_up(const SdpaArgs& a, uint32_t p, uint32_t hkv) {
-    uint32_t up = 0;
+// The flag words of one (plane, KV head), a word per lane (there are 64 pack splits at most), as one
+// vector load that stays in flight with whatever the caller requests next; any lane's result
+// non-zero = the flag is up.  (Read one after the other through the scalar cache they were a chain
+// of up to 64 dependent loads at the head of every workgroup.)
+__device__ __forceinline__ uint32_t sdpa_flag_words(const SdpaArgs& a, uint32_t p, uint32_t hkv, uint32_t lane) {
     const uint64_t pair = (uint64_t)p * a.Hkv + hkv;
-    for (uint32_t i = 0; i < a.pack_splits; ++i) up |= a.flags[pair * a.pack_splits + i];
-    return up != 0;                       // uniform: every lane reads the same words
+    uint32_t up = 0;
+    for (uint32_t i = lane; i < a.pack_splits; i += 64) up |= a.flags[pair * a.pack_splits + i];
+    return up;
 }
 
 // MODE 0: a workgroup of four waves = four heads of one row tile, each wave walks
@@ -372,11 +384,18 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t kv_ring[SHARE ? 3 * kStage : 16];
     constexpr int NW = sdpa_waves(DT16, MODE);
     constexpr int D32 = (DT16 + 1) / 2;
+    // FULLD: D is a multiple of 32, i.e. exactly DT16 whole tiles -- a constant to the compiler
+    const uint32_t head_dim = FULLD ? (uint32_t)DT16 * kTile : a.D;
+    const uint32_t d_tiles = FULLD ? (uint32_t)DT16 : a.d_tiles;
     constexpr float kLog2e = 1.44269504088896340736f;
     // stands in for a maximum of -infinity (nothing seen yet) in exponent arguments
     constexpr float kFloor = -1.0e30f;
     __shared__ float wave_stats[NW][16][5];
     __shared__ f32x4_t wave_out[SPLIT ? NW - 1 : 1][SPLIT ? DT16 : 1][64];
+    // raised by a wave whose rows need the passes of the special rows (the waves that share a ring
+    // decide together); cleared here, and the barriers of pass 1 lie between this and its first use
+    __shared__ uint32_t special_rows;
+    if (SHARE && threadIdx.x == 0) special_rows = 0;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
@@ -411,24 +430,16 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     // lane offset of the body alive across it, far beyond the register file)
     {
         const uint32_t p = a.plane0 + blockIdx.y;
-        if (sdpa_flag_up(a, p, hkv)) {
-            // V of this KV head holds an infinity or NaN.  A masked probability is +0, and on the
-            // matrix cores +0 times an infinite V of a token the row must not see would poison
-            // the row: these rows are formed in the reference's order instead.  (All waves of a
-            // workgroup that meets at barriers share the KV head and leave together.)
-            float* pbuf = &wave_stats[wave][0][0];
-            for (uint32_t r = SPLIT ? wave : 0; r < kTile; r += SPLIT ? NW : 1)
-                if (first_row + r < a.R) sdpa_reference_row(a, p, hkv, head, first_row + r, lane, pbuf);
-            return;
-        }
+        // requested now, looked at once Q and the first K groups are on their way too
+        const uint32_t flag_words = sdpa_flag_words(a, p, hkv, lane);
         uint64_t plane[4];
         walk_planes(a.walk, p, plane);
         const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
         // wave-uniform bases and 32-bit lane offsets: the packed region of one KV head is far
         // below 4 GiB, and 64-bit addresses per load would cost the registers of a whole wave slot
-        const uint8_t* vf = a.packed_v + (((uint64_t)p * a.Hkv + hkv) * a.groups) * a.d_tiles * kFrag;
+        const uint8_t* vf = a.packed_v + (((uint64_t)p * a.Hkv + hkv) * a.groups) * d_tiles * kFrag;
         const uint32_t vf_lane = lane * 16;
-        const uint8_t* kp = a.packed_k + (((uint64_t)p * a.Hkv + hkv) * a.groups * 2) * a.d_tiles * kTileBytes;
+        const uint8_t* kp = a.packed_k + (((uint64_t)p * a.Hkv + hkv) * a.groups * 2) * d_tiles * kTileBytes;
         const uint32_t kp_lane = l16 * kRowBytes + c0 * 2;
         // One direct load of a wave's share of the K group (and of the V group) g into ring stage buf:
         // wave w brings in KiB chunks w, w+4, .. ; lane i fetches 16-byte piece i of a chunk, and the
@@ -454,15 +465,30 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             issue(std::false_type{}, 1, 1);
         }
         // the row tile of Q, flushed, as the B operand of every score tile
-        bf16x8_t qf[D32];
+        u32x4 q_bits[D32];
 #pragma unroll
         for (int c = 0; c < D32; ++c) {
             const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
-            qf[c] = __builtin_bit_cast(bf16x8_t, u32x4{0, 0, 0, 0});
+            q_bits[c] = u32x4{0, 0, 0, 0};
             if (FULLD || i0 < a.D)
-                qf[c] = daz8(load_k8_bits(qb + ((uint64_t)(qrow >> 4) * a.d_tiles + tile) * kTileBytes
-                                                  + (qrow & 15u) * kRowBytes, c0, i0, a.D));
+                q_bits[c] = load_k8_bits(qb + ((uint64_t)(qrow >> 4) * d_tiles + tile) * kTileBytes
+                                            + (qrow & 15u) * kRowBytes, c0, i0, head_dim);
         }
+        if (__any(flag_words != 0)) {
+            // V of this KV head holds an infinity or NaN.  A masked probability is +0, and on the
+            // matrix cores +0 times an infinite V of a token the row must not see would poison
+            // the row: these rows are formed in the reference's order instead.  (All waves of a
+            // workgroup that meets at barriers share the KV head and leave together; the K groups
+            // requested above land in the ring, which nothing reads on this path.)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            float* pbuf = &wave_stats[wave][0][0];
+            for (uint32_t r = SPLIT ? wave : 0; r < kTile; r += SPLIT ? NW : 1)
+                if (first_row + r < a.R) sdpa_reference_row(a, p, hkv, head, first_row + r, lane, pbuf);
+            return;
+        }
+        bf16x8_t qf[D32];
+#pragma unroll
+        for (int c = 0; c < D32; ++c) qf[c] = daz8(q_bits[c]);
         // K of the 32 tokens of group g, from the flushed copy: two 16-token tiles, lane
         // (token l16, features 8*kg..); tokens past the prefix and columns past D are zeros there
         struct KGroup { u32x4 w[2][D32]; };
@@ -475,14 +501,17 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                     kgp.w[half][c] = u32x4{0, 0, 0, 0};
                     if (FULLD || i0 < a.D)
                         kgp.w[half][c] = *reinterpret_cast<const u32x4*>(
-                                kp + (((2 * g + half) * a.d_tiles + tile) * kTileBytes + kp_lane));
+                                kp + (((2 * g + half) * d_tiles + tile) * kTileBytes + kp_lane));
                 }
         };
         // scores: lane gets tokens 32g + 16*half + 4*kg + j (j < 4) of row l16.  `bare` (plain
         // passes, sqrt(D) a power of two): the dot products themselves -- the division is exact
         // there, so the passes fold it into the constant of their exponent argument and get the
         // same bits with one multiplication less per score.
-        auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2], bool bare) {
+        // `checked` (the passes of the special rows): an infinite dot product stays infinite.  The
+        // plain passes leave that select out: the remainder of an infinite quotient is NaN, the NaN
+        // reaches the row's sum, and the tile repeats with the special rows' passes.
+        auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2], bool bare, bool checked) {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -501,7 +530,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float refined = __builtin_fmaf(__builtin_fmaf(-q[j], a.scale, acc[j]), a.inv_scale, q[j]);
-                        q[j] = __builtin_fabsf(q[j]) < __builtin_inff() ? refined : q[j];   // inf - inf is not a remainder
+                        q[j] = !checked || __builtin_fabsf(q[j]) < __builtin_inff() ? refined : q[j];   // inf - inf is not a remainder
                     }
                 }
                 s[half] = q;
@@ -510,7 +539,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         // the visible groups of this wave, K one group ahead where the mode says so; WITH_V: the
         // V fragments of the group are requested before its scores are formed
         // `primed`: the first two stages of the ring have been requested already
-        auto walk_groups = [&](auto with_v, bool bare, bool primed, auto&& body) {
+        auto walk_groups = [&](auto with_v, bool bare, bool checked, bool primed, auto&& body) {
             constexpr bool WITH_V = decltype(with_v)::value;
             if constexpr (SHARE) {
                 constexpr int LPS = (WITH_V ? 2 : 1) * (DT16 / 4);        // direct loads per wave and stage
@@ -558,7 +587,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                         for (int dt = 0; dt < DT16; ++dt) asm volatile("" : "+v"(vfr[dt]));
                     }
                     f32x4_t s[2];
-                    scores(cur, s, bare);
+                    scores(cur, s, bare, checked);
                     body(g, s, vfr);
                 }
                 // nothing in flight and nobody reading when the next pass (or the next workgroup)
@@ -577,10 +606,10 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 if constexpr (WITH_V) {
 #pragma unroll
                     for (int dt = 0; dt < DT16; ++dt)
-                        vfr[dt] = *reinterpret_cast<const u32x4*>(vf + ((g * a.d_tiles + dt) * kFrag + vf_lane));
+                        vfr[dt] = *reinterpret_cast<const u32x4*>(vf + ((g * d_tiles + dt) * kFrag + vf_lane));
                 }
                 f32x4_t s[2];
-                scores(cur, s, bare);
+                scores(cur, s, bare, checked);
                 body(g, s, vfr);
                 if (AHEAD) cur = nxt;
             }
@@ -616,7 +645,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 
         // ---- plain pass 1: running maximum and sum of exp(score - maximum)
         float pm = -inf, psum = 0.0f;
-        walk_groups(std::false_type{}, bare, true, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+        walk_groups(std::false_type{}, bare, false, true, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
             if (g >= full_groups) mask_group(g, s);
             // (the maximum instruction itself: a NaN among its operands is passed over, and the
             // row's sum below turns NaN from that score's exponential all the same)
@@ -631,6 +660,14 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 for (int j = 0; j < 4; ++j) psum += __builtin_amdgcn_exp2f(__builtin_fmaf(s[half][j], kls, nb));
             pm = newm;
         });
+        // the first two groups of pass 2 (K and V) are on their way while the statistics are
+        // joined: the ring is free (pass 1 ended at a barrier with nothing in flight).  Should the
+        // tile turn out to need the special rows' passes, those request their own first groups
+        // over these: the same K bytes into the same places.
+        if (SHARE && ring_groups != 0) {
+            issue(std::true_type{}, 0, 0);
+            issue(std::true_type{}, 1, 1);
+        }
 #pragma unroll
         for (int off = 16; off <= 32; off *= 2) {
             const float m2 = __shfl_xor(pm, off), s2 = __shfl_xor(psum, off);
@@ -651,7 +688,15 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         // workgroup holds the same joined values and decides alike
         const bool odd = !ghost && !(psum > 0.0f && psum < inf && pm < inf);
         // (sharing the groups, the four waves also share the decision: they meet at barriers)
-        const bool plain = SHARE ? !__syncthreads_or(odd ? 1 : 0) : !__any(odd);
+        bool plain = !__any(odd);
+        if constexpr (SHARE) {
+            // (a bare barrier and a read the compiler does not see as one: a fence here, or an LDS
+            // read it knows of, would first wait for the groups of pass 2 requested above)
+            if (!plain && lane == 0) special_rows = 1;
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            plain = __builtin_amdgcn_readfirstlane(lds_read_b32(lds_address(&special_rows))) == 0;
+        }
 
         f32x4_t o[DT16];
 #pragma unroll
@@ -660,7 +705,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         if (plain) {
             // ---- plain pass 2: probabilities, rounded once to BF16 and flushed, times V
             const float inv_sum = 1.0f / psum, nb = -pm * kls;
-            walk_groups(std::true_type{}, bare, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+            walk_groups(std::true_type{}, bare, false, SHARE, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
                 if (g >= full_groups) mask_group(g, s);
                 float e[8];
 #pragma unroll
@@ -674,7 +719,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         } else {
             // ---- pass 1 with the bookkeeping of the special rows
             RowStats st = {-inf, 0.0f, 0u, false, false};
-            walk_groups(std::false_type{}, false, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+            walk_groups(std::false_type{}, false, true, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
                 // the finite maximum of the lane's eight scores first, then one rescale; written
                 // with selects only (a branch per element would cost more than the arithmetic)
                 float local = -inf;
@@ -727,7 +772,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
             const float inv_sum = 1.0f / st.sum;
             // ---- pass 2 of the special rows
-            walk_groups(std::true_type{}, false, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+            walk_groups(std::true_type{}, false, true, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
                 float pr[8];
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
@@ -762,6 +807,17 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         if (!row_ok) return;
         uint8_t* ob = a.out + plane[3] * a.out_plane_bytes
                 + (uint64_t)(row >> 4) * a.out_tile_cols * kTileBytes + (row & 15u) * kRowBytes;
+        if (FULLD && plain) {
+            // whole tiles and no special row: a lane's four outputs of a tile are one 8-byte piece of
+            // tile head * DT16 + dt.  Adding +0 stores -0 as +0; the sums are no NaN here (finite V,
+            // probabilities that add up to about one).
+            uint8_t* ot = ob + (uint64_t)head * (DT16 * kTileBytes) + kg * 8;
+#pragma unroll
+            for (int dt = 0; dt < DT16; ++dt)
+                *reinterpret_cast<u32x2*>(ot + dt * kTileBytes) =
+                        u32x2{cvt_bf16x2(o[dt][0] + 0.0f, o[dt][1] + 0.0f), cvt_bf16x2(o[dt][2] + 0.0f, o[dt][3] + 0.0f)};
+            return;
+        }
 #pragma unroll
         for (int dt = 0; dt < DT16; ++dt) {
             float val[4];
@@ -770,10 +826,10 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 val[j] = o[dt][j];
                 if (val[j] == 0.0f) val[j] = 0.0f;                    // -0 is stored as +0
             }
-            const uint32_t d = dt * kTile + 4 * kg, col = head * a.D + d;
-            if ((a.D & 3u) == 0) {
+            const uint32_t d = dt * kTile + 4 * kg, col = head * head_dim + d;
+            if ((head_dim & 3u) == 0) {
                 // the four outputs lie in one tile row of out
-                if (d >= a.D) continue;
+                if (d >= head_dim) continue;
                 const u32x2 bits = nan_row ? u32x2{0x7FC07FC0u, 0x7FC07FC0u}
                                            : u32x2{pack_bf16(val[0], val[1]), pack_bf16(val[2], val[3])};
                 *reinterpret_cast<u32x2*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) = bits;
@@ -781,7 +837,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                if (d + j >= a.D) continue;
+                if (d + j >= head_dim) continue;
                 const uint32_t bits = nan_row ? 0x7FC0u : bf16_rne_sw(as_u32(val[j]));
                 const uint32_t cj = col + j;
                 *reinterpret_cast<uint16_t*>(ob + (uint64_t)(cj >> 4) * kTileBytes + (cj & 15u) * 2) = (uint16_t)bits;
