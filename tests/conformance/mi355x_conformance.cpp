@@ -14,6 +14,7 @@
 #include <doctest/doctest.h>
 
 #include <array>
+#include <cmath>
 #include <cstddef>
 #include <cstdint>
 #include <cstdlib>
@@ -731,6 +732,116 @@ TEST_CASE("MI355X backend: SiLU launch evidence, accepted failure, recovery, and
         const std::string mismatch = conf::silu_compare(
                 iom::DataType::BF16, conf::read_logical(fresh_output->view()), expected, "activation on fresh operands");
         CHECK_MESSAGE(mismatch.empty(), mismatch);
+    }
+}
+
+TEST_CASE("MI355X backend: SiLU submitted through views that die before the wait, input owner destroyed first") {
+    // the reference driver's scenario (test/rocm/test_rocm_conformance.cpp:1494-1572): both
+    // descriptors handed to silu() are temporaries of the submitting call, the input owner goes
+    // away before the token is observed, and the poisoned padding of the output owner survives
+    const auto device = make_candidate();
+    const iom::TensorSpec owner_spec = conf::silu_make_spec({3, 4, 2, 17}, iom::DataType::F16);
+    const conf::SiluReferenceCase fixture = conf::silu_make_pattern_case(
+            conf::SiluReferenceCaseKind::ordinary, iom::DataType::F16, {2, 2}, 2, 17, "mi355x-temporary/F16");
+    const iom::TensorSpec logical_spec = conf::silu_case_spec(fixture);
+    const std::vector<std::byte> input_logical = conf::silu_pack_bits(iom::DataType::F16, fixture.input_bits);
+    const std::vector<conf::SiluReferenceValue> expected = conf::silu_evaluate(fixture);
+    const std::vector<std::byte> poison(logical_spec.logical_nbytes(), conf::kReadbackSentinel);
+    auto input_owner = device->create_tensor(owner_spec);
+    auto output_owner = device->create_tensor(owner_spec);
+    RawStorageOracle storage;
+    {
+        iom::TensorView input_view = conf::silu_transformed_view(*input_owner);
+        iom::TensorView output_view = conf::silu_transformed_view(*output_owner);
+        REQUIRE(input_view.spec() == logical_spec);
+        REQUIRE(output_view.spec() == logical_spec);
+        storage.set_owner_spec(owner_spec);
+        storage.seed(input_view, conf::silu_storage_image(owner_spec, input_view, input_logical, std::byte{0x5A}));
+        storage.set_owner_spec(owner_spec);
+        storage.seed(output_view, conf::silu_storage_image(owner_spec, output_view, poison, std::byte{0xA5}));
+        auto queue = device->create_ops();
+        const auto submit = [&queue](iom::Tensor& input, iom::Tensor& output) {
+            const iom::TensorView in = conf::silu_transformed_view(input);
+            iom::TensorView out = conf::silu_transformed_view(output);
+            return queue->silu(in, out);
+        };
+        const iom::oid token = submit(*input_owner, *output_owner);
+        REQUIRE(iom::oid_is_token(token));
+        input_owner.reset();
+        CHECK_NOTHROW(queue->wait(token));
+        CHECK_NOTHROW(queue->wait(token));
+        const std::vector<std::byte> activated = conf::read_logical(output_view);
+        const std::string mismatch = conf::silu_compare(
+                iom::DataType::F16, activated, expected, "activation through temporary views");
+        CHECK_MESSAGE(mismatch.empty(), mismatch);
+        std::vector<std::byte> want(owner_spec.tiled_storage_nbytes(), std::byte{0xA5});
+        conf::apply_standard_tiled_view(output_view, owner_spec, activated, want);
+        storage.set_owner_spec(owner_spec);
+        CHECK(storage.observe(output_view) == want);
+    }
+    output_owner.reset();
+}
+
+TEST_CASE("MI355X backend: one SiLU kernel per accepted request of every floating leaf, none for a rejected one, negative subnormal tails kept") {
+    // test/rocm/test_rocm_conformance.cpp:1578-1676 against this backend's launch counter
+    const auto device = make_candidate();
+    auto queue = device->create_ops();
+    for (const iom::DataType type : conf::kSiluRocmExpectedSupported) {
+        CAPTURE(static_cast<int>(type));
+        const iom::TensorSpec spec = conf::silu_make_spec({2, 17, 17}, type);
+        auto input = device->create_tensor(spec);
+        auto output = device->create_tensor(spec);
+        const std::size_t before = seams::silu_launch_count_for_testing.load();
+        const iom::oid token = queue->silu(input->view(), output->view());
+        REQUIRE(iom::oid_is_token(token));
+        CHECK_NOTHROW(queue->wait(token));
+        CHECK_NOTHROW(queue->wait(token));
+        CHECK_EQ(seams::silu_launch_count_for_testing.load(), before + 1);
+    }
+    {
+        const iom::TensorSpec spec = conf::silu_make_spec({2, 17, 17}, iom::DataType::F32);
+        const iom::TensorSpec other = conf::silu_make_spec({2, 17, 18}, iom::DataType::F32);
+        auto input = device->create_tensor(spec);
+        auto output = device->create_tensor(other);
+        const std::size_t before = seams::silu_launch_count_for_testing.load();
+        CHECK_EQ(queue->silu(input->view(), output->view()), iom::to_oid(iom::OidError::InvalidArgument));
+        CHECK_EQ(seams::silu_launch_count_for_testing.load(), before);
+        CHECK_EQ(queue->silu(input->view(), input->view()), iom::to_oid(iom::OidError::InvalidArgument));
+        CHECK_EQ(seams::silu_launch_count_for_testing.load(), before);
+    }
+    for (const iom::DataType type : {iom::DataType::F32, iom::DataType::F64}) {
+        CAPTURE(static_cast<int>(type));
+        const conf::SiluReferenceCase tails = conf::silu_make_tail_case(type);
+        const iom::TensorSpec spec = conf::silu_case_spec(tails);
+        auto input = device->create_tensor(spec);
+        auto output = device->create_tensor(spec);
+        conf::copy_from_host(input->view(), conf::silu_pack_bits(type, tails.input_bits));
+        conf::copy_from_host(output->view(), std::vector<std::byte>(spec.logical_nbytes(), conf::kReadbackSentinel));
+        const iom::oid token = queue->silu(input->view(), output->view());
+        REQUIRE(iom::oid_is_token(token));
+        CHECK_NOTHROW(queue->wait(token));
+        const std::vector<std::byte> observed = conf::read_logical(output->view());
+        const std::vector<conf::SiluReferenceValue> expected = conf::silu_evaluate(tails);
+        const std::uint64_t tail_input =
+                conf::silu_oracle::value_bits(type, type == iom::DataType::F64 ? -746.0 : -104.0);
+        std::size_t seen = 0;
+        for (std::size_t i = 0; i < expected.size(); ++i) {
+            if (tails.input_bits[i] != tail_input) continue;
+            ++seen;
+            const std::uint64_t bits = conf::silu_read_bits(observed, type, i);
+            CHECK_EQ(bits, expected[i].bits);
+            // classified in the leaf's own domain: a binary32 subnormal widened to binary64 is normal
+            bool negative_subnormal = false;
+            if (type == iom::DataType::F64) {
+                const double v = conf::silu_oracle::decode_f64(bits);
+                negative_subnormal = std::fpclassify(v) == FP_SUBNORMAL && std::signbit(v);
+            } else {
+                const float v = conf::silu_oracle::decode_f32(type, bits);
+                negative_subnormal = std::fpclassify(v) == FP_SUBNORMAL && std::signbit(v);
+            }
+            CHECK_MESSAGE(negative_subnormal, "the tail must stay a nonzero negative subnormal");
+        }
+        CHECK(seen > 0);
     }
 }
 

@@ -64,6 +64,10 @@ BACKEND_CASES = {
         "ROCm embedding status transfer failure retires safely",
     "MI355X backend: SiLU launch evidence, accepted failure, recovery, and quarantine after an unrecorded completion":
         "ROCm SiLU accepted native failure / failed drain",
+    "MI355X backend: SiLU submitted through views that die before the wait, input owner destroyed first":
+        "ROCm SiLU retains snapshot and owners across temporary views",
+    "MI355X backend: one SiLU kernel per accepted request of every floating leaf, none for a rejected one, negative subnormal tails kept":
+        "ROCm SiLU native launch evidence and negative subnormal tails",
     "MI355X backend: TinyLlama-shaped attention, prefill of 17 rows and the decode step that follows it":
         "ROCm TinyLlama SDPA native QK/PV decode and prefill",
     "MI355X backend: workspaces are ranges of the one arena, and requirement queries are pure":
