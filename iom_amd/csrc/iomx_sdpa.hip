@@ -49,6 +49,7 @@ struct SdpaArgs {
     float scale;                // sqrtf(D)
     float inv_scale;            // 1 / scale, rounded
     uint32_t scale_pow2;        // scale is a power of two: the product with inv_scale is the quotient
+    float exp_scale;            // log2(e) / scale, rounded once: exp((dot - max) / scale) = 2^((dot - max) * exp_scale)
 };
 
 constexpr uint32_t kTileBytes = 512, kRowBytes = 32, kFrag = 1024;
@@ -504,14 +505,11 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                                 kp + (((2 * g + half) * d_tiles + tile) * kTileBytes + kp_lane));
                 }
         };
-        // scores: lane gets tokens 32g + 16*half + 4*kg + j (j < 4) of row l16.  `bare` (plain
-        // passes, sqrt(D) a power of two): the dot products themselves -- the division is exact
-        // there, so the passes fold it into the constant of their exponent argument and get the
-        // same bits with one multiplication less per score.
-        // `checked` (the passes of the special rows): an infinite dot product stays infinite.  The
-        // plain passes leave that select out: the remainder of an infinite quotient is NaN, the NaN
-        // reaches the row's sum, and the tile repeats with the special rows' passes.
-        auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2], bool bare, bool checked) {
+        // scores: lane gets tokens 32g + 16*half + 4*kg + j (j < 4) of row l16.  `bare` (the plain
+        // passes): the dot products themselves; the division by sqrt(D) is folded into the constant
+        // of the passes' exponent argument (see there).  Otherwise (the passes of the special rows,
+        // whose values are compared and counted as scores): dot / sqrt(D).
+        auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2], bool bare) {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -530,7 +528,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float refined = __builtin_fmaf(__builtin_fmaf(-q[j], a.scale, acc[j]), a.inv_scale, q[j]);
-                        q[j] = !checked || __builtin_fabsf(q[j]) < __builtin_inff() ? refined : q[j];   // inf - inf is not a remainder
+                        q[j] = __builtin_fabsf(q[j]) < __builtin_inff() ? refined : q[j];   // inf - inf is not a remainder
                     }
                 }
                 s[half] = q;
@@ -539,7 +537,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         // the visible groups of this wave, K one group ahead where the mode says so; WITH_V: the
         // V fragments of the group are requested before its scores are formed
         // `primed`: the first two stages of the ring have been requested already
-        auto walk_groups = [&](auto with_v, bool bare, bool checked, bool primed, auto&& body) {
+        auto walk_groups = [&](auto with_v, bool bare, bool primed, auto&& body) {
             constexpr bool WITH_V = decltype(with_v)::value;
             if constexpr (SHARE) {
                 constexpr int LPS = (WITH_V ? 2 : 1) * (DT16 / 4);        // direct loads per wave and stage
@@ -587,7 +585,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                         for (int dt = 0; dt < DT16; ++dt) asm volatile("" : "+v"(vfr[dt]));
                     }
                     f32x4_t s[2];
-                    scores(cur, s, bare, checked);
+                    scores(cur, s, bare);
                     body(g, s, vfr);
                 }
                 // nothing in flight and nobody reading when the next pass (or the next workgroup)
@@ -609,7 +607,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                         vfr[dt] = *reinterpret_cast<const u32x4*>(vf + ((g * d_tiles + dt) * kFrag + vf_lane));
                 }
                 f32x4_t s[2];
-                scores(cur, s, bare, checked);
+                scores(cur, s, bare);
                 body(g, s, vfr);
                 if (AHEAD) cur = nxt;
             }
@@ -622,13 +620,17 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) s[half][j] = 16 * half + j < rem ? s[half][j] : -inf;
         };
-        // The plain passes work on the dot products themselves where dividing by sqrt(D) is exact
-        // (a power of two): the division moves into the constant of the exponent argument,
-        // 2^(dot * (log2 e / sqrt(D)) - max * (log2 e / sqrt(D))), which is the same binary32 value as
-        // 2^((dot / sqrt(D)) * log2 e - ...) bit for bit, since scaling by a power of two commutes
-        // with rounding.  The running maximum is then a maximum of dot products.
-        const bool bare = a.scale_pow2 != 0;
-        const float kls = bare ? kLog2e * a.inv_scale : kLog2e;
+        // The plain passes work on the dot products themselves: the division by sqrt(D) moves into
+        // the constant of the exponent argument, 2^(dot * c - max * c) with c = log2(e) / sqrt(D)
+        // rounded once, and the running maximum is a maximum of dot products.  Where sqrt(D) is a
+        // power of two that is the same binary32 value as 2^((dot / sqrt(D)) * log2 e - ...) bit for
+        // bit (scaling by a power of two commutes with rounding); for the other head sizes the
+        // argument differs from the divided form's by a few units of its last place, which is the
+        // size of the rounding of dot / sqrt(D) itself and far inside the contract's allowance for
+        // a native kernel, and costs three vector instructions per score and pass less than a
+        // correctly rounded quotient.
+        constexpr bool bare = true;
+        const float kls = a.exp_scale;
         // (maximum, sum) of one part of a row joined with another part's
         auto join = [&](float& m, float& sum, float m2, float sum2) {
             const float mm = __builtin_fmaxf(m, m2), base = __builtin_fmaxf(mm, kFloor);
@@ -645,7 +647,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 
         // ---- plain pass 1: running maximum and sum of exp(score - maximum)
         float pm = -inf, psum = 0.0f;
-        walk_groups(std::false_type{}, bare, false, true, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+        walk_groups(std::false_type{}, bare, true, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
             if (g >= full_groups) mask_group(g, s);
             // (the maximum instruction itself: a NaN among its operands is passed over, and the
             // row's sum below turns NaN from that score's exponential all the same)
@@ -705,7 +707,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         if (plain) {
             // ---- plain pass 2: probabilities, rounded once to BF16 and flushed, times V
             const float inv_sum = 1.0f / psum, nb = -pm * kls;
-            walk_groups(std::true_type{}, bare, false, SHARE, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+            walk_groups(std::true_type{}, bare, SHARE, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
                 if (g >= full_groups) mask_group(g, s);
                 float e[8];
 #pragma unroll
@@ -719,7 +721,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         } else {
             // ---- pass 1 with the bookkeeping of the special rows
             RowStats st = {-inf, 0.0f, 0u, false, false};
-            walk_groups(std::false_type{}, false, true, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+            walk_groups(std::false_type{}, false, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
                 // the finite maximum of the lane's eight scores first, then one rescale; written
                 // with selects only (a branch per element would cost more than the arithmetic)
                 float local = -inf;
@@ -772,7 +774,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
             const float inv_sum = 1.0f / st.sum;
             // ---- pass 2 of the special rows
-            walk_groups(std::true_type{}, false, true, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+            walk_groups(std::true_type{}, false, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
                 float pr[8];
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
@@ -1452,6 +1454,7 @@ static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const 
         int e = 0;
         g.scale_pow2 = frexpf(g.scale, &e) == 0.5f ? 1u : 0u;
         g.inv_scale = 1.0f / g.scale;
+        g.exp_scale = (float)(1.4426950408889634074 / (double)g.scale);
     }
     if (s.Hq > 65535u || s.R > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
     const hipStream_t st = native(stream);
