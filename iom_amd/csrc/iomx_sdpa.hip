@@ -335,6 +335,16 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
     return r;
 }
 
+// Results of the matrix instructions that are about to be read by instructions the compiler
+// cannot see (max3 / max2 above).  A vector instruction may read a register the matrix pipeline
+// writes only a fixed number of issue slots after the matrix instruction; the compiler counts those
+// slots for the instructions it schedules and knows nothing of the ones inside an asm statement,
+// so the wait is written out here (sixteen slots cover the eight passes of a 16x16x32 product),
+// tied to the values so that it stays between their producers and their readers.
+__device__ __forceinline__ void settle_matrix_results(f32x4_t (&s)[2]) {
+    asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s[0]), "+v"(s[1]));
+}
+
 __device__ __forceinline__ float max2(float a, float b) {
     float r;
     asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
@@ -537,8 +547,13 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         // the visible groups of this wave, K one group ahead where the mode says so; WITH_V: the
         // V fragments of the group are requested before its scores are formed
         // `primed`: the first two stages of the ring have been requested already
-        auto walk_groups = [&](auto with_v, bool bare, bool primed, auto&& body) {
+        // `edge` (plain passes): the groups below full_groups get body(.., false_type) and the ones
+        // from there on body(.., true_type), which masks -- as two loops over one step, because a
+        // mask under a branch inside one loop costs a register copy per score in every group.  The
+        // special rows' passes do their own bookkeeping per score and take one loop.
+        auto walk_groups = [&](auto with_v, bool bare, bool primed, auto edge, auto&& body) {
             constexpr bool WITH_V = decltype(with_v)::value;
+            constexpr bool EDGE = decltype(edge)::value;
             if constexpr (SHARE) {
                 constexpr int LPS = (WITH_V ? 2 : 1) * (DT16 / 4);        // direct loads per wave and stage
                 if (!primed) {
@@ -546,8 +561,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                     issue(with_v, 1, 1);
                 }
                 uint32_t buf = 0;
-#pragma unroll 1
-                for (uint32_t g = 0; g < ring_groups; ++g) {
+                auto step = [&](uint32_t g, auto masked) {
                     // the own loads of group g have landed; past the barrier everybody's have, and
                     // nobody reads the buffer of group g-1 any more: it takes group g+2
                     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPS) : "memory");
@@ -555,7 +569,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                     issue(with_v, g + 2, buf == 0 ? 2 : buf - 1);
                     const uint8_t* stage = kv_ring + buf * kStage;
                     buf = buf == 2 ? 0 : buf + 1;
-                    if (MODE == 3 && g >= groups) continue;               // uniform: past this wave's own tile
+                    if (MODE == 3 && g >= groups) return;                 // uniform: past this wave's own tile
                     // The operands come out of LDS through ds_read instructions the compiler does
                     // not see as such.  Left to itself it waits, before every LDS read, for every
                     // direct load still in flight (it cannot tell the ring's stages apart), which
@@ -586,8 +600,16 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                     }
                     f32x4_t s[2];
                     scores(cur, s, bare);
-                    body(g, s, vfr);
+                    body(g, s, vfr, masked);
+                };
+                uint32_t g = 0;
+                if constexpr (EDGE) {
+                    const uint32_t whole = full_groups < ring_groups ? full_groups : ring_groups;
+#pragma unroll 1
+                    for (; g < whole; ++g) step(g, std::false_type{});
                 }
+#pragma unroll 1
+                for (; g < ring_groups; ++g) step(g, std::true_type{});
                 // nothing in flight and nobody reading when the next pass (or the next workgroup)
                 // takes the ring
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -596,8 +618,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             }
             KGroup cur, nxt;
             if (AHEAD && g_first < groups) load_k(g_first, cur);
-#pragma unroll 1
-            for (uint32_t g = g_first; g < groups; g += g_step) {
+            auto step = [&](uint32_t g, auto masked) {
                 if (!AHEAD) load_k(g, cur);
                 else if (g + g_step < groups) load_k(g + g_step, nxt);     // the next group is in flight meanwhile
                 u32x4 vfr[WITH_V ? DT16 : 1];
@@ -608,9 +629,17 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
                 }
                 f32x4_t s[2];
                 scores(cur, s, bare);
-                body(g, s, vfr);
+                body(g, s, vfr, masked);
                 if (AHEAD) cur = nxt;
+            };
+            uint32_t g = g_first;
+            if constexpr (EDGE) {
+                const uint32_t whole = full_groups < groups ? full_groups : groups;
+#pragma unroll 1
+                for (; g < whole; g += g_step) step(g, std::false_type{});
             }
+#pragma unroll 1
+            for (; g < groups; g += g_step) step(g, std::true_type{});
         };
         // scores of tokens the lane's row must not see become -infinity (plain passes)
         auto mask_group = [&](uint32_t g, f32x4_t (&s)[2]) {
@@ -647,8 +676,9 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
 
         // ---- plain pass 1: running maximum and sum of exp(score - maximum)
         float pm = -inf, psum = 0.0f;
-        walk_groups(std::false_type{}, bare, true, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
-            if (g >= full_groups) mask_group(g, s);
+        walk_groups(std::false_type{}, bare, true, std::true_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1], auto masked) {
+            if constexpr (decltype(masked)::value) mask_group(g, s);     // (selects the compiler schedules)
+            else settle_matrix_results(s);
             // (the maximum instruction itself: a NaN among its operands is passed over, and the
             // row's sum below turns NaN from that score's exponential all the same)
             const float newm = max3(max3(s[0][0], s[0][1], s[0][2]), max3(s[0][3], s[1][0], s[1][1]),
@@ -707,8 +737,8 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         if (plain) {
             // ---- plain pass 2: probabilities, rounded once to BF16 and flushed, times V
             const float inv_sum = 1.0f / psum, nb = -pm * kls;
-            walk_groups(std::true_type{}, bare, SHARE, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
-                if (g >= full_groups) mask_group(g, s);
+            walk_groups(std::true_type{}, bare, SHARE, std::true_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16], auto masked) {
+                if constexpr (decltype(masked)::value) mask_group(g, s);
                 float e[8];
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
@@ -721,7 +751,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
         } else {
             // ---- pass 1 with the bookkeeping of the special rows
             RowStats st = {-inf, 0.0f, 0u, false, false};
-            walk_groups(std::false_type{}, false, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1]) {
+            walk_groups(std::false_type{}, false, false, std::false_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&)[1], auto) {
                 // the finite maximum of the lane's eight scores first, then one rescale; written
                 // with selects only (a branch per element would cost more than the arithmetic)
                 float local = -inf;
@@ -774,7 +804,7 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
             const float pinf_p = st.pinf ? 1.0f / (float)st.pinf : 0.0f;
             const float inv_sum = 1.0f / st.sum;
             // ---- pass 2 of the special rows
-            walk_groups(std::true_type{}, false, false, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16]) {
+            walk_groups(std::true_type{}, false, false, std::false_type{}, [&](uint32_t g, f32x4_t (&s)[2], const u32x4 (&vfr)[DT16], auto) {
                 float pr[8];
 #pragma unroll
                 for (int half = 0; half < 2; ++half)
