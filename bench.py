@@ -494,7 +494,7 @@ def wl_sdpa(timer, steps, warmup):
                    2 * (B * Hq * R * D * 2 + 2 * B * Hkv * L * D), B * Hq * R * D, wall, ev,
                    iomx.last_launch().kernel.decode())
         r["TFLOP_per_s"] = round(flops / (ev * 1e-3) / 1e12, 2)
-        r["launches"] = "sdpa_decode" if nbytes == 0 else "sdpa_pack + sdpa_mfma"
+        r["launches"] = "sdpa_decode" if nbytes == 0 else "sdpa_pack + " + iomx.last_launch().kernel.decode()
         out.append(r)
         for t in (q, k, v, o) + ((ws,) if ws else ()):
             t.free()

@@ -337,7 +337,9 @@ int iomx_launch_linear(int dtype, const iomx_view* x, const iomx_view* w, const 
  * P*V on the vector units straight from the cache) for the few-row requests, else the
  * pack kernel and the matrix-core kernel (D <= 128), which forms the rows of a KV head
  * whose V holds an infinity or NaN in the reference's order instead; path 1 runs the
- * reference-order kernel alone (D <= 256, no workspace).
+ * reference-order kernel alone (D <= 256, no workspace); path 2 is path 0 with the kernel
+ * that gives a wave two row tiles (chosen by path 0 from 1024 rows on, where four query
+ * heads share a KV head and D is 64 or 128) for any number of rows: for tests.
  */
 int iomx_sdpa_workspace(int dtype, const iomx_view* q, const iomx_view* k, const iomx_view* v,
                         const iomx_view* out, uint64_t a, uint64_t L, uint64_t* bytes,

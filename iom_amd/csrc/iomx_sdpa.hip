@@ -878,6 +878,299 @@ void sdpa_mfma_bf16_kernel(const SdpaArgs a) {
     }
 }
 
+// The shared-ring mapping (MODE 2 above: four heads of one KV head per workgroup, D = 64 or 128)
+// with TWO neighbouring row tiles per wave: every K and V group read from LDS feeds two score tiles
+// and two output tiles, which halves the LDS traffic per product (what bounds the one-tile kernel
+// at D = 128) and gives a wave two independent chains of matrix and exponent instructions per group
+// where few waves fit a SIMD.  (Pairing tile j with tile N-1-j instead, which makes every
+// workgroup's walk equally long, was measured and lost: half of its steps have one tile's work.)
+// Plain passes only: a workgroup whose rows turn out special (a NaN or +infinity score, no finite
+// score, or an infinity / NaN in V) forms its rows in the reference's order instead
+// (sdpa_reference_row), all four waves together.  Grid (Hq / 4, planes, ceil(N / 2)); with N odd
+// the last tile is alone.  The walk below does not assume the two tiles are neighbours: tile 0 is
+// any tile above tile 1.
+struct TileAbsent {};
+struct TilePlain {};
+struct TileMasked {};
+
+template <int DT16>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+void sdpa_mfma_pair_bf16_kernel(const SdpaArgs a) {
+    static_assert(DT16 % 4 == 0, "whole KiB chunks per wave");
+    constexpr int T = 2;                                   // row tiles per wave: 0 the short one, 1 the long one
+    constexpr uint32_t kStage = 2 * DT16 * 1024;           // K group + V group
+    constexpr int D32 = DT16 / 2;
+    constexpr float kFloor = -1.0e30f;                     // stands in for a maximum of -infinity
+    __shared__ __attribute__((aligned(16))) uint8_t kv_ring[3 * kStage];
+    __shared__ float row_buffer[4][64];
+    __shared__ uint32_t special_rows;
+    if (threadIdx.x == 0) special_rows = 0;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t l16 = lane & 15u, kg = lane >> 4;
+    const uint32_t head = blockIdx.x * 4 + wave;
+    const uint32_t hkv = head / a.grouping;
+    const uint32_t row_tiles = (a.R + kTile - 1) / kTile;
+    // pairs of neighbouring tiles, the pairs with the longest prefixes dispatched first
+    const uint32_t pair = gridDim.z - 1 - blockIdx.z;
+    const uint32_t slab[T] = {2 * pair, 2 * pair + 1 < row_tiles ? 2 * pair + 1 : 2 * pair};
+    const bool both = slab[0] < slab[1];
+    const float inf = __builtin_inff();
+    // per tile: the lane's row, what it sees (rows past R mirror the tile's last row: their results
+    // are dropped), the groups its rows reach and the groups all of them see whole
+    uint32_t row[T], vis_plain[T], groups[T], full[T], first_row[T], last_row[T];
+    bool row_ok[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        first_row[t] = slab[t] * kTile;
+        last_row[t] = first_row[t] + kTile - 1 < a.R ? first_row[t] + kTile - 1 : a.R - 1;
+        const uint32_t vis_last = a.a + last_row[t] + 1 < a.L ? a.a + last_row[t] + 1 : a.L;
+        row[t] = first_row[t] + l16;
+        row_ok[t] = row[t] < a.R && (t == 1 || both);
+        const uint32_t reach = a.a + row[t] + 1;
+        vis_plain[t] = row[t] < a.R ? (reach < a.L ? reach : a.L) : vis_last;
+        const uint32_t reach_min = a.a + first_row[t] + 1;
+        groups[t] = (vis_last + 31) / 32;
+        full[t] = (reach_min < a.L ? reach_min : a.L) / 32;
+    }
+    if (!both) {
+        groups[0] = 0;
+        full[0] = 0;
+    }
+    const uint32_t ring_groups = groups[1];
+    const uint32_t c0 = (kg & 1u) * 8u;
+    const uint32_t p = a.plane0 + blockIdx.y;
+    const uint32_t flag_words = sdpa_flag_words(a, p, hkv, lane);
+    uint64_t plane[4];
+    walk_planes(a.walk, p, plane);
+    const uint8_t* qb = a.q + (plane[0] + (uint64_t)head * a.q_head_stride) * a.q_plane_bytes;
+    const uint8_t* vf = a.packed_v + (((uint64_t)p * a.Hkv + hkv) * a.groups) * DT16 * kFrag;
+    const uint32_t vf_lane = lane * 16;
+    const uint8_t* kp = a.packed_k + (((uint64_t)p * a.Hkv + hkv) * a.groups * 2) * DT16 * kTileBytes;
+    const uint32_t kp_lane = l16 * kRowBytes + c0 * 2;
+    // a wave's share of K group g (and V group g) into ring stage buf, as in sdpa_mfma
+    auto issue = [&](auto with_v, uint32_t g, uint32_t buf) {
+        const uint32_t gg = g < ring_groups ? g : ring_groups - 1;
+        uint8_t* stage = kv_ring + buf * kStage;
+#pragma unroll
+        for (int j = 0; j < DT16 / 4; ++j) {
+            const uint32_t chunk = wave + 4 * j;
+            __builtin_amdgcn_global_load_lds((gptr_t)(kp + ((gg * DT16 + chunk) * kFrag + vf_lane)),
+                                             (lptr_t)(stage + chunk * kFrag), 16, 0, 0);
+            if constexpr (decltype(with_v)::value)
+                __builtin_amdgcn_global_load_lds((gptr_t)(vf + ((gg * DT16 + chunk) * kFrag + vf_lane)),
+                                                 (lptr_t)(stage + (DT16 + chunk) * kFrag), 16, 0, 0);
+        }
+    };
+    issue(std::false_type{}, 0, 0);
+    issue(std::false_type{}, 1, 1);
+    u32x4 q_bits[T][D32];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        const uint32_t qrow = row[t] < a.R ? row[t] : a.R - 1;
+#pragma unroll
+        for (int c = 0; c < D32; ++c)
+            q_bits[t][c] = *reinterpret_cast<const u32x4*>(
+                    qb + ((uint64_t)(qrow >> 4) * DT16 + (2 * c + (kg >> 1))) * kTileBytes + (qrow & 15u) * kRowBytes + c0 * 2);
+    }
+    // every row of the wave's tiles in the reference's order
+    auto reference_rows = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        for (int t = both ? 0 : 1; t < T; ++t)
+            for (uint32_t r = first_row[t]; r <= last_row[t]; ++r)
+                sdpa_reference_row(a, p, hkv, head, r, lane, &row_buffer[wave][0]);
+    };
+    if (__any(flag_words != 0)) {           // an infinity or NaN in V of this KV head: all four waves alike
+        reference_rows();
+        return;
+    }
+    bf16x8_t qf[T][D32];
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int c = 0; c < D32; ++c) qf[t][c] = daz8(q_bits[t][c]);
+
+    // One pass over the groups of the long tile: group g's K (and V) out of the ring, then
+    // body(g, k, v, state of tile 0, state of tile 1).  Tile 0 sees its groups whole, then masked,
+    // then not at all; tile 1 whole, then masked; the combinations that occur, in their order:
+    auto walk = [&](auto with_v, bool primed, auto&& body) {
+        constexpr bool WITH_V = decltype(with_v)::value;
+        constexpr int LPS = (WITH_V ? 2 : 1) * (DT16 / 4);
+        if (!primed) {
+            issue(with_v, 0, 0);
+            issue(with_v, 1, 1);
+        }
+        uint32_t buf = 0;
+        auto step = [&](uint32_t g, auto tile0, auto tile1) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPS) : "memory");
+            __builtin_amdgcn_s_barrier();
+            issue(with_v, g + 2, buf == 0 ? 2 : buf - 1);
+            const uint8_t* stage = kv_ring + buf * kStage;
+            buf = buf == 2 ? 0 : buf + 1;
+            u32x4 kw[2][D32];
+            const uint32_t k_at = lds_address(stage + ((kg >> 1) * kTileBytes + kp_lane));
+            static_for<2 * D32>([&](auto index) {
+                constexpr int half = decltype(index)::value / D32, c = decltype(index)::value % D32;
+                kw[half][c] = lds_read_b128<(half * DT16 + 2 * c) * (int)kTileBytes>(k_at);
+            });
+            u32x4 vfr[WITH_V ? DT16 : 1];
+            if constexpr (WITH_V) {
+                const uint32_t v_at = lds_address(stage + vf_lane);
+                static_for<DT16>([&](auto index) {
+                    constexpr int dt = decltype(index)::value;
+                    vfr[dt] = lds_read_b128<(DT16 + dt) * (int)kFrag>(v_at);
+                });
+            }
+            lds_reads_landed();
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int c = 0; c < D32; ++c) asm volatile("" : "+v"(kw[half][c]));
+            if constexpr (WITH_V) {
+#pragma unroll
+                for (int dt = 0; dt < DT16; ++dt) asm volatile("" : "+v"(vfr[dt]));
+            }
+            body(g, kw, vfr, tile0, tile1);
+        };
+        const uint32_t meet = groups[0] < full[1] ? groups[0] : full[1];
+        uint32_t g = 0;
+#pragma unroll 1
+        for (; g < full[0]; ++g) step(g, TilePlain{}, TilePlain{});
+#pragma unroll 1
+        for (; g < meet; ++g) step(g, TileMasked{}, TilePlain{});
+#pragma unroll 1
+        for (; g < full[1]; ++g) step(g, TileAbsent{}, TilePlain{});       // (runs when groups[0] < full[1])
+#pragma unroll 1
+        for (; g < groups[0]; ++g) step(g, TileMasked{}, TileMasked{});    // (runs when full[1] < groups[0])
+#pragma unroll 1
+        for (; g < groups[1]; ++g) step(g, TileAbsent{}, TileMasked{});
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+    };
+    // the dot products of tile t's rows with the 32 tokens of the group (lane: tokens
+    // 16*half + 4*kg + j of row l16), masked where the row must not see the token
+    auto scores = [&](auto tile, auto state, const u32x4 (&kw)[2][D32], uint32_t g, f32x4_t (&s)[2]) {
+        constexpr int t = decltype(tile)::value;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int c = 0; c < D32; ++c)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kw[half][c]), qf[t][c], acc, 0, 0, 0);
+            s[half] = acc;
+        }
+        if constexpr (std::is_same_v<decltype(state), TileMasked>) {
+            const int rem = (int)vis_plain[t] - (int)(32 * g + 4 * kg);
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) s[half][j] = 16 * half + j < rem ? s[half][j] : -inf;
+        } else {
+            settle_matrix_results(s);
+        }
+    };
+    const float kls = a.exp_scale;
+    auto join = [&](float& m, float& sum, float m2, float sum2) {
+        const float mm = __builtin_fmaxf(m, m2), base = __builtin_fmaxf(mm, kFloor);
+        sum = sum * __builtin_amdgcn_exp2f((__builtin_fmaxf(m, kFloor) - base) * kls)
+            + sum2 * __builtin_amdgcn_exp2f((__builtin_fmaxf(m2, kFloor) - base) * kls);
+        m = mm;
+    };
+
+    // ---- pass 1: running maximum and sum of exponentials of both tiles
+    float pm[T], psum[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        pm[t] = -inf;
+        psum[t] = 0.0f;
+    }
+    auto statistics = [&](auto tile, auto state, const u32x4 (&kw)[2][D32], uint32_t g) {
+        constexpr int t = decltype(tile)::value;
+        if constexpr (!std::is_same_v<decltype(state), TileAbsent>) {
+            f32x4_t s[2];
+            scores(tile, state, kw, g, s);
+            const float newm = max3(max3(s[0][0], s[0][1], s[0][2]), max3(s[0][3], s[1][0], s[1][1]),
+                                    max3(s[1][2], s[1][3], pm[t]));
+            const float base = max2(newm, kFloor);
+            psum[t] *= __builtin_amdgcn_exp2f((max2(pm[t], kFloor) - base) * kls);
+            const float nb = -base * kls;
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) psum[t] += __builtin_amdgcn_exp2f(__builtin_fmaf(s[half][j], kls, nb));
+            pm[t] = newm;
+        }
+    };
+    walk(std::false_type{}, true, [&](uint32_t g, const u32x4 (&kw)[2][D32], const u32x4 (&)[1], auto tile0, auto tile1) {
+        statistics(std::integral_constant<int, 0>{}, tile0, kw, g);
+        statistics(std::integral_constant<int, 1>{}, tile1, kw, g);
+    });
+    // pass 2's first groups are on their way while the statistics are joined
+    issue(std::true_type{}, 0, 0);
+    issue(std::true_type{}, 1, 1);
+    bool odd = false;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+#pragma unroll
+        for (int off = 16; off <= 32; off *= 2) {
+            const float m2 = __shfl_xor(pm[t], off), s2 = __shfl_xor(psum[t], off);
+            join(pm[t], psum[t], m2, s2);
+        }
+        if (t == 1 || both) odd = odd || !(psum[t] > 0.0f && psum[t] < inf && pm[t] < inf);
+    }
+    bool plain = !__any(odd);
+    if (!plain && lane == 0) special_rows = 1;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    plain = __builtin_amdgcn_readfirstlane(lds_read_b32(lds_address(&special_rows))) == 0;
+    if (!plain) {
+        reference_rows();
+        return;
+    }
+
+    // ---- pass 2: probabilities, rounded once to BF16 and flushed, times V
+    f32x4_t o[T][DT16];
+    float inv_sum[T], nb[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt) o[t][dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        inv_sum[t] = 1.0f / psum[t];
+        nb[t] = -pm[t] * kls;
+    }
+    auto products = [&](auto tile, auto state, const u32x4 (&kw)[2][D32], const u32x4 (&vfr)[DT16], uint32_t g) {
+        constexpr int t = decltype(tile)::value;
+        if constexpr (!std::is_same_v<decltype(state), TileAbsent>) {
+            f32x4_t s[2];
+            scores(tile, state, kw, g, s);
+            float e[8];
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) e[half * 4 + j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[half][j], kls, nb[t]));
+            const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, scaled_flushed_bf16x8(e, inv_sum[t]));
+#pragma unroll
+            for (int dt = 0; dt < DT16; ++dt)
+                o[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vfr[dt]), pf, o[t][dt], 0, 0, 0);
+        }
+    };
+    walk(std::true_type{}, true, [&](uint32_t g, const u32x4 (&kw)[2][D32], const u32x4 (&vfr)[DT16], auto tile0, auto tile1) {
+        products(std::integral_constant<int, 0>{}, tile0, kw, vfr, g);
+        products(std::integral_constant<int, 1>{}, tile1, kw, vfr, g);
+    });
+    // lane holds out[row][head*D + 16*dt + 4*kg + j]: one 8-byte piece of tile head * DT16 + dt
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        if (!row_ok[t]) continue;
+        uint8_t* ot = a.out + plane[3] * a.out_plane_bytes + (uint64_t)(row[t] >> 4) * a.out_tile_cols * kTileBytes
+                + (row[t] & 15u) * kRowBytes + (uint64_t)head * (DT16 * kTileBytes) + kg * 8;
+#pragma unroll
+        for (int dt = 0; dt < DT16; ++dt)
+            *reinterpret_cast<u32x2*>(ot + dt * kTileBytes) =
+                    u32x2{cvt_bf16x2(o[t][dt][0] + 0.0f, o[t][dt][1] + 0.0f), cvt_bf16x2(o[t][dt][2] + 0.0f, o[t][dt][3] + 0.0f)};
+    }
+}
+
 // Few rows per KV head (grouping * R <= 16: a decode step): one workgroup of eight waves
 // = one KV head of one plane, the 16 rows of its tile = the rows of all query heads of
 // that KV head, the waves share out the 32-token groups.  Scores come from the matrix
@@ -1445,6 +1738,9 @@ static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const 
     IOMX_TRY(sdpa_shape(q, k, v, out, a, L, &s));
     if (dtype != IOMX_DT_BF16) return IOMX_ERR_UNSUPPORTED;
     if (s.D > 256) return IOMX_ERR_UNSUPPORTED;
+    // path 2 = path 0 with the two-tile kernel wherever its mapping applies, however few the rows
+    const bool pairs_always = path == 2;
+    if (path == 2) path = 0;
     const Matrix qm = matrix_of(*q), km = matrix_of(*k), om = matrix_of(*out);
     SdpaArgs g = {};
     uint64_t strides[4][kMaxLead] = {};
@@ -1537,8 +1833,10 @@ static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const 
         // and when all rows of a KV head's query heads fit one tile they share it
         const uint32_t row_tiles = (g.R + kTile - 1) / kTile;
         int mode = 0;
-        if ((uint64_t)row_tiles * g.Hq * g.planes < 4096 && g.groups >= 8) mode = 1;
-        else if ((g.D == 64 || g.D == 128) && g.grouping % 4 == 0) mode = 2;
+        const bool four_heads_share = (g.D == 64 || g.D == 128) && g.grouping % 4 == 0;
+        if (pairs_always && four_heads_share) mode = 2;
+        else if ((uint64_t)row_tiles * g.Hq * g.planes < 4096 && g.groups >= 8) mode = 1;
+        else if (four_heads_share) mode = 2;
         else if ((g.D == 64 || g.D == 128) && row_tiles >= 4) mode = 3;
         g.flags = static_cast<uint32_t*>(workspace);
         g.packed_v = static_cast<uint8_t*>(workspace) + header;
@@ -1546,6 +1844,9 @@ static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const 
         g.pack_splits = sdpa_pack_splits(s, L);
         hipLaunchKernelGGL(sdpa_pack_kernel, dim3(g.Hkv * g.pack_splits, gz), dim3(256), 0, st, g);
         const bool full_d = (g.D & 31u) == 0;
+        // two row tiles per wave from 1024 rows on (measured on one sequence of 4096 rows against the
+        // one-tile kernel in the same process: 2 % at D = 64, 8 % at D = 128; at 512 rows no gain)
+        const bool in_pairs = mode == 2 && (pairs_always || row_tiles >= 64);
         for (g.plane0 = 0; g.plane0 < g.planes; g.plane0 += 65535u) {
         const uint32_t layers = g.planes - g.plane0 < 65535u ? g.planes - g.plane0 : 65535u;
         const dim3 grid(mode == 1 || mode == 3 ? g.Hq : (g.Hq + 3) / 4, layers, mode == 3 ? (row_tiles + 3) / 4 : row_tiles);
@@ -1557,7 +1858,11 @@ static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const 
         if (mode == 1) { IOMX_SDPA_MODE(N, 1); } \
         else { IOMX_SDPA_MODE(N, 0); } \
         break;
-        if (mode == 2 && g.d_tiles == 4)
+        if (in_pairs) {
+            const dim3 pairs(g.Hq / 4, layers, (row_tiles + 1) / 2);
+            if (g.d_tiles == 4) hipLaunchKernelGGL((sdpa_mfma_pair_bf16_kernel<4>), pairs, dim3(256), 0, st, g);
+            else hipLaunchKernelGGL((sdpa_mfma_pair_bf16_kernel<8>), pairs, dim3(256), 0, st, g);
+        } else if (mode == 2 && g.d_tiles == 4)
             hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<4, 2, true>), grid, dim3(256), 0, st, g);
         else if (mode == 2)
             hipLaunchKernelGGL((sdpa_mfma_bf16_kernel<8, 2, true>), grid, dim3(256), 0, st, g);
@@ -1573,8 +1878,9 @@ static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const 
 #undef IOMX_SDPA_MODE
 #undef IOMX_SDPA
         }
-        record_launch("sdpa_mfma", (mode == 3 ? (row_tiles + 3) / 4 : row_tiles) * (mode == 1 || mode == 3 ? g.Hq : (g.Hq + 3) / 4) * gz, 256,
-                      (uint64_t)g.planes * g.Hq * g.R);
+        if (in_pairs) record_launch("sdpa_mfma_pair", (row_tiles + 1) / 2 * (g.Hq / 4) * gz, 256, (uint64_t)g.planes * g.Hq * g.R);
+        else record_launch("sdpa_mfma", (mode == 3 ? (row_tiles + 3) / 4 : row_tiles) * (mode == 1 || mode == 3 ? g.Hq : (g.Hq + 3) / 4) * gz, 256,
+                           (uint64_t)g.planes * g.Hq * g.R);
         IOMX_HIP(hipGetLastError());
         return IOMX_OK;
     }
@@ -1637,7 +1943,7 @@ extern "C" int iomx_launch_sdpa_static(int dtype, const iomx_view* q, const iomx
                                        uint64_t L, int path, iomx_stream_t stream) {
     uint64_t need = 0, alignment = 1;
     IOMX_TRY(iomx_sdpa_workspace(dtype, q, k, v, out, a, L, &need, &alignment));
-    if (path != 0) need = 0;  // the reference-order kernel keeps nothing outside its operands
+    if (path == 1) need = 0;  // the reference-order kernel keeps nothing outside its operands
     if (need > IOMX_SDPA_STATIC_BYTES) return IOMX_ERR_EXHAUSTED;
     void* address = nullptr;
     IOMX_TRY(scratch_of_current_device(native(stream), &address));

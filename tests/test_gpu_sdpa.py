@@ -38,7 +38,7 @@ def run(case, path, fill=0x5A, expect_kernel=None):
     q, k, v, o = device_operands(case, fill)
     before = o.raw().copy()
     ws = None
-    if path == 0:
+    if path in (0, 2):
         rc, nbytes, align = iomx.sdpa_workspace(q.view(), k.view(), v.view(), o.view(), case["a"], case["L"])
         assert rc == 0 and align in (1, 256)
         ws = iomx.Buffer(nbytes) if nbytes else None
@@ -122,7 +122,7 @@ def float64_attention(case):
 FIXTURE_RULE_CAP = {((2,), 8, 2, 40, 64, 100, 50, 90): 4}
 
 
-@pytest.mark.parametrize("path", [0, 1], ids=["matrix_cores", "reference_order"])
+@pytest.mark.parametrize("path", [0, 1, 2], ids=["matrix_cores", "reference_order", "two_tiles_a_wave"])
 @pytest.mark.parametrize("spec", SEEDED, ids=[str(i) for i in range(len(SEEDED))])
 def test_seeded_shapes_against_the_oracle(spec, path):
     lead, Hq, Hkv, R, D, C, a, L = spec
@@ -152,6 +152,79 @@ def test_seeded_shapes_against_the_oracle(spec, path):
         # rule is not a bound under cancellation; the float64 budget above is, on every element).
         # That count is a cap: a kernel change that worsens it fails here.
         assert len(outside) <= FIXTURE_RULE_CAP.get(spec, 0), (spec, len(outside))
+
+
+PAIRS = [((2,), 8, 2, 33, 64, 60, 20, 53), ((), 8, 2, 100, 128, 128, 0, 100), ((3,), 4, 1, 64, 64, 64, 0, 64),
+         ((), 16, 4, 75, 128, 300, 200, 275), ((2,), 8, 2, 16, 64, 40, 3, 19), ((), 8, 2, 130, 64, 200, 50, 180)]
+
+
+@pytest.mark.parametrize("spec", PAIRS, ids=[str(i) for i in range(len(PAIRS))])
+def test_two_row_tiles_a_wave_equal_the_one_tile_kernel(spec):
+    """The kernel that gives a wave two neighbouring row tiles (path 2; path 0 picks it from 1024 rows
+    on) forms every row with the arithmetic of the one-tile kernel in the same order, so the outputs
+    are the same bits: odd and even numbers of row tiles, a ragged last tile, rows that start behind
+    a cached prefix, several planes."""
+    lead, Hq, Hkv, R, D, C, a, L = spec
+    case = random_case(71, lead, Hq, Hkv, R, D, C, a, L)
+    two = run(case, 2, fill=0xFF, expect_kernel="sdpa_mfma_pair")
+    one = run(case, 0, fill=0xFF, expect_kernel="sdpa_mfma")
+    if (L + 31) // 32 < 8:
+        assert np.array_equal(two, one)
+    else:
+        # (a long prefix on few rows: path 0 shares the token groups out over the waves of a workgroup,
+        # another order of additions)
+        assert np.mean(two == one) > 0.99
+    assert close_to_oracle(two, oracle(case)) == []
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_a_prefill_of_1024_rows_takes_two_tiles_a_wave_by_itself(D):
+    """From 1024 rows on (and enough row tiles, heads and planes to fill the chip without sharing a
+    head's tokens among waves) path 0 itself gives a wave two row tiles."""
+    n, Hq, Hkv, R = 4, 32, 8, 1024
+    case = random_case(79, (n,), Hq, Hkv, R, D, R, 0, R)
+    got = run(case, 0, expect_kernel="sdpa_mfma_pair").reshape(n, R, Hq * D)
+    # the same bits as the one-tile kernel gives: both halves of the rows by themselves (512 rows a
+    # call stay below the switch), the second half against a prefix that ends with it
+    q = np.array(case["q"], np.uint16).reshape(n, Hq, R, D)
+    for first in (0, 512):
+        part = dict(case, R=512, a=first, L=first + 512, q=q[:, :, first:first + 512].reshape(-1).tolist())
+        one = run(part, 0, expect_kernel="sdpa_mfma").reshape(n, 512, Hq * D)
+        assert np.array_equal(got[:, first:first + 512], one)
+    # one plane against the oracle: held to the float64 budget of the BF16 probability on every element,
+    # like the seeded shapes (with 1024 terms a sum, outputs that cancel to near zero leave the fixture
+    # rule in both kernels alike)
+    k = np.array(case["k"], np.uint16).reshape(n, Hkv, R, D)
+    v = np.array(case["v"], np.uint16).reshape(n, Hkv, R, D)
+    plane = dict(case, leading=[], q=q[1].reshape(-1).tolist(), k=k[1].reshape(-1).tolist(), v=v[1].reshape(-1).tolist())
+    want = oracle(plane)
+    ref64, budget = float64_attention(plane)
+    g = datagen.bf16_to_f32(got[1].reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    w = datagen.bf16_to_f32(want.reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    assert np.all(np.abs(g - ref64) <= budget)
+    assert np.all(np.abs(w - ref64) <= budget)
+    assert len(close_to_oracle(got[1], want)) <= got[1].size // 100000
+
+
+def test_two_row_tiles_a_wave_with_special_scores_and_values():
+    """A workgroup of the two-tile kernel whose rows meet a NaN or infinite score, or whose KV head
+    has an infinity in V, forms its rows in the reference's order: same value classes as the oracle
+    everywhere, and the bits of the plain case in the KV heads that have nothing special."""
+    R, D = 70, 64
+    case = random_case(73, (2,), 8, 2, R, D, 100, 20, 20 + R)
+    q = np.array(case["q"], np.uint16).reshape(2, 8, R, D).copy()
+    k = np.array(case["k"], np.uint16).reshape(2, 2, 100, D).copy()
+    v = np.array(case["v"], np.uint16).reshape(2, 2, 100, D).copy()
+    k[0, 0, 5, 3] = 0x7F80            # +inf in one feature of one token: scores of +inf / -inf
+    q[0, 6, 3, 7] = 0x7FC0            # a NaN row (plane 0, head 6 -> KV head 1)
+    v[1, 1, 40, 2] = 0x7F80           # an infinity in V of plane 1, KV head 1
+    special = dict(case, q=q.reshape(-1).tolist(), k=k.reshape(-1).tolist(), v=v.reshape(-1).tolist())
+    got = run(special, 2, expect_kernel="sdpa_mfma_pair")
+    assert close_to_oracle(got, oracle(special)) == []
+    g = got.reshape(2, R, 8, D)
+    assert np.all((g[0, 3, 6] & 0x7FFF) > 0x7F80)
+    plain = run(case, 2).reshape(2, R, 8, D)
+    assert np.array_equal(g[1][:, :4], plain[1][:, :4])              # plane 1, KV head 0: untouched by any of it
 
 
 @pytest.mark.parametrize("R", [6, 20], ids=["decode_kernel", "tiled_kernel_and_guard"])
