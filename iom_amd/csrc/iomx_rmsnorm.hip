@@ -35,17 +35,28 @@ struct RmsArgsT {
 };
 using RmsArgs = RmsArgsT<2>;
 
+constexpr bool is_f8(int dt) { return dt == IOMX_DT_F8_E4M3FN || dt == IOMX_DT_F8_E5M2; }
+
+// (The two 8-bit floating leaves take the resident kernel as well: a 16-byte chunk is one tile
+// row of sixteen elements, decoded and encoded by the conversion instructions of the tile-row
+// kernels.)
 template <int DT>
 struct RLeaf {
-    static constexpr uint32_t kBytes = (DT == IOMX_DT_BF16 || DT == IOMX_DT_F16) ? 2 : 4;
+    static constexpr uint32_t kBytes = is_f8(DT) ? 1 : (DT == IOMX_DT_BF16 || DT == IOMX_DT_F16) ? 2 : 4;
     static constexpr uint32_t kPerChunk = 16 / kBytes;
-    static constexpr uint32_t kChunksPerRow = kTile / kPerChunk;     // 2 | 4
-    static constexpr uint32_t kChunksPerTile = kTileSlots / kPerChunk; // 32 | 64
+    static constexpr uint32_t kChunksPerRow = kTile / kPerChunk;     // 1 | 2 | 4
+    static constexpr uint32_t kChunksPerTile = kTileSlots / kPerChunk; // 16 | 32 | 64
 };
 
 template <int DT>
 __device__ __forceinline__ void unpack(const u32x4& v, float* f) {
-    if constexpr (DT == IOMX_DT_BF16) {
+    if constexpr (is_f8(DT)) {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        float row[kTile];
+        hw_decode_row<DT>(w, row);
+#pragma unroll
+        for (int i = 0; i < (int)kTile; ++i) f[i] = row[i];
+    } else if constexpr (DT == IOMX_DT_BF16) {
         f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
         f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z); f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
     } else if constexpr (DT == IOMX_DT_F16) {
@@ -59,7 +70,14 @@ __device__ __forceinline__ void unpack(const u32x4& v, float* f) {
 template <int DT>
 __device__ __forceinline__ u32x4 pack(const float* f) {
     u32x4 r;
-    if constexpr (DT == IOMX_DT_BF16) {
+    if constexpr (is_f8(DT)) {
+        float row[kTile];
+#pragma unroll
+        for (int i = 0; i < (int)kTile; ++i) row[i] = f[i];
+        uint32_t w[4];
+        hw_encode_row<DT>(row, w);
+        r = u32x4{w[0], w[1], w[2], w[3]};
+    } else if constexpr (DT == IOMX_DT_BF16) {
         r.x = pack_bf16(f[0], f[1]); r.y = pack_bf16(f[2], f[3]);
         r.z = pack_bf16(f[4], f[5]); r.w = pack_bf16(f[6], f[7]);
     } else if constexpr (DT == IOMX_DT_F16) {
@@ -210,7 +228,7 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_band_kernel(const RmsArgsT<AD
 #pragma unroll
         for (uint32_t e = 0; e < L::kPerChunk; ++e) acc = __builtin_fmaf(f[e], f[e], acc);
     }
-    if constexpr (L::kBytes == 2) {
+    if constexpr (L::kBytes <= 2) {
 #pragma unroll
         for (int k = 0; k < K; ++k) asm volatile("" : "+v"(cur[k]));
     }
@@ -398,6 +416,22 @@ void launch_resident(const RmsArgsT<ADD ? 4 : 2>& a, hipStream_t s) {
     }
 }
 
+// The 8-bit floating leaves: n = F chunks per band (a tile is 256 bytes, sixteen chunks); whole
+// bands per workgroup up to 8192 features, two parts of eight rows beyond.
+constexpr uint32_t kF8BandLimit = 16384;
+template <int DT>
+void launch_resident_f8(const RmsArgs& a, hipStream_t s) {
+    const uint32_t n = a.band_chunks;
+    if (n <= 64) launch_band<DT, 1, 1, 64, false, true>(a, s);
+    else if (n <= 256) launch_band<DT, 1, 1, 256, false, true>(a, s);
+    else if (n <= 512) launch_band<DT, 2, 1, 256, false, true>(a, s);
+    else if (n <= 1024) launch_band<DT, 2, 1, 512, false, true>(a, s);
+    else if (n <= 2048) launch_band<DT, 4, 1, 512, false, true>(a, s);
+    else if (n <= 4096) launch_band<DT, 4, 1, 1024, false, true>(a, s);
+    else if (n <= 8192) launch_band<DT, 8, 1, 1024, false, false>(a, s);
+    else launch_band<DT, 8, 2, 1024, false, false>(a, s);
+}
+
 template <int DT>
 int launch(const RmsArgs& a, bool band_ok, hipStream_t s) {
     if (!band_ok || !band_kernel_serves<DT>(a.band_chunks, a.total_bands)) {
@@ -432,7 +466,15 @@ extern "C" int iomx_launch_rmsnorm(int dtype, const iomx_view* x, const iomx_vie
     if (scale->rank != 2 || scale->dims[0] != 1 || scale->dims[1] != m.cols) return IOMX_ERR_INVALID;
     if (out->base == x->base || out->base == scale->base) return IOMX_ERR_INVALID;
     if (!(eps >= 0.0f) || eps > 3.4028234e38f) return IOMX_ERR_INVALID;
-    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32 && dtype != IOMX_DT_F16) {
+    // (the 8-bit floating leaves take the resident kernel where a band is whole tiles and fits it)
+    bool f8_resident = is_f8(dtype) && m.cols % kTile == 0 && m.tile_cols * 16 <= kF8BandLimit;
+    if (f8_resident) {
+        uint64_t bands = m.tile_rows;            // of all leading planes: two workgroups a band at most
+        for (uint32_t i = 0; i + 2 < x->rank; ++i)
+            if (mul_overflows(bands, x->dims[i], &bands)) bands = ~0ull;
+        f8_resident = bands <= 0x7FFFFFFFull / 8;
+    }
+    if (dtype != IOMX_DT_BF16 && dtype != IOMX_DT_F32 && dtype != IOMX_DT_F16 && !f8_resident) {
         // the other floating leaves: one workgroup per row on packed tile rows
         RowsRmsnormRequest r = {};
         uint64_t rstrides[2][kMaxLead] = {};
@@ -493,6 +535,8 @@ extern "C" int iomx_launch_rmsnorm(int dtype, const iomx_view* x, const iomx_vie
     const hipStream_t s = native(stream);
     if (dtype == IOMX_DT_BF16) IOMX_TRY(launch<IOMX_DT_BF16>(a, band_ok, s));
     else if (dtype == IOMX_DT_F16) IOMX_TRY(launch<IOMX_DT_F16>(a, band_ok, s));
+    else if (dtype == IOMX_DT_F8_E4M3FN) launch_resident_f8<IOMX_DT_F8_E4M3FN>(a, s);
+    else if (dtype == IOMX_DT_F8_E5M2) launch_resident_f8<IOMX_DT_F8_E5M2>(a, s);
     else IOMX_TRY(launch<IOMX_DT_F32>(a, band_ok, s));
     IOMX_HIP(hipGetLastError());
     return IOMX_OK;
