@@ -655,8 +655,8 @@ def wl_chain(timer, steps, warmup):
     public = report("tinyllama_layer_non_gemm_chain_bf16_[64,512]", alg, 4 * nh + 2 * nf, wall, ev,
                     "6 launches: the public operations")
 
-    # The same chain as BASELINE words it (RMSNorm -> residual ADD -> RMSNorm -> SiLU*up -> residual
-    # ADD) with what may be fused privately fused: add + rmsnorm in one launch (x2 stored once and
+    # The same chain (RMSNorm -> residual ADD -> RMSNorm -> SiLU*up -> residual ADD) with what may be
+    # fused privately fused: add + rmsnorm in one launch (x2 stored once and
     # normalised from the registers that hold it) and SiLU*up in one launch.  Same bits in n1, x2,
     # n2, prod and next; act is never stored.  Fewer bytes have to cross HBM, so this row's
     # algorithmic bytes are its own: 4nh + 8nh + 6nf + 6nh (+ the two weight rows).
