@@ -362,10 +362,19 @@ namespace {
 template <int DT, int K, int S, int THREADS, bool ADD, bool PRE = (K * (int)RLeaf<DT>::kPerChunk <= 32)>
 void launch_band(const RmsArgsT<ADD ? 4 : 2>& a, hipStream_t s) {
     const uint32_t grid = a.total_bands * S;
+    // Workgroups per CU.  A workgroup of the 2-byte leaves that holds 32 KiB on 512 lanes would fit a
+    // CU four times (2048 lanes); three of them stream faster: four loads of 32 KiB each in flight,
+    // then four bursts of stores, is more than the memory side of a CU takes without queueing.  An
+    // LDS request nobody uses, of a size that fits three times into a CU's 160 KiB, sets that
+    // (BF16 [32768,2048]: 5830 -> 5950 GB/s, [65536,1024]: 6010 -> 6060; with two, 5800; the
+    // 16 KiB and 64 KiB workgroups of the other shapes and the F32 shapes of any size: no change or
+    // a loss).  The fused add + norm holds twice the bytes and takes two per CU (5560 -> 5610).
+    uint32_t lds = 0;
+    if (RLeaf<DT>::kBytes == 2 && K == 4 && THREADS == 512) lds = ADD ? 72u * 1024 : 48u * 1024;
     if ((uint32_t)(K * THREADS * S) == a.band_chunks)
-        hipLaunchKernelGGL((rmsnorm_band_kernel<DT, K, S, THREADS, true, PRE, ADD>), dim3(grid), dim3(THREADS), 0, s, a);
+        hipLaunchKernelGGL((rmsnorm_band_kernel<DT, K, S, THREADS, true, PRE, ADD>), dim3(grid), dim3(THREADS), lds, s, a);
     else
-        hipLaunchKernelGGL((rmsnorm_band_kernel<DT, K, S, THREADS, false, PRE, ADD>), dim3(grid), dim3(THREADS), 0, s, a);
+        hipLaunchKernelGGL((rmsnorm_band_kernel<DT, K, S, THREADS, false, PRE, ADD>), dim3(grid), dim3(THREADS), lds, s, a);
     record_launch(ADD ? (S == 1 ? "add_rmsnorm_band" : "add_rmsnorm_split") : (S == 1 ? "rmsnorm_band" : "rmsnorm_split"),
                   grid, THREADS, grid);
 }
