@@ -126,12 +126,23 @@ struct FlatArgs {
 enum { SHAPE_FLAT = 0, SHAPE_BANDS = 1, SHAPE_AXIS1 = 2, SHAPE_AXIS2 = 3, SHAPE_PLANES = 4,
        SHAPE_AXIS2B = 5 };
 
+// chunk of row 0 of the lane's tile column, for row-vector operands
+template <int DT>
+__device__ __forceinline__ uint64_t rowvec_offset(uint64_t cb) {
+    using L = Leaf<DT>;
+    return ((cb & ~(uint64_t)(L::kChunksPerTile - 1)) | (cb & (L::kChunksPerRow - 1))) * 16;
+}
+
+// Whole-plane operands stream past the caches; the row vector is reused by every row and stays
+// cached.  (Fetching the vector's 64 bytes a wave through the scalar cache instead, each lane
+// selecting its chunk, was built: a bare copy-plus-add probe gained 3 % from it, the real
+// operations lost 2-3 %, because the selects are vector instructions and a wave of these kernels
+// has about 680 cycles of its SIMD per KiB at full bandwidth -- sixty instructions are a third of
+// that.  Four lanes fetching and a cross-lane read per word: +0.5 % on ADD, -1 % on DIV.)
 template <int DT, int OP, int LM, int RM>
 __device__ __forceinline__ void stream_chunk(const uint8_t* lbase, const uint8_t* rbase,
                                              uint8_t* obase, uint64_t off, uint64_t voff) {
     constexpr int kInputs = Arity<OP>::kInputs;
-    // whole-plane operands stream past the caches; the row vector is reused by
-    // every row and stays cached
     u32x4 va, vb = u32x4{0, 0, 0, 0};
     if constexpr (LM == MODE_ROWVEC) va = *reinterpret_cast<const u32x4*>(lbase + voff);
     else va = load_stream(lbase + off);
@@ -142,38 +153,39 @@ __device__ __forceinline__ void stream_chunk(const uint8_t* lbase, const uint8_t
     store_stream(obase + off, op_chunk<DT, OP>(va, vb));
 }
 
-// chunk of row 0 of the lane's tile column, for row-vector operands
-template <int DT>
-__device__ __forceinline__ uint64_t rowvec_offset(uint64_t cb) {
-    using L = Leaf<DT>;
-    return ((cb & ~(uint64_t)(L::kChunksPerTile - 1)) | (cb & (L::kChunksPerRow - 1))) * 16;
-}
-
-template <int DT, int OP, int LM, int RM, int SHAPE>
+// ONCE: the grid has a workgroup for every (axis 0, axis 1 / band) pair -- no extent above 65535 --
+// so nothing loops: the wave reads one batch of arguments, loads, computes, stores and ends.  The
+// bandwidth of these kernels is the bytes in flight over the lifetime of a wave, and the loop
+// bounds and the grid's extents (fetched for the loops' steps) were two more trips to the scalar
+// cache in that lifetime: broadcast ADD BF16 [64,512,2048] 6490 -> 6570 GB/s, DIV 6480 -> 6550.
+template <int DT, int OP, int LM, int RM, int SHAPE, bool ONCE>
 __global__ __launch_bounds__(kPlanesBlock) void elementwise_stream_kernel(const FlatArgs a) {
     const uint64_t cb = (uint64_t)blockIdx.x * kPlanesBlock + threadIdx.x;
     if (cb >= a.seg_chunks) return;
     // with a row-vector operand and a single segment (a plane of one band) FLAT and AXIS2 still
     // need the lane's chunk of the vector
     constexpr bool kVector = LM == MODE_ROWVEC || RM == MODE_ROWVEC;
+    const uint64_t voff = kVector ? rowvec_offset<DT>(cb) : 0;
+    // the (z, y) pairs of this workgroup: one, or a stride of the grid's extents
+    const uint32_t z_step = ONCE ? 1u : gridDim.z, y_step = ONCE ? 1u : gridDim.y;
     if constexpr (SHAPE == SHAPE_FLAT) {
-        stream_chunk<DT, OP, LM, RM>(a.src[0], a.src[1], a.out, cb * 16, kVector ? rowvec_offset<DT>(cb) : 0);
+        stream_chunk<DT, OP, LM, RM>(a.src[0], a.src[1], a.out, cb * 16, voff);
     } else if constexpr (SHAPE == SHAPE_BANDS) {
-        const uint64_t voff = rowvec_offset<DT>(cb);
-        for (uint32_t y = blockIdx.y; y < a.segments; y += gridDim.y)
+        const uint32_t y_end = ONCE ? blockIdx.y + 1 : a.segments;
+        for (uint32_t y = blockIdx.y; y < y_end; y += y_step)
             stream_chunk<DT, OP, LM, RM>(a.src[0], a.src[1], a.out,
                                          ((uint64_t)y * a.seg_chunks + cb) * 16, voff);
     } else if constexpr (SHAPE == SHAPE_AXIS1) {
-        const uint64_t voff = rowvec_offset<DT>(cb);
-        for (uint32_t z = blockIdx.z; z < a.n0; z += gridDim.z)
-            for (uint32_t y = blockIdx.y; y < a.segments; y += gridDim.y)
+        const uint32_t z_end = ONCE ? blockIdx.z + 1 : a.n0, y_end = ONCE ? blockIdx.y + 1 : a.segments;
+        for (uint32_t z = blockIdx.z; z < z_end; z += z_step)
+            for (uint32_t y = blockIdx.y; y < y_end; y += y_step)
                 stream_chunk<DT, OP, LM, RM>(a.src[0] + z * a.step0[0], a.src[1] + z * a.step0[1],
                                              a.out + z * a.step0[2],
                                              ((uint64_t)y * a.seg_chunks + cb) * 16, voff);
     } else if constexpr (SHAPE == SHAPE_AXIS2B) {
-        const uint64_t voff = rowvec_offset<DT>(cb);
-        for (uint32_t z = blockIdx.z; z < a.n0; z += gridDim.z)
-            for (uint32_t y = blockIdx.y; y < a.n1 * a.segments; y += gridDim.y) {
+        const uint32_t z_end = ONCE ? blockIdx.z + 1 : a.n0, y_end = ONCE ? blockIdx.y + 1 : a.n1 * a.segments;
+        for (uint32_t z = blockIdx.z; z < z_end; z += z_step)
+            for (uint32_t y = blockIdx.y; y < y_end; y += y_step) {
                 const uint32_t j = fast_div(y, a.div_segments);  // segments >= 2 here
                 const uint32_t seg = y - j * a.segments;
                 stream_chunk<DT, OP, LM, RM>(a.src[0] + z * a.step0[0] + j * a.step1[0],
@@ -182,12 +194,12 @@ __global__ __launch_bounds__(kPlanesBlock) void elementwise_stream_kernel(const 
                                              ((uint64_t)seg * a.seg_chunks + cb) * 16, voff);
             }
     } else {
-        for (uint32_t z = blockIdx.z; z < a.n0; z += gridDim.z)
-            for (uint32_t y = blockIdx.y; y < a.n1; y += gridDim.y)
+        const uint32_t z_end = ONCE ? blockIdx.z + 1 : a.n0, y_end = ONCE ? blockIdx.y + 1 : a.n1;
+        for (uint32_t z = blockIdx.z; z < z_end; z += z_step)
+            for (uint32_t y = blockIdx.y; y < y_end; y += y_step)
                 stream_chunk<DT, OP, LM, RM>(a.src[0] + z * a.step0[0] + y * a.step1[0],
                                              a.src[1] + z * a.step0[1] + y * a.step1[1],
-                                             a.out + z * a.step0[2] + y * a.step1[2], cb * 16,
-                                             kVector ? rowvec_offset<DT>(cb) : 0);
+                                             a.out + z * a.step0[2] + y * a.step1[2], cb * 16, voff);
     }
 }
 
@@ -391,6 +403,7 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
         int shape = SHAPE_PLANES;
         dim3 grid3((uint32_t)gx, pa.segments < 65535u ? pa.segments : 65535u,
                    pa.planes < 65535u ? pa.planes : 65535u);
+        uint64_t y_extent = pa.segments, z_extent = pa.planes;    // what grid3.y and grid3.z stand for
         if (pa.planes == 1 && pa.walk.nlead == 0) {
             shape = pa.segments == 1 ? SHAPE_FLAT : SHAPE_BANDS;
         } else if (pa.walk.nlead == 1 || pa.walk.nlead == 2) {
@@ -404,20 +417,31 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
                 fa.step0[k] = pa.walk.stride[k][0] * pa.plane_bytes[k];
                 fa.step1[k] = pa.walk.nlead == 2 ? pa.walk.stride[k][1] * pa.plane_bytes[k] : 0;
             }
-            if (shape == SHAPE_AXIS2) grid3 = dim3((uint32_t)gx, fa.n1 < 65535u ? fa.n1 : 65535u,
-                                                   fa.n0 < 65535u ? fa.n0 : 65535u);
-            else if (shape == SHAPE_AXIS2B) {
+            z_extent = fa.n0;
+            if (shape == SHAPE_AXIS2) {
+                grid3 = dim3((uint32_t)gx, fa.n1 < 65535u ? fa.n1 : 65535u, fa.n0 < 65535u ? fa.n0 : 65535u);
+                y_extent = fa.n1;
+            } else if (shape == SHAPE_AXIS2B) {
                 const uint64_t ys = (uint64_t)fa.n1 * pa.segments;
                 fa.div_segments = make_fast_div(pa.segments);
                 grid3 = dim3((uint32_t)gx, (uint32_t)(ys < 65535u ? ys : 65535u),
                              fa.n0 < 65535u ? fa.n0 : 65535u);
+                y_extent = ys;
                 if (ys > 0xFFFFFFFFull) shape = SHAPE_PLANES;
             }
             else grid3.z = fa.n0 < 65535u ? fa.n0 : 65535u;
         }
+        // a workgroup for every (axis 0, axis 1 / band) pair: the kernel without loops
+        const bool once = grid3.y == y_extent && grid3.z == z_extent;
 #define IOMX_STREAM(LMV, RMV, SH)                                                               \
-    hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SH>), grid3,                \
-                       dim3(kPlanesBlock), 0, s, fa)
+    do {                                                                                        \
+        if (once || SH == SHAPE_FLAT)                                                           \
+            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SH, true>), grid3,  \
+                               dim3(kPlanesBlock), 0, s, fa);                                   \
+        else                                                                                    \
+            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SH, SH != SHAPE_FLAT ? false : true>), grid3, \
+                               dim3(kPlanesBlock), 0, s, fa);                                   \
+    } while (0)
 #define IOMX_PLANES(LMV, RMV)                                                                   \
     do {                                                                                        \
         if (shape == SHAPE_FLAT) IOMX_STREAM(LMV, RMV, SHAPE_FLAT);                             \
