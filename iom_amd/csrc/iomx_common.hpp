@@ -258,15 +258,14 @@ __device__ __forceinline__ uint32_t fast_div(uint32_t n, FastDiv f) {
 
 // e^x for x <= 0 (-inf gives 0; NaN gives a finite value, callers handle NaN
 // themselves), to about two units in the last place for |x| < 32, with gradual
-// underflow.  The rounding error of x*log2(e) is recovered by one FMA; the power
-// of two is applied by v_ldexp_f32, which denormalises correctly where v_exp_f32
-// alone would flush.
+// underflow.  n is the nearest integer to x*log2(e) and one FMA forms x*log2(e) - n
+// from the exact product, so the rounding error of the product never reaches the
+// fraction; the power of two is applied by v_ldexp_f32, which denormalises
+// correctly where v_exp_f32 alone would flush.
 __device__ __forceinline__ float exp_nonpos(float x) {
     const float a = fmaxf(x, -256.0f);  // bounds the integer part
-    const float hi = a * 1.44269502e+00f;
-    const float lo = __builtin_fmaf(a, 1.44269502e+00f, -hi);
-    const float n = __builtin_rintf(hi);
-    const float f = (hi - n) + lo;
+    const float n = __builtin_rintf(a * 1.44269502e+00f);
+    const float f = __builtin_fmaf(a, 1.44269502e+00f, -n);
     return __builtin_amdgcn_ldexpf(__builtin_amdgcn_exp2f(f), (int)n);
 }
 

@@ -3,8 +3,8 @@
 // One wave owns one row.  In the fast kernel the lane holds the whole row in
 // registers (K 128-bit loads, fully coalesced across the wave), so HBM sees
 // every visible score once and every probability once; the maximum and the sum
-// are wave-wide butterfly reductions.  Rows are independent, so four waves of a
-// workgroup work on four rows without LDS or barriers.
+// are wave-wide butterfly reductions.  Rows are independent: a workgroup is one wave
+// with one row, without LDS or barriers.
 //
 //   softmax_rows     unit column strides, 16-byte aligned score rows, at most
 //                    4096 physical columns.
@@ -45,7 +45,6 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
     return v;
 }
 
-constexpr uint32_t kThrottleLds = 40000;   // bytes of dynamic LDS asked for and never used
 constexpr uint32_t kNegInf = 0xFF800000u;
 constexpr uint32_t kPosInf = 0x7F800000u;
 
@@ -55,10 +54,9 @@ __device__ __forceinline__ uint64_t stage_offset(const iomx_stage_layout& l, uin
 }
 
 template <int K>
-__global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) {
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t g = blockIdx.x * 4u + (threadIdx.x >> 6);
-    if (g >= (uint32_t)a.total_rows) return;
+__global__ __launch_bounds__(64) void softmax_rows_kernel(const SoftmaxArgs a) {
+    const uint32_t lane = threadIdx.x;
+    const uint32_t g = blockIdx.x;   // the grid has one workgroup of one wave per row
     // row -> (plane, head, r) with multiply-shift divisions
     uint32_t ph = g, r = 0;
     if (a.prows32 > 1) {
@@ -99,36 +97,39 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
     float vmax = as_f32(kNegInf);
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const uint32_t col = (k * 64u + lane) * 4u;
-        if (k * 256u >= visible) {
+        if (k * 256u >= visible) {                         // uniform: nothing of this chunk is seen
 #pragma unroll
             for (int j = 0; j < 4; ++j) s[k][j] = as_f32(kNegInf);
             continue;
         }
-        const uint32_t nvis = visible > col ? visible - col : 0u;
         float x[4] = {as_f32(raw[k].x) * a.scale, as_f32(raw[k].y) * a.scale,
                       as_f32(raw[k].z) * a.scale, as_f32(raw[k].w) * a.scale};
-        if (col < visible && col + 4 > a.scols32) {
-            // the physical row ends inside this chunk: element by element (at most one
-            // lane of a row, and only where the row length is not a multiple of four)
+        if ((k + 1) * 256u > visible || (k + 1) * 256u > a.scols32) {
+            // uniform: the visible range or the physical row ends inside this chunk
+            const uint32_t col = (k * 64u + lane) * 4u;
+            const uint32_t nvis = visible > col ? visible - col : 0u;
+            if (col < visible && col + 4 > a.scols32) {
+                // the physical row ends inside this lane's four scores: element by element (at
+                // most one lane of a row, and only where the row length is not a multiple of four)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if ((uint32_t)j < nvis) x[j] = srow[col + j] * a.scale;
+                for (int j = 0; j < 4; ++j)
+                    if ((uint32_t)j < nvis) x[j] = srow[col + j] * a.scale;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) x[j] = (uint32_t)j < nvis ? x[j] : as_f32(kNegInf);
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            x[j] = (uint32_t)j < nvis ? x[j] : as_f32(kNegInf);
-            s[k][j] = x[j];
-            has_nan = has_nan || (x[j] != x[j]);
-            vmax = fmaxf(vmax, x[j]);  // fmaxf skips NaN; NaN rows are decided by has_nan
-        }
+        for (int j = 0; j < 4; ++j) s[k][j] = x[j];
+        // one unordered compare sees a NaN in either of two scores; fmaxf skips NaN
+        has_nan = has_nan || __builtin_isunordered(x[0], x[1]) || __builtin_isunordered(x[2], x[3]);
+        vmax = fmaxf(fmaxf(vmax, x[0]), fmaxf(x[1], fmaxf(x[2], x[3])));
     }
     const bool row_nan = __any(has_nan);
     const float m = wave_max(vmax);
     const bool poisoned = row_nan || as_u32(m) == kNegInf;
     if (poisoned || as_u32(m) == kPosInf) {
         // rare rows: NaN / all -inf -> NaN over the visible range; k scores of +inf
-        // share 1/k
+        // share 1/k; everything at or beyond the visible limit is +0
         float share = as_f32(kQuietNanF32);
         if (!poisoned) {
             uint32_t cnt = 0;
@@ -141,8 +142,11 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
 #pragma unroll
         for (int k = 0; k < K; ++k)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                s[k][j] = (poisoned || as_u32(s[k][j]) == kPosInf) ? share : 0.0f;
+            for (int j = 0; j < 4; ++j) {
+                const bool seen = (k * 64u + lane) * 4u + j < visible;
+                const float v = (poisoned || as_u32(s[k][j]) == kPosInf) ? share : 0.0f;
+                s[k][j] = seen ? v : 0.0f;
+            }
     } else {
         float part = 0.0f;
 #pragma unroll
@@ -150,13 +154,13 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
             if (k * 256u >= visible) continue;            // uniform; stored as +0 below
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float e = exp_nonpos(s[k][j] - m);  // 0 for masked and -inf scores
+                const float e = exp_nonpos(s[k][j] - m);  // +0 for masked and -inf scores
                 s[k][j] = e;
                 part = part + e;
             }
         }
         // e * (1/sum) instead of e / sum: at most one binary32 unit apart, which a
-        // BF16 result shows only at a rounding boundary
+        // BF16 result shows only at a rounding boundary.  A masked score's +0 stays +0.
         const float inv_sum = 1.0f / wave_sum(part);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
@@ -169,15 +173,10 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const SoftmaxArgs a) 
     for (int k = 0; k < K; ++k) {
         const uint32_t col = (k * 64u + lane) * 4u;
         if (col >= a.pcols32) continue;
-        // elements at or beyond the visible limit are +0
-        const uint32_t nvis = visible > col ? visible - col : 0u;
-        uint32_t lo = 0, hi = 0;
+        uint32_t lo = 0, hi = 0;                           // a chunk nobody sees is +0
         if (k * 256u < visible) {                          // uniform
-            float pr[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) pr[j] = ((uint32_t)j < nvis) ? s[k][j] : 0.0f;
-            lo = pack_bf16(pr[0], pr[1]);
-            hi = pack_bf16(pr[2], pr[3]);
+            lo = pack_bf16(s[k][0], s[k][1]);
+            hi = pack_bf16(s[k][2], s[k][3]);
         }
         if (col + 4 <= a.pcols32) {
             __builtin_nontemporal_store(u32x2{lo, hi}, reinterpret_cast<u32x2*>(prow + col));
@@ -290,13 +289,11 @@ extern "C" int iomx_launch_softmax(const iomx_softmax_desc* d, iomx_stream_t str
             && sl.row_stride % 4 == 0
             && pl.plane_offset % 4 == 0 && pl.plane_stride % 4 == 0 && pl.head_stride % 4 == 0
             && pl.row_stride % 4 == 0;
-    const uint64_t blocks = (total + 3) / 4;
-    uint32_t grid = (uint32_t)(blocks < (1u << 20) ? blocks : (1u << 20));
     const hipStream_t s = native(stream);
     const uint64_t cols = pl.columns;
-    if (aligned && cols <= 4096 && sl.columns >= 4 && blocks <= 0x7FFFFFFFull && d->rows <= 0xFFFFFFFFull
+    if (aligned && cols <= 4096 && sl.columns >= 4 && total <= 0x7FFFFFFFull && d->rows <= 0xFFFFFFFFull
         && pl.rows <= 0xFFFFFFFFull && d->heads <= 0xFFFFFFFFull) {
-        grid = (uint32_t)blocks;  // one wave per row, one-shot
+        const uint32_t grid = (uint32_t)total;  // one wave per row, one-shot
         a.rows32 = (uint32_t)d->rows;
         a.prows32 = (uint32_t)pl.rows;
         a.heads32 = (uint32_t)d->heads;
@@ -306,18 +303,29 @@ extern "C" int iomx_launch_softmax(const iomx_softmax_desc* d, iomx_stream_t str
         a.a32 = (uint32_t)(d->a < d->L ? d->a : d->L);
         a.div_prows = make_fast_div(a.prows32);
         a.div_heads = make_fast_div(a.heads32);
-        if (cols <= 256) hipLaunchKernelGGL(softmax_rows_kernel<1>, dim3(grid), dim3(256), 0, s, a);
-        else if (cols <= 512) hipLaunchKernelGGL(softmax_rows_kernel<2>, dim3(grid), dim3(256), 0, s, a);
-        else if (cols <= 1024) hipLaunchKernelGGL(softmax_rows_kernel<4>, dim3(grid), dim3(256), 0, s, a);
-        // Rows of 1025..2048 columns: a wave has 8 KiB of loads in flight, and with all 32
-        // wave slots of a compute unit taken the memory system has 64 MB outstanding, past
-        // the point where more requests in flight help (measured on [32,32,2048,2048]: 72-74 %
-        // of peak with eight workgroups per compute unit, 77-78 % with four, 67 % with two).
-        // The unused dynamic LDS request (40 KB of 160 KB) is that limit of four.
-        else if (cols <= 2048) hipLaunchKernelGGL(softmax_rows_kernel<8>, dim3(grid), dim3(256), kThrottleLds, s, a);
-        else hipLaunchKernelGGL(softmax_rows_kernel<16>, dim3(grid), dim3(256), 0, s, a);
-        record_launch("softmax_rows", grid, 256, total);
+        // One wave per workgroup (the dispatcher then starts and retires rows one by one instead
+        // of four at a time), and fewer of them on a compute unit than its 32 wave slots: a wave
+        // has K KiB of loads in flight, and past about 100 KiB per compute unit more requests in
+        // flight only lengthen every wave's wait.  Measured on 2^32 scores, GB/s at the best
+        // count against four-wave workgroups at theirs: rows of 4096 columns 6170 (10 per compute
+        // unit) against 5400, 2048 columns 6500 (12) against 6110, 1024 columns 6250 (20) against
+        // 6250, 512 columns 6500 (32) against 6330; where a row sees only a part of its columns
+        // (half of them on average with a = 0) the best counts are 16, 16, 28 and 32.  The limit
+        // is an LDS request that nobody uses (160 KiB per compute unit).
+        const bool sees_all = a.a32 + 1 >= a.L32;
+        const auto lds_for = [](uint32_t per_cu) { return (163840u / per_cu) & ~511u; };
+        if (cols <= 256) hipLaunchKernelGGL(softmax_rows_kernel<1>, dim3(grid), dim3(64), 0, s, a);
+        else if (cols <= 512) hipLaunchKernelGGL(softmax_rows_kernel<2>, dim3(grid), dim3(64), 0, s, a);
+        else if (cols <= 1024)
+            hipLaunchKernelGGL(softmax_rows_kernel<4>, dim3(grid), dim3(64), lds_for(sees_all ? 20 : 28), s, a);
+        else if (cols <= 2048)
+            hipLaunchKernelGGL(softmax_rows_kernel<8>, dim3(grid), dim3(64), lds_for(sees_all ? 12 : 16), s, a);
+        else
+            hipLaunchKernelGGL(softmax_rows_kernel<16>, dim3(grid), dim3(64), lds_for(sees_all ? 10 : 16), s, a);
+        record_launch("softmax_rows", grid, 64, total);
     } else {
+        const uint64_t blocks = (total + 3) / 4;
+        const uint32_t grid = (uint32_t)(blocks < (1u << 20) ? blocks : (1u << 20));
         hipLaunchKernelGGL(softmax_generic_kernel, dim3(grid), dim3(256), 0, s, a);
         record_launch("softmax_generic", grid, 256, total);
     }
