@@ -1291,23 +1291,35 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         // loaded straight from the cache in the operand order (lane (feature l16, kg): tokens
         // 32g + 4kg + j and 32g + 16 + 4kg + j), flushed in registers
         const uint32_t vis_min = a.a + 1 < a.L ? a.a + 1 : a.L;          // what row 0 sees: the least
-        const uint32_t full_groups = vis_min / 32;
+        // Where every row in use sees the same prefix (one row per sequence -- the decode step --
+        // or every row reaches the end of the prefix) no visible token is hidden from any row, so
+        // the ragged last group takes the matrix cores as well: its tokens past the prefix get a
+        // probability of +0 and their V, whatever the cache holds there, is taken as zero.
+        const bool one_prefix = vis_min == vis_max;
+        const uint32_t full_groups = one_prefix ? groups : vis_min / 32;
         // of this share: the fully visible groups end at full_hi, the others start at tail_lo
         const uint32_t full_hi = full_groups < g_hi ? full_groups : g_hi;
         const uint32_t tail_lo = full_groups > g_lo ? full_groups : g_lo;
         struct VFrag { u32x4 w[DT16]; };
+        // (the ragged last group may end in the cache's last token tile: the second tile of the
+        // group is then not there, and its lanes read the first tile again -- their tokens lie past
+        // the prefix and are taken as zero below.  A wave-uniform offset, so every address stays a
+        // group base plus constants.)
+        const uint32_t last_token_tile = (vis_max - 1) >> 4;
         auto load_vf = [&](uint32_t g, VFrag& vf) {
+            const uint32_t second = 2 * g + 1 <= last_token_tile ? 2 * g + 1 : 2 * g;
+            const uint8_t* tiles[2] = {vb + (uint64_t)(2 * g) * a.d_tiles * kTileBytes,
+                                       vb + (uint64_t)second * a.d_tiles * kTileBytes};
 #pragma unroll
             for (int dt = 0; dt < DT16; ++dt) {
                 // pairs of 16-bit loads into the halves of one register
                 u16x2_t h[4];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const uint32_t token = 32 * g + (j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4));   // < vis_min <= L
                     uint16_t bits = 0;
                     if (dt * kTile + l16 < a.D)
                         bits = *reinterpret_cast<const uint16_t*>(
-                                vb + ((token >> 4) * a.d_tiles + dt) * kTileBytes + (token & 15u) * kRowBytes + l16 * 2);
+                                tiles[j >> 2] + dt * kTileBytes + (4 * kg + (j & 3)) * kRowBytes + l16 * 2);
                     h[j >> 1][j & 1] = bits;
                 }
                 // raw bits: they are flushed where they are used, so a request does not wait here
@@ -1456,6 +1468,15 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                     scores(kr[slot], s);
                     if (g + PD * NW < full_hi) load_k(g + PD * NW, kr[slot]);
                     const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, probabilities(g, s));
+                    if (32 * g + 32 > vis_max) {                              // uniform: the ragged last group
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const uint32_t t0 = 32 * g + (q < 2 ? 4 * kg + 2 * q : 16 + 4 * kg + 2 * (q - 2));
+                            const uint32_t keep = (t0 < vis_max ? 0x0000FFFFu : 0u) | (t0 + 1 < vis_max ? 0xFFFF0000u : 0u);
+#pragma unroll
+                            for (int dt = 0; dt < DT16; ++dt) vr[slot].w[dt][q] &= keep;
+                        }
+                    }
 #pragma unroll
                     for (int dt = 0; dt < DT16; ++dt)
                         om[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(daz8(vr[slot].w[dt]), pf, om[dt], 0, 0, 0);

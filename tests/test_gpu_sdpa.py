@@ -326,6 +326,38 @@ def test_decode_step_against_a_long_prefix_in_shares(spec):
     assert close_to_oracle(got, want) == []                    # and the reference's fixture rule holds
 
 
+RAGGED_DECODE = [((2,), 8, 2, 1, 64, 500, 499, 500), ((), 32, 4, 1, 64, 490, 485, 486),
+                 ((2,), 16, 8, 1, 128, 77, 69, 70), ((), 4, 2, 1, 40, 100, 50, 51),
+                 ((), 8, 2, 2, 64, 300, 298, 300), ((2,), 8, 2, 1, 64, 2300, 2210, 2211)]
+
+
+@pytest.mark.parametrize("spec", RAGGED_DECODE, ids=[str(i) for i in range(len(RAGGED_DECODE))])
+def test_decode_step_whose_prefix_ends_inside_a_token_group(spec):
+    """A decode step at a position that is not a multiple of 32 (31 of 32 steps of a session): every
+    row in use sees the same prefix, and the ragged last group takes the matrix cores with the V of
+    its tokens past the prefix taken as zero.  The cache tail holds NaN and infinities (the bits of
+    the result do not depend on it), a cache that ends in the group's first token tile is not read
+    past its end, and the results hold the fixture rule and the float64 budget against the oracle.
+    Cases: the cache ends with the prefix; the group's second tile is not there; D = 128 and a D
+    that is no multiple of 16; two rows that both reach the end of the prefix; in shares."""
+    lead, Hq, Hkv, R, D, C, a, L = spec
+    case = random_case(131 + L, lead, Hq, Hkv, R, D, C, a, L)
+    n = int(np.prod(lead)) if lead else 1
+    k = np.array(case["k"], np.uint16).reshape(n, Hkv, C, D).copy()
+    v = np.array(case["v"], np.uint16).reshape(n, Hkv, C, D).copy()
+    k[:, :, L:, :] = 0x7FC0
+    v[:, :, L:, 0::2] = 0xFF80
+    v[:, :, L:, 1::2] = 0x7FC0
+    tail = dict(case, k=k.reshape(-1).tolist(), v=v.reshape(-1).tolist())
+    got = run(tail, 0, fill=0xFF, expect_kernel="sdpa_decode")
+    assert np.array_equal(got, run(case, 0, expect_kernel="sdpa_decode"))
+    want = oracle(case)
+    ref64, budget = float64_attention(case)
+    g = datagen.bf16_to_f32(got.reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    assert np.all(np.abs(g - ref64) <= budget)
+    assert close_to_oracle(got, want) == []
+
+
 def test_decode_in_shares_with_special_scores_and_values():
     """Special scores that fall into different shares (a +infinity score in the first and the last
     share, a NaN query row, a row of -infinity scores), an infinite V at a token only the second
