@@ -41,6 +41,7 @@ struct SdpaArgs {
     uint32_t plane0;            // first plane of this launch
     float* decode_stats;        // sdpa_decode in shares: [pair][share][row][8] statistics
     float* decode_sums;         // ... and [pair][share][row][D] partial output sums
+    uint32_t kept_wave_bytes;   // sdpa_decode with kept scores: bytes of a wave's area in dynamic LDS
     uint8_t* packed_v;          // [plane][kv head][group][d tile] fragments of 1 KiB
     uint8_t* packed_k;          // [plane][kv head][token tile][d tile] flushed tiles (null: not packed)
     uint32_t* flags;            // [plane][kv head][pack split]: nonzero = that part of the V prefix
@@ -1186,15 +1187,29 @@ void sdpa_mfma_pair_bf16_kernel(const SdpaArgs a) {
 // shares (every workgroup in the same order, so all hold the same values), forms the
 // probabilities of its share and leaves its partial output sums; sdpa_decode_join_kernel adds the
 // partial sums in share order and stores the rows.
-template <int DT16, int PHASE>
+//
+// KEPT (one launch, prefixes past what the K ring holds): the scores of pass 1 stay in LDS
+// (128 bytes per group and tile row in use: [tile row][kg][8] binary32; every wave its own
+// groups), and pass 2 takes them from there instead of reading K and multiplying a second time
+// -- the same bits, a third less traffic.  KEPT = 1: the scores lie behind the kernel's own
+// arrays, [group] by [group].  KEPT = 2, for prefixes that do not fit that way: every wave has
+// an area of its own for its groups, and its probabilities of the vector path and its partial
+// outputs take the start of that area over once the wave is through with its scores (a wave's
+// LDS operations complete in order, and no other wave looks at the area before the barrier
+// behind the partial outputs).
+template <int DT16, int PHASE, int KEPT = 0>
 __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a) {
+    static_assert(KEPT == 0 || PHASE == 0, "scores are kept inside one launch");
+    extern __shared__ __attribute__((aligned(16))) uint8_t kept_scores[];
     constexpr int D32 = (DT16 + 1) / 2;
     constexpr int NW = 8;
     constexpr int DL = (DT16 + 3) / 4;                 // features per lane (lane, lane + 64)
     constexpr int PD = DT16 > 6 ? 1 : 2;               // groups in flight per wave (registers allow one at D > 96)
     __shared__ float wave_stats[NW][16][5];
-    __shared__ __attribute__((aligned(16))) float p_tile[NW][16][32];
-    __shared__ float o_part[NW][16][DL * 64];
+    // the probabilities of a group on the vector path and the waves' partial outputs
+    constexpr uint32_t kPBytes = 16 * 32 * 4;
+    __shared__ __attribute__((aligned(16))) float p_tile_own[KEPT == 2 ? 1 : NW][16][32];
+    __shared__ float o_part_own[KEPT == 2 ? 1 : NW][16][DL * 64];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t l16 = lane & 15u, kg = lane >> 4;
@@ -1204,6 +1219,21 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
     const bool row_ok = row < a.R;
     const uint32_t qrow = row_ok ? row : a.R - 1;
     const uint32_t nrows = a.grouping * a.R;                          // tile rows in use
+    auto p_tile = [&](uint32_t r, uint32_t t) -> float* {
+        if constexpr (KEPT == 2) return reinterpret_cast<float*>(kept_scores + wave * a.kept_wave_bytes + (r * 32 + t) * 4);
+        else return &p_tile_own[wave][r][t];
+    };
+    auto o_part = [&](uint32_t w, uint32_t r, uint32_t d) -> float& {
+        if constexpr (KEPT == 2)
+            return *reinterpret_cast<float*>(kept_scores + w * a.kept_wave_bytes + kPBytes + (r * (DL * 64) + d) * 4);
+        else return o_part_own[w][r][d];
+    };
+    // where the lane's eight scores of group g are kept
+    auto kept_at = [&](uint32_t g, uint32_t r) -> f32x4_t* {
+        if constexpr (KEPT == 2)
+            return reinterpret_cast<f32x4_t*>(kept_scores + wave * a.kept_wave_bytes + (((g / NW) * nrows + r) * 4 + kg) * 32);
+        else return reinterpret_cast<f32x4_t*>(kept_scores + ((g * nrows + r) * 4 + kg) * 32);
+    };
     const uint32_t reach = a.a + row + 1, reach_max = a.a + a.R;
     const uint32_t vis = row_ok ? (reach < a.L ? reach : a.L) : 0;
     const uint32_t vis_max = reach_max < a.L ? reach_max : a.L;
@@ -1359,6 +1389,13 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             f32x4_t s[2];
             scores(kr[slot], s);
             if (g + PD * NW < g_hi) load_k(g + PD * NW, kr[slot]);
+            if constexpr (KEPT != 0) {
+                if (l16 < nrows) {
+                    f32x4_t* dst = kept_at(g, l16);
+                    dst[0] = s[0];
+                    dst[1] = s[1];
+                }
+            }
             float local = -inf;
 #pragma unroll
             for (int half = 0; half < 2; ++half)
@@ -1455,7 +1492,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
 #pragma unroll
             for (int slot = 0; slot < PD; ++slot)
                 if (g_lo + wave + slot * NW < full_hi) {
-                    if (!ring_kept) load_k(g_lo + wave + slot * NW, kr[slot]);
+                    if (!ring_kept && KEPT == 0) load_k(g_lo + wave + slot * NW, kr[slot]);
                     if (PHASE != 0) load_vf(g_lo + wave + slot * NW, vr[slot]);
                 }
 #pragma unroll 1
@@ -1465,8 +1502,15 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                     const uint32_t g = g0 + slot * NW;
                     if (g >= full_hi) break;                                  // uniform
                     f32x4_t s[2];
-                    scores(kr[slot], s);
-                    if (g + PD * NW < full_hi) load_k(g + PD * NW, kr[slot]);
+                    if constexpr (KEPT != 0) {
+                        // (a wave reads what it wrote itself; rows not in use get no probability)
+                        const f32x4_t* src = kept_at(g, l16 < nrows ? l16 : 0);
+                        s[0] = src[0];
+                        s[1] = src[1];
+                    } else {
+                        scores(kr[slot], s);
+                        if (g + PD * NW < full_hi) load_k(g + PD * NW, kr[slot]);
+                    }
                     const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, probabilities(g, s));
                     if (32 * g + 32 > vis_max) {                              // uniform: the ragged last group
 #pragma unroll
@@ -1505,7 +1549,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                     const uint32_t pair = pw[half * 2 + (j >> 1)];
                     pe[j] = as_f32((j & 1) ? (pair & 0xFFFF0000u) : (pair << 16));
                 }
-                *reinterpret_cast<f32x4_t*>(&p_tile[wave][l16][16 * half + 4 * kg]) = pe;
+                *reinterpret_cast<f32x4_t*>(p_tile(l16, 16 * half + 4 * kg)) = pe;
             }
             // the wave reads only what it wrote itself: LDS operations of a wave complete in order
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -1521,8 +1565,8 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                     f32x4_t pa[4], pb[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        pa[q] = *reinterpret_cast<const f32x4_t*>(&p_tile[wave][r4 + q][t0]);
-                        pb[q] = *reinterpret_cast<const f32x4_t*>(&p_tile[wave][r4 + q][t0 + 4]);
+                        pa[q] = *reinterpret_cast<const f32x4_t*>(p_tile(r4 + q, t0));
+                        pb[q] = *reinterpret_cast<const f32x4_t*>(p_tile(r4 + q, t0 + 4));
                     }
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
@@ -1547,11 +1591,11 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
 #pragma unroll
-            for (int c = 0; c < DL; ++c) o_part[wave][r][lane + 64 * c] = o[r][c];
+            for (int c = 0; c < DL; ++c) o_part(wave, r, lane + 64 * c) = o[r][c];
 #pragma unroll
         for (int dt = 0; dt < DT16; ++dt)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) o_part[wave][l16][dt * 16 + 4 * kg + j] += om[dt][j];
+            for (int j = 0; j < 4; ++j) o_part(wave, l16, dt * 16 + 4 * kg + j) += om[dt][j];
         __syncthreads();
         // thread = (tile row, feature): 16 x D outputs over 512 threads
         for (uint32_t idx = threadIdx.x; idx < 16 * DL * 64; idx += 512) {
@@ -1559,7 +1603,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             if (r >= nrows || d >= a.D) continue;
             float sum = 0.0f;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) sum += o_part[w][r][d];
+            for (int w = 0; w < NW; ++w) sum += o_part(w, r, d);
             if (PHASE == 2) {
                 // [pair][share][row][D] partial sums of the workspace
                 a.decode_sums[((((uint64_t)p * a.Hkv + hkv) * shares + share) * 16 + r) * a.D + d] = sum;
@@ -1817,11 +1861,39 @@ static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const 
             g.decode_stats = static_cast<float*>(workspace);
             g.decode_sums = g.decode_stats + sdpa_decode_stats_floats(s, shares);
         }
+        // The scores of pass 1 kept in LDS for pass 2, where the K ring does not hold the whole prefix
+        // anyway (more than 16 groups; 8 where the ring has one slot) and they fit beside the
+        // kernel's own arrays (160 KiB per workgroup, one workgroup per CU): 128 bytes per group and
+        // tile row in use.
+        uint32_t kept_bytes = 0, kept_mode = 0;
+        {
+            const uint64_t reach = a + s.R, vis = reach < L ? reach : L, groups = (vis + 31) / 32;
+            const uint64_t ring = g.d_tiles > 6 ? 8 : 16, room = 159 * 1024;
+            const uint64_t arrays = 16 * 32 * 4 + 16 * ((g.d_tiles + 3) / 4) * 64 * 4;   // probabilities, partial outputs: per wave
+            const uint64_t group_bytes = (uint64_t)(g.grouping * s.R) * 128;
+            // a wave's area (mode 2): its ceil(groups / 8) groups, and not less than the two arrays
+            uint64_t per_wave = ((groups + 7) / 8) * group_bytes;
+            if (per_wave < arrays) per_wave = arrays;
+            if (shares == 1 && groups > ring) {
+                if (2560 + 8 * arrays + groups * group_bytes <= room) {
+                    kept_mode = 1;
+                    kept_bytes = (uint32_t)(groups * group_bytes);
+                } else if (2560 + 8 * per_wave <= room) {
+                    kept_mode = 2;
+                    kept_bytes = (uint32_t)(8 * per_wave);
+                    g.kept_wave_bytes = (uint32_t)per_wave;
+                }
+            }
+        }
         for (g.plane0 = 0; g.plane0 < g.planes; g.plane0 += 65535u) {
             const dim3 grid(g.Hkv, g.planes - g.plane0 < 65535u ? g.planes - g.plane0 : 65535u, shares);
 #define IOMX_SDPA_DECODE(N) \
     case N: \
-        if (shares == 1) { \
+        if (shares == 1 && kept_mode == 1) { \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0, 1>), grid, dim3(512), kept_bytes, st, g); \
+        } else if (shares == 1 && kept_mode == 2) { \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0, 2>), grid, dim3(512), kept_bytes, st, g); \
+        } else if (shares == 1) { \
             hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0>), grid, dim3(512), 0, st, g); \
         } else { \
             hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 1>), grid, dim3(512), 0, st, g); \

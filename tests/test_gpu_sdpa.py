@@ -358,6 +358,42 @@ def test_decode_step_whose_prefix_ends_inside_a_token_group(spec):
     assert close_to_oracle(got, want) == []
 
 
+KEPT_SCORES = [((2,), 8, 2, 1, 64, 1100, 1049, 1050), ((), 16, 2, 1, 128, 700, 650, 651),
+               ((), 8, 2, 2, 64, 900, 800, 802), ((), 16, 1, 1, 64, 1900, 1899, 1900),
+               ((), 8, 1, 2, 128, 1800, 1700, 1702), ((), 4, 4, 4, 96, 640, 600, 604)]
+
+
+@pytest.mark.parametrize("spec", KEPT_SCORES, ids=[str(i) for i in range(len(KEPT_SCORES))])
+def test_decode_step_that_keeps_its_scores_between_the_passes(spec):
+    """One launch against a prefix of 17 to 63 token groups: more than the K ring holds, so the
+    scores of pass 1 stay in LDS and pass 2 reads neither K nor multiplies again.  Cases 0-2 fit
+    behind the kernel's own arrays (D = 64 and 128; two rows per head, whose diagonal group takes
+    the vector path); cases 3-4 have 16 tile rows in use and 55 or more groups, which fit only as
+    per-wave areas that the partial outputs take over (case 4 with the vector path's probabilities
+    in the same area); case 5 is D = 96 with four rows.  Against the oracle (fixture rule, float64
+    budget), with NaN and infinities in the cache tail, which the result's bits do not depend on."""
+    lead, Hq, Hkv, R, D, C, a, L = spec
+    case = random_case(171 + L, lead, Hq, Hkv, R, D, C, a, L)
+    q, k, v, o = device_operands(case)
+    rc, nbytes, align = iomx.sdpa_workspace(q.view(), k.view(), v.view(), o.view(), a, L)
+    assert rc == 0 and nbytes == 0                                  # one launch, no workspace
+    for t in (q, k, v, o):
+        t.free()
+    n = int(np.prod(lead)) if lead else 1
+    kk = np.array(case["k"], np.uint16).reshape(n, Hkv, C, D).copy()
+    vv = np.array(case["v"], np.uint16).reshape(n, Hkv, C, D).copy()
+    kk[:, :, L:, :] = 0x7FC0
+    vv[:, :, L:, :] = 0x7F80
+    tail = dict(case, k=kk.reshape(-1).tolist(), v=vv.reshape(-1).tolist())
+    got = run(tail, 0, fill=0xFF, expect_kernel="sdpa_decode")
+    assert np.array_equal(got, run(case, 0, expect_kernel="sdpa_decode"))
+    want = oracle(case)
+    ref64, budget = float64_attention(case)
+    g = datagen.bf16_to_f32(got.reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    assert np.all(np.abs(g - ref64) <= budget)
+    assert close_to_oracle(got, want) == []
+
+
 def test_decode_in_shares_with_special_scores_and_values():
     """Special scores that fall into different shares (a +infinity score in the first and the last
     share, a NaN query row, a row of -infinity scores), an infinite V at a token only the second
