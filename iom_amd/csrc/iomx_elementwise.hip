@@ -231,6 +231,8 @@ struct PaddedArgs {
     uint32_t tile_rows;       // bands of one plane
     FastDiv div_tile_rows;
     uint32_t folded;          // segments run over several planes: band = segment mod tile_rows
+    uint32_t row_shift;       // lanes cover 2^row_shift rows of a band (4: all sixteen)
+    uint64_t lanes;           // lanes of one band: tile columns * 2^row_shift rows * chunks per row
 };
 
 // One operand's chunk: streamed for whole planes; for the broadcast shapes the one
@@ -255,11 +257,18 @@ template <int DT, int OP, int LM, int RM>
 __global__ __launch_bounds__(kPlanesBlock) void elementwise_padded_kernel(const PaddedArgs a) {
     using L = Leaf<DT>;
     constexpr int kInputs = Arity<OP>::kInputs;
-    const uint64_t cb = (uint64_t)blockIdx.x * kPlanesBlock + threadIdx.x;
-    if (cb >= a.b.seg_chunks) return;
-    const uint32_t in_tile = (uint32_t)cb & (L::kChunksPerTile - 1);
-    const uint32_t row = in_tile / L::kChunksPerRow;
-    const uint32_t col0 = (uint32_t)(cb / L::kChunksPerTile) * kTile + (in_tile & (L::kChunksPerRow - 1)) * L::kPerChunk;
+    // A plane of one band with eight rows or fewer (a decode step's [.,1,F] planes) gets lanes for
+    // the first 1, 2, 4 or 8 rows of its tiles only: the others would drop out at once, fifteen
+    // lanes in sixteen for a single row.  row_shift = 4 is the plain chunk order of the band.
+    const uint64_t lane_id = (uint64_t)blockIdx.x * kPlanesBlock + threadIdx.x;
+    if (lane_id >= a.lanes) return;
+    constexpr uint32_t kRowBits = L::kChunksPerRow == 1 ? 0 : L::kChunksPerRow == 2 ? 1 : L::kChunksPerRow == 4 ? 2 : 3;
+    static_assert((1u << kRowBits) == L::kChunksPerRow, "chunks per row: a power of two up to eight");
+    const uint32_t piece = (uint32_t)lane_id & (L::kChunksPerRow - 1);
+    const uint32_t row = (uint32_t)(lane_id >> kRowBits) & ((1u << a.row_shift) - 1);
+    const uint64_t tile = lane_id >> (kRowBits + a.row_shift);
+    const uint64_t cb = tile * L::kChunksPerTile + row * L::kChunksPerRow + piece;
+    const uint32_t col0 = (uint32_t)tile * kTile + piece * L::kPerChunk;
     if (col0 >= a.cols) return;
     const uint32_t left = a.cols - col0;
     const uint32_t valid = left < L::kPerChunk ? left : L::kPerChunk;
@@ -493,7 +502,7 @@ int dispatch(int op, bool planes, int lm, int rm, const BinaryArgs& pa, const Ge
 
 template <int DT, int OP>
 int launch_padded(int lm, int rm, const PaddedArgs& pa, hipStream_t s) {
-    const uint64_t gx = (pa.b.seg_chunks + kPlanesBlock - 1) / kPlanesBlock;
+    const uint64_t gx = (pa.lanes + kPlanesBlock - 1) / kPlanesBlock;
     if (gx > 0x7FFFFFFFull) return IOMX_ERR_OVERFLOW;
     const dim3 grid((uint32_t)gx, pa.b.segments < 65535u ? pa.b.segments : 65535u,
                     pa.b.planes < 65535u ? pa.b.planes : 65535u);
@@ -670,6 +679,9 @@ int run(int op, int dtype, const iomx_view* lhs, const iomx_view* rhs, const iom
         pd.cols = (uint32_t)cols;
         pd.tile_rows = (uint32_t)m[2].tile_rows;
         pd.div_tile_rows = make_fast_div(pd.tile_rows);
+        pd.row_shift = 4;
+        if (m[2].tile_rows == 1 && rows <= 8) pd.row_shift = rows <= 1 ? 0 : rows <= 2 ? 1 : rows <= 4 ? 2 : 3;
+        pd.lanes = (b.seg_chunks >> 4) << pd.row_shift;
         const hipStream_t ps = native(stream);
         int prc = IOMX_ERR_UNSUPPORTED;
         switch (cls) {
