@@ -467,13 +467,15 @@ def wl_vendor_stream(timer, steps, warmup):
 def wl_sdpa(timer, steps, warmup):
     """BF16 causal grouped-query attention at TinyLlama's head shape (32 query heads, 4 KV
     heads, D = 64): a 512-token prefill of 8 sequences and a decode step of 64 sequences
-    against a 512-token cache; and a 4096-token prefill of one sequence at D = 64 and at
-    D = 128 with 8 KV heads.  Algorithmic bytes: q, the visible K and V prefix and out,
+    against a 512-token cache; a 4096-token prefill of one sequence at D = 64 and at
+    D = 128 with 8 KV heads; and a decode step of 64 sequences at position 2046 (a prefix
+    that ends inside a token group and is longer than the kernel's K ring).  Algorithmic bytes: q, the visible K and V prefix and out,
     once each; flops: 4 * D per (row, visible token, head)."""
     out = []
     for name, B, R, a, L, Hq, Hkv, D in (("prefill", 8, 512, 0, 512, 32, 4, 64), ("decode", 64, 1, 511, 512, 32, 4, 64),
                                          ("prefill", 1, 4096, 0, 4096, 32, 4, 64),
-                                         ("prefill", 1, 4096, 0, 4096, 32, 8, 128)):
+                                         ("prefill", 1, 4096, 0, 4096, 32, 8, 128),
+                                         ("decode", 64, 1, 2046, 2047, 32, 4, 64)):
         C = L
         q = device_tensor(BF16, (B, Hq, R, D), "normal", 111)
         k = device_tensor(BF16, (B, Hkv, C, D), "normal", 112)

@@ -396,6 +396,20 @@ const char* family(int op, bool planes, bool rowvec) {
     return rowvec ? "binary_rowvec" : "binary_planes";
 }
 
+// The loop-free instance where the grid has a workgroup for every (axis, band) pair; FLAT has
+// no loops to begin with.
+template <int DT, int OP, int LM, int RM, int SH>
+void launch_stream(bool once, dim3 grid3, hipStream_t s, const FlatArgs& fa) {
+    if constexpr (SH == SHAPE_FLAT) {
+        hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LM, RM, SH, true>), grid3, dim3(kPlanesBlock), 0, s, fa);
+    } else {
+        if (once)
+            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LM, RM, SH, true>), grid3, dim3(kPlanesBlock), 0, s, fa);
+        else
+            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LM, RM, SH, false>), grid3, dim3(kPlanesBlock), 0, s, fa);
+    }
+}
+
 template <int DT, int OP>
 int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs& ga,
            hipStream_t s) {
@@ -442,15 +456,7 @@ int launch(bool planes, int lm, int rm, const BinaryArgs& pa, const GeneralArgs&
         }
         // a workgroup for every (axis 0, axis 1 / band) pair: the kernel without loops
         const bool once = grid3.y == y_extent && grid3.z == z_extent;
-#define IOMX_STREAM(LMV, RMV, SH)                                                               \
-    do {                                                                                        \
-        if (once || SH == SHAPE_FLAT)                                                           \
-            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SH, true>), grid3,  \
-                               dim3(kPlanesBlock), 0, s, fa);                                   \
-        else                                                                                    \
-            hipLaunchKernelGGL((elementwise_stream_kernel<DT, OP, LMV, RMV, SH, SH != SHAPE_FLAT ? false : true>), grid3, \
-                               dim3(kPlanesBlock), 0, s, fa);                                   \
-    } while (0)
+#define IOMX_STREAM(LMV, RMV, SH) launch_stream<DT, OP, LMV, RMV, SH>(once, grid3, s, fa)
 #define IOMX_PLANES(LMV, RMV)                                                                   \
     do {                                                                                        \
         if (shape == SHAPE_FLAT) IOMX_STREAM(LMV, RMV, SHAPE_FLAT);                             \
