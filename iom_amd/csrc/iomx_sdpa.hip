@@ -1362,16 +1362,19 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         // a ring of PD groups of K (and of V in pass 2): group g + PD*NW is requested as soon as
         // group g has been multiplied, so PD groups per wave are in flight -- one wave's chain of
         // dependent loads is what a long prefix costs here
-        KGroup kr[PD];
-        VFrag vr[PD];
+        // (with kept scores every pass streams one operand, and one group per wave in flight is
+        // enough: measured at 2048 tokens, 64 sequences, two groups 31.2 us, four 33.1, one 29.5)
+        constexpr int PR = KEPT != 0 ? 1 : PD;
+        KGroup kr[PR];
+        VFrag vr[PR];
         // a wave whose groups all fit the ring still holds their K after pass 1; V of the first
         // groups of pass 2 is requested here, together with K, so the step waits for memory once
         const bool ring_kept = PHASE == 0 && g_lo + wave + PD * NW >= g_hi;
         if (PHASE != 2) {
 #pragma unroll
-        for (int slot = 0; slot < PD; ++slot)
+        for (int slot = 0; slot < PR; ++slot)
             if (g_lo + wave + slot * NW < g_hi) load_k(g_lo + wave + slot * NW, kr[slot]);
-        if (PHASE == 0) {
+        if (PHASE == 0 && KEPT == 0) {
 #pragma unroll
             for (int slot = 0; slot < PD; ++slot)
                 if (g_lo + wave + slot * NW < full_hi) load_vf(g_lo + wave + slot * NW, vr[slot]);
@@ -1381,14 +1384,14 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         for (int c = 0; c < D32; ++c) qf[c] = daz8(q_bits[c]);
         if (PHASE != 2) {
 #pragma unroll 1
-        for (uint32_t g0 = g_lo + wave; g0 < g_hi; g0 += PD * NW) {
+        for (uint32_t g0 = g_lo + wave; g0 < g_hi; g0 += PR * NW) {
 #pragma unroll
-          for (int slot = 0; slot < PD; ++slot) {
+          for (int slot = 0; slot < PR; ++slot) {
             const uint32_t g = g0 + slot * NW;
             if (g >= g_hi) break;                                     // uniform
             f32x4_t s[2];
             scores(kr[slot], s);
-            if (g + PD * NW < g_hi) load_k(g + PD * NW, kr[slot]);
+            if (g + PR * NW < g_hi) load_k(g + PR * NW, kr[slot]);
             if constexpr (KEPT != 0) {
                 if (l16 < nrows) {
                     f32x4_t* dst = kept_at(g, l16);
@@ -1490,15 +1493,15 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         };
         {
 #pragma unroll
-            for (int slot = 0; slot < PD; ++slot)
+            for (int slot = 0; slot < PR; ++slot)
                 if (g_lo + wave + slot * NW < full_hi) {
                     if (!ring_kept && KEPT == 0) load_k(g_lo + wave + slot * NW, kr[slot]);
-                    if (PHASE != 0) load_vf(g_lo + wave + slot * NW, vr[slot]);
+                    if (PHASE != 0 || KEPT != 0) load_vf(g_lo + wave + slot * NW, vr[slot]);
                 }
 #pragma unroll 1
-            for (uint32_t g0 = g_lo + wave; g0 < full_hi; g0 += PD * NW) {
+            for (uint32_t g0 = g_lo + wave; g0 < full_hi; g0 += PR * NW) {
 #pragma unroll
-                for (int slot = 0; slot < PD; ++slot) {
+                for (int slot = 0; slot < PR; ++slot) {
                     const uint32_t g = g0 + slot * NW;
                     if (g >= full_hi) break;                                  // uniform
                     f32x4_t s[2];
@@ -1509,7 +1512,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                         s[1] = src[1];
                     } else {
                         scores(kr[slot], s);
-                        if (g + PD * NW < full_hi) load_k(g + PD * NW, kr[slot]);
+                        if (g + PR * NW < full_hi) load_k(g + PR * NW, kr[slot]);
                     }
                     const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, probabilities(g, s));
                     if (32 * g + 32 > vis_max) {                              // uniform: the ragged last group
@@ -1524,7 +1527,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
 #pragma unroll
                     for (int dt = 0; dt < DT16; ++dt)
                         om[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(daz8(vr[slot].w[dt]), pf, om[dt], 0, 0, 0);
-                    if (g + PD * NW < full_hi) load_vf(g + PD * NW, vr[slot]);
+                    if (g + PR * NW < full_hi) load_vf(g + PR * NW, vr[slot]);
                 }
             }
         }
