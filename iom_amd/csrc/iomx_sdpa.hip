@@ -1383,22 +1383,9 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
 #pragma unroll
         for (int c = 0; c < D32; ++c) qf[c] = daz8(q_bits[c]);
         if (PHASE != 2) {
-#pragma unroll 1
-        for (uint32_t g0 = g_lo + wave; g0 < g_hi; g0 += PR * NW) {
-#pragma unroll
-          for (int slot = 0; slot < PR; ++slot) {
-            const uint32_t g = g0 + slot * NW;
-            if (g >= g_hi) break;                                     // uniform
-            f32x4_t s[2];
-            scores(kr[slot], s);
-            if (g + PR * NW < g_hi) load_k(g + PR * NW, kr[slot]);
-            if constexpr (KEPT != 0) {
-                if (l16 < nrows) {
-                    f32x4_t* dst = kept_at(g, l16);
-                    dst[0] = s[0];
-                    dst[1] = s[1];
-                }
-            }
+        // The statistics of a group, with everything the special scores need: which tokens the
+        // row sees, NaN, the count of +infinity, non-finite scores kept out of maximum and sum.
+        auto careful_stats = [&](uint32_t g, f32x4_t (&s)[2]) {
             float local = -inf;
 #pragma unroll
             for (int half = 0; half < 2; ++half)
@@ -1419,7 +1406,81 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             for (int half = 0; half < 2; ++half)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) st.sum += s[half][e] == -inf ? 0.0f : __expf(s[half][e] - newm);
+        };
+        // The same statistics, bit for bit, for a group that every row in use sees whole and whose
+        // scores are finite or -infinity -- less than half the instructions: no per-token test, and
+        // exp(-infinity) is the +0 the careful form selects.  kFloor stands in for a maximum of
+        // -infinity in the exponent arguments.  A NaN, a +infinity or a maximum below kFloor raises
+        // `suspicious`, and the wave then forms all its statistics again in the careful form.
+        constexpr float kFloor = -1.0e30f;
+        bool suspicious = false;
+        auto fast_stats = [&](const f32x4_t (&s)[2]) {
+            suspicious = suspicious | __builtin_isunordered(s[0][0], s[0][1]) | __builtin_isunordered(s[0][2], s[0][3])
+                    | __builtin_isunordered(s[1][0], s[1][1]) | __builtin_isunordered(s[1][2], s[1][3]);
+            const float local = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(s[0][0], s[0][1]), __builtin_fmaxf(s[0][2], s[0][3])),
+                                                __builtin_fmaxf(__builtin_fmaxf(s[1][0], s[1][1]), __builtin_fmaxf(s[1][2], s[1][3])));
+            const float newm = __builtin_fmaxf(st.m, local);
+            suspicious = suspicious | (local == inf) | ((newm < kFloor) & (newm > -inf));
+            const float m_eff = __builtin_fmaxf(newm, kFloor);
+            st.sum = st.sum * __expf(__builtin_fmaxf(st.m, kFloor) - m_eff);
+            st.m = newm;
+            st.finite = st.finite | (local > -inf);
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) st.sum += __expf(s[half][e] - m_eff);
+        };
+        // groups below whole_hi are seen whole by every row in use
+        const uint32_t whole_groups = vis_min / 32, whole_hi = whole_groups < g_hi ? whole_groups : g_hi;
+        uint32_t g0 = g_lo + wave;
+#pragma unroll 1
+        for (; g0 + (PR - 1) * NW < whole_hi; g0 += PR * NW) {
+#pragma unroll
+          for (int slot = 0; slot < PR; ++slot) {
+            const uint32_t g = g0 + slot * NW;
+            f32x4_t s[2];
+            scores(kr[slot], s);
+            if (g + PR * NW < g_hi) load_k(g + PR * NW, kr[slot]);
+            if constexpr (KEPT != 0) {
+                if (l16 < nrows) {
+                    f32x4_t* dst = kept_at(g, l16);
+                    dst[0] = s[0];
+                    dst[1] = s[1];
+                }
+            }
+            fast_stats(s);
           }
+        }
+#pragma unroll 1
+        for (; g0 < g_hi; g0 += PR * NW) {
+#pragma unroll
+          for (int slot = 0; slot < PR; ++slot) {
+            const uint32_t g = g0 + slot * NW;
+            if (g >= g_hi) break;                                     // uniform
+            f32x4_t s[2];
+            scores(kr[slot], s);
+            if (g + PR * NW < g_hi) load_k(g + PR * NW, kr[slot]);
+            if constexpr (KEPT != 0) {
+                if (l16 < nrows) {
+                    f32x4_t* dst = kept_at(g, l16);
+                    dst[0] = s[0];
+                    dst[1] = s[1];
+                }
+            }
+            careful_stats(g, s);
+          }
+        }
+        if (__any(suspicious)) {
+            // rare: a special score among the whole groups -- all of the wave's groups again
+            st = RowStats{-inf, 0.0f, 0u, false, false};
+#pragma unroll 1
+            for (uint32_t g = g_lo + wave; g < g_hi; g += NW) {
+                KGroup kt;
+                load_k(g, kt);
+                f32x4_t s[2];
+                scores(kt, s);
+                careful_stats(g, s);
+            }
         }
 #pragma unroll
         for (int off = 16; off <= 32; off *= 2) {
@@ -1491,6 +1552,20 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             return u32x4{daz2(pack_bf16(pr[0], pr[1])), daz2(pack_bf16(pr[2], pr[3])),
                          daz2(pack_bf16(pr[4], pr[5])), daz2(pack_bf16(pr[6], pr[7]))};
         };
+        // The same probabilities, bit for bit, where no row of the tile is special (no NaN, no
+        // +infinity, a finite maximum) and every row in use sees the whole group: the careful
+        // form's selects all pick exp(v - max) / sum there, and exp(-infinity) is its +0.  (Tile
+        // rows not in use get probabilities too; their outputs are never stored.)
+        const bool plain_rows = !__any(nan_row || st.pinf != 0);
+        auto plain_probabilities = [&](const f32x4_t (&s)[2]) -> u32x4 {
+            float pr[8];
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) pr[half * 4 + j] = __expf(s[half][j] - st.m) * inv_sum;
+            return u32x4{daz2(pack_bf16(pr[0], pr[1])), daz2(pack_bf16(pr[2], pr[3])),
+                         daz2(pack_bf16(pr[4], pr[5])), daz2(pack_bf16(pr[6], pr[7]))};
+        };
         {
 #pragma unroll
             for (int slot = 0; slot < PR; ++slot)
@@ -1514,7 +1589,8 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                         scores(kr[slot], s);
                         if (g + PR * NW < full_hi) load_k(g + PR * NW, kr[slot]);
                     }
-                    const bf16x8_t pf = __builtin_bit_cast(bf16x8_t, probabilities(g, s));
+                    const bf16x8_t pf = __builtin_bit_cast(
+                            bf16x8_t, plain_rows && 32 * g + 32 <= vis_min ? plain_probabilities(s) : probabilities(g, s));
                     if (32 * g + 32 > vis_max) {                              // uniform: the ragged last group
 #pragma unroll
                         for (int q = 0; q < 4; ++q) {

@@ -394,6 +394,43 @@ def test_decode_step_that_keeps_its_scores_between_the_passes(spec):
     assert close_to_oracle(got, want) == []
 
 
+@pytest.mark.parametrize("L", [151, 700], ids=["k_ring", "kept_scores"])
+def test_decode_step_with_special_scores_among_whole_groups(L):
+    """One launch, several token groups that every row sees whole: their statistics and probabilities
+    take the short forms, which hold for finite and -infinity scores only; a +infinity score, a NaN
+    query row, a KV head whose every score is -infinity, +infinity or NaN, and a head whose scores
+    all lie below -1e30 (the stand-in for "no maximum yet" in the short form's exponent arguments)
+    must send the wave back to the careful form.  Against the oracle under the fixture rule."""
+    Hq, Hkv, R, D, C, a = 8, 2, 1, 64, L + 40, L - 1
+    case = random_case(191 + L, (2,), Hq, Hkv, R, D, C, a, L)
+    q = np.array(case["q"], np.uint16).reshape(2, Hq, R, D).copy()
+    k = np.array(case["k"], np.uint16).reshape(2, Hkv, C, D).copy()
+    k[0, 0, 3, 5] = 0x7F80            # +inf or -inf scores of plane 0, heads 0-3, by the sign of q
+    q[1, 2, 0, 9] = 0x7FC0            # a NaN row
+    k[1, 1, :, :] = 0x0000
+    k[1, 1, :L, 0] = 0xFF80           # every score of plane 1, heads 4-7: -inf, +inf or NaN
+    q[0, 4:, 0, :] = 0x0000
+    q[0, 4:, 0, 0] = 0x5B00           # 2^55 ...
+    k[0, 1, :, :] = 0x0000
+    k[0, 1, :L, 0] = 0xDB00 + (np.arange(L) % 5).astype(np.uint16)   # ... times about -2^55: scores near -1.6e32
+    special = dict(case, q=q.reshape(-1).tolist(), k=k.reshape(-1).tolist())
+    qd, kd, vd, od = device_operands(special)
+    rc, nbytes, _ = iomx.sdpa_workspace(qd.view(), kd.view(), vd.view(), od.view(), a, L)
+    assert rc == 0 and nbytes == 0
+    for t in (qd, kd, vd, od):
+        t.free()
+    got = run(special, 0, expect_kernel="sdpa_decode")
+    want = oracle(special)
+    assert close_to_oracle(got, want) == []
+    g = got.reshape(2, R, Hq, D)
+    assert np.all((g[1, 0, 2] & 0x7FFF) > 0x7F80)                        # the NaN row
+    w = want.reshape(2, R, Hq, D)
+    assert np.array_equal((g[0, 0, 4:] & 0x7F80) == 0x7F80, (w[0, 0, 4:] & 0x7F80) == 0x7F80)
+    # the untouched half (plane 1, heads 0-3 except the NaN row) equals the run without special values
+    plain = run(case, 0).reshape(2, R, Hq, D)
+    assert np.array_equal(g[1, 0, [0, 1, 3]], plain[1, 0, [0, 1, 3]])
+
+
 def test_decode_in_shares_with_special_scores_and_values():
     """Special scores that fall into different shares (a +infinity score in the first and the last
     share, a NaN query row, a row of -infinity scores), an infinite V at a token only the second
