@@ -1197,9 +1197,12 @@ void sdpa_mfma_pair_bf16_kernel(const SdpaArgs a) {
 // outputs take the start of that area over once the wave is through with its scores (a wave's
 // LDS operations complete in order, and no other wave looks at the area before the barrier
 // behind the partial outputs).
-template <int DT16, int PHASE, int KEPT = 0>
+// FULLD: D is DT16 whole tiles and a multiple of 32 -- a constant to the compiler, and no operand
+// load needs a path for a head that ends inside its eight features.
+template <int DT16, int PHASE, int KEPT = 0, bool FULLD = false>
 __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a) {
     static_assert(KEPT == 0 || PHASE == 0, "scores are kept inside one launch");
+    static_assert(!FULLD || DT16 % 2 == 0, "whole 32-feature slices");
     extern __shared__ __attribute__((aligned(16))) uint8_t kept_scores[];
     constexpr int D32 = (DT16 + 1) / 2;
     constexpr int NW = 8;
@@ -1219,6 +1222,8 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
     const bool row_ok = row < a.R;
     const uint32_t qrow = row_ok ? row : a.R - 1;
     const uint32_t nrows = a.grouping * a.R;                          // tile rows in use
+    const uint32_t head_dim = FULLD ? (uint32_t)DT16 * kTile : a.D;
+    const uint32_t d_tiles = FULLD ? (uint32_t)DT16 : a.d_tiles;
     auto p_tile = [&](uint32_t r, uint32_t t) -> float* {
         if constexpr (KEPT == 2) return reinterpret_cast<float*>(kept_scores + wave * a.kept_wave_bytes + (r * 32 + t) * 4);
         else return &p_tile_own[wave][r][t];
@@ -1261,9 +1266,9 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         for (int c = 0; c < D32; ++c) {
             const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
             q_bits[c] = u32x4{0, 0, 0, 0};
-            if (i0 < a.D)
-                q_bits[c] = load_k8_bits(qb + ((uint64_t)(qrow >> 4) * a.d_tiles + tile) * kTileBytes
-                                            + (qrow & 15u) * kRowBytes, c0, i0, a.D);
+            if (FULLD || i0 < head_dim)
+                q_bits[c] = load_k8_bits(qb + ((uint64_t)(qrow >> 4) * d_tiles + tile) * kTileBytes
+                                            + (qrow & 15u) * kRowBytes, c0, i0, head_dim);
         }
         // K of group g (two 16-token tiles), requested one group ahead of its use
         struct KGroup { u32x4 w[2][D32]; };
@@ -1272,12 +1277,13 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             for (int half = 0; half < 2; ++half) {
                 uint32_t token = 32 * g + 16 * half + l16;
                 if (token >= a.L) token = a.L - 1;                    // the cache tail is never touched
-                const uint8_t* krow = kb + (uint64_t)(token >> 4) * a.d_tiles * kTileBytes + (token & 15u) * kRowBytes;
+                const uint8_t* krow = kb + (uint64_t)(token >> 4) * d_tiles * kTileBytes + (token & 15u) * kRowBytes;
 #pragma unroll
                 for (int c = 0; c < D32; ++c) {
                     const uint32_t i0 = 32 * c + 8 * kg, tile = 2 * c + (kg >> 1);
                     kgp.w[half][c] = u32x4{0, 0, 0, 0};
-                    if (i0 < a.D) kgp.w[half][c] = load_k8_bits(krow + (uint64_t)tile * kTileBytes, c0, i0, a.D);
+                    if (FULLD || i0 < head_dim)
+                        kgp.w[half][c] = load_k8_bits(krow + (uint64_t)tile * kTileBytes, c0, i0, head_dim);
                 }
             }
         };
@@ -1307,11 +1313,11 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
             for (int i = 0; i < 8; ++i) {
                 uint32_t token = 32 * g + t0 + i;
                 if (token >= vis_max) token = vis_max - 1;            // its probability is +0 and it is masked below
-                const uint8_t* vrow = vb + (uint64_t)(token >> 4) * a.d_tiles * kTileBytes + (token & 15u) * kRowBytes;
+                const uint8_t* vrow = vb + (uint64_t)(token >> 4) * d_tiles * kTileBytes + (token & 15u) * kRowBytes;
 #pragma unroll
                 for (int c = 0; c < DL; ++c) {
                     const uint32_t d = lane + 64 * c;
-                    value[i][c] = d < a.D ? daz_bf16(*reinterpret_cast<const uint16_t*>(
+                    value[i][c] = (FULLD || d < head_dim) ? daz_bf16(*reinterpret_cast<const uint16_t*>(
                                                     vrow + (uint64_t)(d >> 4) * kTileBytes + (d & 15u) * 2))
                                           : 0.0f;
                 }
@@ -1338,8 +1344,8 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         const uint32_t last_token_tile = (vis_max - 1) >> 4;
         auto load_vf = [&](uint32_t g, VFrag& vf) {
             const uint32_t second = 2 * g + 1 <= last_token_tile ? 2 * g + 1 : 2 * g;
-            const uint8_t* tiles[2] = {vb + (uint64_t)(2 * g) * a.d_tiles * kTileBytes,
-                                       vb + (uint64_t)second * a.d_tiles * kTileBytes};
+            const uint8_t* tiles[2] = {vb + (uint64_t)(2 * g) * d_tiles * kTileBytes,
+                                       vb + (uint64_t)second * d_tiles * kTileBytes};
 #pragma unroll
             for (int dt = 0; dt < DT16; ++dt) {
                 // pairs of 16-bit loads into the halves of one register
@@ -1347,7 +1353,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     uint16_t bits = 0;
-                    if (dt * kTile + l16 < a.D)
+                    if (FULLD || dt * kTile + l16 < head_dim)
                         bits = *reinterpret_cast<const uint16_t*>(
                                 tiles[j >> 2] + dt * kTileBytes + (4 * kg + (j & 3)) * kRowBytes + l16 * 2);
                     h[j >> 1][j & 1] = bits;
@@ -1679,13 +1685,13 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         // thread = (tile row, feature): 16 x D outputs over 512 threads
         for (uint32_t idx = threadIdx.x; idx < 16 * DL * 64; idx += 512) {
             const uint32_t r = idx / (DL * 64), d = idx - r * (DL * 64);
-            if (r >= nrows || d >= a.D) continue;
+            if (r >= nrows || d >= head_dim) continue;
             float sum = 0.0f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) sum += o_part(w, r, d);
             if (PHASE == 2) {
                 // [pair][share][row][D] partial sums of the workspace
-                a.decode_sums[((((uint64_t)p * a.Hkv + hkv) * shares + share) * 16 + r) * a.D + d] = sum;
+                a.decode_sums[((((uint64_t)p * a.Hkv + hkv) * shares + share) * 16 + r) * head_dim + d] = sum;
                 continue;
             }
             if (sum == 0.0f) sum = 0.0f;                                   // -0 is stored as +0
@@ -1701,7 +1707,7 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                 pinf += as_u32(ws[w * 16 * 5 + 2]);
             }
             const bool nan_out = nan || (pinf == 0 && !finite);
-            const uint32_t col = hh * a.D + d;
+            const uint32_t col = hh * head_dim + d;
             uint8_t* ob = a.out + plane[3] * a.out_plane_bytes
                     + (uint64_t)(rr >> 4) * a.out_tile_cols * kTileBytes + (rr & 15u) * kRowBytes;
             *reinterpret_cast<uint16_t*>(ob + (uint64_t)(col >> 4) * kTileBytes + (col & 15u) * 2) =
@@ -1966,26 +1972,36 @@ static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const 
         }
         for (g.plane0 = 0; g.plane0 < g.planes; g.plane0 += 65535u) {
             const dim3 grid(g.Hkv, g.planes - g.plane0 < 65535u ? g.planes - g.plane0 : 65535u, shares);
+#define IOMX_SDPA_DECODE_AS(N, F) \
+        if (shares == 1 && kept_mode == 1) { \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0, 1, F>), grid, dim3(512), kept_bytes, st, g); \
+        } else if (shares == 1 && kept_mode == 2) { \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0, 2, F>), grid, dim3(512), kept_bytes, st, g); \
+        } else if (shares == 1) { \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0, 0, F>), grid, dim3(512), 0, st, g); \
+        } else { \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 1, 0, F>), grid, dim3(512), 0, st, g); \
+            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 2, 0, F>), grid, dim3(512), 0, st, g); \
+            hipLaunchKernelGGL(sdpa_decode_join_kernel, dim3(grid.x, grid.y), dim3(512), 0, st, g, shares); \
+        }
 #define IOMX_SDPA_DECODE(N) \
     case N: \
-        if (shares == 1 && kept_mode == 1) { \
-            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0, 1>), grid, dim3(512), kept_bytes, st, g); \
-        } else if (shares == 1 && kept_mode == 2) { \
-            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0, 2>), grid, dim3(512), kept_bytes, st, g); \
-        } else if (shares == 1) { \
-            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 0>), grid, dim3(512), 0, st, g); \
-        } else { \
-            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 1>), grid, dim3(512), 0, st, g); \
-            hipLaunchKernelGGL((sdpa_decode_bf16_kernel<N, 2>), grid, dim3(512), 0, st, g); \
-            hipLaunchKernelGGL(sdpa_decode_join_kernel, dim3(grid.x, grid.y), dim3(512), 0, st, g, shares); \
-        } \
+        IOMX_SDPA_DECODE_AS(N, false) \
         break;
+            // the two head sizes of the model families (64, 128) as compile-time constants
+            const bool whole_head = g.D == g.d_tiles * 16;
             switch (g.d_tiles) {
-                IOMX_SDPA_DECODE(1) IOMX_SDPA_DECODE(2) IOMX_SDPA_DECODE(3) IOMX_SDPA_DECODE(4)
+                IOMX_SDPA_DECODE(1) IOMX_SDPA_DECODE(2) IOMX_SDPA_DECODE(3)
+                case 4:
+                    if (whole_head) { IOMX_SDPA_DECODE_AS(4, true) } else { IOMX_SDPA_DECODE_AS(4, false) }
+                    break;
                 IOMX_SDPA_DECODE(5) IOMX_SDPA_DECODE(6) IOMX_SDPA_DECODE(7)
-                default: IOMX_SDPA_DECODE(8)
+                default:
+                    if (whole_head) { IOMX_SDPA_DECODE_AS(8, true) } else { IOMX_SDPA_DECODE_AS(8, false) }
+                    break;
             }
 #undef IOMX_SDPA_DECODE
+#undef IOMX_SDPA_DECODE_AS
         }
         record_launch("sdpa_decode", g.Hkv * gz * shares, 512, (uint64_t)g.planes * g.Hq * g.R);
         IOMX_HIP(hipGetLastError());
