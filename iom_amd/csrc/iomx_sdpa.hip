@@ -1988,19 +1988,22 @@ static int sdpa_launch(int dtype, const iomx_view* q, const iomx_view* k, const 
     case N: \
         IOMX_SDPA_DECODE_AS(N, false) \
         break;
-            // the two head sizes of the model families (64, 128) as compile-time constants
+#define IOMX_SDPA_DECODE_EVEN(N) \
+    case N: \
+        if (whole_head) { IOMX_SDPA_DECODE_AS(N, true) } else { IOMX_SDPA_DECODE_AS(N, false) } \
+        break;
+            // head sizes that are whole multiples of 32 (64 and 128 are the model families') as
+            // compile-time constants
             const bool whole_head = g.D == g.d_tiles * 16;
             switch (g.d_tiles) {
-                IOMX_SDPA_DECODE(1) IOMX_SDPA_DECODE(2) IOMX_SDPA_DECODE(3)
-                case 4:
-                    if (whole_head) { IOMX_SDPA_DECODE_AS(4, true) } else { IOMX_SDPA_DECODE_AS(4, false) }
-                    break;
-                IOMX_SDPA_DECODE(5) IOMX_SDPA_DECODE(6) IOMX_SDPA_DECODE(7)
+                IOMX_SDPA_DECODE(1) IOMX_SDPA_DECODE_EVEN(2) IOMX_SDPA_DECODE(3) IOMX_SDPA_DECODE_EVEN(4)
+                IOMX_SDPA_DECODE(5) IOMX_SDPA_DECODE_EVEN(6) IOMX_SDPA_DECODE(7)
                 default:
                     if (whole_head) { IOMX_SDPA_DECODE_AS(8, true) } else { IOMX_SDPA_DECODE_AS(8, false) }
                     break;
             }
 #undef IOMX_SDPA_DECODE
+#undef IOMX_SDPA_DECODE_EVEN
 #undef IOMX_SDPA_DECODE_AS
         }
         record_launch("sdpa_decode", g.Hkv * gz * shares, 512, (uint64_t)g.planes * g.Hq * g.R);
