@@ -67,6 +67,28 @@ __device__ __forceinline__ uint32_t daz2(uint32_t w) {
 __device__ __forceinline__ bf16x8_t daz8(u32x4 v) {
     return __builtin_bit_cast(bf16x8_t, u32x4{daz2(v[0]), daz2(v[1]), daz2(v[2]), daz2(v[3])});
 }
+// The smaller exponent field of each half, over a run of words: zero in a half exactly if some
+// word of the run has a zero exponent field there (a zero or a subnormal).
+typedef unsigned short u16x2_min_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t least_exponents(uint32_t least, uint32_t w) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(u16x2_min_t, least),
+                                                                  __builtin_bit_cast(u16x2_min_t, w & 0x7F807F80u)));
+}
+// N operand words with their subnormals flushed.  Two instructions a word find out whether any
+// lane of the wave holds a zero exponent field at all; only then the six-instruction flush runs
+// (operands of a model hold neither zeros nor subnormals as a rule).
+template <int N>
+__device__ __forceinline__ void daz_words(u32x4 (&v)[N]) {
+    uint32_t least = 0xFFFFFFFFu;
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) least = least_exponents(least, v[i][j]);
+    if (__any((least & 0xFFFFu) == 0u || (least >> 16) == 0u)) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = u32x4{daz2(v[i][0]), daz2(v[i][1]), daz2(v[i][2]), daz2(v[i][3])};
+    }
+}
 __device__ __forceinline__ float daz_bf16(uint32_t h) {
     return as_f32(((h & 0x7F80u) ? h : (h & 0x8000u)) << 16);
 }
@@ -1289,12 +1311,18 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
         };
         // scores: lane gets tokens 32g + 16*half + 4*kg + j (j < 4) of tile row l16
         auto scores = [&](const KGroup& kgp, f32x4_t (&s)[2]) {
+            // (whole heads: one test for the group's words, the flush only if a lane asks for it)
+            u32x4 kw[2 * D32];
+#pragma unroll
+            for (int i = 0; i < 2 * D32; ++i) kw[i] = kgp.w[i / D32][i % D32];
+            if constexpr (FULLD) daz_words(kw);
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int c = 0; c < D32; ++c)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(daz8(kgp.w[half][c]), qf[c], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            FULLD ? __builtin_bit_cast(bf16x8_t, kw[half * D32 + c]) : daz8(kw[half * D32 + c]), qf[c], acc, 0, 0, 0);
                 f32x4_t q = acc * a.inv_scale;
                 if (!a.scale_pow2) {
 #pragma unroll
@@ -1606,9 +1634,11 @@ __global__ __launch_bounds__(512) void sdpa_decode_bf16_kernel(const SdpaArgs a)
                             for (int dt = 0; dt < DT16; ++dt) vr[slot].w[dt][q] &= keep;
                         }
                     }
+                    if constexpr (FULLD) daz_words(vr[slot].w);
 #pragma unroll
                     for (int dt = 0; dt < DT16; ++dt)
-                        om[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(daz8(vr[slot].w[dt]), pf, om[dt], 0, 0, 0);
+                        om[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                FULLD ? __builtin_bit_cast(bf16x8_t, vr[slot].w[dt]) : daz8(vr[slot].w[dt]), pf, om[dt], 0, 0, 0);
                     if (g + PR * NW < full_hi) load_vf(g + PR * NW, vr[slot]);
                 }
             }
