@@ -431,6 +431,39 @@ def test_decode_step_with_special_scores_among_whole_groups(L):
     assert np.array_equal(g[1, 0, [0, 1, 3]], plain[1, 0, [0, 1, 3]])
 
 
+@pytest.mark.parametrize("spec,kernel", [(((), 8, 2, 1, 64, 300, 299, 300), "sdpa_decode"),
+                                         (((), 8, 2, 1, 128, 700, 699, 700), "sdpa_decode"),
+                                         (((), 8, 2, 64, 64, 64, 0, 64), "sdpa_mfma")],
+                         ids=["decode", "decode_kept_scores", "prefill"])
+def test_a_subnormal_k_against_a_huge_q_is_flushed(spec, kernel):
+    """The dot product flushes subnormal operands (src/cpu/sdpa.cpp:57-60).  Sixteen K elements of
+    nearly 2^-126 meet q elements of 2^127: unflushed, the products would raise one token's score of
+    every row by 4 (D = 64), far outside any tolerance.  The other K elements of those features are
+    zeros, so the matrix-core kernels' test for zero exponent fields finds something in every wave
+    that meets these features; the rest of K and all of V hold none."""
+    lead, Hq, Hkv, R, D, C, a, L = spec
+    case = random_case(211 + L, lead, Hq, Hkv, R, D, C, a, L)
+    q = np.array(case["q"], np.uint16).reshape(1, Hq, R, D).copy()
+    k = np.array(case["k"], np.uint16).reshape(1, Hkv, C, D).copy()
+    q[:, :, :, 5:21] = 0x7F00         # 2^127 in sixteen features
+    k[:, :, :, 5:21] = 0x0000
+    k[0, 0, 17, 5:21] = 0x007F        # the largest subnormal, nearly 2^-126: unflushed, +32 on the dot product,
+    k[0, 1, L - 3, 5:21] = 0x807F     # +4 (D = 64) on the score and a factor of 55 on that token's weight
+    case = dict(case, q=q.reshape(-1).tolist(), k=k.reshape(-1).tolist())
+    got = run(case, 0, expect_kernel=kernel)
+    want = oracle(case)
+    assert close_to_oracle(got, want) == []
+    # the check is a sharp one: the same operands with the subnormals made the smallest normal number
+    # give visibly different rows
+    k2 = k.copy()
+    k2[0, 0, 17, 5:21] = 0x0080
+    moved = oracle(dict(case, k=k2.reshape(-1).tolist()))
+    assert close_to_oracle(moved, want) != []
+    ref64, budget = float64_attention(case)                       # (flushes the operands as well)
+    g = datagen.bf16_to_f32(got.reshape(-1)).astype(np.float64).reshape(ref64.shape)
+    assert np.all(np.abs(g - ref64) <= budget)
+
+
 def test_decode_in_shares_with_special_scores_and_values():
     """Special scores that fall into different shares (a +infinity score in the first and the last
     share, a NaN query row, a row of -infinity scores), an infinite V at a token only the second
